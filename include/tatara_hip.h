@@ -1,0 +1,226 @@
+/*
+ * tatara_hip.h — C ABI of the MI355X (gfx950) backend for Tatara's
+ * attention-family hot path.
+ *
+ * This is the drop-in boundary: the entry points below are what a binding of
+ * the reference's backend operator interface
+ * (include/tatara/backend/metal/{resources,pipeline,commands}.h) would bind on
+ * an AMD host.  Plain pointers, sizes and integer status codes only.  Each
+ * declaration cites the reference interface it replaces.
+ *
+ * Model: a device owns HBM buffers; a kernel library resolves the reference's
+ * kernel names ("attn_qk_rope", "attention_decode", "gdn_recurrence", ...) to
+ * pipelines whose buffer-index argument tables are the reference's; a command
+ * buffer records a compute pass (set_pipeline / set_buffer / set_bytes /
+ * dispatch / barrier) and blit commands, `tt_commit` submits the recording to
+ * the queue's HIP stream and `tt_wait` blocks until it has completed.
+ * Validation (null handles, index > 30, offset >= size, zero extents, operand
+ * shapes a kernel assumes) happens on the host before anything is launched and
+ * is reported through the status codes; nothing throws.
+ *
+ * Memory model: buffers live in HBM.  `tt_buffer_contents` exposes a pinned
+ * host staging view of the same size (allocated on first use);
+ * `tt_buffer_did_modify` publishes host writes to HBM and
+ * `tt_buffer_synchronize` fetches device results, the managed-storage idiom
+ * (didModifyRange / synchronizeResource) standing in for the reference's
+ * unified-memory `contents()`.  `tt_buffer_write/read` move bytes without a
+ * staging view; `tt_buffer_wrap` adopts device memory owned by someone else
+ * (a torch tensor, another allocator) without copying.
+ */
+#ifndef TATARA_HIP_H
+#define TATARA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TT_ABI_VERSION 1u
+/* commands.h:29,32 */
+#define TT_MAX_BUFFER_ARGUMENT_INDEX 30u
+#define TT_MAX_INLINE_CONSTANT_BYTES 4096u
+/* commands.h:299 */
+#define TT_DIAGNOSTIC_STORAGE_BYTES 512u
+
+typedef struct tt_device tt_device;
+typedef struct tt_queue tt_queue;
+typedef struct tt_buffer tt_buffer;
+typedef struct tt_library tt_library;
+typedef struct tt_pipeline tt_pipeline;
+typedef struct tt_command_buffer tt_command_buffer;
+
+/* Status codes.  0 is success in every family.  Command errors keep the
+ * numbering of MetalCommandError (commands.h:232-262); resource errors are
+ * MetalResourceError (resources.h:174-184) + 100; pipeline errors are
+ * MetalPipelineError (pipeline.h:99-110) + 200. */
+typedef enum tt_status {
+    TT_OK = 0,
+    TT_CMD_INVALID_COMMAND_QUEUE = 1,
+    TT_CMD_INVALID_COMMAND_BUFFER = 2,
+    TT_CMD_INVALID_EVENT = 3,
+    TT_CMD_INVALID_EVENT_VALUE = 4,
+    TT_CMD_INVALID_COMPUTE_PASS = 5,
+    TT_CMD_INVALID_BLIT_PASS = 6,
+    TT_CMD_INVALID_PIPELINE = 7,
+    TT_CMD_INVALID_BUFFER = 8,
+    TT_CMD_INVALID_BUFFER_INDEX = 9,
+    TT_CMD_INVALID_BUFFER_OFFSET = 10,
+    TT_CMD_INVALID_SOURCE_RANGE = 11,
+    TT_CMD_INVALID_DESTINATION_RANGE = 12,
+    TT_CMD_INVALID_COPY_EXTENT = 13,
+    TT_CMD_INVALID_FILL_EXTENT = 14,
+    TT_CMD_INVALID_DISPATCH_EXTENT = 15,
+    TT_CMD_CONTEXT_OUT_OF_RANGE = 16,
+    TT_CMD_STATE_SLOT_MISMATCH = 17,
+    TT_CMD_INVALID_PENDING_EXECUTION = 18,
+    TT_CMD_COMMAND_BUFFER_CREATION_FAILED = 19,
+    TT_CMD_ENCODER_CREATION_FAILED = 20,
+    TT_CMD_INVALID_DEVICE = 27,
+    TT_CMD_INVALID_STREAM_GROUP = 28,
+    TT_RES_INVALID_DEVICE = 101,
+    TT_RES_SYSTEM_DEVICE_UNAVAILABLE = 102,
+    TT_RES_COMMAND_QUEUE_CREATION_FAILED = 103,
+    TT_RES_INVALID_BUFFER_SIZE = 105,
+    TT_RES_BUFFER_CREATION_FAILED = 106,
+    TT_RES_OWNERSHIP_FAILURE = 107,
+    TT_RES_BUFFER_WINDOW_UNSUPPORTED = 108,
+    TT_PIPE_INVALID_DEVICE = 201,
+    TT_PIPE_INVALID_LIBRARY = 202,
+    TT_PIPE_INVALID_FUNCTION_NAME = 205,
+    TT_PIPE_LIBRARY_COMPILATION_FAILED = 206,
+    TT_PIPE_FUNCTION_LOOKUP_FAILED = 207,
+    TT_PIPE_PIPELINE_CREATION_FAILED = 208
+} tt_status;
+
+/* MetalExecutionFailure (commands.h:281-295). */
+typedef enum tt_failure {
+    TT_FAILURE_NONE = 0,
+    TT_FAILURE_INTERNAL = 1,
+    TT_FAILURE_TIMEOUT = 2,
+    TT_FAILURE_PAGE_FAULT = 3,
+    TT_FAILURE_OUT_OF_MEMORY = 6,
+    TT_FAILURE_INVALID_RESOURCE = 7,
+    TT_FAILURE_DEVICE_REMOVED = 9,
+    TT_FAILURE_UNKNOWN_ERROR = 11
+} tt_failure;
+
+/* MetalExecutionResult + MetalExecutionTiming (commands.h:374-416).  gpu_ms is
+ * the device time between the first and the last recorded command, measured
+ * with HIP events on the queue's stream. */
+typedef struct tt_execution_result {
+    int32_t status;
+    int32_t completed;
+    int32_t failure;
+    int32_t has_native_error_code;
+    int64_t native_error_code;
+    double gpu_ms;
+    uint64_t diagnostic_length;
+    char diagnostic[TT_DIAGNOSTIC_STORAGE_BYTES];
+} tt_execution_result;
+
+uint32_t tt_abi_version(void);
+/* Human-readable name of a status code; never NULL. */
+const char* tt_status_name(int32_t status);
+
+/* ---- resources (resources.h:237-252) ---- */
+/* create_system_device (resources.h:237): HIP device 0 of the process. */
+int32_t tt_device_create(tt_device** out);
+void tt_device_destroy(tt_device* device);
+/* MetalDevice::name (resources.h:41). */
+const char* tt_device_name(const tt_device* device);
+/* Number of compute units of the device (no reference counterpart; used to size
+ * split-K grids). */
+uint32_t tt_device_compute_units(const tt_device* device);
+/* create_command_queue (resources.h:239): one in-order HIP stream. */
+int32_t tt_queue_create(tt_device* device, tt_queue** out);
+void tt_queue_destroy(tt_queue* queue);
+/* The HIP stream (hipStream_t) behind a queue, for event timing by the caller. */
+void* tt_queue_native_stream(tt_queue* queue);
+
+/* create_shared_buffer (resources.h:241) with the zeroed-allocation rule of
+ * decode_step.cpp:49-57 built in: the HBM allocation is zero-filled. */
+int32_t tt_buffer_create(tt_device* device, uint64_t size_bytes, tt_buffer** out);
+/* create_striped_pool_buffer (resources.h:247): count equal stripes,
+ * *stride_out bytes apart (stripe_bytes rounded up to 256). */
+int32_t tt_pool_create(tt_device* device, uint64_t stripe_bytes, uint32_t stripe_count,
+                       tt_buffer** out, uint64_t* stride_out);
+/* create_buffer_window (resources.h:250): aliasing view; keeps the parent alive. */
+int32_t tt_buffer_window(tt_buffer* parent, uint64_t offset, uint64_t length, tt_buffer** out);
+/* Adopt caller-owned device memory (no reference counterpart). */
+int32_t tt_buffer_wrap(tt_device* device, void* device_pointer, uint64_t size_bytes,
+                       tt_buffer** out);
+void tt_buffer_destroy(tt_buffer* buffer);
+/* MetalBuffer::size_bytes / contents (resources.h:133-134). */
+uint64_t tt_buffer_size(const tt_buffer* buffer);
+void* tt_buffer_contents(tt_buffer* buffer);
+void* tt_buffer_device_pointer(tt_buffer* buffer);
+int32_t tt_buffer_did_modify(tt_buffer* buffer, uint64_t offset, uint64_t length);
+int32_t tt_buffer_synchronize(tt_buffer* buffer, uint64_t offset, uint64_t length);
+int32_t tt_buffer_write(tt_buffer* buffer, uint64_t offset, const void* source, uint64_t length);
+int32_t tt_buffer_read(tt_buffer* buffer, uint64_t offset, void* destination, uint64_t length);
+
+/* ---- pipelines (pipeline.h:141-144) ---- */
+/* create_library_with_source (pipeline.h:141): the library is the gfx950 code
+ * object linked into this shared object, so there is no source argument. */
+int32_t tt_library_create(tt_device* device, tt_library** out);
+void tt_library_destroy(tt_library* library);
+/* Number of kernel names the library resolves and the i-th name. */
+uint32_t tt_library_function_count(const tt_library* library);
+const char* tt_library_function_name(const tt_library* library, uint32_t index);
+/* create_function + create_compute_pipeline (pipeline.h:142-143) in one step. */
+int32_t tt_pipeline_create(tt_library* library, const char* function_name, tt_pipeline** out);
+void tt_pipeline_destroy(tt_pipeline* pipeline);
+const char* tt_pipeline_name(const tt_pipeline* pipeline);
+
+/* ---- command encoding (commands.h:418-507) ---- */
+/* create_command_buffer (commands.h:418). */
+int32_t tt_command_buffer_create(tt_queue* queue, tt_command_buffer** out);
+void tt_command_buffer_destroy(tt_command_buffer* command_buffer);
+/* begin_compute_pass / end_compute_pass (commands.h:420, 492).  At most one
+ * pass is open at a time; pass commands outside one return
+ * TT_CMD_INVALID_COMPUTE_PASS. */
+int32_t tt_pass_begin(tt_command_buffer* command_buffer);
+int32_t tt_pass_end(tt_command_buffer* command_buffer);
+/* set_compute_pipeline (commands.h:440). */
+int32_t tt_pass_set_pipeline(tt_command_buffer* command_buffer, const tt_pipeline* pipeline);
+/* set_buffer (commands.h:442): index <= 30, offset < size. */
+int32_t tt_pass_set_buffer(tt_command_buffer* command_buffer, const tt_buffer* buffer,
+                           uint64_t offset_bytes, uint32_t index);
+/* set_bytes (commands.h:456): 1..4096 bytes copied into the recording. */
+int32_t tt_pass_set_bytes(tt_command_buffer* command_buffer, const void* bytes,
+                          uint32_t length_bytes, uint32_t index);
+/* dispatch_threadgroups (commands.h:444).  The grid is the reference call
+ * site's; a pipeline validates it against the shape its operator is
+ * dispatched with and derives its own HIP launch geometry from it. */
+int32_t tt_pass_dispatch(tt_command_buffer* command_buffer, uint64_t groups_x, uint64_t groups_y,
+                         uint64_t groups_z, uint64_t threads_x, uint64_t threads_y,
+                         uint64_t threads_z);
+/* memory_barrier (commands.h:461): the stream is in-order, so this only
+ * validates the pass. */
+int32_t tt_pass_barrier(tt_command_buffer* command_buffer);
+/* copy_buffer / fill_buffer of a blit pass (commands.h:493-498), recorded
+ * directly on the command buffer (outside a compute pass). */
+int32_t tt_blit_copy(tt_command_buffer* command_buffer, const tt_buffer* source,
+                     uint64_t source_offset, tt_buffer* destination, uint64_t destination_offset,
+                     uint64_t length);
+int32_t tt_blit_fill(tt_command_buffer* command_buffer, tt_buffer* destination,
+                     uint64_t destination_offset, uint64_t length, uint8_t value);
+/* Number of commands recorded so far. */
+uint32_t tt_command_count(const tt_command_buffer* command_buffer);
+/* commit (commands.h:500): launches every recorded command on the queue's
+ * stream, bracketed by HIP events.  The recording is kept, so the same command
+ * buffer may be committed again after tt_wait (the per-token walk re-submits
+ * an identical recording). */
+int32_t tt_commit(tt_command_buffer* command_buffer);
+/* wait_until_completed(_timed) (commands.h:501, 506). */
+int32_t tt_wait(tt_command_buffer* command_buffer, tt_execution_result* result);
+/* Discards the recording so the command buffer can be encoded afresh. */
+int32_t tt_command_buffer_reset(tt_command_buffer* command_buffer);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TATARA_HIP_H */

@@ -1,0 +1,864 @@
+// Full-attention decode for gfx950: qk-RMSNorm + partial rotary + cache append,
+// split-K flash-decode over bf16 KV lanes, and the partial-record combine with
+// the sigmoid output gate.
+//
+// Operators registered here, with the reference kernels whose argument tables
+// they accept (src/backend/metal/kernels/attention.metal):
+//   attn_qk_rope (:43), attn_qk_rope_ms (:119)
+//   attention_decode (:200), attention_decode_ms (:283)
+//   attention_decode_scores_values_gqa8 (:674), attention_decode_combine (:1086)
+//   attention_decode_scores_gqa4 (:373), attention_decode_values_gqa8 (:995)
+// plus the lane-batched split path the reference lacks (it re-dispatches the
+// one-lane split path per long row, src/runtime/decode_step.cpp:1249-1259):
+//   attention_decode_split_ms, attention_decode_combine_ms.
+//
+// Flash-decode layout.  One workgroup = 4 wave64 = one (row, kv head, key
+// range).  Each wave owns every 4th block of 32 keys and keeps an online
+// softmax state for the 8 query heads of the kv group:
+//   S^T[key][head] = K[key][:] . Q[head][:]   v_mfma_f32_16x16x32_bf16,
+//       A = K tile read from a per-wave LDS stage (rows padded to 528 B so the
+//       16-lane operand reads are conflict-free), B = Q^T held in registers.
+//       MFMA columns 8..15 repeat heads 0..7.
+//   O^T[dim][head] += V^T[dim][key] P^T[key][head]
+//       A = V^T built in registers: each lane loads 16 B runs of 8 value rows
+//       (a 16-lane group reads 256 contiguous bytes of one row) and transposes
+//       8x8 with v_perm_b32; B = P^T straight from the S^T accumulators.
+//       Columns 0..7 carry bf16(p), columns 8..15 carry bf16(p - bf16(p)), so
+//       the probability enters the product with ~16 mantissa bits at no extra
+//       MFMA cost; the two column sets are added once at the end.
+// HBM traffic is the K and V rows once each (1 KiB per key per kv head); the
+// arithmetic runs at a few percent of MFMA peak, so the kernel is bound by how
+// many loads are in flight, not by compute.
+#include "../tt_internal.h"
+
+namespace tt {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr uint32_t kD = kAttnHeadDim;
+constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
+constexpr uint32_t kLdsRowBytes = 528;      // 512 B key row + 16 B pad
+constexpr uint32_t kWaveLdsBytes = kBlockKeys * kLdsRowBytes;  // 16896
+constexpr uint32_t kWaves = 4;
+constexpr uint32_t kMergeHeadFloats = 260;  // padded head stride of the wave merge
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+    return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+// round-to-nearest-even, NaN/inf truncated; matches the host conversion
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
+    const uint32_t b = __float_as_uint(v);
+    if ((b & 0x7F800000u) == 0x7F800000u) return static_cast<uint16_t>(b >> 16);
+    return static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float round_bf16(float v) {
+    return bf16_bits_to_f32(f32_to_bf16_bits(v));
+}
+__device__ __forceinline__ float sigmoid_gate(uint16_t g) {
+    return 1.0f / (1.0f + __expf(-bf16_bits_to_f32(g)));
+}
+
+// ---------------------------------------------------------------- qk rope ---
+
+struct RopeArgs {
+    const uint16_t* projection;
+    const uint16_t* q_weight;
+    const uint16_t* k_weight;
+    uint16_t* q_out;
+    uint16_t* gate_out;
+    uint16_t* keys;
+    uint16_t* values;
+    const uint32_t* table;      // per row {kv element offset, context}; null = one lane
+    uint32_t context;           // position of row 0 when table is null
+    uint32_t capacity;
+    uint32_t projection_stride; // elements between rows
+    uint32_t query_stride;
+    uint32_t position_per_row;  // 1: block prefill (row r sits at context + r)
+};
+
+// grid (18, rows) x 256: one head per workgroup, one dimension per thread.
+// Sum of squares: 64 threads x 4 values, a 32-lane adjacent-pairs tree per
+// half-wave, then the two halves added (attention.metal:63-88).
+__global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
+    __shared__ float normed[kD];
+    __shared__ float inverse_shared;
+    const uint32_t head = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t d = threadIdx.x;
+    uint32_t position = a.context + (a.position_per_row ? row : 0u);
+    uint64_t kv_offset = 0;
+    if (a.table != nullptr) {
+        kv_offset = a.table[row * 4];
+        position = a.table[row * 4 + 1];
+    }
+    if (position >= a.capacity) return;  // a bad table row must not write outside the cache
+    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const bool is_query = head < kAttnQueryHeads;
+    const uint32_t local = is_query ? head : head - kAttnQueryHeads;
+    const uint32_t base = is_query ? head * 2 * kD : kAttnQGateRows + local * kD;
+    const float x = bf16_bits_to_f32(proj[base + d]);
+    if (d < 64) {
+        float acc = 0.0f;
+        for (uint32_t j = 0; j < 4; ++j) {
+            const float v = bf16_bits_to_f32(proj[base + d * 4 + j]);
+            acc += v * v;
+        }
+        for (uint32_t off = 1; off < 32; off <<= 1) acc += __shfl_xor(acc, off, 64);
+        const float total = acc + __shfl_xor(acc, 32, 64);
+        if (d == 0) {
+            inverse_shared = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+        }
+    }
+    __syncthreads();
+    const float inverse = inverse_shared;
+    const uint16_t weight = is_query ? a.q_weight[d] : a.k_weight[d];
+    // w * bf16(x * inv), the product rounded to bf16 again
+    const float n = round_bf16(bf16_bits_to_f32(weight) * round_bf16(x * inverse));
+    normed[d] = n;
+    __syncthreads();
+    float rotated = n;
+    if (d < 2 * kAttnRopePairs) {
+        const uint32_t pair = d & (kAttnRopePairs - 1);
+        const float theta = static_cast<float>(position) /
+                            powf(kAttnRopeBase, static_cast<float>(pair) /
+                                                    static_cast<float>(kAttnRopePairs));
+        const float c = cosf(theta);
+        const float s = sinf(theta);
+        rotated = d < kAttnRopePairs ? fmaf(-normed[d + kAttnRopePairs], s, n * c)
+                                     : fmaf(normed[d - kAttnRopePairs], s, n * c);
+    }
+    const uint16_t stored = f32_to_bf16_bits(rotated);
+    if (is_query) {
+        const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+        a.q_out[at] = stored;
+        a.gate_out[at] = proj[head * 2 * kD + kD + d];
+    } else {
+        const uint64_t at =
+            kv_offset + (static_cast<uint64_t>(local) * a.capacity + position) * kD + d;
+        a.keys[at] = stored;
+        a.values[at] = proj[kAttnVRowOffset + local * kD + d];
+    }
+}
+
+// ------------------------------------------------------------ flash decode ---
+
+struct FlashArgs {
+    const uint16_t* q;          // [rows][query_stride], head-major 16 x 256 per row
+    const uint16_t* gate;       // same layout (final mode only)
+    const uint16_t* keys;       // pool base; row r's cache at + kv element offset
+    const uint16_t* values;
+    const uint32_t* table;      // per row {kv element offset, context}; null = one lane
+    const uint32_t* row_list;   // optional indirection blockIdx.z -> row
+    float* partials;            // [row][16][record_splits][258]
+    uint16_t* out;              // [rows][query_stride] (final mode only)
+    uint32_t context;           // when table is null
+    uint32_t capacity;
+    uint32_t part;              // keys per workgroup
+    uint32_t record_splits;     // record stride per head
+    uint32_t query_stride;      // elements between rows of q / gate / out
+    uint64_t partial_row_floats;
+    uint32_t final_mode;        // 1: one workgroup sees every key, writes bf16 output
+    uint32_t long_rows_only;    // 1: rows with a single partition are skipped
+    uint32_t single_partition;  // keys of one reference partition (256)
+};
+
+__device__ __forceinline__ uint32_t pack_low(uint32_t a, uint32_t b) {
+    // {a.lo16, b.lo16}
+    return __builtin_amdgcn_perm(b, a, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
+    // {a.hi16, b.hi16}
+    return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+
+__global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t split = blockIdx.x;
+    const uint32_t kvh = blockIdx.y;
+    uint32_t row = blockIdx.z;
+    if (a.row_list != nullptr) row = a.row_list[row];
+    uint64_t kv_offset = 0;
+    uint32_t context = a.context;
+    if (a.table != nullptr) {
+        kv_offset = a.table[row * 4];
+        context = a.table[row * 4 + 1];
+    }
+    if (context >= a.capacity) return;  // a bad table row must not read outside the cache
+    const uint32_t n = context + 1;
+    if (a.long_rows_only && n <= a.single_partition) return;
+    const uint32_t part = a.final_mode ? n : a.part;
+    const uint32_t k0 = split * part;
+    if (k0 >= n) return;
+    const uint32_t k1 = min(n, k0 + part);
+
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+
+    // B operand of S^T: Q^T, column m holds head (m & 7)
+    const uint16_t* qh = a.q + static_cast<uint64_t>(row) * a.query_stride +
+                         (kvh * kAttnHeadsPerKv + (m & 7)) * kD;
+    bf16x8 qreg[8];
+#pragma unroll
+    for (uint32_t kb = 0; kb < 8; ++kb) {
+        qreg[kb] = __builtin_bit_cast(
+            bf16x8, *reinterpret_cast<const u32x4*>(qh + kb * 32 + g * 8));
+    }
+
+    const uint16_t* kbase = a.keys + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
+    const uint16_t* vbase = a.values + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
+    uint8_t* stage = lds + wave * kWaveLdsBytes;
+
+    f32x4 o[16];
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j) o[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY;
+    float l_run = 0.0f;
+
+    const uint32_t nblocks = (k1 - k0 + kBlockKeys - 1) / kBlockKeys;
+    for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
+        const uint32_t key0 = k0 + blk * kBlockKeys;
+        const uint32_t valid = min(kBlockKeys, k1 - key0);
+        // K rows: instruction i moves keys 2i, 2i+1 (1 KiB contiguous per wave)
+        u32x4 kreg[16];
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i) {
+            const uint32_t key = min(2 * i + (lane >> 5), valid - 1);
+            kreg[i] = *reinterpret_cast<const u32x4*>(
+                kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8);
+        }
+        // V rows: contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3)
+        u32x4 vreg[2][8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
+            const uint16_t* vrow = vbase + static_cast<uint64_t>(key0 + key) * kD + m * 8;
+            vreg[0][e] = *reinterpret_cast<const u32x4*>(vrow);
+            vreg[1][e] = *reinterpret_cast<const u32x4*>(vrow + 128);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i) {
+            *reinterpret_cast<u32x4*>(stage + (2 * i + (lane >> 5)) * kLdsRowBytes +
+                                      (lane & 31) * 16) = kreg[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f};
+        f32x4 s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (uint32_t kb = 0; kb < 8; ++kb) {
+            const bf16x8 a0 = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsRowBytes +
+                                                        (kb * 4 + g) * 16));
+            const bf16x8 a1 = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(stage + (16 + m) * kLdsRowBytes +
+                                                        (kb * 4 + g) * 16));
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[kb], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[kb], s1, 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+        // scores of keys g*4+i (s0) and 16+g*4+i (s1) for head m&7
+        float sc[8];
+        float block_max = -INFINITY;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            sc[i] = (g * 4 + i) < valid ? s0[i] * kAttnScale : -INFINITY;
+            sc[4 + i] = (16 + g * 4 + i) < valid ? s1[i] * kAttnScale : -INFINITY;
+            block_max = fmaxf(block_max, fmaxf(sc[i], sc[4 + i]));
+        }
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
+        const float m_new = fmaxf(m_run, block_max);
+        const float alpha = __expf(m_run - m_new);  // 0 on the first block
+        float p[8];
+        float block_sum = 0.0f;
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) {
+            p[e] = __expf(sc[e] - m_new);
+            block_sum += p[e];
+        }
+        block_sum += __shfl_xor(block_sum, 16, 64);
+        block_sum += __shfl_xor(block_sum, 32, 64);
+        l_run = l_run * alpha + block_sum;
+        m_run = m_new;
+        // P^T operand: columns 0..7 the bf16 head, columns 8..15 the residual
+        uint32_t pw[4];
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            float x0 = p[2 * c];
+            float x1 = p[2 * c + 1];
+            if (m >= 8) {
+                x0 -= round_bf16(x0);
+                x1 -= round_bf16(x1);
+            }
+            pw[c] = static_cast<uint32_t>(f32_to_bf16_bits(x0)) |
+                    (static_cast<uint32_t>(f32_to_bf16_bits(x1)) << 16);
+        }
+        const bf16x8 pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) o[j] *= alpha;
+        }
+        // O^T += V^T P^T; MFMA j covers dims (j>>3)*128 + row*8 + (j&7)
+#pragma unroll
+        for (uint32_t hh = 0; hh < 2; ++hh) {
+#pragma unroll
+            for (uint32_t dw = 0; dw < 4; ++dw) {
+                u32x4 lo, hi;
+                lo.x = pack_low(vreg[hh][0][dw], vreg[hh][1][dw]);
+                lo.y = pack_low(vreg[hh][2][dw], vreg[hh][3][dw]);
+                lo.z = pack_low(vreg[hh][4][dw], vreg[hh][5][dw]);
+                lo.w = pack_low(vreg[hh][6][dw], vreg[hh][7][dw]);
+                hi.x = pack_high(vreg[hh][0][dw], vreg[hh][1][dw]);
+                hi.y = pack_high(vreg[hh][2][dw], vreg[hh][3][dw]);
+                hi.z = pack_high(vreg[hh][4][dw], vreg[hh][5][dw]);
+                hi.w = pack_high(vreg[hh][6][dw], vreg[hh][7][dw]);
+                o[hh * 8 + 2 * dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, lo), pb, o[hh * 8 + 2 * dw], 0, 0, 0);
+                o[hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, hi), pb, o[hh * 8 + 2 * dw + 1], 0, 0, 0);
+            }
+        }
+    }
+
+    // fold the residual columns into the head columns, then stage each wave's
+    // {O[8][256], max, sum} in its own LDS region for the cross-wave merge
+    float* merge = reinterpret_cast<float*>(stage);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const float total = o[j][i] + __shfl_xor(o[j][i], 8, 64);
+            if (m < 8) {
+                const uint32_t dim = (j >> 3) * 128 + (g * 4 + i) * 8 + (j & 7);
+                merge[m * kMergeHeadFloats + dim] = total;
+            }
+        }
+    }
+    if (lane < 8) {
+        merge[8 * kMergeHeadFloats + lane * 2] = m_run;
+        merge[8 * kMergeHeadFloats + lane * 2 + 1] = l_run;
+    }
+    __syncthreads();
+
+    const uint32_t t = threadIdx.x;
+    for (uint32_t h = 0; h < kAttnHeadsPerKv; ++h) {
+        float wmax[kWaves];
+        float gmax = -INFINITY;
+#pragma unroll
+        for (uint32_t w = 0; w < kWaves; ++w) {
+            const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
+            wmax[w] = wm[8 * kMergeHeadFloats + h * 2];
+            gmax = fmaxf(gmax, wmax[w]);
+        }
+        float acc = 0.0f;
+        float denom = 0.0f;
+#pragma unroll
+        for (uint32_t w = 0; w < kWaves; ++w) {
+            const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
+            const float scale = wmax[w] == -INFINITY ? 0.0f : __expf(wmax[w] - gmax);
+            acc = fmaf(scale, wm[h * kMergeHeadFloats + t], acc);
+            denom = fmaf(scale, wm[8 * kMergeHeadFloats + h * 2 + 1], denom);
+        }
+        const uint32_t head = kvh * kAttnHeadsPerKv + h;
+        if (a.final_mode) {
+            const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + t;
+            a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
+        } else {
+            float* record = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
+                            (static_cast<uint64_t>(head) * a.record_splits + split) *
+                                kAttnRecordFloats;
+            record[t] = acc;
+            if (t == 0) {
+                record[kD] = gmax;
+                record[kD + 1] = denom;
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------- combine ---
+
+struct CombineArgs {
+    const float* partials;   // [row][16][record_splits][258]
+    const uint16_t* gate;
+    uint16_t* out;
+    const uint32_t* table;   // per row {kv offset, context}; null: nparts is explicit
+    uint32_t nparts;
+    uint32_t part;
+    uint32_t record_splits;
+    uint32_t query_stride;
+    uint64_t partial_row_floats;
+    uint32_t long_rows_only;
+    uint32_t single_partition;
+};
+
+// grid (16, rows) x 256.  out = bf16((sum_p w_p num_p / sum_p w_p sum_p) * sigmoid(gate)),
+// w_p = exp(max_p - max) (attention.metal:1086-1108).
+__global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
+    const uint32_t head = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t d = threadIdx.x;
+    uint32_t nparts = a.nparts;
+    if (a.table != nullptr) {
+        const uint32_t n = a.table[row * 4 + 1] + 1;
+        if (a.long_rows_only && n <= a.single_partition) return;
+        nparts = (n + a.part - 1) / a.part;
+    }
+    const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
+                        static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
+    float gmax = -INFINITY;
+    for (uint32_t p = 0; p < nparts; ++p) gmax = fmaxf(gmax, base[p * kAttnRecordFloats + kD]);
+    float acc = 0.0f;
+    float denom = 0.0f;
+    for (uint32_t p = 0; p < nparts; ++p) {
+        const float* rec = base + static_cast<uint64_t>(p) * kAttnRecordFloats;
+        const float pmax = rec[kD];
+        const float w = pmax == -INFINITY ? 0.0f : __expf(pmax - gmax);
+        acc = fmaf(w, rec[d], acc);
+        denom = fmaf(w, rec[kD + 1], denom);
+    }
+    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+    a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
+}
+
+// ---------------------------------------- separate score / value stages ------
+
+// attention_decode_scores_gqa4: one workgroup per (head, partition); thread t
+// scores key t of the partition; record = {p[0..255], max, sum}
+// (attention.metal:373-448).  Scalar loads; this two-stage path exists for
+// argument-table compatibility, the fused split path is the fast one.
+__global__ __launch_bounds__(256) void attention_scores_kernel(const uint16_t* q,
+                                                               const uint16_t* keys,
+                                                               uint32_t context, uint32_t capacity,
+                                                               uint32_t part, float* weights,
+                                                               uint32_t nparts) {
+    __shared__ float red[256];
+    __shared__ float qs[kD];
+    const uint32_t head = blockIdx.x;
+    const uint32_t partition = blockIdx.y;
+    const uint32_t t = threadIdx.x;
+    const uint32_t n = context + 1;
+    const uint32_t start = partition * part;
+    const uint32_t count = start < n ? min(n - start, part) : 0u;
+    qs[t] = bf16_bits_to_f32(q[head * kD + t]);
+    __syncthreads();
+    float s = -INFINITY;
+    if (t < count) {
+        const uint16_t* k =
+            keys + (static_cast<uint64_t>(head / kAttnHeadsPerKv) * capacity + start + t) * kD;
+        float dot = 0.0f;
+        for (uint32_t d = 0; d < kD; d += 8) {
+            const u32x4 w = *reinterpret_cast<const u32x4*>(k + d);
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                dot = fmaf(qs[d + 2 * c], __uint_as_float(w[c] << 16), dot);
+                dot = fmaf(qs[d + 2 * c + 1], __uint_as_float(w[c] & 0xFFFF0000u), dot);
+            }
+        }
+        s = dot * kAttnScale;
+    }
+    red[t] = s;
+    __syncthreads();
+    for (uint32_t off = 128; off; off >>= 1) {
+        if (t < off) red[t] = fmaxf(red[t], red[t + off]);
+        __syncthreads();
+    }
+    const float pmax = red[0];
+    __syncthreads();
+    const float p = t < count ? __expf(s - pmax) : 0.0f;
+    red[t] = p;
+    __syncthreads();
+    for (uint32_t off = 128; off; off >>= 1) {
+        if (t < off) red[t] += red[t + off];
+        __syncthreads();
+    }
+    float* record = weights + (static_cast<uint64_t>(head) * nparts + partition) * kAttnRecordFloats;
+    record[t] = p;
+    if (t == 0) {
+        record[kD] = pmax;
+        record[kD + 1] = red[0];
+    }
+}
+
+// attention_decode_values_gqa8: one workgroup per (head, partition); thread d
+// accumulates sum_p w_p V[p][d] in ascending p (attention.metal:995-1036).
+__global__ __launch_bounds__(256) void attention_values_kernel(const float* weights,
+                                                               const uint16_t* values,
+                                                               uint32_t context, uint32_t capacity,
+                                                               uint32_t part, float* partials,
+                                                               uint32_t nparts) {
+    __shared__ float w[256];
+    const uint32_t head = blockIdx.x;
+    const uint32_t partition = blockIdx.y;
+    const uint32_t d = threadIdx.x;
+    const uint32_t n = context + 1;
+    const uint32_t start = partition * part;
+    const uint32_t count = start < n ? min(n - start, part) : 0u;
+    const uint64_t rec = (static_cast<uint64_t>(head) * nparts + partition) * kAttnRecordFloats;
+    w[d] = weights[rec + d];
+    __syncthreads();
+    const uint16_t* v =
+        values + (static_cast<uint64_t>(head / kAttnHeadsPerKv) * capacity + start) * kD + d;
+    float acc = 0.0f;
+    for (uint32_t p = 0; p < count; ++p) {
+        acc = fmaf(w[p], bf16_bits_to_f32(v[static_cast<uint64_t>(p) * kD]), acc);
+    }
+    partials[rec + d] = acc;
+    if (d == 0) {
+        partials[rec + kD] = weights[rec + kD];
+        partials[rec + kD + 1] = weights[rec + kD + 1];
+    }
+}
+
+// ---------------------------------------------------------------- launchers --
+
+constexpr uint64_t kQueryBytes = kAttnQueryValues * 2;
+
+uint64_t cache_bytes(uint32_t capacity) {
+    return static_cast<uint64_t>(kAttnKvHeads) * capacity * kD * 2;
+}
+
+int32_t launch_rope(const RopeArgs& r, uint32_t rows, hipStream_t stream) {
+    hipLaunchKernelGGL(attn_qk_rope_kernel, dim3(kAttnQueryHeads + kAttnKvHeads, rows), dim3(256),
+                       0, stream, r);
+    return TT_OK;
+}
+
+// attn_qk_rope: b0 projection, b1 q_w, b2 k_w, b3 q, b4 gate, b5 keys, b6 values,
+// c7 context, c8 capacity; grid 18 x 256 (decode_step.cpp:713-723).
+int32_t op_attn_qk_rope(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only) {
+    Args a(b);
+    RopeArgs r{};
+    r.context = a.constant(7);
+    r.capacity = a.constant(8);
+    a.require(context_ok(r.context, r.capacity), TT_CMD_CONTEXT_OUT_OF_RANGE);
+    r.projection = a.buffer<const uint16_t>(0, kAttnProjectionRows * 2);
+    r.q_weight = a.buffer<const uint16_t>(1, kD * 2);
+    r.k_weight = a.buffer<const uint16_t>(2, kD * 2);
+    r.q_out = a.buffer<uint16_t>(3, kQueryBytes);
+    r.gate_out = a.buffer<uint16_t>(4, kQueryBytes);
+    r.keys = a.buffer<uint16_t>(5, cache_bytes(r.capacity));
+    r.values = a.buffer<uint16_t>(6, cache_bytes(r.capacity));
+    r.projection_stride = kAttnProjectionRows;
+    r.query_stride = kAttnQueryValues;
+    a.require(grid_is(g, 18, 1, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_rope(r, 1, stream);
+}
+
+// Host-side bound of the rows a state table may carry (decode_step.cpp:1007-1009).
+constexpr uint32_t kMaxBatchRows = 16;
+
+// attn_qk_rope_ms: b0 projection slab, b1 q_w, b2 k_w, b3 q slab, b4 gate slab,
+// b5 keys_pool, b6 values_pool, c7 capacity, b8 state_table, c9 projection
+// stride, c10 query stride; grid (18, rows) x 256 (decode_step.cpp:1231-1243).
+// The per-row kv offsets and contexts live in device memory, so pool extents
+// cannot be checked here; the runtime that writes the table guarantees
+// offset + cache <= pool and context < capacity (decode_step.cpp:1022-1062).
+int32_t op_attn_qk_rope_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                           bool validate_only) {
+    Args a(b);
+    RopeArgs r{};
+    r.capacity = a.constant(7);
+    r.projection_stride = a.constant(9);
+    r.query_stride = a.constant(10);
+    const uint32_t rows = static_cast<uint32_t>(g.gy);
+    a.require(g.gx == 18 && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1 && rows >= 1 &&
+                  rows <= kMaxBatchRows,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(r.capacity != 0 && r.projection_stride >= kAttnProjectionRows &&
+                  r.query_stride >= kAttnQueryValues,
+              TT_CMD_INVALID_BUFFER);
+    const uint64_t last = rows - 1;
+    r.projection = a.buffer<const uint16_t>(0, (last * r.projection_stride + kAttnProjectionRows) * 2);
+    r.q_weight = a.buffer<const uint16_t>(1, kD * 2);
+    r.k_weight = a.buffer<const uint16_t>(2, kD * 2);
+    r.q_out = a.buffer<uint16_t>(3, (last * r.query_stride + kAttnQueryValues) * 2);
+    r.gate_out = a.buffer<uint16_t>(4, (last * r.query_stride + kAttnQueryValues) * 2);
+    r.keys = a.buffer<uint16_t>(5, cache_bytes(r.capacity));
+    r.values = a.buffer<uint16_t>(6, cache_bytes(r.capacity));
+    r.table = a.buffer<const uint32_t>(8, rows * 16);
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_rope(r, rows, stream);
+}
+
+}  // namespace
+
+// attn_qk_rope_blk: b0 projection[rows][9216], b1 q_w, b2 k_w, b3 query[rows][16][256],
+// b4 gate[rows][16][256], b5 keys, b6 values, c7 context of row 0, c8 capacity;
+// grid (18, rows) x 256 (prefill_step.cpp:1450-1465; prefill_attention.metal:1-92).
+int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                            bool validate_only) {
+    Args a(b);
+    RopeArgs r{};
+    r.context = a.constant(7);
+    r.capacity = a.constant(8);
+    const uint64_t rows = g.gy;
+    a.require(g.gx == 18 && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1 && rows >= 1 &&
+                  rows <= 65535,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(r.capacity != 0 && static_cast<uint64_t>(r.context) + rows <= r.capacity,
+              TT_CMD_CONTEXT_OUT_OF_RANGE);
+    r.projection = a.buffer<const uint16_t>(0, rows * kAttnProjectionRows * 2);
+    r.q_weight = a.buffer<const uint16_t>(1, kD * 2);
+    r.k_weight = a.buffer<const uint16_t>(2, kD * 2);
+    r.q_out = a.buffer<uint16_t>(3, rows * kQueryBytes);
+    r.gate_out = a.buffer<uint16_t>(4, rows * kQueryBytes);
+    r.keys = a.buffer<uint16_t>(5, cache_bytes(r.capacity));
+    r.values = a.buffer<uint16_t>(6, cache_bytes(r.capacity));
+    r.projection_stride = kAttnProjectionRows;
+    r.query_stride = kAttnQueryValues;
+    r.position_per_row = 1;
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_rope(r, static_cast<uint32_t>(rows), stream);
+}
+
+namespace {
+
+int32_t launch_flash(const FlashArgs& f, uint32_t splits, uint32_t rows, hipStream_t stream) {
+    // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
+    static const hipError_t opted = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(flash_decode_kernel),
+        hipFuncAttributeMaxDynamicSharedMemorySize, kWaves * kWaveLdsBytes);
+    if (opted != hipSuccess) return TT_CMD_INVALID_PIPELINE;
+    hipLaunchKernelGGL(flash_decode_kernel, dim3(splits, kAttnKvHeads, rows), dim3(256),
+                       kWaves * kWaveLdsBytes, stream, f);
+    return TT_OK;
+}
+
+// attention_decode: b0 q, b1 gate, b2 keys, b3 values, c4 context, b5 out,
+// c6 capacity; grid 16 x 256 (decode_step.cpp:239-247).  Any context.
+int32_t op_attention_decode(const Bindings& b, const Grid& g, hipStream_t stream,
+                            bool validate_only) {
+    Args a(b);
+    FlashArgs f{};
+    f.context = a.constant(4);
+    f.capacity = a.constant(6);
+    a.require(context_ok(f.context, f.capacity), TT_CMD_CONTEXT_OUT_OF_RANGE);
+    f.q = a.buffer<const uint16_t>(0, kQueryBytes);
+    f.gate = a.buffer<const uint16_t>(1, kQueryBytes);
+    f.keys = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
+    f.values = a.buffer<const uint16_t>(3, cache_bytes(f.capacity));
+    f.out = a.buffer<uint16_t>(5, kQueryBytes);
+    f.query_stride = kAttnQueryValues;
+    f.final_mode = 1;
+    a.require(grid_is(g, 16, 1, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_flash(f, 1, 1, stream);
+}
+
+// attention_decode_ms: b0 q slab, b1 gate slab, b2 keys_pool, b3 values_pool,
+// b4 state_table, b5 out slab, c6 capacity, b7 bucket_rows, c8 query stride;
+// grid (16, bucket_rows) x 256 (decode_step.cpp:1261-1272).
+int32_t op_attention_decode_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                               bool validate_only) {
+    Args a(b);
+    FlashArgs f{};
+    f.capacity = a.constant(6);
+    f.query_stride = a.constant(8);
+    const uint32_t rows = static_cast<uint32_t>(g.gy);
+    a.require(g.gx == 16 && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1 && rows >= 1 &&
+                  rows <= kMaxBatchRows,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(f.capacity != 0 && f.query_stride >= kAttnQueryValues, TT_CMD_INVALID_BUFFER);
+    f.q = a.buffer<const uint16_t>(0, kQueryBytes);
+    f.gate = a.buffer<const uint16_t>(1, kQueryBytes);
+    f.keys = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
+    f.values = a.buffer<const uint16_t>(3, cache_bytes(f.capacity));
+    f.table = a.buffer<const uint32_t>(4, kMaxBatchRows * 16);
+    f.out = a.buffer<uint16_t>(5, kQueryBytes);
+    f.row_list = a.buffer<const uint32_t>(7, rows * 4);
+    f.final_mode = 1;
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_flash(f, 1, rows, stream);
+}
+
+// attention_decode_scores_values_gqa8: b0 q, b1 keys, b2 values, c3 context,
+// c4 capacity, c5 part, b6 partials[16][nparts][258], c7 nparts;
+// grid (2, nparts) x (256, 4) (decode_step.cpp:296-306).  part may be any
+// positive multiple of 32.
+int32_t op_attention_scores_values(const Bindings& b, const Grid& g, hipStream_t stream,
+                                   bool validate_only) {
+    Args a(b);
+    FlashArgs f{};
+    f.context = a.constant(3);
+    f.capacity = a.constant(4);
+    f.part = a.constant(5);
+    const uint32_t nparts = a.constant(7);
+    a.require(context_ok(f.context, f.capacity), TT_CMD_CONTEXT_OUT_OF_RANGE);
+    a.require(f.part != 0 && f.part % kBlockKeys == 0 && nparts != 0 &&
+                  static_cast<uint64_t>(nparts) * f.part >= static_cast<uint64_t>(f.context) + 1,
+              TT_CMD_INVALID_BUFFER);
+    a.require(g.gx == 2 && g.gy == nparts && g.gz == 1, TT_CMD_INVALID_DISPATCH_EXTENT);
+    f.q = a.buffer<const uint16_t>(0, kQueryBytes);
+    f.keys = a.buffer<const uint16_t>(1, cache_bytes(f.capacity));
+    f.values = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
+    f.partials = a.buffer<float>(
+        6, static_cast<uint64_t>(kAttnQueryHeads) * nparts * kAttnRecordFloats * 4);
+    f.record_splits = nparts;
+    f.query_stride = kAttnQueryValues;
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_flash(f, nparts, 1, stream);
+}
+
+// attention_decode_combine: b0 partials, b1 gate, c2 nparts, b3 out; grid 16 x 256
+// (decode_step.cpp:332-337).
+int32_t op_attention_combine(const Bindings& b, const Grid& g, hipStream_t stream,
+                             bool validate_only) {
+    Args a(b);
+    CombineArgs c{};
+    c.nparts = a.constant(2);
+    a.require(c.nparts != 0, TT_CMD_INVALID_BUFFER);
+    c.partials = a.buffer<const float>(
+        0, static_cast<uint64_t>(kAttnQueryHeads) * c.nparts * kAttnRecordFloats * 4);
+    c.gate = a.buffer<const uint16_t>(1, kQueryBytes);
+    c.out = a.buffer<uint16_t>(3, kQueryBytes);
+    c.record_splits = c.nparts;
+    c.query_stride = kAttnQueryValues;
+    a.require(grid_is(g, 16, 1, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(kAttnQueryHeads, 1), dim3(256), 0, stream, c);
+    return TT_OK;
+}
+
+// attention_decode_split_ms (no reference counterpart; folds every long row of
+// a lane batch into one split-K grid): b0 q slab, b1 keys_pool, b2 values_pool,
+// b3 state_table, b4 partials [rows][16][max_splits][258], c5 capacity,
+// c6 query stride, c7 part (keys per workgroup, multiple of 32), c8 max_splits,
+// c9 long_rows_only (1: rows whose context fits one 256-key partition are left
+// to attention_decode_ms); grid (max_splits, 2, rows) x 256.
+int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                              bool validate_only) {
+    Args a(b);
+    FlashArgs f{};
+    f.capacity = a.constant(5);
+    f.query_stride = a.constant(6);
+    f.part = a.constant(7);
+    f.record_splits = a.constant(8);
+    f.long_rows_only = a.constant(9);
+    f.single_partition = kAttnPartition;
+    const uint32_t rows = static_cast<uint32_t>(g.gz);
+    a.require(f.capacity != 0 && f.query_stride >= kAttnQueryValues && f.part != 0 &&
+                  f.part % kBlockKeys == 0 && f.record_splits != 0 &&
+                  static_cast<uint64_t>(f.record_splits) * f.part >= f.capacity,
+              TT_CMD_INVALID_BUFFER);
+    a.require(g.gx == f.record_splits && g.gy == 2 && rows >= 1 && rows <= kMaxBatchRows &&
+                  g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint64_t last = rows - 1;
+    f.partial_row_floats =
+        static_cast<uint64_t>(kAttnQueryHeads) * f.record_splits * kAttnRecordFloats;
+    f.q = a.buffer<const uint16_t>(0, (last * f.query_stride + kAttnQueryValues) * 2);
+    f.keys = a.buffer<const uint16_t>(1, cache_bytes(f.capacity));
+    f.values = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
+    f.table = a.buffer<const uint32_t>(3, rows * 16);
+    f.partials = a.buffer<float>(4, f.partial_row_floats * rows * 4);
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_flash(f, f.record_splits, rows, stream);
+}
+
+// attention_decode_combine_ms: b0 partials, b1 gate slab, b2 state_table,
+// b3 out slab, c4 part, c5 max_splits, c6 query stride, c7 long_rows_only;
+// grid (16, rows) x 256.
+int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                                bool validate_only) {
+    Args a(b);
+    CombineArgs c{};
+    c.part = a.constant(4);
+    c.record_splits = a.constant(5);
+    c.query_stride = a.constant(6);
+    c.long_rows_only = a.constant(7);
+    c.single_partition = kAttnPartition;
+    const uint32_t rows = static_cast<uint32_t>(g.gy);
+    a.require(c.part != 0 && c.record_splits != 0 && c.query_stride >= kAttnQueryValues,
+              TT_CMD_INVALID_BUFFER);
+    a.require(g.gx == 16 && g.gz == 1 && rows >= 1 && rows <= kMaxBatchRows && g.tx == 256 &&
+                  g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint64_t last = rows - 1;
+    c.partial_row_floats =
+        static_cast<uint64_t>(kAttnQueryHeads) * c.record_splits * kAttnRecordFloats;
+    c.partials = a.buffer<const float>(0, c.partial_row_floats * rows * 4);
+    c.gate = a.buffer<const uint16_t>(1, (last * c.query_stride + kAttnQueryValues) * 2);
+    c.table = a.buffer<const uint32_t>(2, rows * 16);
+    c.out = a.buffer<uint16_t>(3, (last * c.query_stride + kAttnQueryValues) * 2);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
+                       c);
+    return TT_OK;
+}
+
+// attention_decode_scores_gqa4: b0 q, b1 keys, c2 context, c3 capacity, c4 part,
+// b5 weights[16][nparts][258], c6 nparts; grid (4, nparts) x (256, 4)
+// (decode_step.cpp:309-318).
+int32_t op_attention_scores(const Bindings& b, const Grid& g, hipStream_t stream,
+                            bool validate_only) {
+    Args a(b);
+    const uint32_t context = a.constant(2);
+    const uint32_t capacity = a.constant(3);
+    const uint32_t part = a.constant(4);
+    const uint32_t nparts = a.constant(6);
+    a.require(context_ok(context, capacity), TT_CMD_CONTEXT_OUT_OF_RANGE);
+    a.require(part != 0 && part <= 256 && nparts != 0, TT_CMD_INVALID_BUFFER);
+    a.require(g.gx == 4 && g.gy == nparts && g.gz == 1, TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint16_t* q = a.buffer<const uint16_t>(0, kQueryBytes);
+    const uint16_t* keys = a.buffer<const uint16_t>(1, cache_bytes(capacity));
+    float* weights = a.buffer<float>(
+        5, static_cast<uint64_t>(kAttnQueryHeads) * nparts * kAttnRecordFloats * 4);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_scores_kernel, dim3(kAttnQueryHeads, nparts), dim3(256), 0, stream,
+                       q, keys, context, capacity, part, weights, nparts);
+    return TT_OK;
+}
+
+// attention_decode_values_gqa8: b0 weights, b1 values, c2 context, c3 capacity,
+// c4 part, b5 partials, c6 nparts; grid (2, nparts) x (32, 4, 8)
+// (decode_step.cpp:320-329).
+int32_t op_attention_values(const Bindings& b, const Grid& g, hipStream_t stream,
+                            bool validate_only) {
+    Args a(b);
+    const uint32_t context = a.constant(2);
+    const uint32_t capacity = a.constant(3);
+    const uint32_t part = a.constant(4);
+    const uint32_t nparts = a.constant(6);
+    a.require(context_ok(context, capacity), TT_CMD_CONTEXT_OUT_OF_RANGE);
+    a.require(part != 0 && part <= 256 && nparts != 0, TT_CMD_INVALID_BUFFER);
+    a.require(g.gx == 2 && g.gy == nparts && g.gz == 1, TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint64_t record_bytes =
+        static_cast<uint64_t>(kAttnQueryHeads) * nparts * kAttnRecordFloats * 4;
+    const float* weights = a.buffer<const float>(0, record_bytes);
+    const uint16_t* values = a.buffer<const uint16_t>(1, cache_bytes(capacity));
+    float* partials = a.buffer<float>(5, record_bytes);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_values_kernel, dim3(kAttnQueryHeads, nparts), dim3(256), 0, stream,
+                       weights, values, context, capacity, part, partials, nparts);
+    return TT_OK;
+}
+
+}  // namespace
+
+#if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
+const KernelDesc kAttentionDecodeKernels[] = {
+    {"attn_qk_rope", op_attn_qk_rope},
+    {"attn_qk_rope_ms", op_attn_qk_rope_ms},
+    {"attention_decode", op_attention_decode},
+    {"attention_decode_ms", op_attention_decode_ms},
+    {"attention_decode_scores_values_gqa8", op_attention_scores_values},
+    {"attention_decode_combine", op_attention_combine},
+    {"attention_decode_scores_gqa4", op_attention_scores},
+    {"attention_decode_values_gqa8", op_attention_values},
+    {"attention_decode_split_ms", op_attention_split_ms},
+    {"attention_decode_combine_ms", op_attention_combine_ms},
+};
+const uint32_t kAttentionDecodeKernelCount =
+    sizeof(kAttentionDecodeKernels) / sizeof(kAttentionDecodeKernels[0]);
+
+#endif
+
+}  // namespace tt

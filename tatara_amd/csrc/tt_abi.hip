@@ -1,0 +1,674 @@
+// C-ABI core: devices, HBM buffers with a pinned staging view, the kernel
+// library (reference kernel names -> launchers), command recording, submission
+// on an in-order HIP stream and completion reporting.  Mirrors the contract of
+// the reference's backend (src/backend/metal/{resources,pipeline,commands}.mm):
+// typed status codes, validation before any native call, no exceptions.
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "tt_internal.h"
+
+using tt::Bindings;
+using tt::Grid;
+using tt::KernelDesc;
+
+struct tt_device {
+    int ordinal = 0;
+    std::string name;
+    uint32_t compute_units = 0;
+};
+
+struct tt_queue {
+    tt_device* device = nullptr;
+    hipStream_t stream = nullptr;
+};
+
+struct tt_buffer {
+    tt_device* device = nullptr;
+    uint8_t* dptr = nullptr;
+    uint64_t size = 0;
+    uint8_t* host = nullptr;  // pinned staging view, allocated on first contents()
+    bool owns_device = false;
+    tt_buffer* parent = nullptr;  // windows keep their parent alive
+    uint64_t parent_offset = 0;
+    std::atomic<int> refs{1};
+};
+
+struct tt_library {
+    tt_device* device = nullptr;
+    std::vector<KernelDesc> kernels;
+};
+
+struct tt_pipeline {
+    KernelDesc desc{};
+};
+
+namespace {
+
+enum class CommandKind : uint8_t { Dispatch, Copy, Fill };
+
+struct Command {
+    CommandKind kind;
+    tt::LaunchFn launch;
+    Bindings bindings;
+    Grid grid;
+    uint8_t* a;
+    uint8_t* b;
+    uint64_t length;
+    uint8_t value;
+};
+
+__global__ void tt_fill_bytes(uint8_t* dst, uint64_t length, uint8_t value) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < length;
+         i += stride) {
+        dst[i] = value;
+    }
+}
+
+void release_buffer(tt_buffer* buffer) {
+    if (buffer == nullptr) return;
+    if (buffer->refs.fetch_sub(1) != 1) return;
+    if (buffer->parent != nullptr) {
+        release_buffer(buffer->parent);
+    } else {
+        if (buffer->host != nullptr) (void)hipHostFree(buffer->host);
+        if (buffer->owns_device && buffer->dptr != nullptr) (void)hipFree(buffer->dptr);
+    }
+    delete buffer;
+}
+
+int32_t classify(hipError_t error) {
+    switch (error) {
+    case hipSuccess:
+        return TT_FAILURE_NONE;
+    case hipErrorOutOfMemory:
+        return TT_FAILURE_OUT_OF_MEMORY;
+    case hipErrorIllegalAddress:
+        return TT_FAILURE_PAGE_FAULT;
+    case hipErrorLaunchTimeOut:
+        return TT_FAILURE_TIMEOUT;
+    case hipErrorInvalidValue:
+    case hipErrorInvalidDevicePointer:
+    case hipErrorInvalidHandle:
+        return TT_FAILURE_INVALID_RESOURCE;
+    case hipErrorNoDevice:
+    case hipErrorInvalidDevice:
+        return TT_FAILURE_DEVICE_REMOVED;
+    case hipErrorLaunchFailure:
+        return TT_FAILURE_INTERNAL;
+    default:
+        return TT_FAILURE_UNKNOWN_ERROR;
+    }
+}
+
+}  // namespace
+
+struct tt_command_buffer {
+    tt_queue* queue = nullptr;
+    std::vector<Command> commands;
+    bool pass_open = false;
+    const tt_pipeline* pipeline = nullptr;
+    Bindings table{};
+    hipEvent_t begin = nullptr;
+    hipEvent_t end = nullptr;
+    bool committed = false;
+    hipError_t submit_error = hipSuccess;
+};
+
+extern "C" {
+
+uint32_t tt_abi_version(void) { return TT_ABI_VERSION; }
+
+const char* tt_status_name(int32_t status) {
+    switch (status) {
+    case TT_OK: return "None";
+    case TT_CMD_INVALID_COMMAND_QUEUE: return "InvalidCommandQueue";
+    case TT_CMD_INVALID_COMMAND_BUFFER: return "InvalidCommandBuffer";
+    case TT_CMD_INVALID_EVENT: return "InvalidEvent";
+    case TT_CMD_INVALID_EVENT_VALUE: return "InvalidEventValue";
+    case TT_CMD_INVALID_COMPUTE_PASS: return "InvalidComputePass";
+    case TT_CMD_INVALID_BLIT_PASS: return "InvalidBlitPass";
+    case TT_CMD_INVALID_PIPELINE: return "InvalidPipeline";
+    case TT_CMD_INVALID_BUFFER: return "InvalidBuffer";
+    case TT_CMD_INVALID_BUFFER_INDEX: return "InvalidBufferIndex";
+    case TT_CMD_INVALID_BUFFER_OFFSET: return "InvalidBufferOffset";
+    case TT_CMD_INVALID_SOURCE_RANGE: return "InvalidSourceRange";
+    case TT_CMD_INVALID_DESTINATION_RANGE: return "InvalidDestinationRange";
+    case TT_CMD_INVALID_COPY_EXTENT: return "InvalidCopyExtent";
+    case TT_CMD_INVALID_FILL_EXTENT: return "InvalidFillExtent";
+    case TT_CMD_INVALID_DISPATCH_EXTENT: return "InvalidDispatchExtent";
+    case TT_CMD_CONTEXT_OUT_OF_RANGE: return "ContextOutOfRange";
+    case TT_CMD_STATE_SLOT_MISMATCH: return "StateSlotMismatch";
+    case TT_CMD_INVALID_PENDING_EXECUTION: return "InvalidPendingExecution";
+    case TT_CMD_COMMAND_BUFFER_CREATION_FAILED: return "CommandBufferCreationFailed";
+    case TT_CMD_ENCODER_CREATION_FAILED: return "EncoderCreationFailed";
+    case TT_CMD_INVALID_DEVICE: return "InvalidDevice";
+    case TT_CMD_INVALID_STREAM_GROUP: return "InvalidStreamGroup";
+    case TT_RES_INVALID_DEVICE: return "Resource.InvalidDevice";
+    case TT_RES_SYSTEM_DEVICE_UNAVAILABLE: return "Resource.SystemDeviceUnavailable";
+    case TT_RES_COMMAND_QUEUE_CREATION_FAILED: return "Resource.CommandQueueCreationFailed";
+    case TT_RES_INVALID_BUFFER_SIZE: return "Resource.InvalidBufferSize";
+    case TT_RES_BUFFER_CREATION_FAILED: return "Resource.BufferCreationFailed";
+    case TT_RES_OWNERSHIP_FAILURE: return "Resource.OwnershipFailure";
+    case TT_RES_BUFFER_WINDOW_UNSUPPORTED: return "Resource.BufferWindowUnsupported";
+    case TT_PIPE_INVALID_DEVICE: return "Pipeline.InvalidDevice";
+    case TT_PIPE_INVALID_LIBRARY: return "Pipeline.InvalidLibrary";
+    case TT_PIPE_INVALID_FUNCTION_NAME: return "Pipeline.InvalidFunctionName";
+    case TT_PIPE_LIBRARY_COMPILATION_FAILED: return "Pipeline.LibraryCompilationFailed";
+    case TT_PIPE_FUNCTION_LOOKUP_FAILED: return "Pipeline.FunctionLookupFailed";
+    case TT_PIPE_PIPELINE_CREATION_FAILED: return "Pipeline.PipelineCreationFailed";
+    default: return "Unknown";
+    }
+}
+
+/* ---------------------------------------------------------------- resources */
+
+int32_t tt_device_create(tt_device** out) {
+    if (out == nullptr) return TT_RES_INVALID_DEVICE;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return TT_RES_SYSTEM_DEVICE_UNAVAILABLE;
+    }
+    hipDeviceProp_t properties;
+    if (hipSetDevice(0) != hipSuccess || hipGetDeviceProperties(&properties, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_RES_SYSTEM_DEVICE_UNAVAILABLE;
+    }
+    tt_device* device = new (std::nothrow) tt_device;
+    if (device == nullptr) return TT_RES_OWNERSHIP_FAILURE;
+    device->ordinal = 0;
+    device->name = std::string(properties.name) + " (" + properties.gcnArchName + ")";
+    device->compute_units = static_cast<uint32_t>(properties.multiProcessorCount);
+    *out = device;
+    return TT_OK;
+}
+
+void tt_device_destroy(tt_device* device) { delete device; }
+
+const char* tt_device_name(const tt_device* device) {
+    return device != nullptr ? device->name.c_str() : "";
+}
+
+uint32_t tt_device_compute_units(const tt_device* device) {
+    return device != nullptr ? device->compute_units : 0;
+}
+
+int32_t tt_queue_create(tt_device* device, tt_queue** out) {
+    if (out == nullptr) return TT_RES_INVALID_DEVICE;
+    *out = nullptr;
+    if (device == nullptr) return TT_RES_INVALID_DEVICE;
+    hipStream_t stream = nullptr;
+    if (hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_RES_COMMAND_QUEUE_CREATION_FAILED;
+    }
+    tt_queue* queue = new (std::nothrow) tt_queue;
+    if (queue == nullptr) {
+        (void)hipStreamDestroy(stream);
+        return TT_RES_OWNERSHIP_FAILURE;
+    }
+    queue->device = device;
+    queue->stream = stream;
+    *out = queue;
+    return TT_OK;
+}
+
+void tt_queue_destroy(tt_queue* queue) {
+    if (queue == nullptr) return;
+    if (queue->stream != nullptr) {
+        (void)hipStreamSynchronize(queue->stream);
+        (void)hipStreamDestroy(queue->stream);
+    }
+    delete queue;
+}
+
+void* tt_queue_native_stream(tt_queue* queue) {
+    return queue != nullptr ? static_cast<void*>(queue->stream) : nullptr;
+}
+
+int32_t tt_buffer_create(tt_device* device, uint64_t size_bytes, tt_buffer** out) {
+    if (out == nullptr) return TT_RES_INVALID_BUFFER_SIZE;
+    *out = nullptr;
+    if (device == nullptr) return TT_RES_INVALID_DEVICE;
+    if (size_bytes == 0) return TT_RES_INVALID_BUFFER_SIZE;
+    void* dptr = nullptr;
+    if (hipMalloc(&dptr, size_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_RES_BUFFER_CREATION_FAILED;
+    }
+    if (hipMemset(dptr, 0, size_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(dptr);
+        return TT_RES_BUFFER_CREATION_FAILED;
+    }
+    tt_buffer* buffer = new (std::nothrow) tt_buffer;
+    if (buffer == nullptr) {
+        (void)hipFree(dptr);
+        return TT_RES_OWNERSHIP_FAILURE;
+    }
+    buffer->device = device;
+    buffer->dptr = static_cast<uint8_t*>(dptr);
+    buffer->size = size_bytes;
+    buffer->owns_device = true;
+    *out = buffer;
+    return TT_OK;
+}
+
+int32_t tt_pool_create(tt_device* device, uint64_t stripe_bytes, uint32_t stripe_count,
+                       tt_buffer** out, uint64_t* stride_out) {
+    if (out == nullptr || stride_out == nullptr) return TT_RES_INVALID_BUFFER_SIZE;
+    *out = nullptr;
+    *stride_out = 0;
+    if (device == nullptr) return TT_RES_INVALID_DEVICE;
+    if (stripe_bytes == 0 || stripe_count == 0) return TT_RES_INVALID_BUFFER_SIZE;
+    const uint64_t stride = (stripe_bytes + 255u) & ~uint64_t{255};
+    if (stride > UINT64_MAX / stripe_count) return TT_RES_INVALID_BUFFER_SIZE;
+    const int32_t status = tt_buffer_create(device, stride * stripe_count, out);
+    if (status == TT_OK) *stride_out = stride;
+    return status;
+}
+
+int32_t tt_buffer_window(tt_buffer* parent, uint64_t offset, uint64_t length, tt_buffer** out) {
+    if (out == nullptr) return TT_RES_INVALID_BUFFER_SIZE;
+    *out = nullptr;
+    if (parent == nullptr) return TT_RES_BUFFER_WINDOW_UNSUPPORTED;
+    if (length == 0 || offset > parent->size || parent->size - offset < length) {
+        return TT_RES_INVALID_BUFFER_SIZE;
+    }
+    tt_buffer* root = parent->parent != nullptr ? parent->parent : parent;
+    tt_buffer* window = new (std::nothrow) tt_buffer;
+    if (window == nullptr) return TT_RES_OWNERSHIP_FAILURE;
+    window->device = parent->device;
+    window->dptr = parent->dptr + offset;
+    window->size = length;
+    window->parent = root;
+    window->parent_offset = parent->parent_offset + offset;
+    root->refs.fetch_add(1);
+    *out = window;
+    return TT_OK;
+}
+
+int32_t tt_buffer_wrap(tt_device* device, void* device_pointer, uint64_t size_bytes,
+                       tt_buffer** out) {
+    if (out == nullptr) return TT_RES_INVALID_BUFFER_SIZE;
+    *out = nullptr;
+    if (device == nullptr) return TT_RES_INVALID_DEVICE;
+    if (device_pointer == nullptr || size_bytes == 0) return TT_RES_INVALID_BUFFER_SIZE;
+    tt_buffer* buffer = new (std::nothrow) tt_buffer;
+    if (buffer == nullptr) return TT_RES_OWNERSHIP_FAILURE;
+    buffer->device = device;
+    buffer->dptr = static_cast<uint8_t*>(device_pointer);
+    buffer->size = size_bytes;
+    buffer->owns_device = false;
+    *out = buffer;
+    return TT_OK;
+}
+
+void tt_buffer_destroy(tt_buffer* buffer) { release_buffer(buffer); }
+
+uint64_t tt_buffer_size(const tt_buffer* buffer) { return buffer != nullptr ? buffer->size : 0; }
+
+void* tt_buffer_contents(tt_buffer* buffer) {
+    if (buffer == nullptr) return nullptr;
+    tt_buffer* root = buffer->parent != nullptr ? buffer->parent : buffer;
+    if (root->host == nullptr) {
+        void* host = nullptr;
+        if (hipHostMalloc(&host, root->size, hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        std::memset(host, 0, root->size);
+        root->host = static_cast<uint8_t*>(host);
+    }
+    return root->host + buffer->parent_offset;
+}
+
+void* tt_buffer_device_pointer(tt_buffer* buffer) {
+    return buffer != nullptr ? buffer->dptr : nullptr;
+}
+
+static int32_t range_ok(const tt_buffer* buffer, uint64_t offset, uint64_t length) {
+    if (buffer == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (offset > buffer->size || buffer->size - offset < length) return TT_CMD_INVALID_BUFFER_OFFSET;
+    return TT_OK;
+}
+
+int32_t tt_buffer_did_modify(tt_buffer* buffer, uint64_t offset, uint64_t length) {
+    const int32_t status = range_ok(buffer, offset, length);
+    if (status != TT_OK) return status;
+    if (length == 0) return TT_OK;
+    uint8_t* host = static_cast<uint8_t*>(tt_buffer_contents(buffer));
+    if (host == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (hipMemcpy(buffer->dptr + offset, host + offset, length, hipMemcpyHostToDevice) !=
+        hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_INVALID_DESTINATION_RANGE;
+    }
+    return TT_OK;
+}
+
+int32_t tt_buffer_synchronize(tt_buffer* buffer, uint64_t offset, uint64_t length) {
+    const int32_t status = range_ok(buffer, offset, length);
+    if (status != TT_OK) return status;
+    if (length == 0) return TT_OK;
+    uint8_t* host = static_cast<uint8_t*>(tt_buffer_contents(buffer));
+    if (host == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (hipMemcpy(host + offset, buffer->dptr + offset, length, hipMemcpyDeviceToHost) !=
+        hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_INVALID_SOURCE_RANGE;
+    }
+    return TT_OK;
+}
+
+int32_t tt_buffer_write(tt_buffer* buffer, uint64_t offset, const void* source, uint64_t length) {
+    const int32_t status = range_ok(buffer, offset, length);
+    if (status != TT_OK) return status;
+    if (length == 0) return TT_OK;
+    if (source == nullptr) return TT_CMD_INVALID_SOURCE_RANGE;
+    if (hipMemcpy(buffer->dptr + offset, source, length, hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_INVALID_DESTINATION_RANGE;
+    }
+    return TT_OK;
+}
+
+int32_t tt_buffer_read(tt_buffer* buffer, uint64_t offset, void* destination, uint64_t length) {
+    const int32_t status = range_ok(buffer, offset, length);
+    if (status != TT_OK) return status;
+    if (length == 0) return TT_OK;
+    if (destination == nullptr) return TT_CMD_INVALID_DESTINATION_RANGE;
+    if (hipMemcpy(destination, buffer->dptr + offset, length, hipMemcpyDeviceToHost) !=
+        hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_INVALID_SOURCE_RANGE;
+    }
+    return TT_OK;
+}
+
+/* ---------------------------------------------------------------- pipelines */
+
+int32_t tt_library_create(tt_device* device, tt_library** out) {
+    if (out == nullptr) return TT_PIPE_INVALID_LIBRARY;
+    *out = nullptr;
+    if (device == nullptr) return TT_PIPE_INVALID_DEVICE;
+    tt_library* library = new (std::nothrow) tt_library;
+    if (library == nullptr) return TT_PIPE_LIBRARY_COMPILATION_FAILED;
+    library->device = device;
+    const struct {
+        const KernelDesc* table;
+        uint32_t count;
+    } families[] = {
+        {tt::kAttentionDecodeKernels, tt::kAttentionDecodeKernelCount},
+        {tt::kAttentionPrefillKernels, tt::kAttentionPrefillKernelCount},
+        {tt::kGdnDecodeKernels, tt::kGdnDecodeKernelCount},
+        {tt::kGdnPrefillKernels, tt::kGdnPrefillKernelCount},
+    };
+    for (const auto& family : families) {
+        for (uint32_t i = 0; i < family.count; ++i) library->kernels.push_back(family.table[i]);
+    }
+    *out = library;
+    return TT_OK;
+}
+
+void tt_library_destroy(tt_library* library) { delete library; }
+
+uint32_t tt_library_function_count(const tt_library* library) {
+    return library != nullptr ? static_cast<uint32_t>(library->kernels.size()) : 0;
+}
+
+const char* tt_library_function_name(const tt_library* library, uint32_t index) {
+    if (library == nullptr || index >= library->kernels.size()) return nullptr;
+    return library->kernels[index].name;
+}
+
+int32_t tt_pipeline_create(tt_library* library, const char* function_name, tt_pipeline** out) {
+    if (out == nullptr) return TT_PIPE_PIPELINE_CREATION_FAILED;
+    *out = nullptr;
+    if (library == nullptr) return TT_PIPE_INVALID_LIBRARY;
+    if (function_name == nullptr || function_name[0] == '\0') return TT_PIPE_INVALID_FUNCTION_NAME;
+    for (const KernelDesc& desc : library->kernels) {
+        if (std::strcmp(desc.name, function_name) == 0) {
+            tt_pipeline* pipeline = new (std::nothrow) tt_pipeline;
+            if (pipeline == nullptr) return TT_PIPE_PIPELINE_CREATION_FAILED;
+            pipeline->desc = desc;
+            *out = pipeline;
+            return TT_OK;
+        }
+    }
+    return TT_PIPE_FUNCTION_LOOKUP_FAILED;
+}
+
+void tt_pipeline_destroy(tt_pipeline* pipeline) { delete pipeline; }
+
+const char* tt_pipeline_name(const tt_pipeline* pipeline) {
+    return pipeline != nullptr ? pipeline->desc.name : "";
+}
+
+/* ----------------------------------------------------------------- commands */
+
+int32_t tt_command_buffer_create(tt_queue* queue, tt_command_buffer** out) {
+    if (out == nullptr) return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+    *out = nullptr;
+    if (queue == nullptr || queue->stream == nullptr) return TT_CMD_INVALID_COMMAND_QUEUE;
+    tt_command_buffer* cb = new (std::nothrow) tt_command_buffer;
+    if (cb == nullptr) return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+    if (hipEventCreate(&cb->begin) != hipSuccess || hipEventCreate(&cb->end) != hipSuccess) {
+        (void)hipGetLastError();
+        if (cb->begin != nullptr) (void)hipEventDestroy(cb->begin);
+        delete cb;
+        return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+    }
+    cb->queue = queue;
+    *out = cb;
+    return TT_OK;
+}
+
+void tt_command_buffer_destroy(tt_command_buffer* cb) {
+    if (cb == nullptr) return;
+    if (cb->committed) (void)hipEventSynchronize(cb->end);
+    if (cb->begin != nullptr) (void)hipEventDestroy(cb->begin);
+    if (cb->end != nullptr) (void)hipEventDestroy(cb->end);
+    delete cb;
+}
+
+int32_t tt_pass_begin(tt_command_buffer* cb) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_ENCODER_CREATION_FAILED;
+    cb->pass_open = true;
+    cb->pipeline = nullptr;
+    std::memset(&cb->table, 0, sizeof(cb->table));
+    return TT_OK;
+}
+
+int32_t tt_pass_end(tt_command_buffer* cb) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    cb->pass_open = false;
+    cb->pipeline = nullptr;
+    return TT_OK;
+}
+
+int32_t tt_pass_set_pipeline(tt_command_buffer* cb, const tt_pipeline* pipeline) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    if (pipeline == nullptr || pipeline->desc.launch == nullptr) return TT_CMD_INVALID_PIPELINE;
+    cb->pipeline = pipeline;
+    return TT_OK;
+}
+
+int32_t tt_pass_set_buffer(tt_command_buffer* cb, const tt_buffer* buffer, uint64_t offset_bytes,
+                           uint32_t index) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    if (buffer == nullptr || buffer->dptr == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (index > TT_MAX_BUFFER_ARGUMENT_INDEX) return TT_CMD_INVALID_BUFFER_INDEX;
+    if (offset_bytes >= buffer->size) return TT_CMD_INVALID_BUFFER_OFFSET;
+    cb->table.ptr[index] = buffer->dptr + offset_bytes;
+    cb->table.bytes[index] = buffer->size - offset_bytes;
+    cb->table.has_buffer |= 1u << index;
+    cb->table.clen[index] = 0;
+    return TT_OK;
+}
+
+int32_t tt_pass_set_bytes(tt_command_buffer* cb, const void* bytes, uint32_t length_bytes,
+                          uint32_t index) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    if (bytes == nullptr || length_bytes == 0 || length_bytes > TT_MAX_INLINE_CONSTANT_BYTES) {
+        return TT_CMD_INVALID_BUFFER;
+    }
+    if (index > TT_MAX_BUFFER_ARGUMENT_INDEX) return TT_CMD_INVALID_BUFFER_INDEX;
+    uint32_t word = 0;
+    std::memcpy(&word, bytes, length_bytes < 4 ? length_bytes : 4);
+    cb->table.cval[index] = word;
+    cb->table.clen[index] = length_bytes;
+    cb->table.has_buffer &= ~(1u << index);
+    return TT_OK;
+}
+
+int32_t tt_pass_dispatch(tt_command_buffer* cb, uint64_t gx, uint64_t gy, uint64_t gz, uint64_t tx,
+                         uint64_t ty, uint64_t tz) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    if (cb->pipeline == nullptr) return TT_CMD_INVALID_PIPELINE;
+    constexpr uint64_t kLimit = 0x7fffffffull;
+    if (gx == 0 || gy == 0 || gz == 0 || tx == 0 || ty == 0 || tz == 0 || gx > kLimit ||
+        gy > kLimit || gz > kLimit || tx * ty * tz > 1024) {
+        return TT_CMD_INVALID_DISPATCH_EXTENT;
+    }
+    Command command{};
+    command.kind = CommandKind::Dispatch;
+    command.launch = cb->pipeline->desc.launch;
+    command.bindings = cb->table;
+    command.grid = Grid{gx, gy, gz, tx, ty, tz};
+    const int32_t status = command.launch(command.bindings, command.grid, nullptr, true);
+    if (status != TT_OK) return status;
+    cb->commands.push_back(command);
+    return TT_OK;
+}
+
+int32_t tt_pass_barrier(tt_command_buffer* cb) {
+    if (cb == nullptr || !cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    return TT_OK;
+}
+
+int32_t tt_blit_copy(tt_command_buffer* cb, const tt_buffer* source, uint64_t source_offset,
+                     tt_buffer* destination, uint64_t destination_offset, uint64_t length) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_BLIT_PASS;
+    if (source == nullptr || destination == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (length == 0) return TT_CMD_INVALID_COPY_EXTENT;
+    if (source_offset > source->size || source->size - source_offset < length) {
+        return TT_CMD_INVALID_SOURCE_RANGE;
+    }
+    if (destination_offset > destination->size || destination->size - destination_offset < length) {
+        return TT_CMD_INVALID_DESTINATION_RANGE;
+    }
+    Command command{};
+    command.kind = CommandKind::Copy;
+    command.a = source->dptr + source_offset;
+    command.b = destination->dptr + destination_offset;
+    command.length = length;
+    cb->commands.push_back(command);
+    return TT_OK;
+}
+
+int32_t tt_blit_fill(tt_command_buffer* cb, tt_buffer* destination, uint64_t destination_offset,
+                     uint64_t length, uint8_t value) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_BLIT_PASS;
+    if (destination == nullptr) return TT_CMD_INVALID_BUFFER;
+    if (length == 0) return TT_CMD_INVALID_FILL_EXTENT;
+    if (destination_offset > destination->size || destination->size - destination_offset < length) {
+        return TT_CMD_INVALID_DESTINATION_RANGE;
+    }
+    Command command{};
+    command.kind = CommandKind::Fill;
+    command.b = destination->dptr + destination_offset;
+    command.length = length;
+    command.value = value;
+    cb->commands.push_back(command);
+    return TT_OK;
+}
+
+uint32_t tt_command_count(const tt_command_buffer* cb) {
+    return cb != nullptr ? static_cast<uint32_t>(cb->commands.size()) : 0;
+}
+
+int32_t tt_commit(tt_command_buffer* cb) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    hipStream_t stream = cb->queue->stream;
+    cb->submit_error = hipSuccess;
+    (void)hipEventRecord(cb->begin, stream);
+    for (const Command& command : cb->commands) {
+        hipError_t error = hipSuccess;
+        if (command.kind == CommandKind::Dispatch) {
+            const int32_t status = command.launch(command.bindings, command.grid, stream, false);
+            error = hipGetLastError();
+            if (status != TT_OK && error == hipSuccess) error = hipErrorInvalidValue;
+        } else if (command.kind == CommandKind::Copy) {
+            error = hipMemcpyAsync(command.b, command.a, command.length, hipMemcpyDeviceToDevice,
+                                   stream);
+        } else {
+            const uint64_t blocks = (command.length + 255) / 256;
+            const unsigned grid = static_cast<unsigned>(blocks < 4096 ? blocks : 4096);
+            hipLaunchKernelGGL(tt_fill_bytes, dim3(grid), dim3(256), 0, stream, command.b,
+                               command.length, command.value);
+            error = hipGetLastError();
+        }
+        if (error != hipSuccess) {
+            cb->submit_error = error;
+            break;
+        }
+    }
+    (void)hipEventRecord(cb->end, stream);
+    cb->committed = true;
+    return TT_OK;
+}
+
+int32_t tt_wait(tt_command_buffer* cb, tt_execution_result* result) {
+    if (result != nullptr) std::memset(result, 0, sizeof(*result));
+    if (cb == nullptr || !cb->committed) {
+        if (result != nullptr) result->status = TT_CMD_INVALID_PENDING_EXECUTION;
+        return TT_CMD_INVALID_PENDING_EXECUTION;
+    }
+    hipError_t error = hipEventSynchronize(cb->end);
+    if (error == hipSuccess) error = cb->submit_error;
+    float ms = 0.0f;
+    if (error == hipSuccess && hipEventElapsedTime(&ms, cb->begin, cb->end) != hipSuccess) {
+        (void)hipGetLastError();
+        ms = 0.0f;
+    }
+    cb->committed = false;
+    if (result != nullptr) {
+        result->status = TT_OK;
+        result->completed = error == hipSuccess ? 1 : 0;
+        result->failure = classify(error);
+        result->gpu_ms = ms;
+        if (error != hipSuccess) {
+            result->has_native_error_code = 1;
+            result->native_error_code = static_cast<int64_t>(error);
+            const char* text = hipGetErrorString(error);
+            std::snprintf(result->diagnostic, sizeof(result->diagnostic), "%s",
+                          text != nullptr ? text : "unknown HIP error");
+            result->diagnostic_length = std::strlen(result->diagnostic);
+        }
+    }
+    return TT_OK;
+}
+
+int32_t tt_command_buffer_reset(tt_command_buffer* cb) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->committed) (void)hipEventSynchronize(cb->end);
+    cb->committed = false;
+    cb->commands.clear();
+    cb->pass_open = false;
+    cb->pipeline = nullptr;
+    return TT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,293 @@
+"""Full-attention decode on the GPU against the CPU checker, through the C ABI.
+Tolerance of the path: max-abs <= 2e-2, mean-abs <= 2e-3 on bf16 outputs; slot
+indexing (which cache rows are written, raw V and gate copies) is exact."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from golden import cases
+from gpu_util import check_bf16, gpu, run
+
+pytestmark = pytest.mark.gpu
+o = ol.oracle
+
+
+def _weights():
+    q_w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x5157, 256))
+    k_w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x4B57, 256))
+    return q_w, k_w
+
+
+def test_qk_rope_chain_matches_reference_vectors():
+    """Five chained positions on the reference's own fixture inputs (capacity 512)."""
+    print("[case] qk_rope chain, seed 0xA77E1755, capacity 512", flush=True)
+    B, dev, queue, lib = gpu()
+    G = np.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
+    proj, q_w, k_w = cases.attention_chain_inputs(ol.banded_bf16)
+    cap, n = cases.ATTN_CAPACITY, cases.ATTN_CHAIN_POSITIONS
+    b_proj = [dev.buffer_from(proj[p]) for p in range(n)]
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g = dev.create_buffer(8192), dev.create_buffer(8192)
+    b_k, b_v = dev.create_buffer(2 * cap * 512), dev.create_buffer(2 * cap * 512)
+    rope = lib.pipeline("attn_qk_rope")
+
+    def rec(cb):
+        for p in range(n):
+            cb.encode(rope, {0: b_proj[p], 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: b_k, 6: b_v},
+                      {7: p, 8: cap}, (18,), (256,))
+            cb.barrier()
+    run(rec)
+    keys = b_k.read(np.uint16).reshape(2, cap, 256)
+    vals = b_v.read(np.uint16).reshape(2, cap, 256)
+    assert np.array_equal(b_g.read(np.uint16), G["chain_gate"])          # raw copy: exact
+    assert np.array_equal(vals[:, :n], G["chain_values"])                # raw copy: exact
+    assert not keys[:, n:].any() and not vals[:, n:].any()               # slot indexing: exact
+    # banded fixture values reach 2^8, so compare relative to magnitude
+    for got, want, what in ((b_q.read(np.uint16), G["chain_q"], "q"),
+                            (keys[:, :n], G["chain_keys"], "k rows")):
+        g, w = ol.bf16_to_f32(got.reshape(-1)), ol.bf16_to_f32(want.reshape(-1))
+        rel = np.abs(g - w) / np.maximum(np.abs(w), 1e-3)
+        print(f"[parity] rope {what}: exact {np.mean(got.reshape(-1) == want.reshape(-1)):.4f} "
+              f"max-rel {rel.max():.3e}", flush=True)
+        assert rel.max() <= 2 ** -7     # at most one bf16 ulp
+        assert np.mean(got.reshape(-1) == want.reshape(-1)) > 0.99
+
+
+def _fill_cache_by_rope(seed, rows, cap):
+    """K rows normed+roped at their own positions, V raw, through the block rope
+    operator on the GPU and the checker on the CPU; returns both caches."""
+    B, dev, queue, lib = gpu()
+    q_w, k_w = _weights()
+    proj = ol.gaussian_bf16(seed, rows * 9216)
+    keys = np.zeros(2 * cap * 256, np.uint16)
+    values = np.zeros_like(keys)
+    query = np.zeros(rows * 4096, np.uint16)
+    gate = np.zeros_like(query)
+    att = np.zeros_like(query)
+    sel = np.zeros(1, np.uint32)
+    o.tto_attention_prefill(proj, q_w, k_w, rows, 0, cap, query, gate, keys, values, sel, 0, att, 8)
+    b_proj = dev.buffer_from(proj)
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g = dev.create_buffer(rows * 8192), dev.create_buffer(rows * 8192)
+    b_k, b_v = dev.create_buffer(2 * cap * 512), dev.create_buffer(2 * cap * 512)
+    run(lambda cb: cb.encode(lib.pipeline("attn_qk_rope_blk"),
+                             {0: b_proj, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: b_k, 6: b_v},
+                             {7: 0, 8: cap}, (18, rows), (256,)))
+    return dict(proj=proj, q_w=q_w, k_w=k_w, keys=keys, values=values, query=query, gate=gate,
+                b_q=b_q, b_g=b_g, b_k=b_k, b_v=b_v, b_qw=b_qw, b_kw=b_kw)
+
+
+def test_config1_single_decode_step_4096():
+    """Batch 1, 16 q / 2 kv heads, 4096 keys, position 4095: qk-RMSNorm, rotary on
+    64 dims at theta 1e7, softmax(qK^T/16)V * sigmoid(gate)."""
+    print("[case] config 1: decode, context 4095, capacity 4096", flush=True)
+    B, dev, queue, lib = gpu()
+    cap, ctx = 4096, 4095
+    c = _fill_cache_by_rope(0xC0F1, cap, cap)
+    gk = c["b_k"].read(np.uint16)
+    gv = c["b_v"].read(np.uint16)
+    assert np.array_equal(gv, c["values"])                                # raw V: exact
+    check_bf16(gk, c["keys"], "config1 K cache", max_abs=4e-2, mean_abs=1e-4)
+    assert np.mean(gk == c["keys"]) > 0.995
+    # the decode token itself: last row's projection through the one-token operator
+    q_w, k_w = c["q_w"], c["k_w"]
+    proj_last = c["proj"][ctx * 9216:(ctx + 1) * 9216]
+    q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16)
+    keys, values = c["keys"].copy(), c["values"].copy()
+    o.tto_attn_qk_rope(proj_last, q_w, k_w, ctx, cap, q, gate, keys, values)
+    want_tiled = np.zeros(4096, np.uint16); want_split = np.zeros(4096, np.uint16)
+    o.tto_attention_decode(q, gate, keys, values, ctx, cap, want_tiled, 8)
+    o.tto_attention_decode_split(q, gate, keys, values, ctx, cap, 256, None, want_split, 8)
+
+    b_p = dev.buffer_from(proj_last)
+    b_q, b_g, b_o = dev.create_buffer(8192), dev.create_buffer(8192), dev.create_buffer(8192)
+    nparts = (ctx + 256) // 256
+    b_part = dev.create_buffer(16 * nparts * 258 * 4)
+    b_wts = dev.create_buffer(16 * nparts * 258 * 4)
+    outs = {}
+
+    def rec(cb):
+        cb.encode(lib.pipeline("attn_qk_rope"),
+                  {0: b_p, 1: c["b_qw"], 2: c["b_kw"], 3: b_q, 4: b_g, 5: c["b_k"], 6: c["b_v"]},
+                  {7: ctx, 8: cap}, (18,), (256,))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode"),
+                  {0: b_q, 1: b_g, 2: c["b_k"], 3: c["b_v"], 5: b_o}, {4: ctx, 6: cap},
+                  (16,), (256,))
+    run(rec)
+    outs["single"] = b_o.read(np.uint16)
+    check_bf16(b_q.read(np.uint16), q, "config1 q")
+    assert np.array_equal(b_g.read(np.uint16), gate)
+
+    def rec_fused(cb):
+        cb.encode(lib.pipeline("attention_decode_scores_values_gqa8"),
+                  {0: b_q, 1: c["b_k"], 2: c["b_v"], 6: b_part},
+                  {3: ctx, 4: cap, 5: 256, 7: nparts}, (2, nparts), (256, 4))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode_combine"), {0: b_part, 1: b_g, 3: b_o},
+                  {2: nparts}, (16,), (256,))
+    b_o.write(np.zeros(4096, np.uint16))
+    run(rec_fused)
+    outs["fused split"] = b_o.read(np.uint16)
+
+    def rec_two_stage(cb):
+        cb.encode(lib.pipeline("attention_decode_scores_gqa4"), {0: b_q, 1: c["b_k"], 5: b_wts},
+                  {2: ctx, 3: cap, 4: 256, 6: nparts}, (4, nparts), (256, 4))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode_values_gqa8"), {0: b_wts, 1: c["b_v"], 5: b_part},
+                  {2: ctx, 3: cap, 4: 256, 6: nparts}, (2, nparts), (32, 4, 8))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode_combine"), {0: b_part, 1: b_g, 3: b_o},
+                  {2: nparts}, (16,), (256,))
+    b_o.write(np.zeros(4096, np.uint16))
+    run(rec_two_stage)
+    outs["two-stage split"] = b_o.read(np.uint16)
+    check_bf16(outs["single"], want_tiled, "config1 attention_decode vs tiled checker")
+    check_bf16(outs["fused split"], want_split, "config1 scores_values_gqa8+combine")
+    check_bf16(outs["two-stage split"], want_split, "config1 scores+values+combine")
+
+
+@pytest.mark.parametrize("ctx", [0, 1, 30, 31, 32, 33, 63, 64, 127, 255, 256, 257, 300, 511, 512,
+                                 1000])
+def test_decode_context_edges(ctx):
+    print(f"[case] decode edge context {ctx}, capacity 1100", flush=True)
+    B, dev, queue, lib = gpu()
+    cap = 1100
+    q = ol.gaussian_bf16(100 + ctx, 4096); gate = ol.gaussian_bf16(200 + ctx, 4096)
+    keys = ol.gaussian_bf16(300 + ctx, 2 * cap * 256)
+    values = ol.gaussian_bf16(400 + ctx, 2 * cap * 256)
+    # rows past the context hold NaN: they must never be read into the result
+    keys.reshape(2, cap, 256)[:, ctx + 1:] = 0x7FC0
+    values.reshape(2, cap, 256)[:, ctx + 1:] = 0x7FC0
+    want = np.zeros(4096, np.uint16)
+    o.tto_attention_decode_split(q, gate, keys, values, ctx, cap, 256, None, want, 4)
+    b_q, b_g = dev.buffer_from(q), dev.buffer_from(gate)
+    b_k, b_v = dev.buffer_from(keys), dev.buffer_from(values)
+    b_o = dev.create_buffer(8192)
+    run(lambda cb: cb.encode(lib.pipeline("attention_decode"),
+                             {0: b_q, 1: b_g, 2: b_k, 3: b_v, 5: b_o}, {4: ctx, 6: cap},
+                             (16,), (256,)))
+    check_bf16(b_o.read(np.uint16), want, f"attention_decode ctx {ctx}")
+    for part in (256, 64):
+        nparts = (ctx + part) // part
+        b_part = dev.create_buffer(16 * nparts * 258 * 4)
+        b_o2 = dev.create_buffer(8192)
+
+        def rec(cb):
+            cb.encode(lib.pipeline("attention_decode_scores_values_gqa8"),
+                      {0: b_q, 1: b_k, 2: b_v, 6: b_part}, {3: ctx, 4: cap, 5: part, 7: nparts},
+                      (2, nparts), (256, 4))
+            cb.barrier()
+            cb.encode(lib.pipeline("attention_decode_combine"), {0: b_part, 1: b_g, 3: b_o2},
+                      {2: nparts}, (16,), (256,))
+        run(rec)
+        check_bf16(b_o2.read(np.uint16), want, f"split part {part} ctx {ctx}")
+
+
+def _lane_batch(contexts, cap, part, seed):
+    """Lane-batched decode over a striped pool with a state table, long rows
+    through attention_decode_split_ms and short rows through attention_decode_ms."""
+    B, dev, queue, lib = gpu()
+    rows = len(contexts)
+    stripe = 2 * cap * 256          # elements per lane cache
+    k_pool, stride = dev.create_pool(stripe * 2, rows)
+    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    assert stride == stripe * 2
+    q = np.zeros((rows, 4096), np.uint16); gate = np.zeros_like(q)
+    want = np.zeros_like(q)
+    # lanes are placed on stripes in reverse order so row != stripe
+    stripes = list(range(rows))[::-1]
+    table = np.zeros(64, np.uint32)
+    for r, ctx in enumerate(contexts):
+        lane_seed = seed ^ (r * 0x9E3779B97F4A7C15 & 0xFFFFFFFFFFFFFFFF)
+        q[r] = ol.gaussian_bf16(lane_seed + 1, 4096)
+        gate[r] = ol.gaussian_bf16(lane_seed + 2, 4096)
+        n = ctx + 1
+        k = np.zeros((2, cap, 256), np.uint16); v = np.zeros_like(k)
+        k[:, :n] = ol.gaussian_bf16(lane_seed + 3, 2 * n * 256).reshape(2, n, 256)
+        v[:, :n] = ol.gaussian_bf16(lane_seed + 4, 2 * n * 256).reshape(2, n, 256)
+        o.tto_attention_decode_split(q[r], gate[r], k.reshape(-1), v.reshape(-1), ctx, cap, 256,
+                                     None, want[r], 8)
+        k_pool.write(k, stripes[r] * stride)
+        v_pool.write(v, stripes[r] * stride)
+        table[r * 4] = stripes[r] * (stride // 2)
+        table[r * 4 + 1] = ctx
+    short = [r for r, c in enumerate(contexts) if c + 1 <= 256]
+    bucket = np.zeros(16, np.uint32)
+    bucket[:len(short)] = short
+    b_tab = dev.buffer_from(np.concatenate([table, bucket]))
+    b_q, b_g = dev.buffer_from(q), dev.buffer_from(gate)
+    b_o = dev.create_buffer(rows * 8192)
+    max_splits = (cap + part - 1) // part
+    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
+
+    def rec(cb):
+        cb.encode(lib.pipeline("attention_decode_split_ms"),
+                  {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
+                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1}, (max_splits, 2, rows), (256,))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode_combine_ms"),
+                  {0: b_part, 1: b_g, 2: b_tab, 3: b_o},
+                  {4: part, 5: max_splits, 6: 4096, 7: 1}, (16, rows), (256,))
+        if short:
+            cb.encode(lib.pipeline("attention_decode_ms"),
+                      {0: b_q, 1: b_g, 2: k_pool, 3: v_pool, 4: b_tab, 5: b_o,
+                       7: (b_tab, 256)}, {6: cap, 8: 4096}, (16, len(short)), (256,))
+    ms = run(rec)
+    got = b_o.read(np.uint16).reshape(rows, 4096)
+    for r, ctx in enumerate(contexts):
+        check_bf16(got[r], want[r], f"lane {r} ctx {ctx} (stripe {stripes[r]}, part {part})")
+    return ms
+
+
+def test_lane_batch_small_ragged():
+    print("[case] lane batch ragged small", flush=True)
+    _lane_batch([2000, 1499, 700, 100, 255, 256, 0], 2048, 128, 0xBEEF)
+
+
+def test_config3_four_ragged_lanes_at_depth():
+    """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
+    capacity-32768 pool."""
+    print("[case] config 3: 4 ragged lanes 32768/30000/24576/8192", flush=True)
+    _lane_batch([32767, 29999, 24575, 8191], 32768, 512, 0xC0F3)
+
+
+def test_config3_single_lane_100k():
+    print("[case] config 3: 1 lane, 100000 visible keys, capacity 100096", flush=True)
+    _lane_batch([99999], 100096, 512, 0xC0F4)
+
+
+def test_binding_validation_precedes_dispatch():
+    """Typed errors are returned before anything is launched
+    (commands.mm:607-648 behaviour)."""
+    B, dev, queue, lib = gpu()
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    small = dev.create_buffer(64)
+    cb.set_pipeline(lib.pipeline("attention_decode"))
+    with pytest.raises(B.BackendError) as e:
+        cb.set_buffer(small, 64, 0)
+    assert e.value.status == 10          # InvalidBufferOffset
+    with pytest.raises(B.BackendError) as e:
+        cb.set_buffer(small, 0, 31)
+    assert e.value.status == 9           # InvalidBufferIndex
+    with pytest.raises(B.BackendError) as e:
+        cb.dispatch((16, 0, 1), (256,))
+    assert e.value.status == 15          # InvalidDispatchExtent
+    # context == capacity is one past the cache
+    big = dev.create_buffer(2 * 8 * 512)
+    q = dev.create_buffer(8192)
+    for i, b in {0: q, 1: q, 2: big, 3: big, 5: q}.items():
+        cb.set_buffer(b, 0, i)
+    cb.set_bytes(8, 4); cb.set_bytes(8, 6)
+    with pytest.raises(B.BackendError) as e:
+        cb.dispatch((16,), (256,))
+    assert e.value.status == 16          # ContextOutOfRange
+    # a cache smaller than capacity says is refused, not read out of bounds
+    cb.set_bytes(3, 4); cb.set_bytes(4096, 6)
+    with pytest.raises(B.BackendError) as e:
+        cb.dispatch((16,), (256,))
+    assert e.value.status == 10
+    assert cb.command_count == 0

@@ -1,0 +1,174 @@
+"""Gated DeltaNet decode on the GPU against the CPU checker, through the C ABI
+(config: 4 lanes, q/k [16,128], v [32,128], conv history [4,8192] N(0,0.5),
+beta = sigmoid(N(0,1)), decay = exp(U[-0.1,0]), state fp32 [32,128,128] N(0,0.02))."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_util import check_bf16, check_f32, gpu, run
+
+pytestmark = pytest.mark.gpu
+o = ol.oracle
+LANES = 4
+
+
+def _lane_inputs(lane):
+    s = 0x6D2 ^ (lane * 0x9E3779B97F4A7C15 & 0xFFFFFFFFFFFFFFFF)
+    proj = ol.gaussian_bf16(s + 1, 12352, 0.0, 0.5)          # newest conv sample + z + b + a
+    proj[12288:12320] = ol.gaussian_bf16(s + 2, 32)          # b ~ N(0,1): beta = sigmoid(b)
+    conv_state = ol.gaussian_bf16(s + 3, 3 * 8192, 0.0, 0.5)  # three older samples
+    state = ol.gaussian_f32(s + 4, 32 * 128 * 128, 0.0, 0.02)
+    return proj, conv_state, state
+
+
+def _weights():
+    conv_w = ol.gaussian_bf16(0x77, 4 * 8192, 0.0, 0.5)
+    # decay = exp(-exp(A_log) softplus(a + dt_bias)) lands in about [0.9, 1] for these draws
+    a_log = ol.f32_to_bf16(ol.uniform_f32(0x78, 32, -4.0, -2.5))
+    dt_bias = ol.gaussian_bf16(0x79, 32, 0.0, 0.3)
+    norm_w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x7A, 128))
+    return conv_w, a_log, dt_bias, norm_w
+
+
+def test_single_lane_stages_and_chain():
+    """prepare / recurrence / gate-norm one at a time, then a 3-token chain with
+    the ping-pong planes swapped by the host after every token."""
+    print("[case] gdn decode stages, one lane", flush=True)
+    B, dev, queue, lib = gpu()
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    proj, conv_state, state = _lane_inputs(0)
+    b_w, b_al, b_dt, b_nw = (dev.buffer_from(x) for x in (conv_w, a_log, dt_bias, norm_w))
+    b_proj = dev.create_buffer(12352 * 2)
+    conv = [dev.buffer_from(conv_state), dev.create_buffer(3 * 8192 * 2)]
+    rec_ = [dev.buffer_from(state), dev.create_buffer(32 * 128 * 128 * 4)]
+    b_qk, b_v, b_z, b_y, b_out = (dev.create_buffer(8192) for _ in range(5))
+    cs, st = conv_state, state
+    swapped = False
+    for token in range(3):
+        if token:
+            proj = ol.gaussian_bf16(0x900 + token, 12352, 0.0, 0.5)
+        b_proj.write(proj)
+        ci, co = (conv[1], conv[0]) if swapped else (conv[0], conv[1])
+        ri, ro = (rec_[1], rec_[0]) if swapped else (rec_[0], rec_[1])
+
+        def rec(cb):
+            cb.encode(lib.pipeline("gdn_prepare"),
+                      {0: b_proj, 1: ci, 2: b_w, 3: b_qk, 4: b_v, 5: b_z, 6: co}, {}, (96,), (128,))
+            cb.barrier()
+            cb.encode(lib.pipeline("gdn_recurrence"),
+                      {0: b_qk, 1: b_v, 2: b_proj, 3: b_al, 4: b_dt, 5: ri, 6: b_y, 7: ro}, {},
+                      (1, 32, 32), (32, 4, 1))
+            cb.barrier()
+            cb.encode(lib.pipeline("gdn_gate_norm"), {0: b_y, 1: b_z, 2: b_nw, 3: b_out}, {},
+                      (32,), (128,))
+        run(rec)
+        qk = np.zeros(4096, np.uint16); v = np.zeros(4096, np.uint16)
+        z = np.zeros(4096, np.uint16); ncs = np.zeros(3 * 8192, np.uint16)
+        o.tto_gdn_prepare(proj, cs, conv_w, qk, v, z, ncs)
+        decay = np.zeros(32, np.float32); beta = np.zeros(32, np.float32)
+        o.tto_gdn_gates(proj, a_log, dt_bias, decay, beta)
+        y = np.zeros(4096, np.uint16); so = np.zeros_like(st)
+        o.tto_gdn_recurrence(qk, v, decay, beta, st, 16, 32, y, so, 8)
+        gated = np.zeros(4096, np.uint16)
+        o.tto_gdn_gate_norm(y, z, norm_w, 32, gated)
+        check_bf16(b_qk.read(np.uint16), qk, f"token {token} qk")
+        check_bf16(b_v.read(np.uint16), v, f"token {token} v")
+        assert np.array_equal(b_z.read(np.uint16), z)                       # copy: exact
+        assert np.array_equal(co.read(np.uint16), ncs)                      # conv shift: exact
+        check_bf16(b_y.read(np.uint16), y, f"token {token} y")
+        check_f32(ro.read(np.float32), so, f"token {token} state", 2e-3, 2e-5)
+        check_bf16(b_out.read(np.uint16), gated, f"token {token} gated")
+        # continue both sides from the checker's state so errors do not compound in the test
+        cs, st = ncs, so
+        swapped = not swapped
+        ro.write(so); co.write(ncs)
+
+
+def test_recurrence_with_direct_inputs_is_float_exact():
+    """The recurrence alone on L2-normalised q/k fed directly, gates bypassed by
+    a_log/dt_bias/a/b chosen so decay and beta are what the checker derives:
+    the state update has no transcendental, so only the gates can differ."""
+    print("[case] gdn recurrence direct inputs", flush=True)
+    B, dev, queue, lib = gpu()
+    rng = np.random.default_rng(5)
+    qn = rng.standard_normal((16, 128)); kn = rng.standard_normal((16, 128))
+    qn /= np.linalg.norm(qn, axis=1, keepdims=True) * np.sqrt(128.0)
+    kn /= np.linalg.norm(kn, axis=1, keepdims=True)
+    qk = ol.f32_to_bf16(np.concatenate([qn.reshape(-1), kn.reshape(-1)]).astype(np.float32))
+    v = ol.gaussian_bf16(51, 4096)
+    proj = np.zeros(12352, np.uint16)
+    proj[12288:12320] = ol.gaussian_bf16(52, 32)
+    proj[12320:12352] = ol.gaussian_bf16(53, 32)
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    state = ol.gaussian_f32(54, 32 * 128 * 128, 0.0, 0.02)
+    decay = np.zeros(32, np.float32); beta = np.zeros(32, np.float32)
+    o.tto_gdn_gates(proj, a_log, dt_bias, decay, beta)
+    y = np.zeros(4096, np.uint16); so = np.zeros_like(state)
+    o.tto_gdn_recurrence(qk, v, decay, beta, state, 16, 32, y, so, 8)
+    bufs = {0: dev.buffer_from(qk), 1: dev.buffer_from(v), 2: dev.buffer_from(proj),
+            3: dev.buffer_from(a_log), 4: dev.buffer_from(dt_bias), 5: dev.buffer_from(state),
+            6: dev.create_buffer(8192), 7: dev.create_buffer(state.nbytes)}
+    run(lambda cb: cb.encode(lib.pipeline("gdn_recurrence"), bufs, {}, (1, 32, 32), (32, 4, 1)))
+    check_bf16(bufs[6].read(np.uint16), y, "recurrence y")
+    check_f32(bufs[7].read(np.float32), so, "recurrence state", 1e-3, 1e-5)
+
+
+def test_config2_four_lanes_batched():
+    """Four lanes on pool stripes with mixed ping-pong parities through the _ms
+    operators and the state table {conv_in, conv_out, rec_in, rec_out}."""
+    print("[case] config 2: gdn decode x4 lanes, pooled state", flush=True)
+    B, dev, queue, lib = gpu()
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    b_w, b_al, b_dt, b_nw = (dev.buffer_from(x) for x in (conv_w, a_log, dt_bias, norm_w))
+    conv_bytes, rec_bytes = 3 * 8192 * 2, 32 * 128 * 128 * 4
+    conv_pool, conv_stride = dev.create_pool(conv_bytes, 2 * LANES)
+    rec_pool, rec_stride = dev.create_pool(rec_bytes, 2 * LANES)
+    proj = np.zeros((LANES, 12352), np.uint16)
+    swapped = [False, True, True, False]
+    stripes = [2, 0, 3, 1]
+    table = np.zeros(64, np.uint32)
+    want = []
+    for r in range(LANES):
+        p, cs, st = _lane_inputs(r)
+        proj[r] = p
+        par = 1 if swapped[r] else 0
+        conv_pool.write(cs, (2 * stripes[r] + par) * conv_stride)
+        rec_pool.write(st, (2 * stripes[r] + par) * rec_stride)
+        table[r * 4 + 0] = (2 * stripes[r] + par) * (conv_stride // 2)
+        table[r * 4 + 1] = (2 * stripes[r] + 1 - par) * (conv_stride // 2)
+        table[r * 4 + 2] = (2 * stripes[r] + par) * (rec_stride // 4)
+        table[r * 4 + 3] = (2 * stripes[r] + 1 - par) * (rec_stride // 4)
+        ncs = np.zeros(3 * 8192, np.uint16); so = np.zeros_like(st)
+        gated = np.zeros(4096, np.uint16)
+        o.tto_gdn_decode_step(p, cs, conv_w, a_log, dt_bias, norm_w, st, ncs, so, gated, 8)
+        want.append((ncs, so, gated))
+    b_tab = dev.buffer_from(table)
+    b_proj = dev.buffer_from(proj)
+    b_qk, b_v, b_z, b_y, b_out = (dev.create_buffer(LANES * 8192) for _ in range(5))
+
+    def rec(cb):
+        cb.encode(lib.pipeline("gdn_prepare_ms"),
+                  {0: b_proj, 1: conv_pool, 2: b_w, 3: b_qk, 4: b_v, 5: b_z, 6: b_tab},
+                  {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, LANES), (128,))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_recurrence_ms"),
+                  {0: b_qk, 1: b_v, 2: b_proj, 3: b_al, 4: b_dt, 5: rec_pool, 6: b_y, 7: b_tab},
+                  {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32 * LANES), (32, 4, 1))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_gate_norm_ms"), {0: b_y, 1: b_z, 2: b_nw, 3: b_out}, {4: 4096},
+                  (32, LANES), (128,))
+    ms = run(rec)
+    print(f"[time] gdn decode x{LANES} lanes (3 kernels, first run): {ms * 1e3:.1f} us", flush=True)
+    out = b_out.read(np.uint16).reshape(LANES, 4096)
+    for r in range(LANES):
+        ncs, so, gated = want[r]
+        par = 1 if swapped[r] else 0
+        got_cs = conv_pool.read(np.uint16, 3 * 8192, (2 * stripes[r] + 1 - par) * conv_stride)
+        got_st = rec_pool.read(np.float32, 32 * 128 * 128, (2 * stripes[r] + 1 - par) * rec_stride)
+        assert np.array_equal(got_cs, ncs), f"lane {r} conv state plane"
+        check_f32(got_st, so, f"lane {r} state (stripe {stripes[r]}, parity {par})", 2e-3, 2e-5)
+        check_bf16(out[r], gated, f"lane {r} gated")
+        # the input planes are read-only for the step
+        p, cs, st = _lane_inputs(r)
+        assert np.array_equal(conv_pool.read(np.uint16, 3 * 8192,
+                                             (2 * stripes[r] + par) * conv_stride), cs)
