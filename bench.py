@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention-family hot path on one MI355X.
+
+A step is one decode token wave of 4 lanes at 32768 visible keys through one
+hybrid period of the layer stack, G,G,G,A (three Gated DeltaNet layers, one
+full-attention layer), with the lane-batched operators:
+    GDN:       gdn_prepare_ms -> gdn_recurrence_ms -> gdn_gate_norm_ms
+    attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms
+Projections (the reference's Q4 GEMVs) are not on the path: their outputs are
+resident random bf16 slabs.  KV caches, GDN state and all scratch are in HBM
+before the timed region; two copies of the attention layer's KV pools (537 MB in
+total) alternate from step to step so the 256 MB last-level cache cannot serve
+the stream.  The step is compiled into a HIP graph and replayed.
+
+Prints ONE JSON line: `value` = microseconds per layer over the period,
+`roofline` for the dominant kernel (the split-K flash-decode), `cpu_baseline` =
+the CPU checker timed on this box's host cores on the same period."""
+import argparse
+import ctypes as C
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LANES = 4
+VISIBLE = 32768
+CAPACITY = 32768
+PART = 512                      # keys per split-K workgroup
+HBM_PEAK_GBS = 8000.0
+ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
+GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
+
+
+def build_workload(B, dev, lib, torch):
+    """Allocates and fills every buffer of the period; returns the two step
+    recorders (even/odd KV copy) and bookkeeping."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x7A7A)
+    keep = []
+
+    def rand_bf16(n, sigma=1.0):
+        t = (torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma).to(
+            torch.bfloat16)
+        keep.append(t)
+        return dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t)
+
+    def rand_f32(n, sigma):
+        t = torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma
+        keep.append(t)
+        return dev.wrap(t.data_ptr(), t.numel() * 4, keepalive=t)
+
+    def from_np(a):
+        return dev.buffer_from(a)
+
+    rows = LANES
+    context = VISIBLE - 1
+    stripe_elems = 2 * CAPACITY * 256
+    max_splits = (CAPACITY + PART - 1) // PART
+    # attention layer: two alternating KV copies, 4 stripes each
+    kv = [(rand_bf16(rows * stripe_elems), rand_bf16(rows * stripe_elems)) for _ in range(2)]
+    attn_table = np.zeros(64, np.uint32)
+    for r in range(rows):
+        attn_table[r * 4] = r * stripe_elems
+        attn_table[r * 4 + 1] = context
+    b_attn_table = from_np(attn_table)
+    attn_proj = rand_bf16(rows * 9216)
+    q_w = from_np(np.full(256, 0x3F80, np.uint16))
+    k_w = from_np(np.full(256, 0x3F80, np.uint16))
+    b_q, b_gate, b_att = (dev.create_buffer(rows * 8192) for _ in range(3))
+    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
+
+    # three GDN layers, each with its own pooled state and weights
+    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
+    gdn_layers = []
+    for _ in range(3):
+        conv_pool = rand_bf16(2 * rows * conv_elems, 0.5)
+        rec_pool = rand_f32(2 * rows * rec_elems, 0.02)
+        table = np.zeros(64, np.uint32)
+        for r in range(rows):
+            table[r * 4 + 0] = (2 * r) * conv_elems
+            table[r * 4 + 1] = (2 * r + 1) * conv_elems
+            table[r * 4 + 2] = (2 * r) * rec_elems
+            table[r * 4 + 3] = (2 * r + 1) * rec_elems
+        rng = np.random.default_rng(len(gdn_layers) + 1)
+        a_log = (rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16).astype(
+            np.uint16)
+        dt_bias = (rng.normal(0, 0.3, 32).astype(np.float32).view(np.uint32) >> 16).astype(
+            np.uint16)
+        gdn_layers.append(dict(conv=conv_pool, rec=rec_pool, table=from_np(table),
+                               proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
+                               a_log=from_np(a_log), dt_bias=from_np(dt_bias),
+                               norm_w=from_np(np.full(128, 0x3F80, np.uint16))))
+    g_qk, g_v, g_z, g_y, g_out = (dev.create_buffer(rows * 8192) for _ in range(5))
+
+    P = lib.pipeline
+
+    def record(cb, copy):
+        for layer in gdn_layers:
+            cb.encode(P("gdn_prepare_ms"),
+                      {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: g_qk, 4: g_v,
+                       5: g_z, 6: layer["table"]},
+                      {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, rows), (128,))
+            cb.barrier()
+            cb.encode(P("gdn_recurrence_ms"),
+                      {0: g_qk, 1: g_v, 2: layer["proj"], 3: layer["a_log"], 4: layer["dt_bias"],
+                       5: layer["rec"], 6: g_y, 7: layer["table"]},
+                      {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32 * rows),
+                      (32, 4, 1))
+            cb.barrier()
+            cb.encode(P("gdn_gate_norm_ms"), {0: g_y, 1: g_z, 2: layer["norm_w"], 3: g_out},
+                      {4: 4096}, (32, rows), (128,))
+            cb.barrier()
+        keys, values = kv[copy]
+        cb.encode(P("attn_qk_rope_ms"),
+                  {0: attn_proj, 1: q_w, 2: k_w, 3: b_q, 4: b_gate, 5: keys, 6: values,
+                   8: b_attn_table}, {7: CAPACITY, 9: 9216, 10: 4096}, (18, rows), (256,))
+        cb.barrier()
+        cb.encode(P("attention_decode_split_ms"),
+                  {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
+                  {5: CAPACITY, 6: 4096, 7: PART, 8: max_splits, 9: 0}, (max_splits, 2, rows),
+                  (256,))
+        cb.barrier()
+        cb.encode(P("attention_decode_combine_ms"),
+                  {0: b_part, 1: b_gate, 2: b_attn_table, 3: b_att},
+                  {4: PART, 5: max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
+
+    return record, keep
+
+
+def cpu_baseline(threads):
+    """The CPU checker (reference arithmetic restated, oracle/liboracle.so) on one
+    G,G,G,A period at the same shapes: 4 lanes x 32768 keys of attention decode and
+    3 x 4 lanes of GDN decode.  Baseline only; never part of the product path."""
+    path = os.path.join(ROOT, "oracle", "liboracle.so")
+    if not os.path.exists(path):
+        return None
+    L = C.CDLL(path)
+    u16 = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
+    f32 = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+    L.tto_attention_decode_split.argtypes = [u16, u16, u16, u16, C.c_uint32, C.c_uint32,
+                                             C.c_uint32, C.c_void_p, u16, C.c_uint32]
+    L.tto_attention_decode_split.restype = None
+    L.tto_gdn_decode_step.argtypes = [u16] * 6 + [f32, u16, f32, u16, C.c_uint32]
+    L.tto_gdn_decode_step.restype = None
+    rng = np.random.default_rng(7)
+
+    def bf16(n, sigma=1.0):
+        x = rng.standard_normal(n, dtype=np.float32) * np.float32(sigma)
+        return (x.view(np.uint32) >> 16).astype(np.uint16)   # truncation is fine for random data
+
+    keys = bf16(2 * CAPACITY * 256)
+    values = bf16(2 * CAPACITY * 256)
+    q, gate = bf16(4096), bf16(4096)
+    out = np.zeros(4096, np.uint16)
+    proj, cs, cw = bf16(12352, 0.5), bf16(3 * 8192, 0.5), bf16(4 * 8192, 0.5)
+    a_log = np.full(32, 0xC040, np.uint16)   # -3.0
+    dtb = np.zeros(32, np.uint16)
+    nw = np.full(128, 0x3F80, np.uint16)
+    st = (rng.standard_normal(32 * 128 * 128, dtype=np.float32) * 0.02)
+    ncs = np.zeros(3 * 8192, np.uint16)
+    so = np.zeros_like(st)
+    gated = np.zeros(4096, np.uint16)
+    t0 = time.perf_counter()
+    for _ in range(LANES):   # lanes are independent; same-shape data per lane
+        L.tto_attention_decode_split(q, gate, keys, values, VISIBLE - 1, CAPACITY, 256, None, out,
+                                     threads)
+    t_attn = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    for _ in range(3 * LANES):
+        L.tto_gdn_decode_step(proj, cs, cw, a_log, dtb, nw, st, ncs, so, gated, threads)
+    t_gdn = time.perf_counter() - t0
+    return {"value": round((t_attn + t_gdn) * 1e6 / 4.0, 1), "unit": "us/layer",
+            "cores": threads, "kind": "port",
+            "sample": "one full G,G,G,A period, 4 lanes x 32768 keys (attention layer "
+                      f"{t_attn * 1e6:.0f} us, GDN layer {t_gdn * 1e6 / 3:.0f} us)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (lanes and heads "
+              "would shard without exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from tatara_amd import backend as B
+    if not torch.cuda.is_available():
+        print("no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    dev = B.Device()
+    queue = dev.create_queue()
+    lib = dev.create_library()
+    record, keep = build_workload(B, dev, lib, torch)
+
+    steps = []
+    for copy in range(2):
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        record(cb, copy)
+        cb.end_compute_pass()
+        cb.compile()
+        steps.append(cb)
+
+    for k in range(args.warmup):
+        steps[k & 1].commit()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        steps[k & 1].commit()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-kernel device time: eager commits with an event after every command
+    prof = []
+    for copy in range(2):
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        record(cb, copy)
+        cb.end_compute_pass()
+        cb.set_profiling(True)
+        prof.append(cb)
+    per_kernel = {}
+    reps = 30
+    for k in range(reps):
+        cb = prof[k & 1]
+        cb.commit().wait()
+        for name, ms in cb.command_times():
+            per_kernel.setdefault(name, []).append(ms)
+    # one list entry per launch: average launch duration of each kernel
+    kernel_us = {name: round(statistics.mean(v) * 1e3, 2) for name, v in per_kernel.items()}
+    split_us = kernel_us["attention_decode_split_ms"]
+    algo_bytes = LANES * VISIBLE * ATTN_BYTES_PER_KEY
+    achieved = algo_bytes / (split_us * 1e-6) / 1e9
+    attn_layer_us = sum(kernel_us[k] for k in ("attn_qk_rope_ms", "attention_decode_split_ms",
+                                               "attention_decode_combine_ms"))
+    gdn_layer_us = sum(kernel_us[k] for k in ("gdn_prepare_ms", "gdn_recurrence_ms",
+                                              "gdn_gate_norm_ms"))
+    gdn_gbs = LANES * GDN_BYTES_PER_LANE_LAYER / (gdn_layer_us * 1e-6) / 1e9
+
+    line = {
+        "metric": "decode attn+GDN us/layer @32k ctx x4 lanes",
+        "value": round(ms_per_step * 1e3 / 4.0, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "decode wave, 4 lanes x 32768 visible keys, one G,G,G,A period "
+                               "(3 GDN layers + 1 full-attention layer), HIP-graph replay",
+                   "lanes": LANES, "visible_keys": VISIBLE, "capacity": CAPACITY,
+                   "split_keys": PART, "device": dev.name},
+        "roofline": {"bound": "hbm", "kernel": "attention_decode_split_ms (flash_decode_kernel)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": algo_bytes, "avg_launch_us": split_us},
+        "detail": {"attention_layer_us": round(attn_layer_us, 2),
+                   "gdn_layer_us": round(gdn_layer_us, 2),
+                   "gdn_layer_gbs": round(gdn_gbs, 1),
+                   "kernel_avg_us": kernel_us},
+    }
+    if not args.no_cpu_baseline:
+        threads = min(16, os.cpu_count() or 1)
+        line["cpu_baseline"] = cpu_baseline(threads)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -216,6 +216,20 @@ uint32_t tt_command_count(const tt_command_buffer* command_buffer);
 int32_t tt_commit(tt_command_buffer* command_buffer);
 /* wait_until_completed(_timed) (commands.h:501, 506). */
 int32_t tt_wait(tt_command_buffer* command_buffer, tt_execution_result* result);
+/* Compiles the recording into a HIP graph (stream capture); later commits
+ * replay the graph in one launch instead of one launch per command.  Counterpart
+ * of the reference's indirect-command-buffer command graph
+ * (src/runtime/prefill_step.cpp:4165-5415) for launch-bound walks.  Row-batched
+ * (_ms) recordings read contexts and state offsets from the state table in
+ * device memory, so one compiled walk serves every token of a lane group. */
+int32_t tt_command_buffer_compile(tt_command_buffer* command_buffer);
+/* Per-command device timing, the dispatch-boundary counter sampling of
+ * include/tatara/backend/metal/counter_sampling.h: when enabled, an eager
+ * (uncompiled) commit brackets every command with HIP events; after tt_wait,
+ * tt_command_gpu_ms reports command `index`'s device time. */
+int32_t tt_command_buffer_set_profiling(tt_command_buffer* command_buffer, int32_t enabled);
+const char* tt_command_name(const tt_command_buffer* command_buffer, uint32_t index);
+int32_t tt_command_gpu_ms(tt_command_buffer* command_buffer, uint32_t index, double* ms_out);
 /* Discards the recording so the command buffer can be encoded afresh. */
 int32_t tt_command_buffer_reset(tt_command_buffer* command_buffer);
 

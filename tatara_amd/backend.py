@@ -25,7 +25,8 @@ EXPORTED_SYMBOLS = [
     "tt_command_buffer_destroy", "tt_pass_begin", "tt_pass_end", "tt_pass_set_pipeline",
     "tt_pass_set_buffer", "tt_pass_set_bytes", "tt_pass_dispatch", "tt_pass_barrier",
     "tt_blit_copy", "tt_blit_fill", "tt_command_count", "tt_commit", "tt_wait",
-    "tt_command_buffer_reset",
+    "tt_command_buffer_reset", "tt_command_buffer_compile", "tt_command_buffer_set_profiling",
+    "tt_command_name", "tt_command_gpu_ms",
 ]
 
 
@@ -93,6 +94,10 @@ def lib():
         "tt_command_count": (u32, [vp]),
         "tt_commit": (i32, [vp]), "tt_wait": (i32, [vp, C.POINTER(ExecutionResult)]),
         "tt_command_buffer_reset": (i32, [vp]),
+        "tt_command_buffer_compile": (i32, [vp]),
+        "tt_command_buffer_set_profiling": (i32, [vp, i32]),
+        "tt_command_name": (C.c_char_p, [vp, u32]),
+        "tt_command_gpu_ms": (i32, [vp, u32, C.POINTER(C.c_double)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -349,6 +354,24 @@ class CommandBuffer:
     def reset(self):
         _check(lib().tt_command_buffer_reset(self.handle), "reset")
         self._refs.clear()
+
+    def compile(self):
+        """Turns the recording into a HIP graph; later commits replay it."""
+        _check(lib().tt_command_buffer_compile(self.handle), "compile")
+        return self
+
+    def set_profiling(self, enabled=True):
+        _check(lib().tt_command_buffer_set_profiling(self.handle, 1 if enabled else 0),
+               "set_profiling")
+
+    def command_times(self):
+        """[(kernel name, device ms)] of the last eager commit made with profiling on."""
+        out = []
+        for i in range(self.command_count):
+            ms = C.c_double()
+            _check(lib().tt_command_gpu_ms(self.handle, i, C.byref(ms)), "command_gpu_ms")
+            out.append((lib().tt_command_name(self.handle, i).decode(), ms.value))
+        return out
 
     def __del__(self):
         if getattr(self, "handle", None):

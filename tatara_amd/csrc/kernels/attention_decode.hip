@@ -622,11 +622,6 @@ int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream
 namespace {
 
 int32_t launch_flash(const FlashArgs& f, uint32_t splits, uint32_t rows, hipStream_t stream) {
-    // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
-    static const hipError_t opted = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(flash_decode_kernel),
-        hipFuncAttributeMaxDynamicSharedMemorySize, kWaves * kWaveLdsBytes);
-    if (opted != hipSuccess) return TT_CMD_INVALID_PIPELINE;
     hipLaunchKernelGGL(flash_decode_kernel, dim3(splits, kAttnKvHeads, rows), dim3(256),
                        kWaves * kWaveLdsBytes, stream, f);
     return TT_OK;
@@ -844,6 +839,13 @@ int32_t op_attention_values(const Bindings& b, const Grid& g, hipStream_t stream
 }  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
+bool prepare_kernels() {
+    // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kWaves * kWaveLdsBytes) == hipSuccess;
+}
+
 const KernelDesc kAttentionDecodeKernels[] = {
     {"attn_qk_rope", op_attn_qk_rope},
     {"attn_qk_rope_ms", op_attn_qk_rope_ms},

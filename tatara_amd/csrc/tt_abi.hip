@@ -53,6 +53,7 @@ enum class CommandKind : uint8_t { Dispatch, Copy, Fill };
 
 struct Command {
     CommandKind kind;
+    const char* name;
     tt::LaunchFn launch;
     Bindings bindings;
     Grid grid;
@@ -118,7 +119,14 @@ struct tt_command_buffer {
     hipEvent_t end = nullptr;
     bool committed = false;
     hipError_t submit_error = hipSuccess;
+    hipGraph_t graph = nullptr;          // compiled form of the recording
+    hipGraphExec_t graph_exec = nullptr;
+    bool profiling = false;              // eager commits bracket every command with events
+    std::vector<hipEvent_t> marks;       // marks[i], marks[i+1] bracket command i
+    bool marks_valid = false;
 };
+
+static void drop_graph(tt_command_buffer* cb);
 
 extern "C" {
 
@@ -402,6 +410,10 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
     tt_library* library = new (std::nothrow) tt_library;
     if (library == nullptr) return TT_PIPE_LIBRARY_COMPILATION_FAILED;
     library->device = device;
+    if (!tt::prepare_kernels()) {
+        delete library;
+        return TT_PIPE_LIBRARY_COMPILATION_FAILED;
+    }
     const struct {
         const KernelDesc* table;
         uint32_t count;
@@ -476,6 +488,8 @@ void tt_command_buffer_destroy(tt_command_buffer* cb) {
     if (cb->committed) (void)hipEventSynchronize(cb->end);
     if (cb->begin != nullptr) (void)hipEventDestroy(cb->begin);
     if (cb->end != nullptr) (void)hipEventDestroy(cb->end);
+    for (hipEvent_t event : cb->marks) (void)hipEventDestroy(event);
+    drop_graph(cb);
     delete cb;
 }
 
@@ -541,6 +555,7 @@ int32_t tt_pass_dispatch(tt_command_buffer* cb, uint64_t gx, uint64_t gy, uint64
     }
     Command command{};
     command.kind = CommandKind::Dispatch;
+    command.name = cb->pipeline->desc.name;
     command.launch = cb->pipeline->desc.launch;
     command.bindings = cb->table;
     command.grid = Grid{gx, gy, gz, tx, ty, tz};
@@ -569,6 +584,7 @@ int32_t tt_blit_copy(tt_command_buffer* cb, const tt_buffer* source, uint64_t so
     }
     Command command{};
     command.kind = CommandKind::Copy;
+    command.name = "copy_buffer";
     command.a = source->dptr + source_offset;
     command.b = destination->dptr + destination_offset;
     command.length = length;
@@ -587,6 +603,7 @@ int32_t tt_blit_fill(tt_command_buffer* cb, tt_buffer* destination, uint64_t des
     }
     Command command{};
     command.kind = CommandKind::Fill;
+    command.name = "fill_buffer";
     command.b = destination->dptr + destination_offset;
     command.length = length;
     command.value = value;
@@ -598,12 +615,25 @@ uint32_t tt_command_count(const tt_command_buffer* cb) {
     return cb != nullptr ? static_cast<uint32_t>(cb->commands.size()) : 0;
 }
 
-int32_t tt_commit(tt_command_buffer* cb) {
-    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
-    if (cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
-    hipStream_t stream = cb->queue->stream;
-    cb->submit_error = hipSuccess;
-    (void)hipEventRecord(cb->begin, stream);
+static void drop_graph(tt_command_buffer* cb) {
+    if (cb->graph_exec != nullptr) (void)hipGraphExecDestroy(cb->graph_exec);
+    if (cb->graph != nullptr) (void)hipGraphDestroy(cb->graph);
+    cb->graph_exec = nullptr;
+    cb->graph = nullptr;
+}
+
+// Launches every recorded command on the stream in order; with marks, an event
+// is recorded before the first and after each command.
+static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool with_marks) {
+    if (with_marks) {
+        while (cb->marks.size() < cb->commands.size() + 1) {
+            hipEvent_t event = nullptr;
+            if (hipEventCreate(&event) != hipSuccess) return hipGetLastError();
+            cb->marks.push_back(event);
+        }
+        (void)hipEventRecord(cb->marks[0], stream);
+    }
+    size_t index = 0;
     for (const Command& command : cb->commands) {
         hipError_t error = hipSuccess;
         if (command.kind == CommandKind::Dispatch) {
@@ -620,13 +650,76 @@ int32_t tt_commit(tt_command_buffer* cb) {
                                command.length, command.value);
             error = hipGetLastError();
         }
-        if (error != hipSuccess) {
-            cb->submit_error = error;
-            break;
-        }
+        if (error != hipSuccess) return error;
+        ++index;
+        if (with_marks) (void)hipEventRecord(cb->marks[index], stream);
+    }
+    return hipSuccess;
+}
+
+int32_t tt_commit(tt_command_buffer* cb) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    hipStream_t stream = cb->queue->stream;
+    cb->submit_error = hipSuccess;
+    cb->marks_valid = false;
+    (void)hipEventRecord(cb->begin, stream);
+    if (cb->graph_exec != nullptr) {
+        cb->submit_error = hipGraphLaunch(cb->graph_exec, stream);
+    } else {
+        cb->submit_error = issue_commands(cb, stream, cb->profiling);
+        cb->marks_valid = cb->profiling && cb->submit_error == hipSuccess;
     }
     (void)hipEventRecord(cb->end, stream);
     cb->committed = true;
+    return TT_OK;
+}
+
+int32_t tt_command_buffer_compile(tt_command_buffer* cb) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
+    if (cb->commands.empty()) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->committed) (void)hipEventSynchronize(cb->end);
+    drop_graph(cb);
+    hipStream_t stream = cb->queue->stream;
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+    }
+    const hipError_t issued = issue_commands(cb, stream, false);
+    const hipError_t ended = hipStreamEndCapture(stream, &cb->graph);
+    if (issued != hipSuccess || ended != hipSuccess || cb->graph == nullptr ||
+        hipGraphInstantiate(&cb->graph_exec, cb->graph, nullptr, nullptr, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        drop_graph(cb);
+        return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+    }
+    return TT_OK;
+}
+
+int32_t tt_command_buffer_set_profiling(tt_command_buffer* cb, int32_t enabled) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    cb->profiling = enabled != 0;
+    return TT_OK;
+}
+
+const char* tt_command_name(const tt_command_buffer* cb, uint32_t index) {
+    if (cb == nullptr || index >= cb->commands.size()) return nullptr;
+    return cb->commands[index].name;
+}
+
+int32_t tt_command_gpu_ms(tt_command_buffer* cb, uint32_t index, double* ms_out) {
+    if (cb == nullptr || ms_out == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    *ms_out = 0.0;
+    if (!cb->marks_valid || cb->committed || index >= cb->commands.size()) {
+        return TT_CMD_INVALID_PENDING_EXECUTION;
+    }
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, cb->marks[index], cb->marks[index + 1]) != hipSuccess) {
+        (void)hipGetLastError();
+        return TT_CMD_INVALID_PENDING_EXECUTION;
+    }
+    *ms_out = ms;
     return TT_OK;
 }
 
@@ -666,6 +759,8 @@ int32_t tt_command_buffer_reset(tt_command_buffer* cb) {
     if (cb->committed) (void)hipEventSynchronize(cb->end);
     cb->committed = false;
     cb->commands.clear();
+    cb->marks_valid = false;
+    drop_graph(cb);
     cb->pass_open = false;
     cb->pipeline = nullptr;
     return TT_OK;

@@ -87,6 +87,10 @@ inline bool grid_is(const Grid& g, uint64_t gx, uint64_t gy, uint64_t gz, uint64
 int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream,
                             bool validate_only);
 
+// One-time kernel attribute set-up (large dynamic LDS opt-in); called when a
+// library is created, so it never runs inside a stream capture.
+bool prepare_kernels();
+
 extern const KernelDesc kAttentionDecodeKernels[];
 extern const uint32_t kAttentionDecodeKernelCount;
 extern const KernelDesc kAttentionPrefillKernels[];
