@@ -31,13 +31,13 @@ sys.path.insert(0, ROOT)
 LANES = 4
 VISIBLE = 32768
 CAPACITY = 32768
-PART = 512                      # keys per split-K workgroup
+DEFAULT_SPLIT_KEYS = 1024       # keys per split-K workgroup
 HBM_PEAK_GBS = 8000.0
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 
 
-def build_workload(B, dev, lib, torch):
+def build_workload(B, dev, lib, torch, PART):
     """Allocates and fills every buffer of the period; returns the two step
     recorders (even/odd KV copy) and bookkeeping."""
     gen = torch.Generator(device="cuda")
@@ -130,7 +130,14 @@ def build_workload(B, dev, lib, torch):
                   {0: b_part, 1: b_gate, 2: b_attn_table, 3: b_att},
                   {4: PART, 5: max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
 
-    return record, keep
+    def record_split_only(cb, copy):
+        keys, values = kv[copy]
+        cb.encode(P("attention_decode_split_ms"),
+                  {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
+                  {5: CAPACITY, 6: 4096, 7: PART, 8: max_splits, 9: 0}, (max_splits, 2, rows),
+                  (256,))
+
+    return record, record_split_only, keep
 
 
 def cpu_baseline(threads):
@@ -187,6 +194,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--split-keys", type=int, default=DEFAULT_SPLIT_KEYS,
+                    help="keys per split-K workgroup (multiple of 32)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (lanes and heads "
@@ -201,7 +210,8 @@ def main():
     dev = B.Device()
     queue = dev.create_queue()
     lib = dev.create_library()
-    record, keep = build_workload(B, dev, lib, torch)
+    PART = args.split_keys
+    record, record_split_only, keep = build_workload(B, dev, lib, torch, PART)
 
     steps = []
     for copy in range(2):
@@ -240,7 +250,16 @@ def main():
             per_kernel.setdefault(name, []).append(ms)
     # one list entry per launch: average launch duration of each kernel
     kernel_us = {name: round(statistics.mean(v) * 1e3, 2) for name, v in per_kernel.items()}
-    split_us = kernel_us["attention_decode_split_ms"]
+    # the dominant kernel alone, back to back between one pair of events on its
+    # stream, alternating the two KV copies: average launch duration
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    launches = 40
+    for k in range(launches):
+        record_split_only(cb, k & 1)
+    cb.end_compute_pass()
+    cb.commit().wait()
+    split_us = round(cb.commit().wait() * 1e3 / launches, 2)
     algo_bytes = LANES * VISIBLE * ATTN_BYTES_PER_KEY
     achieved = algo_bytes / (split_us * 1e-6) / 1e9
     attn_layer_us = sum(kernel_us[k] for k in ("attn_qk_rope_ms", "attention_decode_split_ms",

@@ -11,7 +11,9 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIBRARY_PATH = os.path.join(_HERE, "lib", "libtatara_hip.so")
+# TATARA_HIP_LIBRARY selects another build of the same C ABI (e.g. a debug build).
+LIBRARY_PATH = os.environ.get("TATARA_HIP_LIBRARY") or os.path.join(_HERE, "lib",
+                                                                    "libtatara_hip.so")
 
 EXPORTED_SYMBOLS = [
     "tt_abi_version", "tt_status_name", "tt_device_create", "tt_device_destroy",

@@ -16,8 +16,9 @@
 // range).  Each wave owns every 4th block of 32 keys and keeps an online
 // softmax state for the 8 query heads of the kv group:
 //   S^T[key][head] = K[key][:] . Q[head][:]   v_mfma_f32_16x16x32_bf16,
-//       A = K tile read from a per-wave LDS stage (rows padded to 528 B so the
-//       16-lane operand reads are conflict-free), B = Q^T held in registers.
+//       A = K tile read from a per-wave LDS stage that HBM fills directly
+//       (global_load_lds, no registers; row pairs padded to 1040 B so the
+//       16-lane operand reads spread over the banks), B = Q^T in registers.
 //       MFMA columns 8..15 repeat heads 0..7.
 //   O^T[dim][head] += V^T[dim][key] P^T[key][head]
 //       A = V^T built in registers: each lane loads 16 B runs of 8 value rows
@@ -40,10 +41,11 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr uint32_t kD = kAttnHeadDim;
 constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
-constexpr uint32_t kLdsRowBytes = 528;      // 512 B key row + 16 B pad
-constexpr uint32_t kWaveLdsBytes = kBlockKeys * kLdsRowBytes;  // 16896
+constexpr uint32_t kLdsPairBytes = 1040;    // key i row | key 16+i row | 16 B pad
+constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16640
 constexpr uint32_t kWaves = 4;
-constexpr uint32_t kMergeHeadFloats = 260;  // padded head stride of the wave merge
+constexpr uint32_t kMergeTileFloats = 20;   // 16 accumulator words of one MFMA + 4 pad
+constexpr uint32_t kMergeHeadFloats = 16 * kMergeTileFloats + 4;  // 324: head stride of the merge
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -165,6 +167,12 @@ struct FlashArgs {
     uint32_t single_partition;  // keys of one reference partition (256)
 };
 
+// value of lane (l ^ 8) within each row of 16 lanes
+__device__ __forceinline__ float dpp_row_ror8(float v) {
+    return __int_as_float(
+        __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));
+}
+
 __device__ __forceinline__ uint32_t pack_low(uint32_t a, uint32_t b) {
     // {a.lo16, b.lo16}
     return __builtin_amdgcn_perm(b, a, 0x05040100u);
@@ -174,7 +182,7 @@ __device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
     return __builtin_amdgcn_perm(b, a, 0x07060302u);
 }
 
-__global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
+__global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t split = blockIdx.x;
     const uint32_t kvh = blockIdx.y;
@@ -220,48 +228,69 @@ __global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
     float l_run = 0.0f;
 
     const uint32_t nblocks = (k1 - k0 + kBlockKeys - 1) / kBlockKeys;
-    for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
+
+    // K rows go from HBM straight into the wave's LDS stage (no registers): one
+    // instruction lands 1 KiB contiguous in LDS, lanes 0..31 fetching key i
+    // (tile 0) and lanes 32..63 key 16+i (tile 1), so the two rows sharing LDS
+    // banks are never read by the same operand load.
+    auto stage_keys = [&](uint32_t blk) {
         const uint32_t key0 = k0 + blk * kBlockKeys;
         const uint32_t valid = min(kBlockKeys, k1 - key0);
-        // K rows: instruction i moves keys 2i, 2i+1 (1 KiB contiguous per wave)
-        u32x4 kreg[16];
 #pragma unroll
         for (uint32_t i = 0; i < 16; ++i) {
-            const uint32_t key = min(2 * i + (lane >> 5), valid - 1);
-            kreg[i] = *reinterpret_cast<const u32x4*>(
-                kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8);
+            const uint32_t key = min(i + (lane >> 5) * 16, valid - 1);
+            const uint16_t* src = kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(src),
+                (__attribute__((address_space(3))) void*)(stage + i * kLdsPairBytes),
+                16, 0, 0);
         }
-        // V rows: contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3)
-        u32x4 vreg[2][8];
+    };
+
+    // V rows: contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3);
+    // one call fetches one 128-dim half (8 x 16 B per lane)
+    auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
+        const uint32_t key0 = k0 + blk * kBlockKeys;
+        const uint32_t valid = min(kBlockKeys, k1 - key0);
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) {
             const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
-            const uint16_t* vrow = vbase + static_cast<uint64_t>(key0 + key) * kD + m * 8;
-            vreg[0][e] = *reinterpret_cast<const u32x4*>(vrow);
-            vreg[1][e] = *reinterpret_cast<const u32x4*>(vrow + 128);
+            vhalf[e] = *reinterpret_cast<const u32x4*>(
+                vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8);
         }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (uint32_t i = 0; i < 16; ++i) {
-            *reinterpret_cast<u32x4*>(stage + (2 * i + (lane >> 5)) * kLdsRowBytes +
-                                      (lane & 31) * 16) = kreg[i];
-        }
+    };
+
+    // Software pipeline per wave: the K transfer of block b+1 starts as soon as
+    // the S^T operand reads of block b are done, and each V half of block b+1 is
+    // requested as soon as the P.V products of block b have consumed that half's
+    // registers, so a wave always has its next block in flight.
+    u32x4 vreg[2][8];
+    if (wave < nblocks) {
+        stage_keys(wave);
+        load_values(vreg[0], wave, 0);
+        load_values(vreg[1], wave, 1);
+    }
+    for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
+        const uint32_t valid = min(kBlockKeys, k1 - (k0 + blk * kBlockKeys));
+        const bool more = blk + kWaves < nblocks;
+        // every transfer issued so far (this block's K and V) has landed
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         __builtin_amdgcn_wave_barrier();
         f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f};
         f32x4 s1 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (uint32_t kb = 0; kb < 8; ++kb) {
             const bf16x8 a0 = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsRowBytes +
+                bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes +
                                                         (kb * 4 + g) * 16));
             const bf16x8 a1 = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u32x4*>(stage + (16 + m) * kLdsRowBytes +
+                bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes + 512 +
                                                         (kb * 4 + g) * 16));
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[kb], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[kb], s1, 0, 0, 0);
         }
-        __builtin_amdgcn_wave_barrier();
-        // scores of keys g*4+i (s0) and 16+g*4+i (s1) for head m&7
+        // scores of keys g*4+i (s0) and 16+g*4+i (s1) for head m&7; reading the
+        // accumulators also retires every LDS operand read of this block
         float sc[8];
         float block_max = -INFINITY;
 #pragma unroll
@@ -270,6 +299,9 @@ __global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
             sc[4 + i] = (16 + g * 4 + i) < valid ? s1[i] * kAttnScale : -INFINITY;
             block_max = fmaxf(block_max, fmaxf(sc[i], sc[4 + i]));
         }
+        __builtin_amdgcn_wave_barrier();
+        // the stage is free again: start the next block's K transfer now
+        if (more) stage_keys(blk + kWaves);
         block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
         block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
         const float m_new = fmaxf(m_run, block_max);
@@ -322,22 +354,29 @@ __global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
                 o[hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                     __builtin_bit_cast(bf16x8, hi), pb, o[hh * 8 + 2 * dw + 1], 0, 0, 0);
             }
+            if (more) load_values(vreg[hh], blk + kWaves, hh);
         }
     }
+    // every transfer into the stage has landed before the stage is reused below
+    __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    // fold the residual columns into the head columns, then stage each wave's
-    // {O[8][256], max, sum} in its own LDS region for the cross-wave merge
+    // Fold the residual columns into the head columns (lanes m and m^8, a DPP
+    // rotate by 8 inside each row of 16 lanes: no LDS traffic), then stage each
+    // wave's {O[8][256], max, sum} in its own LDS region for the cross-wave
+    // merge.  Stage layout per head: word j*20 + g*4 + i for MFMA j, lane group
+    // g, accumulator element i (one 16-byte store per MFMA per lane); head
+    // stride 324 words.  Both the stores and the strided reads of the merge
+    // spread over the banks.
     float* merge = reinterpret_cast<float*>(stage);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j) {
+        f32x4 total;
 #pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            const float total = o[j][i] + __shfl_xor(o[j][i], 8, 64);
-            if (m < 8) {
-                const uint32_t dim = (j >> 3) * 128 + (g * 4 + i) * 8 + (j & 7);
-                merge[m * kMergeHeadFloats + dim] = total;
-            }
+        for (uint32_t i = 0; i < 4; ++i) total[i] = o[j][i] + dpp_row_ror8(o[j][i]);
+        if (m < 8) {
+            *reinterpret_cast<f32x4*>(merge + m * kMergeHeadFloats + j * kMergeTileFloats +
+                                      g * 4) = total;
         }
     }
     if (lane < 8) {
@@ -346,38 +385,54 @@ __global__ __launch_bounds__(256) void flash_decode_kernel(FlashArgs a) {
     }
     __syncthreads();
 
-    const uint32_t t = threadIdx.x;
-    for (uint32_t h = 0; h < kAttnHeadsPerKv; ++h) {
-        float wmax[kWaves];
+    // Cross-wave merge: wave w finishes heads 2w and 2w+1; lane l owns output
+    // dimensions l, l+64, l+128, l+192 (coalesced stores).  Dimension d sits in
+    // the stage at word ((d>>7)*8 + (d&7))*20 + ((d&127)>>3).
+#pragma unroll
+    for (uint32_t hl = 0; hl < 2; ++hl) {
+        const uint32_t h = wave * 2 + hl;
+        float scale[kWaves];
         float gmax = -INFINITY;
+        float lsum[kWaves];
 #pragma unroll
         for (uint32_t w = 0; w < kWaves; ++w) {
             const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
-            wmax[w] = wm[8 * kMergeHeadFloats + h * 2];
-            gmax = fmaxf(gmax, wmax[w]);
+            scale[w] = wm[8 * kMergeHeadFloats + h * 2];
+            lsum[w] = wm[8 * kMergeHeadFloats + h * 2 + 1];
+            gmax = fmaxf(gmax, scale[w]);
         }
-        float acc = 0.0f;
         float denom = 0.0f;
 #pragma unroll
         for (uint32_t w = 0; w < kWaves; ++w) {
-            const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
-            const float scale = wmax[w] == -INFINITY ? 0.0f : __expf(wmax[w] - gmax);
-            acc = fmaf(scale, wm[h * kMergeHeadFloats + t], acc);
-            denom = fmaf(scale, wm[8 * kMergeHeadFloats + h * 2 + 1], denom);
+            scale[w] = scale[w] == -INFINITY ? 0.0f : __expf(scale[w] - gmax);
+            denom = fmaf(scale[w], lsum[w], denom);
         }
         const uint32_t head = kvh * kAttnHeadsPerKv + h;
-        if (a.final_mode) {
-            const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + t;
-            a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
-        } else {
-            float* record = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
-                            (static_cast<uint64_t>(head) * a.record_splits + split) *
-                                kAttnRecordFloats;
-            record[t] = acc;
-            if (t == 0) {
-                record[kD] = gmax;
-                record[kD + 1] = denom;
+        float* record = a.final_mode
+                            ? nullptr
+                            : a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
+                                  (static_cast<uint64_t>(head) * a.record_splits + split) *
+                                      kAttnRecordFloats;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            const uint32_t d = lane + 64 * c;
+            const uint32_t slot = ((d >> 7) * 8 + (d & 7)) * kMergeTileFloats + ((d & 127) >> 3);
+            float acc = 0.0f;
+#pragma unroll
+            for (uint32_t w = 0; w < kWaves; ++w) {
+                const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
+                acc = fmaf(scale[w], wm[h * kMergeHeadFloats + slot], acc);
             }
+            if (a.final_mode) {
+                const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+                a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
+            } else {
+                record[d] = acc;
+            }
+        }
+        if (!a.final_mode && lane == 0) {
+            record[kD] = gmax;
+            record[kD + 1] = denom;
         }
     }
 }
@@ -412,16 +467,52 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
     }
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                         static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
-    float gmax = -INFINITY;
-    for (uint32_t p = 0; p < nparts; ++p) gmax = fmaxf(gmax, base[p * kAttnRecordFloats + kD]);
+    __shared__ float red[256];
+    __shared__ float weight[256];
+    __shared__ float wsum[256];
+    // global maximum: partitions strided over the threads, then a block reduction
+    float local = -INFINITY;
+    for (uint32_t p = d; p < nparts; p += 256) {
+        local = fmaxf(local, base[static_cast<uint64_t>(p) * kAttnRecordFloats + kD]);
+    }
+    red[d] = local;
+    __syncthreads();
+    for (uint32_t off = 128; off; off >>= 1) {
+        if (d < off) red[d] = fmaxf(red[d], red[d + off]);
+        __syncthreads();
+    }
+    const float gmax = red[0];
     float acc = 0.0f;
     float denom = 0.0f;
-    for (uint32_t p = 0; p < nparts; ++p) {
-        const float* rec = base + static_cast<uint64_t>(p) * kAttnRecordFloats;
-        const float pmax = rec[kD];
-        const float w = pmax == -INFINITY ? 0.0f : __expf(pmax - gmax);
-        acc = fmaf(w, rec[d], acc);
-        denom = fmaf(w, rec[kD + 1], denom);
+    for (uint32_t chunk = 0; chunk < nparts; chunk += 256) {
+        const uint32_t count = min(256u, nparts - chunk);
+        __syncthreads();
+        if (d < count) {
+            const float* rec = base + static_cast<uint64_t>(chunk + d) * kAttnRecordFloats;
+            const float pmax = rec[kD];
+            const float w = pmax == -INFINITY ? 0.0f : __expf(pmax - gmax);
+            weight[d] = w;
+            wsum[d] = w * rec[kD + 1];
+        }
+        __syncthreads();
+        const float* rec = base + static_cast<uint64_t>(chunk) * kAttnRecordFloats + d;
+        uint32_t p = 0;
+        for (; p + 8 <= count; p += 8) {
+            float v[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                v[u] = rec[static_cast<uint64_t>(p + u) * kAttnRecordFloats];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                acc = fmaf(weight[p + u], v[u], acc);
+                denom += wsum[p + u];
+            }
+        }
+        for (; p < count; ++p) {
+            acc = fmaf(weight[p], rec[static_cast<uint64_t>(p) * kAttnRecordFloats], acc);
+            denom += wsum[p];
+        }
     }
     const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
     a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
