@@ -930,7 +930,7 @@ int32_t op_attention_values(const Bindings& b, const Grid& g, hipStream_t stream
 }  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
-bool prepare_kernels() {
+bool prepare_decode_kernels() {
     // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
     return hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -1,17 +1,491 @@
-// Block-prefill full attention for gfx950.  Operators registered here, with the
-// reference kernels whose argument tables they accept
-// (src/backend/metal/kernels/prefill_attention.metal): attn_qk_rope_blk (:1).
+// Block-prefill full attention for gfx950: causal flash attention on bf16 MFMA
+// with K/V tiles double-buffered in LDS, plus the exact partial/combine control
+// path.
+//
+// Operators registered here, with the reference kernels whose argument tables
+// they accept (src/backend/metal/kernels/prefill_attention.metal):
+//   attn_qk_rope_blk (:1)
+//   attention_streaming_blk (:860), attention_flash_v2_blk (:1233)  -> flash kernel
+//   attention_partial_blk (:97), attention_combine_blk (:207)        -> control path
+//
+// Flash kernel.  One workgroup = 4 wave64 = 16 consecutive query positions x
+// the 8 query heads of one kv head (128 score rows); wave w owns heads 2w and
+// 2w+1.  Keys are walked in tiles of 32 up to the causal limit of the tile.
+// The four waves share each K/V tile through LDS: HBM/L2 fills the next tile's
+// stage directly (global_load_lds, no registers) while the current one is
+// consumed, two stages of 32.25 KiB each.
+//   S^T[key][pos] = K[key][:] . Q[pos][:]    v_mfma_f32_16x16x32_bf16,
+//       A = K from LDS, B = Q^T held in registers for the whole walk.
+//   O^T[dim][pos] += V^T[dim][key] P^T[key][pos]
+//       A = V^T: each lane reads 16-byte runs of 8 value rows from LDS and
+//       transposes 8x8 in registers (v_perm_b32), shared by both heads of the
+//       wave; B = P^T = bf16 of the S^T accumulators, no LDS round trip.
+// Row r of the dispatch sees keys [0, tile_context + r], which makes every row
+// a decode step at context tile_context + r over the same cache
+// (prefill_attention.metal:117-119).  Algorithmic work: 1024 flop per visible
+// (query, key) pair per head.
 #include "../tt_internal.h"
 
 namespace tt {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr uint32_t kD = kAttnHeadDim;
+constexpr uint32_t kTilePositions = 16;
+constexpr uint32_t kTileKeys = 32;
+constexpr uint32_t kKeyPairBytes = 1040;                 // key i | key 16+i | 16 B pad
+constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16640
+constexpr uint32_t kValueStageBytes = kTileKeys * 512;   // 16384
+constexpr uint32_t kStageBytes = kKeyStageBytes + kValueStageBytes;
+constexpr uint32_t kFlashLdsBytes = 2 * kStageBytes;     // 66048
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+    return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
+    const uint32_t b = __float_as_uint(v);
+    if ((b & 0x7F800000u) == 0x7F800000u) return static_cast<uint16_t>(b >> 16);
+    return static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ uint32_t pack_low(uint32_t a, uint32_t b) {
+    return __builtin_amdgcn_perm(b, a, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
+    return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+
+struct FlashPrefillArgs {
+    const uint16_t* query;   // [rows][16][256]
+    const uint16_t* gate;    // [rows][16][256]
+    const uint16_t* keys;    // [2][capacity][256]
+    const uint16_t* values;
+    uint16_t* out;           // [rows][16][256]
+    uint32_t rows;
+    uint32_t tile_context;   // cache position of row 0
+    uint32_t capacity;
+};
+
+__global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPrefillArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // longest key walks first: the last position tile is dispatched first
+    const uint32_t tile = gridDim.x - 1 - blockIdx.x;
+    const uint32_t kvh = blockIdx.y;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t p0 = tile * kTilePositions;
+    const uint32_t pos = min(p0 + m, a.rows - 1);         // this lane's query row (column n = m)
+    const uint32_t limit = a.tile_context + p0 + m;       // last visible key of that row
+    const uint32_t tile_keys = a.tile_context + min(p0 + kTilePositions, a.rows);  // visible count
+    const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
+
+    // B operand of S^T for the wave's two heads: Q^T, column n = position p0+n
+    bf16x8 q[2][8];
+#pragma unroll
+    for (uint32_t t = 0; t < 2; ++t) {
+        const uint16_t* qrow = a.query + (static_cast<uint64_t>(pos) * kAttnQueryHeads +
+                                          kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
+#pragma unroll
+        for (uint32_t kb = 0; kb < 8; ++kb) {
+            q[t][kb] = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(qrow + kb * 32 + g * 8));
+        }
+    }
+
+    const uint16_t* kbase = a.keys + static_cast<uint64_t>(kvh) * a.capacity * kD;
+    const uint16_t* vbase = a.values + static_cast<uint64_t>(kvh) * a.capacity * kD;
+
+    // each wave moves a quarter of a tile: 4 K transfers (key pairs 4w..4w+3) and
+    // 4 V transfers (rows 8w..8w+7), 1 KiB each
+    auto stage_tile = [&](uint32_t kb, uint32_t stage_index) {
+        uint8_t* kstage = lds + stage_index * kStageBytes;
+        uint8_t* vstage = kstage + kKeyStageBytes;
+        const uint32_t key0 = kb * kTileKeys;
+        const uint32_t last = tile_keys - 1 - key0;  // rows past the walk repeat the last key
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint32_t pair = wave * 4 + i;
+            const uint32_t key = min(pair + (lane >> 5) * 16, last);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(
+                    kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8),
+                (__attribute__((address_space(3))) void*)(kstage + pair * kKeyPairBytes), 16, 0, 0);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint32_t row2 = wave * 4 + i;  // rows 2*row2, 2*row2+1
+            const uint32_t key = min(row2 * 2 + (lane >> 5), last);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(
+                    vbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8),
+                (__attribute__((address_space(3))) void*)(vstage + row2 * 1024), 16, 0, 0);
+        }
+    };
+
+    f32x4 o[2][16];
+#pragma unroll
+    for (uint32_t t = 0; t < 2; ++t) {
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) o[t][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    float m_run[2] = {-INFINITY, -INFINITY};  // in units of log2
+    float l_run[2] = {0.0f, 0.0f};
+    const float scale = kAttnScale * kLog2e;
+
+    stage_tile(0, 0);
+    for (uint32_t kb = 0; kb < nkb; ++kb) {
+        const bool more = kb + 1 < nkb;
+        if (more) {
+            stage_tile(kb + 1, (kb + 1) & 1);
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // all but the 8 transfers just issued
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();  // every wave's quarter of tile kb has landed
+        const uint8_t* kstage = lds + (kb & 1) * kStageBytes;
+        const uint8_t* vstage = kstage + kKeyStageBytes;
+        const uint32_t key0 = kb * kTileKeys;
+
+        f32x4 s[2][2];  // [key tile][head]
+#pragma unroll
+        for (uint32_t kt = 0; kt < 2; ++kt) {
+            s[kt][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            s[kt][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (uint32_t kk = 0; kk < 8; ++kk) {
+#pragma unroll
+            for (uint32_t kt = 0; kt < 2; ++kt) {
+                const bf16x8 ka = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(kstage + m * kKeyPairBytes + kt * 512 +
+                                                            (kk * 4 + g) * 16));
+                s[kt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[0][kk], s[kt][0], 0, 0, 0);
+                s[kt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[1][kk], s[kt][1], 0, 0, 0);
+            }
+        }
+        // lane holds keys key0 + kt*16 + g*4 + i of column (position) m
+        const bool needs_mask = key0 + kTileKeys - 1 > a.tile_context + p0;
+        bf16x8 pb[2];
+        bool rescale = false;
+        float alpha[2];
+#pragma unroll
+        for (uint32_t t = 0; t < 2; ++t) {
+            float sc[8];
+            float block_max = -INFINITY;
+#pragma unroll
+            for (uint32_t kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    float v = s[kt][t][i] * scale;
+                    if (needs_mask && key0 + kt * 16 + g * 4 + i > limit) v = -INFINITY;
+                    sc[kt * 4 + i] = v;
+                    block_max = fmaxf(block_max, v);
+                }
+            }
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
+            const float m_new = fmaxf(m_run[t], block_max);
+            // a row with no visible key yet keeps max = -inf; exp2(-inf - -inf) is avoided
+            const float base = m_new == -INFINITY ? 0.0f : m_new;
+            alpha[t] = __builtin_amdgcn_exp2f(m_run[t] - base);
+            float block_sum = 0.0f;
+            uint32_t pw[4];
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                const float x0 = __builtin_amdgcn_exp2f(sc[2 * c] - base);
+                const float x1 = __builtin_amdgcn_exp2f(sc[2 * c + 1] - base);
+                block_sum += x0 + x1;
+                pw[c] = static_cast<uint32_t>(f32_to_bf16_bits(x0)) |
+                        (static_cast<uint32_t>(f32_to_bf16_bits(x1)) << 16);
+            }
+            block_sum += __shfl_xor(block_sum, 16, 64);
+            block_sum += __shfl_xor(block_sum, 32, 64);
+            l_run[t] = l_run[t] * alpha[t] + block_sum;
+            m_run[t] = m_new;
+            pb[t] = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+            rescale = rescale || alpha[t] != 1.0f;
+        }
+        if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+#pragma unroll
+            for (uint32_t t = 0; t < 2; ++t) {
+#pragma unroll
+                for (uint32_t j = 0; j < 16; ++j) o[t][j] *= alpha[t];
+            }
+        }
+        // O^T += V^T P^T; contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3);
+        // MFMA j covers dims (j>>3)*128 + row*8 + (j&7)
+#pragma unroll
+        for (uint32_t hh = 0; hh < 2; ++hh) {
+            u32x4 v[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                const uint32_t key = (e >> 2) * 16 + g * 4 + (e & 3);
+                v[e] = *reinterpret_cast<const u32x4*>(vstage + key * 512 + hh * 256 + m * 16);
+            }
+#pragma unroll
+            for (uint32_t dw = 0; dw < 4; ++dw) {
+                u32x4 lo, hi;
+                lo.x = pack_low(v[0][dw], v[1][dw]);
+                lo.y = pack_low(v[2][dw], v[3][dw]);
+                lo.z = pack_low(v[4][dw], v[5][dw]);
+                lo.w = pack_low(v[6][dw], v[7][dw]);
+                hi.x = pack_high(v[0][dw], v[1][dw]);
+                hi.y = pack_high(v[2][dw], v[3][dw]);
+                hi.z = pack_high(v[4][dw], v[5][dw]);
+                hi.w = pack_high(v[6][dw], v[7][dw]);
+                const bf16x8 va = __builtin_bit_cast(bf16x8, lo);
+                const bf16x8 vb = __builtin_bit_cast(bf16x8, hi);
+#pragma unroll
+                for (uint32_t t = 0; t < 2; ++t) {
+                    o[t][hh * 8 + 2 * dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        va, pb[t], o[t][hh * 8 + 2 * dw], 0, 0, 0);
+                    o[t][hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        vb, pb[t], o[t][hh * 8 + 2 * dw + 1], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();  // stage kb&1 may be refilled by the next iteration's transfers
+    }
+
+    // out[(row*16 + head)*256 + dim] = bf16((O/l) * sigmoid(gate)); lane holds, for
+    // position m, dims (j>>3)*128 + (g*4+i)*8 + (j&7)
+    if (p0 + m < a.rows) {
+#pragma unroll
+        for (uint32_t t = 0; t < 2; ++t) {
+            const uint64_t row_base = (static_cast<uint64_t>(p0 + m) * kAttnQueryHeads +
+                                       kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
+            const float inv = 1.0f / l_run[t];
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    const uint32_t dim = (j >> 3) * 128 + (g * 4 + i) * 8 + (j & 7);
+                    const float gate = bf16_bits_to_f32(a.gate[row_base + dim]);
+                    const float sig = 1.0f / (1.0f + __expf(-gate));
+                    a.out[row_base + dim] = f32_to_bf16_bits((o[t][j][i] * inv) * sig);
+                }
+            }
+        }
+    }
+}
+
+// --------------------------------------------------- exact control path ------
+
+// attention_partial_blk: grid (16, partitions, tile_rows) x 256; one record
+// {numerator[256], max, sum} per (head, row, partition of 256 keys) with the
+// causal limit visible = context + row + 1 (prefill_attention.metal:97-205).
+// Scalar and simple on purpose: this is the reference the fast kernels are
+// judged against, not a fast path.
+__global__ __launch_bounds__(256) void attention_partial_blk_kernel(
+    const uint16_t* query, const uint16_t* keys, const uint16_t* values, uint32_t context,
+    uint32_t capacity, uint32_t partition, float* partials, uint32_t partition_count,
+    uint32_t block) {
+    __shared__ float scores[256];
+    __shared__ float red[256];
+    __shared__ float qs[kD];
+    const uint32_t head = blockIdx.x;
+    const uint32_t part = blockIdx.y;
+    const uint32_t row = blockIdx.z;
+    const uint32_t t = threadIdx.x;
+    const uint32_t visible = context + row + 1;
+    const uint32_t start = part * partition;
+    const uint32_t end = min(visible, start + partition);
+    const uint32_t kv = head / kAttnHeadsPerKv;
+    qs[t] = bf16_bits_to_f32(query[(static_cast<uint64_t>(row) * kAttnQueryHeads + head) * kD + t]);
+    float running = -INFINITY;
+    float denom = 0.0f;
+    float acc = 0.0f;
+    __syncthreads();
+    for (uint32_t tile = start; tile < end; tile += 256) {
+        const uint32_t count = min(end - tile, 256u);
+        float s = -INFINITY;
+        if (t < count) {
+            const uint16_t* k = keys + (static_cast<uint64_t>(kv) * capacity + tile + t) * kD;
+            float dot = 0.0f;
+            for (uint32_t d = 0; d < kD; ++d) dot = fmaf(qs[d], bf16_bits_to_f32(k[d]), dot);
+            s = dot * kAttnScale;
+        }
+        red[t] = s;
+        __syncthreads();
+        for (uint32_t off = 128; off; off >>= 1) {
+            if (t < off) red[t] = fmaxf(red[t], red[t + off]);
+            __syncthreads();
+        }
+        const float next = fmaxf(running, red[0]);
+        const float rescale = running == -INFINITY ? 0.0f : expf(running - next);
+        __syncthreads();
+        const float p = t < count ? expf(s - next) : 0.0f;
+        scores[t] = p;
+        red[t] = p;
+        __syncthreads();
+        for (uint32_t off = 128; off; off >>= 1) {
+            if (t < off) red[t] += red[t + off];
+            __syncthreads();
+        }
+        acc *= rescale;
+        const uint16_t* v = values + (static_cast<uint64_t>(kv) * capacity + tile) * kD + t;
+        for (uint32_t p2 = 0; p2 < count; ++p2) {
+            acc = fmaf(scores[p2], bf16_bits_to_f32(v[static_cast<uint64_t>(p2) * kD]), acc);
+        }
+        denom = denom * rescale + red[0];
+        running = next;
+        __syncthreads();
+    }
+    float* dst = partials + ((static_cast<uint64_t>(head) * block + row) * partition_count + part) *
+                                kAttnRecordFloats;
+    dst[t] = acc;
+    if (t == 0) {
+        dst[kD] = running;
+        dst[kD + 1] = denom;
+    }
+}
+
+// attention_combine_blk: grid (16, tile_rows) x 256 (prefill_attention.metal:207-254);
+// an all-masked partition (max = -inf) carries weight zero.
+__global__ __launch_bounds__(256) void attention_combine_blk_kernel(const float* partials,
+                                                                    const uint16_t* gate,
+                                                                    uint32_t partition_count,
+                                                                    uint16_t* out, uint32_t block) {
+    const uint32_t head = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t d = threadIdx.x;
+    const float* base = partials + (static_cast<uint64_t>(head) * block + row) * partition_count *
+                                       kAttnRecordFloats;
+    float gmax = -INFINITY;
+    for (uint32_t p = 0; p < partition_count; ++p) {
+        gmax = fmaxf(gmax, base[static_cast<uint64_t>(p) * kAttnRecordFloats + kD]);
+    }
+    float acc = 0.0f;
+    float denom = 0.0f;
+    for (uint32_t p = 0; p < partition_count; ++p) {
+        const float* rec = base + static_cast<uint64_t>(p) * kAttnRecordFloats;
+        const float w = rec[kD] == -INFINITY ? 0.0f : expf(rec[kD] - gmax);
+        acc = fmaf(w, rec[d], acc);
+        denom = fmaf(w, rec[kD + 1], denom);
+    }
+    const uint64_t at = (static_cast<uint64_t>(row) * kAttnQueryHeads + head) * kD + d;
+    const float g = bf16_bits_to_f32(gate[at]);
+    out[at] = f32_to_bf16_bits((acc / denom) * (1.0f / (1.0f + expf(-g))));
+}
+
+// ---------------------------------------------------------------- launchers --
+
+uint64_t cache_bytes(uint32_t capacity) {
+    return static_cast<uint64_t>(kAttnKvHeads) * capacity * kD * 2;
+}
+
+// attention_streaming_blk / attention_flash_v2_blk: b0 query(+tile), b1 keys,
+// b2 values, b3 gate(+tile), b4 attended(+tile), c5 visible, c6 capacity,
+// c7 tile_rows, c8 tile_context; grid (16, ceil(tile_rows/16)) x 256
+// (prefill_step.cpp:1657-1717).  tile_rows is not limited to the reference's
+// 256-row query tile: one dispatch may cover a whole block.
+int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                               bool validate_only) {
+    Args a(b);
+    FlashPrefillArgs f{};
+    const uint32_t visible = a.constant(5);
+    f.capacity = a.constant(6);
+    f.rows = a.constant(7);
+    f.tile_context = a.constant(8);
+    a.require(f.rows >= 1 && f.rows <= (1u << 24), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    const uint32_t tiles = (f.rows + kTilePositions - 1) / kTilePositions;
+    a.require(g.gx == 16 && g.gy == tiles && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(f.capacity != 0 &&
+                  static_cast<uint64_t>(f.tile_context) + f.rows == visible &&
+                  visible <= f.capacity,
+              TT_CMD_CONTEXT_OUT_OF_RANGE);
+    const uint64_t row_bytes = static_cast<uint64_t>(f.rows) * kAttnQueryValues * 2;
+    f.query = a.buffer<const uint16_t>(0, row_bytes);
+    f.keys = a.buffer<const uint16_t>(1, cache_bytes(f.capacity));
+    f.values = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
+    f.gate = a.buffer<const uint16_t>(3, row_bytes);
+    f.out = a.buffer<uint16_t>(4, row_bytes);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_flash_prefill_kernel, dim3(tiles, kAttnKvHeads), dim3(256),
+                       kFlashLdsBytes, stream, f);
+    return TT_OK;
+}
+
+// attention_partial_blk: b0 query(+tile), b1 keys, b2 values, c3 tile_context,
+// c4 capacity, c5 partition=256, b6 partials[16][tile_rows][parts][258],
+// c7 partitions, c8 tile_rows; grid (16, partitions, tile_rows) x 256
+// (prefill_step.cpp:1782-1800).
+int32_t op_attention_partial_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                                 bool validate_only) {
+    Args a(b);
+    const uint32_t context = a.constant(3);
+    const uint32_t capacity = a.constant(4);
+    const uint32_t partition = a.constant(5);
+    const uint32_t partitions = a.constant(7);
+    const uint32_t rows = a.constant(8);
+    a.require(rows >= 1 && rows <= 65535 && partitions >= 1 && partitions <= 65535 &&
+                  partition >= 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(g.gx == 16 && g.gy == partitions && g.gz == rows && g.tx == 256 && g.ty == 1 &&
+                  g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(capacity != 0 && static_cast<uint64_t>(context) + rows <= capacity,
+              TT_CMD_CONTEXT_OUT_OF_RANGE);
+    const uint16_t* query =
+        a.buffer<const uint16_t>(0, static_cast<uint64_t>(rows) * kAttnQueryValues * 2);
+    const uint16_t* keys = a.buffer<const uint16_t>(1, cache_bytes(capacity));
+    const uint16_t* values = a.buffer<const uint16_t>(2, cache_bytes(capacity));
+    float* partials = a.buffer<float>(
+        6, static_cast<uint64_t>(kAttnQueryHeads) * rows * partitions * kAttnRecordFloats * 4);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_partial_blk_kernel, dim3(16, partitions, rows), dim3(256), 0,
+                       stream, query, keys, values, context, capacity, partition, partials,
+                       partitions, rows);
+    return TT_OK;
+}
+
+// attention_combine_blk: b0 partials, b1 gate(+tile), c2 partitions,
+// b3 attended(+tile), c4 tile_rows; grid (16, tile_rows) x 256
+// (prefill_step.cpp:1802-1817).
+int32_t op_attention_combine_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                                 bool validate_only) {
+    Args a(b);
+    const uint32_t partitions = a.constant(2);
+    const uint32_t rows = a.constant(4);
+    a.require(rows >= 1 && rows <= 65535 && partitions >= 1, TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(g.gx == 16 && g.gy == rows && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    const float* partials = a.buffer<const float>(
+        0, static_cast<uint64_t>(kAttnQueryHeads) * rows * partitions * kAttnRecordFloats * 4);
+    const uint64_t row_bytes = static_cast<uint64_t>(rows) * kAttnQueryValues * 2;
+    const uint16_t* gate = a.buffer<const uint16_t>(1, row_bytes);
+    uint16_t* out = a.buffer<uint16_t>(3, row_bytes);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_combine_blk_kernel, dim3(16, rows), dim3(256), 0, stream, partials,
+                       gate, partitions, out, rows);
+    return TT_OK;
+}
+
+}  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
+bool prepare_prefill_kernels() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kFlashLdsBytes) == hipSuccess;
+}
+
 const KernelDesc kAttentionPrefillKernels[] = {
     {"attn_qk_rope_blk", op_attn_qk_rope_blk},
+    {"attention_streaming_blk", op_attention_flash_blk},
+    {"attention_flash_v2_blk", op_attention_flash_blk},
+    {"attention_partial_blk", op_attention_partial_blk},
+    {"attention_combine_blk", op_attention_combine_blk},
 };
 const uint32_t kAttentionPrefillKernelCount =
     sizeof(kAttentionPrefillKernels) / sizeof(kAttentionPrefillKernels[0]);
-
 #endif
 
 }  // namespace tt

@@ -410,7 +410,7 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
     tt_library* library = new (std::nothrow) tt_library;
     if (library == nullptr) return TT_PIPE_LIBRARY_COMPILATION_FAILED;
     library->device = device;
-    if (!tt::prepare_kernels()) {
+    if (!tt::prepare_decode_kernels() || !tt::prepare_prefill_kernels()) {
         delete library;
         return TT_PIPE_LIBRARY_COMPILATION_FAILED;
     }

@@ -89,7 +89,8 @@ int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream
 
 // One-time kernel attribute set-up (large dynamic LDS opt-in); called when a
 // library is created, so it never runs inside a stream capture.
-bool prepare_kernels();
+bool prepare_decode_kernels();
+bool prepare_prefill_kernels();
 
 extern const KernelDesc kAttentionDecodeKernels[];
 extern const uint32_t kAttentionDecodeKernelCount;

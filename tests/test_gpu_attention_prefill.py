@@ -1,0 +1,120 @@
+"""Block-prefill full attention on the GPU against the CPU checker (exact
+partial/combine semantics, row r sees keys [0, context + r]).  Tolerance of the
+path: max-abs <= 2e-2, mean-abs <= 2e-3; cache rows written by the rope stage are
+compared at the decode tests' bar."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_util import check_bf16, gpu, run
+
+pytestmark = pytest.mark.gpu
+o = ol.oracle
+
+
+def _weights():
+    q_w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x5157, 256))
+    k_w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x4B57, 256))
+    return q_w, k_w
+
+
+def _prefill_case(rows, base, cap, seed, select=None, control=False):
+    """Runs rope + flash prefill on the GPU for `rows` new tokens after `base`
+    cached ones and compares the selected rows with the checker."""
+    B, dev, queue, lib = gpu()
+    q_w, k_w = _weights()
+    proj = ol.gaussian_bf16(seed, rows * 9216)
+    keys = np.zeros(2 * cap * 256, np.uint16); values = np.zeros_like(keys)
+    if base:
+        keys.reshape(2, cap, 256)[:, :base] = ol.gaussian_bf16(seed + 1, 2 * base * 256).reshape(
+            2, base, 256)
+        values.reshape(2, cap, 256)[:, :base] = ol.gaussian_bf16(seed + 2, 2 * base * 256).reshape(
+            2, base, 256)
+    b_k, b_v = dev.buffer_from(keys), dev.buffer_from(values)
+    sel = np.arange(rows, dtype=np.uint32) if select is None else np.asarray(select, np.uint32)
+    query = np.zeros(rows * 4096, np.uint16); gate = np.zeros_like(query)
+    want = np.zeros_like(query)
+    o.tto_attention_prefill(proj, q_w, k_w, rows, base, cap, query, gate, keys, values, sel,
+                            len(sel), want, 8)
+    b_p = dev.buffer_from(proj)
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g, b_o = (dev.create_buffer(rows * 8192) for _ in range(3))
+    tiles = (rows + 15) // 16
+
+    def rec(cb):
+        cb.encode(lib.pipeline("attn_qk_rope_blk"),
+                  {0: b_p, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: b_k, 6: b_v}, {7: base, 8: cap},
+                  (18, rows), (256,))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_flash_v2_blk"),
+                  {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: b_o},
+                  {5: base + rows, 6: cap, 7: rows, 8: base}, (16, tiles), (256,))
+    ms = run(rec)
+    got = b_o.read(np.uint16).reshape(rows, 4096)
+    w = want.reshape(rows, 4096)
+    check_bf16(got[sel], w[sel], f"flash prefill rows {rows} base {base}")
+    # cache: raw V exact, roped K at the decode bar, rows beyond untouched
+    gk = b_k.read(np.uint16).reshape(2, cap, 256)
+    gv = b_v.read(np.uint16).reshape(2, cap, 256)
+    assert np.array_equal(gv, values.reshape(2, cap, 256))
+    check_bf16(gk, keys, "prefill K cache", max_abs=4e-2, mean_abs=1e-4)
+    assert np.array_equal(b_g.read(np.uint16), gate)
+    if control:
+        parts = (base + rows + 255) // 256
+        b_part = dev.create_buffer(16 * rows * parts * 258 * 4)
+        b_o2 = dev.create_buffer(rows * 8192)
+
+        def rec2(cb):
+            cb.encode(lib.pipeline("attention_partial_blk"), {0: b_q, 1: b_k, 2: b_v, 6: b_part},
+                      {3: base, 4: cap, 5: 256, 7: parts, 8: rows}, (16, parts, rows), (256,))
+            cb.barrier()
+            cb.encode(lib.pipeline("attention_combine_blk"), {0: b_part, 1: b_g, 3: b_o2},
+                      {2: parts, 4: rows}, (16, rows), (256,))
+        run(rec2)
+        got2 = b_o2.read(np.uint16).reshape(rows, 4096)
+        check_bf16(got2[sel], w[sel], f"partial/combine control rows {rows} base {base}")
+        # fast vs control, the reference's own band (normalised error <= 0.02,
+        # attention_fixture_probe.cpp:1241-1269)
+        a, c = ol.bf16_to_f32(got.reshape(-1)), ol.bf16_to_f32(got2.reshape(-1))
+        assert np.abs(a - c).max() / max(np.abs(c).max(), 1e-6) <= 0.02
+    return ms, dict(b_q=b_q, b_g=b_g, b_k=b_k, b_v=b_v, got=got, cap=cap, base=base)
+
+
+def test_block_13_rows_at_context_300():
+    """The reference probe's block: 13 rows at context 300 -> 313 visible, capacity 512."""
+    print("[case] prefill 13 rows at context 300", flush=True)
+    _prefill_case(13, 300, 512, 0xB10C, control=True)
+
+
+@pytest.mark.parametrize("rows,base", [(1, 0), (16, 0), (17, 0), (48, 0), (100, 1000), (256, 31),
+                                       (300, 33)])
+def test_block_shapes(rows, base):
+    print(f"[case] prefill rows {rows} base {base}", flush=True)
+    _prefill_case(rows, base, 2048, 0x5EED + rows, control=rows <= 48)
+
+
+def test_prefill_row_equals_decode_step_on_gpu():
+    """Row r of a block at context c is the decode operator at context c + r over
+    the same cache (prefill_attention.metal:117-119)."""
+    print("[case] prefill rows vs decode operator", flush=True)
+    B, dev, queue, lib = gpu()
+    rows, base, cap = 40, 500, 1024
+    _, c = _prefill_case(rows, base, cap, 0xD3C0)
+    for r in (0, 15, 16, 39):
+        b_o = dev.create_buffer(8192)
+        run(lambda cb: cb.encode(lib.pipeline("attention_decode"),
+                                 {0: (c["b_q"], r * 8192), 1: (c["b_g"], r * 8192), 2: c["b_k"],
+                                  3: c["b_v"], 5: b_o}, {4: base + r, 6: cap}, (16,), (256,)))
+        check_bf16(b_o.read(np.uint16), c["got"][r], f"decode vs prefill row {r}",
+                   max_abs=8e-3, mean_abs=2e-4)
+
+
+def test_config4_prefill_16384_rows():
+    """Config 4: 16384 new tokens into an empty capacity-16384 cache.  The checker
+    computes a strided subset of query rows (every 256th plus the first and last
+    16); the K/V cache written by the rope stage is compared in full."""
+    print("[case] config 4: prefill 16384 rows", flush=True)
+    rows = 16384
+    sel = sorted(set(list(range(16)) + list(range(0, rows, 256)) + list(range(rows - 16, rows))))
+    ms, _ = _prefill_case(rows, 0, rows, 0xC0F4, select=sel)
+    print(f"[time] rope + flash prefill 16384 rows (first run): {ms:.3f} ms", flush=True)
