@@ -1,0 +1,1085 @@
+#include "runtime.h"
+
+#include <algorithm>
+#include <cstring>
+#include <limits>
+
+namespace tatara::model::qwen36 {
+
+std::vector<LayerKind> make_hybrid_layer_schedule(std::size_t layer_count, std::size_t period,
+                                                  std::size_t first) {
+    std::vector<LayerKind> layers(layer_count, LayerKind::GatedDelta);
+    if (period == 0) return layers;
+    for (std::size_t index = first; index < layer_count; index += period) {
+        layers[index] = LayerKind::FullAttention;
+    }
+    return layers;
+}
+
+ModelPlan qwen36_35b_a3b_plan() {
+    return ModelPlan{
+        .hidden = 2048,
+        .vocabulary = 248320,
+        .query_heads = 16,
+        .key_value_heads = 2,
+        .head_dimension = 256,
+        .recurrent_heads = 32,
+        .state_dimension = 128,
+        .initial_serving_capacity = 16384,
+        .layers = make_hybrid_layer_schedule(40, 4, 3),
+    };
+}
+
+}  // namespace tatara::model::qwen36
+
+namespace tatara::runtime {
+
+using namespace backend::hip;
+
+namespace {
+
+bool is_gated(LayerKind kind) { return kind == LayerKind::GatedDelta; }
+
+// Row counts shared by byte sizes and dispatch shapes (decode_geometry.h:188-203).
+struct FamilyRows {
+    std::uint32_t gdn_qk, gdn_values, gdn_conv, gdn_prepare, gdn_projection, attn_projection,
+        attn_query;
+};
+FamilyRows family_rows(const model::qwen36::ModelPlan& plan) {
+    FamilyRows r{};
+    r.gdn_qk = 2u * (plan.recurrent_heads / 2u) * plan.state_dimension;
+    r.gdn_values = plan.recurrent_heads * plan.state_dimension;
+    r.gdn_conv = r.gdn_qk + r.gdn_values;
+    r.gdn_prepare = r.gdn_conv + r.gdn_values;
+    r.gdn_projection = r.gdn_prepare + 2u * plan.recurrent_heads;
+    r.attn_projection = plan.query_heads * 2u * plan.head_dimension +
+                        2u * plan.key_value_heads * plan.head_dimension;
+    r.attn_query = plan.query_heads * plan.head_dimension;
+    return r;
+}
+
+bool allocate_zeroed(const HipDevice& device, std::uint64_t bytes, HipBuffer& out) {
+    // create_shared_buffer zero-fills the HBM allocation (zeroed-allocation rule,
+    // decode_step.h:252-255), so no host memset is needed here.
+    auto made = create_shared_buffer(device, bytes);
+    if (!made) return false;
+    out = std::move(*made.buffer);
+    return true;
+}
+
+// Issues calls in order and latches the first error: once one is held every
+// later call is skipped, so a rejected bind can never be followed by a recorded
+// dispatch (decode_step.cpp:95-184).
+struct Walk {
+    HipComputePass& pass;
+    HipCommandError error = HipCommandError::None;
+
+    bool failed() const { return error != HipCommandError::None; }
+    void check(HipCommandError result) {
+        if (error == HipCommandError::None && result != HipCommandError::None) error = result;
+    }
+    void pipeline(const HipComputePipeline& p) {
+        if (!failed()) check(set_compute_pipeline(pass, p));
+    }
+    void buffer(const HipBuffer& b, std::uint64_t offset, std::uint32_t index) {
+        if (!failed()) check(set_buffer(pass, b, offset, index));
+    }
+    void weight(const HipBuffer* b, std::uint32_t index) {
+        if (failed()) return;
+        if (b == nullptr) {
+            check(HipCommandError::InvalidBuffer);
+            return;
+        }
+        check(set_buffer(pass, *b, 0, index));
+    }
+    void constant(std::uint32_t value, std::uint32_t index) {
+        if (!failed()) check(set_bytes(pass, &value, sizeof(value), index));
+    }
+    void dispatch(HipSize groups, HipSize threads) {
+        if (!failed()) check(dispatch_threadgroups(pass, groups, threads));
+    }
+    void dispatch(std::uint64_t gx, std::uint64_t tx, std::uint64_t gy = 1, std::uint64_t ty = 1,
+                  std::uint64_t tz = 1) {
+        dispatch(HipSize{gx, gy, 1}, HipSize{tx, ty, tz});
+    }
+    void barrier() {
+        if (!failed()) check(memory_barrier(pass));
+    }
+    void hook(HipCommandError (*fn)(void*, HipComputePass&, std::size_t, LayerKind, std::uint32_t),
+              void* user, std::size_t layer, LayerKind kind, std::uint32_t rows) {
+        if (failed() || fn == nullptr) return;
+        check(fn(user, pass, layer, kind, rows));
+    }
+};
+
+HipCommandError stream_admissible(const DecodeStep& step, const DecodeStateSlot& state,
+                                  std::uint32_t context) {
+    if (!decode_state_slot_compatible(step, state)) return HipCommandError::StateSlotMismatch;
+    if (!context_in_capacity(context, step.capacity)) return HipCommandError::ContextOutOfRange;
+    if (!decode_state_slot_ready(step, state)) return HipCommandError::StateSlotMismatch;
+    return HipCommandError::None;
+}
+
+template <typename Pipelines, typename Member>
+bool resolve(const HipLibrary& library, Pipelines& out, Member member, const char* name,
+             HipPipelineError& error) {
+    auto made = create_compute_pipeline(library, name);
+    if (!made) {
+        error = made.error;
+        return false;
+    }
+    out.*member = std::move(*made.pipeline);
+    return true;
+}
+
+}  // namespace
+
+DecodeGeometry make_decode_geometry(const model::qwen36::ModelPlan& plan, std::uint32_t capacity) {
+    const FamilyRows rows = family_rows(plan);
+    std::uint32_t gated = 0;
+    std::uint32_t attention = 0;
+    for (const LayerKind kind : plan.layers) (is_gated(kind) ? gated : attention) += 1;
+    const std::uint32_t partitions = (capacity + kAttentionPartition - 1u) / kAttentionPartition;
+    DecodeGeometry g{};
+    g.gated_delta_layers = gated;
+    g.attention_layers = attention;
+    g.hidden_bytes = std::uint64_t{plan.hidden} * kBf16Bytes;
+    g.layer_stream_bytes = plan.layers.size() * std::uint64_t{plan.hidden} * kBf16Bytes;
+    g.gdn_projection_bytes = std::uint64_t{rows.gdn_projection} * kBf16Bytes;
+    g.gdn_qk_bytes = std::uint64_t{rows.gdn_qk} * kBf16Bytes;
+    g.gdn_value_bytes = std::uint64_t{rows.gdn_values} * kBf16Bytes;
+    g.gdn_gate_bytes = g.gdn_value_bytes;
+    g.gdn_conv_state_bytes = std::uint64_t{kConvShiftSteps} * rows.gdn_conv * kBf16Bytes;
+    g.gdn_recurrent_state_bytes = std::uint64_t{plan.recurrent_heads} * plan.state_dimension *
+                                  plan.state_dimension * kF32Bytes;
+    g.attn_projection_bytes = std::uint64_t{rows.attn_projection} * kBf16Bytes;
+    g.attn_query_bytes = std::uint64_t{rows.attn_query} * kBf16Bytes;
+    g.attn_record_scratch_bytes =
+        std::uint64_t{plan.query_heads} * partitions * kAttentionRecordFloats * kF32Bytes;
+    g.attn_cache_bytes =
+        std::uint64_t{plan.key_value_heads} * capacity * plan.head_dimension * kBf16Bytes;
+    g.gdn_prepare = {rows.gdn_prepare / plan.state_dimension, plan.state_dimension};
+    g.gdn_recurrence = {plan.state_dimension / 4u, plan.recurrent_heads, 32u, 4u};
+    g.gdn_gate_norm = {plan.recurrent_heads, plan.state_dimension};
+    g.attn_qk_rope = {plan.query_heads + plan.key_value_heads, plan.head_dimension};
+    g.attention_head = {plan.query_heads, plan.head_dimension};
+    g.attention_split = {plan.query_heads / 4u,
+                         kAttentionPartition,
+                         4u,
+                         plan.key_value_heads,
+                         32u,
+                         plan.head_dimension / 64u,
+                         plan.query_heads / plan.key_value_heads};
+    g.rms = {1u, plan.hidden / 4u};
+    return g;
+}
+
+std::uint32_t attention_partitions(std::uint32_t context) {
+    const std::uint32_t count = context + 1;
+    return count <= kAttentionPartition ? 1u
+                                        : (count + kAttentionPartition - 1) / kAttentionPartition;
+}
+
+DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
+    DecodePipelines p;
+    HipPipelineError error = HipPipelineError::None;
+    using P = DecodePipelines;
+    const bool ok =
+        resolve(library, p, &P::gdn_prepare, "gdn_prepare", error) &&
+        resolve(library, p, &P::gdn_recurrence, "gdn_recurrence", error) &&
+        resolve(library, p, &P::gdn_gate_norm, "gdn_gate_norm", error) &&
+        resolve(library, p, &P::attn_qk_rope, "attn_qk_rope", error) &&
+        resolve(library, p, &P::attention_decode, "attention_decode", error) &&
+        resolve(library, p, &P::attention_scores_values_fused,
+                "attention_decode_scores_values_gqa8", error) &&
+        resolve(library, p, &P::attention_combine, "attention_decode_combine", error) &&
+        resolve(library, p, &P::gdn_prepare_ms, "gdn_prepare_ms", error) &&
+        resolve(library, p, &P::gdn_recurrence_ms, "gdn_recurrence_ms", error) &&
+        resolve(library, p, &P::gate_norm_ms, "gdn_gate_norm_ms", error) &&
+        resolve(library, p, &P::attn_qk_rope_ms, "attn_qk_rope_ms", error) &&
+        resolve(library, p, &P::attention_decode_ms, "attention_decode_ms", error) &&
+        resolve(library, p, &P::attention_split_ms, "attention_decode_split_ms", error) &&
+        resolve(library, p, &P::attention_combine_ms, "attention_decode_combine_ms", error);
+    if (!ok) return {error, std::nullopt};
+    return {HipPipelineError::None, std::move(p)};
+}
+
+namespace {
+
+DecodeStateSlotResult allocate_state_slot(const HipDevice& device, const DecodeGeometry& geometry,
+                                          std::uint32_t capacity,
+                                          std::span<const LayerKind> schedule,
+                                          const LayerKind* schedule_identity) {
+    if (!device) return {DecodeStepError::InvalidDevice, std::nullopt};
+    if (capacity == 0 || schedule.empty() || schedule_identity == nullptr) {
+        return {DecodeStepError::OffsetCountMismatch, std::nullopt};
+    }
+    DecodeStateSlot slot;
+    slot.capacity = capacity;
+    slot.schedule_identity = schedule_identity;
+    slot.layers.reserve(schedule.size());
+    for (const LayerKind kind : schedule) {
+        DecodeLayerState state;
+        const bool gated = is_gated(kind);
+        const std::uint64_t first = gated ? geometry.gdn_conv_state_bytes : geometry.attn_cache_bytes;
+        const std::uint64_t second =
+            gated ? geometry.gdn_recurrent_state_bytes : geometry.attn_cache_bytes;
+        if (!allocate_zeroed(device, first, state.first) ||
+            !allocate_zeroed(device, second, state.second) ||
+            (gated && (!allocate_zeroed(device, first, state.first_out) ||
+                       !allocate_zeroed(device, second, state.second_out)))) {
+            return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+        }
+        slot.layers.push_back(std::move(state));
+    }
+    return {DecodeStepError::None, std::move(slot)};
+}
+
+}  // namespace
+
+DecodeStepResult create_decode_step(const HipDevice& device, const DecodeGeometry& geometry,
+                                    std::uint32_t capacity, std::span<const LayerKind> schedule,
+                                    DecodePipelines pipelines) {
+    if (!device) return {DecodeStepError::InvalidDevice, std::nullopt};
+    if (schedule.empty() || capacity == 0) return {DecodeStepError::OffsetCountMismatch, std::nullopt};
+    DecodeStep step;
+    step.geometry = geometry;
+    step.capacity = capacity;
+    step.schedule.assign(schedule.begin(), schedule.end());
+    step.pipelines = std::move(pipelines);
+    auto state = allocate_state_slot(device, geometry, capacity, step.schedule, step.schedule.data());
+    if (!state) return {state.error, std::nullopt};
+    step.state = std::move(*state.slot);
+    return {DecodeStepError::None, std::move(step)};
+}
+
+DecodeStateSlotResult create_decode_state_slot(const HipDevice& device, const DecodeStep& step) {
+    return allocate_state_slot(device, step.geometry, step.capacity, step.schedule,
+                               step.schedule.data());
+}
+
+DecodeStateSlotPoolResult create_decode_state_slot_pool(const HipDevice& device,
+                                                        const DecodeStep& step,
+                                                        std::uint32_t count) {
+    DecodeStateSlotPoolResult result{DecodeStepError::None, std::nullopt, {}};
+    if (!device) {
+        result.error = DecodeStepError::InvalidDevice;
+        return result;
+    }
+    if (count == 0 || step.capacity == 0 || step.schedule.empty()) {
+        result.error = DecodeStepError::OffsetCountMismatch;
+        return result;
+    }
+    DecodeStatePool pool;
+    pool.stripes = count;
+    result.slots.resize(count);
+    for (DecodeStateSlot& slot : result.slots) {
+        slot.capacity = step.capacity;
+        slot.schedule_identity = step.schedule.data();
+        slot.layers.reserve(step.schedule.size());
+    }
+    const auto fail = [&result]() {
+        result.error = DecodeStepError::BufferAllocationFailed;
+        result.slots.clear();
+        return std::move(result);
+    };
+    for (const LayerKind kind : step.schedule) {
+        const bool gated = is_gated(kind);
+        const std::uint64_t first_bytes =
+            gated ? step.geometry.gdn_conv_state_bytes : step.geometry.attn_cache_bytes;
+        const std::uint64_t second_bytes =
+            gated ? step.geometry.gdn_recurrent_state_bytes : step.geometry.attn_cache_bytes;
+        const std::uint32_t stripes = gated ? 2u * count : count;
+        DecodeStatePoolLayer layer;
+        auto first = create_striped_pool_buffer(device, first_bytes, stripes);
+        auto second = create_striped_pool_buffer(device, second_bytes, stripes);
+        // offsets in the state table are u32 element counts (decode_step.cpp:476)
+        if (!first || !second || first.buffer->size_bytes() > 0xffffffffull * 2 ||
+            second.buffer->size_bytes() > 0xffffffffull * 2) {
+            return fail();
+        }
+        layer.first = std::move(*first.buffer);
+        layer.second = std::move(*second.buffer);
+        layer.first_stride = first.stripe_stride_bytes;
+        layer.second_stride = second.stripe_stride_bytes;
+        for (std::uint32_t slot = 0; slot < count; ++slot) {
+            DecodeLayerState state;
+            const std::uint64_t base = gated ? std::uint64_t{slot} * 2 : std::uint64_t{slot};
+            auto w0 = create_buffer_window(layer.first, base * layer.first_stride, first_bytes);
+            auto w1 = create_buffer_window(layer.second, base * layer.second_stride, second_bytes);
+            if (!w0 || !w1) return fail();
+            state.first = std::move(*w0.buffer);
+            state.second = std::move(*w1.buffer);
+            if (gated) {
+                auto o0 =
+                    create_buffer_window(layer.first, (base + 1) * layer.first_stride, first_bytes);
+                auto o1 = create_buffer_window(layer.second, (base + 1) * layer.second_stride,
+                                               second_bytes);
+                if (!o0 || !o1) return fail();
+                state.first_out = std::move(*o0.buffer);
+                state.second_out = std::move(*o1.buffer);
+            }
+            result.slots[slot].layers.push_back(std::move(state));
+        }
+        pool.layers.push_back(std::move(layer));
+    }
+    result.pool = std::move(pool);
+    return result;
+}
+
+DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
+                                                     const DecodeStep& step, std::uint32_t rows) {
+    if (rows == 0 || rows > kMaximumBatchRows) {
+        return {DecodeStepError::OffsetCountMismatch, std::nullopt};
+    }
+    const DecodeGeometry& g = step.geometry;
+    DecodeBatchScratch b;
+    b.rows = rows;
+    const std::uint64_t table_bytes = step.schedule.size() * 16 * 4 * 4 + 64;
+    // split records: capacity / 32 partitions is the finest split the kernels take
+    const std::uint64_t record_bytes = std::uint64_t{rows} * g.attn_record_scratch_bytes;
+    if (!allocate_zeroed(device, rows * g.gdn_projection_bytes, b.gdn_projection) ||
+        !allocate_zeroed(device, rows * g.gdn_qk_bytes, b.gdn_qk) ||
+        !allocate_zeroed(device, rows * g.gdn_value_bytes, b.gdn_value) ||
+        !allocate_zeroed(device, rows * g.gdn_gate_bytes, b.gdn_z) ||
+        !allocate_zeroed(device, rows * g.gdn_value_bytes, b.gdn_y) ||
+        !allocate_zeroed(device, rows * g.gdn_value_bytes, b.gdn_gated) ||
+        !allocate_zeroed(device, rows * g.attn_projection_bytes, b.attn_projection) ||
+        !allocate_zeroed(device, rows * g.attn_query_bytes, b.attn_query) ||
+        !allocate_zeroed(device, rows * g.attn_query_bytes, b.attn_gate) ||
+        !allocate_zeroed(device, rows * g.attn_query_bytes, b.attn_attended) ||
+        !allocate_zeroed(device, record_bytes, b.attn_partials) ||
+        !allocate_zeroed(device, table_bytes, b.state_offsets)) {
+        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+    }
+    return {DecodeStepError::None, std::move(b)};
+}
+
+bool decode_state_slot_compatible(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
+    return step.capacity != 0 && state.capacity == step.capacity &&
+           state.schedule_identity == step.schedule.data() &&
+           state.layers.size() == step.schedule.size();
+}
+
+bool decode_state_slot_complete(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
+    if (!decode_state_slot_compatible(step, state)) return false;
+    const auto enough = [](const HipBuffer& buffer, std::uint64_t bytes) {
+        return buffer && buffer.size_bytes() >= bytes;
+    };
+    const DecodeGeometry& g = step.geometry;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        const DecodeLayerState& s = state.layers[layer];
+        if (is_gated(step.schedule[layer])) {
+            if (!enough(s.first, g.gdn_conv_state_bytes) ||
+                !enough(s.first_out, g.gdn_conv_state_bytes) ||
+                !enough(s.second, g.gdn_recurrent_state_bytes) ||
+                !enough(s.second_out, g.gdn_recurrent_state_bytes)) {
+                return false;
+            }
+        } else if (!enough(s.first, g.attn_cache_bytes) || !enough(s.second, g.attn_cache_bytes)) {
+            return false;
+        }
+    }
+    return true;
+}
+
+bool decode_state_slot_available(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
+    return decode_state_slot_compatible(step, state) &&
+           state.status == DecodeStateSlotStatus::Ready && state.active_transfer_generation == 0 &&
+           state.active_reset_generation == 0 && state.active_reset_segments == 0 &&
+           state.active_reset_bytes == 0;
+}
+
+bool decode_state_slot_ready(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
+    return decode_state_slot_available(step, state) && decode_state_slot_complete(step, state);
+}
+
+HipCommandError build_state_offset_table(const DecodeStep& step,
+                                         std::span<const DecodeStream> streams,
+                                         const DecodeStatePool& pool, StateOffsetTable& out) {
+    const std::size_t layers = step.schedule.size();
+    const std::uint32_t rows = static_cast<std::uint32_t>(streams.size());
+    if (rows == 0 || rows > kMaximumBatchRows || pool.layers.size() != layers ||
+        pool.stripes == 0) {
+        return HipCommandError::InvalidStreamGroup;
+    }
+    out.words.assign(layers * 64 + 16, 0u);
+    for (std::size_t layer = 0; layer < layers; ++layer) {
+        const DecodeStatePoolLayer& pool_layer = pool.layers[layer];
+        const bool gated = is_gated(step.schedule[layer]);
+        for (std::uint32_t r = 0; r < rows; ++r) {
+            if (streams[r].state == nullptr || streams[r].stripe >= pool.stripes ||
+                streams[r].state->layers.size() != layers) {
+                return HipCommandError::InvalidStreamGroup;
+            }
+            const std::uint32_t stripe = streams[r].stripe;
+            std::uint32_t* entry = out.words.data() + layer * 64 + std::size_t{r} * 4;
+            if (gated) {
+                const auto conv_elems = static_cast<std::uint32_t>(pool_layer.first_stride / 2);
+                const auto rec_elems = static_cast<std::uint32_t>(pool_layer.second_stride / 4);
+                const std::uint32_t parity = streams[r].state->layers[layer].swapped ? 1u : 0u;
+                entry[0] = (2u * stripe + parity) * conv_elems;
+                entry[1] = (2u * stripe + 1u - parity) * conv_elems;
+                entry[2] = (2u * stripe + parity) * rec_elems;
+                entry[3] = (2u * stripe + 1u - parity) * rec_elems;
+            } else {
+                entry[0] = stripe * static_cast<std::uint32_t>(pool_layer.first_stride / 2);
+                entry[1] = streams[r].context;
+            }
+        }
+    }
+    out.bucket_rows = 0;
+    for (std::uint32_t r = 0; r < rows; ++r) {
+        if (attention_partitions(streams[r].context) == 1) {
+            out.words[layers * 64 + out.bucket_rows] = r;
+            ++out.bucket_rows;
+        }
+    }
+    return HipCommandError::None;
+}
+
+HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStream> streams,
+                                   const DecodeStatePool& pool, DecodeBatchScratch& batch,
+                                   std::span<const LayerWeights> weights,
+                                   const LayerStageHooks& hooks, HipComputePass& pass) {
+    const std::uint32_t rows = static_cast<std::uint32_t>(streams.size());
+    if (rows == 0 || rows > batch.rows || rows > kMaximumBatchRows ||
+        pool.layers.size() != step.schedule.size() || pool.stripes == 0 || !batch.state_offsets ||
+        weights.size() != step.schedule.size() || batch.split_keys == 0 ||
+        batch.split_keys % 32u != 0) {
+        return HipCommandError::InvalidStreamGroup;
+    }
+    for (std::size_t index = 0; index < streams.size(); ++index) {
+        if (streams[index].state == nullptr || streams[index].stripe >= pool.stripes) {
+            return HipCommandError::InvalidStreamGroup;
+        }
+        const HipCommandError admissible =
+            stream_admissible(step, *streams[index].state, streams[index].context);
+        if (admissible != HipCommandError::None) return admissible;
+        for (std::size_t other = 0; other < index; ++other) {
+            if (streams[other].state == streams[index].state) {
+                return HipCommandError::InvalidStreamGroup;
+            }
+        }
+    }
+    StateOffsetTable table;
+    const HipCommandError built = build_state_offset_table(step, streams, pool, table);
+    if (built != HipCommandError::None) return built;
+    void* host = batch.state_offsets.contents();
+    const std::uint64_t table_bytes = table.words.size() * sizeof(std::uint32_t);
+    if (host == nullptr || batch.state_offsets.size_bytes() < table_bytes) {
+        return HipCommandError::InvalidBuffer;
+    }
+    std::memcpy(host, table.words.data(), table_bytes);
+    const HipCommandError published = did_modify_range(batch.state_offsets, 0, table_bytes);
+    if (published != HipCommandError::None) return published;
+
+    const DecodeGeometry& g = step.geometry;
+    const std::uint64_t bucket_offset = step.schedule.size() * 256;
+    bool any_long = false;
+    for (const DecodeStream& s : streams) any_long |= attention_partitions(s.context) != 1;
+    const std::uint32_t max_splits = (step.capacity + batch.split_keys - 1) / batch.split_keys;
+    if (any_long && batch.attn_partials.size_bytes() <
+                        std::uint64_t{rows} * 16 * max_splits * kAttentionRecordFloats * kF32Bytes) {
+        return HipCommandError::InvalidBuffer;
+    }
+    Walk walk{pass};
+    const DecodePipelines& k = step.pipelines;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        const LayerKind kind = step.schedule[layer];
+        const LayerWeights& w = weights[layer];
+        walk.barrier();
+        walk.hook(hooks.project, hooks.user, layer, kind, rows);
+        walk.barrier();
+        if (is_gated(kind)) {
+            walk.pipeline(k.gdn_prepare_ms);
+            walk.buffer(batch.gdn_projection, 0, 0);
+            walk.buffer(pool.layers[layer].first, 0, 1);
+            walk.weight(w.conv_weight, 2);
+            walk.buffer(batch.gdn_qk, 0, 3);
+            walk.buffer(batch.gdn_value, 0, 4);
+            walk.buffer(batch.gdn_z, 0, 5);
+            walk.buffer(batch.state_offsets, layer * 256, 6);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_projection_bytes / 2), 7);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_qk_bytes / 2), 8);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 9);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_gate_bytes / 2), 10);
+            walk.dispatch(g.gdn_prepare.groups, g.gdn_prepare.threads, rows);
+            walk.barrier();
+            walk.pipeline(k.gdn_recurrence_ms);
+            walk.buffer(batch.gdn_qk, 0, 0);
+            walk.buffer(batch.gdn_value, 0, 1);
+            walk.buffer(batch.gdn_projection, 0, 2);
+            walk.weight(w.a_log, 3);
+            walk.weight(w.dt_bias, 4);
+            walk.buffer(pool.layers[layer].second, 0, 5);
+            walk.buffer(batch.gdn_y, 0, 6);
+            walk.buffer(batch.state_offsets, layer * 256, 7);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_qk_bytes / 2), 8);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 9);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_projection_bytes / 2), 10);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 11);
+            walk.constant(g.gdn_recurrence.head_groups, 12);
+            walk.dispatch(HipSize{1, g.gdn_recurrence.dimension_groups,
+                                  std::uint64_t{g.gdn_recurrence.head_groups} * rows},
+                          HipSize{g.gdn_recurrence.lane_threads,
+                                  g.gdn_recurrence.dimension_threads, 1});
+            walk.barrier();
+            walk.pipeline(k.gate_norm_ms);
+            walk.buffer(batch.gdn_y, 0, 0);
+            walk.buffer(batch.gdn_z, 0, 1);
+            walk.weight(w.norm_weight, 2);
+            walk.buffer(batch.gdn_gated, 0, 3);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 4);
+            walk.dispatch(g.gdn_gate_norm.groups, g.gdn_gate_norm.threads, rows);
+        } else {
+            walk.pipeline(k.attn_qk_rope_ms);
+            walk.buffer(batch.attn_projection, 0, 0);
+            walk.weight(w.query_norm, 1);
+            walk.weight(w.key_norm, 2);
+            walk.buffer(batch.attn_query, 0, 3);
+            walk.buffer(batch.attn_gate, 0, 4);
+            walk.buffer(pool.layers[layer].first, 0, 5);
+            walk.buffer(pool.layers[layer].second, 0, 6);
+            walk.constant(step.capacity, 7);
+            walk.buffer(batch.state_offsets, layer * 256, 8);
+            walk.constant(static_cast<std::uint32_t>(g.attn_projection_bytes / 2), 9);
+            walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 10);
+            walk.dispatch(g.attn_qk_rope.groups, g.attn_qk_rope.threads, rows);
+            walk.barrier();
+            if (any_long) {
+                // every long row of the batch in one split-K grid + one combine
+                walk.pipeline(k.attention_split_ms);
+                walk.buffer(batch.attn_query, 0, 0);
+                walk.buffer(pool.layers[layer].first, 0, 1);
+                walk.buffer(pool.layers[layer].second, 0, 2);
+                walk.buffer(batch.state_offsets, layer * 256, 3);
+                walk.buffer(batch.attn_partials, 0, 4);
+                walk.constant(step.capacity, 5);
+                walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
+                walk.constant(batch.split_keys, 7);
+                walk.constant(max_splits, 8);
+                walk.constant(1u, 9);
+                walk.dispatch(HipSize{max_splits, 2, rows}, HipSize{256, 1, 1});
+                walk.barrier();
+                walk.pipeline(k.attention_combine_ms);
+                walk.buffer(batch.attn_partials, 0, 0);
+                walk.buffer(batch.attn_gate, 0, 1);
+                walk.buffer(batch.state_offsets, layer * 256, 2);
+                walk.buffer(batch.attn_attended, 0, 3);
+                walk.constant(batch.split_keys, 4);
+                walk.constant(max_splits, 5);
+                walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
+                walk.constant(1u, 7);
+                walk.dispatch(g.attention_head.groups, g.attention_head.threads, rows);
+            }
+            if (table.bucket_rows != 0) {
+                walk.pipeline(k.attention_decode_ms);
+                walk.buffer(batch.attn_query, 0, 0);
+                walk.buffer(batch.attn_gate, 0, 1);
+                walk.buffer(pool.layers[layer].first, 0, 2);
+                walk.buffer(pool.layers[layer].second, 0, 3);
+                walk.buffer(batch.state_offsets, layer * 256, 4);
+                walk.buffer(batch.attn_attended, 0, 5);
+                walk.constant(step.capacity, 6);
+                walk.buffer(batch.state_offsets, bucket_offset, 7);
+                walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 8);
+                walk.dispatch(g.attention_head.groups, g.attention_head.threads, table.bucket_rows);
+            }
+        }
+        walk.barrier();
+        walk.hook(hooks.finish, hooks.user, layer, kind, rows);
+    }
+    return walk.error;
+}
+
+HipCommandError encode_token(DecodeStep& step, DecodeStateSlot& state, DecodeBatchScratch& scratch,
+                             std::span<const LayerWeights> weights, const LayerStageHooks& hooks,
+                             HipComputePass& pass, std::uint32_t context) {
+    const HipCommandError admissible = stream_admissible(step, state, context);
+    if (admissible != HipCommandError::None) return admissible;
+    if (weights.size() != step.schedule.size() || scratch.rows == 0) {
+        return HipCommandError::InvalidStreamGroup;
+    }
+    const DecodeGeometry& g = step.geometry;
+    const DecodePipelines& k = step.pipelines;
+    Walk walk{pass};
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        const LayerKind kind = step.schedule[layer];
+        const LayerWeights& w = weights[layer];
+        DecodeLayerState& s = state.layers[layer];
+        walk.barrier();
+        walk.hook(hooks.project, hooks.user, layer, kind, 1);
+        walk.barrier();
+        if (is_gated(kind)) {
+            const HipBuffer& conv_in = s.swapped ? s.first_out : s.first;
+            const HipBuffer& conv_out = s.swapped ? s.first : s.first_out;
+            const HipBuffer& rec_in = s.swapped ? s.second_out : s.second;
+            const HipBuffer& rec_out = s.swapped ? s.second : s.second_out;
+            walk.pipeline(k.gdn_prepare);
+            walk.buffer(scratch.gdn_projection, 0, 0);
+            walk.buffer(conv_in, 0, 1);
+            walk.weight(w.conv_weight, 2);
+            walk.buffer(scratch.gdn_qk, 0, 3);
+            walk.buffer(scratch.gdn_value, 0, 4);
+            walk.buffer(scratch.gdn_z, 0, 5);
+            walk.buffer(conv_out, 0, 6);
+            walk.dispatch(g.gdn_prepare.groups, g.gdn_prepare.threads);
+            walk.barrier();
+            walk.pipeline(k.gdn_recurrence);
+            walk.buffer(scratch.gdn_qk, 0, 0);
+            walk.buffer(scratch.gdn_value, 0, 1);
+            walk.buffer(scratch.gdn_projection, 0, 2);
+            walk.weight(w.a_log, 3);
+            walk.weight(w.dt_bias, 4);
+            walk.buffer(rec_in, 0, 5);
+            walk.buffer(scratch.gdn_y, 0, 6);
+            walk.buffer(rec_out, 0, 7);
+            walk.dispatch(HipSize{1, g.gdn_recurrence.dimension_groups, g.gdn_recurrence.head_groups},
+                          HipSize{g.gdn_recurrence.lane_threads, g.gdn_recurrence.dimension_threads,
+                                  1});
+            walk.barrier();
+            walk.pipeline(k.gdn_gate_norm);
+            walk.buffer(scratch.gdn_y, 0, 0);
+            walk.buffer(scratch.gdn_z, 0, 1);
+            walk.weight(w.norm_weight, 2);
+            walk.buffer(scratch.gdn_gated, 0, 3);
+            walk.dispatch(g.gdn_gate_norm.groups, g.gdn_gate_norm.threads);
+        } else {
+            walk.pipeline(k.attn_qk_rope);
+            walk.buffer(scratch.attn_projection, 0, 0);
+            walk.weight(w.query_norm, 1);
+            walk.weight(w.key_norm, 2);
+            walk.buffer(scratch.attn_query, 0, 3);
+            walk.buffer(scratch.attn_gate, 0, 4);
+            walk.buffer(s.first, 0, 5);
+            walk.buffer(s.second, 0, 6);
+            walk.constant(context, 7);
+            walk.constant(step.capacity, 8);
+            walk.dispatch(g.attn_qk_rope.groups, g.attn_qk_rope.threads);
+            walk.barrier();
+            const std::uint32_t partitions = attention_partitions(context);
+            if (partitions == 1) {
+                walk.pipeline(k.attention_decode);
+                walk.buffer(scratch.attn_query, 0, 0);
+                walk.buffer(scratch.attn_gate, 0, 1);
+                walk.buffer(s.first, 0, 2);
+                walk.buffer(s.second, 0, 3);
+                walk.constant(context, 4);
+                walk.buffer(scratch.attn_attended, 0, 5);
+                walk.constant(step.capacity, 6);
+                walk.dispatch(g.attention_head.groups, g.attention_head.threads);
+            } else {
+                walk.pipeline(k.attention_scores_values_fused);
+                walk.buffer(scratch.attn_query, 0, 0);
+                walk.buffer(s.first, 0, 1);
+                walk.buffer(s.second, 0, 2);
+                walk.constant(context, 3);
+                walk.constant(step.capacity, 4);
+                walk.constant(kAttentionPartition, 5);
+                walk.buffer(scratch.attn_partials, 0, 6);
+                walk.constant(partitions, 7);
+                walk.dispatch(g.attention_split.value_groups, g.attention_split.score_threads,
+                              partitions, g.attention_split.score_cohort_threads);
+                walk.barrier();
+                walk.pipeline(k.attention_combine);
+                walk.buffer(scratch.attn_partials, 0, 0);
+                walk.buffer(scratch.attn_gate, 0, 1);
+                walk.constant(partitions, 2);
+                walk.buffer(scratch.attn_attended, 0, 3);
+                walk.dispatch(g.attention_head.groups, g.attention_head.threads);
+            }
+        }
+        walk.barrier();
+        walk.hook(hooks.finish, hooks.user, layer, kind, 1);
+    }
+    return walk.error;
+}
+
+void advance_decode_state(const DecodeStep& step, DecodeStateSlot& state) {
+    if (!decode_state_slot_available(step, state)) return;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (is_gated(step.schedule[layer])) {
+            state.layers[layer].swapped = !state.layers[layer].swapped;
+        }
+    }
+}
+
+void advance_decode_state(DecodeStep& step) { advance_decode_state(step, step.state); }
+
+void advance_prefill_state(const DecodeStep& step, DecodeStateSlot& state, std::uint32_t chunks) {
+    if (!decode_state_slot_available(step, state)) return;
+    if ((chunks & 1u) == 0u) return;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (is_gated(step.schedule[layer])) {
+            state.layers[layer].swapped = !state.layers[layer].swapped;
+        }
+    }
+}
+
+StateSlotResetResult encode_state_slot_reset(const DecodeStep& step, DecodeStateSlot& state,
+                                             HipBlitPass& blit_pass) noexcept {
+    const auto failure = [](StateSlotResetError error,
+                            HipCommandError command = HipCommandError::None) {
+        return StateSlotResetResult{error, command, 0, 0, std::nullopt};
+    };
+    if (state.status == DecodeStateSlotStatus::Poisoned) {
+        return failure(StateSlotResetError::PoisonedStateSlot);
+    }
+    if (!decode_state_slot_compatible(step, state) || !decode_state_slot_complete(step, state)) {
+        return failure(StateSlotResetError::InvalidStateSlot);
+    }
+    if (!decode_state_slot_ready(step, state)) return failure(StateSlotResetError::StateSlotNotReady);
+    if (state.next_reset_generation == 0) return failure(StateSlotResetError::GenerationExhausted);
+    if (!blit_pass) {
+        return failure(StateSlotResetError::CommandEncodingFailed, HipCommandError::InvalidBlitPass);
+    }
+    std::uint32_t segments = 0;
+    std::uint64_t bytes = 0;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (!is_gated(step.schedule[layer])) continue;
+        DecodeLayerState& s = state.layers[layer];
+        // only the two live-capable planes that hold carried state need zeroing
+        // at the canonical phase: first/second (state_slot_reset.cpp:265-286)
+        HipBuffer* planes[2] = {&s.first, &s.second};
+        const std::uint64_t lengths[2] = {step.geometry.gdn_conv_state_bytes,
+                                          step.geometry.gdn_recurrent_state_bytes};
+        for (int p = 0; p < 2; ++p) {
+            const HipCommandError command =
+                fill_buffer(blit_pass, *planes[p], 0, lengths[p], std::byte{0});
+            if (command != HipCommandError::None) {
+                state.status = DecodeStateSlotStatus::Poisoned;
+                state.active_reset_generation = 0;
+                state.active_reset_segments = 0;
+                state.active_reset_bytes = 0;
+                return failure(StateSlotResetError::CommandEncodingFailed, command);
+            }
+            ++segments;
+            bytes += lengths[p];
+        }
+    }
+    const std::uint64_t generation = state.next_reset_generation;
+    state.next_reset_generation =
+        generation == std::numeric_limits<std::uint64_t>::max() ? 0 : generation + 1u;
+    state.active_reset_generation = generation;
+    state.active_reset_segments = segments;
+    state.active_reset_bytes = bytes;
+    state.status = DecodeStateSlotStatus::ResetPending;
+    return StateSlotResetResult{
+        StateSlotResetError::None, HipCommandError::None, segments, bytes,
+        StateSlotResetTicket{&step, &state, segments, bytes, generation, true}};
+}
+
+StateSlotResetError complete_state_slot_reset(StateSlotResetTicket& ticket, const DecodeStep& step,
+                                              DecodeStateSlot& state) noexcept {
+    if (!ticket.pending) return StateSlotResetError::AlreadyCompleted;
+    if (state.status == DecodeStateSlotStatus::Poisoned) return StateSlotResetError::PoisonedStateSlot;
+    if (ticket.owner != &step || ticket.state_owner != &state ||
+        state.status != DecodeStateSlotStatus::ResetPending ||
+        ticket.generation != state.active_reset_generation ||
+        ticket.segment_count != state.active_reset_segments ||
+        ticket.state_bytes != state.active_reset_bytes) {
+        return StateSlotResetError::StaleTicket;
+    }
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (is_gated(step.schedule[layer])) state.layers[layer].swapped = false;
+    }
+    state.active_reset_generation = 0;
+    state.active_reset_segments = 0;
+    state.active_reset_bytes = 0;
+    state.status = DecodeStateSlotStatus::Ready;
+    ticket.pending = false;
+    return StateSlotResetError::None;
+}
+
+// ------------------------------------------------------------ block prefill --
+
+namespace {
+PrefillRequestValidation validate_common(const PrefillPolicy& policy, std::uint32_t live_context,
+                                         std::uint32_t context_base,
+                                         std::span<const std::uint32_t> tokens,
+                                         std::uint32_t vocabulary, bool bounded_block) noexcept {
+    if (tokens.empty()) return {PrefillRequestError::EmptyPrefix, 0};
+    if (bounded_block && tokens.size() > policy.maximum_block_rows) {
+        return {PrefillRequestError::BlockOutOfRange, 0};
+    }
+    if (context_base != live_context || context_base > policy.context_capacity) {
+        return {PrefillRequestError::ContextOutOfRange, 0};
+    }
+    if (tokens.size() > policy.context_capacity - context_base) {
+        return {PrefillRequestError::ContextOverflow, 0};
+    }
+    for (const std::uint32_t token : tokens) {
+        if (token >= vocabulary) return {PrefillRequestError::TokenOutOfRange, 0};
+    }
+    return {PrefillRequestError::None, context_base + static_cast<std::uint32_t>(tokens.size())};
+}
+
+bool mul(std::uint64_t a, std::uint64_t b, std::uint64_t& out) {
+    if (a != 0 && b > std::numeric_limits<std::uint64_t>::max() / a) return false;
+    out = a * b;
+    return true;
+}
+}  // namespace
+
+PrefillRequestValidation validate_prefill_request(const PrefillPolicy& policy,
+                                                  std::uint32_t live_context,
+                                                  std::uint32_t context_base,
+                                                  std::span<const std::uint32_t> tokens,
+                                                  std::uint32_t vocabulary) noexcept {
+    return validate_common(policy, live_context, context_base, tokens, vocabulary, true);
+}
+
+PrefillRequestValidation validate_prefill_prefix(const PrefillPolicy& policy,
+                                                 std::uint32_t live_context,
+                                                 std::uint32_t context_base,
+                                                 std::span<const std::uint32_t> tokens,
+                                                 std::uint32_t vocabulary) noexcept {
+    return validate_common(policy, live_context, context_base, tokens, vocabulary, false);
+}
+
+PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan,
+                                            const PrefillPolicy& policy) {
+    if (plan.layers.empty() || plan.hidden == 0 || plan.vocabulary == 0 || plan.query_heads == 0 ||
+        plan.key_value_heads == 0 || plan.query_heads % plan.key_value_heads != 0 ||
+        plan.query_heads / plan.key_value_heads != 8 || plan.head_dimension != kAttentionPartition ||
+        plan.recurrent_heads == 0 || plan.recurrent_heads % 2 != 0 || plan.state_dimension != 128) {
+        return {PrefillGeometryError::InvalidPlan, {}};
+    }
+    if ((policy.schedule != PrefillSchedule::ChunkMajor &&
+         policy.schedule != PrefillSchedule::LayerMajor) ||
+        policy.context_capacity == 0 || policy.context_capacity > kPrefillMaximumContext ||
+        policy.maximum_block_rows == 0 || policy.maximum_block_rows > kPrefillMaximumBlockRows ||
+        policy.first_chunk_rows == 0 || policy.first_chunk_rows > policy.maximum_block_rows ||
+        policy.query_tile_rows == 0 || policy.query_tile_rows > policy.maximum_block_rows ||
+        policy.query_tile_rows % kPrefillQueryTileMultiple != 0 ||
+        policy.attention_partition != kAttentionPartition) {
+        return {PrefillGeometryError::InvalidPolicy, {}};
+    }
+    PrefillGeometry g;
+    g.policy = policy;
+    for (const LayerKind kind : plan.layers) {
+        (is_gated(kind) ? g.gated_delta_layers : g.attention_layers) += 1;
+    }
+    if (g.gated_delta_layers == 0 || g.attention_layers == 0) {
+        return {PrefillGeometryError::InvalidPlan, {}};
+    }
+    const FamilyRows rows = family_rows(plan);
+    const std::uint64_t block = policy.maximum_block_rows;
+    const std::uint64_t capacity = policy.context_capacity;
+    g.attention_partitions =
+        (policy.context_capacity + policy.attention_partition - 1u) / policy.attention_partition;
+    g.gdn_projection_rows = rows.gdn_projection;
+    g.gdn_qk_values = rows.gdn_qk;
+    g.gdn_value_values = rows.gdn_values;
+    g.attention_projection_rows = rows.attn_projection;
+    g.attention_vector_values = rows.attn_query;
+    g.gdn_projection_bytes = block * rows.gdn_projection * kBf16Bytes;
+    g.gdn_qk_bytes = block * rows.gdn_qk * kBf16Bytes;
+    g.gdn_value_bytes = block * rows.gdn_values * kBf16Bytes;
+    g.gdn_parameter_bytes = policy.gdn_gate_hoist ? block * plan.recurrent_heads * kF32Bytes : 0;
+    g.attention_projection_bytes = block * rows.attn_projection * kBf16Bytes;
+    g.attention_vector_bytes = block * rows.attn_query * kBf16Bytes;
+    std::uint64_t records = 0;
+    if (!mul(std::uint64_t{plan.query_heads} * policy.query_tile_rows, g.attention_partitions,
+             records) ||
+        !mul(records, (plan.head_dimension + 2u) * std::uint64_t{kF32Bytes},
+             g.attention_partial_bytes)) {
+        return {PrefillGeometryError::Overflow, {}};
+    }
+    const std::uint64_t conv = std::uint64_t{kConvShiftSteps} * rows.gdn_conv * kBf16Bytes;
+    const std::uint64_t recurrent = std::uint64_t{plan.recurrent_heads} * plan.state_dimension *
+                                    plan.state_dimension * kF32Bytes;
+    const std::uint64_t cache_plane =
+        std::uint64_t{plan.key_value_heads} * capacity * plan.head_dimension * kBf16Bytes;
+    g.gdn_live_state_bytes_per_layer = conv + recurrent;
+    g.gdn_slot_state_bytes_per_layer = 2u * g.gdn_live_state_bytes_per_layer;
+    g.attention_state_bytes_per_position_per_layer =
+        2ull * plan.key_value_heads * plan.head_dimension * kBf16Bytes;
+    g.attention_slot_state_bytes_per_layer = 2u * cache_plane;
+    g.slot_state_bytes = g.gated_delta_layers * g.gdn_slot_state_bytes_per_layer +
+                         g.attention_layers * g.attention_slot_state_bytes_per_layer;
+    return {PrefillGeometryError::None, g};
+}
+
+PrefixStateSnapshotGeometry make_prefix_state_snapshot_geometry(const PrefillGeometry& geometry,
+                                                                std::uint32_t positions) noexcept {
+    PrefixStateSnapshotGeometry s;
+    if (geometry.policy.context_capacity == 0 || geometry.gated_delta_layers == 0 ||
+        geometry.attention_layers == 0 || positions == 0 ||
+        positions > geometry.policy.context_capacity) {
+        return s;
+    }
+    s.valid = true;
+    s.positions = positions;
+    s.gated_delta_bytes = geometry.gated_delta_layers * geometry.gdn_live_state_bytes_per_layer;
+    s.attention_bytes = std::uint64_t{geometry.attention_layers} * positions *
+                        geometry.attention_state_bytes_per_position_per_layer;
+    s.total_bytes = s.gated_delta_bytes + s.attention_bytes;
+    return s;
+}
+
+namespace {
+std::uint32_t first_rows(const PrefillPolicy& policy, std::uint32_t context_base) {
+    return policy.schedule == PrefillSchedule::LayerMajor && context_base == 0
+               ? policy.first_chunk_rows
+               : policy.maximum_block_rows;
+}
+}  // namespace
+
+std::uint32_t prefill_chunk_count(const PrefillPolicy& policy, std::uint32_t context_base,
+                                  std::uint32_t rows) {
+    const std::uint32_t first = first_rows(policy, context_base);
+    if (rows <= first) return 1;
+    return 1u + (rows - first + policy.maximum_block_rows - 1u) / policy.maximum_block_rows;
+}
+
+PrefillChunk prefill_chunk_at(const PrefillPolicy& policy, std::uint32_t context_base,
+                              std::uint32_t total_rows, std::uint32_t ordinal) {
+    const std::uint32_t first = first_rows(policy, context_base);
+    if (ordinal == 0) return {0, std::min(total_rows, first), 0};
+    const std::uint32_t offset = first + (ordinal - 1u) * policy.maximum_block_rows;
+    return {offset, std::min(total_rows - offset, policy.maximum_block_rows), ordinal};
+}
+
+PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library) {
+    PrefillPipelines p;
+    HipPipelineError error = HipPipelineError::None;
+    using P = PrefillPipelines;
+    const bool ok =
+        resolve(library, p, &P::attn_qk_rope_blk, "attn_qk_rope_blk", error) &&
+        resolve(library, p, &P::attention_flash_blk, "attention_flash_v2_blk", error) &&
+        resolve(library, p, &P::gdn_conv_blk, "gdn_conv_blk", error) &&
+        resolve(library, p, &P::gdn_gates_blk, "gdn_gates_blk", error) &&
+        resolve(library, p, &P::gdn_recurrence_gates_blk, "gdn_recurrence_gates_blk", error) &&
+        resolve(library, p, &P::gdn_recurrence_blk, "gdn_recurrence_blk", error) &&
+        resolve(library, p, &P::gdn_gate_norm_blk, "gdn_gate_norm_blk", error);
+    if (!ok) return {error, std::nullopt};
+    return {HipPipelineError::None, std::move(p)};
+}
+
+PrefillScratchResult create_prefill_scratch(const HipDevice& device,
+                                            const PrefillGeometry& geometry) {
+    if (!device) return {DecodeStepError::InvalidDevice, std::nullopt};
+    PrefillScratch s;
+    s.block_rows = geometry.policy.maximum_block_rows;
+    const std::uint64_t parameter_bytes =
+        std::uint64_t{s.block_rows} * 32u * kF32Bytes;  // [rows][32] decay / beta
+    if (!allocate_zeroed(device, geometry.gdn_projection_bytes, s.gdn_projection) ||
+        !allocate_zeroed(device, geometry.gdn_qk_bytes, s.gdn_qk) ||
+        !allocate_zeroed(device, geometry.gdn_value_bytes, s.gdn_value) ||
+        !allocate_zeroed(device, geometry.gdn_value_bytes, s.gdn_gate) ||
+        !allocate_zeroed(device, geometry.gdn_value_bytes, s.gdn_recurrence) ||
+        !allocate_zeroed(device, geometry.gdn_value_bytes, s.gdn_gated) ||
+        !allocate_zeroed(device, parameter_bytes, s.gdn_decay) ||
+        !allocate_zeroed(device, parameter_bytes, s.gdn_beta) ||
+        !allocate_zeroed(device, geometry.attention_projection_bytes, s.attn_projection) ||
+        !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_query) ||
+        !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_gate) ||
+        !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_attended)) {
+        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+    }
+    return {DecodeStepError::None, std::move(s)};
+}
+
+HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
+                                         const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                         const DecodeLayerState& state, const LayerWeights& weights,
+                                         const PrefillChunk& chunk, std::uint32_t context_base,
+                                         HipComputePass& pass) {
+    const std::uint32_t rows = chunk.rows;
+    const std::uint32_t capacity = geometry.policy.context_capacity;
+    if (rows == 0 || rows > scratch.block_rows) return HipCommandError::InvalidDispatchExtent;
+    const std::uint64_t position = std::uint64_t{context_base} + chunk.offset;
+    if (position + rows > capacity) return HipCommandError::ContextOutOfRange;
+    Walk walk{pass};
+    walk.pipeline(pipelines.attn_qk_rope_blk);
+    walk.buffer(scratch.attn_projection, 0, 0);
+    walk.weight(weights.query_norm, 1);
+    walk.weight(weights.key_norm, 2);
+    walk.buffer(scratch.attn_query, 0, 3);
+    walk.buffer(scratch.attn_gate, 0, 4);
+    walk.buffer(state.first, 0, 5);
+    walk.buffer(state.second, 0, 6);
+    walk.constant(static_cast<std::uint32_t>(position), 7);
+    walk.constant(capacity, 8);
+    walk.dispatch(18, 256, rows);
+    walk.barrier();
+    walk.pipeline(pipelines.attention_flash_blk);
+    walk.buffer(scratch.attn_query, 0, 0);
+    walk.buffer(state.first, 0, 1);
+    walk.buffer(state.second, 0, 2);
+    walk.buffer(scratch.attn_gate, 0, 3);
+    walk.buffer(scratch.attn_attended, 0, 4);
+    walk.constant(static_cast<std::uint32_t>(position) + rows, 5);
+    walk.constant(capacity, 6);
+    walk.constant(rows, 7);
+    walk.constant(static_cast<std::uint32_t>(position), 8);
+    walk.dispatch(16, 256, (rows + 15u) / 16u);
+    return walk.error;
+}
+
+HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
+                                           const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                           const DecodeLayerState& state,
+                                           const LayerWeights& weights, const PrefillChunk& chunk,
+                                           std::uint32_t recurrence_ordinal, HipComputePass& pass) {
+    const std::uint32_t rows = chunk.rows;
+    if (rows == 0 || rows > scratch.block_rows) return HipCommandError::InvalidDispatchExtent;
+    const bool phase = state.swapped ^ ((recurrence_ordinal & 1u) != 0u);
+    const HipBuffer& conv_in = phase ? state.first_out : state.first;
+    const HipBuffer& conv_out = phase ? state.first : state.first_out;
+    const HipBuffer& recurrent_in = phase ? state.second_out : state.second;
+    const HipBuffer& recurrent_out = phase ? state.second : state.second_out;
+    Walk walk{pass};
+    walk.pipeline(pipelines.gdn_conv_blk);
+    walk.buffer(scratch.gdn_projection, 0, 0);
+    walk.buffer(conv_in, 0, 1);
+    walk.weight(weights.conv_weight, 2);
+    walk.buffer(scratch.gdn_qk, 0, 3);
+    walk.buffer(scratch.gdn_value, 0, 4);
+    walk.buffer(scratch.gdn_gate, 0, 5);
+    walk.buffer(conv_out, 0, 6);
+    walk.constant(rows, 7);
+    walk.dispatch(96, 128, rows);
+    walk.barrier();
+    if (geometry.policy.gdn_gate_hoist) {
+        walk.pipeline(pipelines.gdn_gates_blk);
+        walk.buffer(scratch.gdn_projection, 0, 0);
+        walk.weight(weights.a_log, 1);
+        walk.weight(weights.dt_bias, 2);
+        walk.buffer(scratch.gdn_decay, 0, 3);
+        walk.buffer(scratch.gdn_beta, 0, 4);
+        walk.constant(rows, 5);
+        walk.dispatch(HipSize{1, (rows + 3u) / 4u, 1}, HipSize{32, 4, 1});
+        walk.barrier();
+        walk.pipeline(pipelines.gdn_recurrence_gates_blk);
+        walk.buffer(scratch.gdn_qk, 0, 0);
+        walk.buffer(scratch.gdn_value, 0, 1);
+        walk.buffer(scratch.gdn_decay, 0, 2);
+        walk.weight(weights.a_log, 3);
+        walk.buffer(scratch.gdn_beta, 0, 4);
+    } else {
+        walk.pipeline(pipelines.gdn_recurrence_blk);
+        walk.buffer(scratch.gdn_qk, 0, 0);
+        walk.buffer(scratch.gdn_value, 0, 1);
+        walk.buffer(scratch.gdn_projection, 0, 2);
+        walk.weight(weights.a_log, 3);
+        walk.weight(weights.dt_bias, 4);
+    }
+    walk.buffer(recurrent_in, 0, 5);
+    walk.buffer(scratch.gdn_recurrence, 0, 6);
+    walk.buffer(recurrent_out, 0, 7);
+    walk.constant(rows, 8);
+    walk.dispatch(HipSize{1, 32, 32}, HipSize{32, 4, 1});
+    walk.barrier();
+    walk.pipeline(pipelines.gdn_gate_norm_blk);
+    walk.buffer(scratch.gdn_recurrence, 0, 0);
+    walk.buffer(scratch.gdn_gate, 0, 1);
+    walk.weight(weights.norm_weight, 2);
+    walk.buffer(scratch.gdn_gated, 0, 3);
+    walk.dispatch(32, 128, rows);
+    return walk.error;
+}
+
+}  // namespace tatara::runtime

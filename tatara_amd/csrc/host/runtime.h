@@ -1,0 +1,494 @@
+// tatara::runtime — host side of the attention-family path over the HIP
+// backend: model plan, buffer geometry, per-lane state slots and striped pools,
+// the state-offset table of a lane batch, the per-token layer walk and the
+// block-prefill layer walk.  Types and functions keep the reference's names and
+// meaning (include/tatara/runtime/{decode_geometry,decode_step,
+// prefill_geometry}.h, src/runtime/{decode_step,prefill_step,
+// state_slot_reset}.cpp) so call sites and contract tests read the same; only
+// the attention and Gated DeltaNet branches of the walk are real.  The stages
+// around them (input norm, Q4 projections, MoE, LM head) are a caller-supplied
+// hook: this repository ships a bf16 dense stand-in for them (StackStages).
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <optional>
+#include <span>
+#include <vector>
+
+#include "backend_hip.h"
+
+namespace tatara::model::qwen36 {
+
+// include/tatara/model/qwen36_plan.h:12-15
+enum class LayerKind : std::uint8_t { GatedDelta, FullAttention };
+
+// The fields of StaticModelPlan (qwen36_plan.h:118-131) the path depends on.
+struct ModelPlan {
+    std::uint32_t hidden;
+    std::uint32_t vocabulary;
+    std::uint32_t query_heads;
+    std::uint32_t key_value_heads;
+    std::uint32_t head_dimension;
+    std::uint32_t recurrent_heads;
+    std::uint32_t state_dimension;
+    std::uint32_t initial_serving_capacity;
+    std::vector<LayerKind> layers;
+};
+
+// qwen36-35b-a3b (catalog/model_packages/qwen36-35b-a3b/model.toml:9-34):
+// 40 layers, full attention at 3, 7, ..., 39 (make_hybrid_layer_schedule,
+// qwen36_plan.h:101-113 with period 4, first 3).
+ModelPlan qwen36_35b_a3b_plan();
+std::vector<LayerKind> make_hybrid_layer_schedule(std::size_t layer_count, std::size_t period,
+                                                  std::size_t first);
+
+}  // namespace tatara::model::qwen36
+
+namespace tatara::runtime {
+
+using backend::hip::HipBuffer;
+using backend::hip::HipCommandError;
+using backend::hip::HipComputePass;
+using backend::hip::HipBlitPass;
+using backend::hip::HipComputePipeline;
+using backend::hip::HipDevice;
+using backend::hip::HipLibrary;
+using model::qwen36::LayerKind;
+
+inline constexpr std::uint32_t kAttentionRecordFloats = 258;   // decode_geometry.h:111
+inline constexpr std::uint32_t kAttentionPartition = 256;      // decode_geometry.h:112
+inline constexpr std::uint32_t kConvShiftSteps = 3;
+inline constexpr std::uint32_t kBf16Bytes = 2;
+inline constexpr std::uint32_t kF32Bytes = 4;
+inline constexpr std::uint32_t kMaximumBatchRows = 16;         // decode_step.cpp:554, 1008
+inline constexpr std::uint32_t kPrefillMaximumContext = 262144;   // prefill_geometry.h:14
+inline constexpr std::uint32_t kPrefillMaximumBlockRows = 2048;   // prefill_geometry.h:15
+inline constexpr std::uint32_t kPrefillQueryTileMultiple = 16;    // prefill_geometry.h:16
+
+// decode_geometry.h:133-135
+constexpr bool context_in_capacity(std::uint32_t context, std::uint32_t capacity) {
+    return capacity != 0 && context < capacity;
+}
+
+struct DispatchShape {
+    std::uint32_t groups;
+    std::uint32_t threads;
+};
+struct RecurrenceDispatch {
+    std::uint32_t dimension_groups, head_groups, lane_threads, dimension_threads;
+};
+struct AttentionSplitDispatch {
+    std::uint32_t score_groups, score_threads, score_cohort_threads;
+    std::uint32_t value_groups, value_lane_threads, value_dimension_threads, value_head_threads;
+};
+
+// Attention-family subset of DecodeGeometry / DecodeDispatch
+// (decode_geometry.h:43-108); field names and values are the reference's.
+struct DecodeGeometry {
+    std::uint32_t gated_delta_layers;
+    std::uint32_t attention_layers;
+    std::uint64_t hidden_bytes;
+    std::uint64_t layer_stream_bytes;
+    std::uint64_t gdn_projection_bytes;
+    std::uint64_t gdn_qk_bytes;
+    std::uint64_t gdn_value_bytes;
+    std::uint64_t gdn_gate_bytes;
+    std::uint64_t gdn_conv_state_bytes;
+    std::uint64_t gdn_recurrent_state_bytes;
+    std::uint64_t attn_projection_bytes;
+    std::uint64_t attn_query_bytes;
+    std::uint64_t attn_record_scratch_bytes;
+    std::uint64_t attn_cache_bytes;
+    DispatchShape gdn_prepare;
+    RecurrenceDispatch gdn_recurrence;
+    DispatchShape gdn_gate_norm;
+    DispatchShape attn_qk_rope;
+    DispatchShape attention_head;
+    AttentionSplitDispatch attention_split;
+    DispatchShape rms;
+};
+
+DecodeGeometry make_decode_geometry(const model::qwen36::ModelPlan& plan, std::uint32_t capacity);
+
+// decode_step.cpp:15-19
+std::uint32_t attention_partitions(std::uint32_t context);
+
+// decode_step.h:66-100
+struct DecodeLayerState {
+    HipBuffer first;
+    HipBuffer first_out;
+    HipBuffer second;
+    HipBuffer second_out;
+    bool swapped{false};
+};
+
+enum class DecodeStateSlotStatus : std::uint8_t {
+    Ready,
+    SnapshotPending,
+    RestorePending,
+    ResetPending,
+    Poisoned,
+};
+
+struct DecodeStateSlot {
+    std::uint32_t capacity{0};
+    const LayerKind* schedule_identity{nullptr};
+    std::vector<DecodeLayerState> layers;
+    DecodeStateSlotStatus status{DecodeStateSlotStatus::Ready};
+    std::uint64_t next_transfer_generation{1};
+    std::uint64_t active_transfer_generation{0};
+    std::uint64_t next_reset_generation{1};
+    std::uint64_t active_reset_generation{0};
+    std::uint32_t active_reset_segments{0};
+    std::uint64_t active_reset_bytes{0};
+};
+
+enum class DecodeStepError : std::uint8_t {
+    None,
+    InvalidDevice,
+    InvalidImage,
+    OffsetCountMismatch,
+    BufferAllocationFailed,
+};
+
+// Pipelines of the attention-family walk, resolved by name from the kernel
+// library (decode_step.h:26-61, 322-345).  attention_split_ms/combine_ms fold
+// every long row of a batch into one split-K grid; the reference re-dispatches
+// the one-lane split path per long row (decode_step.cpp:1249-1259).
+struct DecodePipelines {
+    HipComputePipeline gdn_prepare, gdn_recurrence, gdn_gate_norm;
+    HipComputePipeline attn_qk_rope, attention_decode, attention_scores_values_fused,
+        attention_combine;
+    HipComputePipeline gdn_prepare_ms, gdn_recurrence_ms, gate_norm_ms;
+    HipComputePipeline attn_qk_rope_ms, attention_decode_ms, attention_split_ms,
+        attention_combine_ms;
+};
+struct DecodePipelinesResult {
+    backend::hip::HipPipelineError error;
+    std::optional<DecodePipelines> pipelines;
+    explicit operator bool() const noexcept {
+        return error == backend::hip::HipPipelineError::None && pipelines.has_value();
+    }
+};
+DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library);
+
+// Every per-token buffer as a [rows x stride] slab (decode_step.h:202-231,
+// 281-305); strides are the single-stream byte sizes of DecodeGeometry.
+struct DecodeBatchScratch {
+    std::uint32_t rows{0};
+    HipBuffer gdn_projection, gdn_qk, gdn_value, gdn_z, gdn_y, gdn_gated;
+    HipBuffer attn_projection, attn_query, attn_gate, attn_attended, attn_partials;
+    HipBuffer state_offsets;
+    std::uint32_t split_keys{1024};      // keys per split-K workgroup of the batched path
+};
+
+// The step: geometry, schedule and pipelines; its own primary slot (decode_step.h:115-153).
+struct DecodeStep {
+    DecodeGeometry geometry{};
+    std::uint32_t capacity{0};
+    std::vector<LayerKind> schedule;
+    DecodePipelines pipelines;
+    DecodeStateSlot state;
+};
+struct DecodeStepResult {
+    DecodeStepError error;
+    std::optional<DecodeStep> step;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && step.has_value();
+    }
+};
+struct DecodeStateSlotResult {
+    DecodeStepError error;
+    std::optional<DecodeStateSlot> slot;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && slot.has_value();
+    }
+};
+
+// decode_step.h:177-197
+struct DecodeStatePoolLayer {
+    HipBuffer first;
+    HipBuffer second;
+    std::uint64_t first_stride{0};
+    std::uint64_t second_stride{0};
+};
+struct DecodeStatePool {
+    std::uint32_t stripes{0};
+    std::vector<DecodeStatePoolLayer> layers;
+};
+struct DecodeStateSlotPoolResult {
+    DecodeStepError error;
+    std::optional<DecodeStatePool> pool;
+    std::vector<DecodeStateSlot> slots;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && pool.has_value();
+    }
+};
+struct DecodeBatchScratchResult {
+    DecodeStepError error;
+    std::optional<DecodeBatchScratch> scratch;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && scratch.has_value();
+    }
+};
+
+// decode_step.h:245-250
+struct DecodeStream {
+    DecodeStateSlot* state{nullptr};
+    std::uint32_t context{0};
+    std::uint32_t stripe{0};
+};
+
+DecodeStepResult create_decode_step(const HipDevice& device, const DecodeGeometry& geometry,
+                                    std::uint32_t capacity, std::span<const LayerKind> schedule,
+                                    DecodePipelines pipelines);
+DecodeStateSlotResult create_decode_state_slot(const HipDevice& device, const DecodeStep& step);
+DecodeStateSlotPoolResult create_decode_state_slot_pool(const HipDevice& device,
+                                                        const DecodeStep& step,
+                                                        std::uint32_t count);
+DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
+                                                     const DecodeStep& step, std::uint32_t rows);
+
+bool decode_state_slot_compatible(const DecodeStep& step, const DecodeStateSlot& state) noexcept;
+bool decode_state_slot_complete(const DecodeStep& step, const DecodeStateSlot& state) noexcept;
+bool decode_state_slot_available(const DecodeStep& step, const DecodeStateSlot& state) noexcept;
+bool decode_state_slot_ready(const DecodeStep& step, const DecodeStateSlot& state) noexcept;
+
+// Host image of the per-layer state-offset table of a lane batch: 64 u32 per
+// layer (16 rows x 4), then the bucket list of short-context rows
+// (decode_step.cpp:1037-1071).  Pure integers; exact by construction.
+struct StateOffsetTable {
+    std::vector<std::uint32_t> words;   // layers*64 entries + 16 bucket rows
+    std::uint32_t bucket_rows{0};
+};
+HipCommandError build_state_offset_table(const DecodeStep& step,
+                                         std::span<const DecodeStream> streams,
+                                         const DecodeStatePool& pool, StateOffsetTable& out);
+
+// Stages of the walk outside the attention family.  project() must fill
+// scratch.gdn_projection / attn_projection ([rows][stride] bf16) for `layer`
+// from the caller's hidden stream; finish() consumes scratch.gdn_gated /
+// attn_attended.  Both encode into the same pass; returning an error aborts
+// the walk.  A null hook leaves the projection slabs as the caller filled them.
+struct LayerStageHooks {
+    void* user{nullptr};
+    HipCommandError (*project)(void* user, HipComputePass& pass, std::size_t layer, LayerKind kind,
+                               std::uint32_t rows){nullptr};
+    HipCommandError (*finish)(void* user, HipComputePass& pass, std::size_t layer, LayerKind kind,
+                              std::uint32_t rows){nullptr};
+};
+
+struct LayerWeights {
+    // GatedDelta: conv_weight [8192][4], a_log [32], dt_bias [32], norm_weight [128];
+    // FullAttention: query_norm [256], key_norm [256] (all bf16).
+    const HipBuffer* conv_weight{nullptr};
+    const HipBuffer* a_log{nullptr};
+    const HipBuffer* dt_bias{nullptr};
+    const HipBuffer* norm_weight{nullptr};
+    const HipBuffer* query_norm{nullptr};
+    const HipBuffer* key_norm{nullptr};
+};
+
+// One batched token step for up to 16 streams over pool-striped slots
+// (encode_token_batch, decode_step.cpp:1002-1426, attention-family branches).
+// Admission errors (StateSlotMismatch, ContextOutOfRange, InvalidStreamGroup)
+// are returned before anything is encoded.  The host writes the state-offset
+// table first, so the previous step must have completed.
+HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStream> streams,
+                                   const DecodeStatePool& pool, DecodeBatchScratch& batch,
+                                   std::span<const LayerWeights> weights,
+                                   const LayerStageHooks& hooks, HipComputePass& pass);
+
+// One token, one lane, un-batched operators (encode_token, decode_step.cpp:828-842).
+HipCommandError encode_token(DecodeStep& step, DecodeStateSlot& state, DecodeBatchScratch& scratch,
+                             std::span<const LayerWeights> weights, const LayerStageHooks& hooks,
+                             HipComputePass& pass, std::uint32_t context);
+
+// decode_step.cpp:1432-1441: toggles `swapped` on Gated DeltaNet layers of an
+// available, compatible slot; anything else is left untouched.
+void advance_decode_state(const DecodeStep& step, DecodeStateSlot& state);
+void advance_decode_state(DecodeStep& step);
+// prefill_step.cpp:3526-3538: toggles iff the chunk count is odd.
+void advance_prefill_state(const DecodeStep& step, DecodeStateSlot& state, std::uint32_t chunks);
+
+// Lane recycle (state_slot_reset.cpp:176-286): zero-fill both planes of every
+// Gated DeltaNet layer through a blit pass, then complete -> swapped=false,
+// Ready.  Attention KV is never cleared: validity is `context`.
+enum class StateSlotResetError : std::uint8_t {
+    None,
+    InvalidStateSlot,
+    StateSlotNotReady,
+    PoisonedStateSlot,
+    GenerationExhausted,
+    CommandEncodingFailed,
+    StaleTicket,
+    AlreadyCompleted,
+};
+struct StateSlotResetTicket {
+    const DecodeStep* owner{nullptr};
+    DecodeStateSlot* state_owner{nullptr};
+    std::uint32_t segment_count{0};
+    std::uint64_t state_bytes{0};
+    std::uint64_t generation{0};
+    bool pending{false};
+};
+struct StateSlotResetResult {
+    StateSlotResetError error;
+    HipCommandError command_error;
+    std::uint32_t segment_count;
+    std::uint64_t state_bytes;
+    std::optional<StateSlotResetTicket> ticket;
+};
+StateSlotResetResult encode_state_slot_reset(const DecodeStep& step, DecodeStateSlot& state,
+                                             HipBlitPass& blit_pass) noexcept;
+StateSlotResetError complete_state_slot_reset(StateSlotResetTicket& ticket, const DecodeStep& step,
+                                              DecodeStateSlot& state) noexcept;
+
+// ---- block prefill ----
+enum class PrefillSchedule : std::uint8_t { ChunkMajor, LayerMajor };
+
+// prefill_geometry.h:25-34 (attention-family fields)
+struct PrefillPolicy {
+    PrefillSchedule schedule{PrefillSchedule::ChunkMajor};
+    std::uint32_t context_capacity{0};
+    std::uint32_t maximum_block_rows{0};
+    std::uint32_t first_chunk_rows{0};
+    std::uint32_t query_tile_rows{0};
+    std::uint32_t attention_partition{kAttentionPartition};
+    bool gdn_gate_hoist{false};
+};
+
+enum class PrefillRequestError : std::uint8_t {
+    None,
+    EmptyPrefix,
+    BlockOutOfRange,
+    ContextOutOfRange,
+    ContextOverflow,
+    TokenOutOfRange,
+};
+struct PrefillRequestValidation {
+    PrefillRequestError error{PrefillRequestError::EmptyPrefix};
+    std::uint32_t next_context{0};
+    explicit constexpr operator bool() const noexcept {
+        return error == PrefillRequestError::None;
+    }
+};
+// prefill_geometry.h:248-299
+PrefillRequestValidation validate_prefill_request(const PrefillPolicy& policy,
+                                                  std::uint32_t live_context,
+                                                  std::uint32_t context_base,
+                                                  std::span<const std::uint32_t> tokens,
+                                                  std::uint32_t vocabulary) noexcept;
+PrefillRequestValidation validate_prefill_prefix(const PrefillPolicy& policy,
+                                                 std::uint32_t live_context,
+                                                 std::uint32_t context_base,
+                                                 std::span<const std::uint32_t> tokens,
+                                                 std::uint32_t vocabulary) noexcept;
+
+enum class PrefillGeometryError : std::uint8_t { None, InvalidPlan, InvalidPolicy, Overflow };
+
+// Persistent-state and attention-family extents of PrefillGeometry
+// (prefill_geometry.h:65-131, 301-496).
+struct PrefillGeometry {
+    PrefillPolicy policy;
+    std::uint32_t gated_delta_layers{0};
+    std::uint32_t attention_layers{0};
+    std::uint32_t attention_partitions{0};
+    std::uint32_t gdn_projection_rows{0};
+    std::uint32_t gdn_qk_values{0};
+    std::uint32_t gdn_value_values{0};
+    std::uint32_t attention_projection_rows{0};
+    std::uint32_t attention_vector_values{0};
+    std::uint64_t gdn_live_state_bytes_per_layer{0};
+    std::uint64_t gdn_slot_state_bytes_per_layer{0};
+    std::uint64_t attention_state_bytes_per_position_per_layer{0};
+    std::uint64_t attention_slot_state_bytes_per_layer{0};
+    std::uint64_t slot_state_bytes{0};
+    std::uint64_t gdn_projection_bytes{0};
+    std::uint64_t gdn_qk_bytes{0};
+    std::uint64_t gdn_value_bytes{0};
+    std::uint64_t gdn_parameter_bytes{0};
+    std::uint64_t attention_projection_bytes{0};
+    std::uint64_t attention_vector_bytes{0};
+    std::uint64_t attention_partial_bytes{0};
+};
+struct PrefillGeometryResult {
+    PrefillGeometryError error;
+    PrefillGeometry geometry;
+    explicit operator bool() const noexcept { return error == PrefillGeometryError::None; }
+};
+PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan,
+                                            const PrefillPolicy& policy);
+
+// Canonical snapshot payload sizes (prefill_geometry.h:215-246).
+struct PrefixStateSnapshotGeometry {
+    bool valid{false};
+    std::uint32_t positions{0};
+    std::uint64_t gated_delta_bytes{0};
+    std::uint64_t attention_bytes{0};
+    std::uint64_t total_bytes{0};
+};
+PrefixStateSnapshotGeometry make_prefix_state_snapshot_geometry(const PrefillGeometry& geometry,
+                                                                std::uint32_t positions) noexcept;
+
+// prefill_step.cpp:511-550
+struct PrefillChunk {
+    std::uint32_t offset;
+    std::uint32_t rows;
+    std::uint32_t ordinal;
+};
+std::uint32_t prefill_chunk_count(const PrefillPolicy& policy, std::uint32_t context_base,
+                                  std::uint32_t rows);
+PrefillChunk prefill_chunk_at(const PrefillPolicy& policy, std::uint32_t context_base,
+                              std::uint32_t total_rows, std::uint32_t ordinal);
+
+struct PrefillPipelines {
+    HipComputePipeline attn_qk_rope_blk, attention_flash_blk;
+    HipComputePipeline gdn_conv_blk, gdn_gates_blk, gdn_recurrence_gates_blk, gdn_recurrence_blk,
+        gdn_gate_norm_blk;
+};
+struct PrefillPipelinesResult {
+    backend::hip::HipPipelineError error;
+    std::optional<PrefillPipelines> pipelines;
+    explicit operator bool() const noexcept {
+        return error == backend::hip::HipPipelineError::None && pipelines.has_value();
+    }
+};
+PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library);
+
+// Block scratch: [maximum_block_rows x width] slabs of the family's stages.
+struct PrefillScratch {
+    std::uint32_t block_rows{0};
+    HipBuffer gdn_projection, gdn_qk, gdn_value, gdn_gate, gdn_recurrence, gdn_gated;
+    HipBuffer gdn_decay, gdn_beta;
+    HipBuffer attn_projection, attn_query, attn_gate, attn_attended;
+};
+struct PrefillScratchResult {
+    DecodeStepError error;
+    std::optional<PrefillScratch> scratch;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && scratch.has_value();
+    }
+};
+PrefillScratchResult create_prefill_scratch(const HipDevice& device,
+                                            const PrefillGeometry& geometry);
+
+// encode_attention (prefill_step.cpp:1386-1851): rope + append the chunk's rows
+// at context_base + chunk.offset, then causal attention of the chunk (one flash
+// dispatch for the whole chunk; the reference walks 256-row query tiles).
+HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
+                                         const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                         const DecodeLayerState& state, const LayerWeights& weights,
+                                         const PrefillChunk& chunk, std::uint32_t context_base,
+                                         HipComputePass& pass);
+// encode_gated_delta (prefill_step.cpp:1854-2081): phase = swapped ^ (ordinal & 1)
+// selects the ping-pong planes; conv over the block, gates (hoisted or inline),
+// register-loop scan, gate-norm.
+HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
+                                           const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                           const DecodeLayerState& state,
+                                           const LayerWeights& weights, const PrefillChunk& chunk,
+                                           std::uint32_t recurrence_ordinal, HipComputePass& pass);
+
+}  // namespace tatara::runtime

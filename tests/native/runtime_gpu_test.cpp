@@ -1,0 +1,364 @@
+// The C++ host layer end to end on the GPU against the CPU checker: a 4-layer
+// stack (G,G,G,A) over pooled lanes, two batched token steps with the ping-pong
+// flip in between, a two-chunk block prefill on a private slot, and a lane
+// reset.  Returns a distinct non-zero code per failed check and prints the
+// error figures it accepts (max-abs <= 2e-2, mean-abs <= 2e-3 on bf16 outputs;
+// cache/state slot placement exact).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "runtime.h"
+#include "tatara_oracle.h"
+
+using namespace tatara::runtime;
+using namespace tatara::backend::hip;
+
+namespace {
+
+constexpr std::uint32_t kCapacity = 1024;
+constexpr std::uint32_t kLanes = 3;
+
+std::vector<std::uint16_t> gauss16(std::uint64_t seed, std::size_t n, double sigma = 1.0) {
+    std::vector<std::uint16_t> v(n);
+    tto_fill_gaussian_bf16(seed, 0.0, sigma, v.data(), n);
+    return v;
+}
+std::vector<float> gauss32(std::uint64_t seed, std::size_t n, double sigma) {
+    std::vector<float> v(n);
+    tto_fill_gaussian_f32(seed, 0.0, sigma, v.data(), n);
+    return v;
+}
+
+template <typename T> bool upload(const HipBuffer& b, const std::vector<T>& v, std::uint64_t off = 0) {
+    return tt_buffer_write(b.native(), off, v.data(), v.size() * sizeof(T)) == TT_OK;
+}
+template <typename T> std::vector<T> download(const HipBuffer& b, std::size_t n, std::uint64_t off = 0) {
+    std::vector<T> v(n);
+    if (tt_buffer_read(b.native(), off, v.data(), n * sizeof(T)) != TT_OK) v.clear();
+    return v;
+}
+
+bool close16(const std::vector<std::uint16_t>& got, const std::uint16_t* want, std::size_t n,
+             const char* what) {
+    if (got.size() != n) return false;
+    double max_abs = 0.0, sum = 0.0;
+    for (std::size_t i = 0; i < n; ++i) {
+        const double e = std::fabs(double(tto_f32_from_bf16(got[i])) - tto_f32_from_bf16(want[i]));
+        if (!(e == e)) return false;
+        max_abs = std::max(max_abs, e);
+        sum += e;
+    }
+    std::printf("[parity] %s: max-abs %.3e mean-abs %.3e\n", what, max_abs, sum / double(n));
+    std::fflush(stdout);
+    return max_abs <= 2e-2 && sum / double(n) <= 2e-3;
+}
+bool close32(const std::vector<float>& got, const std::vector<float>& want, const char* what) {
+    if (got.size() != want.size()) return false;
+    double max_abs = 0.0;
+    for (std::size_t i = 0; i < got.size(); ++i) {
+        max_abs = std::max(max_abs, std::fabs(double(got[i]) - want[i]));
+    }
+    std::printf("[parity] %s: max-abs %.3e\n", what, max_abs);
+    std::fflush(stdout);
+    return max_abs <= 2e-3;
+}
+
+struct Weights {
+    std::vector<std::uint16_t> conv_w, a_log, dt_bias, norm_w, q_norm, k_norm;
+    HipBuffer b_conv_w, b_a_log, b_dt_bias, b_norm_w, b_q_norm, b_k_norm;
+};
+
+struct Submit {
+    const HipCommandQueue& queue;
+    // encodes `body` into one compute pass, commits, waits; 0 on success
+    template <typename Body> int run(Body body) const {
+        auto cb = create_command_buffer(queue);
+        if (!cb) return 1;
+        auto pass = begin_compute_pass(std::move(*cb.command_buffer));
+        if (!pass) return 2;
+        const HipCommandError encoded = body(*pass.compute_pass);
+        if (encoded != HipCommandError::None) {
+            std::printf("encode error %d\n", int(encoded));
+            return 3;
+        }
+        auto ended = end_compute_pass(std::move(*pass.compute_pass));
+        if (!ended) return 4;
+        auto pending = commit(std::move(*ended.command_buffer));
+        if (!pending) return 5;
+        const HipExecutionResult done = wait_until_completed(std::move(*pending.pending_execution));
+        if (!done) {
+            std::printf("execution failed: %s\n", done.failure_description.data());
+            return 6;
+        }
+        return 0;
+    }
+};
+
+}  // namespace
+
+int main() {
+    auto device = create_system_device();
+    if (!device) return 1;
+    auto queue = create_command_queue(*device.device);
+    auto library = create_kernel_library(*device.device);
+    if (!queue || !library) return 2;
+    auto decode_pipes = resolve_decode_pipelines(*library.library);
+    auto prefill_pipes = resolve_prefill_pipelines(*library.library);
+    if (!decode_pipes || !prefill_pipes) return 3;
+    const Submit submit{*queue.command_queue};
+
+    auto plan = tatara::model::qwen36::qwen36_35b_a3b_plan();
+    plan.layers = tatara::model::qwen36::make_hybrid_layer_schedule(4, 4, 3);
+    const DecodeGeometry geometry = make_decode_geometry(plan, kCapacity);
+    auto made = create_decode_step(*device.device, geometry, kCapacity, plan.layers,
+                                   std::move(*decode_pipes.pipelines));
+    if (!made) return 4;
+    DecodeStep& step = *made.step;
+    if (!decode_state_slot_ready(step, step.state)) return 5;
+
+    // per-layer weights
+    std::vector<Weights> weights(4);
+    std::vector<LayerWeights> bound(4);
+    for (std::size_t l = 0; l < 4; ++l) {
+        Weights& w = weights[l];
+        w.conv_w = gauss16(100 + l, 4 * 8192, 0.5);
+        w.a_log.assign(32, 0xC040);  // -3.0
+        w.dt_bias = gauss16(120 + l, 32, 0.3);
+        w.norm_w.assign(128, 0x3F80);
+        w.q_norm.assign(256, 0x3F80);
+        w.k_norm.assign(256, 0x3F80);
+        HipBuffer* dst[6] = {&w.b_conv_w, &w.b_a_log, &w.b_dt_bias, &w.b_norm_w, &w.b_q_norm,
+                             &w.b_k_norm};
+        const std::vector<std::uint16_t>* src[6] = {&w.conv_w, &w.a_log, &w.dt_bias, &w.norm_w,
+                                                    &w.q_norm, &w.k_norm};
+        for (int i = 0; i < 6; ++i) {
+            auto b = create_shared_buffer(*device.device, src[i]->size() * 2);
+            if (!b) return 6;
+            *dst[i] = std::move(*b.buffer);
+            if (!upload(*dst[i], *src[i])) return 7;
+        }
+        bound[l] = LayerWeights{&w.b_conv_w, &w.b_a_log, &w.b_dt_bias,
+                                &w.b_norm_w, &w.b_q_norm, &w.b_k_norm};
+    }
+
+    // ---- pooled lanes, two batched token steps -------------------------------
+    auto pooled = create_decode_state_slot_pool(*device.device, step, kLanes);
+    if (!pooled) return 10;
+    auto batch_made = create_decode_batch_scratch(*device.device, step, kLanes);
+    if (!batch_made) return 11;
+    DecodeBatchScratch& batch = *batch_made.scratch;
+    batch.split_keys = 256;
+    std::uint32_t contexts[kLanes] = {700, 100, 300};
+    const std::uint32_t stripes[kLanes] = {2, 0, 1};  // lane r lives on stripe stripes[r]
+    // host copies of every lane's state (the checker's side)
+    struct LaneState {
+        std::vector<std::uint16_t> conv[3];
+        std::vector<float> rec[3];
+        std::vector<std::uint16_t> keys, values;
+    };
+    std::vector<LaneState> lanes(kLanes);
+    for (std::uint32_t r = 0; r < kLanes; ++r) {
+        DecodeStateSlot& slot = pooled.slots[stripes[r]];
+        for (int l = 0; l < 3; ++l) {
+            lanes[r].conv[l] = gauss16(1000 + r * 10 + l, 3 * 8192, 0.5);
+            lanes[r].rec[l] = gauss32(2000 + r * 10 + l, 32 * 128 * 128, 0.02);
+            if (!upload(slot.layers[l].first, lanes[r].conv[l]) ||
+                !upload(slot.layers[l].second, lanes[r].rec[l])) {
+                return 12;
+            }
+        }
+        lanes[r].keys.assign(2 * kCapacity * 256, 0);
+        lanes[r].values.assign(2 * kCapacity * 256, 0);
+        const auto k = gauss16(3000 + r, 2 * kCapacity * 256);
+        const auto v = gauss16(4000 + r, 2 * kCapacity * 256);
+        for (std::uint32_t h = 0; h < 2; ++h) {
+            const std::size_t n = std::size_t{contexts[r]} * 256;
+            std::memcpy(&lanes[r].keys[h * kCapacity * 256], &k[h * kCapacity * 256], n * 2);
+            std::memcpy(&lanes[r].values[h * kCapacity * 256], &v[h * kCapacity * 256], n * 2);
+        }
+        if (!upload(slot.layers[3].first, lanes[r].keys) ||
+            !upload(slot.layers[3].second, lanes[r].values)) {
+            return 13;
+        }
+    }
+    const LayerStageHooks no_hooks{};
+    for (int token = 0; token < 2; ++token) {
+        std::vector<std::uint16_t> gdn_proj, attn_proj;
+        for (std::uint32_t r = 0; r < kLanes; ++r) {
+            const auto g = gauss16(5000 + token * 10 + r, 12352, 0.5);
+            const auto a = gauss16(6000 + token * 10 + r, 9216);
+            gdn_proj.insert(gdn_proj.end(), g.begin(), g.end());
+            attn_proj.insert(attn_proj.end(), a.begin(), a.end());
+        }
+        if (!upload(batch.gdn_projection, gdn_proj) || !upload(batch.attn_projection, attn_proj)) {
+            return 14;
+        }
+        std::vector<DecodeStream> streams;
+        for (std::uint32_t r = 0; r < kLanes; ++r) {
+            streams.push_back({&pooled.slots[stripes[r]], contexts[r], stripes[r]});
+        }
+        const int rc = submit.run([&](HipComputePass& pass) {
+            return encode_token_batch(step, streams, *pooled.pool, batch, bound, no_hooks, pass);
+        });
+        if (rc != 0) return 20 + rc;
+        const auto gated = download<std::uint16_t>(batch.gdn_gated, kLanes * 4096);
+        const auto attended = download<std::uint16_t>(batch.attn_attended, kLanes * 4096);
+        for (std::uint32_t r = 0; r < kLanes; ++r) {
+            DecodeStateSlot& slot = pooled.slots[stripes[r]];
+            std::vector<std::uint16_t> want_gated(4096);
+            for (int l = 0; l < 3; ++l) {
+                std::vector<std::uint16_t> ncs(3 * 8192);
+                std::vector<float> so(32 * 128 * 128);
+                tto_gdn_decode_step(&gdn_proj[r * 12352], lanes[r].conv[l].data(),
+                                    weights[l].conv_w.data(), weights[l].a_log.data(),
+                                    weights[l].dt_bias.data(), weights[l].norm_w.data(),
+                                    lanes[r].rec[l].data(), ncs.data(), so.data(),
+                                    want_gated.data(), 4);
+                const DecodeLayerState& s = slot.layers[l];
+                const HipBuffer& conv_out = s.swapped ? s.first : s.first_out;
+                const HipBuffer& rec_out = s.swapped ? s.second : s.second_out;
+                if (download<std::uint16_t>(conv_out, 3 * 8192) != ncs) return 30 + l;
+                if (!close32(download<float>(rec_out, so.size()), so, "pooled recurrent state")) {
+                    return 33 + l;
+                }
+                lanes[r].conv[l] = ncs;
+                lanes[r].rec[l] = so;
+            }
+            if (!close16(std::vector<std::uint16_t>(gated.begin() + r * 4096,
+                                                    gated.begin() + (r + 1) * 4096),
+                         want_gated.data(), 4096, "batched gdn gated (layer 2)")) {
+                return 36;
+            }
+            std::vector<std::uint16_t> q(4096), gate(4096), want(4096);
+            tto_attn_qk_rope(&attn_proj[r * 9216], weights[3].q_norm.data(),
+                             weights[3].k_norm.data(), contexts[r], kCapacity, q.data(), gate.data(),
+                             lanes[r].keys.data(), lanes[r].values.data());
+            tto_attention_decode_split(q.data(), gate.data(), lanes[r].keys.data(),
+                                       lanes[r].values.data(), contexts[r], kCapacity, 256, nullptr,
+                                       want.data(), 4);
+            if (!close16(std::vector<std::uint16_t>(attended.begin() + r * 4096,
+                                                    attended.begin() + (r + 1) * 4096),
+                         want.data(), 4096, "batched attention")) {
+                return 37;
+            }
+            // the appended V row is a raw copy at exactly (head, context)
+            const auto got_v = download<std::uint16_t>(slot.layers[3].second, 2 * kCapacity * 256);
+            if (got_v != lanes[r].values) return 38;
+            advance_decode_state(step, slot);
+            contexts[r] += 1;
+        }
+        for (int l = 0; l < 3; ++l) {
+            if (pooled.slots[0].layers[l].swapped != (token == 0)) return 39;
+        }
+    }
+
+    // ---- block prefill on a private slot: 100 rows in chunks of 64 -----------
+    auto slot_made = create_decode_state_slot(*device.device, step);
+    if (!slot_made) return 50;
+    DecodeStateSlot& slot = *slot_made.slot;
+    const PrefillPolicy policy{.schedule = PrefillSchedule::ChunkMajor,
+                               .context_capacity = kCapacity,
+                               .maximum_block_rows = 64,
+                               .first_chunk_rows = 64,
+                               .query_tile_rows = 64,
+                               .attention_partition = 256,
+                               .gdn_gate_hoist = true};
+    const auto pg = make_prefill_geometry(plan, policy);
+    if (!pg) return 51;
+    auto scratch_made = create_prefill_scratch(*device.device, pg.geometry);
+    if (!scratch_made) return 52;
+    PrefillScratch& ps = *scratch_made.scratch;
+    const std::uint32_t total_rows = 100;
+    const std::uint32_t chunks = prefill_chunk_count(policy, 0, total_rows);
+    if (chunks != 2) return 53;
+    const auto gproj = gauss16(7000, total_rows * 12352, 0.5);
+    const auto aproj = gauss16(7001, total_rows * 9216);
+    std::vector<std::uint16_t> conv0(3 * 8192, 0), keys(2 * kCapacity * 256, 0),
+        values(2 * kCapacity * 256, 0);
+    std::vector<float> rec0(32 * 128 * 128, 0.0f);
+    for (std::uint32_t c = 0; c < chunks; ++c) {
+        const PrefillChunk chunk = prefill_chunk_at(policy, 0, total_rows, c);
+        const std::vector<std::uint16_t> gp(gproj.begin() + chunk.offset * 12352,
+                                            gproj.begin() + (chunk.offset + chunk.rows) * 12352);
+        const std::vector<std::uint16_t> ap(aproj.begin() + chunk.offset * 9216,
+                                            aproj.begin() + (chunk.offset + chunk.rows) * 9216);
+        if (!upload(ps.gdn_projection, gp) || !upload(ps.attn_projection, ap)) return 54;
+        const int rc = submit.run([&](HipComputePass& pass) {
+            HipCommandError e = encode_prefill_gated_delta(*prefill_pipes.pipelines, pg.geometry, ps,
+                                                           slot.layers[0], bound[0], chunk, c, pass);
+            if (e != HipCommandError::None) return e;
+            e = memory_barrier(pass);
+            if (e != HipCommandError::None) return e;
+            return encode_prefill_attention(*prefill_pipes.pipelines, pg.geometry, ps,
+                                            slot.layers[3], bound[3], chunk, 0, pass);
+        });
+        if (rc != 0) return 60 + rc;
+        std::vector<std::uint16_t> ncs(3 * 8192), want_gated(chunk.rows * 4096);
+        std::vector<float> so(rec0.size());
+        tto_gdn_prefill(gp.data(), chunk.rows, conv0.data(), weights[0].conv_w.data(),
+                        weights[0].a_log.data(), weights[0].dt_bias.data(), weights[0].norm_w.data(),
+                        rec0.data(), ncs.data(), so.data(), want_gated.data(), nullptr, nullptr,
+                        nullptr, 4);
+        if (!close16(download<std::uint16_t>(ps.gdn_gated, chunk.rows * 4096), want_gated.data(),
+                     want_gated.size(), "prefill gdn gated")) {
+            return 70;
+        }
+        // phase = swapped ^ (ordinal & 1): chunk 0 writes the out planes, chunk 1 the in planes
+        const bool phase = (c & 1u) != 0u;
+        const HipBuffer& conv_out = phase ? slot.layers[0].first : slot.layers[0].first_out;
+        const HipBuffer& rec_out = phase ? slot.layers[0].second : slot.layers[0].second_out;
+        if (download<std::uint16_t>(conv_out, 3 * 8192) != ncs) return 71;
+        if (!close32(download<float>(rec_out, so.size()), so, "prefill recurrent state")) return 72;
+        conv0 = ncs;
+        rec0 = so;
+        std::vector<std::uint16_t> query(chunk.rows * 4096), gate(chunk.rows * 4096),
+            want(chunk.rows * 4096);
+        tto_attention_prefill(ap.data(), weights[3].q_norm.data(), weights[3].k_norm.data(),
+                              chunk.rows, chunk.offset, kCapacity, query.data(), gate.data(),
+                              keys.data(), values.data(), nullptr, 0, want.data(), 4);
+        if (!close16(download<std::uint16_t>(ps.attn_attended, chunk.rows * 4096), want.data(),
+                     want.size(), "prefill attention")) {
+            return 73;
+        }
+    }
+    if (download<std::uint16_t>(slot.layers[3].second, values.size()) != values) return 74;
+    advance_prefill_state(step, slot, chunks);  // even chunk count: live planes unchanged
+    if (slot.layers[0].swapped) return 75;
+    if (download<std::uint16_t>(slot.layers[0].first, 3 * 8192) != conv0) return 76;
+
+    // ---- lane reset -----------------------------------------------------------
+    {
+        auto cb = create_command_buffer(*queue.command_queue);
+        if (!cb) return 80;
+        auto blit = begin_blit_pass(std::move(*cb.command_buffer));
+        if (!blit) return 81;
+        slot.layers[0].swapped = true;
+        StateSlotResetResult reset = encode_state_slot_reset(step, slot, *blit.blit_pass);
+        if (reset.error != StateSlotResetError::None || !reset.ticket ||
+            reset.segment_count != 6 || reset.state_bytes != 3ull * (49152 + 2097152)) {
+            return 82;
+        }
+        if (slot.status != DecodeStateSlotStatus::ResetPending) return 83;
+        if (decode_state_slot_available(step, slot)) return 84;
+        auto ended = end_blit_pass(std::move(*blit.blit_pass));
+        auto pending = commit(std::move(*ended.command_buffer));
+        if (!pending || !wait_until_completed(std::move(*pending.pending_execution))) return 85;
+        if (complete_state_slot_reset(*reset.ticket, step, slot) != StateSlotResetError::None) {
+            return 86;
+        }
+        if (slot.status != DecodeStateSlotStatus::Ready || slot.layers[0].swapped) return 87;
+        for (const float v : download<float>(slot.layers[0].second, 32 * 128 * 128)) {
+            if (v != 0.0f) return 88;
+        }
+        if (complete_state_slot_reset(*reset.ticket, step, slot) !=
+            StateSlotResetError::AlreadyCompleted) {
+            return 89;
+        }
+        // attention KV is never cleared by a reset
+        if (download<std::uint16_t>(slot.layers[3].second, values.size()) != values) return 90;
+    }
+    std::printf("runtime gpu test ok\n");
+    return 0;
+}
