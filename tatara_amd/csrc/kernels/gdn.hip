@@ -10,6 +10,8 @@
 //   gdn_gate_norm (:174), gdn_gate_norm_ms (:552), gdn_gate_norm_blk (prefill_gdn.metal:283)
 //   gdn_gates_blk (prefill_gdn.metal:94), gdn_recurrence_gates_blk (:137),
 //   gdn_recurrence_blk (:204)
+// plus the chunked evaluation of the block recurrence the reference lacks:
+//   gdn_chunk_prepare_blk, gdn_chunk_scan_blk.
 //
 // State row layout: S[h][j][0..127] with the key index contiguous; one half
 // wave (32 lanes x 4 floats = 512 B) owns one row, so a wave64 load
@@ -284,6 +286,491 @@ __global__ __launch_bounds__(128) void gdn_gate_norm_kernel(const uint16_t* y, c
     out[at] = narrow((g * sig) * normed);
 }
 
+// ------------------------------------------- chunked (WY) block prefill ------
+//
+// The reference walks a block token by token (prefill_gdn.metal:204-281).  The
+// same recurrence is evaluated here 64 tokens at a time so that its products run
+// on MFMA.  With g_t the product of the decays up to token t inside a chunk,
+// L[t][s] = beta_t (g_t/g_s)(k_t.k_s) for s < t and A[t][s] = (g_t/g_s)(q_t.k_s)
+// for s <= t, the per-token deltas u_t of the delta rule satisfy
+//     (I + L) U = beta o (V - (g o K) S0^T)
+// so with Wk = (I+L)^-1 (beta o g o K) and Wv = (I+L)^-1 (beta o V):
+//     U  = Wv - Wk S0^T
+//     Y  = (g o Q) S0^T + A U
+//     S' = g_C S0 + U^T ((g_C/g) o K)
+// Stage 1 (parallel over chunks and heads) builds Wk, Wv, g o Q, (g_C/g) o K and
+// A for every chunk: the k.k and q.k Gram tiles on MFMA, the unit-triangular
+// solve by forward substitution in fp32 (one right-hand-side column per thread).
+// Stage 2 walks the chunks in order, one workgroup per (value head, 32-wide
+// slice of the value dimension), with the fp32 state slice held in MFMA
+// accumulators and every product on v_mfma_f32_16x16x32_bf16.
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr uint32_t kChunk = 64;
+// per (chunk, head) record, byte offsets.  Everything that feeds the recurrent
+// state or the output keeps fp32-grade precision: bf16 MFMA operands that are
+// not exact already are stored as hi/lo pairs, Wv in fp32 (it is only added).
+constexpr uint32_t kRecWkHi = 0;                        // bf16 [64 tokens][128 dk]
+constexpr uint32_t kRecWkLo = 16384;                    // bf16 [64 tokens][128 dk]
+constexpr uint32_t kRecKt = 32768;                      // bf16 [128 dk][64 tokens], exact keys
+constexpr uint32_t kRecAqkHi = 49152;                   // bf16 [64 tokens][64 tokens]
+constexpr uint32_t kRecAqkLo = 57344;                   // bf16 [64 tokens][64 tokens]
+constexpr uint32_t kRecWvT = 65536;                     // f32  [128 dv][64 tokens]
+constexpr uint32_t kRecRatio = 98304;                   // f32  [64]: g_C / g_t
+constexpr uint32_t kRecGam = 98560;                     // f32  [64]: g_t
+constexpr uint32_t kRecGamma = 98816;                   // f32: g_C
+constexpr uint32_t kRecBytes = 99072;
+
+struct ChunkPrepareArgs {
+    const uint16_t* qk;      // [rows][4096]
+    const uint16_t* value;   // [rows][4096]
+    const float* decay;      // [rows][32]
+    const float* beta;       // [rows][32]
+    uint8_t* scratch;        // [chunks][32] records
+    uint32_t rows;
+};
+
+__device__ __forceinline__ bf16x8 operand(const uint16_t* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p));
+}
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+// Two floats to a packed bf16 pair with the hardware conversion (round to
+// nearest even).  Used for MFMA operands only: operator outputs go through
+// narrow().
+__device__ __forceinline__ uint32_t pack_pair(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+// x ~ hi + lo to 2^-17: the pair's hi parts, then the remainders.
+__device__ __forceinline__ void split_pair(float a, float b, uint32_t& hi, uint32_t& lo) {
+    hi = pack_pair(a, b);
+    lo = pack_pair(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xFFFF0000u));
+}
+
+// Four floats to packed hi and lo bf16 quads.
+__device__ __forceinline__ void split4(const f32x4 v, u32x2& hi, u32x2& lo) {
+    uint32_t h0, h1, l0, l1;
+    split_pair(v[0], v[1], h0, l0);
+    split_pair(v[2], v[3], h1, l1);
+    hi = u32x2{h0, h1};
+    lo = u32x2{l0, l1};
+}
+
+// Splits eight floats into bf16 hi and lo MFMA operands.
+__device__ __forceinline__ void split8(const float* x, bf16x8& hi, bf16x8& lo) {
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (uint32_t e = 0; e < 4; ++e) split_pair(x[2 * e], x[2 * e + 1], h[e], l[e]);
+    hi = __builtin_bit_cast(bf16x8, u32x4{h[0], h[1], h[2], h[3]});
+    lo = __builtin_bit_cast(bf16x8, u32x4{l[0], l[1], l[2], l[3]});
+}
+
+// Stage 1, grid (chunks, 32) x 256: decay products, Gram tiles on MFMA, the
+// inverse T of the unit lower-triangular I + L (diagonal 16x16 blocks by forward
+// substitution in registers, the rest by block recursion, all fp32), then
+// [Wk | Wv] = T (beta o [g o K | V]) on MFMA with hi/lo operands.
+__global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs a) {
+    constexpr uint32_t kLd = 68;  // fp32 row stride: 16-byte aligned, bank-skewed
+    __shared__ __attribute__((aligned(16))) float lower[kChunk][kLd];
+    __shared__ __attribute__((aligned(16))) float tinv[kChunk][kLd];
+    __shared__ __attribute__((aligned(16))) float mtmp[16][52];
+    __shared__ __attribute__((aligned(16))) float log_g[kChunk];
+    __shared__ __attribute__((aligned(16))) float scale_k[kChunk];  // beta_t g_t
+    __shared__ __attribute__((aligned(16))) float scale_v[kChunk];  // beta_t
+    const uint32_t chunk = blockIdx.x;
+    const uint32_t h = blockIdx.y;
+    const uint32_t kh = h >> 1;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t wave = tid >> 6;
+    const uint32_t lane = tid & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t t0 = chunk * kChunk;
+    const uint32_t valid = min(kChunk, a.rows - t0);
+    uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
+
+    if (tid < kChunk) {
+        float dec = 1.0f;
+        float b = 0.0f;
+        if (tid < valid) {
+            dec = a.decay[static_cast<uint64_t>(t0 + tid) * kGdnValueHeads + h];
+            b = a.beta[static_cast<uint64_t>(t0 + tid) * kGdnValueHeads + h];
+        }
+        float lg = fmaxf(logf(dec), -87.0f);  // a zero decay acts as exp(-87)
+        for (uint32_t off = 1; off < kChunk; off <<= 1) {
+            const float up = __shfl_up(lg, off, 64);
+            if (lane >= off) lg += up;
+        }
+        log_g[tid] = lg;
+        scale_k[tid] = b * __expf(lg);
+        scale_v[tid] = b;
+        const float log_gc = __shfl(lg, kChunk - 1, 64);
+        reinterpret_cast<float*>(rec + kRecRatio)[tid] = __expf(log_gc - lg);
+        reinterpret_cast<float*>(rec + kRecGam)[tid] = __expf(lg);
+        if (tid == kChunk - 1) *reinterpret_cast<float*>(rec + kRecGamma) = __expf(lg);
+    }
+    for (uint32_t e = tid; e < kChunk * kLd; e += 256) (&tinv[0][0])[e] = 0.0f;
+    __syncthreads();
+
+    const uint16_t* qrows = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kh * kGD;
+    const uint16_t* krows = qrows + kGdnKOffset;
+    {
+        uint16_t* aqk_hi = reinterpret_cast<uint16_t*>(rec + kRecAqkHi);
+        uint16_t* aqk_lo = reinterpret_cast<uint16_t*>(rec + kRecAqkLo);
+        // wave w owns token rows 16w..16w+15 against all 64 columns
+        const uint32_t trow = min(wave * 16 + m, valid - 1);
+        bf16x8 ak[4], aq[4];
+#pragma unroll
+        for (uint32_t kk = 0; kk < 4; ++kk) {
+            ak[kk] = operand(krows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
+            aq[kk] = operand(qrows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
+        }
+#pragma unroll
+        for (uint32_t nt = 0; nt < 4; ++nt) {
+            const uint32_t srow = min(nt * 16 + m, valid - 1);
+            f32x4 kkacc = {0.0f, 0.0f, 0.0f, 0.0f};
+            f32x4 qkacc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t kk = 0; kk < 4; ++kk) {
+                const bf16x8 bk =
+                    operand(krows + static_cast<uint64_t>(srow) * kGdnQkValues + kk * 32 + g * 8);
+                kkacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[kk], bk, kkacc, 0, 0, 0);
+                qkacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aq[kk], bk, qkacc, 0, 0, 0);
+            }
+            const uint32_t s = nt * 16 + m;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                const uint32_t t = wave * 16 + g * 4 + i;
+                const float ratio = s <= t ? __expf(log_g[t] - log_g[s]) : 0.0f;
+                lower[t][s] = (s < t && t < valid) ? scale_v[t] * ratio * kkacc[i] : 0.0f;
+                const float aqk = (s <= t && t < valid) ? ratio * qkacc[i] : 0.0f;
+                const uint16_t hi = narrow(aqk);
+                aqk_hi[t * kChunk + s] = hi;
+                aqk_lo[t * kChunk + s] = narrow(aqk - widen(hi));
+            }
+        }
+    }
+    __syncthreads();
+
+    // diagonal blocks: thread (block b, column c) solves (I + L_bb) x = e_c
+    if (tid < kChunk) {
+        const uint32_t b = tid >> 4;
+        const uint32_t c = tid & 15;
+        float x[16];
+#pragma unroll
+        for (uint32_t r = 0; r < 16; ++r) {
+            float acc = r == c ? 1.0f : 0.0f;
+#pragma unroll
+            for (uint32_t s = 0; s < r; ++s) acc = fmaf(-lower[b * 16 + r][b * 16 + s], x[s], acc);
+            x[r] = acc;
+        }
+#pragma unroll
+        for (uint32_t r = 0; r < 16; ++r) tinv[b * 16 + r][b * 16 + c] = x[r];
+    }
+    __syncthreads();
+    // block rows 1..3: T_i,<i = -T_ii (L_i,<i T_<i,<i)
+    for (uint32_t i = 1; i < 4; ++i) {
+        const uint32_t width = 16 * i;
+        for (uint32_t e = tid; e < 16 * width; e += 256) {
+            const uint32_t r = e / width;
+            const uint32_t c = e - r * width;
+            float acc = 0.0f;
+            for (uint32_t s = c & ~15u; s < width; ++s) {
+                acc = fmaf(lower[16 * i + r][s], tinv[s][c], acc);
+            }
+            mtmp[r][c] = acc;
+        }
+        __syncthreads();
+        for (uint32_t e = tid; e < 16 * width; e += 256) {
+            const uint32_t r = e / width;
+            const uint32_t c = e - r * width;
+            float acc = 0.0f;
+            for (uint32_t s = 0; s <= r; ++s) {
+                acc = fmaf(tinv[16 * i + r][16 * i + s], mtmp[s][c], acc);
+            }
+            tinv[16 * i + r][c] = -acc;
+        }
+        __syncthreads();
+    }
+
+    // [Wk | Wv] = T B: waves 0,1 take the 128 key columns, waves 2,3 the values
+    bf16x8 t_hi[4][2], t_lo[4][2];
+#pragma unroll
+    for (uint32_t mt = 0; mt < 4; ++mt) {
+#pragma unroll
+        for (uint32_t ks = 0; ks < 2; ++ks) {
+            split8(&tinv[mt * 16 + m][ks * 32 + g * 8], t_hi[mt][ks], t_lo[mt][ks]);
+        }
+    }
+    const bool is_k = wave < 2;
+    const uint16_t* src =
+        is_k ? krows : a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
+    const uint32_t src_stride = is_k ? kGdnQkValues : kGdnValueValues;
+    const float* scale = is_k ? scale_k : scale_v;
+    float sc[2][8];
+#pragma unroll
+    for (uint32_t ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) sc[ks][e] = scale[ks * 32 + g * 8 + e];
+    }
+#pragma unroll 1
+    for (uint32_t ct = 0; ct < 4; ++ct) {
+        const uint32_t col = (wave & 1) * 64 + ct * 16 + m;
+        bf16x8 b_hi[2], b_lo[2];
+#pragma unroll
+        for (uint32_t ks = 0; ks < 2; ++ks) {
+            float x[8];
+            uint32_t bits[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                const uint32_t s = ks * 32 + g * 8 + e;
+                bits[e] = s < valid ? src[static_cast<uint64_t>(s) * src_stride + col] : 0u;
+                x[e] = widen(static_cast<uint16_t>(bits[e])) * sc[ks][e];
+            }
+            split8(x, b_hi[ks], b_lo[ks]);
+            if (is_k) {  // the exact keys, token-contiguous
+                *reinterpret_cast<u32x4*>(rec + kRecKt + (col * kChunk + ks * 32 + g * 8) * 2) =
+                    u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                          bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
+            }
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < 4; ++mt) {
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t ks = 0; ks < 2; ++ks) {
+                if (ks * 32 > mt * 16 + 15) continue;  // T is lower triangular
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_lo[mt][ks], b_hi[ks], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_hi[mt][ks], b_lo[ks], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_hi[mt][ks], b_hi[ks], acc, 0, 0, 0);
+            }
+            // lane holds tokens 16mt+4g+i of column col
+            if (is_k) {
+                uint16_t* wk_hi = reinterpret_cast<uint16_t*>(rec + kRecWkHi);
+                uint16_t* wk_lo = reinterpret_cast<uint16_t*>(rec + kRecWkLo);
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    const uint32_t t = mt * 16 + g * 4 + i;
+                    const uint16_t hi = narrow(acc[i]);
+                    wk_hi[t * kGD + col] = hi;
+                    wk_lo[t * kGD + col] = narrow(acc[i] - widen(hi));
+                }
+            } else {
+                *reinterpret_cast<f32x4*>(rec + kRecWvT + (col * kChunk + mt * 16 + g * 4) * 4) = acc;
+            }
+        }
+    }
+}
+
+struct ChunkScanArgs {
+    const uint8_t* scratch;
+    const uint16_t* qk;      // [rows][4096]
+    const float* state_in;
+    float* state_out;
+    uint16_t* y;             // [rows][4096]
+    uint32_t rows;
+};
+
+// One chunk's operands of one wave, loaded a chunk ahead of their use.
+template <uint32_t NT>
+struct ChunkOperands {
+    bf16x8 wk_hi[4], wk_lo[4], q[4], aq_hi[2], aq_lo[2], kt[2][2];
+    f32x4 wv[NT];
+    f32x4 ratio, gam;
+    float gamma_c;
+};
+
+template <uint32_t NT>
+__device__ __forceinline__ ChunkOperands<NT> load_chunk(const ChunkScanArgs& a, uint32_t chunk,
+                                                        uint32_t h, uint32_t slice, uint32_t wave,
+                                                        uint32_t m, uint32_t g) {
+    ChunkOperands<NT> o;
+    const uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
+    const uint16_t* wk_hi = reinterpret_cast<const uint16_t*>(rec + kRecWkHi);
+    const uint16_t* wk_lo = reinterpret_cast<const uint16_t*>(rec + kRecWkLo);
+    const uint16_t* kt = reinterpret_cast<const uint16_t*>(rec + kRecKt);
+    const uint16_t* aq_hi = reinterpret_cast<const uint16_t*>(rec + kRecAqkHi);
+    const uint16_t* aq_lo = reinterpret_cast<const uint16_t*>(rec + kRecAqkLo);
+    const float* wvt = reinterpret_cast<const float*>(rec + kRecWvT);
+    const uint32_t trow = wave * 16 + m;
+    const uint32_t qrow = min(chunk * kChunk + trow, a.rows - 1);
+    const uint16_t* q = a.qk + static_cast<uint64_t>(qrow) * kGdnQkValues + (h >> 1) * kGD;
+#pragma unroll
+    for (uint32_t kk = 0; kk < 4; ++kk) {
+        o.wk_hi[kk] = operand(wk_hi + trow * kGD + kk * 32 + g * 8);
+        o.wk_lo[kk] = operand(wk_lo + trow * kGD + kk * 32 + g * 8);
+        o.q[kk] = operand(q + kk * 32 + g * 8);
+    }
+#pragma unroll
+    for (uint32_t k2 = 0; k2 < 2; ++k2) {
+        o.aq_hi[k2] = operand(aq_hi + trow * kChunk + k2 * 32 + g * 8);
+        o.aq_lo[k2] = operand(aq_lo + trow * kChunk + k2 * 32 + g * 8);
+#pragma unroll
+        for (uint32_t nt = 0; nt < 2; ++nt) {
+            o.kt[nt][k2] = operand(kt + (wave * 32 + nt * 16 + m) * kChunk + k2 * 32 + g * 8);
+        }
+    }
+#pragma unroll
+    for (uint32_t nt = 0; nt < NT; ++nt) {
+        o.wv[nt] = *reinterpret_cast<const f32x4*>(
+            wvt + (slice * 16 * NT + nt * 16 + m) * kChunk + wave * 16 + g * 4);
+    }
+    o.ratio = *reinterpret_cast<const f32x4*>(rec + kRecRatio + (wave * 16 + g * 4) * 4);
+    o.gam = *reinterpret_cast<const f32x4*>(rec + kRecGam + (wave * 16 + g * 4) * 4);
+    o.gamma_c = *reinterpret_cast<const float*>(rec + kRecGamma);
+    return o;
+}
+
+// Stage 2.  grid (8, 4 * 128 / (16 NT)) x 256: a workgroup owns a
+// 16*NT-wide slice of the value dimension.  Wave w owns token rows 16w..16w+15
+// of the chunk products and key columns 32w..32w+31 of the state slice, whose
+// fp32 master copy lives in MFMA accumulators for the whole block.
+template <uint32_t NT>
+__global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
+    constexpr uint32_t DV = 16 * NT;
+    __shared__ __attribute__((aligned(16))) uint16_t s_hi[DV][136];  // bf16 S slice [dv][dk+pad]
+    __shared__ __attribute__((aligned(16))) uint16_t s_lo[DV][136];  // S - s_hi
+    __shared__ __attribute__((aligned(16))) uint16_t u_hi[DV][72];   // U^T [dv][token+pad]
+    __shared__ __attribute__((aligned(16))) uint16_t u_lo[DV][72];
+    __shared__ __attribute__((aligned(16))) uint16_t d_hi[DV][72];   // ((g_C/g) o U)^T
+    __shared__ __attribute__((aligned(16))) uint16_t d_lo[DV][72];
+    // Workgroups are dealt round-robin over the 8 XCDs, each with its own L2, in
+    // linear order (x fastest): blockIdx.x names the XCD.  All slices of a head
+    // read the same chunk records, so a head's slices stay on one XCD.
+    constexpr uint32_t kSlicesPerHead = kGD / DV;
+    const uint32_t local = blockIdx.y;
+    const uint32_t slice = local % kSlicesPerHead;
+    const uint32_t h = blockIdx.x * (kGdnValueHeads / 8) + local / kSlicesPerHead;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t chunks = (a.rows + kChunk - 1) / kChunk;
+
+    // State slice transposed, [dk tile][dv tile]: this lane holds key rows
+    // 32w+16mt+4g+i of value column 16nt+m, four consecutive keys of one state row.
+    f32x4 sacc[2][NT];
+#pragma unroll
+    for (uint32_t mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (uint32_t nt = 0; nt < NT; ++nt) {
+            const uint32_t j = nt * 16 + m;
+            const uint32_t dk = wave * 32 + mt * 16 + g * 4;
+            const f32x4 v = *reinterpret_cast<const f32x4*>(
+                a.state_in + (static_cast<uint64_t>(h) * kGD + slice * DV + j) * kGD + dk);
+            sacc[mt][nt] = v;
+            u32x2 hi, lo;
+            split4(v, hi, lo);
+            *reinterpret_cast<u32x2*>(&s_hi[j][dk]) = hi;
+            *reinterpret_cast<u32x2*>(&s_lo[j][dk]) = lo;
+        }
+    }
+    ChunkOperands<NT> cur = load_chunk<NT>(a, 0, h, slice, wave, m, g);
+    __syncthreads();
+
+    for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+#ifdef TT_EXP_SAMEREC
+        const ChunkOperands<NT> nxt = load_chunk<NT>(a, (chunk + 1) & 1, h, slice, wave, m, g);
+#else
+        const ChunkOperands<NT> nxt =
+            load_chunk<NT>(a, min(chunk + 1, chunks - 1), h, slice, wave, m, g);
+#endif
+        // P1 = Wk S^T and P2 = Q S^T for token tile w: [16 x DV]
+        f32x4 y[NT];
+        const uint32_t at = wave * 16 + g * 4;
+#pragma unroll
+        for (uint32_t nt = 0; nt < NT; ++nt) {
+            f32x4 p1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            f32x4 p2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t kk = 0; kk < 4; ++kk) {
+                const bf16x8 sh = operand(&s_hi[nt * 16 + m][kk * 32 + g * 8]);
+                const bf16x8 sl = operand(&s_lo[nt * 16 + m][kk * 32 + g * 8]);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_lo[kk], sh, p1, 0, 0, 0);
+                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sl, p2, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sl, p1, 0, 0, 0);
+                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sh, p2, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sh, p1, 0, 0, 0);
+            }
+            // U = Wv - P1; this lane holds tokens 16w+4g+i of value column 16nt+m
+            const f32x4 u = cur.wv[nt] - p1;
+            const f32x4 d = u * cur.ratio;
+            y[nt] = p2 * cur.gam;
+            u32x2 uh, ul, dh, dl;
+            split4(u, uh, ul);
+            split4(d, dh, dl);
+            *reinterpret_cast<u32x2*>(&u_hi[nt * 16 + m][at]) = uh;
+            *reinterpret_cast<u32x2*>(&u_lo[nt * 16 + m][at]) = ul;
+            *reinterpret_cast<u32x2*>(&d_hi[nt * 16 + m][at]) = dh;
+            *reinterpret_cast<u32x2*>(&d_lo[nt * 16 + m][at]) = dl;
+        }
+        __syncthreads();  // U^T complete; every read of the old state copy is done
+        // Y = g o (Q S^T) + A U
+#pragma unroll
+        for (uint32_t nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                const bf16x8 bh = operand(&u_hi[nt * 16 + m][k2 * 32 + g * 8]);
+                const bf16x8 bl = operand(&u_lo[nt * 16 + m][k2 * 32 + g * 8]);
+                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_lo[k2], bh, y[nt], 0, 0, 0);
+                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bl, y[nt], 0, 0, 0);
+                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bh, y[nt], 0, 0, 0);
+            }
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                const uint32_t token = chunk * kChunk + at + i;
+#ifdef TT_EXP_NOSTORE
+                if (token < a.rows && y[nt][i] == 123.456f) {
+#else
+                if (token < a.rows) {
+#endif
+                    a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV +
+                        nt * 16 + m] = narrow(y[nt][i]);
+                }
+            }
+        }
+        // S^T = g_C S^T + K^T ((g_C/g) o U) for key rows 32w..32w+31
+#pragma unroll
+        for (uint32_t mt = 0; mt < 2; ++mt) {
+#pragma unroll
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                sacc[mt][nt] *= cur.gamma_c;
+#pragma unroll
+                for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                    const bf16x8 dl = operand(&d_lo[nt * 16 + m][k2 * 32 + g * 8]);
+                    const bf16x8 dh = operand(&d_hi[nt * 16 + m][k2 * 32 + g * 8]);
+                    sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dl,
+                                                                           sacc[mt][nt], 0, 0, 0);
+                    sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dh,
+                                                                           sacc[mt][nt], 0, 0, 0);
+                }
+                const f32x4 v = sacc[mt][nt];
+                u32x2 hi, lo;
+                split4(v, hi, lo);
+                const uint32_t dk = wave * 32 + mt * 16 + g * 4;
+                *reinterpret_cast<u32x2*>(&s_hi[nt * 16 + m][dk]) = hi;
+                *reinterpret_cast<u32x2*>(&s_lo[nt * 16 + m][dk]) = lo;
+            }
+        }
+        __syncthreads();  // new state copy visible; U^T free for the next chunk
+        cur = nxt;
+    }
+#pragma unroll
+    for (uint32_t mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (uint32_t nt = 0; nt < NT; ++nt) {
+            const uint32_t j = slice * DV + nt * 16 + m;
+            const uint32_t dk = wave * 32 + mt * 16 + g * 4;
+            *reinterpret_cast<f32x4*>(a.state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + dk) =
+                sacc[mt][nt];
+        }
+    }
+}
+
 // ---------------------------------------------------------------- launchers --
 
 int32_t launch_prepare(const PrepareArgs& p, hipStream_t stream) {
@@ -546,6 +1033,59 @@ int32_t op_gdn_gate_norm_blk(const Bindings& b, const Grid& g, hipStream_t strea
     return gate_norm_common(a, g, rows, kGdnValueValues, stream, validate_only);
 }
 
+
+uint64_t chunk_scratch_bytes(uint32_t rows) {
+    const uint64_t chunks = (static_cast<uint64_t>(rows) + kChunk - 1) / kChunk;
+    return chunks * kGdnValueHeads * kRecBytes;
+}
+
+// gdn_chunk_prepare_blk (no reference counterpart: stage 1 of the chunked
+// evaluation of gdn_recurrence_gates_blk): b0 qk[rows][4096], b1 value[rows][4096],
+// b2 decay[rows][32], b3 beta[rows][32], b4 scratch (ceil(rows/64)*32 records of
+// 99072 B), c5 rows; grid (ceil(rows/64), 32) x 256.
+int32_t op_gdn_chunk_prepare(const Bindings& b, const Grid& g, hipStream_t stream,
+                             bool validate_only) {
+    Args a(b);
+    ChunkPrepareArgs p{};
+    p.rows = a.constant(5);
+    a.require(p.rows >= 1 && p.rows <= (1u << 22), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    const uint32_t chunks = (p.rows + kChunk - 1) / kChunk;
+    a.require(g.gx == chunks && g.gy == 32 && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint64_t rows = p.rows;
+    p.qk = a.buffer<const uint16_t>(0, rows * kGdnQkValues * 2);
+    p.value = a.buffer<const uint16_t>(1, rows * kGdnValueValues * 2);
+    p.decay = a.buffer<const float>(2, rows * kGdnValueHeads * 4);
+    p.beta = a.buffer<const float>(3, rows * kGdnValueHeads * 4);
+    p.scratch = a.buffer<uint8_t>(4, chunk_scratch_bytes(p.rows));
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(gdn_chunk_prepare_kernel, dim3(chunks, kGdnValueHeads), dim3(256), 0, stream,
+                       p);
+    return TT_OK;
+}
+
+// gdn_chunk_scan_blk (stage 2): b0 scratch, b1 qk[rows][4096], b2 state_in,
+// b3 y[rows][4096], b4 state_out, c5 rows; grid (8, 32) x 256.  state_in and
+// state_out may be the same plane.
+int32_t op_gdn_chunk_scan(const Bindings& b, const Grid& g, hipStream_t stream,
+                          bool validate_only) {
+    Args a(b);
+    ChunkScanArgs p{};
+    p.rows = a.constant(5);
+    a.require(p.rows >= 1 && p.rows <= (1u << 22), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    a.require(grid_is(g, 8, 32, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    p.scratch = a.buffer<const uint8_t>(0, chunk_scratch_bytes(p.rows));
+    p.qk = a.buffer<const uint16_t>(1, static_cast<uint64_t>(p.rows) * kGdnQkValues * 2);
+    p.state_in = a.buffer<const float>(2, kGdnStateFloats * 4ull);
+    p.y = a.buffer<uint16_t>(3, static_cast<uint64_t>(p.rows) * kGdnValueValues * 2);
+    p.state_out = a.buffer<float>(4, kGdnStateFloats * 4ull);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(256), 0, stream, p);
+    return TT_OK;
+}
+
 }  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
@@ -565,6 +1105,8 @@ const KernelDesc kGdnPrefillKernels[] = {
     {"gdn_recurrence_gates_blk", op_gdn_recurrence_gates_blk},
     {"gdn_recurrence_blk", op_gdn_recurrence_blk},
     {"gdn_gate_norm_blk", op_gdn_gate_norm_blk},
+    {"gdn_chunk_prepare_blk", op_gdn_chunk_prepare},
+    {"gdn_chunk_scan_blk", op_gdn_chunk_scan},
 };
 const uint32_t kGdnPrefillKernelCount = sizeof(kGdnPrefillKernels) / sizeof(kGdnPrefillKernels[0]);
 
