@@ -877,7 +877,12 @@ PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan
     g.gdn_projection_bytes = block * rows.gdn_projection * kBf16Bytes;
     g.gdn_qk_bytes = block * rows.gdn_qk * kBf16Bytes;
     g.gdn_value_bytes = block * rows.gdn_values * kBf16Bytes;
-    g.gdn_parameter_bytes = policy.gdn_gate_hoist ? block * plan.recurrent_heads * kF32Bytes : 0;
+    g.gdn_parameter_bytes = (policy.gdn_gate_hoist || policy.gdn_chunked)
+                                ? block * plan.recurrent_heads * kF32Bytes
+                                : 0;
+    g.gdn_chunk_bytes = policy.gdn_chunked ? ((block + kGdnChunkRows - 1u) / kGdnChunkRows) *
+                                                 plan.recurrent_heads * kGdnChunkRecordBytes
+                                           : 0;
     g.attention_projection_bytes = block * rows.attn_projection * kBf16Bytes;
     g.attention_vector_bytes = block * rows.attn_query * kBf16Bytes;
     std::uint64_t records = 0;
@@ -953,7 +958,9 @@ PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::gdn_gates_blk, "gdn_gates_blk", error) &&
         resolve(library, p, &P::gdn_recurrence_gates_blk, "gdn_recurrence_gates_blk", error) &&
         resolve(library, p, &P::gdn_recurrence_blk, "gdn_recurrence_blk", error) &&
-        resolve(library, p, &P::gdn_gate_norm_blk, "gdn_gate_norm_blk", error);
+        resolve(library, p, &P::gdn_gate_norm_blk, "gdn_gate_norm_blk", error) &&
+        resolve(library, p, &P::gdn_chunk_prepare_blk, "gdn_chunk_prepare_blk", error) &&
+        resolve(library, p, &P::gdn_chunk_scan_blk, "gdn_chunk_scan_blk", error);
     if (!ok) return {error, std::nullopt};
     return {HipPipelineError::None, std::move(p)};
 }
@@ -973,6 +980,8 @@ PrefillScratchResult create_prefill_scratch(const HipDevice& device,
         !allocate_zeroed(device, geometry.gdn_value_bytes, s.gdn_gated) ||
         !allocate_zeroed(device, parameter_bytes, s.gdn_decay) ||
         !allocate_zeroed(device, parameter_bytes, s.gdn_beta) ||
+        (geometry.gdn_chunk_bytes != 0 &&
+         !allocate_zeroed(device, geometry.gdn_chunk_bytes, s.gdn_chunk)) ||
         !allocate_zeroed(device, geometry.attention_projection_bytes, s.attn_projection) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_query) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_gate) ||
@@ -1043,6 +1052,43 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
     walk.constant(rows, 7);
     walk.dispatch(96, 128, rows);
     walk.barrier();
+    if (geometry.policy.gdn_chunked) {
+        if (!scratch.gdn_chunk) return HipCommandError::InvalidBuffer;
+        const std::uint32_t chunks = (rows + kGdnChunkRows - 1u) / kGdnChunkRows;
+        walk.pipeline(pipelines.gdn_gates_blk);
+        walk.buffer(scratch.gdn_projection, 0, 0);
+        walk.weight(weights.a_log, 1);
+        walk.weight(weights.dt_bias, 2);
+        walk.buffer(scratch.gdn_decay, 0, 3);
+        walk.buffer(scratch.gdn_beta, 0, 4);
+        walk.constant(rows, 5);
+        walk.dispatch(HipSize{1, (rows + 3u) / 4u, 1}, HipSize{32, 4, 1});
+        walk.barrier();
+        walk.pipeline(pipelines.gdn_chunk_prepare_blk);
+        walk.buffer(scratch.gdn_qk, 0, 0);
+        walk.buffer(scratch.gdn_value, 0, 1);
+        walk.buffer(scratch.gdn_decay, 0, 2);
+        walk.buffer(scratch.gdn_beta, 0, 3);
+        walk.buffer(scratch.gdn_chunk, 0, 4);
+        walk.constant(rows, 5);
+        walk.dispatch(HipSize{chunks, 32, 1}, HipSize{256, 1, 1});
+        walk.barrier();
+        walk.pipeline(pipelines.gdn_chunk_scan_blk);
+        walk.buffer(scratch.gdn_chunk, 0, 0);
+        walk.buffer(recurrent_in, 0, 1);
+        walk.buffer(scratch.gdn_recurrence, 0, 2);
+        walk.buffer(recurrent_out, 0, 3);
+        walk.constant(rows, 4);
+        walk.dispatch(HipSize{8, 32, 1}, HipSize{256, 1, 1});
+        walk.barrier();
+        walk.pipeline(pipelines.gdn_gate_norm_blk);
+        walk.buffer(scratch.gdn_recurrence, 0, 0);
+        walk.buffer(scratch.gdn_gate, 0, 1);
+        walk.weight(weights.norm_weight, 2);
+        walk.buffer(scratch.gdn_gated, 0, 3);
+        walk.dispatch(32, 128, rows);
+        return walk.error;
+    }
     if (geometry.policy.gdn_gate_hoist) {
         walk.pipeline(pipelines.gdn_gates_blk);
         walk.buffer(scratch.gdn_projection, 0, 0);

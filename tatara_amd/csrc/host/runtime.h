@@ -59,6 +59,8 @@ using model::qwen36::LayerKind;
 inline constexpr std::uint32_t kAttentionRecordFloats = 258;   // decode_geometry.h:111
 inline constexpr std::uint32_t kAttentionPartition = 256;      // decode_geometry.h:112
 inline constexpr std::uint32_t kConvShiftSteps = 3;
+inline constexpr std::uint32_t kGdnChunkRows = 64;             // tokens per chunk of the MFMA recurrence
+inline constexpr std::uint32_t kGdnChunkRecordBytes = 115712;  // scratch per (chunk, value head)
 inline constexpr std::uint32_t kBf16Bytes = 2;
 inline constexpr std::uint32_t kF32Bytes = 4;
 inline constexpr std::uint32_t kMaximumBatchRows = 16;         // decode_step.cpp:554, 1008
@@ -357,6 +359,10 @@ struct PrefillPolicy {
     std::uint32_t query_tile_rows{0};
     std::uint32_t attention_partition{kAttentionPartition};
     bool gdn_gate_hoist{false};
+    // Evaluate the block recurrence 64 tokens at a time on MFMA (gdn_chunk_prepare_blk
+    // + gdn_chunk_scan_blk) instead of the reference's token-by-token register loop.
+    // Implies hoisted gates.  The reference has no such switch.
+    bool gdn_chunked{false};
 };
 
 enum class PrefillRequestError : std::uint8_t {
@@ -409,6 +415,7 @@ struct PrefillGeometry {
     std::uint64_t gdn_qk_bytes{0};
     std::uint64_t gdn_value_bytes{0};
     std::uint64_t gdn_parameter_bytes{0};
+    std::uint64_t gdn_chunk_bytes{0};  // chunk records of the MFMA recurrence; 0 when unused
     std::uint64_t attention_projection_bytes{0};
     std::uint64_t attention_vector_bytes{0};
     std::uint64_t attention_partial_bytes{0};
@@ -446,7 +453,7 @@ PrefillChunk prefill_chunk_at(const PrefillPolicy& policy, std::uint32_t context
 struct PrefillPipelines {
     HipComputePipeline attn_qk_rope_blk, attention_flash_blk;
     HipComputePipeline gdn_conv_blk, gdn_gates_blk, gdn_recurrence_gates_blk, gdn_recurrence_blk,
-        gdn_gate_norm_blk;
+        gdn_gate_norm_blk, gdn_chunk_prepare_blk, gdn_chunk_scan_blk;
 };
 struct PrefillPipelinesResult {
     backend::hip::HipPipelineError error;
@@ -461,7 +468,7 @@ PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library);
 struct PrefillScratch {
     std::uint32_t block_rows{0};
     HipBuffer gdn_projection, gdn_qk, gdn_value, gdn_gate, gdn_recurrence, gdn_gated;
-    HipBuffer gdn_decay, gdn_beta;
+    HipBuffer gdn_decay, gdn_beta, gdn_chunk;
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended;
 };
 struct PrefillScratchResult {
@@ -484,7 +491,8 @@ HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
                                          HipComputePass& pass);
 // encode_gated_delta (prefill_step.cpp:1854-2081): phase = swapped ^ (ordinal & 1)
 // selects the ping-pong planes; conv over the block, gates (hoisted or inline),
-// register-loop scan, gate-norm.
+// register-loop scan or, with policy.gdn_chunked, the chunked MFMA recurrence,
+// gate-norm.
 HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
                                            const PrefillGeometry& geometry, PrefillScratch& scratch,
                                            const DecodeLayerState& state,

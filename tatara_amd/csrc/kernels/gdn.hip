@@ -312,16 +312,34 @@ constexpr uint32_t kChunk = 64;
 // per (chunk, head) record, byte offsets.  Everything that feeds the recurrent
 // state or the output keeps fp32-grade precision: bf16 MFMA operands that are
 // not exact already are stored as hi/lo pairs, Wv in fp32 (it is only added).
-constexpr uint32_t kRecWkHi = 0;                        // bf16 [64 tokens][128 dk]
-constexpr uint32_t kRecWkLo = 16384;                    // bf16 [64 tokens][128 dk]
-constexpr uint32_t kRecKt = 32768;                      // bf16 [128 dk][64 tokens], exact keys
-constexpr uint32_t kRecAqkHi = 49152;                   // bf16 [64 tokens][64 tokens]
-constexpr uint32_t kRecAqkLo = 57344;                   // bf16 [64 tokens][64 tokens]
-constexpr uint32_t kRecWvT = 65536;                     // f32  [128 dv][64 tokens]
-constexpr uint32_t kRecRatio = 98304;                   // f32  [64]: g_C / g_t
-constexpr uint32_t kRecGam = 98560;                     // f32  [64]: g_t
-constexpr uint32_t kRecGamma = 98816;                   // f32: g_C
-constexpr uint32_t kRecBytes = 99072;
+// Operands are stored in the order stage 2 consumes them: one 1 KiB fragment per
+// wave-level load (64 lanes x 16 B, lane = 16 g + m), so every load instruction
+// of stage 2 reads whole cache lines.
+//   token-by-key operands (Wk hi, Wk lo, Q): fragment (token tile w, key step kk),
+//     lane (m, g) = token 16w+m, keys 32kk+8g..+7
+//   K^T: fragment (key tile 2w+mt, token step k2), lane = key 16(2w+mt)+m, tokens 32k2+8g..+7
+//   A hi/lo: fragment (token tile w, token step k2), lane = token 16w+m, tokens 32k2+8g..+7
+//   Wv (fp32): fragment (value slice of 16, token tile w), lane = value 16 slice+m, tokens 16w+4g..+3
+constexpr uint32_t kRecWkHi = 0;
+constexpr uint32_t kRecWkLo = 16384;
+constexpr uint32_t kRecQ = 32768;
+constexpr uint32_t kRecKt = 49152;
+constexpr uint32_t kRecAqkHi = 65536;
+constexpr uint32_t kRecAqkLo = 73728;
+constexpr uint32_t kRecWv = 81920;
+constexpr uint32_t kRecRatio = 114688;                  // f32  [64]: g_C / g_t
+constexpr uint32_t kRecGam = 114944;                    // f32  [64]: g_t
+constexpr uint32_t kRecGamma = 115200;                  // f32: g_C
+constexpr uint32_t kRecBytes = 115712;
+
+// byte offset of element (token t, key dk) inside a token-by-key operand
+__device__ __forceinline__ uint32_t frag_token_key(uint32_t t, uint32_t dk) {
+    return ((((t >> 4) * 4 + (dk >> 5)) * 64 + ((dk >> 3) & 3) * 16 + (t & 15)) * 8 + (dk & 7)) * 2;
+}
+// byte offset of element (token t, token s) inside an A operand
+__device__ __forceinline__ uint32_t frag_token_token(uint32_t t, uint32_t s) {
+    return ((((t >> 4) * 2 + (s >> 5)) * 64 + ((s >> 3) & 3) * 16 + (t & 15)) * 8 + (s & 7)) * 2;
+}
 
 struct ChunkPrepareArgs {
     const uint16_t* qk;      // [rows][4096]
@@ -419,8 +437,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     const uint16_t* qrows = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kh * kGD;
     const uint16_t* krows = qrows + kGdnKOffset;
     {
-        uint16_t* aqk_hi = reinterpret_cast<uint16_t*>(rec + kRecAqkHi);
-        uint16_t* aqk_lo = reinterpret_cast<uint16_t*>(rec + kRecAqkLo);
         // wave w owns token rows 16w..16w+15 against all 64 columns
         const uint32_t trow = min(wave * 16 + m, valid - 1);
         bf16x8 ak[4], aq[4];
@@ -428,6 +444,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
         for (uint32_t kk = 0; kk < 4; ++kk) {
             ak[kk] = operand(krows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
             aq[kk] = operand(qrows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
+            *reinterpret_cast<u32x4*>(rec + kRecQ + ((wave * 4 + kk) * 64 + lane) * 16) =
+                __builtin_bit_cast(u32x4, aq[kk]);
         }
 #pragma unroll
         for (uint32_t nt = 0; nt < 4; ++nt) {
@@ -449,8 +467,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
                 lower[t][s] = (s < t && t < valid) ? scale_v[t] * ratio * kkacc[i] : 0.0f;
                 const float aqk = (s <= t && t < valid) ? ratio * qkacc[i] : 0.0f;
                 const uint16_t hi = narrow(aqk);
-                aqk_hi[t * kChunk + s] = hi;
-                aqk_lo[t * kChunk + s] = narrow(aqk - widen(hi));
+                *reinterpret_cast<uint16_t*>(rec + kRecAqkHi + frag_token_token(t, s)) = hi;
+                *reinterpret_cast<uint16_t*>(rec + kRecAqkLo + frag_token_token(t, s)) =
+                    narrow(aqk - widen(hi));
             }
         }
     }
@@ -533,7 +552,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             }
             split8(x, b_hi[ks], b_lo[ks]);
             if (is_k) {  // the exact keys, token-contiguous
-                *reinterpret_cast<u32x4*>(rec + kRecKt + (col * kChunk + ks * 32 + g * 8) * 2) =
+                *reinterpret_cast<u32x4*>(rec + kRecKt +
+                                          (((col >> 4) * 2 + ks) * 64 + g * 16 + (col & 15)) * 16) =
                     u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
                           bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
             }
@@ -550,17 +570,16 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             }
             // lane holds tokens 16mt+4g+i of column col
             if (is_k) {
-                uint16_t* wk_hi = reinterpret_cast<uint16_t*>(rec + kRecWkHi);
-                uint16_t* wk_lo = reinterpret_cast<uint16_t*>(rec + kRecWkLo);
 #pragma unroll
                 for (uint32_t i = 0; i < 4; ++i) {
-                    const uint32_t t = mt * 16 + g * 4 + i;
+                    const uint32_t at = frag_token_key(mt * 16 + g * 4 + i, col);
                     const uint16_t hi = narrow(acc[i]);
-                    wk_hi[t * kGD + col] = hi;
-                    wk_lo[t * kGD + col] = narrow(acc[i] - widen(hi));
+                    *reinterpret_cast<uint16_t*>(rec + kRecWkHi + at) = hi;
+                    *reinterpret_cast<uint16_t*>(rec + kRecWkLo + at) = narrow(acc[i] - widen(hi));
                 }
             } else {
-                *reinterpret_cast<f32x4*>(rec + kRecWvT + (col * kChunk + mt * 16 + g * 4) * 4) = acc;
+                *reinterpret_cast<f32x4*>(rec + kRecWv +
+                                          (((col >> 4) * 4 + mt) * 64 + g * 16 + (col & 15)) * 16) = acc;
             }
         }
     }
@@ -568,7 +587,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
 
 struct ChunkScanArgs {
     const uint8_t* scratch;
-    const uint16_t* qk;      // [rows][4096]
     const float* state_in;
     float* state_out;
     uint16_t* y;             // [rows][4096]
@@ -590,34 +608,28 @@ __device__ __forceinline__ ChunkOperands<NT> load_chunk(const ChunkScanArgs& a, 
                                                         uint32_t m, uint32_t g) {
     ChunkOperands<NT> o;
     const uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
-    const uint16_t* wk_hi = reinterpret_cast<const uint16_t*>(rec + kRecWkHi);
-    const uint16_t* wk_lo = reinterpret_cast<const uint16_t*>(rec + kRecWkLo);
-    const uint16_t* kt = reinterpret_cast<const uint16_t*>(rec + kRecKt);
-    const uint16_t* aq_hi = reinterpret_cast<const uint16_t*>(rec + kRecAqkHi);
-    const uint16_t* aq_lo = reinterpret_cast<const uint16_t*>(rec + kRecAqkLo);
-    const float* wvt = reinterpret_cast<const float*>(rec + kRecWvT);
-    const uint32_t trow = wave * 16 + m;
-    const uint32_t qrow = min(chunk * kChunk + trow, a.rows - 1);
-    const uint16_t* q = a.qk + static_cast<uint64_t>(qrow) * kGdnQkValues + (h >> 1) * kGD;
+    const uint32_t lane = g * 16 + m;
+    const auto fragment = [&](uint32_t base, uint32_t index) {
+        return *reinterpret_cast<const u32x4*>(rec + base + (index * 64 + lane) * 16);
+    };
 #pragma unroll
     for (uint32_t kk = 0; kk < 4; ++kk) {
-        o.wk_hi[kk] = operand(wk_hi + trow * kGD + kk * 32 + g * 8);
-        o.wk_lo[kk] = operand(wk_lo + trow * kGD + kk * 32 + g * 8);
-        o.q[kk] = operand(q + kk * 32 + g * 8);
+        o.wk_hi[kk] = __builtin_bit_cast(bf16x8, fragment(kRecWkHi, wave * 4 + kk));
+        o.wk_lo[kk] = __builtin_bit_cast(bf16x8, fragment(kRecWkLo, wave * 4 + kk));
+        o.q[kk] = __builtin_bit_cast(bf16x8, fragment(kRecQ, wave * 4 + kk));
     }
 #pragma unroll
     for (uint32_t k2 = 0; k2 < 2; ++k2) {
-        o.aq_hi[k2] = operand(aq_hi + trow * kChunk + k2 * 32 + g * 8);
-        o.aq_lo[k2] = operand(aq_lo + trow * kChunk + k2 * 32 + g * 8);
+        o.aq_hi[k2] = __builtin_bit_cast(bf16x8, fragment(kRecAqkHi, wave * 2 + k2));
+        o.aq_lo[k2] = __builtin_bit_cast(bf16x8, fragment(kRecAqkLo, wave * 2 + k2));
 #pragma unroll
-        for (uint32_t nt = 0; nt < 2; ++nt) {
-            o.kt[nt][k2] = operand(kt + (wave * 32 + nt * 16 + m) * kChunk + k2 * 32 + g * 8);
+        for (uint32_t mt = 0; mt < 2; ++mt) {
+            o.kt[mt][k2] = __builtin_bit_cast(bf16x8, fragment(kRecKt, (wave * 2 + mt) * 2 + k2));
         }
     }
 #pragma unroll
     for (uint32_t nt = 0; nt < NT; ++nt) {
-        o.wv[nt] = *reinterpret_cast<const f32x4*>(
-            wvt + (slice * 16 * NT + nt * 16 + m) * kChunk + wave * 16 + g * 4);
+        o.wv[nt] = __builtin_bit_cast(f32x4, fragment(kRecWv, (slice * NT + nt) * 4 + wave));
     }
     o.ratio = *reinterpret_cast<const f32x4*>(rec + kRecRatio + (wave * 16 + g * 4) * 4);
     o.gam = *reinterpret_cast<const f32x4*>(rec + kRecGam + (wave * 16 + g * 4) * 4);
@@ -673,12 +685,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
     __syncthreads();
 
     for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-#ifdef TT_EXP_SAMEREC
-        const ChunkOperands<NT> nxt = load_chunk<NT>(a, (chunk + 1) & 1, h, slice, wave, m, g);
-#else
+        // the next chunk's operands are requested before this chunk's products
         const ChunkOperands<NT> nxt =
             load_chunk<NT>(a, min(chunk + 1, chunks - 1), h, slice, wave, m, g);
-#endif
         // P1 = Wk S^T and P2 = Q S^T for token tile w: [16 x DV]
         f32x4 y[NT];
         const uint32_t at = wave * 16 + g * 4;
@@ -723,11 +732,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
 #pragma unroll
             for (uint32_t i = 0; i < 4; ++i) {
                 const uint32_t token = chunk * kChunk + at + i;
-#ifdef TT_EXP_NOSTORE
-                if (token < a.rows && y[nt][i] == 123.456f) {
-#else
                 if (token < a.rows) {
-#endif
                     a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV +
                         nt * 16 + m] = narrow(y[nt][i]);
                 }
@@ -1042,7 +1047,7 @@ uint64_t chunk_scratch_bytes(uint32_t rows) {
 // gdn_chunk_prepare_blk (no reference counterpart: stage 1 of the chunked
 // evaluation of gdn_recurrence_gates_blk): b0 qk[rows][4096], b1 value[rows][4096],
 // b2 decay[rows][32], b3 beta[rows][32], b4 scratch (ceil(rows/64)*32 records of
-// 99072 B), c5 rows; grid (ceil(rows/64), 32) x 256.
+// 115712 B), c5 rows; grid (ceil(rows/64), 32) x 256.
 int32_t op_gdn_chunk_prepare(const Bindings& b, const Grid& g, hipStream_t stream,
                              bool validate_only) {
     Args a(b);
@@ -1065,22 +1070,21 @@ int32_t op_gdn_chunk_prepare(const Bindings& b, const Grid& g, hipStream_t strea
     return TT_OK;
 }
 
-// gdn_chunk_scan_blk (stage 2): b0 scratch, b1 qk[rows][4096], b2 state_in,
-// b3 y[rows][4096], b4 state_out, c5 rows; grid (8, 32) x 256.  state_in and
-// state_out may be the same plane.
+// gdn_chunk_scan_blk (stage 2): b0 scratch, b1 state_in, b2 y[rows][4096],
+// b3 state_out, c4 rows; grid (8, 32) x 256.  state_in and state_out may be the
+// same plane.
 int32_t op_gdn_chunk_scan(const Bindings& b, const Grid& g, hipStream_t stream,
                           bool validate_only) {
     Args a(b);
     ChunkScanArgs p{};
-    p.rows = a.constant(5);
+    p.rows = a.constant(4);
     a.require(p.rows >= 1 && p.rows <= (1u << 22), TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK) return a.status;
     a.require(grid_is(g, 8, 32, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
     p.scratch = a.buffer<const uint8_t>(0, chunk_scratch_bytes(p.rows));
-    p.qk = a.buffer<const uint16_t>(1, static_cast<uint64_t>(p.rows) * kGdnQkValues * 2);
-    p.state_in = a.buffer<const float>(2, kGdnStateFloats * 4ull);
-    p.y = a.buffer<uint16_t>(3, static_cast<uint64_t>(p.rows) * kGdnValueValues * 2);
-    p.state_out = a.buffer<float>(4, kGdnStateFloats * 4ull);
+    p.state_in = a.buffer<const float>(1, kGdnStateFloats * 4ull);
+    p.y = a.buffer<uint16_t>(2, static_cast<uint64_t>(p.rows) * kGdnValueValues * 2);
+    p.state_out = a.buffer<float>(3, kGdnStateFloats * 4ull);
     if (a.status != TT_OK || validate_only) return a.status;
     hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(256), 0, stream, p);
     return TT_OK;
