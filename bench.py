@@ -33,6 +33,12 @@ VISIBLE = 32768
 CAPACITY = 32768
 DEFAULT_SPLIT_KEYS = 1024       # keys per split-K workgroup
 HBM_PEAK_GBS = 8000.0
+CALIBRATION_COPY_BYTES = 256 << 20
+# HBM traffic of one launch of the split-K kernel at this workload, from two
+# rocprofv3 counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
+# scaled by what the same counter read for a plain 256 MiB copy of known size.
+FLASH_FETCH_KIB, FETCH_SCALE = 131289.5, 262144.0 / 131083.3
+FLASH_WRITE_KIB, WRITE_SCALE = 2112.0, 262144.0 / 262144.0
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 
@@ -196,6 +202,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--split-keys", type=int, default=DEFAULT_SPLIT_KEYS,
                     help="keys per split-K workgroup (multiple of 32)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device-to-device copies first, so a "
+                         "counter run has a kernel of known traffic to scale its readings by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (lanes and heads "
@@ -211,6 +220,13 @@ def main():
     queue = dev.create_queue()
     lib = dev.create_library()
     PART = args.split_keys
+    if args.calibrate_copy:
+        src = dev.create_buffer(CALIBRATION_COPY_BYTES)
+        dst = dev.create_buffer(CALIBRATION_COPY_BYTES)
+        for _ in range(3):
+            cb = queue.create_command_buffer()
+            cb.copy_buffer(src, 0, dst, 0, CALIBRATION_COPY_BYTES)
+            cb.commit().wait()
     record, record_split_only, keep = build_workload(B, dev, lib, torch, PART)
 
     steps = []
@@ -287,7 +303,10 @@ def main():
                    "split_keys": PART, "device": dev.name},
         "roofline": {"bound": "hbm", "kernel": "attention_decode_split_ms (flash_decode_kernel)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": (round((FLASH_FETCH_KIB * FETCH_SCALE +
+                                        FLASH_WRITE_KIB * WRITE_SCALE) * 1024)
+                                 if PART == DEFAULT_SPLIT_KEYS else None),
                      "algorithmic_bytes": algo_bytes, "avg_launch_us": split_us},
         "detail": {"attention_layer_us": round(attn_layer_us, 2),
                    "gdn_layer_us": round(gdn_layer_us, 2),

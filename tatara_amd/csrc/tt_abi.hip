@@ -71,6 +71,23 @@ __global__ void tt_fill_bytes(uint8_t* dst, uint64_t length, uint8_t value) {
     }
 }
 
+// Plain device-to-device copy: 16 bytes per thread where both ends allow it.
+// Overlapping ranges are the caller's business, as with the reference's blit.
+__global__ void tt_copy_bytes(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                              uint64_t length, uint32_t wide) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint64_t done = 0;
+    if (wide != 0u) {
+        const uint64_t vectors = length / 16;
+        const uint4* s = reinterpret_cast<const uint4*>(src);
+        uint4* d = reinterpret_cast<uint4*>(dst);
+        for (uint64_t i = first; i < vectors; i += stride) d[i] = s[i];
+        done = vectors * 16;
+    }
+    for (uint64_t i = done + first; i < length; i += stride) dst[i] = src[i];
+}
+
 void release_buffer(tt_buffer* buffer) {
     if (buffer == nullptr) return;
     if (buffer->refs.fetch_sub(1) != 1) return;
@@ -641,8 +658,14 @@ static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool
             error = hipGetLastError();
             if (status != TT_OK && error == hipSuccess) error = hipErrorInvalidValue;
         } else if (command.kind == CommandKind::Copy) {
-            error = hipMemcpyAsync(command.b, command.a, command.length, hipMemcpyDeviceToDevice,
-                                   stream);
+            const bool wide = ((reinterpret_cast<uintptr_t>(command.a) |
+                                reinterpret_cast<uintptr_t>(command.b)) & 15u) == 0;
+            const uint64_t units = wide ? command.length / 16 + 15 : command.length;
+            const uint64_t blocks = (units + 255) / 256;
+            const unsigned grid = static_cast<unsigned>(blocks < 8192 ? (blocks ? blocks : 1) : 8192);
+            hipLaunchKernelGGL(tt_copy_bytes, dim3(grid), dim3(256), 0, stream, command.a,
+                               command.b, command.length, wide ? 1u : 0u);
+            error = hipGetLastError();
         } else {
             const uint64_t blocks = (command.length + 255) / 256;
             const unsigned grid = static_cast<unsigned>(blocks < 4096 ? blocks : 4096);
