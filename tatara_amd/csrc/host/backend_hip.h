@@ -213,7 +213,6 @@ class HipCommandBuffer {
     friend struct HipCommandBufferResult end_compute_pass(class HipComputePass&&);
     friend struct HipCommandBufferResult end_blit_pass(class HipBlitPass&&);
     friend struct HipPendingExecutionResult commit(HipCommandBuffer&&);
-    friend struct HipCommandBufferResult reuse_command_buffer(class HipPendingExecution&&);
     detail::Handle<tt_command_buffer, tt_command_buffer_destroy> h_;
 };
 
@@ -249,7 +248,6 @@ class HipPendingExecution {
   private:
     friend struct HipPendingExecutionResult commit(HipCommandBuffer&&);
     friend struct HipExecutionResult wait_until_completed(HipPendingExecution&&);
-    friend struct HipCommandBufferResult reuse_command_buffer(HipPendingExecution&&);
     detail::Handle<tt_command_buffer, tt_command_buffer_destroy> h_;
 };
 
