@@ -8,18 +8,23 @@
 //   attention_streaming_blk (:860), attention_flash_v2_blk (:1233)  -> flash kernel
 //   attention_partial_blk (:97), attention_combine_blk (:207)        -> control path
 //
-// Flash kernel.  One workgroup = 4 wave64 = 16 consecutive query positions x
-// the 8 query heads of one kv head (128 score rows); wave w owns heads 2w and
-// 2w+1.  Keys are walked in tiles of 32 up to the causal limit of the tile.
-// The four waves share each K/V tile through LDS: HBM/L2 fills the next tile's
-// stage directly (global_load_lds, no registers) while the current one is
-// consumed, two stages of 32.25 KiB each.
+// Flash kernel.  One workgroup = 4 wave64 = 32 consecutive query positions x
+// the 8 query heads of one kv head (256 score rows); wave w owns heads 2w and
+// 2w+1 at both 16-position halves, four 16x16 blocks that share every K and V
+// fragment read from LDS.  Keys are walked in tiles of 32 up to the causal
+// limit of the tile.  The four waves share each K/V tile through LDS: HBM/L2
+// fills stages two tiles ahead directly (global_load_lds, no registers), four
+// stages of 32.25 KiB each, one barrier per tile.
 //   S^T[key][pos] = K[key][:] . Q[pos][:]    v_mfma_f32_16x16x32_bf16,
 //       A = K from LDS, B = Q^T held in registers for the whole walk.
 //   O^T[dim][pos] += V^T[dim][key] P^T[key][pos]
 //       A = V^T: each lane reads 16-byte runs of 8 value rows from LDS and
-//       transposes 8x8 in registers (v_perm_b32), shared by both heads of the
-//       wave; B = P^T = bf16 of the S^T accumulators, no LDS round trip.
+//       transposes 8x8 in registers (v_perm_b32), shared by the wave's four
+//       blocks; B = P^T = bf16 of the S^T accumulators, no LDS round trip.
+// The loop is skewed by one tile: the softmax of tile kb (VALU) sits next to
+// the PV products of tile kb-1 (MFMA) so the two pipes overlap.  The running
+// maximum is only raised when a tile exceeds it by more than 2^8, so the
+// 256-register rescale of O is rare; probabilities then reach at most 2^8.
 // Row r of the dispatch sees keys [0, tile_context + r], which makes every row
 // a decode step at context tile_context + r over the same cache
 // (prefill_attention.metal:117-119).  Algorithmic work: 1024 flop per visible
@@ -32,16 +37,18 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr uint32_t kD = kAttnHeadDim;
-constexpr uint32_t kTilePositions = 16;
 constexpr uint32_t kTileKeys = 32;
 constexpr uint32_t kKeyPairBytes = 1040;                 // key i | key 16+i | 16 B pad
 constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16640
 constexpr uint32_t kValueStageBytes = kTileKeys * 512;   // 16384
 constexpr uint32_t kStageBytes = kKeyStageBytes + kValueStageBytes;
-constexpr uint32_t kFlashLdsBytes = 2 * kStageBytes;     // 66048
+constexpr uint32_t kStages = 4;
+constexpr uint32_t kFlashLdsBytes = kStages * kStageBytes;  // 132096
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kReferenceSlack = 100.0f;  // log2 units a score may exceed the fixed reference by
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -57,6 +64,12 @@ __device__ __forceinline__ uint32_t pack_low(uint32_t a, uint32_t b) {
 __device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
     return __builtin_amdgcn_perm(b, a, 0x07060302u);
 }
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+// two probabilities to a packed bf16 pair (hardware round to nearest even)
+__device__ __forceinline__ uint32_t pack_probabilities(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
 
 struct FlashPrefillArgs {
     const uint16_t* query;   // [rows][16][256]
@@ -69,7 +82,12 @@ struct FlashPrefillArgs {
     uint32_t capacity;
 };
 
-__global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPrefillArgs a) {
+// PH = 16-position halves per workgroup; a wave owns NB = 2*PH blocks.
+template <uint32_t PH>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void attention_flash_prefill_kernel(FlashPrefillArgs a) {
+    constexpr uint32_t NB = 2 * PH;
+    constexpr uint32_t kTilePositions = 16 * PH;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // longest key walks first: the last position tile is dispatched first
     const uint32_t tile = gridDim.x - 1 - blockIdx.x;
@@ -79,21 +97,26 @@ __global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPr
     const uint32_t m = lane & 15;
     const uint32_t g = lane >> 4;
     const uint32_t p0 = tile * kTilePositions;
-    const uint32_t pos = min(p0 + m, a.rows - 1);         // this lane's query row (column n = m)
-    const uint32_t limit = a.tile_context + p0 + m;       // last visible key of that row
     const uint32_t tile_keys = a.tile_context + min(p0 + kTilePositions, a.rows);  // visible count
     const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
 
-    // B operand of S^T for the wave's two heads: Q^T, column n = position p0+n
-    bf16x8 q[2][8];
+    // block b = 2*t + ph: head 2*wave + t, positions p0 + 16*ph + (column n = m).
+    // B operand of S^T: Q^T, held for the whole walk.
+    bf16x8 q[NB][8];
+    uint32_t limit[PH];  // last visible key of this lane's column in each position half
 #pragma unroll
-    for (uint32_t t = 0; t < 2; ++t) {
-        const uint16_t* qrow = a.query + (static_cast<uint64_t>(pos) * kAttnQueryHeads +
-                                          kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
+    for (uint32_t ph = 0; ph < PH; ++ph) {
+        limit[ph] = a.tile_context + p0 + ph * 16 + m;
+        const uint32_t pos = min(p0 + ph * 16 + m, a.rows - 1);
 #pragma unroll
-        for (uint32_t kb = 0; kb < 8; ++kb) {
-            q[t][kb] = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u32x4*>(qrow + kb * 32 + g * 8));
+        for (uint32_t t = 0; t < 2; ++t) {
+            const uint16_t* qrow = a.query + (static_cast<uint64_t>(pos) * kAttnQueryHeads +
+                                              kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
+#pragma unroll
+            for (uint32_t kb = 0; kb < 8; ++kb) {
+                q[t * PH + ph][kb] = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(qrow + kb * 32 + g * 8));
+            }
         }
     }
 
@@ -102,8 +125,8 @@ __global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPr
 
     // each wave moves a quarter of a tile: 4 K transfers (key pairs 4w..4w+3) and
     // 4 V transfers (rows 8w..8w+7), 1 KiB each
-    auto stage_tile = [&](uint32_t kb, uint32_t stage_index) {
-        uint8_t* kstage = lds + stage_index * kStageBytes;
+    auto stage_tile = [&](uint32_t kb) {
+        uint8_t* kstage = lds + (kb % kStages) * kStageBytes;
         uint8_t* vstage = kstage + kKeyStageBytes;
         const uint32_t key0 = kb * kTileKeys;
         const uint32_t last = tile_keys - 1 - key0;  // rows past the walk repeat the last key
@@ -127,35 +150,27 @@ __global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPr
         }
     };
 
-    f32x4 o[2][16];
+    f32x4 o[NB][16];
 #pragma unroll
-    for (uint32_t t = 0; t < 2; ++t) {
+    for (uint32_t b = 0; b < NB; ++b) {
 #pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) o[t][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t j = 0; j < 16; ++j) o[b][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    float m_run[2] = {-INFINITY, -INFINITY};  // in units of log2
-    float l_run[2] = {0.0f, 0.0f};
+    float m_run[NB], l_run[NB];  // maximum in log2 units; this lane's share of the row sum
+#pragma unroll
+    for (uint32_t b = 0; b < NB; ++b) {
+        m_run[b] = -INFINITY;
+        l_run[b] = 0.0f;
+    }
     const float scale = kAttnScale * kLog2e;
 
-    stage_tile(0, 0);
-    for (uint32_t kb = 0; kb < nkb; ++kb) {
-        const bool more = kb + 1 < nkb;
-        if (more) {
-            stage_tile(kb + 1, (kb + 1) & 1);
-            __builtin_amdgcn_s_waitcnt(0x0F78);  // all but the 8 transfers just issued
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        __syncthreads();  // every wave's quarter of tile kb has landed
-        const uint8_t* kstage = lds + (kb & 1) * kStageBytes;
-        const uint8_t* vstage = kstage + kKeyStageBytes;
-        const uint32_t key0 = kb * kTileKeys;
-
-        f32x4 s[2][2];  // [key tile][head]
+    // S^T of tile kb for the wave's four blocks
+    auto scores = [&](uint32_t kb, f32x4 (&s)[2][NB]) {
+        const uint8_t* kstage = lds + (kb % kStages) * kStageBytes;
 #pragma unroll
         for (uint32_t kt = 0; kt < 2; ++kt) {
-            s[kt][0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            s[kt][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) s[kt][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll
         for (uint32_t kk = 0; kk < 8; ++kk) {
@@ -164,102 +179,203 @@ __global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPr
                 const bf16x8 ka = __builtin_bit_cast(
                     bf16x8, *reinterpret_cast<const u32x4*>(kstage + m * kKeyPairBytes + kt * 512 +
                                                             (kk * 4 + g) * 16));
-                s[kt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[0][kk], s[kt][0], 0, 0, 0);
-                s[kt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[1][kk], s[kt][1], 0, 0, 0);
-            }
-        }
-        // lane holds keys key0 + kt*16 + g*4 + i of column (position) m
-        const bool needs_mask = key0 + kTileKeys - 1 > a.tile_context + p0;
-        bf16x8 pb[2];
-        bool rescale = false;
-        float alpha[2];
 #pragma unroll
-        for (uint32_t t = 0; t < 2; ++t) {
-            float sc[8];
-            float block_max = -INFINITY;
-#pragma unroll
-            for (uint32_t kt = 0; kt < 2; ++kt) {
-#pragma unroll
-                for (uint32_t i = 0; i < 4; ++i) {
-                    float v = s[kt][t][i] * scale;
-                    if (needs_mask && key0 + kt * 16 + g * 4 + i > limit) v = -INFINITY;
-                    sc[kt * 4 + i] = v;
-                    block_max = fmaxf(block_max, v);
+                for (uint32_t b = 0; b < NB; ++b) {
+                    s[kt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[b][kk], s[kt][b], 0, 0, 0);
                 }
             }
-            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
-            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
-            const float m_new = fmaxf(m_run[t], block_max);
-            // a row with no visible key yet keeps max = -inf; exp2(-inf - -inf) is avoided
-            const float base = m_new == -INFINITY ? 0.0f : m_new;
-            alpha[t] = __builtin_amdgcn_exp2f(m_run[t] - base);
-            float block_sum = 0.0f;
-            uint32_t pw[4];
-#pragma unroll
-            for (uint32_t c = 0; c < 4; ++c) {
-                const float x0 = __builtin_amdgcn_exp2f(sc[2 * c] - base);
-                const float x1 = __builtin_amdgcn_exp2f(sc[2 * c + 1] - base);
-                block_sum += x0 + x1;
-                pw[c] = static_cast<uint32_t>(f32_to_bf16_bits(x0)) |
-                        (static_cast<uint32_t>(f32_to_bf16_bits(x1)) << 16);
-            }
-            block_sum += __shfl_xor(block_sum, 16, 64);
-            block_sum += __shfl_xor(block_sum, 32, 64);
-            l_run[t] = l_run[t] * alpha[t] + block_sum;
-            m_run[t] = m_new;
-            pb[t] = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
-            rescale = rescale || alpha[t] != 1.0f;
         }
-        if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+    };
+
+    // Scaled and masked scores of tile kb for block b.  Lane holds keys
+    // key0 + kt*16 + g*4 + i of its position column.
+    auto scaled = [&](uint32_t kb, const f32x4 (&s)[2][NB], uint32_t b, float (&sc)[8]) {
+        const uint32_t key0 = kb * kTileKeys;
+        const bool needs_mask = key0 + kTileKeys - 1 > a.tile_context + p0;
 #pragma unroll
-            for (uint32_t t = 0; t < 2; ++t) {
+        for (uint32_t kt = 0; kt < 2; ++kt) {
 #pragma unroll
-                for (uint32_t j = 0; j < 16; ++j) o[t][j] *= alpha[t];
+            for (uint32_t i = 0; i < 4; ++i) {
+                float v = s[kt][b][i] * scale;
+                if (needs_mask && key0 + kt * 16 + g * 4 + i > limit[b % PH]) v = -INFINITY;
+                sc[kt * 4 + i] = v;
             }
         }
-        // O^T += V^T P^T; contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3);
-        // MFMA j covers dims (j>>3)*128 + row*8 + (j&7)
+    };
+    // P^T operand of block b against the reference m_run[b]; adds to the row sum share
+    auto probabilities = [&](const float (&sc)[8], uint32_t b, bf16x8& pb) {
+        float block_sum = 0.0f;
+        uint32_t pw[4];
 #pragma unroll
-        for (uint32_t hh = 0; hh < 2; ++hh) {
-            u32x4 v[8];
+        for (uint32_t c = 0; c < 4; ++c) {
+            const float x0 = __builtin_amdgcn_exp2f(sc[2 * c] - m_run[b]);
+            const float x1 = __builtin_amdgcn_exp2f(sc[2 * c + 1] - m_run[b]);
+            block_sum += x0 + x1;
+            pw[c] = pack_probabilities(x0, x1);
+        }
+        l_run[b] += block_sum;
+        pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+    };
+    // Exact online softmax step of block b: raises the reference to the tile's
+    // maximum and returns the factor O and the row sum are scaled by.
+    auto raise_reference = [&](const float (&sc)[8], uint32_t b) -> float {
+        float block_max = sc[0];
+#pragma unroll
+        for (uint32_t e = 1; e < 8; ++e) block_max = fmaxf(block_max, sc[e]);
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
+        const float m_new = fmaxf(m_run[b], block_max);  // key 0 is visible: finite from tile 0 on
+        const float alpha = __builtin_amdgcn_exp2f(m_run[b] - m_new);
+        l_run[b] *= alpha;
+        m_run[b] = m_new;
+        return alpha;
+    };
+
+    // O^T += V^T P^T of tile kb; contraction slot e of lane group g is key
+    // (e>>2)*16 + g*4 + (e&3); MFMA j covers dims (j>>3)*128 + row*8 + (j&7)
+    auto accumulate = [&](uint32_t kb, const bf16x8 (&pb)[NB]) {
+        const uint8_t* vstage = lds + (kb % kStages) * kStageBytes + kKeyStageBytes;
+#pragma unroll
+        for (uint32_t hq = 0; hq < 4; ++hq) {  // 8 dwords of a value row = 16 dims per lane
+            u32x2 v[8];
 #pragma unroll
             for (uint32_t e = 0; e < 8; ++e) {
                 const uint32_t key = (e >> 2) * 16 + g * 4 + (e & 3);
-                v[e] = *reinterpret_cast<const u32x4*>(vstage + key * 512 + hh * 256 + m * 16);
+                v[e] = *reinterpret_cast<const u32x2*>(vstage + key * 512 + (hq >> 1) * 256 +
+                                                       m * 16 + (hq & 1) * 8);
             }
 #pragma unroll
-            for (uint32_t dw = 0; dw < 4; ++dw) {
+            for (uint32_t d2 = 0; d2 < 2; ++d2) {
+                const uint32_t dw = (hq & 1) * 2 + d2;
                 u32x4 lo, hi;
-                lo.x = pack_low(v[0][dw], v[1][dw]);
-                lo.y = pack_low(v[2][dw], v[3][dw]);
-                lo.z = pack_low(v[4][dw], v[5][dw]);
-                lo.w = pack_low(v[6][dw], v[7][dw]);
-                hi.x = pack_high(v[0][dw], v[1][dw]);
-                hi.y = pack_high(v[2][dw], v[3][dw]);
-                hi.z = pack_high(v[4][dw], v[5][dw]);
-                hi.w = pack_high(v[6][dw], v[7][dw]);
+                lo.x = pack_low(v[0][d2], v[1][d2]);
+                lo.y = pack_low(v[2][d2], v[3][d2]);
+                lo.z = pack_low(v[4][d2], v[5][d2]);
+                lo.w = pack_low(v[6][d2], v[7][d2]);
+                hi.x = pack_high(v[0][d2], v[1][d2]);
+                hi.y = pack_high(v[2][d2], v[3][d2]);
+                hi.z = pack_high(v[4][d2], v[5][d2]);
+                hi.w = pack_high(v[6][d2], v[7][d2]);
                 const bf16x8 va = __builtin_bit_cast(bf16x8, lo);
                 const bf16x8 vb = __builtin_bit_cast(bf16x8, hi);
+                const uint32_t j = (hq >> 1) * 8 + 2 * dw;
 #pragma unroll
-                for (uint32_t t = 0; t < 2; ++t) {
-                    o[t][hh * 8 + 2 * dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        va, pb[t], o[t][hh * 8 + 2 * dw], 0, 0, 0);
-                    o[t][hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        vb, pb[t], o[t][hh * 8 + 2 * dw + 1], 0, 0, 0);
+                for (uint32_t b = 0; b < NB; ++b) {
+                    o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[b], o[b][j], 0, 0, 0);
+                    o[b][j + 1] =
+                        __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb, pb[b], o[b][j + 1], 0, 0, 0);
                 }
             }
         }
-        __syncthreads();  // stage kb&1 may be refilled by the next iteration's transfers
+    };
+
+    stage_tile(0);
+    if (nkb > 1) stage_tile(1);
+    // Entering tile kb: its transfers (issued two tiles earlier) have landed for
+    // every wave, and every wave is done with tile kb-2, whose stage the transfers
+    // of tile kb+2 overwrite.
+    auto enter_tile = [&](uint32_t kb) {
+        if (kb + 1 < nkb) {
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // all but the 8 transfers of tile kb+1
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();
+        if (kb + 2 < nkb) stage_tile(kb + 2);
+    };
+    bf16x8 pb[NB];
+    {
+        enter_tile(0);
+        f32x4 s[2][NB];
+        scores(0, s);
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+            float sc[8];
+            scaled(0, s, b, sc);
+            (void)raise_reference(sc, b);  // O and the sums are still zero
+            probabilities(sc, b, pb[b]);
+        }
+    }
+    // Steady state.  The reference of every row stays where tile 0 put it: scores
+    // are bounded by |q||k|/16, far inside the 2^127 range of fp32 and bf16, so
+    // P = exp2(s - reference) neither overflows nor, the row maximum being at least
+    // the reference, vanishes.  O is touched by MFMA only.  Should a score ever
+    // exceed the reference by more than 2^kReferenceSlack the walk is finished by
+    // the exact loop below.  The loop is skewed: softmax of tile kb (VALU) next to
+    // P V of tile kb-1 (MFMA).
+    uint32_t kb = 1;
+    bool exact = false;
+    while (kb < nkb) {
+        enter_tile(kb);
+        f32x4 s[2][NB];
+        bf16x8 pb_next[NB];
+        scores(kb, s);
+        bool above = false;
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+            float sc[8];
+            scaled(kb, s, b, sc);
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) above = above || sc[e] > m_run[b] + kReferenceSlack;
+            probabilities(sc, b, pb_next[b]);
+        }
+        accumulate(kb - 1, pb);
+        if (__builtin_amdgcn_ballot_w64(above) != 0) {
+            exact = true;  // tile kb is redone by the exact loop; its sums are taken back there
+            break;
+        }
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) pb[b] = pb_next[b];
+        ++kb;
+    }
+    if (!exact) {
+        accumulate(nkb - 1, pb);
+    } else {
+        // Exact online softmax from tile kb on: raise the reference per tile, scale O.
+        // (Reached only with scores beyond any RMS-normalised q, k.)  The sums of the
+        // abandoned tile are recomputed: undo them by rebuilding l from scratch is not
+        // possible, so the steady loop's contribution of tile kb is subtracted first.
+        f32x4 s[2][NB];
+        scores(kb, s);
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+            float sc[8];
+            scaled(kb, s, b, sc);
+            float taken = 0.0f;
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) taken += __builtin_amdgcn_exp2f(sc[e] - m_run[b]);
+            l_run[b] -= taken;
+        }
+        bool first = true;
+        for (; kb < nkb; ++kb) {
+            if (!first) enter_tile(kb);
+            first = false;
+            scores(kb, s);
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) {
+                float sc[8];
+                scaled(kb, s, b, sc);
+                const float alpha = raise_reference(sc, b);
+#pragma unroll
+                for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
+                probabilities(sc, b, pb[b]);
+            }
+            accumulate(kb, pb);
+        }
     }
 
     // out[(row*16 + head)*256 + dim] = bf16((O/l) * sigmoid(gate)); lane holds, for
-    // position m, dims (j>>3)*128 + (g*4+i)*8 + (j&7)
-    if (p0 + m < a.rows) {
+    // position column m, dims (j>>3)*128 + (g*4+i)*8 + (j&7)
 #pragma unroll
-        for (uint32_t t = 0; t < 2; ++t) {
-            const uint64_t row_base = (static_cast<uint64_t>(p0 + m) * kAttnQueryHeads +
-                                       kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
-            const float inv = 1.0f / l_run[t];
+    for (uint32_t b = 0; b < NB; ++b) {
+        float l = l_run[b];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const uint32_t row = p0 + (b % PH) * 16 + m;
+        if (row < a.rows) {
+            const uint64_t row_base = (static_cast<uint64_t>(row) * kAttnQueryHeads +
+                                       kvh * kAttnHeadsPerKv + wave * 2 + b / PH) * kD;
+            const float inv = 1.0f / l;
 #pragma unroll
             for (uint32_t j = 0; j < 16; ++j) {
 #pragma unroll
@@ -267,7 +383,7 @@ __global__ __launch_bounds__(256, 2) void attention_flash_prefill_kernel(FlashPr
                     const uint32_t dim = (j >> 3) * 128 + (g * 4 + i) * 8 + (j & 7);
                     const float gate = bf16_bits_to_f32(a.gate[row_base + dim]);
                     const float sig = 1.0f / (1.0f + __expf(-gate));
-                    a.out[row_base + dim] = f32_to_bf16_bits((o[t][j][i] * inv) * sig);
+                    a.out[row_base + dim] = f32_to_bf16_bits((o[b][j][i] * inv) * sig);
                 }
             }
         }
@@ -394,9 +510,12 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     f.tile_context = a.constant(8);
     a.require(f.rows >= 1 && f.rows <= (1u << 24), TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK) return a.status;
-    const uint32_t tiles = (f.rows + kTilePositions - 1) / kTilePositions;
-    a.require(g.gx == 16 && g.gy == tiles && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+    // the reference dispatches one threadgroup per (head, 16 query rows)
+    a.require(g.gx == 16 && g.gy == (f.rows + 15) / 16 && g.gz == 1 && g.tx == 256 && g.ty == 1 &&
+                  g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
+    constexpr uint32_t kHalves = 1;  // 16-position halves per workgroup
+    const uint32_t tiles = (f.rows + 16 * kHalves - 1) / (16 * kHalves);
     a.require(f.capacity != 0 &&
                   static_cast<uint64_t>(f.tile_context) + f.rows == visible &&
                   visible <= f.capacity,
@@ -408,7 +527,7 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     f.gate = a.buffer<const uint16_t>(3, row_bytes);
     f.out = a.buffer<uint16_t>(4, row_bytes);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(attention_flash_prefill_kernel, dim3(tiles, kAttnKvHeads), dim3(256),
+    hipLaunchKernelGGL(attention_flash_prefill_kernel<kHalves>, dim3(tiles, kAttnKvHeads), dim3(256),
                        kFlashLdsBytes, stream, f);
     return TT_OK;
 }
@@ -472,7 +591,7 @@ int32_t op_attention_combine_blk(const Bindings& b, const Grid& g, hipStream_t s
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
 bool prepare_prefill_kernels() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel<1>),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                kFlashLdsBytes) == hipSuccess;
 }
