@@ -202,8 +202,9 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
             }
         }
     };
-    // P^T operand of block b against the reference m_run[b]; adds to the row sum share
-    auto probabilities = [&](const float (&sc)[8], uint32_t b, bf16x8& pb) {
+    // P^T operand of block b against the reference m_run[b]; returns this lane's
+    // share of the tile's row sum
+    auto probabilities = [&](const float (&sc)[8], uint32_t b, bf16x8& pb) -> float {
         float block_sum = 0.0f;
         uint32_t pw[4];
 #pragma unroll
@@ -213,8 +214,8 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
             block_sum += x0 + x1;
             pw[c] = pack_probabilities(x0, x1);
         }
-        l_run[b] += block_sum;
         pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+        return block_sum;
     };
     // Exact online softmax step of block b: raises the reference to the tile's
     // maximum and returns the factor O and the row sum are scaled by.
@@ -293,7 +294,7 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
             float sc[8];
             scaled(0, s, b, sc);
             (void)raise_reference(sc, b);  // O and the sums are still zero
-            probabilities(sc, b, pb[b]);
+            l_run[b] += probabilities(sc, b, pb[b]);
         }
     }
     // Steady state.  The reference of every row stays where tile 0 put it: scores
@@ -311,41 +312,34 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         bf16x8 pb_next[NB];
         scores(kb, s);
         bool above = false;
+        float sums[NB];
 #pragma unroll
         for (uint32_t b = 0; b < NB; ++b) {
             float sc[8];
             scaled(kb, s, b, sc);
 #pragma unroll
             for (uint32_t e = 0; e < 8; ++e) above = above || sc[e] > m_run[b] + kReferenceSlack;
-            probabilities(sc, b, pb_next[b]);
+            sums[b] = probabilities(sc, b, pb_next[b]);
         }
         accumulate(kb - 1, pb);
         if (__builtin_amdgcn_ballot_w64(above) != 0) {
-            exact = true;  // tile kb is redone by the exact loop; its sums are taken back there
-            break;
+            exact = true;  // tile kb, whose operands above may have overflowed, is dropped
+            break;         // here and redone by the exact loop
         }
 #pragma unroll
-        for (uint32_t b = 0; b < NB; ++b) pb[b] = pb_next[b];
+        for (uint32_t b = 0; b < NB; ++b) {
+            pb[b] = pb_next[b];
+            l_run[b] += sums[b];
+        }
         ++kb;
     }
     if (!exact) {
         accumulate(nkb - 1, pb);
     } else {
         // Exact online softmax from tile kb on: raise the reference per tile, scale O.
-        // (Reached only with scores beyond any RMS-normalised q, k.)  The sums of the
-        // abandoned tile are recomputed: undo them by rebuilding l from scratch is not
-        // possible, so the steady loop's contribution of tile kb is subtracted first.
+        // (Reached only with scores beyond any RMS-normalised q, k.)  The steady loop
+        // has entered tile kb already.
         f32x4 s[2][NB];
-        scores(kb, s);
-#pragma unroll
-        for (uint32_t b = 0; b < NB; ++b) {
-            float sc[8];
-            scaled(kb, s, b, sc);
-            float taken = 0.0f;
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) taken += __builtin_amdgcn_exp2f(sc[e] - m_run[b]);
-            l_run[b] -= taken;
-        }
         bool first = true;
         for (; kb < nkb; ++kb) {
             if (!first) enter_tile(kb);
@@ -358,7 +352,7 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
                 const float alpha = raise_reference(sc, b);
 #pragma unroll
                 for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
-                probabilities(sc, b, pb[b]);
+                l_run[b] += probabilities(sc, b, pb[b]);
             }
             accumulate(kb, pb);
         }

@@ -18,12 +18,13 @@ def _weights():
     return q_w, k_w
 
 
-def _prefill_case(rows, base, cap, seed, select=None, control=False):
+def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, weights=None):
     """Runs rope + flash prefill on the GPU for `rows` new tokens after `base`
     cached ones and compares the selected rows with the checker."""
     B, dev, queue, lib = gpu()
-    q_w, k_w = _weights()
-    proj = ol.gaussian_bf16(seed, rows * 9216)
+    q_w, k_w = _weights() if weights is None else weights
+    if proj is None:
+        proj = ol.gaussian_bf16(seed, rows * 9216)
     keys = np.zeros(2 * cap * 256, np.uint16); values = np.zeros_like(keys)
     if base:
         keys.reshape(2, cap, 256)[:, :base] = ol.gaussian_bf16(seed + 1, 2 * base * 256).reshape(
@@ -107,6 +108,23 @@ def test_prefill_row_equals_decode_step_on_gpu():
                                   3: c["b_v"], 5: b_o}, {4: base + r, 6: cap}, (16,), (256,)))
         check_bf16(b_o.read(np.uint16), c["got"][r], f"decode vs prefill row {r}",
                    max_abs=8e-3, mean_abs=2e-4)
+
+
+def test_scores_far_above_the_first_tile_take_the_exact_loop():
+    """The flash kernel fixes each row's softmax reference at its first key tile
+    and falls back to an exact online-softmax loop when a later score exceeds it
+    by more than 2^100.  Norm weights of 3 and late keys that repeat the last
+    row's query direction give scores near 150 log2 units above the early ones,
+    so the last position tiles finish in that loop."""
+    print("[case] prefill with scores that force the exact softmax loop", flush=True)
+    rows = 96
+    proj = ol.gaussian_bf16(0xE8AC, rows * 9216).reshape(rows, 9216)
+    for r in range(64, rows):
+        proj[r, 8192:8448] = proj[rows - 1, 0:256]          # kv head 0 key := head 0 query of the last row
+        proj[r, 8448:8704] = proj[rows - 1, 4096:4352]      # kv head 1 key := head 8 query of the last row
+    w = np.full(256, 0x4040, np.uint16)                     # 3.0
+    _prefill_case(rows, 0, 128, 0xE8AD, proj=np.ascontiguousarray(proj).reshape(-1), weights=(w, w),
+                  control=True)
 
 
 def test_config4_prefill_16384_rows():
