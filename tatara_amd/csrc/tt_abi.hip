@@ -437,6 +437,7 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
     } families[] = {
         {tt::kAttentionDecodeKernels, tt::kAttentionDecodeKernelCount},
         {tt::kAttentionPrefillKernels, tt::kAttentionPrefillKernelCount},
+        {tt::kAttentionFamilyKernels, tt::kAttentionFamilyKernelCount},
         {tt::kGdnDecodeKernels, tt::kGdnDecodeKernelCount},
         {tt::kGdnPrefillKernels, tt::kGdnPrefillKernelCount},
     };

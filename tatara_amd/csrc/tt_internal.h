@@ -96,6 +96,8 @@ extern const KernelDesc kAttentionDecodeKernels[];
 extern const uint32_t kAttentionDecodeKernelCount;
 extern const KernelDesc kAttentionPrefillKernels[];
 extern const uint32_t kAttentionPrefillKernelCount;
+extern const KernelDesc kAttentionFamilyKernels[];
+extern const uint32_t kAttentionFamilyKernelCount;
 extern const KernelDesc kGdnDecodeKernels[];
 extern const uint32_t kGdnDecodeKernelCount;
 extern const KernelDesc kGdnPrefillKernels[];
