@@ -684,6 +684,51 @@ void tto_gdn_prefill(const uint16_t* projection, uint32_t rows, const uint16_t* 
     if (y_out) std::memcpy(y_out, y.data(), y.size() * 2);
 }
 
+void tto_rms_only(const uint16_t* input, const uint16_t* weight, uint32_t rows, uint32_t hidden,
+                  uint16_t* output) {
+    // hidden / 4 threads of 4 values, simdgroup trees over 32 lanes, then a tree over
+    // the 32-slot stage (zero padded)
+    const uint32_t simdgroups = hidden / 128;
+    for (uint32_t r = 0; r < rows; ++r) {
+        const uint16_t* in = input + static_cast<size_t>(r) * hidden;
+        uint16_t* out = output + static_cast<size_t>(r) * hidden;
+        float stage[32] = {0};
+        float lanes[32];
+        for (uint32_t sg = 0; sg < simdgroups; ++sg) {
+            for (uint32_t l = 0; l < 32; ++l) lanes[l] = squares4(in + (sg * 32 + l) * 4);
+            stage[sg] = adjacent32(lanes);
+        }
+        const float inverse =
+            1.0f / std::sqrt(adjacent32(stage) / static_cast<float>(hidden) + kEps);
+        for (uint32_t i = 0; i < hidden; ++i) {
+            out[i] = mul16(weight[i], store16(widen(in[i]) * inverse));
+        }
+    }
+}
+
+void tto_dense_bf16(const uint16_t* input, const uint16_t* weights, uint32_t rows, uint32_t in_dim,
+                    uint32_t out_dim, uint16_t* output, uint32_t threads) {
+    parallel_for(out_dim, threads, [=](uint32_t n) {
+        const uint16_t* w = weights + static_cast<size_t>(n) * in_dim;
+        for (uint32_t r = 0; r < rows; ++r) {
+            const uint16_t* x = input + static_cast<size_t>(r) * in_dim;
+            // eight interleaved fp32 partial sums, folded pairwise: fixed order,
+            // vectorisable, and close to what a blocked GPU sum does
+            float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (uint32_t k = 0; k < in_dim; k += 8) {
+                for (uint32_t e = 0; e < 8; ++e) acc[e] += widen(x[k + e]) * widen(w[k + e]);
+            }
+            const float total =
+                ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+            output[static_cast<size_t>(r) * out_dim + n] = store16(total);
+        }
+    });
+}
+
+void tto_add_bf16(const uint16_t* a, const uint16_t* b, uint64_t count, uint16_t* out) {
+    for (uint64_t i = 0; i < count; ++i) out[i] = add16(a[i], b[i]);
+}
+
 void tto_gdn_sequential_f64(const double* q, const double* k, const double* v,
                             const double* decay, const double* beta, uint32_t steps, uint32_t dk,
                             uint32_t dv, double* state, double* y) {

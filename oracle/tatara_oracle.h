@@ -190,6 +190,21 @@ void tto_gdn_scan(const uint16_t* qk, const uint16_t* value, const float* decay,
                   const float* beta, uint32_t steps, const float* state_in, uint16_t* y,
                   float* state_out, uint32_t threads);
 
+/* The steps either side of the path in a stacked run.
+ * tto_rms_only: row RMS norm with the double rounding bf16(w * bf16(x * inv))
+ * (rms_only.metal:5-42; rms_total_of_squares / rms_only_reference
+ * kernel_reference.cpp:174-222), hidden a multiple of 128 up to 4096.
+ * tto_dense_bf16: out[r][n] = bf16(sum_k x[r][k] w[n][k]), fp32 accumulation; a
+ * stand-in for the reference's Q4 projections (no reference counterpart: any
+ * fixed summation order serves, results are compared at tolerance).
+ * tto_add_bf16: bf16(a + b), the residual sum (residual_rms_rounded_sums
+ * kernel_reference.cpp:1160-1165). */
+void tto_rms_only(const uint16_t* input, const uint16_t* weight, uint32_t rows, uint32_t hidden,
+                  uint16_t* output);
+void tto_dense_bf16(const uint16_t* input, const uint16_t* weights, uint32_t rows, uint32_t in_dim,
+                    uint32_t out_dim, uint16_t* output, uint32_t threads);
+void tto_add_bf16(const uint16_t* a, const uint16_t* b, uint64_t count, uint16_t* out);
+
 /* fp64 evaluations used only to pin the algorithms (not reference
  * restatements): sequential delta rule and its chunked WY form for one head.
  * q,k [steps][dk], v [steps][dv], state [dv][dk] (key index contiguous). */

@@ -438,6 +438,7 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
         {tt::kAttentionDecodeKernels, tt::kAttentionDecodeKernelCount},
         {tt::kAttentionPrefillKernels, tt::kAttentionPrefillKernelCount},
         {tt::kAttentionFamilyKernels, tt::kAttentionFamilyKernelCount},
+        {tt::kStackStepKernels, tt::kStackStepKernelCount},
         {tt::kGdnDecodeKernels, tt::kGdnDecodeKernelCount},
         {tt::kGdnPrefillKernels, tt::kGdnPrefillKernelCount},
     };

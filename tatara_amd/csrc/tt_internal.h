@@ -98,6 +98,8 @@ extern const KernelDesc kAttentionPrefillKernels[];
 extern const uint32_t kAttentionPrefillKernelCount;
 extern const KernelDesc kAttentionFamilyKernels[];
 extern const uint32_t kAttentionFamilyKernelCount;
+extern const KernelDesc kStackStepKernels[];
+extern const uint32_t kStackStepKernelCount;
 extern const KernelDesc kGdnDecodeKernels[];
 extern const uint32_t kGdnDecodeKernelCount;
 extern const KernelDesc kGdnPrefillKernels[];

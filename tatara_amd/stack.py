@@ -1,0 +1,260 @@
+"""A stubbed hybrid stack around the attention family, for stacked parity runs and
+context sweeps: `layers` layers in the G,G,G,A pattern at hidden 2048, with the
+reference's Q4/MoE arithmetic replaced by random bf16 dense projections
+(hidden -> 12352 / 9216 in, 4096 -> hidden out) so that only the attention family
+does model-shaped work.  Per layer:
+
+    n = rms_only(x, input_norm);  p = dense(n, W_in)
+    a = GatedDeltaNet(p) | FullAttention(p);  x = x + dense(a, W_out)
+
+and after the last layer  logits = dense(rms_only(x, final_norm), W_vocab).
+
+The walk mirrors the reference's layer loop (src/runtime/decode_step.cpp:1008-1293
+for a token wave over pooled lanes, prefill_step.cpp:1386-2081 for a block of one
+lane): lane state lives in per-layer pools addressed through a state offset table,
+GDN planes ping-pong, attention caches append at the lane's context.
+"""
+import numpy as np
+
+HIDDEN = 2048
+GDN_PROJ = 12352
+ATTN_PROJ = 9216
+CONV_ELEMS = 3 * 8192
+REC_ELEMS = 32 * 128 * 128
+CHUNK_RECORD_BYTES = 115712
+
+
+def layer_kinds(layers):
+    """'G' for Gated DeltaNet, 'A' for full attention: every fourth layer attends."""
+    return ["A" if (i % 4) == 3 else "G" for i in range(layers)]
+
+
+def _bf16(a):
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def make_weights(layers, vocab, seed):
+    """Host-side weights as uint16 bf16 arrays; scales keep the residual stream O(1)."""
+    rng = np.random.default_rng(seed)
+
+    def normal(n, sigma):
+        return _bf16(rng.standard_normal(n, dtype=np.float32) * np.float32(sigma))
+
+    out = {"layers": [], "final_norm": _bf16(1.0 + 0.05 * rng.standard_normal(HIDDEN)),
+           "vocab": normal(vocab * HIDDEN, HIDDEN ** -0.5),
+           "embed": normal(vocab * HIDDEN, 1.0)}
+    for kind in layer_kinds(layers):
+        w = {"kind": kind, "input_norm": _bf16(1.0 + 0.05 * rng.standard_normal(HIDDEN)),
+             "w_out": normal(HIDDEN * 4096, 0.5 * 4096 ** -0.5)}
+        if kind == "G":
+            w["w_in"] = normal(GDN_PROJ * HIDDEN, HIDDEN ** -0.5)
+            w["conv_w"] = normal(4 * 8192, 0.5)
+            w["a_log"] = _bf16(rng.uniform(-4.0, -2.5, 32))
+            w["dt_bias"] = normal(32, 0.3)
+            w["norm_w"] = _bf16(1.0 + 0.1 * rng.standard_normal(128))
+        else:
+            w["w_in"] = normal(ATTN_PROJ * HIDDEN, HIDDEN ** -0.5)
+            w["q_norm"] = _bf16(1.0 + 0.1 * rng.standard_normal(256))
+            w["k_norm"] = _bf16(1.0 + 0.1 * rng.standard_normal(256))
+        out["layers"].append(w)
+    return out
+
+
+class StubStack:
+    """Device side of the stubbed stack: uploads weights, owns the pooled lane
+    state and the scratch, and records token waves and prefill blocks."""
+
+    def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
+                 split_keys=1024):
+        self.dev, self.lib = dev, lib
+        self.lanes, self.capacity, self.vocab = lanes, capacity, vocab
+        self.block_rows = block_rows
+        self.split_keys = split_keys
+        self.max_splits = (capacity + split_keys - 1) // split_keys
+        up = dev.buffer_from
+        self.final_norm = up(weights["final_norm"])
+        self.w_vocab = up(weights["vocab"])
+        self.layers = []
+        self.context = [0] * lanes          # cached positions per lane
+        self.swapped = [False] * lanes      # GDN ping-pong phase per lane
+        stripe = 2 * capacity * 256
+        for w in weights["layers"]:
+            layer = {"kind": w["kind"], "input_norm": up(w["input_norm"]), "w_in": up(w["w_in"]),
+                     "w_out": up(w["w_out"]), "table": dev.create_buffer(256)}
+            if w["kind"] == "G":
+                for name in ("conv_w", "a_log", "dt_bias", "norm_w"):
+                    layer[name] = up(w[name])
+                layer["conv"] = dev.create_buffer(2 * lanes * CONV_ELEMS * 2)
+                layer["rec"] = dev.create_buffer(2 * lanes * REC_ELEMS * 4)
+            else:
+                layer["q_norm"], layer["k_norm"] = up(w["q_norm"]), up(w["k_norm"])
+                layer["keys"] = dev.create_buffer(lanes * stripe * 2)
+                layer["values"] = dev.create_buffer(lanes * stripe * 2)
+            self.layers.append(layer)
+        rows = max(lanes, block_rows)
+        mk = dev.create_buffer
+        self.x = mk(rows * HIDDEN * 2)
+        self.normed = mk(rows * HIDDEN * 2)
+        self.proj = mk(rows * GDN_PROJ * 2)
+        self.mixed = mk(rows * 4096 * 2)
+        self.delta = mk(rows * HIDDEN * 2)
+        self.qk, self.v, self.z, self.y = (mk(rows * 8192) for _ in range(4))
+        self.q, self.gate = mk(rows * 8192), mk(rows * 8192)
+        self.decay, self.beta = mk(rows * 128), mk(rows * 128)
+        self.partials = mk(lanes * 16 * self.max_splits * 258 * 4)
+        self.chunk = mk(((block_rows + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
+        self.logits = mk(rows * vocab * 2)
+        self._write_tables()
+
+    # ---- lane bookkeeping (decode_step.cpp:1044-1060) ----
+    def _gdn_planes(self, lane):
+        a, b = 2 * lane, 2 * lane + 1
+        return (b, a) if self.swapped[lane] else (a, b)   # (in, out)
+
+    def _write_tables(self):
+        stripe = 2 * self.capacity * 256
+        gdn = np.zeros(64, np.uint32)
+        att = np.zeros(64, np.uint32)
+        for lane in range(self.lanes):
+            i, o = self._gdn_planes(lane)
+            gdn[4 * lane:4 * lane + 4] = (i * CONV_ELEMS, o * CONV_ELEMS, i * REC_ELEMS, o * REC_ELEMS)
+            att[4 * lane] = lane * stripe
+            att[4 * lane + 1] = self.context[lane]
+        for layer in self.layers:
+            layer["table"].write(gdn if layer["kind"] == "G" else att)
+
+    # ---- shared steps ----
+    def _dense(self, cb, x, w, out, rows, k, n):
+        cb.encode(self.lib.pipeline("dense_bf16"), {0: x, 1: w, 2: out}, {3: rows, 4: k, 5: n},
+                  ((n + 63) // 64, (rows + 15) // 16), (256,))
+        cb.barrier()
+
+    def _rms(self, cb, x, w, out, rows):
+        cb.encode(self.lib.pipeline("rms_only_ms"), {0: x, 1: w, 2: out}, {3: HIDDEN, 4: HIDDEN},
+                  (1, rows), (HIDDEN // 4,))
+        cb.barrier()
+
+    def _residual(self, cb, rows):
+        n = rows * HIDDEN
+        cb.encode(self.lib.pipeline("add_bf16"), {0: self.x, 1: self.delta, 2: self.x}, {3: n},
+                  ((n + 255) // 256,), (256,))
+        cb.barrier()
+
+    def _head(self, cb, rows):
+        self._rms(cb, self.x, self.final_norm, self.normed, rows)
+        self._dense(cb, self.normed, self.w_vocab, self.logits, rows, HIDDEN, self.vocab)
+
+    # ---- one token for every lane ----
+    def record_token_wave(self, cb, with_head=True):
+        """Records one decode step of all lanes; the lanes' inputs are rows of self.x.
+        Call advance_token_wave() after the recording has been committed."""
+        P, rows = self.lib.pipeline, self.lanes
+        for layer in self.layers:
+            self._rms(cb, self.x, layer["input_norm"], self.normed, rows)
+            if layer["kind"] == "G":
+                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
+                cb.encode(P("gdn_prepare_ms"),
+                          {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: self.qk, 4: self.v,
+                           5: self.z, 6: layer["table"]},
+                          {7: GDN_PROJ, 8: 4096, 9: 4096, 10: 4096}, (96, rows), (128,))
+                cb.barrier()
+                cb.encode(P("gdn_recurrence_ms"),
+                          {0: self.qk, 1: self.v, 2: self.proj, 3: layer["a_log"], 4: layer["dt_bias"],
+                           5: layer["rec"], 6: self.y, 7: layer["table"]},
+                          {8: 4096, 9: 4096, 10: GDN_PROJ, 11: 4096, 12: 32}, (1, 32, 32 * rows),
+                          (32, 4, 1))
+                cb.barrier()
+                cb.encode(P("gdn_gate_norm_ms"), {0: self.y, 1: self.z, 2: layer["norm_w"], 3: self.mixed},
+                          {4: 4096}, (32, rows), (128,))
+            else:
+                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, ATTN_PROJ)
+                cb.encode(P("attn_qk_rope_ms"),
+                          {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,
+                           5: layer["keys"], 6: layer["values"], 8: layer["table"]},
+                          {7: self.capacity, 9: ATTN_PROJ, 10: 4096}, (18, rows), (256,))
+                cb.barrier()
+                cb.encode(P("attention_decode_split_ms"),
+                          {0: self.q, 1: layer["keys"], 2: layer["values"], 3: layer["table"],
+                           4: self.partials},
+                          {5: self.capacity, 6: 4096, 7: self.split_keys, 8: self.max_splits, 9: 0},
+                          (self.max_splits, 2, rows), (256,))
+                cb.barrier()
+                cb.encode(P("attention_decode_combine_ms"),
+                          {0: self.partials, 1: self.gate, 2: layer["table"], 3: self.mixed},
+                          {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
+            cb.barrier()
+            self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
+            self._residual(cb, rows)
+        if with_head:
+            self._head(cb, rows)
+
+    def advance_token_wave(self):
+        """The lanes' GDN planes swap and their contexts grow by one (decode_step.cpp:
+        advance_decode_state); rewrites the state tables."""
+        for lane in range(self.lanes):
+            self.swapped[lane] = not self.swapped[lane]
+            self.context[lane] += 1
+        self._write_tables()
+
+    # ---- a block of rows for one lane ----
+    def record_prefill_block(self, cb, lane, rows, chunked=True, with_head=False):
+        """Records `rows` new tokens of `lane` (inputs are rows of self.x) after its
+        self.context[lane] cached ones.  Call advance_prefill_block(lane, rows) after."""
+        assert 1 <= rows <= self.block_rows and self.context[lane] + rows <= self.capacity
+        P = self.lib.pipeline
+        base = self.context[lane]
+        stripe_bytes = 2 * self.capacity * 256 * 2
+        plane_in, plane_out = self._gdn_planes(lane)
+        for layer in self.layers:
+            self._rms(cb, self.x, layer["input_norm"], self.normed, rows)
+            if layer["kind"] == "G":
+                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
+                conv_in = (layer["conv"], plane_in * CONV_ELEMS * 2)
+                conv_out = (layer["conv"], plane_out * CONV_ELEMS * 2)
+                rec_in = (layer["rec"], plane_in * REC_ELEMS * 4)
+                rec_out = (layer["rec"], plane_out * REC_ELEMS * 4)
+                cb.encode(P("gdn_conv_blk"),
+                          {0: self.proj, 1: conv_in, 2: layer["conv_w"], 3: self.qk, 4: self.v,
+                           5: self.z, 6: conv_out}, {7: rows}, (96, rows), (128,))
+                cb.encode(P("gdn_gates_blk"),
+                          {0: self.proj, 1: layer["a_log"], 2: layer["dt_bias"], 3: self.decay,
+                           4: self.beta}, {5: rows}, (1, (rows + 3) // 4, 1), (32, 4, 1))
+                cb.barrier()
+                if chunked:
+                    chunks = (rows + 63) // 64
+                    cb.encode(P("gdn_chunk_prepare_blk"),
+                              {0: self.qk, 1: self.v, 2: self.decay, 3: self.beta, 4: self.chunk},
+                              {5: rows}, (chunks, 32), (256,))
+                    cb.barrier()
+                    cb.encode(P("gdn_chunk_scan_blk"), {0: self.chunk, 1: rec_in, 2: self.y, 3: rec_out},
+                              {4: rows}, (8, 32), (256,))
+                else:
+                    cb.encode(P("gdn_recurrence_gates_blk"),
+                              {0: self.qk, 1: self.v, 2: self.decay, 3: layer["a_log"], 4: self.beta,
+                               5: rec_in, 6: self.y, 7: rec_out}, {8: rows}, (1, 32, 32), (32, 4, 1))
+                cb.barrier()
+                cb.encode(P("gdn_gate_norm_blk"), {0: self.y, 1: self.z, 2: layer["norm_w"], 3: self.mixed},
+                          {}, (32, rows), (128,))
+            else:
+                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, ATTN_PROJ)
+                keys = (layer["keys"], lane * stripe_bytes)
+                values = (layer["values"], lane * stripe_bytes)
+                cb.encode(P("attn_qk_rope_blk"),
+                          {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,
+                           5: keys, 6: values}, {7: base, 8: self.capacity}, (18, rows), (256,))
+                cb.barrier()
+                cb.encode(P("attention_flash_v2_blk"),
+                          {0: self.q, 1: keys, 2: values, 3: self.gate, 4: self.mixed},
+                          {5: base + rows, 6: self.capacity, 7: rows, 8: base},
+                          (16, (rows + 15) // 16), (256,))
+            cb.barrier()
+            self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
+            self._residual(cb, rows)
+        if with_head:
+            self._head(cb, rows)
+
+    def advance_prefill_block(self, lane, rows):
+        self.swapped[lane] = not self.swapped[lane]
+        self.context[lane] += rows
+        self._write_tables()

@@ -1,0 +1,119 @@
+"""Stacked run of the hybrid 40-layer stub stack (3 GDN : 1 full attention,
+hidden 2048, random bf16 dense projections in place of the Q4/MoE arithmetic) on
+the GPU against the same stack evaluated with the CPU checker: block prefill of two
+lanes with ragged lengths, then greedy decode waves of both lanes through the
+pooled-state operators.  Judged by greedy argmax agreement on the final logits at
+every step.  The per-operator tolerance (max-abs 2e-2, mean-abs 2e-3) is held by
+the single-layer tests; forty layers of bf16 re-rounding put the two evaluations of
+the final logits (bf16, one step = 1.6e-2 at |x| in [2, 4)) a step or two apart, so
+here the logits only have to stay within a loose sanity band."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_util import gpu
+
+pytestmark = pytest.mark.gpu
+o = ol.oracle
+THREADS = 16
+
+
+class OracleLane:
+    """One lane of the stack on the CPU checker."""
+
+    def __init__(self, weights, capacity, vocab):
+        self.w, self.cap, self.vocab = weights, capacity, vocab
+        self.context = 0
+        self.state = []
+        for lw in weights["layers"]:
+            if lw["kind"] == "G":
+                self.state.append({"conv": np.zeros(3 * 8192, np.uint16),
+                                   "rec": np.zeros(32 * 128 * 128, np.float32)})
+            else:
+                self.state.append({"keys": np.zeros(2 * capacity * 256, np.uint16),
+                                   "values": np.zeros(2 * capacity * 256, np.uint16)})
+
+    def block(self, x, rows):
+        """Runs `rows` tokens (x: [rows*2048] bf16); returns logits of every row."""
+        x = x.copy()
+        for lw, st in zip(self.w["layers"], self.state):
+            n = np.zeros(rows * 2048, np.uint16)
+            o.tto_rms_only(x, lw["input_norm"], rows, 2048, n)
+            if lw["kind"] == "G":
+                p = np.zeros(rows * 12352, np.uint16)
+                o.tto_dense_bf16(n, lw["w_in"], rows, 2048, 12352, p, THREADS)
+                conv = np.zeros_like(st["conv"]); rec = np.zeros_like(st["rec"])
+                a = np.zeros(rows * 4096, np.uint16)
+                scratch = [np.zeros(rows * 4096, np.uint16) for _ in range(3)]
+                o.tto_gdn_prefill(p, rows, st["conv"], lw["conv_w"], lw["a_log"], lw["dt_bias"],
+                                  lw["norm_w"], st["rec"], conv, rec, a, *scratch, THREADS)
+                st["conv"], st["rec"] = conv, rec
+            else:
+                p = np.zeros(rows * 9216, np.uint16)
+                o.tto_dense_bf16(n, lw["w_in"], rows, 2048, 9216, p, THREADS)
+                q = np.zeros(rows * 4096, np.uint16); g = np.zeros_like(q); a = np.zeros_like(q)
+                sel = np.arange(rows, dtype=np.uint32)
+                o.tto_attention_prefill(p, lw["q_norm"], lw["k_norm"], rows, self.context, self.cap,
+                                        q, g, st["keys"], st["values"], sel, rows, a, THREADS)
+            d = np.zeros(rows * 2048, np.uint16)
+            o.tto_dense_bf16(a, lw["w_out"], rows, 4096, 2048, d, THREADS)
+            o.tto_add_bf16(x, d, rows * 2048, x)
+        self.context += rows
+        n = np.zeros(rows * 2048, np.uint16)
+        o.tto_rms_only(x, self.w["final_norm"], rows, 2048, n)
+        logits = np.zeros(rows * self.vocab, np.uint16)
+        o.tto_dense_bf16(n, self.w["vocab"], rows, 2048, self.vocab, logits, THREADS)
+        return ol.bf16_to_f32(logits).reshape(rows, self.vocab)
+
+
+def _compare(step, got, want):
+    err = np.abs(got - want)
+    top2 = np.sort(want)[-2:]
+    print(f"[parity] {step}: logits max-abs {err.max():.3e} mean-abs {err.mean():.3e} "
+          f"argmax {got.argmax()} / {want.argmax()} top-2 gap {top2[1] - top2[0]:.3e}", flush=True)
+    assert np.isfinite(got).all()
+    assert err.mean() <= 2e-2 * max(1.0, np.abs(want).max())
+    assert got.argmax() == want.argmax(), step
+
+
+def test_stacked_prefill_and_greedy_decode_match_the_checker():
+    print("[case] 40-layer stub stack: prefill 2 lanes + 3 greedy decode waves", flush=True)
+    from tatara_amd import stack as S
+    B, dev, queue, lib = gpu()
+    layers, vocab, capacity, lanes = 40, 4096, 128, 2
+    weights = S.make_weights(layers, vocab, 0x57AC)
+    embed = weights["embed"].reshape(vocab, 2048)
+    gpu_stack = S.StubStack(dev, lib, weights, lanes, capacity, vocab, block_rows=64, split_keys=64)
+    cpu_lanes = [OracleLane(weights, capacity, vocab) for _ in range(lanes)]
+    rng = np.random.default_rng(5)
+    prompts = [rng.integers(0, vocab, 24), rng.integers(0, vocab, 9)]
+    tokens = []
+    for lane, prompt in enumerate(prompts):
+        rows = len(prompt)
+        x = np.ascontiguousarray(embed[prompt]).reshape(-1)
+        gpu_stack.x.write(x)
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        gpu_stack.record_prefill_block(cb, lane, rows, chunked=True, with_head=True)
+        cb.end_compute_pass()
+        cb.commit().wait()
+        gpu_stack.advance_prefill_block(lane, rows)
+        got = ol.bf16_to_f32(gpu_stack.logits.read(np.uint16, rows * vocab)).reshape(rows, vocab)
+        want = cpu_lanes[lane].block(x, rows)
+        _compare(f"prefill lane {lane} last row", got[-1], want[-1])
+        tokens.append(int(want[-1].argmax()))
+    for step in range(3):
+        x = np.ascontiguousarray(embed[tokens]).reshape(-1)
+        gpu_stack.x.write(x)
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        gpu_stack.record_token_wave(cb)
+        cb.end_compute_pass()
+        cb.commit().wait()
+        gpu_stack.advance_token_wave()
+        got = ol.bf16_to_f32(gpu_stack.logits.read(np.uint16, lanes * vocab)).reshape(lanes, vocab)
+        for lane in range(lanes):
+            want = cpu_lanes[lane].block(np.ascontiguousarray(x[lane * 2048:(lane + 1) * 2048]), 1)
+            _compare(f"decode step {step} lane {lane}", got[lane], want[0])
+            tokens[lane] = int(want[0].argmax())
+    assert gpu_stack.context == [24 + 3, 9 + 3]

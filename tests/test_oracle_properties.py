@@ -347,3 +347,31 @@ def test_scan_matches_fp64_sequential_within_tolerance():
                              st, y64)
     assert np.abs(F(y).reshape(steps, 32, 128)[:, h] - y64).max() < 2e-3
     assert np.abs(s1.reshape(32, 128, 128)[h] - st).max() < 1e-4
+
+
+def test_dense_and_add_against_float64():
+    """The stand-in projection is a plain dot product rounded once to bf16 and the
+    residual sum is one bf16 addition: both against float64 numpy."""
+    rows, k, n = 3, 256, 40
+    x = ol.gaussian_bf16(0xD0, rows * k)
+    w = ol.gaussian_bf16(0xD1, n * k, 0.0, 0.05)
+    out = np.zeros(rows * n, np.uint16)
+    o.tto_dense_bf16(x, w, rows, k, n, out, 4)
+    want = F(x).astype(np.float64).reshape(rows, k) @ F(w).astype(np.float64).reshape(n, k).T
+    got = F(out).reshape(rows, n)
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 1e-6).all()
+    a = ol.gaussian_bf16(0xD2, 1000); b = ol.gaussian_bf16(0xD3, 1000)
+    s = np.zeros(1000, np.uint16)
+    o.tto_add_bf16(a, b, 1000, s)
+    assert np.array_equal(s, ol.f32_to_bf16(F(a) + F(b)))
+
+
+def test_rms_only_closed_forms():
+    # ones -> ones; uniform 2.0 over 2048 -> 2 / sqrt(4 + 1e-6) rounded twice
+    ones = np.full(2048, 0x3F80, np.uint16)
+    out = np.zeros(2048, np.uint16)
+    o.tto_rms_only(ones, ones, 1, 2048, out)
+    assert (out == 0x3F80).all()
+    twos = np.full(2048, 0x4000, np.uint16)
+    o.tto_rms_only(twos, ones, 1, 2048, out)
+    assert (out == 0x3F80).all()

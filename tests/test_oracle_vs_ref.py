@@ -75,3 +75,20 @@ def test_gdn_stages(seed):
                     so.view(np.uint32), out))
     for x, y in zip(*res):
         assert np.array_equal(x, y)
+
+
+@pytest.mark.parametrize("hidden", [256, 2048, 4096])
+@pytest.mark.parametrize("kind", ["banded", "gauss"])
+def test_rms_only_rows(hidden, kind):
+    """tto_rms_only against rms_only_reference (AdjacentPairs tree = 1,
+    1/sqrt = order 0), three rows at once."""
+    rows = 3
+    x = (ol.banded_bf16(0x515 + hidden, rows * hidden) if kind == "banded"
+         else ol.gaussian_bf16(0x516 + hidden, rows * hidden, 0.0, 3.0))
+    w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0x517, hidden))
+    got = np.zeros(rows * hidden, np.uint16)
+    o.tto_rms_only(x, w, rows, hidden, got)
+    for row in range(rows):
+        want = np.zeros(hidden, np.uint16)
+        r.ref_rms_only(np.ascontiguousarray(x[row * hidden:(row + 1) * hidden]), w, hidden, 1, 0, want)
+        assert np.array_equal(got[row * hidden:(row + 1) * hidden], want)
