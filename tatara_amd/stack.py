@@ -61,16 +61,26 @@ def make_weights(layers, vocab, seed):
     return out
 
 
+def choose_split_keys(lanes, capacity):
+    """Keys per split-K workgroup so that one attention layer of a token wave fills
+    the 256 compute units about once: splits * 2 kv heads * lanes ~ 256, between 128
+    and 1024 keys, a multiple of 32."""
+    keys = (capacity * 2 * lanes + 255) // 256
+    keys = ((keys + 31) // 32) * 32
+    return max(128, min(1024, keys))
+
+
 class StubStack:
     """Device side of the stubbed stack: uploads weights, owns the pooled lane
     state and the scratch, and records token waves and prefill blocks."""
 
     def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
-                 split_keys=1024):
+                 split_keys=None):
         self.dev, self.lib = dev, lib
         self.lanes, self.capacity, self.vocab = lanes, capacity, vocab
         self.block_rows = block_rows
-        self.split_keys = split_keys
+        self.split_keys = split_keys or choose_split_keys(lanes, capacity)
+        split_keys = self.split_keys
         self.max_splits = (capacity + split_keys - 1) // split_keys
         up = dev.buffer_from
         self.final_norm = up(weights["final_norm"])
