@@ -4,7 +4,7 @@
 A step is one decode token wave of 4 lanes at 32768 visible keys through one
 hybrid period of the layer stack, G,G,G,A (three Gated DeltaNet layers, one
 full-attention layer), with the lane-batched operators:
-    GDN:       gdn_prepare_ms -> gdn_recurrence_ms -> gdn_gate_norm_ms
+    GDN:       gdn_decode_fused_ms (prepare + recurrence + gate-norm in one dispatch)
     attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms
 Projections (the reference's Q4 GEMVs) are not on the path: their outputs are
 resident random bf16 slabs.  KV caches, GDN state and all scratch are in HBM
@@ -102,25 +102,16 @@ def build_workload(B, dev, lib, torch, PART):
                                proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
                                a_log=from_np(a_log), dt_bias=from_np(dt_bias),
                                norm_w=from_np(np.full(128, 0x3F80, np.uint16))))
-    g_qk, g_v, g_z, g_y, g_out = (dev.create_buffer(rows * 8192) for _ in range(5))
+    g_out = dev.create_buffer(rows * 8192)
 
     P = lib.pipeline
 
     def record(cb, copy):
         for layer in gdn_layers:
-            cb.encode(P("gdn_prepare_ms"),
-                      {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: g_qk, 4: g_v,
-                       5: g_z, 6: layer["table"]},
-                      {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, rows), (128,))
-            cb.barrier()
-            cb.encode(P("gdn_recurrence_ms"),
-                      {0: g_qk, 1: g_v, 2: layer["proj"], 3: layer["a_log"], 4: layer["dt_bias"],
-                       5: layer["rec"], 6: g_y, 7: layer["table"]},
-                      {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32 * rows),
-                      (32, 4, 1))
-            cb.barrier()
-            cb.encode(P("gdn_gate_norm_ms"), {0: g_y, 1: g_z, 2: layer["norm_w"], 3: g_out},
-                      {4: 4096}, (32, rows), (128,))
+            cb.encode(P("gdn_decode_fused_ms"),
+                      {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
+                       4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: g_out,
+                       8: layer["table"]}, {9: 12352, 10: 4096}, (32, rows), (512,))
             cb.barrier()
         keys, values = kv[copy]
         cb.encode(P("attn_qk_rope_ms"),
@@ -280,8 +271,7 @@ def main():
     achieved = algo_bytes / (split_us * 1e-6) / 1e9
     attn_layer_us = sum(kernel_us[k] for k in ("attn_qk_rope_ms", "attention_decode_split_ms",
                                                "attention_decode_combine_ms"))
-    gdn_layer_us = sum(kernel_us[k] for k in ("gdn_prepare_ms", "gdn_recurrence_ms",
-                                              "gdn_gate_norm_ms"))
+    gdn_layer_us = kernel_us["gdn_decode_fused_ms"]
     gdn_gbs = LANES * GDN_BYTES_PER_LANE_LAYER / (gdn_layer_us * 1e-6) / 1e9
 
     line = {

@@ -196,6 +196,7 @@ DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::gdn_prepare_ms, "gdn_prepare_ms", error) &&
         resolve(library, p, &P::gdn_recurrence_ms, "gdn_recurrence_ms", error) &&
         resolve(library, p, &P::gate_norm_ms, "gdn_gate_norm_ms", error) &&
+        resolve(library, p, &P::gdn_decode_fused_ms, "gdn_decode_fused_ms", error) &&
         resolve(library, p, &P::attn_qk_rope_ms, "attn_qk_rope_ms", error) &&
         resolve(library, p, &P::attention_decode_ms, "attention_decode_ms", error) &&
         resolve(library, p, &P::attention_split_ms, "attention_decode_split_ms", error) &&
@@ -491,7 +492,21 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
         walk.barrier();
         walk.hook(hooks.project, hooks.user, layer, kind, rows);
         walk.barrier();
-        if (is_gated(kind)) {
+        if (is_gated(kind) && batch.gdn_fused) {
+            walk.pipeline(k.gdn_decode_fused_ms);
+            walk.buffer(batch.gdn_projection, 0, 0);
+            walk.buffer(pool.layers[layer].first, 0, 1);
+            walk.weight(w.conv_weight, 2);
+            walk.weight(w.a_log, 3);
+            walk.weight(w.dt_bias, 4);
+            walk.buffer(pool.layers[layer].second, 0, 5);
+            walk.weight(w.norm_weight, 6);
+            walk.buffer(batch.gdn_gated, 0, 7);
+            walk.buffer(batch.state_offsets, layer * 256, 8);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_projection_bytes / 2), 9);
+            walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 10);
+            walk.dispatch(HipSize{g.gdn_recurrence.head_groups, rows, 1}, HipSize{512, 1, 1});
+        } else if (is_gated(kind)) {
             walk.pipeline(k.gdn_prepare_ms);
             walk.buffer(batch.gdn_projection, 0, 0);
             walk.buffer(pool.layers[layer].first, 0, 1);

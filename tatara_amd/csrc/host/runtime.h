@@ -162,7 +162,7 @@ struct DecodePipelines {
     HipComputePipeline gdn_prepare, gdn_recurrence, gdn_gate_norm;
     HipComputePipeline attn_qk_rope, attention_decode, attention_scores_values_fused,
         attention_combine;
-    HipComputePipeline gdn_prepare_ms, gdn_recurrence_ms, gate_norm_ms;
+    HipComputePipeline gdn_prepare_ms, gdn_recurrence_ms, gate_norm_ms, gdn_decode_fused_ms;
     HipComputePipeline attn_qk_rope_ms, attention_decode_ms, attention_split_ms,
         attention_combine_ms;
 };
@@ -183,6 +183,9 @@ struct DecodeBatchScratch {
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended, attn_partials;
     HipBuffer state_offsets;
     std::uint32_t split_keys{1024};      // keys per split-K workgroup of the batched path
+    // One dispatch per Gated DeltaNet layer (gdn_decode_fused_ms) instead of the
+    // reference's prepare / recurrence / gate-norm triple; same results bit for bit.
+    bool gdn_fused{true};
 };
 
 // The step: geometry, schedule and pipelines; its own primary slot (decode_step.h:115-153).

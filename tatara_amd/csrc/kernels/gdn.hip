@@ -286,6 +286,157 @@ __global__ __launch_bounds__(128) void gdn_gate_norm_kernel(const uint16_t* y, c
     out[at] = narrow((g * sig) * normed);
 }
 
+// ------------------------------------------------- fused decode step ---------
+
+struct FusedDecodeArgs {
+    const uint16_t* projection;    // [rows][projection_stride]
+    const uint16_t* conv_pool;     // planes addressed through the table
+    uint16_t* conv_pool_out;
+    const uint16_t* conv_weights;  // [8192][4]
+    const uint16_t* a_log;
+    const uint16_t* dt_bias;
+    const float* rec_pool;
+    float* rec_pool_out;
+    const uint16_t* norm_weight;   // [128]
+    uint16_t* out;                 // [rows][out_stride]
+    const uint32_t* table;         // per row {conv_in, conv_out, rec_in, rec_out} element offsets
+    uint32_t projection_stride, out_stride;
+};
+
+// One decode step of a whole value head in one workgroup: conv + SiLU of the
+// head's q, k and v channels, q/k norms, gates, the delta-rule update of the
+// head's 128 x 128 state and the gate-norm of its 128 outputs, with the
+// arithmetic of gdn_prepare / gdn_recurrence / gdn_gate_norm operation for
+// operation (so the results are theirs bit for bit) and none of their
+// intermediates in memory.  grid (32 heads, rows) x 512: sixteen half waves, each
+// walking 8 state rows with 4 key columns per lane.  The two value heads that
+// share a key head both evaluate its q/k channels; the even one writes their new
+// conv history.
+__global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a) {
+    __shared__ float act[3 * kGD];      // activated q | k | v channels (bf16 values)
+    __shared__ float qk_n[2 * kGD];     // normalised, scaled q | k (bf16 values)
+    __shared__ float y_head[kGD];       // bf16 values of the head's outputs
+    __shared__ float inverse[2];
+    __shared__ float gates[2];
+    __shared__ float partial[2];
+    const uint32_t h = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t kh = h >> 1;
+    const uint32_t tid = threadIdx.x;
+    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const uint16_t* conv_in = a.conv_pool + a.table[row * 4];
+    uint16_t* conv_out = a.conv_pool_out + a.table[row * 4 + 1];
+    const float* state_in = a.rec_pool + a.table[row * 4 + 2];
+    float* state_out = a.rec_pool_out + a.table[row * 4 + 3];
+    const uint32_t half = tid >> 5;  // 0..15
+    const uint32_t lane = tid & 31;
+    // the state rows this half wave walks are requested first: their 64 KiB per head
+    // arrive while the conv, norm and gate stages run
+    f32x4 st[8];
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) {
+        const uint32_t j = half * 8 + it;
+        st[it] = *reinterpret_cast<const f32x4*>(
+            state_in + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4);
+    }
+    const uint16_t z_bits = tid < kGD ? proj[kCh + h * kGD + tid] : uint16_t{0};
+    const uint16_t norm_bits = tid < kGD ? a.norm_weight[tid] : uint16_t{0};
+
+    if (tid < 3 * kGD) {
+        const uint32_t part = tid >> 7;  // 0 q, 1 k, 2 v
+        const uint32_t c = (part == 0 ? kh * kGD : part == 1 ? kGdnKOffset + kh * kGD
+                                                             : kGdnQkValues + h * kGD) + (tid & 127);
+        const uint16_t t0 = conv_in[c], t1 = conv_in[kCh + c], t2 = conv_in[2 * kCh + c];
+        const uint16_t t3 = proj[c];
+        const uint16_t* w = a.conv_weights + static_cast<uint64_t>(c) * 4;
+        const float convolved = widen(w[0]) * widen(t0) + widen(w[1]) * widen(t1) +
+                                widen(w[2]) * widen(t2) + widen(w[3]) * widen(t3);
+        const float conv_b = rb(convolved);
+        act[tid] = rb(conv_b * sigmoid_bf16(conv_b));
+        if (part == 2 || (h & 1) == 0) {
+            conv_out[c] = t1;
+            conv_out[kCh + c] = t2;
+            conv_out[2 * kCh + c] = t3;
+        }
+    } else if (tid == 3 * kGD) {
+        float decay, beta;
+        head_gates(proj[kGdnARowOffset + h], proj[kGdnBRowOffset + h], a.a_log[h], a.dt_bias[h],
+                   decay, beta);
+        gates[0] = decay;
+        gates[1] = beta;
+    }
+    __syncthreads();
+    if (tid < 64) {  // lanes 0..31: q head, 32..63: k head; lane l sums squares 4l..4l+3
+        const float* v = act + (tid >> 5) * kGD + (tid & 31) * 4;
+        float sum = ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3];
+        for (uint32_t off = 1; off < 32; off <<= 1) sum += __shfl_xor(sum, off, 64);
+        if ((tid & 31) == 0) {
+            inverse[tid >> 5] = 1.0f / sqrtf(sum / static_cast<float>(kGD) + kRmsNormEpsilon);
+        }
+    }
+    __syncthreads();
+    if (tid < 2 * kGD) {
+        const float scale = widen(tid < kGD ? kGdnQueryScaleBits : kGdnKeyScaleBits);
+        qk_n[tid] = rb(rb(act[tid] * inverse[tid >> 7]) * scale);
+    }
+    __syncthreads();
+
+    const float decay = gates[0];
+    const float beta = gates[1];
+    float q4[4], k4[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        q4[i] = qk_n[lane * 4 + i];
+        k4[i] = qk_n[kGD + lane * 4 + i];
+    }
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) {
+        const uint32_t j = half * 8 + it;
+        float kv = 0.0f;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            st[it][i] *= decay;
+            kv = fmaf(st[it][i], k4[i], kv);
+        }
+        kv = half_wave_sum(kv);
+        const float delta = (act[2 * kGD + j] - kv) * beta;
+        float out = 0.0f;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            st[it][i] = fmaf(k4[i], delta, st[it][i]);
+            out = fmaf(st[it][i], q4[i], out);
+        }
+        out = half_wave_sum(out);
+        *reinterpret_cast<f32x4*>(state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4) =
+            st[it];
+        if (lane == 0) y_head[j] = rb(out);
+    }
+    __syncthreads();
+    if (tid < kGD) {
+        const float v = y_head[tid];
+        const float sq = v * v;
+        const float s1 = __shfl_down(sq, 1, 64);
+        const float s2 = __shfl_down(sq, 2, 64);
+        const float s3 = __shfl_down(sq, 3, 64);
+        const float four = ((sq + s1) + s2) + s3;
+        const uint32_t wl = tid & 63;
+        float t = __shfl(four, (wl & 15) * 4, 64);
+        for (uint32_t off = 1; off < 16; off <<= 1) t += __shfl_xor(t, off, 64);
+        if (wl == 0) partial[tid >> 6] = t;
+    }
+    __syncthreads();
+    if (tid < kGD) {
+        const float v = y_head[tid];
+        const float inv =
+            1.0f / sqrtf((partial[0] + partial[1]) / static_cast<float>(kGD) + kRmsNormEpsilon);
+        const float normed = rb(widen(norm_bits) * rb(v * inv));
+        const float g = widen(z_bits);
+        const float low = 1.0f / (1.0f + expf(fabsf(g)));
+        const float sig = g < 0.0f ? low : 1.0f - low;
+        a.out[static_cast<uint64_t>(row) * a.out_stride + h * kGD + tid] = narrow((g * sig) * normed);
+    }
+}
+
 // ------------------------------------------- chunked (WY) block prefill ------
 //
 // The reference walks a block token by token (prefill_gdn.metal:204-281).  The
@@ -933,6 +1084,44 @@ int32_t op_gdn_recurrence_ms(const Bindings& b, const Grid& g, hipStream_t strea
     return launch_recurrence(r, rows, stream);
 }
 
+// gdn_decode_fused_ms (no reference counterpart: gdn_prepare_ms + gdn_recurrence_ms
+// + gdn_gate_norm_ms of decode_step.cpp:1116-1211 in one dispatch): b0 projection
+// slab, b1 conv pool, b2 conv weights, b3 a_log, b4 dt_bias, b5 recurrent pool,
+// b6 norm weight, b7 gated output slab, b8 state table, c9 projection stride,
+// c10 output stride; grid (32, rows) x 512.
+int32_t op_gdn_decode_fused_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                               bool validate_only) {
+    Args a(b);
+    FusedDecodeArgs f{};
+    f.projection_stride = a.constant(9);
+    f.out_stride = a.constant(10);
+    a.require(g.gx == kGdnValueHeads && g.gy >= 1 && g.gy <= kMaxBatchRows && g.gz == 1 &&
+                  g.tx == 512 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(f.projection_stride >= kGdnProjectionRows && f.out_stride >= kGdnValueValues,
+              TT_CMD_INVALID_BUFFER);
+    if (a.status != TT_OK) return a.status;
+    const uint32_t rows = static_cast<uint32_t>(g.gy);
+    const uint64_t last = rows - 1;
+    f.projection =
+        a.buffer<const uint16_t>(0, (last * f.projection_stride + kGdnProjectionRows) * 2);
+    uint16_t* conv = a.buffer<uint16_t>(1, 2ull * 3 * kCh * 2);
+    f.conv_pool = conv;
+    f.conv_pool_out = conv;
+    f.conv_weights = a.buffer<const uint16_t>(2, 4ull * kCh * 2);
+    f.a_log = a.buffer<const uint16_t>(3, kGdnValueHeads * 2);
+    f.dt_bias = a.buffer<const uint16_t>(4, kGdnValueHeads * 2);
+    float* rec = a.buffer<float>(5, 2 * kStateBytes);
+    f.rec_pool = rec;
+    f.rec_pool_out = rec;
+    f.norm_weight = a.buffer<const uint16_t>(6, kGD * 2);
+    f.out = a.buffer<uint16_t>(7, (last * f.out_stride + kGdnValueValues) * 2);
+    f.table = a.buffer<const uint32_t>(8, rows * 16);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(gdn_decode_fused_kernel, dim3(kGdnValueHeads, rows), dim3(512), 0, stream, f);
+    return TT_OK;
+}
+
 // gdn_gates_blk: b0 projection, b1 a_log, b2 dt_bias, b3 decay[rows][32],
 // b4 beta[rows][32], c5 rows; grid (1, ceil(rows/4)) x (32, 4)
 // (prefill_step.cpp:1989-2001).
@@ -1100,6 +1289,7 @@ const KernelDesc kGdnDecodeKernels[] = {
     {"gdn_recurrence_ms", op_gdn_recurrence_ms},
     {"gdn_gate_norm", op_gdn_gate_norm},
     {"gdn_gate_norm_ms", op_gdn_gate_norm_ms},
+    {"gdn_decode_fused_ms", op_gdn_decode_fused_ms},
 };
 const uint32_t kGdnDecodeKernelCount = sizeof(kGdnDecodeKernels) / sizeof(kGdnDecodeKernels[0]);
 

@@ -164,19 +164,10 @@ class StubStack:
             self._rms(cb, self.x, layer["input_norm"], self.normed, rows)
             if layer["kind"] == "G":
                 self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
-                cb.encode(P("gdn_prepare_ms"),
-                          {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: self.qk, 4: self.v,
-                           5: self.z, 6: layer["table"]},
-                          {7: GDN_PROJ, 8: 4096, 9: 4096, 10: 4096}, (96, rows), (128,))
-                cb.barrier()
-                cb.encode(P("gdn_recurrence_ms"),
-                          {0: self.qk, 1: self.v, 2: self.proj, 3: layer["a_log"], 4: layer["dt_bias"],
-                           5: layer["rec"], 6: self.y, 7: layer["table"]},
-                          {8: 4096, 9: 4096, 10: GDN_PROJ, 11: 4096, 12: 32}, (1, 32, 32 * rows),
-                          (32, 4, 1))
-                cb.barrier()
-                cb.encode(P("gdn_gate_norm_ms"), {0: self.y, 1: self.z, 2: layer["norm_w"], 3: self.mixed},
-                          {4: 4096}, (32, rows), (128,))
+                cb.encode(P("gdn_decode_fused_ms"),
+                          {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
+                           4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: self.mixed,
+                           8: layer["table"]}, {9: GDN_PROJ, 10: 4096}, (32, rows), (512,))
             else:
                 self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, ATTN_PROJ)
                 cb.encode(P("attn_qk_rope_ms"),

@@ -172,3 +172,66 @@ def test_config2_four_lanes_batched():
         p, cs, st = _lane_inputs(r)
         assert np.array_equal(conv_pool.read(np.uint16, 3 * 8192,
                                              (2 * stripes[r] + par) * conv_stride), cs)
+
+
+def test_fused_decode_step_equals_the_three_operators():
+    """gdn_decode_fused_ms against gdn_prepare_ms + gdn_recurrence_ms +
+    gdn_gate_norm_ms on the same pooled lanes: bit-identical outputs and state
+    planes, and the checker's bar on top."""
+    print("[case] gdn fused decode step x4 lanes", flush=True)
+    B, dev, queue, lib = gpu()
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    b_w, b_al, b_dt, b_nw = (dev.buffer_from(x) for x in (conv_w, a_log, dt_bias, norm_w))
+    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
+    swapped = [False, True, True, False]
+    proj = np.zeros((LANES, 12352), np.uint16)
+    conv0 = np.zeros(2 * LANES * conv_elems, np.uint16)
+    rec0 = np.zeros(2 * LANES * rec_elems, np.float32)
+    table = np.zeros(64, np.uint32)
+    want = []
+    for r in range(LANES):
+        p, cs, st = _lane_inputs(r)
+        proj[r] = p
+        i, o_ = (2 * r + 1, 2 * r) if swapped[r] else (2 * r, 2 * r + 1)
+        conv0[i * conv_elems:(i + 1) * conv_elems] = cs
+        rec0[i * rec_elems:(i + 1) * rec_elems] = st
+        table[4 * r:4 * r + 4] = (i * conv_elems, o_ * conv_elems, i * rec_elems, o_ * rec_elems)
+        gated = np.zeros(4096, np.uint16)
+        ncs = np.zeros(conv_elems, np.uint16); so = np.zeros(rec_elems, np.float32)
+        o.tto_gdn_decode_step(p, cs, conv_w, a_log, dt_bias, norm_w, st, ncs, so, gated, 8)
+        want.append(gated)
+    b_tab, b_proj = dev.buffer_from(table), dev.buffer_from(proj)
+    pools = [(dev.buffer_from(conv0), dev.buffer_from(rec0)) for _ in range(2)]
+    b_qk, b_v, b_z, b_y = (dev.create_buffer(LANES * 8192) for _ in range(4))
+    outs = [dev.create_buffer(LANES * 8192) for _ in range(2)]
+
+    def rec(cb):
+        conv, rec_ = pools[0]
+        cb.encode(lib.pipeline("gdn_prepare_ms"),
+                  {0: b_proj, 1: conv, 2: b_w, 3: b_qk, 4: b_v, 5: b_z, 6: b_tab},
+                  {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, LANES), (128,))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_recurrence_ms"),
+                  {0: b_qk, 1: b_v, 2: b_proj, 3: b_al, 4: b_dt, 5: rec_, 6: b_y, 7: b_tab},
+                  {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32 * LANES), (32, 4, 1))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_gate_norm_ms"), {0: b_y, 1: b_z, 2: b_nw, 3: outs[0]}, {4: 4096},
+                  (32, LANES), (128,))
+        conv, rec_ = pools[1]
+        cb.encode(lib.pipeline("gdn_decode_fused_ms"),
+                  {0: b_proj, 1: conv, 2: b_w, 3: b_al, 4: b_dt, 5: rec_, 6: b_nw, 7: outs[1],
+                   8: b_tab}, {9: 12352, 10: 4096}, (32, LANES), (512,))
+    run(rec)
+    assert np.array_equal(outs[0].read(np.uint16), outs[1].read(np.uint16))
+    assert np.array_equal(pools[0][0].read(np.uint16), pools[1][0].read(np.uint16))
+    assert np.array_equal(pools[0][1].read(np.float32), pools[1][1].read(np.float32))
+    got = outs[1].read(np.uint16).reshape(LANES, 4096)
+    for r in range(LANES):
+        check_bf16(got[r], want[r], f"fused lane {r} gated")
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    with pytest.raises(B.BackendError) as e:
+        cb.encode(lib.pipeline("gdn_decode_fused_ms"),
+                  {0: b_proj, 1: pools[0][0], 2: b_w, 3: b_al, 4: b_dt, 5: pools[0][1], 6: b_nw,
+                   7: outs[1], 8: b_tab}, {9: 12352, 10: 4096}, (32, 17), (512,))
+    assert e.value.status == 15
