@@ -12,6 +12,10 @@ before the timed region; two copies of the attention layer's KV pools (537 MB in
 total) alternate from step to step so the 256 MB last-level cache cannot serve
 the stream.  The step is compiled into a HIP graph and replayed.
 
+`detail.prefill_16k` adds the block-prefill side of the metric: 16384 new tokens of
+one lane through a full-attention layer (causal flash attention on MFMA) and a
+Gated DeltaNet layer (chunk-64 recurrence on MFMA), tok/s and fraction of MFMA peak.
+
 Prints ONE JSON line: `value` = microseconds per layer over the period,
 `roofline` for the dominant kernel (the split-K flash-decode), `cpu_baseline` =
 the CPU checker timed on this box's host cores on the same period."""
@@ -137,6 +141,82 @@ def build_workload(B, dev, lib, torch, PART):
     return record, record_split_only, keep
 
 
+def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
+    """Block prefill of `rows` new tokens into an empty cache, one lane, resident
+    random inputs: the causal flash attention kernel (rope stage timed beside it) and
+    the chunk-64 Gated DeltaNet recurrence (conv, gates and gate-norm beside it).
+    Per-command device time, best of `repeats`."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0xF1A5)
+    keep = []
+
+    def rb(n, sigma=1.0):
+        t = (torch.randn(n, generator=gen, device="cuda") * sigma).to(torch.bfloat16)
+        keep.append(t)
+        return dev.wrap(t.data_ptr(), n * 2, keepalive=t)
+
+    P = lib.pipeline
+    mk = dev.create_buffer
+    # attention layer
+    a_proj = rb(rows * 9216)
+    ones = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
+    q, gate, out = mk(rows * 8192), mk(rows * 8192), mk(rows * 8192)
+    keys, values = mk(2 * rows * 256 * 2), mk(2 * rows * 256 * 2)
+    # GDN layer
+    g_proj = rb(rows * 12352, 0.5)
+    conv_w = rb(4 * 8192, 0.5)
+    rng = np.random.default_rng(3)
+    a_log = dev.buffer_from((rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16)
+                            .astype(np.uint16))
+    dt_bias = dev.buffer_from(np.zeros(32, np.uint16))
+    norm_w = dev.buffer_from(np.full(128, 0x3F80, np.uint16))
+    conv_in, conv_out = mk(3 * 8192 * 2), mk(3 * 8192 * 2)
+    rec = mk(32 * 128 * 128 * 4)
+    qk, v, z, y, gated = (mk(rows * 8192) for _ in range(5))
+    decay, beta = mk(rows * 128), mk(rows * 128)
+    chunks = (rows + 63) // 64
+    chunk = mk(chunks * 32 * 115712)
+    best = {}
+    for _ in range(repeats):
+        cb = queue.create_command_buffer()
+        cb.set_profiling(True)
+        cb.begin_compute_pass()
+        cb.encode(P("attn_qk_rope_blk"), {0: a_proj, 1: ones, 2: ones, 3: q, 4: gate, 5: keys, 6: values},
+                  {7: 0, 8: rows}, (18, rows), (256,))
+        cb.barrier()
+        cb.encode(P("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: out},
+                  {5: rows, 6: rows, 7: rows, 8: 0}, (16, (rows + 15) // 16), (256,))
+        cb.encode(P("gdn_conv_blk"), {0: g_proj, 1: conv_in, 2: conv_w, 3: qk, 4: v, 5: z, 6: conv_out},
+                  {7: rows}, (96, rows), (128,))
+        cb.encode(P("gdn_gates_blk"), {0: g_proj, 1: a_log, 2: dt_bias, 3: decay, 4: beta}, {5: rows},
+                  (1, (rows + 3) // 4, 1), (32, 4, 1))
+        cb.barrier()
+        cb.encode(P("gdn_chunk_prepare_blk"), {0: qk, 1: v, 2: decay, 3: beta, 4: chunk}, {5: rows},
+                  (chunks, 32), (256,))
+        cb.barrier()
+        cb.encode(P("gdn_chunk_scan_blk"), {0: chunk, 1: rec, 2: y, 3: rec}, {4: rows}, (8, 32), (256,))
+        cb.barrier()
+        cb.encode(P("gdn_gate_norm_blk"), {0: y, 1: z, 2: norm_w, 3: gated}, {}, (32, rows), (128,))
+        cb.end_compute_pass()
+        cb.commit().wait()
+        for name, ms in cb.command_times():
+            best[name] = min(best.get(name, ms), ms)
+    flash_ms = best["attention_flash_v2_blk"]
+    flops = 16 * 4 * 256 * rows * (rows + 1) / 2
+    attn_ms = flash_ms + best["attn_qk_rope_blk"]
+    gdn_ms = sum(best[k] for k in ("gdn_conv_blk", "gdn_gates_blk", "gdn_chunk_prepare_blk",
+                                   "gdn_chunk_scan_blk", "gdn_gate_norm_blk"))
+    return {"rows": rows,
+            "attention_layer_ms": round(attn_ms, 3),
+            "attention_layer_tok_per_s": round(rows / (attn_ms * 1e-3)),
+            "flash_kernel_ms": round(flash_ms, 3),
+            "flash_kernel_tflops": round(flops / (flash_ms * 1e-3) / 1e12, 1),
+            "flash_kernel_frac_of_bf16_mfma_peak": round(flops / (flash_ms * 1e-3) / 2.5e15, 4),
+            "gdn_layer_ms": round(gdn_ms, 3),
+            "gdn_layer_tok_per_s": round(rows / (gdn_ms * 1e-3)),
+            "kernel_ms": {k: round(v, 3) for k, v in best.items()}}
+
+
 def cpu_baseline(threads):
     """The CPU checker (reference arithmetic restated, oracle/liboracle.so) on one
     G,G,G,A period at the same shapes: 4 lanes x 32768 keys of attention decode and
@@ -191,6 +271,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true",
+                    help="skip the 16384-row block prefill figures in detail.prefill_16k")
     ap.add_argument("--split-keys", type=int, default=DEFAULT_SPLIT_KEYS,
                     help="keys per split-K workgroup (multiple of 32)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -266,7 +348,7 @@ def main():
         record_split_only(cb, k & 1)
     cb.end_compute_pass()
     cb.commit().wait()
-    split_us = round(cb.commit().wait() * 1e3 / launches, 2)
+    split_us = round(statistics.mean(cb.commit().wait() for _ in range(3)) * 1e3 / launches, 2)
     algo_bytes = LANES * VISIBLE * ATTN_BYTES_PER_KEY
     achieved = algo_bytes / (split_us * 1e-6) / 1e9
     attn_layer_us = sum(kernel_us[k] for k in ("attn_qk_rope_ms", "attention_decode_split_ms",
@@ -303,6 +385,8 @@ def main():
                    "gdn_layer_gbs": round(gdn_gbs, 1),
                    "kernel_avg_us": kernel_us},
     }
+    if not args.no_prefill:
+        line["detail"]["prefill_16k"] = prefill_figures(B, dev, queue, lib, torch)
     if not args.no_cpu_baseline:
         threads = min(16, os.cpu_count() or 1)
         line["cpu_baseline"] = cpu_baseline(threads)
