@@ -79,69 +79,77 @@ struct RopeArgs {
     uint32_t projection_stride; // elements between rows
     uint32_t query_stride;
     uint32_t position_per_row;  // 1: block prefill (row r sits at context + r)
+    uint32_t rows;
+    uint32_t rows_per_group;    // rows one workgroup walks (1 for decode)
 };
 
-// grid (18, rows) x 256: one head per workgroup, one dimension per thread.
-// Sum of squares: 64 threads x 4 values, a 32-lane adjacent-pairs tree per
-// half-wave, then the two halves added (attention.metal:63-88).
+// grid (18, ceil(rows / rows_per_group)) x 256: one head per workgroup, one
+// dimension per thread.  Sum of squares: 64 threads x 4 values, a 32-lane
+// adjacent-pairs tree per half-wave, then the two halves added
+// (attention.metal:63-88).
 __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
     __shared__ float normed[kD];
     __shared__ float inverse_shared;
     const uint32_t head = blockIdx.x;
-    const uint32_t row = blockIdx.y;
     const uint32_t d = threadIdx.x;
-    uint32_t position = a.context + (a.position_per_row ? row : 0u);
-    uint64_t kv_offset = 0;
-    if (a.table != nullptr) {
-        kv_offset = a.table[row * 4];
-        position = a.table[row * 4 + 1];
-    }
-    if (position >= a.capacity) return;  // a bad table row must not write outside the cache
-    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
     const bool is_query = head < kAttnQueryHeads;
     const uint32_t local = is_query ? head : head - kAttnQueryHeads;
     const uint32_t base = is_query ? head * 2 * kD : kAttnQGateRows + local * kD;
-    const float x = bf16_bits_to_f32(proj[base + d]);
-    if (d < 64) {
-        float acc = 0.0f;
-        for (uint32_t j = 0; j < 4; ++j) {
-            const float v = bf16_bits_to_f32(proj[base + d * 4 + j]);
-            acc += v * v;
+    const float weight = bf16_bits_to_f32(is_query ? a.q_weight[d] : a.k_weight[d]);
+    const uint32_t pair = d & (kAttnRopePairs - 1);
+    const float inverse_frequency =
+        d < 2 * kAttnRopePairs
+            ? powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs))
+            : 1.0f;
+    const uint32_t row_end = min(a.rows, (blockIdx.y + 1) * a.rows_per_group);
+    for (uint32_t row = blockIdx.y * a.rows_per_group; row < row_end; ++row) {
+        uint32_t position = a.context + (a.position_per_row ? row : 0u);
+        uint64_t kv_offset = 0;
+        if (a.table != nullptr) {
+            kv_offset = a.table[row * 4];
+            position = a.table[row * 4 + 1];
         }
-        for (uint32_t off = 1; off < 32; off <<= 1) acc += __shfl_xor(acc, off, 64);
-        const float total = acc + __shfl_xor(acc, 32, 64);
-        if (d == 0) {
-            inverse_shared = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+        if (position >= a.capacity) continue;  // a bad table row must not write outside the cache
+        const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+        const float x = bf16_bits_to_f32(proj[base + d]);
+        __syncthreads();  // the previous row's readers are done with the shared values
+        if (d < 64) {
+            float acc = 0.0f;
+            for (uint32_t j = 0; j < 4; ++j) {
+                const float v = bf16_bits_to_f32(proj[base + d * 4 + j]);
+                acc += v * v;
+            }
+            for (uint32_t off = 1; off < 32; off <<= 1) acc += __shfl_xor(acc, off, 64);
+            const float total = acc + __shfl_xor(acc, 32, 64);
+            if (d == 0) {
+                inverse_shared = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+            }
         }
-    }
-    __syncthreads();
-    const float inverse = inverse_shared;
-    const uint16_t weight = is_query ? a.q_weight[d] : a.k_weight[d];
-    // w * bf16(x * inv), the product rounded to bf16 again
-    const float n = round_bf16(bf16_bits_to_f32(weight) * round_bf16(x * inverse));
-    normed[d] = n;
-    __syncthreads();
-    float rotated = n;
-    if (d < 2 * kAttnRopePairs) {
-        const uint32_t pair = d & (kAttnRopePairs - 1);
-        const float theta = static_cast<float>(position) /
-                            powf(kAttnRopeBase, static_cast<float>(pair) /
-                                                    static_cast<float>(kAttnRopePairs));
-        const float c = cosf(theta);
-        const float s = sinf(theta);
-        rotated = d < kAttnRopePairs ? fmaf(-normed[d + kAttnRopePairs], s, n * c)
-                                     : fmaf(normed[d - kAttnRopePairs], s, n * c);
-    }
-    const uint16_t stored = f32_to_bf16_bits(rotated);
-    if (is_query) {
-        const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
-        a.q_out[at] = stored;
-        a.gate_out[at] = proj[head * 2 * kD + kD + d];
-    } else {
-        const uint64_t at =
-            kv_offset + (static_cast<uint64_t>(local) * a.capacity + position) * kD + d;
-        a.keys[at] = stored;
-        a.values[at] = proj[kAttnVRowOffset + local * kD + d];
+        __syncthreads();
+        const float inverse = inverse_shared;
+        // w * bf16(x * inv), the product rounded to bf16 again
+        const float n = round_bf16(weight * round_bf16(x * inverse));
+        normed[d] = n;
+        __syncthreads();
+        float rotated = n;
+        if (d < 2 * kAttnRopePairs) {
+            const float theta = static_cast<float>(position) / inverse_frequency;
+            const float c = cosf(theta);
+            const float s = sinf(theta);
+            rotated = d < kAttnRopePairs ? fmaf(-normed[d + kAttnRopePairs], s, n * c)
+                                         : fmaf(normed[d - kAttnRopePairs], s, n * c);
+        }
+        const uint16_t stored = f32_to_bf16_bits(rotated);
+        if (is_query) {
+            const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+            a.q_out[at] = stored;
+            a.gate_out[at] = proj[head * 2 * kD + kD + d];
+        } else {
+            const uint64_t at =
+                kv_offset + (static_cast<uint64_t>(local) * a.capacity + position) * kD + d;
+            a.keys[at] = stored;
+            a.values[at] = proj[kAttnVRowOffset + local * kD + d];
+        }
     }
 }
 
@@ -615,9 +623,13 @@ uint64_t cache_bytes(uint32_t capacity) {
     return static_cast<uint64_t>(kAttnKvHeads) * capacity * kD * 2;
 }
 
-int32_t launch_rope(const RopeArgs& r, uint32_t rows, hipStream_t stream) {
-    hipLaunchKernelGGL(attn_qk_rope_kernel, dim3(kAttnQueryHeads + kAttnKvHeads, rows), dim3(256),
-                       0, stream, r);
+int32_t launch_rope(const RopeArgs& args, uint32_t rows, hipStream_t stream) {
+    RopeArgs r = args;
+    r.rows = rows;
+    r.rows_per_group = r.position_per_row ? 8u : 1u;  // blocks walk 8 rows per workgroup
+    const uint32_t groups = (rows + r.rows_per_group - 1) / r.rows_per_group;
+    hipLaunchKernelGGL(attn_qk_rope_kernel, dim3(kAttnQueryHeads + kAttnKvHeads, groups),
+                       dim3(256), 0, stream, r);
     return TT_OK;
 }
 

@@ -85,75 +85,81 @@ struct PrepareArgs {
     uint32_t rows;
 };
 
-// grid (96, rows) x 128: groups 0..63 convolve one 128-channel head each
-// (0..15 q, 16..31 k, 32..63 v), groups 64..95 copy the z gate.
+constexpr uint32_t kBlockRowsPerGroup = 16;  // block mode: rows one workgroup walks
+
+// grid (96, rows) x 128 (decode) or (96, ceil(rows/16)) (block mode, a workgroup
+// walks 16 consecutive rows with a sliding tap window): groups 0..63 convolve one
+// 128-channel head each (0..15 q, 16..31 k, 32..63 v), groups 64..95 copy the z gate.
 __global__ __launch_bounds__(128) void gdn_prepare_kernel(PrepareArgs a) {
     __shared__ float partial[2];
     const uint32_t group = blockIdx.x;
-    const uint32_t row = blockIdx.y;
     const uint32_t lane = threadIdx.x;
-    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const uint32_t row_begin = a.block_mode ? blockIdx.y * kBlockRowsPerGroup : blockIdx.y;
+    const uint32_t row_end = a.block_mode ? min(a.rows, row_begin + kBlockRowsPerGroup) : row_begin + 1;
     if (group >= kCh / kGD) {
         const uint32_t index = (group - kCh / kGD) * kGD + lane;
-        a.z[static_cast<uint64_t>(row) * a.z_stride + index] = proj[kCh + index];
+        for (uint32_t row = row_begin; row < row_end; ++row) {
+            a.z[static_cast<uint64_t>(row) * a.z_stride + index] =
+                a.projection[static_cast<uint64_t>(row) * a.projection_stride + kCh + index];
+        }
         return;
     }
     const uint16_t* conv_in = a.conv_in;
     uint16_t* conv_out = a.conv_out;
     if (a.table != nullptr) {
-        conv_in += a.table[row * 4];
-        conv_out += a.table[row * 4 + 1];
+        conv_in += a.table[row_begin * 4];
+        conv_out += a.table[row_begin * 4 + 1];
     }
     const uint32_t c = group * kGD + lane;
-    float taps[4];
-    uint16_t tap_bits[4];
-#pragma unroll
-    for (uint32_t tap = 0; tap < 4; ++tap) {
-        // logical sequence = three state rows then the block's projection rows
-        const uint32_t logical = (a.block_mode ? row : 0u) + tap;
-        tap_bits[tap] = logical < 3
-                            ? conv_in[logical * kCh + c]
-                            : (a.block_mode
-                                   ? a.projection[static_cast<uint64_t>(logical - 3) *
-                                                      a.projection_stride + c]
-                                   : proj[c]);
-        taps[tap] = widen(tap_bits[tap]);
-    }
+    // logical sequence = three state rows then the block's projection rows; a decode
+    // row is a block of one
+    const uint32_t first = a.block_mode ? row_begin : 0u;
+    auto logical = [&](uint32_t index) -> uint16_t {
+        if (index < 3) return conv_in[index * kCh + c];
+        const uint32_t prow = a.block_mode ? index - 3 : row_begin;
+        return a.projection[static_cast<uint64_t>(prow) * a.projection_stride + c];
+    };
+    uint16_t t0 = logical(first), t1 = logical(first + 1), t2 = logical(first + 2);
     const uint16_t* w = a.conv_weights + static_cast<uint64_t>(c) * 4;
-    // fixed four-term shape; bf16 x bf16 products are exact in fp32
-    const float convolved = widen(w[0]) * taps[0] + widen(w[1]) * taps[1] +
-                            widen(w[2]) * taps[2] + widen(w[3]) * taps[3];
-    const float conv_b = rb(convolved);
-    const float act = rb(conv_b * sigmoid_bf16(conv_b));
-    if (!a.block_mode || row == a.rows - 1) {
-        conv_out[c] = tap_bits[1];
-        conv_out[kCh + c] = tap_bits[2];
-        conv_out[2 * kCh + c] = tap_bits[3];
-    }
-    if (group < kGdnQkValues / kGD) {
-        // RMS over the head: lane l (< 32) sums values 4l..4l+3, then the tree
-        const float neighbour_sum = [&]() {
+    const float w0 = widen(w[0]), w1 = widen(w[1]), w2 = widen(w[2]), w3 = widen(w[3]);
+    for (uint32_t row = row_begin; row < row_end; ++row) {
+        const uint16_t t3 = a.projection[static_cast<uint64_t>(row) * a.projection_stride + c];
+        // fixed four-term shape; bf16 x bf16 products are exact in fp32
+        const float convolved = w0 * widen(t0) + w1 * widen(t1) + w2 * widen(t2) + w3 * widen(t3);
+        const float conv_b = rb(convolved);
+        const float act = rb(conv_b * sigmoid_bf16(conv_b));
+        if (!a.block_mode || row == a.rows - 1) {
+            conv_out[c] = t1;
+            conv_out[kCh + c] = t2;
+            conv_out[2 * kCh + c] = t3;
+        }
+        if (group < kGdnQkValues / kGD) {
+            // RMS over the head: lane l (< 32) sums values 4l..4l+3, then the tree
             float sq = act * act;
             // gather 4 consecutive squares in ascending order onto lane 4k
             const float s1 = __shfl_down(sq, 1, 64);
             const float s2 = __shfl_down(sq, 2, 64);
             const float s3 = __shfl_down(sq, 3, 64);
-            return ((sq + s1) + s2) + s3;
-        }();
-        // lanes 4k hold thread-k partials; bring them to lanes 0..15 of each wave
-        const uint32_t wave = lane >> 6;
-        const uint32_t wl = lane & 63;
-        float v = __shfl(neighbour_sum, (wl & 15) * 4, 64);  // 16 partials per wave
-        // adjacent-pairs over 32 partials = pairs within each wave, then across
-        for (uint32_t off = 1; off < 16; off <<= 1) v += __shfl_xor(v, off, 64);
-        if (wl == 0) partial[wave] = v;
-        __syncthreads();
-        const float total = partial[0] + partial[1];
-        const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
-        const float scale = widen(group < kGdnKeyHeads ? kGdnQueryScaleBits : kGdnKeyScaleBits);
-        a.qk[static_cast<uint64_t>(row) * a.qk_stride + c] = narrow(rb(act * inverse) * scale);
-    } else {
-        a.value[static_cast<uint64_t>(row) * a.value_stride + c - kGdnQkValues] = narrow(act);
+            const float neighbour_sum = ((sq + s1) + s2) + s3;
+            // lanes 4k hold thread-k partials; bring them to lanes 0..15 of each wave
+            const uint32_t wave = lane >> 6;
+            const uint32_t wl = lane & 63;
+            float v = __shfl(neighbour_sum, (wl & 15) * 4, 64);  // 16 partials per wave
+            // adjacent-pairs over 32 partials = pairs within each wave, then across
+            for (uint32_t off = 1; off < 16; off <<= 1) v += __shfl_xor(v, off, 64);
+            __syncthreads();  // the previous row's readers are done with `partial`
+            if (wl == 0) partial[wave] = v;
+            __syncthreads();
+            const float total = partial[0] + partial[1];
+            const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
+            const float scale = widen(group < kGdnKeyHeads ? kGdnQueryScaleBits : kGdnKeyScaleBits);
+            a.qk[static_cast<uint64_t>(row) * a.qk_stride + c] = narrow(rb(act * inverse) * scale);
+        } else {
+            a.value[static_cast<uint64_t>(row) * a.value_stride + c - kGdnQkValues] = narrow(act);
+        }
+        t0 = t1;
+        t1 = t2;
+        t2 = t3;
     }
 }
 
@@ -256,34 +262,40 @@ __global__ void gdn_gates_kernel(const uint16_t* projection, const uint16_t* a_l
 
 // --------------------------------------------------------------- gate norm ---
 
-// grid (32, rows) x 128: y * rsqrt(mean y^2 + eps) rounded to bf16, times the
-// weight rounded to bf16, times fp32 SiLU(z); one bf16 rounding at the end
-// (gdn.metal:174-207).
+// grid (32, ceil(rows / rows_per_group)) x 128: y * rsqrt(mean y^2 + eps) rounded to
+// bf16, times the weight rounded to bf16, times fp32 SiLU(z); one bf16 rounding at
+// the end (gdn.metal:174-207).
 __global__ __launch_bounds__(128) void gdn_gate_norm_kernel(const uint16_t* y, const uint16_t* z,
                                                             const uint16_t* weight, uint16_t* out,
-                                                            uint32_t stride) {
+                                                            uint32_t stride, uint32_t rows,
+                                                            uint32_t rows_per_group) {
     __shared__ float partial[2];
     const uint32_t head = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint64_t at = static_cast<uint64_t>(blockIdx.y) * stride + head * kGD + lane;
-    const float v = widen(y[at]);
-    const float sq = v * v;
-    const float s1 = __shfl_down(sq, 1, 64);
-    const float s2 = __shfl_down(sq, 2, 64);
-    const float s3 = __shfl_down(sq, 3, 64);
-    const float four = ((sq + s1) + s2) + s3;
-    const uint32_t wl = lane & 63;
-    float t = __shfl(four, (wl & 15) * 4, 64);
-    for (uint32_t off = 1; off < 16; off <<= 1) t += __shfl_xor(t, off, 64);
-    if (wl == 0) partial[lane >> 6] = t;
-    __syncthreads();
-    const float inverse =
-        1.0f / sqrtf((partial[0] + partial[1]) / static_cast<float>(kGD) + kRmsNormEpsilon);
-    const float normed = rb(widen(weight[lane]) * rb(v * inverse));
-    const float g = widen(z[at]);
-    const float low = 1.0f / (1.0f + expf(fabsf(g)));
-    const float sig = g < 0.0f ? low : 1.0f - low;
-    out[at] = narrow((g * sig) * normed);
+    const float w = widen(weight[lane]);
+    const uint32_t row_end = min(rows, (blockIdx.y + 1) * rows_per_group);
+    for (uint32_t row = blockIdx.y * rows_per_group; row < row_end; ++row) {
+        const uint64_t at = static_cast<uint64_t>(row) * stride + head * kGD + lane;
+        const float v = widen(y[at]);
+        const float sq = v * v;
+        const float s1 = __shfl_down(sq, 1, 64);
+        const float s2 = __shfl_down(sq, 2, 64);
+        const float s3 = __shfl_down(sq, 3, 64);
+        const float four = ((sq + s1) + s2) + s3;
+        const uint32_t wl = lane & 63;
+        float t = __shfl(four, (wl & 15) * 4, 64);
+        for (uint32_t off = 1; off < 16; off <<= 1) t += __shfl_xor(t, off, 64);
+        __syncthreads();  // the previous row's readers are done with `partial`
+        if (wl == 0) partial[lane >> 6] = t;
+        __syncthreads();
+        const float inverse =
+            1.0f / sqrtf((partial[0] + partial[1]) / static_cast<float>(kGD) + kRmsNormEpsilon);
+        const float normed = rb(w * rb(v * inverse));
+        const float g = widen(z[at]);
+        const float low = 1.0f / (1.0f + expf(fabsf(g)));
+        const float sig = g < 0.0f ? low : 1.0f - low;
+        out[at] = narrow((g * sig) * normed);
+    }
 }
 
 // ------------------------------------------------- fused decode step ---------
@@ -930,7 +942,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
 // ---------------------------------------------------------------- launchers --
 
 int32_t launch_prepare(const PrepareArgs& p, hipStream_t stream) {
-    hipLaunchKernelGGL(gdn_prepare_kernel, dim3(96, p.rows), dim3(128), 0, stream, p);
+    const uint32_t groups =
+        p.block_mode ? (p.rows + kBlockRowsPerGroup - 1) / kBlockRowsPerGroup : p.rows;
+    hipLaunchKernelGGL(gdn_prepare_kernel, dim3(96, groups), dim3(128), 0, stream, p);
     return TT_OK;
 }
 
@@ -1194,8 +1208,9 @@ int32_t gate_norm_common(Args& a, const Grid& g, uint32_t rows, uint32_t stride,
     a.require(g.gx == 32 && g.gy == rows && g.gz == 1 && g.tx == 128 && g.ty == 1 && g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(gdn_gate_norm_kernel, dim3(32, rows), dim3(128), 0, stream, y, z, w, out,
-                       stride);
+    const uint32_t per_group = rows > kMaxBatchRows ? 8u : 1u;  // blocks walk 8 rows per group
+    hipLaunchKernelGGL(gdn_gate_norm_kernel, dim3(32, (rows + per_group - 1) / per_group), dim3(128),
+                       0, stream, y, z, w, out, stride, rows, per_group);
     return TT_OK;
 }
 
