@@ -174,8 +174,7 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
     rec = mk(32 * 128 * 128 * 4)
     qk, v, z, y, gated = (mk(rows * 8192) for _ in range(5))
     decay, beta = mk(rows * 128), mk(rows * 128)
-    chunks = (rows + 63) // 64
-    chunk = mk(chunks * 32 * 115712)
+    chunk = mk(((min(rows, 2048) + 63) // 64) * 32 * 115712)
     best = {}
     for _ in range(repeats):
         cb = queue.create_command_buffer()
@@ -191,10 +190,9 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
         cb.encode(P("gdn_gates_blk"), {0: g_proj, 1: a_log, 2: dt_bias, 3: decay, 4: beta}, {5: rows},
                   (1, (rows + 3) // 4, 1), (32, 4, 1))
         cb.barrier()
-        cb.encode(P("gdn_chunk_prepare_blk"), {0: qk, 1: v, 2: decay, 3: beta, 4: chunk}, {5: rows},
-                  (chunks, 32), (256,))
-        cb.barrier()
-        cb.encode(P("gdn_chunk_scan_blk"), {0: chunk, 1: rec, 2: y, 3: rec}, {4: rows}, (8, 32), (256,))
+        cb.encode(P("gdn_chunk_recurrence_blk"),
+                  {0: qk, 1: v, 2: decay, 3: beta, 4: chunk, 5: rec, 6: y, 7: rec}, {8: rows},
+                  (8, 32), (256,))
         cb.barrier()
         cb.encode(P("gdn_gate_norm_blk"), {0: y, 1: z, 2: norm_w, 3: gated}, {}, (32, rows), (128,))
         cb.end_compute_pass()
@@ -204,8 +202,8 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
     flash_ms = best["attention_flash_v2_blk"]
     flops = 16 * 4 * 256 * rows * (rows + 1) / 2
     attn_ms = flash_ms + best["attn_qk_rope_blk"]
-    gdn_ms = sum(best[k] for k in ("gdn_conv_blk", "gdn_gates_blk", "gdn_chunk_prepare_blk",
-                                   "gdn_chunk_scan_blk", "gdn_gate_norm_blk"))
+    gdn_ms = sum(best[k] for k in ("gdn_conv_blk", "gdn_gates_blk", "gdn_chunk_recurrence_blk",
+                                   "gdn_gate_norm_blk"))
     return {"rows": rows,
             "attention_layer_ms": round(attn_ms, 3),
             "attention_layer_tok_per_s": round(rows / (attn_ms * 1e-3)),

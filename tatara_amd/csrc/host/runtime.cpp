@@ -895,7 +895,8 @@ PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan
     g.gdn_parameter_bytes = (policy.gdn_gate_hoist || policy.gdn_chunked)
                                 ? block * plan.recurrent_heads * kF32Bytes
                                 : 0;
-    g.gdn_chunk_bytes = policy.gdn_chunked ? ((block + kGdnChunkRows - 1u) / kGdnChunkRows) *
+    g.gdn_chunk_bytes = policy.gdn_chunked ? ((std::min<std::uint64_t>(block, kGdnChunkGroupRows) +
+                                               kGdnChunkRows - 1u) / kGdnChunkRows) *
                                                  plan.recurrent_heads * kGdnChunkRecordBytes
                                            : 0;
     g.attention_projection_bytes = block * rows.attn_projection * kBf16Bytes;
@@ -974,8 +975,7 @@ PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::gdn_recurrence_gates_blk, "gdn_recurrence_gates_blk", error) &&
         resolve(library, p, &P::gdn_recurrence_blk, "gdn_recurrence_blk", error) &&
         resolve(library, p, &P::gdn_gate_norm_blk, "gdn_gate_norm_blk", error) &&
-        resolve(library, p, &P::gdn_chunk_prepare_blk, "gdn_chunk_prepare_blk", error) &&
-        resolve(library, p, &P::gdn_chunk_scan_blk, "gdn_chunk_scan_blk", error);
+        resolve(library, p, &P::gdn_chunk_recurrence_blk, "gdn_chunk_recurrence_blk", error);
     if (!ok) return {error, std::nullopt};
     return {HipPipelineError::None, std::move(p)};
 }
@@ -1069,7 +1069,6 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
     walk.barrier();
     if (geometry.policy.gdn_chunked) {
         if (!scratch.gdn_chunk) return HipCommandError::InvalidBuffer;
-        const std::uint32_t chunks = (rows + kGdnChunkRows - 1u) / kGdnChunkRows;
         walk.pipeline(pipelines.gdn_gates_blk);
         walk.buffer(scratch.gdn_projection, 0, 0);
         walk.weight(weights.a_log, 1);
@@ -1079,21 +1078,16 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
         walk.constant(rows, 5);
         walk.dispatch(HipSize{1, (rows + 3u) / 4u, 1}, HipSize{32, 4, 1});
         walk.barrier();
-        walk.pipeline(pipelines.gdn_chunk_prepare_blk);
+        walk.pipeline(pipelines.gdn_chunk_recurrence_blk);
         walk.buffer(scratch.gdn_qk, 0, 0);
         walk.buffer(scratch.gdn_value, 0, 1);
         walk.buffer(scratch.gdn_decay, 0, 2);
         walk.buffer(scratch.gdn_beta, 0, 3);
         walk.buffer(scratch.gdn_chunk, 0, 4);
-        walk.constant(rows, 5);
-        walk.dispatch(HipSize{chunks, 32, 1}, HipSize{256, 1, 1});
-        walk.barrier();
-        walk.pipeline(pipelines.gdn_chunk_scan_blk);
-        walk.buffer(scratch.gdn_chunk, 0, 0);
-        walk.buffer(recurrent_in, 0, 1);
-        walk.buffer(scratch.gdn_recurrence, 0, 2);
-        walk.buffer(recurrent_out, 0, 3);
-        walk.constant(rows, 4);
+        walk.buffer(recurrent_in, 0, 5);
+        walk.buffer(scratch.gdn_recurrence, 0, 6);
+        walk.buffer(recurrent_out, 0, 7);
+        walk.constant(rows, 8);
         walk.dispatch(HipSize{8, 32, 1}, HipSize{256, 1, 1});
         walk.barrier();
         walk.pipeline(pipelines.gdn_gate_norm_blk);

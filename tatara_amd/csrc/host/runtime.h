@@ -61,6 +61,7 @@ inline constexpr std::uint32_t kAttentionPartition = 256;      // decode_geometr
 inline constexpr std::uint32_t kConvShiftSteps = 3;
 inline constexpr std::uint32_t kGdnChunkRows = 64;             // tokens per chunk of the MFMA recurrence
 inline constexpr std::uint32_t kGdnChunkRecordBytes = 115712;  // scratch per (chunk, value head)
+inline constexpr std::uint32_t kGdnChunkGroupRows = 2048;      // rows whose records are live at once
 inline constexpr std::uint32_t kBf16Bytes = 2;
 inline constexpr std::uint32_t kF32Bytes = 4;
 inline constexpr std::uint32_t kMaximumBatchRows = 16;         // decode_step.cpp:554, 1008
@@ -362,8 +363,8 @@ struct PrefillPolicy {
     std::uint32_t query_tile_rows{0};
     std::uint32_t attention_partition{kAttentionPartition};
     bool gdn_gate_hoist{false};
-    // Evaluate the block recurrence 64 tokens at a time on MFMA (gdn_chunk_prepare_blk
-    // + gdn_chunk_scan_blk) instead of the reference's token-by-token register loop.
+    // Evaluate the block recurrence 64 tokens at a time on MFMA (gdn_chunk_recurrence_blk)
+    // instead of the reference's token-by-token register loop.
     // Implies hoisted gates.  The reference has no such switch.
     bool gdn_chunked{false};
 };
@@ -456,7 +457,7 @@ PrefillChunk prefill_chunk_at(const PrefillPolicy& policy, std::uint32_t context
 struct PrefillPipelines {
     HipComputePipeline attn_qk_rope_blk, attention_flash_blk;
     HipComputePipeline gdn_conv_blk, gdn_gates_blk, gdn_recurrence_gates_blk, gdn_recurrence_blk,
-        gdn_gate_norm_blk, gdn_chunk_prepare_blk, gdn_chunk_scan_blk;
+        gdn_gate_norm_blk, gdn_chunk_recurrence_blk;
 };
 struct PrefillPipelinesResult {
     backend::hip::HipPipelineError error;

@@ -495,15 +495,6 @@ constexpr uint32_t kRecGam = 114944;                    // f32  [64]: g_t
 constexpr uint32_t kRecGamma = 115200;                  // f32: g_C
 constexpr uint32_t kRecBytes = 115712;
 
-// byte offset of element (token t, key dk) inside a token-by-key operand
-__device__ __forceinline__ uint32_t frag_token_key(uint32_t t, uint32_t dk) {
-    return ((((t >> 4) * 4 + (dk >> 5)) * 64 + ((dk >> 3) & 3) * 16 + (t & 15)) * 8 + (dk & 7)) * 2;
-}
-// byte offset of element (token t, token s) inside an A operand
-__device__ __forceinline__ uint32_t frag_token_token(uint32_t t, uint32_t s) {
-    return ((((t >> 4) * 2 + (s >> 5)) * 64 + ((s >> 3) & 3) * 16 + (t & 15)) * 8 + (s & 7)) * 2;
-}
-
 struct ChunkPrepareArgs {
     const uint16_t* qk;      // [rows][4096]
     const uint16_t* value;   // [rows][4096]
@@ -550,6 +541,34 @@ __device__ __forceinline__ void split8(const float* x, bf16x8& hi, bf16x8& lo) {
     lo = __builtin_bit_cast(bf16x8, u32x4{l[0], l[1], l[2], l[3]});
 }
 
+// A wave's 16 x 16 MFMA result tile (this lane: rows 4g+i of column m) as bf16 hi/lo
+// pairs into fragment order: through a per-wave LDS tile so that every lane ends
+// up with eight consecutive columns of one row and stores 16 bytes; lanes 0..31
+// write the hi fragment piece, lanes 32..63 the lo piece, 512 contiguous bytes each.
+// `piece` is the byte offset of the tile's 512-byte run inside a fragment array.
+__device__ __forceinline__ void store_tile_hi_lo(uint16_t (*tile)[16][24], const f32x4 acc,
+                                                 uint32_t lane, uint8_t* hi_base, uint8_t* lo_base,
+                                                 uint32_t piece) {
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        const uint16_t hi = narrow(acc[i]);
+        tile[0][g * 4 + i][m] = hi;
+        tile[1][g * 4 + i][m] = narrow(acc[i] - widen(hi));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint32_t half = lane >> 5;
+    const uint32_t row = lane & 15;
+    const uint32_t group = (lane >> 4) & 1;  // which run of eight columns
+    const u32x4 v = *reinterpret_cast<const u32x4*>(&tile[half][row][group * 8]);
+    *reinterpret_cast<u32x4*>((half ? lo_base : hi_base) + piece + (group * 16 + row) * 16) = v;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 // Stage 1, grid (chunks, 32) x 256: decay products, Gram tiles on MFMA, the
 // inverse T of the unit lower-triangular I + L (diagonal 16x16 blocks by forward
 // substitution in registers, the rest by block recursion, all fp32), then
@@ -559,6 +578,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     __shared__ __attribute__((aligned(16))) float lower[kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float tinv[kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float mtmp[16][52];
+    __shared__ __attribute__((aligned(16))) uint16_t tiles[4][2][16][24];  // per-wave store staging
     __shared__ __attribute__((aligned(16))) float log_g[kChunk];
     __shared__ __attribute__((aligned(16))) float scale_k[kChunk];  // beta_t g_t
     __shared__ __attribute__((aligned(16))) float scale_v[kChunk];  // beta_t
@@ -573,6 +593,30 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     const uint32_t t0 = chunk * kChunk;
     const uint32_t valid = min(kChunk, a.rows - t0);
     uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
+
+    // The right-hand sides of the last stage ([K | V] columns, token-contiguous per
+    // lane: 2-byte gathers) are requested now and consumed at the end, behind the
+    // Gram and inverse stages.  Waves 0,1 take the 128 key columns, waves 2,3 the values.
+    const bool is_k = wave < 2;
+    uint32_t rhs_bits[4][2][8];
+    {
+        const uint16_t* src =
+            is_k ? a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kGdnKOffset + kh * kGD
+                 : a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
+        const uint32_t src_stride = is_k ? kGdnQkValues : kGdnValueValues;
+#pragma unroll
+        for (uint32_t ct = 0; ct < 4; ++ct) {
+            const uint32_t col = (wave & 1) * 64 + ct * 16 + m;
+#pragma unroll
+            for (uint32_t ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (uint32_t e = 0; e < 8; ++e) {
+                    const uint32_t s = min(ks * 32 + g * 8 + e, valid - 1);
+                    rhs_bits[ct][ks][e] = src[static_cast<uint64_t>(s) * src_stride + col];
+                }
+            }
+        }
+    }
 
     if (tid < kChunk) {
         float dec = 1.0f;
@@ -623,17 +667,17 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
                 qkacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aq[kk], bk, qkacc, 0, 0, 0);
             }
             const uint32_t s = nt * 16 + m;
+            f32x4 aqk;
 #pragma unroll
             for (uint32_t i = 0; i < 4; ++i) {
                 const uint32_t t = wave * 16 + g * 4 + i;
                 const float ratio = s <= t ? __expf(log_g[t] - log_g[s]) : 0.0f;
                 lower[t][s] = (s < t && t < valid) ? scale_v[t] * ratio * kkacc[i] : 0.0f;
-                const float aqk = (s <= t && t < valid) ? ratio * qkacc[i] : 0.0f;
-                const uint16_t hi = narrow(aqk);
-                *reinterpret_cast<uint16_t*>(rec + kRecAqkHi + frag_token_token(t, s)) = hi;
-                *reinterpret_cast<uint16_t*>(rec + kRecAqkLo + frag_token_token(t, s)) =
-                    narrow(aqk - widen(hi));
+                aqk[i] = (s <= t && t < valid) ? ratio * qkacc[i] : 0.0f;
             }
+            // fragment (token tile `wave`, token step nt >> 1), column groups 2(nt&1), +1
+            store_tile_hi_lo(tiles[wave], aqk, lane, rec + kRecAqkHi, rec + kRecAqkLo,
+                             ((wave * 2 + (nt >> 1)) * 64 + (nt & 1) * 32) * 16);
         }
     }
     __syncthreads();
@@ -688,10 +732,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             split8(&tinv[mt * 16 + m][ks * 32 + g * 8], t_hi[mt][ks], t_lo[mt][ks]);
         }
     }
-    const bool is_k = wave < 2;
-    const uint16_t* src =
-        is_k ? krows : a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
-    const uint32_t src_stride = is_k ? kGdnQkValues : kGdnValueValues;
     const float* scale = is_k ? scale_k : scale_v;
     float sc[2][8];
 #pragma unroll
@@ -699,7 +739,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) sc[ks][e] = scale[ks * 32 + g * 8 + e];
     }
-#pragma unroll 1
+#pragma unroll
     for (uint32_t ct = 0; ct < 4; ++ct) {
         const uint32_t col = (wave & 1) * 64 + ct * 16 + m;
         bf16x8 b_hi[2], b_lo[2];
@@ -709,8 +749,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             uint32_t bits[8];
 #pragma unroll
             for (uint32_t e = 0; e < 8; ++e) {
-                const uint32_t s = ks * 32 + g * 8 + e;
-                bits[e] = s < valid ? src[static_cast<uint64_t>(s) * src_stride + col] : 0u;
+                // rows past the block were clamped on load: their scale (beta) is zero,
+                // and the exact keys stored below are zeroed explicitly
+                bits[e] = ks * 32 + g * 8 + e < valid ? rhs_bits[ct][ks][e] : 0u;
                 x[e] = widen(static_cast<uint16_t>(bits[e])) * sc[ks][e];
             }
             split8(x, b_hi[ks], b_lo[ks]);
@@ -733,13 +774,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             }
             // lane holds tokens 16mt+4g+i of column col
             if (is_k) {
-#pragma unroll
-                for (uint32_t i = 0; i < 4; ++i) {
-                    const uint32_t at = frag_token_key(mt * 16 + g * 4 + i, col);
-                    const uint16_t hi = narrow(acc[i]);
-                    *reinterpret_cast<uint16_t*>(rec + kRecWkHi + at) = hi;
-                    *reinterpret_cast<uint16_t*>(rec + kRecWkLo + at) = narrow(acc[i] - widen(hi));
-                }
+                // fragment (token tile mt, key step col0 >> 5), column groups (col0 & 31) >> 3, +1
+                const uint32_t col0 = (wave & 1) * 64 + ct * 16;
+                store_tile_hi_lo(tiles[wave], acc, lane, rec + kRecWkHi, rec + kRecWkLo,
+                                 ((mt * 4 + (col0 >> 5)) * 64 + ((col0 & 31) >> 3) * 16) * 16);
             } else {
                 *reinterpret_cast<f32x4*>(rec + kRecWv +
                                           (((col >> 4) * 4 + mt) * 64 + g * 16 + (col & 15)) * 16) = acc;
@@ -1294,6 +1332,55 @@ int32_t op_gdn_chunk_scan(const Bindings& b, const Grid& g, hipStream_t stream,
     return TT_OK;
 }
 
+// Rows one prepare + scan pair of gdn_chunk_recurrence_blk covers: the chunk records
+// of a group (118 MB) stay in the 256 MB last-level cache between the two stages.
+constexpr uint32_t kChunkGroupRows = 2048;
+
+// gdn_chunk_recurrence_blk (no reference counterpart: the chunked evaluation of
+// gdn_recurrence_gates_blk, prefill_step.cpp:1988-2040, in one dispatch): b0 qk
+// [rows][4096], b1 value [rows][4096], b2 decay [rows][32], b3 beta [rows][32],
+// b4 scratch (chunk records of min(rows, 2048) rows), b5 state_in, b6 y [rows][4096],
+// b7 state_out, c8 rows; grid (8, 32) x 256.  Walks the block in groups of 2048
+// rows, stage 1 then stage 2 per group; state_in and state_out may be the same plane.
+int32_t op_gdn_chunk_recurrence(const Bindings& b, const Grid& g, hipStream_t stream,
+                                bool validate_only) {
+    Args a(b);
+    const uint32_t rows = a.constant(8);
+    a.require(rows >= 1 && rows <= (1u << 22), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    a.require(grid_is(g, 8, 32, 1, 256, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    const uint64_t row_bytes = static_cast<uint64_t>(rows) * kGdnValueValues * 2;
+    const uint16_t* qk = a.buffer<const uint16_t>(0, row_bytes);
+    const uint16_t* value = a.buffer<const uint16_t>(1, row_bytes);
+    const float* decay = a.buffer<const float>(2, static_cast<uint64_t>(rows) * kGdnValueHeads * 4);
+    const float* beta = a.buffer<const float>(3, static_cast<uint64_t>(rows) * kGdnValueHeads * 4);
+    uint8_t* scratch = a.buffer<uint8_t>(4, chunk_scratch_bytes(min(rows, kChunkGroupRows)));
+    const float* state_in = a.buffer<const float>(5, kGdnStateFloats * 4ull);
+    uint16_t* y = a.buffer<uint16_t>(6, row_bytes);
+    float* state_out = a.buffer<float>(7, kGdnStateFloats * 4ull);
+    if (a.status != TT_OK || validate_only) return a.status;
+    for (uint32_t start = 0; start < rows; start += kChunkGroupRows) {
+        const uint32_t count = min(kChunkGroupRows, rows - start);
+        ChunkPrepareArgs p{};
+        p.qk = qk + static_cast<uint64_t>(start) * kGdnQkValues;
+        p.value = value + static_cast<uint64_t>(start) * kGdnValueValues;
+        p.decay = decay + static_cast<uint64_t>(start) * kGdnValueHeads;
+        p.beta = beta + static_cast<uint64_t>(start) * kGdnValueHeads;
+        p.scratch = scratch;
+        p.rows = count;
+        hipLaunchKernelGGL(gdn_chunk_prepare_kernel, dim3((count + kChunk - 1) / kChunk, kGdnValueHeads),
+                           dim3(256), 0, stream, p);
+        ChunkScanArgs c{};
+        c.scratch = scratch;
+        c.state_in = start == 0 ? state_in : state_out;
+        c.state_out = state_out;
+        c.y = y + static_cast<uint64_t>(start) * kGdnValueValues;
+        c.rows = count;
+        hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(256), 0, stream, c);
+    }
+    return TT_OK;
+}
+
 }  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
@@ -1316,6 +1403,7 @@ const KernelDesc kGdnPrefillKernels[] = {
     {"gdn_gate_norm_blk", op_gdn_gate_norm_blk},
     {"gdn_chunk_prepare_blk", op_gdn_chunk_prepare},
     {"gdn_chunk_scan_blk", op_gdn_chunk_scan},
+    {"gdn_chunk_recurrence_blk", op_gdn_chunk_recurrence},
 };
 const uint32_t kGdnPrefillKernelCount = sizeof(kGdnPrefillKernels) / sizeof(kGdnPrefillKernels[0]);
 

@@ -113,7 +113,7 @@ class StubStack:
         self.q, self.gate = mk(rows * 8192), mk(rows * 8192)
         self.decay, self.beta = mk(rows * 128), mk(rows * 128)
         self.partials = mk(lanes * 16 * self.max_splits * 258 * 4)
-        self.chunk = mk(((block_rows + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
+        self.chunk = mk(((min(block_rows, 2048) + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
         self.logits = mk(rows * vocab * 2)
         self._write_tables()
 
@@ -223,13 +223,9 @@ class StubStack:
                            4: self.beta}, {5: rows}, (1, (rows + 3) // 4, 1), (32, 4, 1))
                 cb.barrier()
                 if chunked:
-                    chunks = (rows + 63) // 64
-                    cb.encode(P("gdn_chunk_prepare_blk"),
-                              {0: self.qk, 1: self.v, 2: self.decay, 3: self.beta, 4: self.chunk},
-                              {5: rows}, (chunks, 32), (256,))
-                    cb.barrier()
-                    cb.encode(P("gdn_chunk_scan_blk"), {0: self.chunk, 1: rec_in, 2: self.y, 3: rec_out},
-                              {4: rows}, (8, 32), (256,))
+                    cb.encode(P("gdn_chunk_recurrence_blk"),
+                              {0: self.qk, 1: self.v, 2: self.decay, 3: self.beta, 4: self.chunk,
+                               5: rec_in, 6: self.y, 7: rec_out}, {8: rows}, (8, 32), (256,))
                 else:
                     cb.encode(P("gdn_recurrence_gates_blk"),
                               {0: self.qk, 1: self.v, 2: self.decay, 3: layer["a_log"], 4: self.beta,

@@ -200,3 +200,46 @@ def test_chunked_recurrence_validation():
                   (256, 1, 1))
     assert e.value.status == 15
     assert cb.command_count == 0
+
+
+def test_grouped_chunk_recurrence_equals_the_two_stages():
+    """gdn_chunk_recurrence_blk (stage 1 + stage 2 per group of 2048 rows, scratch for
+    one group only) against gdn_chunk_prepare_blk + gdn_chunk_scan_blk over 2300 rows
+    (two groups, ragged tail): bit-identical outputs and state."""
+    print("[case] gdn grouped chunk recurrence, 2300 rows", flush=True)
+    B, dev, queue, lib = gpu()
+    rows = 2300
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal((rows, 16, 128)); k = rng.standard_normal((rows, 16, 128))
+    q /= np.linalg.norm(q, axis=2, keepdims=True) * np.sqrt(128.0)
+    k /= np.linalg.norm(k, axis=2, keepdims=True)
+    qk = ol.f32_to_bf16(np.concatenate([q.reshape(rows, -1), k.reshape(rows, -1)], axis=1)
+                        .astype(np.float32).reshape(-1))
+    v = ol.gaussian_bf16(0x6701, rows * 4096)
+    decay = np.exp(rng.uniform(-0.1, 0, (rows, 32))).astype(np.float32)
+    beta = (1 / (1 + np.exp(-rng.standard_normal((rows, 32))))).astype(np.float32)
+    state = ol.gaussian_f32(0x6702, STATE, 0.0, 0.02)
+    bufs = {"qk": dev.buffer_from(qk), "value": dev.buffer_from(v),
+            "decay": dev.buffer_from(decay.reshape(-1)), "beta": dev.buffer_from(beta.reshape(-1)),
+            "state_in": dev.buffer_from(state), "state_out": dev.create_buffer(STATE * 4),
+            "y": dev.create_buffer(rows * 8192),
+            "chunk": dev.create_buffer(((rows + 63) // 64) * 32 * 115712)}
+    state2, y2 = dev.create_buffer(STATE * 4), dev.create_buffer(rows * 8192)
+    small = dev.create_buffer(32 * 32 * 115712)          # records of 2048 rows
+
+    def rec(cb):
+        _encode_chunked(cb, lib, bufs, rows)
+        cb.encode(lib.pipeline("gdn_chunk_recurrence_blk"),
+                  {0: bufs["qk"], 1: bufs["value"], 2: bufs["decay"], 3: bufs["beta"], 4: small,
+                   5: bufs["state_in"], 6: y2, 7: state2}, {8: rows}, (8, 32, 1), (256, 1, 1))
+    run(rec)
+    assert np.array_equal(y2.read(np.uint16), bufs["y"].read(np.uint16))
+    assert np.array_equal(state2.read(np.float32), bufs["state_out"].read(np.float32))
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    with pytest.raises(B.BackendError) as e:             # scratch below one group's records
+        cb.encode(lib.pipeline("gdn_chunk_recurrence_blk"),
+                  {0: bufs["qk"], 1: bufs["value"], 2: bufs["decay"], 3: bufs["beta"],
+                   4: dev.create_buffer(1024), 5: bufs["state_in"], 6: y2, 7: state2}, {8: rows},
+                  (8, 32, 1), (256, 1, 1))
+    assert e.value.status == 10
