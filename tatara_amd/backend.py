@@ -113,6 +113,19 @@ def _check(status, where):
     if status != 0:
         raise BackendError(status, where)
 
+def _release(owner, destroy_name):
+    """Finalizer body shared by the handle classes.  During interpreter shutdown the
+    module's globals are already cleared; a handle that outlives them is left to the
+    process exit (the library frees device memory with the HIP context)."""
+    handle = getattr(owner, "handle", None)
+    if not handle:
+        return
+    owner.handle = None
+    if _lib is None:
+        return
+    getattr(_lib, destroy_name)(handle)
+
+
 
 class Device:
     def __init__(self):
@@ -170,10 +183,8 @@ class CommandQueue:
     def create_command_buffer(self):
         return CommandBuffer(self)
 
-    def __del__(self):
-        if getattr(self, "handle", None):
-            lib().tt_queue_destroy(self.handle)
-            self.handle = None
+    def __del__(self, _release=_release):
+        _release(self, "tt_queue_destroy")
 
 
 class Buffer:
@@ -229,10 +240,8 @@ class Buffer:
                                     out.nbytes), "buffer_read")
         return out
 
-    def __del__(self):
-        if getattr(self, "handle", None):
-            lib().tt_buffer_destroy(self.handle)
-            self.handle = None
+    def __del__(self, _release=_release):
+        _release(self, "tt_buffer_destroy")
 
 
 class Library:
@@ -254,21 +263,17 @@ class Library:
             self._cache[name] = Pipeline(h, name)
         return self._cache[name]
 
-    def __del__(self):
+    def __del__(self, _release=_release):
         self._cache.clear()
-        if getattr(self, "handle", None):
-            lib().tt_library_destroy(self.handle)
-            self.handle = None
+        _release(self, "tt_library_destroy")
 
 
 class Pipeline:
     def __init__(self, handle, name):
         self.handle, self.name = handle, name
 
-    def __del__(self):
-        if getattr(self, "handle", None):
-            lib().tt_pipeline_destroy(self.handle)
-            self.handle = None
+    def __del__(self, _release=_release):
+        _release(self, "tt_pipeline_destroy")
 
 
 class CommandBuffer:
@@ -375,7 +380,5 @@ class CommandBuffer:
             out.append((lib().tt_command_name(self.handle, i).decode(), ms.value))
         return out
 
-    def __del__(self):
-        if getattr(self, "handle", None):
-            lib().tt_command_buffer_destroy(self.handle)
-            self.handle = None
+    def __del__(self, _release=_release):
+        _release(self, "tt_command_buffer_destroy")
