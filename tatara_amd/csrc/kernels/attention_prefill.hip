@@ -31,6 +31,8 @@
 // (query, key) pair per head.
 #include "../tt_internal.h"
 
+#include <type_traits>
+
 namespace tt {
 namespace {
 
@@ -384,6 +386,344 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
     }
 }
 
+// ------------------------------------------------- 32-position workgroup ------
+//
+// Workgroup = 8 wave64 = 32 consecutive query positions x the 8 query heads of one
+// kv head.  Wave w owns heads 2(w&3), 2(w&3)+1 at positions 16(w>>2)..+15: two 16x16
+// blocks that share every K and V fragment the wave reads from LDS.  Two waves per
+// SIMD (256 registers each): one wave's softmax (VALU) runs under the other's
+// products (MFMA), and LDS operand reads are issued from eight waves.
+//   K tiles: HBM/L2 -> LDS ring of 3 stages, two tiles ahead (global_load_lds).
+//   V tiles: HBM/L2 -> raw LDS ring of 3 stages, three tiles ahead; one tile ahead
+//   of its use the 512 lanes transpose it once into V^T[dim][key slot] (80-byte
+//   rows: conflict-free 16-byte operand reads), so a wave's V^T operands are plain
+//   LDS reads instead of 64 register permutes per wave and tile.
+// One barrier per tile.  Softmax as in the 16-position kernel: reference fixed by
+// tile 0, exact online loop as the way out.
+constexpr bool kUseWideTile = true;
+constexpr uint32_t kWideWaves = 8;
+constexpr uint32_t kWidePositions = 32;
+constexpr uint32_t kRing = 3;
+constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;      // 49920
+constexpr uint32_t kValueRingBytes = kRing * kValueStageBytes;  // 49152
+constexpr uint32_t kValueRowBytes = 80;                         // 32 key slots of one dim + pad
+constexpr uint32_t kTransposedBytes = kD * kValueRowBytes;      // 20480
+constexpr uint32_t kWideLdsBytes = kKeyRingBytes + kValueRingBytes + 2 * kTransposedBytes;
+
+__global__ __launch_bounds__(kWideWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
+    constexpr uint32_t NB = 2;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t* const key_ring = lds;
+    uint8_t* const value_ring = lds + kKeyRingBytes;
+    uint8_t* const transposed = value_ring + kValueRingBytes;
+    // longest key walks first: the last position tile is dispatched first
+    const uint32_t tile = gridDim.x - 1 - blockIdx.x;
+    const uint32_t kvh = blockIdx.y;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t half = wave >> 2;
+    const uint32_t head0 = kvh * kAttnHeadsPerKv + (wave & 3) * 2;
+    const uint32_t p0 = tile * kWidePositions;
+    const uint32_t tile_keys = a.tile_context + min(p0 + kWidePositions, a.rows);  // visible count
+    const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
+    // this lane's column: query row p0 + 16*half + m, whose last visible key is limit
+    const uint32_t row = p0 + half * 16 + m;
+    const uint32_t limit = a.tile_context + row;
+    // tiles below first_masked lie entirely at or before the first column's limit
+    const uint32_t first_masked = (a.tile_context + p0 + half * 16 + 1) / kTileKeys;
+
+    bf16x8 q[NB][8];
+    {
+        const uint32_t pos = min(row, a.rows - 1);
+#pragma unroll
+        for (uint32_t t = 0; t < NB; ++t) {
+            const uint16_t* qrow =
+                a.query + (static_cast<uint64_t>(pos) * kAttnQueryHeads + head0 + t) * kD;
+#pragma unroll
+            for (uint32_t kk = 0; kk < 8; ++kk) {
+                q[t][kk] = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(qrow + kk * 32 + g * 8));
+            }
+        }
+    }
+
+    const uint16_t* kbase = a.keys + static_cast<uint64_t>(kvh) * a.capacity * kD;
+    const uint16_t* vbase = a.values + static_cast<uint64_t>(kvh) * a.capacity * kD;
+
+    // Each wave moves an eighth of a tile: 2 K transfers (key pairs 2w, 2w+1) and 2 V
+    // transfers (rows 4w..4w+3), 1 KiB each.  Tiles past the walk re-read the last
+    // key, so every batch has the same number of transfers.
+    auto stage_keys = [&](uint32_t kb) {
+        uint8_t* stage = key_ring + (kb % kRing) * kKeyStageBytes;
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            const uint32_t pair = wave * 2 + i;
+            const uint32_t key = min(kb * kTileKeys + pair + (lane >> 5) * 16, tile_keys - 1);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(
+                    kbase + static_cast<uint64_t>(key) * kD + (lane & 31) * 8),
+                (__attribute__((address_space(3))) void*)(stage + pair * kKeyPairBytes), 16, 0, 0);
+        }
+    };
+    auto stage_values = [&](uint32_t kb) {
+        uint8_t* stage = value_ring + (kb % kRing) * kValueStageBytes;
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            const uint32_t row2 = wave * 2 + i;  // rows 2*row2, 2*row2+1
+            const uint32_t key = min(kb * kTileKeys + row2 * 2 + (lane >> 5), tile_keys - 1);
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(
+                    vbase + static_cast<uint64_t>(key) * kD + (lane & 31) * 8),
+                (__attribute__((address_space(3))) void*)(stage + row2 * 1024), 16, 0, 0);
+        }
+    };
+    // V^T of tile kb: thread (slot group gs, dim pair dp) gathers its 8 keys of two
+    // adjacent dims and writes one 16-byte operand run per dim.  Contraction slot e
+    // of group gs is key (e>>2)*16 + gs*4 + (e&3), the order the S^T accumulators
+    // hand the probabilities over in.
+    auto transpose_values = [&](uint32_t kb) {
+        const uint8_t* raw = value_ring + (kb % kRing) * kValueStageBytes;
+        uint8_t* vt = transposed + (kb & 1) * kTransposedBytes;
+        const uint32_t gs = wave >> 1;
+        const uint32_t dp = (wave & 1) * 64 + lane;
+        uint32_t v[8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t key = (e >> 2) * 16 + gs * 4 + (e & 3);
+            v[e] = *reinterpret_cast<const uint32_t*>(raw + key * 512 + dp * 4);
+        }
+        const u32x4 even = {pack_low(v[0], v[1]), pack_low(v[2], v[3]), pack_low(v[4], v[5]),
+                            pack_low(v[6], v[7])};
+        const u32x4 odd = {pack_high(v[0], v[1]), pack_high(v[2], v[3]), pack_high(v[4], v[5]),
+                           pack_high(v[6], v[7])};
+        *reinterpret_cast<u32x4*>(vt + (2 * dp) * kValueRowBytes + gs * 16) = even;
+        *reinterpret_cast<u32x4*>(vt + (2 * dp + 1) * kValueRowBytes + gs * 16) = odd;
+    };
+
+    f32x4 o[NB][16];
+#pragma unroll
+    for (uint32_t b = 0; b < NB; ++b) {
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) o[b][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    float m_run[NB], l_run[NB];  // reference in log2 units; this lane's share of the row sum
+#pragma unroll
+    for (uint32_t b = 0; b < NB; ++b) {
+        m_run[b] = -INFINITY;
+        l_run[b] = 0.0f;
+    }
+    const float scale = kAttnScale * kLog2e;
+
+    auto scores = [&](uint32_t kb, f32x4 (&s)[2][NB]) {
+        const uint8_t* stage = key_ring + (kb % kRing) * kKeyStageBytes;
+#pragma unroll
+        for (uint32_t kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) s[kt][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (uint32_t kk = 0; kk < 8; ++kk) {
+#pragma unroll
+            for (uint32_t kt = 0; kt < 2; ++kt) {
+                const bf16x8 ka = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kKeyPairBytes + kt * 512 +
+                                                            (kk * 4 + g) * 16));
+#pragma unroll
+                for (uint32_t b = 0; b < NB; ++b) {
+                    s[kt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[b][kk], s[kt][b], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // O^T[dim][pos] += V^T[dim][slot] P^T[slot][pos]; MFMA j covers dims 16j..16j+15
+    auto accumulate = [&](uint32_t kb, const bf16x8 (&pb)[NB]) {
+        const uint8_t* vt = transposed + (kb & 1) * kTransposedBytes;
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const bf16x8 va = __builtin_bit_cast(
+                bf16x8,
+                *reinterpret_cast<const u32x4*>(vt + (j * 16 + m) * kValueRowBytes + g * 16));
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) {
+                o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[b], o[b][j], 0, 0, 0);
+            }
+        }
+    };
+    // exponent arguments of block b against the reference: s*scale - m_run, masked
+    // keys at -inf.  Lane holds keys key0 + kt*16 + g*4 + i of its position column.
+    auto arguments = [&](auto masked, uint32_t kb, const f32x4 (&s)[2][NB], uint32_t b,
+                         float (&x)[8]) {
+#pragma unroll
+        for (uint32_t kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                float v = __builtin_fmaf(s[kt][b][i], scale, -m_run[b]);
+                if (decltype(masked)::value && kb * kTileKeys + kt * 16 + g * 4 + i > limit) {
+                    v = -INFINITY;
+                }
+                x[kt * 4 + i] = v;
+            }
+        }
+    };
+    auto probabilities = [&](const float (&x)[8], bf16x8& pb) -> float {
+        float block_sum = 0.0f;
+        uint32_t pw[4];
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            const float x0 = __builtin_amdgcn_exp2f(x[2 * c]);
+            const float x1 = __builtin_amdgcn_exp2f(x[2 * c + 1]);
+            block_sum += x0 + x1;
+            pw[c] = pack_probabilities(x0, x1);
+        }
+        pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+        return block_sum;
+    };
+    // Exact step of block b: scaled, masked scores; raises the reference to the
+    // tile's maximum; returns the factor O and the row sum are scaled by.
+    auto exact_step = [&](uint32_t kb, const f32x4 (&s)[2][NB], uint32_t b, float (&x)[8]) -> float {
+        float block_max = -INFINITY;
+#pragma unroll
+        for (uint32_t kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                float v = s[kt][b][i] * scale;
+                if (kb * kTileKeys + kt * 16 + g * 4 + i > limit) v = -INFINITY;
+                x[kt * 4 + i] = v;
+                block_max = fmaxf(block_max, v);
+            }
+        }
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
+        const float m_new = fmaxf(m_run[b], block_max);  // key 0 is visible: finite from tile 0 on
+        const float alpha = __builtin_amdgcn_exp2f(m_run[b] - m_new);
+        l_run[b] *= alpha;
+        m_run[b] = m_new;
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) x[e] -= m_new;
+        return alpha;
+    };
+
+    // Batch j, issued on entering tile j: keys of tile j+2, values of tile j+3.
+    stage_values(0);
+    stage_keys(0);
+    stage_values(1);
+    stage_keys(1);
+    stage_values(2);
+    __builtin_amdgcn_s_waitcnt(0x0F78);  // the values of tile 0 have landed
+    __syncthreads();
+    transpose_values(0);
+    // Entering tile kb: batch kb-2 (its keys, the values of tile kb+1) has landed for
+    // every wave and every wave is done with tile kb-1, so the stages batch kb refills
+    // (keys of tile kb-1, raw values of tile kb) and the V^T buffer of tile kb+1 are free.
+    auto enter_tile = [&](uint32_t kb) {
+        __builtin_amdgcn_s_waitcnt(0x0F74);  // all but the 4 transfers of batch kb-1
+        __syncthreads();
+        stage_keys(kb + 2);
+        stage_values(kb + 3);
+        if (kb + 1 < nkb) transpose_values(kb + 1);
+    };
+
+    bf16x8 pb[NB];
+    enter_tile(0);
+    {
+        f32x4 s[2][NB];
+        scores(0, s);
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+            float x[8];
+            (void)exact_step(0, s, b, x);  // O and the sums are still zero
+            l_run[b] += probabilities(x, pb[b]);
+        }
+        accumulate(0, pb);
+    }
+    uint32_t kb = 1;
+    if (kb < nkb) enter_tile(kb);
+    // Steady state: the reference of every row stays where tile 0 put it (scores are
+    // bounded by |q||k|/16 with RMS-normalised q and k), so O is touched by MFMA only.
+    // A score beyond the slack leaves for the exact loop with tile kb entered and not
+    // yet accumulated.
+    auto steady = [&](auto masked, uint32_t end) -> bool {
+        while (kb < end) {
+            f32x4 s[2][NB];
+            scores(kb, s);
+            float sums[NB];
+            bf16x8 next[NB];
+            float top = -INFINITY;
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) {
+                float x[8];
+                arguments(masked, kb, s, b, x);
+                top = fmaxf(top, fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                                       fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]))));
+                sums[b] = probabilities(x, next[b]);
+            }
+            if (__builtin_amdgcn_ballot_w64(top > kReferenceSlack) != 0) return true;
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) l_run[b] += sums[b];
+            accumulate(kb, next);
+            ++kb;
+            if (kb < nkb) enter_tile(kb);
+        }
+        return false;
+    };
+    bool above = steady(std::false_type{}, min(first_masked, nkb));
+    if (!above) above = steady(std::true_type{}, nkb);
+    if (above) {
+        for (;;) {
+            f32x4 s[2][NB];
+            scores(kb, s);
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) {
+                float x[8];
+                const float alpha = exact_step(kb, s, b, x);
+#pragma unroll
+                for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
+                l_run[b] += probabilities(x, pb[b]);
+            }
+            accumulate(kb, pb);
+            ++kb;
+            if (kb == nkb) break;
+            enter_tile(kb);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // transfers of the tiles past the walk
+
+    // out[(row*16 + head)*256 + dim] = bf16((O/l) * sigmoid(gate)); lane holds, for
+    // position column m, dims 16j + 4g + i
+    if (row < a.rows) {
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+            float l = l_run[b];
+            l += __shfl_xor(l, 16, 64);
+            l += __shfl_xor(l, 32, 64);
+            const float inv = 1.0f / l;
+            const uint64_t row_base = (static_cast<uint64_t>(row) * kAttnQueryHeads + head0 + b) * kD;
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const uint32_t dim = j * 16 + g * 4;
+                const u32x2 gw = *reinterpret_cast<const u32x2*>(a.gate + row_base + dim);
+                float r[4];
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    const float gate = __uint_as_float(
+                        (i & 1) ? (gw[i >> 1] & 0xFFFF0000u) : (gw[i >> 1] << 16));
+                    const float sig = 1.0f / (1.0f + __expf(-gate));
+                    r[i] = (o[b][j][i] * inv) * sig;
+                }
+                u32x2 ow;
+                ow[0] = static_cast<uint32_t>(f32_to_bf16_bits(r[0])) |
+                        (static_cast<uint32_t>(f32_to_bf16_bits(r[1])) << 16);
+                ow[1] = static_cast<uint32_t>(f32_to_bf16_bits(r[2])) |
+                        (static_cast<uint32_t>(f32_to_bf16_bits(r[3])) << 16);
+                *reinterpret_cast<u32x2*>(a.out + row_base + dim) = ow;
+            }
+        }
+    }
+}
+
 // --------------------------------------------------- exact control path ------
 
 // attention_partial_blk: grid (16, partitions, tile_rows) x 256; one record
@@ -521,6 +861,12 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     f.gate = a.buffer<const uint16_t>(3, row_bytes);
     f.out = a.buffer<uint16_t>(4, row_bytes);
     if (a.status != TT_OK || validate_only) return a.status;
+    if (kUseWideTile) {
+        hipLaunchKernelGGL(attention_flash_prefill_wide_kernel,
+                           dim3((f.rows + kWidePositions - 1) / kWidePositions, kAttnKvHeads),
+                           dim3(kWideWaves * 64), kWideLdsBytes, stream, f);
+        return TT_OK;
+    }
     hipLaunchKernelGGL(attention_flash_prefill_kernel<kHalves>, dim3(tiles, kAttnKvHeads), dim3(256),
                        kFlashLdsBytes, stream, f);
     return TT_OK;
@@ -587,7 +933,10 @@ int32_t op_attention_combine_blk(const Bindings& b, const Grid& g, hipStream_t s
 bool prepare_prefill_kernels() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel<1>),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kFlashLdsBytes) == hipSuccess;
+                               kFlashLdsBytes) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_wide_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kWideLdsBytes) == hipSuccess;
 }
 
 const KernelDesc kAttentionPrefillKernels[] = {
