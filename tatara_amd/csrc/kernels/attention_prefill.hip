@@ -450,57 +450,63 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
         }
     }
 
-    const uint16_t* kbase = a.keys + static_cast<uint64_t>(kvh) * a.capacity * kD;
-    const uint16_t* vbase = a.values + static_cast<uint64_t>(kvh) * a.capacity * kD;
+    // byte addresses inside one kv head stay below 2^32 (capacity * 512 B)
+    const uint8_t* kbase =
+        reinterpret_cast<const uint8_t*>(a.keys + static_cast<uint64_t>(kvh) * a.capacity * kD);
+    const uint8_t* vbase =
+        reinterpret_cast<const uint8_t*>(a.values + static_cast<uint64_t>(kvh) * a.capacity * kD);
+    const uint32_t last_key = tile_keys - 1;
+    const uint32_t column_bytes = (lane & 31) * 16;
+    // staging addresses are wave-uniform: give the compiler the wave index as a scalar
+    const uint32_t swave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t key_lane = swave * 2 + (lane >> 5) * 16;    // + i: key pair 2w+i, second half +16
+    const uint32_t value_lane = swave * 4 + (lane >> 5);       // + 2i: rows 4w+2i, 4w+2i+1
 
     // Each wave moves an eighth of a tile: 2 K transfers (key pairs 2w, 2w+1) and 2 V
     // transfers (rows 4w..4w+3), 1 KiB each.  Tiles past the walk re-read the last
     // key, so every batch has the same number of transfers.
-    auto stage_keys = [&](uint32_t kb) {
-        uint8_t* stage = key_ring + (kb % kRing) * kKeyStageBytes;
+    auto stage_keys = [&](uint32_t kb, uint32_t slot) {
+        uint8_t* stage = key_ring + slot * kKeyStageBytes + swave * 2 * kKeyPairBytes;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
-            const uint32_t pair = wave * 2 + i;
-            const uint32_t key = min(kb * kTileKeys + pair + (lane >> 5) * 16, tile_keys - 1);
+            const uint32_t key = min(kb * kTileKeys + i + key_lane, last_key);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(
-                    kbase + static_cast<uint64_t>(key) * kD + (lane & 31) * 8),
-                (__attribute__((address_space(3))) void*)(stage + pair * kKeyPairBytes), 16, 0, 0);
+                (const __attribute__((address_space(1))) void*)(kbase + (key * 512u + column_bytes)),
+                (__attribute__((address_space(3))) void*)(stage + i * kKeyPairBytes), 16, 0, 0);
         }
     };
-    auto stage_values = [&](uint32_t kb) {
-        uint8_t* stage = value_ring + (kb % kRing) * kValueStageBytes;
+    auto stage_values = [&](uint32_t kb, uint32_t slot) {
+        uint8_t* stage = value_ring + slot * kValueStageBytes + swave * 2048;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
-            const uint32_t row2 = wave * 2 + i;  // rows 2*row2, 2*row2+1
-            const uint32_t key = min(kb * kTileKeys + row2 * 2 + (lane >> 5), tile_keys - 1);
+            const uint32_t key = min(kb * kTileKeys + 2 * i + value_lane, last_key);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(
-                    vbase + static_cast<uint64_t>(key) * kD + (lane & 31) * 8),
-                (__attribute__((address_space(3))) void*)(stage + row2 * 1024), 16, 0, 0);
+                (const __attribute__((address_space(1))) void*)(vbase + (key * 512u + column_bytes)),
+                (__attribute__((address_space(3))) void*)(stage + i * 1024), 16, 0, 0);
         }
     };
-    // V^T of tile kb: thread (slot group gs, dim pair dp) gathers its 8 keys of two
+    // V^T of a tile: thread (slot group gs, dim pair dp) gathers its 8 keys of two
     // adjacent dims and writes one 16-byte operand run per dim.  Contraction slot e
     // of group gs is key (e>>2)*16 + gs*4 + (e&3), the order the S^T accumulators
     // hand the probabilities over in.
-    auto transpose_values = [&](uint32_t kb) {
-        const uint8_t* raw = value_ring + (kb % kRing) * kValueStageBytes;
-        uint8_t* vt = transposed + (kb & 1) * kTransposedBytes;
-        const uint32_t gs = wave >> 1;
-        const uint32_t dp = (wave & 1) * 64 + lane;
+    const uint32_t gs = wave >> 1;
+    const uint32_t dp = (wave & 1) * 64 + lane;
+    const uint32_t gather_bytes = gs * 4 * 512 + dp * 4;
+    const uint32_t scatter_bytes = 2 * dp * kValueRowBytes + gs * 16;
+    auto transpose_values = [&](uint32_t slot, uint32_t parity) {
+        const uint8_t* raw = value_ring + slot * kValueStageBytes + gather_bytes;
+        uint8_t* vt = transposed + parity * kTransposedBytes + scatter_bytes;
         uint32_t v[8];
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) {
-            const uint32_t key = (e >> 2) * 16 + gs * 4 + (e & 3);
-            v[e] = *reinterpret_cast<const uint32_t*>(raw + key * 512 + dp * 4);
+            v[e] = *reinterpret_cast<const uint32_t*>(raw + ((e >> 2) * 16 + (e & 3)) * 512);
         }
         const u32x4 even = {pack_low(v[0], v[1]), pack_low(v[2], v[3]), pack_low(v[4], v[5]),
                             pack_low(v[6], v[7])};
         const u32x4 odd = {pack_high(v[0], v[1]), pack_high(v[2], v[3]), pack_high(v[4], v[5]),
                            pack_high(v[6], v[7])};
-        *reinterpret_cast<u32x4*>(vt + (2 * dp) * kValueRowBytes + gs * 16) = even;
-        *reinterpret_cast<u32x4*>(vt + (2 * dp + 1) * kValueRowBytes + gs * 16) = odd;
+        *reinterpret_cast<u32x4*>(vt) = even;
+        *reinterpret_cast<u32x4*>(vt + kValueRowBytes) = odd;
     };
 
     f32x4 o[NB][16];
@@ -517,38 +523,50 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     }
     const float scale = kAttnScale * kLog2e;
 
-    auto scores = [&](uint32_t kb, f32x4 (&s)[2][NB]) {
-        const uint8_t* stage = key_ring + (kb % kRing) * kKeyStageBytes;
+    const uint32_t key_read_bytes = m * kKeyPairBytes + g * 16;
+    const uint32_t value_read_bytes = m * kValueRowBytes + g * 16;
+    // S^T of the tile in key stage `slot`; operand reads run one contraction step ahead
+    auto scores = [&](uint32_t slot, f32x4 (&s)[2][NB]) {
+        const uint8_t* stage = key_ring + slot * kKeyStageBytes + key_read_bytes;
 #pragma unroll
         for (uint32_t kt = 0; kt < 2; ++kt) {
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) s[kt][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
+        u32x4 ka[2][2];
+        ka[0][0] = *reinterpret_cast<const u32x4*>(stage);
+        ka[0][1] = *reinterpret_cast<const u32x4*>(stage + 512);
 #pragma unroll
         for (uint32_t kk = 0; kk < 8; ++kk) {
+            if (kk + 1 < 8) {
+                ka[(kk + 1) & 1][0] = *reinterpret_cast<const u32x4*>(stage + (kk + 1) * 64);
+                ka[(kk + 1) & 1][1] = *reinterpret_cast<const u32x4*>(stage + (kk + 1) * 64 + 512);
+            }
 #pragma unroll
             for (uint32_t kt = 0; kt < 2; ++kt) {
-                const bf16x8 ka = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kKeyPairBytes + kt * 512 +
-                                                            (kk * 4 + g) * 16));
 #pragma unroll
                 for (uint32_t b = 0; b < NB; ++b) {
-                    s[kt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[b][kk], s[kt][b], 0, 0, 0);
+                    s[kt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, ka[kk & 1][kt]), q[b][kk], s[kt][b], 0, 0, 0);
                 }
             }
         }
     };
     // O^T[dim][pos] += V^T[dim][slot] P^T[slot][pos]; MFMA j covers dims 16j..16j+15
-    auto accumulate = [&](uint32_t kb, const bf16x8 (&pb)[NB]) {
-        const uint8_t* vt = transposed + (kb & 1) * kTransposedBytes;
+    auto accumulate = [&](uint32_t parity, const bf16x8 (&pb)[NB]) {
+        const uint8_t* vt = transposed + parity * kTransposedBytes + value_read_bytes;
+        u32x4 va[2];
+        va[0] = *reinterpret_cast<const u32x4*>(vt);
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
-            const bf16x8 va = __builtin_bit_cast(
-                bf16x8,
-                *reinterpret_cast<const u32x4*>(vt + (j * 16 + m) * kValueRowBytes + g * 16));
+            if (j + 1 < 16) {
+                va[(j + 1) & 1] =
+                    *reinterpret_cast<const u32x4*>(vt + (j + 1) * 16 * kValueRowBytes);
+            }
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) {
-                o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[b], o[b][j], 0, 0, 0);
+                o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, va[j & 1]), pb[b], o[b][j], 0, 0, 0);
             }
         }
     };
@@ -607,30 +625,42 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     };
 
     // Batch j, issued on entering tile j: keys of tile j+2, values of tile j+3.
-    stage_values(0);
-    stage_keys(0);
-    stage_values(1);
-    stage_keys(1);
-    stage_values(2);
+    stage_values(0, 0);
+    stage_keys(0, 0);
+    stage_values(1, 1);
+    stage_keys(1, 1);
+    stage_values(2, 2);
     __builtin_amdgcn_s_waitcnt(0x0F78);  // the values of tile 0 have landed
     __syncthreads();
-    transpose_values(0);
+    transpose_values(0, 0);
+    // Ring positions of the tile being entered: kslot = kb % 3 (its keys; tile kb+2
+    // goes to (kb+2) % 3), vslot = (kb+1) % 3 (raw values of tile kb+1, transposed now;
+    // tile kb+3 goes to kb % 3 = kslot).
+    uint32_t kb = 0;
+    uint32_t kslot = 0;
     // Entering tile kb: batch kb-2 (its keys, the values of tile kb+1) has landed for
     // every wave and every wave is done with tile kb-1, so the stages batch kb refills
     // (keys of tile kb-1, raw values of tile kb) and the V^T buffer of tile kb+1 are free.
-    auto enter_tile = [&](uint32_t kb) {
+    auto enter_tile = [&]() {
+        const uint32_t next = kslot == kRing - 1 ? 0 : kslot + 1;   // (kb+1) % 3
+        const uint32_t prev = kslot == 0 ? kRing - 1 : kslot - 1;   // (kb+2) % 3
         __builtin_amdgcn_s_waitcnt(0x0F74);  // all but the 4 transfers of batch kb-1
         __syncthreads();
-        stage_keys(kb + 2);
-        stage_values(kb + 3);
-        if (kb + 1 < nkb) transpose_values(kb + 1);
+        stage_keys(kb + 2, prev);
+        stage_values(kb + 3, kslot);
+        if (kb + 1 < nkb) transpose_values(next, (kb + 1) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto advance = [&]() {
+        ++kb;
+        kslot = kslot == kRing - 1 ? 0 : kslot + 1;
     };
 
     bf16x8 pb[NB];
-    enter_tile(0);
+    enter_tile();
     {
         f32x4 s[2][NB];
-        scores(0, s);
+        scores(kslot, s);
 #pragma unroll
         for (uint32_t b = 0; b < NB; ++b) {
             float x[8];
@@ -639,8 +669,8 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
         }
         accumulate(0, pb);
     }
-    uint32_t kb = 1;
-    if (kb < nkb) enter_tile(kb);
+    advance();
+    if (kb < nkb) enter_tile();
     // Steady state: the reference of every row stays where tile 0 put it (scores are
     // bounded by |q||k|/16 with RMS-normalised q and k), so O is touched by MFMA only.
     // A score beyond the slack leaves for the exact loop with tile kb entered and not
@@ -648,7 +678,8 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     auto steady = [&](auto masked, uint32_t end) -> bool {
         while (kb < end) {
             f32x4 s[2][NB];
-            scores(kb, s);
+            scores(kslot, s);
+            __builtin_amdgcn_sched_barrier(0);
             float sums[NB];
             bf16x8 next[NB];
             float top = -INFINITY;
@@ -663,9 +694,10 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
             if (__builtin_amdgcn_ballot_w64(top > kReferenceSlack) != 0) return true;
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) l_run[b] += sums[b];
-            accumulate(kb, next);
-            ++kb;
-            if (kb < nkb) enter_tile(kb);
+            __builtin_amdgcn_sched_barrier(0);
+            accumulate(kb & 1, next);
+            advance();
+            if (kb < nkb) enter_tile();
         }
         return false;
     };
@@ -674,7 +706,7 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     if (above) {
         for (;;) {
             f32x4 s[2][NB];
-            scores(kb, s);
+            scores(kslot, s);
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) {
                 float x[8];
@@ -683,10 +715,10 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
                 for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
                 l_run[b] += probabilities(x, pb[b]);
             }
-            accumulate(kb, pb);
-            ++kb;
+            accumulate(kb & 1, pb);
+            advance();
             if (kb == nkb) break;
-            enter_tile(kb);
+            enter_tile();
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // transfers of the tiles past the walk
