@@ -73,6 +73,19 @@ __device__ __forceinline__ uint32_t pack_probabilities(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
+// One 1 KiB transfer HBM/L2 -> LDS: lane l's 16 bytes at base + offset go to LDS byte
+// lds_address + 16 l.  Issued as assembly so that the waits on these transfers are
+// exactly the s_waitcnt instructions written in the kernel: the compiler, seeing an
+// LDS-writing load, would otherwise drain every transfer in flight before the next
+// LDS read of the same array.
+__device__ __forceinline__ void transfer_to_lds(const uint8_t* base, uint32_t offset,
+                                                uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(offset), "s"(base)
+                 : "memory");
+}
+
 struct FlashPrefillArgs {
     const uint16_t* query;   // [rows][16][256]
     const uint16_t* gate;    // [rows][16][256]
@@ -456,6 +469,8 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     const uint8_t* vbase =
         reinterpret_cast<const uint8_t*>(a.values + static_cast<uint64_t>(kvh) * a.capacity * kD);
     const uint32_t last_key = tile_keys - 1;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint8_t*)lds));  // LDS byte address of the key ring
     const uint32_t column_bytes = (lane & 31) * 16;
     // staging addresses are wave-uniform: give the compiler the wave index as a scalar
     const uint32_t swave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -466,23 +481,19 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     // transfers (rows 4w..4w+3), 1 KiB each.  Tiles past the walk re-read the last
     // key, so every batch has the same number of transfers.
     auto stage_keys = [&](uint32_t kb, uint32_t slot) {
-        uint8_t* stage = key_ring + slot * kKeyStageBytes + swave * 2 * kKeyPairBytes;
+        const uint32_t stage = lds_base + slot * kKeyStageBytes + swave * 2 * kKeyPairBytes;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             const uint32_t key = min(kb * kTileKeys + i + key_lane, last_key);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(kbase + (key * 512u + column_bytes)),
-                (__attribute__((address_space(3))) void*)(stage + i * kKeyPairBytes), 16, 0, 0);
+            transfer_to_lds(kbase, key * 512u + column_bytes, stage + i * kKeyPairBytes);
         }
     };
     auto stage_values = [&](uint32_t kb, uint32_t slot) {
-        uint8_t* stage = value_ring + slot * kValueStageBytes + swave * 2048;
+        const uint32_t stage = lds_base + kKeyRingBytes + slot * kValueStageBytes + swave * 2048;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             const uint32_t key = min(kb * kTileKeys + 2 * i + value_lane, last_key);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(vbase + (key * 512u + column_bytes)),
-                (__attribute__((address_space(3))) void*)(stage + i * 1024), 16, 0, 0);
+            transfer_to_lds(vbase, key * 512u + column_bytes, stage + i * 1024);
         }
     };
     // V^T of a tile: thread (slot group gs, dim pair dp) gathers its 8 keys of two
