@@ -406,22 +406,27 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
 // blocks that share every K and V fragment the wave reads from LDS.  Two waves per
 // SIMD (256 registers each): one wave's softmax (VALU) runs under the other's
 // products (MFMA), and LDS operand reads are issued from eight waves.
-//   K tiles: HBM/L2 -> LDS ring of 3 stages, two tiles ahead (global_load_lds).
-//   V tiles: HBM/L2 -> raw LDS ring of 3 stages, three tiles ahead; one tile ahead
-//   of its use the 512 lanes transpose it once into V^T[dim][key slot] (80-byte
-//   rows: conflict-free 16-byte operand reads), so a wave's V^T operands are plain
-//   LDS reads instead of 64 register permutes per wave and tile.
+//   K and V tiles: HBM/L2 -> LDS rings of 3 stages, two tiles ahead (global_load_lds).
+//   Both are stored as 16 row pairs (row i | row 16+i | pad): K pairs of 1040 bytes so
+//   the 16-byte S^T operand reads are conflict-free, V pairs of 1056 bytes so that the
+//   eight rows one half-wave touches in a transposing read fall into eight different
+//   32-byte bank groups.
+//   V^T operands come straight from the row-major V stage with ds_read_b64_tr_b16:
+//   16 lanes hand in the addresses of 4 key rows x 16 dims (4 lanes per row, 4 dims
+//   each) and lane i receives dim i of the 4 rows - two such reads are the 8 contraction
+//   slots of one MFMA operand, no register permutes and no transposed copy in LDS.
 // One barrier per tile.  Softmax as in the 16-position kernel: reference fixed by
 // tile 0, exact online loop as the way out.
 constexpr bool kUseWideTile = true;
 constexpr uint32_t kWideWaves = 8;
 constexpr uint32_t kWidePositions = 32;
 constexpr uint32_t kRing = 3;
-constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;      // 49920
-constexpr uint32_t kValueRingBytes = kRing * kValueStageBytes;  // 49152
-constexpr uint32_t kValueRowBytes = 80;                         // 32 key slots of one dim + pad
-constexpr uint32_t kTransposedBytes = kD * kValueRowBytes;      // 20480
-constexpr uint32_t kWideLdsBytes = kKeyRingBytes + kValueRingBytes + 2 * kTransposedBytes;
+constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 49920
+constexpr uint32_t kValuePairBytes = 1056;                             // row i | row 16+i | 32 B pad
+constexpr uint32_t kValuePairedStageBytes = 16 * kValuePairBytes;      // 16896
+constexpr uint32_t kWideLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 100608
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 __global__ __launch_bounds__(kWideWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
@@ -429,7 +434,6 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t* const key_ring = lds;
     uint8_t* const value_ring = lds + kKeyRingBytes;
-    uint8_t* const transposed = value_ring + kValueRingBytes;
     // longest key walks first: the last position tile is dispatched first
     const uint32_t tile = gridDim.x - 1 - blockIdx.x;
     const uint32_t kvh = blockIdx.y;
@@ -474,50 +478,25 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     const uint32_t column_bytes = (lane & 31) * 16;
     // staging addresses are wave-uniform: give the compiler the wave index as a scalar
     const uint32_t swave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t key_lane = swave * 2 + (lane >> 5) * 16;    // + i: key pair 2w+i, second half +16
-    const uint32_t value_lane = swave * 4 + (lane >> 5);       // + 2i: rows 4w+2i, 4w+2i+1
+    const uint32_t key_lane = swave * 2 + (lane >> 5) * 16;    // + i: row pair 2w+i, second half +16
 
-    // Each wave moves an eighth of a tile: 2 K transfers (key pairs 2w, 2w+1) and 2 V
-    // transfers (rows 4w..4w+3), 1 KiB each.  Tiles past the walk re-read the last
-    // key, so every batch has the same number of transfers.
-    auto stage_keys = [&](uint32_t kb, uint32_t slot) {
-        const uint32_t stage = lds_base + slot * kKeyStageBytes + swave * 2 * kKeyPairBytes;
+    // Each wave moves an eighth of a tile: 2 K transfers and 2 V transfers (row pairs
+    // 2w, 2w+1), 1 KiB each.  Tiles past the walk re-read the last key, so every batch
+    // has the same number of transfers.
+    auto stage_tile = [&](uint32_t kb, uint32_t slot) {
+        const uint32_t kstage = lds_base + slot * kKeyStageBytes + swave * 2 * kKeyPairBytes;
+        const uint32_t vstage =
+            lds_base + kKeyRingBytes + slot * kValuePairedStageBytes + swave * 2 * kValuePairBytes;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             const uint32_t key = min(kb * kTileKeys + i + key_lane, last_key);
-            transfer_to_lds(kbase, key * 512u + column_bytes, stage + i * kKeyPairBytes);
+            transfer_to_lds(kbase, key * 512u + column_bytes, kstage + i * kKeyPairBytes);
         }
-    };
-    auto stage_values = [&](uint32_t kb, uint32_t slot) {
-        const uint32_t stage = lds_base + kKeyRingBytes + slot * kValueStageBytes + swave * 2048;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
-            const uint32_t key = min(kb * kTileKeys + 2 * i + value_lane, last_key);
-            transfer_to_lds(vbase, key * 512u + column_bytes, stage + i * 1024);
+            const uint32_t key = min(kb * kTileKeys + i + key_lane, last_key);
+            transfer_to_lds(vbase, key * 512u + column_bytes, vstage + i * kValuePairBytes);
         }
-    };
-    // V^T of a tile: thread (slot group gs, dim pair dp) gathers its 8 keys of two
-    // adjacent dims and writes one 16-byte operand run per dim.  Contraction slot e
-    // of group gs is key (e>>2)*16 + gs*4 + (e&3), the order the S^T accumulators
-    // hand the probabilities over in.
-    const uint32_t gs = wave >> 1;
-    const uint32_t dp = (wave & 1) * 64 + lane;
-    const uint32_t gather_bytes = gs * 4 * 512 + dp * 4;
-    const uint32_t scatter_bytes = 2 * dp * kValueRowBytes + gs * 16;
-    auto transpose_values = [&](uint32_t slot, uint32_t parity) {
-        const uint8_t* raw = value_ring + slot * kValueStageBytes + gather_bytes;
-        uint8_t* vt = transposed + parity * kTransposedBytes + scatter_bytes;
-        uint32_t v[8];
-#pragma unroll
-        for (uint32_t e = 0; e < 8; ++e) {
-            v[e] = *reinterpret_cast<const uint32_t*>(raw + ((e >> 2) * 16 + (e & 3)) * 512);
-        }
-        const u32x4 even = {pack_low(v[0], v[1]), pack_low(v[2], v[3]), pack_low(v[4], v[5]),
-                            pack_low(v[6], v[7])};
-        const u32x4 odd = {pack_high(v[0], v[1]), pack_high(v[2], v[3]), pack_high(v[4], v[5]),
-                           pack_high(v[6], v[7])};
-        *reinterpret_cast<u32x4*>(vt) = even;
-        *reinterpret_cast<u32x4*>(vt + kValueRowBytes) = odd;
     };
 
     f32x4 o[NB][16];
@@ -535,7 +514,6 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     const float scale = kAttnScale * kLog2e;
 
     const uint32_t key_read_bytes = m * kKeyPairBytes + g * 16;
-    const uint32_t value_read_bytes = m * kValueRowBytes + g * 16;
     // S^T of the tile in key stage `slot`; operand reads run one contraction step ahead
     auto scores = [&](uint32_t slot, f32x4 (&s)[2][NB]) {
         const uint8_t* stage = key_ring + slot * kKeyStageBytes + key_read_bytes;
@@ -563,17 +541,28 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
             }
         }
     };
-    // O^T[dim][pos] += V^T[dim][slot] P^T[slot][pos]; MFMA j covers dims 16j..16j+15
-    auto accumulate = [&](uint32_t parity, const bf16x8 (&pb)[NB]) {
-        const uint8_t* vt = transposed + parity * kTransposedBytes + value_read_bytes;
+    // O^T[dim][pos] += V^T[dim][slot] P^T[slot][pos]; MFMA j covers dims 16j..16j+15.
+    // Contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3), the order the
+    // S^T accumulators hand the probabilities over in: lane (m, g) points at key row
+    // g*4 + (m>>2), dims 16j + 4(m&3)..+3, once in the low and once in the high half
+    // of the row pairs.
+    const uint32_t value_read_bytes = (g * 4 + (m >> 2)) * kValuePairBytes + (m & 3) * 8;
+    auto read_values = [&](const uint8_t* at) -> u32x4 {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(at));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(at + 512));
+        const u32x2 l = __builtin_bit_cast(u32x2, lo);
+        const u32x2 h = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l[0], l[1], h[0], h[1]};
+    };
+    auto accumulate = [&](uint32_t slot, const bf16x8 (&pb)[NB]) {
+        const uint8_t* vt = value_ring + slot * kValuePairedStageBytes + value_read_bytes;
         u32x4 va[2];
-        va[0] = *reinterpret_cast<const u32x4*>(vt);
+        va[0] = read_values(vt);
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
-            if (j + 1 < 16) {
-                va[(j + 1) & 1] =
-                    *reinterpret_cast<const u32x4*>(vt + (j + 1) * 16 * kValueRowBytes);
-            }
+            if (j + 1 < 16) va[(j + 1) & 1] = read_values(vt + (j + 1) * 32);
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) {
                 o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
@@ -635,31 +624,19 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
         return alpha;
     };
 
-    // Batch j, issued on entering tile j: keys of tile j+2, values of tile j+3.
-    stage_values(0, 0);
-    stage_keys(0, 0);
-    stage_values(1, 1);
-    stage_keys(1, 1);
-    stage_values(2, 2);
-    __builtin_amdgcn_s_waitcnt(0x0F78);  // the values of tile 0 have landed
-    __syncthreads();
-    transpose_values(0, 0);
-    // Ring positions of the tile being entered: kslot = kb % 3 (its keys; tile kb+2
-    // goes to (kb+2) % 3), vslot = (kb+1) % 3 (raw values of tile kb+1, transposed now;
-    // tile kb+3 goes to kb % 3 = kslot).
+    // Batch j, issued on entering tile j: keys and values of tile j+2.
+    stage_tile(0, 0);
+    stage_tile(1, 1);
+    // Ring position of the tile being entered: kslot = kb % 3; tile kb+2 goes to
+    // (kb+2) % 3, the stage tile kb-1 has just left.
     uint32_t kb = 0;
     uint32_t kslot = 0;
-    // Entering tile kb: batch kb-2 (its keys, the values of tile kb+1) has landed for
-    // every wave and every wave is done with tile kb-1, so the stages batch kb refills
-    // (keys of tile kb-1, raw values of tile kb) and the V^T buffer of tile kb+1 are free.
+    // Entering tile kb: batch kb-2 (this tile) has landed for every wave and every wave
+    // is done with tile kb-1.
     auto enter_tile = [&]() {
-        const uint32_t next = kslot == kRing - 1 ? 0 : kslot + 1;   // (kb+1) % 3
-        const uint32_t prev = kslot == 0 ? kRing - 1 : kslot - 1;   // (kb+2) % 3
         __builtin_amdgcn_s_waitcnt(0x0F74);  // all but the 4 transfers of batch kb-1
         __syncthreads();
-        stage_keys(kb + 2, prev);
-        stage_values(kb + 3, kslot);
-        if (kb + 1 < nkb) transpose_values(next, (kb + 1) & 1);
+        stage_tile(kb + 2, kslot == 0 ? kRing - 1 : kslot - 1);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto advance = [&]() {
@@ -678,7 +655,7 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
             (void)exact_step(0, s, b, x);  // O and the sums are still zero
             l_run[b] += probabilities(x, pb[b]);
         }
-        accumulate(0, pb);
+        accumulate(kslot, pb);
     }
     advance();
     if (kb < nkb) enter_tile();
@@ -706,7 +683,7 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) l_run[b] += sums[b];
             __builtin_amdgcn_sched_barrier(0);
-            accumulate(kb & 1, next);
+            accumulate(kslot, next);
             advance();
             if (kb < nkb) enter_tile();
         }
@@ -726,7 +703,7 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
                 for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
                 l_run[b] += probabilities(x, pb[b]);
             }
-            accumulate(kb & 1, pb);
+            accumulate(kslot, pb);
             advance();
             if (kb == nkb) break;
             enter_tile();
