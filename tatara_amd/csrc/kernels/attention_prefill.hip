@@ -1,5 +1,5 @@
 // Block-prefill full attention for gfx950: causal flash attention on bf16 MFMA
-// with K/V tiles double-buffered in LDS, plus the exact partial/combine control
+// with K/V tiles staged through LDS rings, plus the exact partial/combine control
 // path.
 //
 // Operators registered here, with the reference kernels whose argument tables
@@ -8,23 +8,14 @@
 //   attention_streaming_blk (:860), attention_flash_v2_blk (:1233)  -> flash kernel
 //   attention_partial_blk (:97), attention_combine_blk (:207)        -> control path
 //
-// Flash kernel.  One workgroup = 4 wave64 = 32 consecutive query positions x
-// the 8 query heads of one kv head (256 score rows); wave w owns heads 2w and
-// 2w+1 at both 16-position halves, four 16x16 blocks that share every K and V
-// fragment read from LDS.  Keys are walked in tiles of 32 up to the causal
-// limit of the tile.  The four waves share each K/V tile through LDS: HBM/L2
-// fills stages two tiles ahead directly (global_load_lds, no registers), four
-// stages of 32.25 KiB each, one barrier per tile.
+// Flash kernel, in short (details above the kernel): one workgroup = 8 wave64 = 32
+// consecutive query positions x the 8 query heads of one kv head; keys are walked
+// in tiles of 32 up to the causal limit of the position tile.
 //   S^T[key][pos] = K[key][:] . Q[pos][:]    v_mfma_f32_16x16x32_bf16,
 //       A = K from LDS, B = Q^T held in registers for the whole walk.
 //   O^T[dim][pos] += V^T[dim][key] P^T[key][pos]
-//       A = V^T: each lane reads 16-byte runs of 8 value rows from LDS and
-//       transposes 8x8 in registers (v_perm_b32), shared by the wave's four
-//       blocks; B = P^T = bf16 of the S^T accumulators, no LDS round trip.
-// The loop is skewed by one tile: the softmax of tile kb (VALU) sits next to
-// the PV products of tile kb-1 (MFMA) so the two pipes overlap.  The running
-// maximum is only raised when a tile exceeds it by more than 2^8, so the
-// 256-register rescale of O is rare; probabilities then reach at most 2^8.
+//       A = V^T read from the row-major V stage with the transposing LDS load,
+//       B = P^T = bf16 of the S^T accumulators, no LDS round trip.
 // Row r of the dispatch sees keys [0, tile_context + r], which makes every row
 // a decode step at context tile_context + r over the same cache
 // (prefill_attention.metal:117-119).  Algorithmic work: 1024 flop per visible
@@ -45,10 +36,6 @@ constexpr uint32_t kD = kAttnHeadDim;
 constexpr uint32_t kTileKeys = 32;
 constexpr uint32_t kKeyPairBytes = 1040;                 // key i | key 16+i | 16 B pad
 constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16640
-constexpr uint32_t kValueStageBytes = kTileKeys * 512;   // 16384
-constexpr uint32_t kStageBytes = kKeyStageBytes + kValueStageBytes;
-constexpr uint32_t kStages = 4;
-constexpr uint32_t kFlashLdsBytes = kStages * kStageBytes;  // 132096
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kReferenceSlack = 100.0f;  // log2 units a score may exceed the fixed reference by
 
@@ -59,12 +46,6 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {
     const uint32_t b = __float_as_uint(v);
     if ((b & 0x7F800000u) == 0x7F800000u) return static_cast<uint16_t>(b >> 16);
     return static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
-}
-__device__ __forceinline__ uint32_t pack_low(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_perm(b, a, 0x05040100u);
-}
-__device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
-    return __builtin_amdgcn_perm(b, a, 0x07060302u);
 }
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
@@ -97,309 +78,7 @@ struct FlashPrefillArgs {
     uint32_t capacity;
 };
 
-// PH = 16-position halves per workgroup; a wave owns NB = 2*PH blocks.
-template <uint32_t PH>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void attention_flash_prefill_kernel(FlashPrefillArgs a) {
-    constexpr uint32_t NB = 2 * PH;
-    constexpr uint32_t kTilePositions = 16 * PH;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    // longest key walks first: the last position tile is dispatched first
-    const uint32_t tile = gridDim.x - 1 - blockIdx.x;
-    const uint32_t kvh = blockIdx.y;
-    const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t m = lane & 15;
-    const uint32_t g = lane >> 4;
-    const uint32_t p0 = tile * kTilePositions;
-    const uint32_t tile_keys = a.tile_context + min(p0 + kTilePositions, a.rows);  // visible count
-    const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
-
-    // block b = 2*t + ph: head 2*wave + t, positions p0 + 16*ph + (column n = m).
-    // B operand of S^T: Q^T, held for the whole walk.
-    bf16x8 q[NB][8];
-    uint32_t limit[PH];  // last visible key of this lane's column in each position half
-#pragma unroll
-    for (uint32_t ph = 0; ph < PH; ++ph) {
-        limit[ph] = a.tile_context + p0 + ph * 16 + m;
-        const uint32_t pos = min(p0 + ph * 16 + m, a.rows - 1);
-#pragma unroll
-        for (uint32_t t = 0; t < 2; ++t) {
-            const uint16_t* qrow = a.query + (static_cast<uint64_t>(pos) * kAttnQueryHeads +
-                                              kvh * kAttnHeadsPerKv + wave * 2 + t) * kD;
-#pragma unroll
-            for (uint32_t kb = 0; kb < 8; ++kb) {
-                q[t * PH + ph][kb] = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const u32x4*>(qrow + kb * 32 + g * 8));
-            }
-        }
-    }
-
-    const uint16_t* kbase = a.keys + static_cast<uint64_t>(kvh) * a.capacity * kD;
-    const uint16_t* vbase = a.values + static_cast<uint64_t>(kvh) * a.capacity * kD;
-
-    // each wave moves a quarter of a tile: 4 K transfers (key pairs 4w..4w+3) and
-    // 4 V transfers (rows 8w..8w+7), 1 KiB each
-    auto stage_tile = [&](uint32_t kb) {
-        uint8_t* kstage = lds + (kb % kStages) * kStageBytes;
-        uint8_t* vstage = kstage + kKeyStageBytes;
-        const uint32_t key0 = kb * kTileKeys;
-        const uint32_t last = tile_keys - 1 - key0;  // rows past the walk repeat the last key
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            const uint32_t pair = wave * 4 + i;
-            const uint32_t key = min(pair + (lane >> 5) * 16, last);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(
-                    kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8),
-                (__attribute__((address_space(3))) void*)(kstage + pair * kKeyPairBytes), 16, 0, 0);
-        }
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            const uint32_t row2 = wave * 4 + i;  // rows 2*row2, 2*row2+1
-            const uint32_t key = min(row2 * 2 + (lane >> 5), last);
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(
-                    vbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8),
-                (__attribute__((address_space(3))) void*)(vstage + row2 * 1024), 16, 0, 0);
-        }
-    };
-
-    f32x4 o[NB][16];
-#pragma unroll
-    for (uint32_t b = 0; b < NB; ++b) {
-#pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) o[b][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    float m_run[NB], l_run[NB];  // maximum in log2 units; this lane's share of the row sum
-#pragma unroll
-    for (uint32_t b = 0; b < NB; ++b) {
-        m_run[b] = -INFINITY;
-        l_run[b] = 0.0f;
-    }
-    const float scale = kAttnScale * kLog2e;
-
-    // S^T of tile kb for the wave's four blocks
-    auto scores = [&](uint32_t kb, f32x4 (&s)[2][NB]) {
-        const uint8_t* kstage = lds + (kb % kStages) * kStageBytes;
-#pragma unroll
-        for (uint32_t kt = 0; kt < 2; ++kt) {
-#pragma unroll
-            for (uint32_t b = 0; b < NB; ++b) s[kt][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        }
-#pragma unroll
-        for (uint32_t kk = 0; kk < 8; ++kk) {
-#pragma unroll
-            for (uint32_t kt = 0; kt < 2; ++kt) {
-                const bf16x8 ka = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const u32x4*>(kstage + m * kKeyPairBytes + kt * 512 +
-                                                            (kk * 4 + g) * 16));
-#pragma unroll
-                for (uint32_t b = 0; b < NB; ++b) {
-                    s[kt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, q[b][kk], s[kt][b], 0, 0, 0);
-                }
-            }
-        }
-    };
-
-    // Scaled and masked scores of tile kb for block b.  Lane holds keys
-    // key0 + kt*16 + g*4 + i of its position column.
-    auto scaled = [&](uint32_t kb, const f32x4 (&s)[2][NB], uint32_t b, float (&sc)[8]) {
-        const uint32_t key0 = kb * kTileKeys;
-        const bool needs_mask = key0 + kTileKeys - 1 > a.tile_context + p0;
-#pragma unroll
-        for (uint32_t kt = 0; kt < 2; ++kt) {
-#pragma unroll
-            for (uint32_t i = 0; i < 4; ++i) {
-                float v = s[kt][b][i] * scale;
-                if (needs_mask && key0 + kt * 16 + g * 4 + i > limit[b % PH]) v = -INFINITY;
-                sc[kt * 4 + i] = v;
-            }
-        }
-    };
-    // P^T operand of block b against the reference m_run[b]; returns this lane's
-    // share of the tile's row sum
-    auto probabilities = [&](const float (&sc)[8], uint32_t b, bf16x8& pb) -> float {
-        float block_sum = 0.0f;
-        uint32_t pw[4];
-#pragma unroll
-        for (uint32_t c = 0; c < 4; ++c) {
-            const float x0 = __builtin_amdgcn_exp2f(sc[2 * c] - m_run[b]);
-            const float x1 = __builtin_amdgcn_exp2f(sc[2 * c + 1] - m_run[b]);
-            block_sum += x0 + x1;
-            pw[c] = pack_probabilities(x0, x1);
-        }
-        pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
-        return block_sum;
-    };
-    // Exact online softmax step of block b: raises the reference to the tile's
-    // maximum and returns the factor O and the row sum are scaled by.
-    auto raise_reference = [&](const float (&sc)[8], uint32_t b) -> float {
-        float block_max = sc[0];
-#pragma unroll
-        for (uint32_t e = 1; e < 8; ++e) block_max = fmaxf(block_max, sc[e]);
-        block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
-        block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
-        const float m_new = fmaxf(m_run[b], block_max);  // key 0 is visible: finite from tile 0 on
-        const float alpha = __builtin_amdgcn_exp2f(m_run[b] - m_new);
-        l_run[b] *= alpha;
-        m_run[b] = m_new;
-        return alpha;
-    };
-
-    // O^T += V^T P^T of tile kb; contraction slot e of lane group g is key
-    // (e>>2)*16 + g*4 + (e&3); MFMA j covers dims (j>>3)*128 + row*8 + (j&7)
-    auto accumulate = [&](uint32_t kb, const bf16x8 (&pb)[NB]) {
-        const uint8_t* vstage = lds + (kb % kStages) * kStageBytes + kKeyStageBytes;
-#pragma unroll
-        for (uint32_t hq = 0; hq < 4; ++hq) {  // 8 dwords of a value row = 16 dims per lane
-            u32x2 v[8];
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) {
-                const uint32_t key = (e >> 2) * 16 + g * 4 + (e & 3);
-                v[e] = *reinterpret_cast<const u32x2*>(vstage + key * 512 + (hq >> 1) * 256 +
-                                                       m * 16 + (hq & 1) * 8);
-            }
-#pragma unroll
-            for (uint32_t d2 = 0; d2 < 2; ++d2) {
-                const uint32_t dw = (hq & 1) * 2 + d2;
-                u32x4 lo, hi;
-                lo.x = pack_low(v[0][d2], v[1][d2]);
-                lo.y = pack_low(v[2][d2], v[3][d2]);
-                lo.z = pack_low(v[4][d2], v[5][d2]);
-                lo.w = pack_low(v[6][d2], v[7][d2]);
-                hi.x = pack_high(v[0][d2], v[1][d2]);
-                hi.y = pack_high(v[2][d2], v[3][d2]);
-                hi.z = pack_high(v[4][d2], v[5][d2]);
-                hi.w = pack_high(v[6][d2], v[7][d2]);
-                const bf16x8 va = __builtin_bit_cast(bf16x8, lo);
-                const bf16x8 vb = __builtin_bit_cast(bf16x8, hi);
-                const uint32_t j = (hq >> 1) * 8 + 2 * dw;
-#pragma unroll
-                for (uint32_t b = 0; b < NB; ++b) {
-                    o[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[b], o[b][j], 0, 0, 0);
-                    o[b][j + 1] =
-                        __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb, pb[b], o[b][j + 1], 0, 0, 0);
-                }
-            }
-        }
-    };
-
-    stage_tile(0);
-    if (nkb > 1) stage_tile(1);
-    // Entering tile kb: its transfers (issued two tiles earlier) have landed for
-    // every wave, and every wave is done with tile kb-2, whose stage the transfers
-    // of tile kb+2 overwrite.
-    auto enter_tile = [&](uint32_t kb) {
-        if (kb + 1 < nkb) {
-            __builtin_amdgcn_s_waitcnt(0x0F78);  // all but the 8 transfers of tile kb+1
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        __syncthreads();
-        if (kb + 2 < nkb) stage_tile(kb + 2);
-    };
-    bf16x8 pb[NB];
-    {
-        enter_tile(0);
-        f32x4 s[2][NB];
-        scores(0, s);
-#pragma unroll
-        for (uint32_t b = 0; b < NB; ++b) {
-            float sc[8];
-            scaled(0, s, b, sc);
-            (void)raise_reference(sc, b);  // O and the sums are still zero
-            l_run[b] += probabilities(sc, b, pb[b]);
-        }
-    }
-    // Steady state.  The reference of every row stays where tile 0 put it: scores
-    // are bounded by |q||k|/16, far inside the 2^127 range of fp32 and bf16, so
-    // P = exp2(s - reference) neither overflows nor, the row maximum being at least
-    // the reference, vanishes.  O is touched by MFMA only.  Should a score ever
-    // exceed the reference by more than 2^kReferenceSlack the walk is finished by
-    // the exact loop below.  The loop is skewed: softmax of tile kb (VALU) next to
-    // P V of tile kb-1 (MFMA).
-    uint32_t kb = 1;
-    bool exact = false;
-    while (kb < nkb) {
-        enter_tile(kb);
-        f32x4 s[2][NB];
-        bf16x8 pb_next[NB];
-        scores(kb, s);
-        bool above = false;
-        float sums[NB];
-#pragma unroll
-        for (uint32_t b = 0; b < NB; ++b) {
-            float sc[8];
-            scaled(kb, s, b, sc);
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) above = above || sc[e] > m_run[b] + kReferenceSlack;
-            sums[b] = probabilities(sc, b, pb_next[b]);
-        }
-        accumulate(kb - 1, pb);
-        if (__builtin_amdgcn_ballot_w64(above) != 0) {
-            exact = true;  // tile kb, whose operands above may have overflowed, is dropped
-            break;         // here and redone by the exact loop
-        }
-#pragma unroll
-        for (uint32_t b = 0; b < NB; ++b) {
-            pb[b] = pb_next[b];
-            l_run[b] += sums[b];
-        }
-        ++kb;
-    }
-    if (!exact) {
-        accumulate(nkb - 1, pb);
-    } else {
-        // Exact online softmax from tile kb on: raise the reference per tile, scale O.
-        // (Reached only with scores beyond any RMS-normalised q, k.)  The steady loop
-        // has entered tile kb already.
-        f32x4 s[2][NB];
-        bool first = true;
-        for (; kb < nkb; ++kb) {
-            if (!first) enter_tile(kb);
-            first = false;
-            scores(kb, s);
-#pragma unroll
-            for (uint32_t b = 0; b < NB; ++b) {
-                float sc[8];
-                scaled(kb, s, b, sc);
-                const float alpha = raise_reference(sc, b);
-#pragma unroll
-                for (uint32_t j = 0; j < 16; ++j) o[b][j] *= alpha;
-                l_run[b] += probabilities(sc, b, pb[b]);
-            }
-            accumulate(kb, pb);
-        }
-    }
-
-    // out[(row*16 + head)*256 + dim] = bf16((O/l) * sigmoid(gate)); lane holds, for
-    // position column m, dims (j>>3)*128 + (g*4+i)*8 + (j&7)
-#pragma unroll
-    for (uint32_t b = 0; b < NB; ++b) {
-        float l = l_run[b];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
-        const uint32_t row = p0 + (b % PH) * 16 + m;
-        if (row < a.rows) {
-            const uint64_t row_base = (static_cast<uint64_t>(row) * kAttnQueryHeads +
-                                       kvh * kAttnHeadsPerKv + wave * 2 + b / PH) * kD;
-            const float inv = 1.0f / l;
-#pragma unroll
-            for (uint32_t j = 0; j < 16; ++j) {
-#pragma unroll
-                for (uint32_t i = 0; i < 4; ++i) {
-                    const uint32_t dim = (j >> 3) * 128 + (g * 4 + i) * 8 + (j & 7);
-                    const float gate = bf16_bits_to_f32(a.gate[row_base + dim]);
-                    const float sig = 1.0f / (1.0f + __expf(-gate));
-                    a.out[row_base + dim] = f32_to_bf16_bits((o[b][j][i] * inv) * sig);
-                }
-            }
-        }
-    }
-}
-
-// ------------------------------------------------- 32-position workgroup ------
+// ---------------------------------------------------------- flash kernel ------
 //
 // Workgroup = 8 wave64 = 32 consecutive query positions x the 8 query heads of one
 // kv head.  Wave w owns heads 2(w&3), 2(w&3)+1 at positions 16(w>>2)..+15: two 16x16
@@ -415,21 +94,23 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
 //   16 lanes hand in the addresses of 4 key rows x 16 dims (4 lanes per row, 4 dims
 //   each) and lane i receives dim i of the 4 rows - two such reads are the 8 contraction
 //   slots of one MFMA operand, no register permutes and no transposed copy in LDS.
-// One barrier per tile.  Softmax as in the 16-position kernel: reference fixed by
-// tile 0, exact online loop as the way out.
-constexpr bool kUseWideTile = true;
-constexpr uint32_t kWideWaves = 8;
-constexpr uint32_t kWidePositions = 32;
+// One barrier per tile.  The softmax reference of a row is fixed by tile 0: with q and
+// k RMS-normalised a later score cannot exceed it by 2^100, so the steady loop never
+// rescales O and the accumulators are touched by MFMA only.  A tile that would exceed
+// the slack leaves the steady loop for an exact online-softmax loop (running maximum
+// raised per tile, O rescaled), which finishes the walk.
+constexpr uint32_t kFlashWaves = 8;
+constexpr uint32_t kTilePositions = 32;
 constexpr uint32_t kRing = 3;
 constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 49920
 constexpr uint32_t kValuePairBytes = 1056;                             // row i | row 16+i | 32 B pad
 constexpr uint32_t kValuePairedStageBytes = 16 * kValuePairBytes;      // 16896
-constexpr uint32_t kWideLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 100608
+constexpr uint32_t kFlashLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 100608
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
-__global__ __launch_bounds__(kWideWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
+__global__ __launch_bounds__(kFlashWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attention_flash_prefill_kernel(FlashPrefillArgs a) {
     constexpr uint32_t NB = 2;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t* const key_ring = lds;
@@ -443,8 +124,8 @@ void attention_flash_prefill_wide_kernel(FlashPrefillArgs a) {
     const uint32_t g = lane >> 4;
     const uint32_t half = wave >> 2;
     const uint32_t head0 = kvh * kAttnHeadsPerKv + (wave & 3) * 2;
-    const uint32_t p0 = tile * kWidePositions;
-    const uint32_t tile_keys = a.tile_context + min(p0 + kWidePositions, a.rows);  // visible count
+    const uint32_t p0 = tile * kTilePositions;
+    const uint32_t tile_keys = a.tile_context + min(p0 + kTilePositions, a.rows);  // visible count
     const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
     // this lane's column: query row p0 + 16*half + m, whose last visible key is limit
     const uint32_t row = p0 + half * 16 + m;
@@ -868,8 +549,6 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     a.require(g.gx == 16 && g.gy == (f.rows + 15) / 16 && g.gz == 1 && g.tx == 256 && g.ty == 1 &&
                   g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
-    constexpr uint32_t kHalves = 1;  // 16-position halves per workgroup
-    const uint32_t tiles = (f.rows + 16 * kHalves - 1) / (16 * kHalves);
     a.require(f.capacity != 0 &&
                   static_cast<uint64_t>(f.tile_context) + f.rows == visible &&
                   visible <= f.capacity,
@@ -881,14 +560,9 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     f.gate = a.buffer<const uint16_t>(3, row_bytes);
     f.out = a.buffer<uint16_t>(4, row_bytes);
     if (a.status != TT_OK || validate_only) return a.status;
-    if (kUseWideTile) {
-        hipLaunchKernelGGL(attention_flash_prefill_wide_kernel,
-                           dim3((f.rows + kWidePositions - 1) / kWidePositions, kAttnKvHeads),
-                           dim3(kWideWaves * 64), kWideLdsBytes, stream, f);
-        return TT_OK;
-    }
-    hipLaunchKernelGGL(attention_flash_prefill_kernel<kHalves>, dim3(tiles, kAttnKvHeads), dim3(256),
-                       kFlashLdsBytes, stream, f);
+    hipLaunchKernelGGL(attention_flash_prefill_kernel,
+                       dim3((f.rows + kTilePositions - 1) / kTilePositions, kAttnKvHeads),
+                       dim3(kFlashWaves * 64), kFlashLdsBytes, stream, f);
     return TT_OK;
 }
 
@@ -951,12 +625,9 @@ int32_t op_attention_combine_blk(const Bindings& b, const Grid& g, hipStream_t s
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
 bool prepare_prefill_kernels() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel<1>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kFlashLdsBytes) == hipSuccess &&
-           hipFuncSetAttribute(reinterpret_cast<const void*>(attention_flash_prefill_wide_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kWideLdsBytes) == hipSuccess;
+                               kFlashLdsBytes) == hipSuccess;
 }
 
 const KernelDesc kAttentionPrefillKernels[] = {
