@@ -24,6 +24,7 @@ namespace tt {
 namespace {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr uint32_t kGD = kGdnHeadDim;
@@ -163,6 +164,98 @@ __global__ __launch_bounds__(128) void gdn_prepare_kernel(PrepareArgs a) {
     }
 }
 
+// Block form of the prepare step for rows that are consecutive tokens of one lane:
+// a lane owns 8 adjacent channels (16-byte loads and stores), a workgroup of 256
+// lanes 2048 channels, and walks kBlockRowsPerGroup rows with the three earlier taps
+// in registers, so every projection element is read once.  grid.x: 0 q heads, 1 k
+// heads, 2..3 value heads, 4..5 the z gate copy.  Same arithmetic, operation for
+// operation, as gdn_prepare_kernel: a head's 128 squares are summed as 32 runs of
+// four, then the adjacent-pairs tree - a lane holds two runs, 16 lanes a head.
+
+__device__ __forceinline__ float widen_half(uint32_t word, uint32_t j) {
+    return __uint_as_float((j & 1) ? (word & 0xFFFF0000u) : (word << 16));
+}
+__device__ __forceinline__ uint32_t narrow_pair(float a, float b) {
+    return static_cast<uint32_t>(narrow(a)) | (static_cast<uint32_t>(narrow(b)) << 16);
+}
+
+__global__ __launch_bounds__(256) void gdn_prepare_block_kernel(PrepareArgs a) {
+    const uint32_t unit = blockIdx.x * 256 + threadIdx.x;  // 8 channels each
+    const uint32_t row_begin = blockIdx.y * kBlockRowsPerGroup;
+    const uint32_t row_end = min(a.rows, row_begin + kBlockRowsPerGroup);
+    if (unit >= kCh / 8) {
+        const uint32_t index = (unit - kCh / 8) * 8;
+        for (uint32_t row = row_begin; row < row_end; ++row) {
+            *reinterpret_cast<u32x4*>(a.z + static_cast<uint64_t>(row) * a.z_stride + index) =
+                *reinterpret_cast<const u32x4*>(
+                    a.projection + static_cast<uint64_t>(row) * a.projection_stride + kCh + index);
+        }
+        return;
+    }
+    const uint32_t c = unit * 8;
+    // logical sequence = three state rows, then the block's projection rows
+    auto logical = [&](uint32_t index) -> u32x4 {
+        if (index < 3) return *reinterpret_cast<const u32x4*>(a.conv_in + index * kCh + c);
+        return *reinterpret_cast<const u32x4*>(
+            a.projection + static_cast<uint64_t>(index - 3) * a.projection_stride + c);
+    };
+    u32x4 t0 = logical(row_begin), t1 = logical(row_begin + 1), t2 = logical(row_begin + 2);
+    float w[8][4];
+    {
+        const u32x4* wp = reinterpret_cast<const u32x4*>(a.conv_weights + static_cast<uint64_t>(c) * 4);
+#pragma unroll
+        for (uint32_t q = 0; q < 4; ++q) {  // 16 bytes = two channels x four taps
+            const u32x4 bits = wp[q];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) w[q * 2 + (e >> 2)][e & 3] = widen_half(bits[e >> 1], e);
+        }
+    }
+    const bool normalised = c < kGdnQkValues;
+    const float scale = widen(c < kGdnQkValues / 2 ? kGdnQueryScaleBits : kGdnKeyScaleBits);
+    for (uint32_t row = row_begin; row < row_end; ++row) {
+        const u32x4 t3 = *reinterpret_cast<const u32x4*>(
+            a.projection + static_cast<uint64_t>(row) * a.projection_stride + c);
+        float act[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            // fixed four-term shape; bf16 x bf16 products are exact in fp32
+            const float convolved = w[j][0] * widen_half(t0[j >> 1], j) +
+                                    w[j][1] * widen_half(t1[j >> 1], j) +
+                                    w[j][2] * widen_half(t2[j >> 1], j) +
+                                    w[j][3] * widen_half(t3[j >> 1], j);
+            const float conv_b = rb(convolved);
+            act[j] = rb(conv_b * sigmoid_bf16(conv_b));
+        }
+        if (row == a.rows - 1) {
+            *reinterpret_cast<u32x4*>(a.conv_out + c) = t1;
+            *reinterpret_cast<u32x4*>(a.conv_out + kCh + c) = t2;
+            *reinterpret_cast<u32x4*>(a.conv_out + 2 * kCh + c) = t3;
+        }
+        u32x4 packed;
+        if (normalised) {
+            const float run0 = ((act[0] * act[0] + act[1] * act[1]) + act[2] * act[2]) + act[3] * act[3];
+            const float run1 = ((act[4] * act[4] + act[5] * act[5]) + act[6] * act[6]) + act[7] * act[7];
+            float total = run0 + run1;
+            for (uint32_t off = 1; off < 16; off <<= 1) total += __shfl_xor(total, off, 64);
+            const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                packed[j] = narrow_pair(rb(act[2 * j] * inverse) * scale,
+                                        rb(act[2 * j + 1] * inverse) * scale);
+            }
+            *reinterpret_cast<u32x4*>(a.qk + static_cast<uint64_t>(row) * a.qk_stride + c) = packed;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) packed[j] = narrow_pair(act[2 * j], act[2 * j + 1]);
+            *reinterpret_cast<u32x4*>(a.value + static_cast<uint64_t>(row) * a.value_stride + c -
+                                      kGdnQkValues) = packed;
+        }
+        t0 = t1;
+        t1 = t2;
+        t2 = t3;
+    }
+}
+
 // ------------------------------------------------------------- recurrence ----
 
 struct RecurrenceArgs {
@@ -295,6 +388,48 @@ __global__ __launch_bounds__(128) void gdn_gate_norm_kernel(const uint16_t* y, c
         const float low = 1.0f / (1.0f + expf(fabsf(g)));
         const float sig = g < 0.0f ? low : 1.0f - low;
         out[at] = narrow((g * sig) * normed);
+    }
+}
+
+// Block form: a lane owns 8 adjacent channels, 16 lanes a head, a workgroup of 256
+// lanes half a row; grid (2, ceil(rows / rows_per_group)).  Same arithmetic as
+// gdn_gate_norm_kernel (two runs of four squares per lane, then the pair tree).
+__global__ __launch_bounds__(256) void gdn_gate_norm_block_kernel(
+    const uint16_t* y, const uint16_t* z, const uint16_t* weight, uint16_t* out, uint32_t stride,
+    uint32_t rows, uint32_t rows_per_group) {
+    const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 8;
+    float w[8];
+    {
+        const u32x4 bits = *reinterpret_cast<const u32x4*>(weight + (c & (kGD - 1)));
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) w[j] = widen_half(bits[j >> 1], j);
+    }
+    const uint32_t row_end = min(rows, (blockIdx.y + 1) * rows_per_group);
+    for (uint32_t row = blockIdx.y * rows_per_group; row < row_end; ++row) {
+        const uint64_t at = static_cast<uint64_t>(row) * stride + c;
+        const u32x4 yb = *reinterpret_cast<const u32x4*>(y + at);
+        const u32x4 zb = *reinterpret_cast<const u32x4*>(z + at);
+        float v[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) v[j] = widen_half(yb[j >> 1], j);
+        const float run0 = ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3];
+        const float run1 = ((v[4] * v[4] + v[5] * v[5]) + v[6] * v[6]) + v[7] * v[7];
+        float total = run0 + run1;
+        for (uint32_t off = 1; off < 16; off <<= 1) total += __shfl_xor(total, off, 64);
+        const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
+        float r[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const float normed = rb(w[j] * rb(v[j] * inverse));
+            const float g = widen_half(zb[j >> 1], j);
+            const float low = 1.0f / (1.0f + expf(fabsf(g)));
+            const float sig = g < 0.0f ? low : 1.0f - low;
+            r[j] = (g * sig) * normed;
+        }
+        u32x4 packed;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) packed[j] = narrow_pair(r[2 * j], r[2 * j + 1]);
+        *reinterpret_cast<u32x4*>(out + at) = packed;
     }
 }
 
@@ -469,7 +604,6 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
 // accumulators and every product on v_mfma_f32_16x16x32_bf16.
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr uint32_t kChunk = 64;
 // per (chunk, head) record, byte offsets.  Everything that feeds the recurrent
@@ -980,9 +1114,14 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
 // ---------------------------------------------------------------- launchers --
 
 int32_t launch_prepare(const PrepareArgs& p, hipStream_t stream) {
-    const uint32_t groups =
-        p.block_mode ? (p.rows + kBlockRowsPerGroup - 1) / kBlockRowsPerGroup : p.rows;
-    hipLaunchKernelGGL(gdn_prepare_kernel, dim3(96, groups), dim3(128), 0, stream, p);
+    if (p.block_mode) {
+        hipLaunchKernelGGL(gdn_prepare_block_kernel,
+                           dim3((kCh + kGdnValueValues) / 8 / 256,
+                                (p.rows + kBlockRowsPerGroup - 1) / kBlockRowsPerGroup),
+                           dim3(256), 0, stream, p);
+        return TT_OK;
+    }
+    hipLaunchKernelGGL(gdn_prepare_kernel, dim3(96, p.rows), dim3(128), 0, stream, p);
     return TT_OK;
 }
 
@@ -1246,9 +1385,13 @@ int32_t gate_norm_common(Args& a, const Grid& g, uint32_t rows, uint32_t stride,
     a.require(g.gx == 32 && g.gy == rows && g.gz == 1 && g.tx == 128 && g.ty == 1 && g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK || validate_only) return a.status;
-    const uint32_t per_group = rows > kMaxBatchRows ? 8u : 1u;  // blocks walk 8 rows per group
-    hipLaunchKernelGGL(gdn_gate_norm_kernel, dim3(32, (rows + per_group - 1) / per_group), dim3(128),
-                       0, stream, y, z, w, out, stride, rows, per_group);
+    if (rows > kMaxBatchRows && stride % 8 == 0) {  // blocks: 8 channels per lane, 8 rows per group
+        hipLaunchKernelGGL(gdn_gate_norm_block_kernel, dim3(kGdnValueValues / 8 / 256, (rows + 7) / 8),
+                           dim3(256), 0, stream, y, z, w, out, stride, rows, 8u);
+        return TT_OK;
+    }
+    hipLaunchKernelGGL(gdn_gate_norm_kernel, dim3(32, rows), dim3(128), 0, stream, y, z, w, out,
+                       stride, rows, 1u);
     return TT_OK;
 }
 
