@@ -153,6 +153,94 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
     }
 }
 
+// Block form for rows that are consecutive positions of one lane: a lane owns 8
+// adjacent dims (16-byte loads and stores), 32 lanes a head, a wave two heads, a
+// workgroup of 192 lanes six of the 18 heads; grid (3, ceil(rows / rows_per_group)).
+// Same arithmetic as attn_qk_rope_kernel: a lane's two runs of four squares are the
+// partials of threads 2l and 2l+1 there, and the xor butterfly is its pair tree.  The
+// 32 rotation angles of a row are the same for every head: lane p of each wave
+// evaluates pair p once and the eight lanes that rotate fetch theirs by shuffle.
+__global__ __launch_bounds__(192) void attn_qk_rope_block_kernel(RopeArgs a) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t head = blockIdx.x * 6 + (threadIdx.x >> 5);
+    const uint32_t l = threadIdx.x & 31;  // dims 8l .. 8l+7
+    const bool is_query = head < kAttnQueryHeads;
+    const uint32_t local = is_query ? head : head - kAttnQueryHeads;
+    const uint32_t base = (is_query ? head * 2 * kD : kAttnQGateRows + local * kD) + l * 8;
+    const uint32_t extra = (is_query ? head * 2 * kD + kD : kAttnVRowOffset + local * kD) + l * 8;
+    float weight[8];
+    {
+        const u32x4 bits =
+            *reinterpret_cast<const u32x4*>((is_query ? a.q_weight : a.k_weight) + l * 8);
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            weight[j] = __uint_as_float((j & 1) ? (bits[j >> 1] & 0xFFFF0000u) : (bits[j >> 1] << 16));
+        }
+    }
+    const float inverse_frequency = powf(
+        kAttnRopeBase, static_cast<float>(lane & (kAttnRopePairs - 1)) / static_cast<float>(kAttnRopePairs));
+    const bool rotates = l < 2 * kAttnRopePairs / 8;
+    const uint32_t row_end = min(a.rows, (blockIdx.y + 1) * a.rows_per_group);
+    for (uint32_t row = blockIdx.y * a.rows_per_group; row < row_end; ++row) {
+        const uint32_t position = a.context + row;
+        if (position >= a.capacity) continue;
+        const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+        const u32x4 xb = *reinterpret_cast<const u32x4*>(proj + base);
+        const u32x4 eb = *reinterpret_cast<const u32x4*>(proj + extra);
+        float x[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            x[j] = __uint_as_float((j & 1) ? (xb[j >> 1] & 0xFFFF0000u) : (xb[j >> 1] << 16));
+        }
+        float run0 = 0.0f, run1 = 0.0f;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            run0 += x[j] * x[j];
+            run1 += x[4 + j] * x[4 + j];
+        }
+        float acc = run0 + run1;
+        for (uint32_t off = 1; off < 16; off <<= 1) acc += __shfl_xor(acc, off, 64);
+        const float total = acc + __shfl_xor(acc, 16, 64);
+        const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+        float n[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) n[j] = round_bf16(weight[j] * round_bf16(x[j] * inverse));
+        // pair p = lane & 31 of this row, shared by the wave's two heads
+        const float theta = static_cast<float>(position) / inverse_frequency;
+        const float c = cosf(theta);
+        const float sn = sinf(theta);
+        u32x4 packed;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t pair = (l * 8 + j) & (kAttnRopePairs - 1);
+            const float cj = __shfl(c, pair, 64);
+            const float sj = __shfl(sn, pair, 64);
+            const float partner = __shfl_xor(n[j], kAttnRopePairs / 8, 64);  // dim +-32: lane l^4
+            float rotated = n[j];
+            if (rotates) {
+                rotated = l < kAttnRopePairs / 8 ? fmaf(-partner, sj, n[j] * cj)
+                                                 : fmaf(partner, sj, n[j] * cj);
+            }
+            const uint32_t bits = f32_to_bf16_bits(rotated);
+            if (j & 1) {
+                packed[j >> 1] |= bits << 16;
+            } else {
+                packed[j >> 1] = bits;
+            }
+        }
+        if (head >= kAttnQueryHeads + kAttnKvHeads) continue;
+        if (is_query) {
+            const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + l * 8;
+            *reinterpret_cast<u32x4*>(a.q_out + at) = packed;
+            *reinterpret_cast<u32x4*>(a.gate_out + at) = eb;
+        } else {
+            const uint64_t at = (static_cast<uint64_t>(local) * a.capacity + position) * kD + l * 8;
+            *reinterpret_cast<u32x4*>(a.keys + at) = packed;
+            *reinterpret_cast<u32x4*>(a.values + at) = eb;
+        }
+    }
+}
+
 // ------------------------------------------------------------ flash decode ---
 
 struct FlashArgs {
@@ -628,6 +716,11 @@ int32_t launch_rope(const RopeArgs& args, uint32_t rows, hipStream_t stream) {
     r.rows = rows;
     r.rows_per_group = r.position_per_row ? 8u : 1u;  // blocks walk 8 rows per workgroup
     const uint32_t groups = (rows + r.rows_per_group - 1) / r.rows_per_group;
+    if (r.position_per_row && r.table == nullptr && r.projection_stride % 8 == 0 &&
+        r.query_stride % 8 == 0) {
+        hipLaunchKernelGGL(attn_qk_rope_block_kernel, dim3(3, groups), dim3(192), 0, stream, r);
+        return TT_OK;
+    }
     hipLaunchKernelGGL(attn_qk_rope_kernel, dim3(kAttnQueryHeads + kAttnKvHeads, groups),
                        dim3(256), 0, stream, r);
     return TT_OK;
