@@ -41,7 +41,7 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # HBM traffic of one launch of the split-K kernel at this workload, from two
 # rocprofv3 counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
 # scaled by what the same counter read for a plain 256 MiB copy of known size.
-FLASH_FETCH_KIB, FETCH_SCALE = 131289.5, 262144.0 / 131083.3
+FLASH_FETCH_KIB, FETCH_SCALE = 131297.0, 262144.0 / 131083.3
 FLASH_WRITE_KIB, WRITE_SCALE = 2112.0, 262144.0 / 262144.0
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
@@ -210,6 +210,12 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
             "flash_kernel_ms": round(flash_ms, 3),
             "flash_kernel_tflops": round(flops / (flash_ms * 1e-3) / 1e12, 1),
             "flash_kernel_frac_of_bf16_mfma_peak": round(flops / (flash_ms * 1e-3) / 2.5e15, 4),
+            "roofline": {"bound": "mfma", "kernel": "attention_flash_v2_blk "
+                                                    "(attention_flash_prefill_kernel)",
+                         "achieved": round(flops / (flash_ms * 1e-3) / 1e12, 1), "peak": 2500.0,
+                         "unit": "TFLOP/s",
+                         "frac": round(flops / (flash_ms * 1e-3) / 2.5e15, 4),
+                         "algorithmic_flops": flops},
             "gdn_layer_ms": round(gdn_ms, 3),
             "gdn_layer_tok_per_s": round(rows / (gdn_ms * 1e-3)),
             "kernel_ms": {k: round(v, 3) for k, v in best.items()}}
