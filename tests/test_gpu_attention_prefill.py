@@ -59,6 +59,7 @@ def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, 
     gv = b_v.read(np.uint16).reshape(2, cap, 256)
     assert np.array_equal(gv, values.reshape(2, cap, 256))
     check_bf16(gk, keys, "prefill K cache", max_abs=4e-2, mean_abs=1e-4)
+    check_bf16(b_q.read(np.uint16), query, "prefill roped Q", max_abs=4e-2, mean_abs=1e-4)
     assert np.array_equal(b_g.read(np.uint16), gate)
     if control:
         parts = (base + rows + 255) // 256

@@ -120,6 +120,31 @@ def test_block_operators_register_loop(hoisted):
     check_bf16(bufs["gated"].read(np.uint16), ref["gated"], "gated")
 
 
+@pytest.mark.parametrize("rows", [1, 15, 16, 17, 33, 130])
+def test_element_wise_block_kernels_bit_for_bit(rows):
+    """conv / L2 norm / z copy / conv-state shift and the gate-norm of a block, at row
+    counts around the 16- and 8-row groups the block kernels walk: the vectorised
+    kernels keep the checker's summation order, so every bf16 output is the same
+    bit pattern.  The gate-norm is fed the checker's y so that only it is tested."""
+    print(f"[case] gdn element-wise block kernels rows={rows}", flush=True)
+    B, dev, queue, lib = gpu()
+    weights = _weights()
+    proj, conv_state, state = _block(rows, 0x5300 + rows)
+    ref = _oracle_block(proj, conv_state, state, weights, rows)
+    bufs = _buffers(dev, proj, conv_state, state, weights, rows)
+    bufs["y"] = dev.buffer_from(ref["y"])
+
+    def rec(cb):
+        _encode_front(cb, lib, bufs, rows)
+        _encode_gate_norm(cb, lib, bufs, rows)
+    run(rec)
+    assert np.array_equal(bufs["qk"].read(np.uint16), ref["qk"])
+    assert np.array_equal(bufs["value"].read(np.uint16), ref["value"])
+    assert np.array_equal(bufs["z"].read(np.uint16).reshape(rows, 4096), proj[:, 8192:12288])
+    assert np.array_equal(bufs["conv_out"].read(np.uint16), ref["conv"])
+    assert np.array_equal(bufs["gated"].read(np.uint16), ref["gated"])
+
+
 def _encode_chunked(cb, lib, bufs, rows, state_in="state_in", state_out="state_out"):
     chunks = (rows + 63) // 64
     cb.encode(lib.pipeline("gdn_chunk_prepare_blk"),
