@@ -644,6 +644,7 @@ __device__ __forceinline__ bf16x8 operand(const uint16_t* p) {
 
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 // Two floats to a packed bf16 pair with the hardware conversion (round to
 // nearest even).  Used for MFMA operands only: operator outputs go through
@@ -709,6 +710,7 @@ __device__ __forceinline__ void store_tile_hi_lo(uint16_t (*tile)[16][24], const
 // [Wk | Wv] = T (beta o [g o K | V]) on MFMA with hi/lo operands.
 __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs a) {
     constexpr uint32_t kLd = 68;  // fp32 row stride: 16-byte aligned, bank-skewed
+    constexpr uint32_t kTileLd = 136;  // bf16 row stride of the key and value tiles
     __shared__ __attribute__((aligned(16))) float lower[kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float tinv[kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float mtmp[16][52];
@@ -716,6 +718,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     __shared__ __attribute__((aligned(16))) float log_g[kChunk];
     __shared__ __attribute__((aligned(16))) float scale_k[kChunk];  // beta_t g_t
     __shared__ __attribute__((aligned(16))) float scale_v[kChunk];  // beta_t
+    // the head's keys and values of the chunk, row-major [token][128], rows padded to
+    // 272 bytes so that 16-byte operand reads of 16 rows spread over the banks
+    __shared__ __attribute__((aligned(16))) uint16_t ktile[kChunk][kTileLd];
+    __shared__ __attribute__((aligned(16))) uint16_t vtile[kChunk][kTileLd];
     const uint32_t chunk = blockIdx.x;
     const uint32_t h = blockIdx.y;
     const uint32_t kh = h >> 1;
@@ -728,27 +734,25 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     const uint32_t valid = min(kChunk, a.rows - t0);
     uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
 
-    // The right-hand sides of the last stage ([K | V] columns, token-contiguous per
-    // lane: 2-byte gathers) are requested now and consumed at the end, behind the
-    // Gram and inverse stages.  Waves 0,1 take the 128 key columns, waves 2,3 the values.
+    // Keys and values of the chunk into LDS with 16-byte loads: 16 lanes per row, 16
+    // rows per pass; rows past the block repeat the last one (their scales are zero).
     const bool is_k = wave < 2;
-    uint32_t rhs_bits[4][2][8];
     {
-        const uint16_t* src =
-            is_k ? a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kGdnKOffset + kh * kGD
-                 : a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
-        const uint32_t src_stride = is_k ? kGdnQkValues : kGdnValueValues;
+        const uint16_t* ksrc = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kGdnKOffset + kh * kGD;
+        const uint16_t* vsrc = a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
+        u32x4 kv[4], vv[4];
 #pragma unroll
-        for (uint32_t ct = 0; ct < 4; ++ct) {
-            const uint32_t col = (wave & 1) * 64 + ct * 16 + m;
+        for (uint32_t pass = 0; pass < 4; ++pass) {
+            const uint32_t r = min(pass * 16 + (tid >> 4), valid - 1);
+            kv[pass] = *reinterpret_cast<const u32x4*>(ksrc + static_cast<uint64_t>(r) * kGdnQkValues +
+                                                       (tid & 15) * 8);
+            vv[pass] = *reinterpret_cast<const u32x4*>(vsrc + static_cast<uint64_t>(r) * kGdnValueValues +
+                                                       (tid & 15) * 8);
+        }
 #pragma unroll
-            for (uint32_t ks = 0; ks < 2; ++ks) {
-#pragma unroll
-                for (uint32_t e = 0; e < 8; ++e) {
-                    const uint32_t s = min(ks * 32 + g * 8 + e, valid - 1);
-                    rhs_bits[ct][ks][e] = src[static_cast<uint64_t>(s) * src_stride + col];
-                }
-            }
+        for (uint32_t pass = 0; pass < 4; ++pass) {
+            *reinterpret_cast<u32x4*>(&ktile[pass * 16 + (tid >> 4)][(tid & 15) * 8]) = kv[pass];
+            *reinterpret_cast<u32x4*>(&vtile[pass * 16 + (tid >> 4)][(tid & 15) * 8]) = vv[pass];
         }
     }
 
@@ -776,27 +780,24 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     __syncthreads();
 
     const uint16_t* qrows = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kh * kGD;
-    const uint16_t* krows = qrows + kGdnKOffset;
     {
         // wave w owns token rows 16w..16w+15 against all 64 columns
         const uint32_t trow = min(wave * 16 + m, valid - 1);
         bf16x8 ak[4], aq[4];
 #pragma unroll
         for (uint32_t kk = 0; kk < 4; ++kk) {
-            ak[kk] = operand(krows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
+            ak[kk] = operand(&ktile[wave * 16 + m][kk * 32 + g * 8]);
             aq[kk] = operand(qrows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
             *reinterpret_cast<u32x4*>(rec + kRecQ + ((wave * 4 + kk) * 64 + lane) * 16) =
                 __builtin_bit_cast(u32x4, aq[kk]);
         }
 #pragma unroll
         for (uint32_t nt = 0; nt < 4; ++nt) {
-            const uint32_t srow = min(nt * 16 + m, valid - 1);
             f32x4 kkacc = {0.0f, 0.0f, 0.0f, 0.0f};
             f32x4 qkacc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (uint32_t kk = 0; kk < 4; ++kk) {
-                const bf16x8 bk =
-                    operand(krows + static_cast<uint64_t>(srow) * kGdnQkValues + kk * 32 + g * 8);
+                const bf16x8 bk = operand(&ktile[nt * 16 + m][kk * 32 + g * 8]);
                 kkacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[kk], bk, kkacc, 0, 0, 0);
                 qkacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aq[kk], bk, qkacc, 0, 0, 0);
             }
@@ -881,11 +882,27 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
         for (uint32_t ks = 0; ks < 2; ++ks) {
             float x[8];
             uint32_t bits[8];
+            {
+                // 16 lanes hand in 4 token rows x 16 columns (4 lanes per row, 4 columns
+                // each) and lane m receives column m of the 4 rows: two reads are the 8
+                // tokens of this lane's contraction slots
+                const uint16_t* at = &(is_k ? ktile : vtile)[ks * 32 + g * 8 + (m >> 2)]
+                                                           [(wave & 1) * 64 + ct * 16 + (m & 3) * 4];
+                const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4*)(at));
+                const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4*)(at + 4 * kTileLd));
+#pragma unroll
+                for (uint32_t e = 0; e < 4; ++e) {
+                    bits[e] = static_cast<uint16_t>(first[e]);
+                    bits[4 + e] = static_cast<uint16_t>(second[e]);
+                }
+            }
 #pragma unroll
             for (uint32_t e = 0; e < 8; ++e) {
                 // rows past the block were clamped on load: their scale (beta) is zero,
                 // and the exact keys stored below are zeroed explicitly
-                bits[e] = ks * 32 + g * 8 + e < valid ? rhs_bits[ct][ks][e] : 0u;
+                if (ks * 32 + g * 8 + e >= valid) bits[e] = 0u;
                 x[e] = widen(static_cast<uint16_t>(bits[e])) * sc[ks][e];
             }
             split8(x, b_hi[ks], b_lo[ks]);
