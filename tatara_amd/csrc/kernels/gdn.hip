@@ -711,10 +711,15 @@ __device__ __forceinline__ void store_tile_hi_lo(uint16_t (*tile)[16][24], const
 __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs a) {
     constexpr uint32_t kLd = 68;  // fp32 row stride: 16-byte aligned, bank-skewed
     constexpr uint32_t kTileLd = 136;  // bf16 row stride of the key and value tiles
+    constexpr uint32_t kStripLd = 72;  // 64 rows + pad: 16-byte reads of 16 columns spread over the banks
     __shared__ __attribute__((aligned(16))) float lower[kChunk][kLd];
-    __shared__ __attribute__((aligned(16))) float tinv[kChunk][kLd];
-    __shared__ __attribute__((aligned(16))) float mtmp[16][52];
-    __shared__ __attribute__((aligned(16))) uint16_t tiles[4][2][16][24];  // per-wave store staging
+    // inverses of the four 16x16 diagonal blocks of I + L: tdiag[16 b + r][c]
+    __shared__ __attribute__((aligned(16))) float tdiag[kChunk][20];
+    // per wave: a 16-column strip of the solution as bf16 hi/lo, [half][column][row]
+    // (rows 0..47 the finished block rows, 48..63 the right-hand side being solved),
+    // rows contiguous so that a lane reads its 8 contraction slots with 16 bytes; the
+    // same memory stages the 16x16 result tiles on their way to the record
+    __shared__ __attribute__((aligned(16))) uint16_t strip[4][2][16][kStripLd];
     __shared__ __attribute__((aligned(16))) float log_g[kChunk];
     __shared__ __attribute__((aligned(16))) float scale_k[kChunk];  // beta_t g_t
     __shared__ __attribute__((aligned(16))) float scale_v[kChunk];  // beta_t
@@ -776,7 +781,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
         reinterpret_cast<float*>(rec + kRecGam)[tid] = __expf(lg);
         if (tid == kChunk - 1) *reinterpret_cast<float*>(rec + kRecGamma) = __expf(lg);
     }
-    for (uint32_t e = tid; e < kChunk * kLd; e += 256) (&tinv[0][0])[e] = 0.0f;
     __syncthreads();
 
     const uint16_t* qrows = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kh * kGD;
@@ -811,7 +815,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
                 aqk[i] = (s <= t && t < valid) ? ratio * qkacc[i] : 0.0f;
             }
             // fragment (token tile `wave`, token step nt >> 1), column groups 2(nt&1), +1
-            store_tile_hi_lo(tiles[wave], aqk, lane, rec + kRecAqkHi, rec + kRecAqkLo,
+            store_tile_hi_lo(reinterpret_cast<uint16_t (*)[16][24]>(&strip[wave][0][0][0]), aqk, lane, rec + kRecAqkHi, rec + kRecAqkLo,
                              ((wave * 2 + (nt >> 1)) * 64 + (nt & 1) * 32) * 16);
         }
     }
@@ -830,108 +834,144 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
             x[r] = acc;
         }
 #pragma unroll
-        for (uint32_t r = 0; r < 16; ++r) tinv[b * 16 + r][b * 16 + c] = x[r];
+        for (uint32_t r = 0; r < 16; ++r) tdiag[b * 16 + r][c] = x[r];
     }
     __syncthreads();
-    // block rows 1..3: T_i,<i = -T_ii (L_i,<i T_<i,<i)
-    for (uint32_t i = 1; i < 4; ++i) {
-        const uint32_t width = 16 * i;
-        for (uint32_t e = tid; e < 16 * width; e += 256) {
-            const uint32_t r = e / width;
-            const uint32_t c = e - r * width;
-            float acc = 0.0f;
-            for (uint32_t s = c & ~15u; s < width; ++s) {
-                acc = fmaf(lower[16 * i + r][s], tinv[s][c], acc);
-            }
-            mtmp[r][c] = acc;
-        }
-        __syncthreads();
-        for (uint32_t e = tid; e < 16 * width; e += 256) {
-            const uint32_t r = e / width;
-            const uint32_t c = e - r * width;
-            float acc = 0.0f;
-            for (uint32_t s = 0; s <= r; ++s) {
-                acc = fmaf(tinv[16 * i + r][16 * i + s], mtmp[s][c], acc);
-            }
-            tinv[16 * i + r][c] = -acc;
-        }
-        __syncthreads();
-    }
+    // [Wk | Wv] = (I + L)^-1 B with B = beta o [g o K | V], solved by block forward
+    // substitution, every wave for its own 64 columns (waves 0,1 the keys, 2,3 the
+    // values): W_i = T_ii (B_i - sum_{j<i} L_ij W_j) with the diagonal inverses T_ii.
+    // All products on MFMA with hi/lo operand pairs; a finished block row goes, as
+    // bf16 hi/lo, into the wave's strip in LDS, from where it is read back as the
+    // right operand of the next products (rows contiguous: one 16-byte read per lane).
+    uint16_t (*hi_strip)[kStripLd] = strip[wave][0];
+    uint16_t (*lo_strip)[kStripLd] = strip[wave][1];
+    // left operands, the same for every column: lane (row m, slot group g).  K = 16
+    // products use slot groups 0 and 1 only; the other lanes hold zeros.
+    const auto left = [&](const float* row8, bool live, bool negate, bf16x8& hi, bf16x8& lo) {
+        float x[8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) x[e] = live ? (negate ? -row8[e] : row8[e]) : 0.0f;
+        split8(x, hi, lo);
+    };
+    bf16x8 t_hi[4], t_lo[4];       // T_ii, K = 16
+    bf16x8 l10_hi, l10_lo;         // -L_10, K = 16
+    bf16x8 l2_hi, l2_lo;           // -L_2,[0 1], K = 32
+    bf16x8 l3_hi, l3_lo;           // -L_3,[0 1], K = 32
+    bf16x8 l32_hi, l32_lo;         // -L_32, K = 16
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) left(&tdiag[16 * i + m][(g & 1) * 8], g < 2, false, t_hi[i], t_lo[i]);
+    left(&lower[16 + m][(g & 1) * 8], g < 2, true, l10_hi, l10_lo);
+    left(&lower[32 + m][g * 8], true, true, l2_hi, l2_lo);
+    left(&lower[48 + m][g * 8], true, true, l3_hi, l3_lo);
+    left(&lower[48 + m][32 + (g & 1) * 8], g < 2, true, l32_hi, l32_lo);
 
-    // [Wk | Wv] = T B: waves 0,1 take the 128 key columns, waves 2,3 the values
-    bf16x8 t_hi[4][2], t_lo[4][2];
-#pragma unroll
-    for (uint32_t mt = 0; mt < 4; ++mt) {
-#pragma unroll
-        for (uint32_t ks = 0; ks < 2; ++ks) {
-            split8(&tinv[mt * 16 + m][ks * 32 + g * 8], t_hi[mt][ks], t_lo[mt][ks]);
+    const auto product = [](const bf16x8 a_hi, const bf16x8 a_lo, const bf16x8 b_hi, const bf16x8 b_lo,
+                            f32x4 acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b_hi, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_lo, acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b_hi, acc, 0, 0, 0);
+    };
+    // a 16x16 tile (this lane: rows 4g+i of column m) into strip rows row0 + 4g + i
+    const auto put = [&](const f32x4 v, uint32_t row0) {
+        u32x2 hi, lo;
+        split4(v, hi, lo);
+        *reinterpret_cast<u32x2*>(&hi_strip[m][row0 + g * 4]) = hi;
+        *reinterpret_cast<u32x2*>(&lo_strip[m][row0 + g * 4]) = lo;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    // right operand from strip rows row0 + 8g .. +7 of column m; with `narrow_k` only
+    // slot groups 0 and 1 are live (K = 16)
+    const auto get = [&](uint32_t row0, bool narrow_k, bf16x8& hi, bf16x8& lo) {
+        const uint32_t row = row0 + (narrow_k ? (g & 1) : g) * 8;
+        u32x4 h = *reinterpret_cast<const u32x4*>(&hi_strip[m][row]);
+        u32x4 l = *reinterpret_cast<const u32x4*>(&lo_strip[m][row]);
+        if (narrow_k && g >= 2) {
+            h = u32x4{0u, 0u, 0u, 0u};
+            l = u32x4{0u, 0u, 0u, 0u};
         }
-    }
+        hi = __builtin_bit_cast(bf16x8, h);
+        lo = __builtin_bit_cast(bf16x8, l);
+    };
+    const uint16_t (*source)[kTileLd] = is_k ? ktile : vtile;
     const float* scale = is_k ? scale_k : scale_v;
-    float sc[2][8];
-#pragma unroll
-    for (uint32_t ks = 0; ks < 2; ++ks) {
-#pragma unroll
-        for (uint32_t e = 0; e < 8; ++e) sc[ks][e] = scale[ks * 32 + g * 8 + e];
-    }
-#pragma unroll
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t ct = 0; ct < 4; ++ct) {
-        const uint32_t col = (wave & 1) * 64 + ct * 16 + m;
-        bf16x8 b_hi[2], b_lo[2];
+        const uint32_t col0 = (wave & 1) * 64 + ct * 16;
+        // right-hand side tiles, this lane: tokens 16i + 4g + r of column col0 + m.  One
+        // transposing read per tile: 16 lanes hand in 4 token rows x 16 columns (4
+        // lanes per row) and lane m receives column m of the 4 rows.
+        f32x4 rhs[4];
 #pragma unroll
-        for (uint32_t ks = 0; ks < 2; ++ks) {
-            float x[8];
-            uint32_t bits[8];
-            {
-                // 16 lanes hand in 4 token rows x 16 columns (4 lanes per row, 4 columns
-                // each) and lane m receives column m of the 4 rows: two reads are the 8
-                // tokens of this lane's contraction slots
-                const uint16_t* at = &(is_k ? ktile : vtile)[ks * 32 + g * 8 + (m >> 2)]
-                                                           [(wave & 1) * 64 + ct * 16 + (m & 3) * 4];
+        for (uint32_t i = 0; i < 4; ++i) {
+            const s16x4 bits = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(&source[16 * i + 4 * g + (m >> 2)]
+                                                                  [col0 + (m & 3) * 4]));
+            const f32x4 sc = *reinterpret_cast<const f32x4*>(&scale[16 * i + 4 * g]);
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) {
+                rhs[i][r] = 16 * i + 4 * g + r < valid
+                                ? widen(static_cast<uint16_t>(bits[r])) * sc[r] : 0.0f;
+            }
+        }
+        if (is_k) {
+            // the exact keys, token-contiguous: fragment (key tile, token step ks), lane =
+            // key col0 + m, tokens 32 ks + 8 g .. +7
+#pragma unroll
+            for (uint32_t ks = 0; ks < 2; ++ks) {
+                const uint16_t* at = &ktile[ks * 32 + g * 8 + (m >> 2)][col0 + (m & 3) * 4];
                 const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) s16x4*)(at));
                 const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) s16x4*)(at + 4 * kTileLd));
+                uint32_t bits[8];
 #pragma unroll
                 for (uint32_t e = 0; e < 4; ++e) {
-                    bits[e] = static_cast<uint16_t>(first[e]);
-                    bits[4 + e] = static_cast<uint16_t>(second[e]);
+                    bits[e] = ks * 32 + g * 8 + e < valid ? static_cast<uint16_t>(first[e]) : 0u;
+                    bits[4 + e] = ks * 32 + g * 8 + 4 + e < valid ? static_cast<uint16_t>(second[e]) : 0u;
                 }
-            }
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) {
-                // rows past the block were clamped on load: their scale (beta) is zero,
-                // and the exact keys stored below are zeroed explicitly
-                if (ks * 32 + g * 8 + e >= valid) bits[e] = 0u;
-                x[e] = widen(static_cast<uint16_t>(bits[e])) * sc[ks][e];
-            }
-            split8(x, b_hi[ks], b_lo[ks]);
-            if (is_k) {  // the exact keys, token-contiguous
-                *reinterpret_cast<u32x4*>(rec + kRecKt +
-                                          (((col >> 4) * 2 + ks) * 64 + g * 16 + (col & 15)) * 16) =
+                *reinterpret_cast<u32x4*>(rec + kRecKt + (((col0 >> 4) * 2 + ks) * 64 + lane) * 16) =
                     u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
                           bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
             }
         }
+        bf16x8 b_hi, b_lo;
+        f32x4 w[4];
+        put(rhs[0], 48);
+        get(48, true, b_hi, b_lo);
+        w[0] = product(t_hi[0], t_lo[0], b_hi, b_lo, zero);
+        put(w[0], 0);
+        get(0, true, b_hi, b_lo);
+        f32x4 x = product(l10_hi, l10_lo, b_hi, b_lo, rhs[1]);
+        put(x, 48);
+        get(48, true, b_hi, b_lo);
+        w[1] = product(t_hi[1], t_lo[1], b_hi, b_lo, zero);
+        put(w[1], 16);
+        bf16x8 w01_hi, w01_lo;
+        get(0, false, w01_hi, w01_lo);
+        x = product(l2_hi, l2_lo, w01_hi, w01_lo, rhs[2]);
+        put(x, 48);
+        get(48, true, b_hi, b_lo);
+        w[2] = product(t_hi[2], t_lo[2], b_hi, b_lo, zero);
+        put(w[2], 32);
+        x = product(l3_hi, l3_lo, w01_hi, w01_lo, rhs[3]);
+        get(32, true, b_hi, b_lo);
+        x = product(l32_hi, l32_lo, b_hi, b_lo, x);
+        put(x, 48);
+        get(48, true, b_hi, b_lo);
+        w[3] = product(t_hi[3], t_lo[3], b_hi, b_lo, zero);
+        // lane holds tokens 16mt+4g+i of column col0 + m
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; ++mt) {
-            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (uint32_t ks = 0; ks < 2; ++ks) {
-                if (ks * 32 > mt * 16 + 15) continue;  // T is lower triangular
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_lo[mt][ks], b_hi[ks], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_hi[mt][ks], b_lo[ks], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t_hi[mt][ks], b_hi[ks], acc, 0, 0, 0);
-            }
-            // lane holds tokens 16mt+4g+i of column col
             if (is_k) {
                 // fragment (token tile mt, key step col0 >> 5), column groups (col0 & 31) >> 3, +1
-                const uint32_t col0 = (wave & 1) * 64 + ct * 16;
-                store_tile_hi_lo(tiles[wave], acc, lane, rec + kRecWkHi, rec + kRecWkLo,
+                store_tile_hi_lo(reinterpret_cast<uint16_t (*)[16][24]>(&strip[wave][0][0][0]), w[mt],
+                                 lane, rec + kRecWkHi, rec + kRecWkLo,
                                  ((mt * 4 + (col0 >> 5)) * 64 + ((col0 & 31) >> 3) * 16) * 16);
             } else {
                 *reinterpret_cast<f32x4*>(rec + kRecWv +
-                                          (((col >> 4) * 4 + mt) * 64 + g * 16 + (col & 15)) * 16) = acc;
+                                          ((((col0 + m) >> 4) * 4 + mt) * 64 + g * 16 + m) * 16) = w[mt];
             }
         }
     }
