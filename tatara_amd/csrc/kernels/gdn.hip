@@ -985,57 +985,80 @@ struct ChunkScanArgs {
     uint32_t rows;
 };
 
-// One chunk's operands of one wave, loaded a chunk ahead of their use.
-template <uint32_t NT>
-struct ChunkOperands {
-    bf16x8 wk_hi[4], wk_lo[4], q[4], aq_hi[2], aq_lo[2], kt[2][2];
-    f32x4 wv[NT];
-    f32x4 ratio, gam;
+// One chunk's operands of one wave, loaded a chunk ahead of their use.  The state
+// waves carry the recurrence, the output waves everything that only leaves it.
+struct StateOperands {
+    bf16x8 wk_hi[4], wk_lo[4], kt[2][2];
+    f32x4 wv, ratio;
     float gamma_c;
 };
+struct OutputOperands {
+    bf16x8 q[4], aq_hi[2], aq_lo[2];
+    f32x4 gam;
+};
 
-template <uint32_t NT>
-__device__ __forceinline__ ChunkOperands<NT> load_chunk(const ChunkScanArgs& a, uint32_t chunk,
-                                                        uint32_t h, uint32_t slice, uint32_t wave,
-                                                        uint32_t m, uint32_t g) {
-    ChunkOperands<NT> o;
-    const uint8_t* rec = a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
-    const uint32_t lane = g * 16 + m;
-    const auto fragment = [&](uint32_t base, uint32_t index) {
-        return *reinterpret_cast<const u32x4*>(rec + base + (index * 64 + lane) * 16);
-    };
+__device__ __forceinline__ const uint8_t* chunk_record(const ChunkScanArgs& a, uint32_t chunk,
+                                                       uint32_t h) {
+    return a.scratch + (static_cast<uint64_t>(chunk) * kGdnValueHeads + h) * kRecBytes;
+}
+__device__ __forceinline__ u32x4 record_fragment(const uint8_t* rec, uint32_t base, uint32_t index,
+                                                 uint32_t lane) {
+    return *reinterpret_cast<const u32x4*>(rec + base + (index * 64 + lane) * 16);
+}
+
+__device__ __forceinline__ StateOperands load_state_operands(const uint8_t* rec, uint32_t slice,
+                                                             uint32_t w, uint32_t lane) {
+    StateOperands o;
+    const uint32_t g = lane >> 4;
 #pragma unroll
     for (uint32_t kk = 0; kk < 4; ++kk) {
-        o.wk_hi[kk] = __builtin_bit_cast(bf16x8, fragment(kRecWkHi, wave * 4 + kk));
-        o.wk_lo[kk] = __builtin_bit_cast(bf16x8, fragment(kRecWkLo, wave * 4 + kk));
-        o.q[kk] = __builtin_bit_cast(bf16x8, fragment(kRecQ, wave * 4 + kk));
+        o.wk_hi[kk] = __builtin_bit_cast(bf16x8, record_fragment(rec, kRecWkHi, w * 4 + kk, lane));
+        o.wk_lo[kk] = __builtin_bit_cast(bf16x8, record_fragment(rec, kRecWkLo, w * 4 + kk, lane));
     }
 #pragma unroll
     for (uint32_t k2 = 0; k2 < 2; ++k2) {
-        o.aq_hi[k2] = __builtin_bit_cast(bf16x8, fragment(kRecAqkHi, wave * 2 + k2));
-        o.aq_lo[k2] = __builtin_bit_cast(bf16x8, fragment(kRecAqkLo, wave * 2 + k2));
 #pragma unroll
         for (uint32_t mt = 0; mt < 2; ++mt) {
-            o.kt[mt][k2] = __builtin_bit_cast(bf16x8, fragment(kRecKt, (wave * 2 + mt) * 2 + k2));
+            o.kt[mt][k2] =
+                __builtin_bit_cast(bf16x8, record_fragment(rec, kRecKt, (w * 2 + mt) * 2 + k2, lane));
         }
     }
-#pragma unroll
-    for (uint32_t nt = 0; nt < NT; ++nt) {
-        o.wv[nt] = __builtin_bit_cast(f32x4, fragment(kRecWv, (slice * NT + nt) * 4 + wave));
-    }
-    o.ratio = *reinterpret_cast<const f32x4*>(rec + kRecRatio + (wave * 16 + g * 4) * 4);
-    o.gam = *reinterpret_cast<const f32x4*>(rec + kRecGam + (wave * 16 + g * 4) * 4);
+    o.wv = __builtin_bit_cast(f32x4, record_fragment(rec, kRecWv, slice * 4 + w, lane));
+    o.ratio = *reinterpret_cast<const f32x4*>(rec + kRecRatio + (w * 16 + g * 4) * 4);
     o.gamma_c = *reinterpret_cast<const float*>(rec + kRecGamma);
     return o;
 }
 
-// Stage 2.  grid (8, 4 * 128 / (16 NT)) x 256: a workgroup owns a
-// 16*NT-wide slice of the value dimension.  Wave w owns token rows 16w..16w+15
-// of the chunk products and key columns 32w..32w+31 of the state slice, whose
-// fp32 master copy lives in MFMA accumulators for the whole block.
+__device__ __forceinline__ OutputOperands load_output_operands(const uint8_t* rec, uint32_t w,
+                                                               uint32_t lane) {
+    OutputOperands o;
+    const uint32_t g = lane >> 4;
+#pragma unroll
+    for (uint32_t kk = 0; kk < 4; ++kk) {
+        o.q[kk] = __builtin_bit_cast(bf16x8, record_fragment(rec, kRecQ, w * 4 + kk, lane));
+    }
+#pragma unroll
+    for (uint32_t k2 = 0; k2 < 2; ++k2) {
+        o.aq_hi[k2] = __builtin_bit_cast(bf16x8, record_fragment(rec, kRecAqkHi, w * 2 + k2, lane));
+        o.aq_lo[k2] = __builtin_bit_cast(bf16x8, record_fragment(rec, kRecAqkLo, w * 2 + k2, lane));
+    }
+    o.gam = *reinterpret_cast<const f32x4*>(rec + kRecGam + (w * 16 + g * 4) * 4);
+    return o;
+}
+
+// Stage 2.  grid (8, 32) x 512: a workgroup owns a 16-wide slice of the value
+// dimension of one head and walks the chunks in order.  Waves 0..3 (state waves)
+// carry the recurrence: wave w owns token rows 16w..16w+15 of U and key columns
+// 32w..32w+31 of the state slice, whose fp32 master copy lives in its MFMA
+// accumulators for the whole block.  Waves 4..7 (output waves) compute what only
+// leaves the recurrence - Y = g o (Q S^T) + A U of token rows 16w..16w+15 - from the
+// state and U copies in LDS, so that their loads, products and stores stay off the
+// chain from one chunk's state to the next.  Two barriers per chunk order the two
+// LDS copies between all eight waves.
 template <uint32_t NT>
-__global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
-    constexpr uint32_t DV = 16 * NT;
+__global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
+    static_assert(NT == 1, "one 16-wide value slice per workgroup");
+    constexpr uint32_t DV = 16;
     __shared__ __attribute__((aligned(16))) uint16_t s_hi[DV][136];  // bf16 S slice [dv][dk+pad]
     __shared__ __attribute__((aligned(16))) uint16_t s_lo[DV][136];  // S - s_hi
     __shared__ __attribute__((aligned(16))) uint16_t u_hi[DV][72];   // U^T [dv][token+pad]
@@ -1049,121 +1072,153 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
     const uint32_t local = blockIdx.y;
     const uint32_t slice = local % kSlicesPerHead;
     const uint32_t h = blockIdx.x * (kGdnValueHeads / 8) + local / kSlicesPerHead;
-    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t w = wave & 3;
+    const bool state_wave = wave < 4;
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t m = lane & 15;
     const uint32_t g = lane >> 4;
     const uint32_t chunks = (a.rows + kChunk - 1) / kChunk;
+    const uint32_t at = w * 16 + g * 4;  // this lane's token rows of a chunk
 
-    // State slice transposed, [dk tile][dv tile]: this lane holds key rows
-    // 32w+16mt+4g+i of value column 16nt+m, four consecutive keys of one state row.
-    f32x4 sacc[2][NT];
+    if (state_wave) {
+        // State slice transposed, [dk tile][dv]: this lane holds key rows
+        // 32w+16mt+4g+i of value column m, four consecutive keys of one state row.
+        f32x4 sacc[2];
 #pragma unroll
-    for (uint32_t mt = 0; mt < 2; ++mt) {
-#pragma unroll
-        for (uint32_t nt = 0; nt < NT; ++nt) {
-            const uint32_t j = nt * 16 + m;
-            const uint32_t dk = wave * 32 + mt * 16 + g * 4;
+        for (uint32_t mt = 0; mt < 2; ++mt) {
+            const uint32_t dk = w * 32 + mt * 16 + g * 4;
             const f32x4 v = *reinterpret_cast<const f32x4*>(
-                a.state_in + (static_cast<uint64_t>(h) * kGD + slice * DV + j) * kGD + dk);
-            sacc[mt][nt] = v;
+                a.state_in + (static_cast<uint64_t>(h) * kGD + slice * DV + m) * kGD + dk);
+            sacc[mt] = v;
             u32x2 hi, lo;
             split4(v, hi, lo);
-            *reinterpret_cast<u32x2*>(&s_hi[j][dk]) = hi;
-            *reinterpret_cast<u32x2*>(&s_lo[j][dk]) = lo;
+            *reinterpret_cast<u32x2*>(&s_hi[m][dk]) = hi;
+            *reinterpret_cast<u32x2*>(&s_lo[m][dk]) = lo;
         }
-    }
-    ChunkOperands<NT> cur = load_chunk<NT>(a, 0, h, slice, wave, m, g);
-    __syncthreads();
-
-    for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-        // the next chunk's operands are requested before this chunk's products
-        const ChunkOperands<NT> nxt =
-            load_chunk<NT>(a, min(chunk + 1, chunks - 1), h, slice, wave, m, g);
-        // P1 = Wk S^T and P2 = Q S^T for token tile w: [16 x DV]
-        f32x4 y[NT];
-        const uint32_t at = wave * 16 + g * 4;
-#pragma unroll
-        for (uint32_t nt = 0; nt < NT; ++nt) {
+        const uint32_t last = chunks - 1;
+        const auto fetch = [&](uint32_t chunk) {
+            return load_state_operands(chunk_record(a, min(chunk, last), h), slice, w, lane);
+        };
+        // one chunk of the recurrence with the operands `cur`
+        const auto step = [&](const StateOperands& cur) {
+            // P1 = Wk S^T for token tile w: [16 x 16]
             f32x4 p1 = {0.0f, 0.0f, 0.0f, 0.0f};
-            f32x4 p2 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (uint32_t kk = 0; kk < 4; ++kk) {
-                const bf16x8 sh = operand(&s_hi[nt * 16 + m][kk * 32 + g * 8]);
-                const bf16x8 sl = operand(&s_lo[nt * 16 + m][kk * 32 + g * 8]);
+                const bf16x8 sh = operand(&s_hi[m][kk * 32 + g * 8]);
+                const bf16x8 sl = operand(&s_lo[m][kk * 32 + g * 8]);
                 p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_lo[kk], sh, p1, 0, 0, 0);
-                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sl, p2, 0, 0, 0);
                 p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sl, p1, 0, 0, 0);
-                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sh, p2, 0, 0, 0);
                 p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sh, p1, 0, 0, 0);
             }
-            // U = Wv - P1; this lane holds tokens 16w+4g+i of value column 16nt+m
-            const f32x4 u = cur.wv[nt] - p1;
+            // U = Wv - P1; this lane holds tokens 16w+4g+i of value column m
+            const f32x4 u = cur.wv - p1;
             const f32x4 d = u * cur.ratio;
-            y[nt] = p2 * cur.gam;
             u32x2 uh, ul, dh, dl;
             split4(u, uh, ul);
             split4(d, dh, dl);
-            *reinterpret_cast<u32x2*>(&u_hi[nt * 16 + m][at]) = uh;
-            *reinterpret_cast<u32x2*>(&u_lo[nt * 16 + m][at]) = ul;
-            *reinterpret_cast<u32x2*>(&d_hi[nt * 16 + m][at]) = dh;
-            *reinterpret_cast<u32x2*>(&d_lo[nt * 16 + m][at]) = dl;
-        }
-        __syncthreads();  // U^T complete; every read of the old state copy is done
-        // Y = g o (Q S^T) + A U
-#pragma unroll
-        for (uint32_t nt = 0; nt < NT; ++nt) {
+            *reinterpret_cast<u32x2*>(&u_hi[m][at]) = uh;
+            *reinterpret_cast<u32x2*>(&u_lo[m][at]) = ul;
+            *reinterpret_cast<u32x2*>(&d_hi[m][at]) = dh;
+            *reinterpret_cast<u32x2*>(&d_lo[m][at]) = dl;
+            __syncthreads();  // U^T complete; every read of the old state copy is done
+            // S^T = g_C S^T + K^T ((g_C/g) o U) for key rows 32w..32w+31
+            bf16x8 dlo[2], dhi[2];
 #pragma unroll
             for (uint32_t k2 = 0; k2 < 2; ++k2) {
-                const bf16x8 bh = operand(&u_hi[nt * 16 + m][k2 * 32 + g * 8]);
-                const bf16x8 bl = operand(&u_lo[nt * 16 + m][k2 * 32 + g * 8]);
-                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_lo[k2], bh, y[nt], 0, 0, 0);
-                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bl, y[nt], 0, 0, 0);
-                y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bh, y[nt], 0, 0, 0);
+                dlo[k2] = operand(&d_lo[m][k2 * 32 + g * 8]);
+                dhi[k2] = operand(&d_hi[m][k2 * 32 + g * 8]);
             }
+#pragma unroll
+            for (uint32_t mt = 0; mt < 2; ++mt) {
+                sacc[mt] *= cur.gamma_c;
+#pragma unroll
+                for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                    sacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dlo[k2], sacc[mt], 0, 0, 0);
+                    sacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dhi[k2], sacc[mt], 0, 0, 0);
+                }
+                u32x2 hi, lo;
+                split4(sacc[mt], hi, lo);
+                const uint32_t dk = w * 32 + mt * 16 + g * 4;
+                *reinterpret_cast<u32x2*>(&s_hi[m][dk]) = hi;
+                *reinterpret_cast<u32x2*>(&s_lo[m][dk]) = lo;
+            }
+            __syncthreads();  // new state copy visible; U^T free for the next chunk
+        };
+        // Operands are requested two chunks ahead of their use, in three register sets
+        // that take turns (no copies: a copy would wait for the newest request).
+        StateOperands set_a = fetch(0);
+        StateOperands set_b = fetch(1);
+        __syncthreads();
+        for (uint32_t chunk = 0; chunk < chunks; chunk += 3) {
+            const StateOperands set_c = fetch(chunk + 2);
+            step(set_a);
+            if (chunk + 1 < chunks) {
+                set_a = fetch(chunk + 3);
+                step(set_b);
+            }
+            if (chunk + 2 < chunks) {
+                set_b = fetch(chunk + 4);
+                step(set_c);
+            }
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < 2; ++mt) {
+            const uint32_t dk = w * 32 + mt * 16 + g * 4;
+            *reinterpret_cast<f32x4*>(a.state_out +
+                                      (static_cast<uint64_t>(h) * kGD + slice * DV + m) * kGD + dk) = sacc[mt];
+        }
+    } else {
+        const uint32_t last = chunks - 1;
+        const auto fetch = [&](uint32_t chunk) {
+            return load_output_operands(chunk_record(a, min(chunk, last), h), w, lane);
+        };
+        const auto step = [&](const OutputOperands& cur, uint32_t chunk) {
+            // P2 = Q S^T for token tile w against the state the chunk starts from
+            f32x4 p2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t kk = 0; kk < 4; ++kk) {
+                const bf16x8 sh = operand(&s_hi[m][kk * 32 + g * 8]);
+                const bf16x8 sl = operand(&s_lo[m][kk * 32 + g * 8]);
+                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sl, p2, 0, 0, 0);
+                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sh, p2, 0, 0, 0);
+            }
+            f32x4 y = p2 * cur.gam;
+            __syncthreads();  // U^T complete; this wave is done with the old state copy
+            // Y = g o (Q S^T) + A U
+#pragma unroll
+            for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                const bf16x8 bh = operand(&u_hi[m][k2 * 32 + g * 8]);
+                const bf16x8 bl = operand(&u_lo[m][k2 * 32 + g * 8]);
+                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_lo[k2], bh, y, 0, 0, 0);
+                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bl, y, 0, 0, 0);
+                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bh, y, 0, 0, 0);
+            }
+            __syncthreads();  // this wave is done with U^T
 #pragma unroll
             for (uint32_t i = 0; i < 4; ++i) {
                 const uint32_t token = chunk * kChunk + at + i;
                 if (token < a.rows) {
-                    a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV +
-                        nt * 16 + m] = narrow(y[nt][i]);
+                    a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV + m] =
+                        narrow(y[i]);
                 }
             }
-        }
-        // S^T = g_C S^T + K^T ((g_C/g) o U) for key rows 32w..32w+31
-#pragma unroll
-        for (uint32_t mt = 0; mt < 2; ++mt) {
-#pragma unroll
-            for (uint32_t nt = 0; nt < NT; ++nt) {
-                sacc[mt][nt] *= cur.gamma_c;
-#pragma unroll
-                for (uint32_t k2 = 0; k2 < 2; ++k2) {
-                    const bf16x8 dl = operand(&d_lo[nt * 16 + m][k2 * 32 + g * 8]);
-                    const bf16x8 dh = operand(&d_hi[nt * 16 + m][k2 * 32 + g * 8]);
-                    sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dl,
-                                                                           sacc[mt][nt], 0, 0, 0);
-                    sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dh,
-                                                                           sacc[mt][nt], 0, 0, 0);
-                }
-                const f32x4 v = sacc[mt][nt];
-                u32x2 hi, lo;
-                split4(v, hi, lo);
-                const uint32_t dk = wave * 32 + mt * 16 + g * 4;
-                *reinterpret_cast<u32x2*>(&s_hi[nt * 16 + m][dk]) = hi;
-                *reinterpret_cast<u32x2*>(&s_lo[nt * 16 + m][dk]) = lo;
+        };
+        OutputOperands set_a = fetch(0);
+        OutputOperands set_b = fetch(1);
+        __syncthreads();
+        for (uint32_t chunk = 0; chunk < chunks; chunk += 3) {
+            const OutputOperands set_c = fetch(chunk + 2);
+            step(set_a, chunk);
+            if (chunk + 1 < chunks) {
+                set_a = fetch(chunk + 3);
+                step(set_b, chunk + 1);
             }
-        }
-        __syncthreads();  // new state copy visible; U^T free for the next chunk
-        cur = nxt;
-    }
-#pragma unroll
-    for (uint32_t mt = 0; mt < 2; ++mt) {
-#pragma unroll
-        for (uint32_t nt = 0; nt < NT; ++nt) {
-            const uint32_t j = slice * DV + nt * 16 + m;
-            const uint32_t dk = wave * 32 + mt * 16 + g * 4;
-            *reinterpret_cast<f32x4*>(a.state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + dk) =
-                sacc[mt][nt];
+            if (chunk + 2 < chunks) {
+                set_b = fetch(chunk + 4);
+                step(set_c, chunk + 2);
+            }
         }
     }
 }
@@ -1528,7 +1583,7 @@ int32_t op_gdn_chunk_scan(const Bindings& b, const Grid& g, hipStream_t stream,
     p.y = a.buffer<uint16_t>(2, static_cast<uint64_t>(p.rows) * kGdnValueValues * 2);
     p.state_out = a.buffer<float>(3, kGdnStateFloats * 4ull);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(512), 0, stream, p);
     return TT_OK;
 }
 
@@ -1576,7 +1631,7 @@ int32_t op_gdn_chunk_recurrence(const Bindings& b, const Grid& g, hipStream_t st
         c.state_out = state_out;
         c.y = y + static_cast<uint64_t>(start) * kGdnValueValues;
         c.rows = count;
-        hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(256), 0, stream, c);
+        hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(512), 0, stream, c);
     }
     return TT_OK;
 }
