@@ -987,9 +987,11 @@ struct ChunkScanArgs {
 
 // One chunk's operands of one wave, loaded a chunk ahead of their use.  The state
 // waves carry the recurrence, the output waves everything that only leaves it.
+template <uint32_t NT>
 struct StateOperands {
     bf16x8 wk_hi[4], wk_lo[4], kt[2][2];
-    f32x4 wv, ratio;
+    f32x4 wv[NT];
+    f32x4 ratio;
     float gamma_c;
 };
 struct OutputOperands {
@@ -1006,9 +1008,10 @@ __device__ __forceinline__ u32x4 record_fragment(const uint8_t* rec, uint32_t ba
     return *reinterpret_cast<const u32x4*>(rec + base + (index * 64 + lane) * 16);
 }
 
-__device__ __forceinline__ StateOperands load_state_operands(const uint8_t* rec, uint32_t slice,
-                                                             uint32_t w, uint32_t lane) {
-    StateOperands o;
+template <uint32_t NT>
+__device__ __forceinline__ StateOperands<NT> load_state_operands(const uint8_t* rec, uint32_t slice,
+                                                                 uint32_t w, uint32_t lane) {
+    StateOperands<NT> o;
     const uint32_t g = lane >> 4;
 #pragma unroll
     for (uint32_t kk = 0; kk < 4; ++kk) {
@@ -1023,7 +1026,10 @@ __device__ __forceinline__ StateOperands load_state_operands(const uint8_t* rec,
                 __builtin_bit_cast(bf16x8, record_fragment(rec, kRecKt, (w * 2 + mt) * 2 + k2, lane));
         }
     }
-    o.wv = __builtin_bit_cast(f32x4, record_fragment(rec, kRecWv, slice * 4 + w, lane));
+#pragma unroll
+    for (uint32_t nt = 0; nt < NT; ++nt) {
+        o.wv[nt] = __builtin_bit_cast(f32x4, record_fragment(rec, kRecWv, (slice * NT + nt) * 4 + w, lane));
+    }
     o.ratio = *reinterpret_cast<const f32x4*>(rec + kRecRatio + (w * 16 + g * 4) * 4);
     o.gamma_c = *reinterpret_cast<const float*>(rec + kRecGamma);
     return o;
@@ -1057,8 +1063,7 @@ __device__ __forceinline__ OutputOperands load_output_operands(const uint8_t* re
 // LDS copies between all eight waves.
 template <uint32_t NT>
 __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
-    static_assert(NT == 1, "one 16-wide value slice per workgroup");
-    constexpr uint32_t DV = 16;
+    constexpr uint32_t DV = 16 * NT;
     __shared__ __attribute__((aligned(16))) uint16_t s_hi[DV][136];  // bf16 S slice [dv][dk+pad]
     __shared__ __attribute__((aligned(16))) uint16_t s_lo[DV][136];  // S - s_hi
     __shared__ __attribute__((aligned(16))) uint16_t u_hi[DV][72];   // U^T [dv][token+pad]
@@ -1084,75 +1089,87 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
     if (state_wave) {
         // State slice transposed, [dk tile][dv]: this lane holds key rows
         // 32w+16mt+4g+i of value column m, four consecutive keys of one state row.
-        f32x4 sacc[2];
+        f32x4 sacc[2][NT];
 #pragma unroll
         for (uint32_t mt = 0; mt < 2; ++mt) {
-            const uint32_t dk = w * 32 + mt * 16 + g * 4;
-            const f32x4 v = *reinterpret_cast<const f32x4*>(
-                a.state_in + (static_cast<uint64_t>(h) * kGD + slice * DV + m) * kGD + dk);
-            sacc[mt] = v;
-            u32x2 hi, lo;
-            split4(v, hi, lo);
-            *reinterpret_cast<u32x2*>(&s_hi[m][dk]) = hi;
-            *reinterpret_cast<u32x2*>(&s_lo[m][dk]) = lo;
+#pragma unroll
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                const uint32_t j = nt * 16 + m;
+                const uint32_t dk = w * 32 + mt * 16 + g * 4;
+                const f32x4 v = *reinterpret_cast<const f32x4*>(
+                    a.state_in + (static_cast<uint64_t>(h) * kGD + slice * DV + j) * kGD + dk);
+                sacc[mt][nt] = v;
+                u32x2 hi, lo;
+                split4(v, hi, lo);
+                *reinterpret_cast<u32x2*>(&s_hi[j][dk]) = hi;
+                *reinterpret_cast<u32x2*>(&s_lo[j][dk]) = lo;
+            }
         }
         const uint32_t last = chunks - 1;
         const auto fetch = [&](uint32_t chunk) {
-            return load_state_operands(chunk_record(a, min(chunk, last), h), slice, w, lane);
+            return load_state_operands<NT>(chunk_record(a, min(chunk, last), h), slice, w, lane);
         };
         // one chunk of the recurrence with the operands `cur`
-        const auto step = [&](const StateOperands& cur) {
-            // P1 = Wk S^T for token tile w: [16 x 16]
-            f32x4 p1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        const auto step = [&](const StateOperands<NT>& cur) {
+            // P1 = Wk S^T for token tile w: [16 x DV]
 #pragma unroll
-            for (uint32_t kk = 0; kk < 4; ++kk) {
-                const bf16x8 sh = operand(&s_hi[m][kk * 32 + g * 8]);
-                const bf16x8 sl = operand(&s_lo[m][kk * 32 + g * 8]);
-                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_lo[kk], sh, p1, 0, 0, 0);
-                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sl, p1, 0, 0, 0);
-                p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sh, p1, 0, 0, 0);
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                f32x4 p1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (uint32_t kk = 0; kk < 4; ++kk) {
+                    const bf16x8 sh = operand(&s_hi[nt * 16 + m][kk * 32 + g * 8]);
+                    const bf16x8 sl = operand(&s_lo[nt * 16 + m][kk * 32 + g * 8]);
+                    p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_lo[kk], sh, p1, 0, 0, 0);
+                    p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sl, p1, 0, 0, 0);
+                    p1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.wk_hi[kk], sh, p1, 0, 0, 0);
+                }
+                // U = Wv - P1; this lane holds tokens 16w+4g+i of value column 16nt+m
+                const f32x4 u = cur.wv[nt] - p1;
+                const f32x4 d = u * cur.ratio;
+                u32x2 uh, ul, dh, dl;
+                split4(u, uh, ul);
+                split4(d, dh, dl);
+                *reinterpret_cast<u32x2*>(&u_hi[nt * 16 + m][at]) = uh;
+                *reinterpret_cast<u32x2*>(&u_lo[nt * 16 + m][at]) = ul;
+                *reinterpret_cast<u32x2*>(&d_hi[nt * 16 + m][at]) = dh;
+                *reinterpret_cast<u32x2*>(&d_lo[nt * 16 + m][at]) = dl;
             }
-            // U = Wv - P1; this lane holds tokens 16w+4g+i of value column m
-            const f32x4 u = cur.wv - p1;
-            const f32x4 d = u * cur.ratio;
-            u32x2 uh, ul, dh, dl;
-            split4(u, uh, ul);
-            split4(d, dh, dl);
-            *reinterpret_cast<u32x2*>(&u_hi[m][at]) = uh;
-            *reinterpret_cast<u32x2*>(&u_lo[m][at]) = ul;
-            *reinterpret_cast<u32x2*>(&d_hi[m][at]) = dh;
-            *reinterpret_cast<u32x2*>(&d_lo[m][at]) = dl;
             __syncthreads();  // U^T complete; every read of the old state copy is done
             // S^T = g_C S^T + K^T ((g_C/g) o U) for key rows 32w..32w+31
-            bf16x8 dlo[2], dhi[2];
 #pragma unroll
-            for (uint32_t k2 = 0; k2 < 2; ++k2) {
-                dlo[k2] = operand(&d_lo[m][k2 * 32 + g * 8]);
-                dhi[k2] = operand(&d_hi[m][k2 * 32 + g * 8]);
-            }
-#pragma unroll
-            for (uint32_t mt = 0; mt < 2; ++mt) {
-                sacc[mt] *= cur.gamma_c;
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                bf16x8 dlo[2], dhi[2];
 #pragma unroll
                 for (uint32_t k2 = 0; k2 < 2; ++k2) {
-                    sacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dlo[k2], sacc[mt], 0, 0, 0);
-                    sacc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dhi[k2], sacc[mt], 0, 0, 0);
+                    dlo[k2] = operand(&d_lo[nt * 16 + m][k2 * 32 + g * 8]);
+                    dhi[k2] = operand(&d_hi[nt * 16 + m][k2 * 32 + g * 8]);
                 }
-                u32x2 hi, lo;
-                split4(sacc[mt], hi, lo);
-                const uint32_t dk = w * 32 + mt * 16 + g * 4;
-                *reinterpret_cast<u32x2*>(&s_hi[m][dk]) = hi;
-                *reinterpret_cast<u32x2*>(&s_lo[m][dk]) = lo;
+#pragma unroll
+                for (uint32_t mt = 0; mt < 2; ++mt) {
+                    sacc[mt][nt] *= cur.gamma_c;
+#pragma unroll
+                    for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                        sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dlo[k2],
+                                                                               sacc[mt][nt], 0, 0, 0);
+                        sacc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kt[mt][k2], dhi[k2],
+                                                                               sacc[mt][nt], 0, 0, 0);
+                    }
+                    u32x2 hi, lo;
+                    split4(sacc[mt][nt], hi, lo);
+                    const uint32_t dk = w * 32 + mt * 16 + g * 4;
+                    *reinterpret_cast<u32x2*>(&s_hi[nt * 16 + m][dk]) = hi;
+                    *reinterpret_cast<u32x2*>(&s_lo[nt * 16 + m][dk]) = lo;
+                }
             }
             __syncthreads();  // new state copy visible; U^T free for the next chunk
         };
         // Operands are requested two chunks ahead of their use, in three register sets
         // that take turns (no copies: a copy would wait for the newest request).
-        StateOperands set_a = fetch(0);
-        StateOperands set_b = fetch(1);
+        StateOperands<NT> set_a = fetch(0);
+        StateOperands<NT> set_b = fetch(1);
         __syncthreads();
         for (uint32_t chunk = 0; chunk < chunks; chunk += 3) {
-            const StateOperands set_c = fetch(chunk + 2);
+            const StateOperands<NT> set_c = fetch(chunk + 2);
             step(set_a);
             if (chunk + 1 < chunks) {
                 set_a = fetch(chunk + 3);
@@ -1165,9 +1182,12 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
         }
 #pragma unroll
         for (uint32_t mt = 0; mt < 2; ++mt) {
-            const uint32_t dk = w * 32 + mt * 16 + g * 4;
-            *reinterpret_cast<f32x4*>(a.state_out +
-                                      (static_cast<uint64_t>(h) * kGD + slice * DV + m) * kGD + dk) = sacc[mt];
+#pragma unroll
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                const uint32_t dk = w * 32 + mt * 16 + g * 4;
+                *reinterpret_cast<f32x4*>(a.state_out + (static_cast<uint64_t>(h) * kGD + slice * DV +
+                                                         nt * 16 + m) * kGD + dk) = sacc[mt][nt];
+            }
         }
     } else {
         const uint32_t last = chunks - 1;
@@ -1176,32 +1196,42 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
         };
         const auto step = [&](const OutputOperands& cur, uint32_t chunk) {
             // P2 = Q S^T for token tile w against the state the chunk starts from
-            f32x4 p2 = {0.0f, 0.0f, 0.0f, 0.0f};
+            f32x4 y[NT];
 #pragma unroll
-            for (uint32_t kk = 0; kk < 4; ++kk) {
-                const bf16x8 sh = operand(&s_hi[m][kk * 32 + g * 8]);
-                const bf16x8 sl = operand(&s_lo[m][kk * 32 + g * 8]);
-                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sl, p2, 0, 0, 0);
-                p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sh, p2, 0, 0, 0);
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+                f32x4 p2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (uint32_t kk = 0; kk < 4; ++kk) {
+                    const bf16x8 sh = operand(&s_hi[nt * 16 + m][kk * 32 + g * 8]);
+                    const bf16x8 sl = operand(&s_lo[nt * 16 + m][kk * 32 + g * 8]);
+                    p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sl, p2, 0, 0, 0);
+                    p2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.q[kk], sh, p2, 0, 0, 0);
+                }
+                y[nt] = p2 * cur.gam;
             }
-            f32x4 y = p2 * cur.gam;
             __syncthreads();  // U^T complete; this wave is done with the old state copy
             // Y = g o (Q S^T) + A U
 #pragma unroll
-            for (uint32_t k2 = 0; k2 < 2; ++k2) {
-                const bf16x8 bh = operand(&u_hi[m][k2 * 32 + g * 8]);
-                const bf16x8 bl = operand(&u_lo[m][k2 * 32 + g * 8]);
-                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_lo[k2], bh, y, 0, 0, 0);
-                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bl, y, 0, 0, 0);
-                y = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bh, y, 0, 0, 0);
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (uint32_t k2 = 0; k2 < 2; ++k2) {
+                    const bf16x8 bh = operand(&u_hi[nt * 16 + m][k2 * 32 + g * 8]);
+                    const bf16x8 bl = operand(&u_lo[nt * 16 + m][k2 * 32 + g * 8]);
+                    y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_lo[k2], bh, y[nt], 0, 0, 0);
+                    y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bl, y[nt], 0, 0, 0);
+                    y[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.aq_hi[k2], bh, y[nt], 0, 0, 0);
+                }
             }
             __syncthreads();  // this wave is done with U^T
 #pragma unroll
-            for (uint32_t i = 0; i < 4; ++i) {
-                const uint32_t token = chunk * kChunk + at + i;
-                if (token < a.rows) {
-                    a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV + m] =
-                        narrow(y[i]);
+            for (uint32_t nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    const uint32_t token = chunk * kChunk + at + i;
+                    if (token < a.rows) {
+                        a.y[static_cast<uint64_t>(token) * kGdnValueValues + h * kGD + slice * DV +
+                            nt * 16 + m] = narrow(y[nt][i]);
+                    }
                 }
             }
         };
@@ -1222,6 +1252,10 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkScanArgs a) {
         }
     }
 }
+
+// value tiles of 16 per scan workgroup: 1 -> 256 workgroups (0.47 ms for 16384 rows),
+// 2 -> 128 workgroups with half the L2 traffic (0.57 ms: the chunk chain gets longer)
+constexpr uint32_t kScanTiles = 1;
 
 // ---------------------------------------------------------------- launchers --
 
@@ -1583,7 +1617,7 @@ int32_t op_gdn_chunk_scan(const Bindings& b, const Grid& g, hipStream_t stream,
     p.y = a.buffer<uint16_t>(2, static_cast<uint64_t>(p.rows) * kGdnValueValues * 2);
     p.state_out = a.buffer<float>(3, kGdnStateFloats * 4ull);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(512), 0, stream, p);
+    hipLaunchKernelGGL(gdn_chunk_scan_kernel<kScanTiles>, dim3(8, kGdnValueHeads / kScanTiles), dim3(512), 0, stream, p);
     return TT_OK;
 }
 
@@ -1631,7 +1665,7 @@ int32_t op_gdn_chunk_recurrence(const Bindings& b, const Grid& g, hipStream_t st
         c.state_out = state_out;
         c.y = y + static_cast<uint64_t>(start) * kGdnValueValues;
         c.rows = count;
-        hipLaunchKernelGGL(gdn_chunk_scan_kernel<1>, dim3(8, kGdnValueHeads), dim3(512), 0, stream, c);
+        hipLaunchKernelGGL(gdn_chunk_scan_kernel<kScanTiles>, dim3(8, kGdnValueHeads / kScanTiles), dim3(512), 0, stream, c);
     }
     return TT_OK;
 }
