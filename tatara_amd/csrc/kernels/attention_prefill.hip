@@ -549,7 +549,8 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     a.require(g.gx == 16 && g.gy == (f.rows + 15) / 16 && g.gz == 1 && g.tx == 256 && g.ty == 1 &&
                   g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
-    a.require(f.capacity != 0 &&
+    // the kernel addresses a kv head's rows with 32-bit byte offsets (512 B per key)
+    a.require(f.capacity != 0 && f.capacity <= (1u << 23) &&
                   static_cast<uint64_t>(f.tile_context) + f.rows == visible &&
                   visible <= f.capacity,
               TT_CMD_CONTEXT_OUT_OF_RANGE);
