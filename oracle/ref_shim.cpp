@@ -51,6 +51,13 @@ void ref_rms_only(const std::uint16_t* in, const std::uint16_t* w, std::uint32_t
                        std::span<std::uint16_t>(out, hidden));
 }
 
+void ref_residual_sums(const std::uint16_t* a, const std::uint16_t* b, std::uint64_t count,
+                       std::uint16_t* out) {
+    residual_rms_rounded_sums(std::span<const std::uint16_t>(a, count),
+                              std::span<const std::uint16_t>(b, count),
+                              std::span<std::uint16_t>(out, count));
+}
+
 void ref_attn_qk_rope(const std::uint16_t* projection, const std::uint16_t* q_weight,
                       const std::uint16_t* k_weight, std::uint32_t position,
                       std::uint32_t capacity, std::uint16_t* q_out, std::uint16_t* gate_out,

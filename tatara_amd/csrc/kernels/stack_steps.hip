@@ -6,6 +6,9 @@
 //   rms_only, rms_only_ms  src/backend/metal/kernels/rms_only.metal:5, :44
 //       (dispatch: decode_step.cpp:641-645, 1103-1109; grid 1 x hidden/4 threads,
 //       _ms adds the row in grid y with element strides in c3 / c4)
+//   residual_rms, residual_rms_ms  src/backend/metal/kernels/moe.metal:1, :551
+//       (dispatch: decode_step.cpp:735-742, 1298-1308): residual = bf16(a + b), then the
+//       same row norm over the rounded sums, both written
 //   dense_bf16, add_bf16   no reference counterpart: the reference projects with
 //       4-bit weights (q4_dot.metal); here the weights are plain bf16.
 #include "../tt_internal.h"
@@ -37,15 +40,34 @@ __device__ __forceinline__ uint16_t fz16(uint16_t h) {
 // hidden/4 threads: thread t squares values 4t..4t+3 in order, 32-lane groups sum
 // in the adjacent-pairs tree (= xor butterfly), the group sums land in a 32-slot
 // stage that is summed by the same tree; out = bf16(w * bf16(x * inverse)).
+// With `addend`, the row normalised is residual = bf16(input + addend), which is also
+// written to `residual_out` (residual_rms): the norm consumes the rounded sums.
 __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, const uint16_t* weight,
                                                         uint16_t* output, uint32_t hidden,
-                                                        uint32_t in_stride, uint32_t out_stride) {
+                                                        uint32_t in_stride, uint32_t out_stride,
+                                                        const uint16_t* addend, uint16_t* residual_out,
+                                                        uint32_t residual_stride) {
     __shared__ float stage[32];
     __shared__ float inverse_norm;
     const uint32_t t = threadIdx.x;
     const uint16_t* in = input + static_cast<uint64_t>(blockIdx.y) * in_stride;
     uint16_t* out = output + static_cast<uint64_t>(blockIdx.y) * out_stride;
-    const u32x2 raw = *reinterpret_cast<const u32x2*>(in + 4 * t);
+    u32x2 raw = *reinterpret_cast<const u32x2*>(in + 4 * t);
+    if (addend != nullptr) {
+        const u32x2 other = *reinterpret_cast<const u32x2*>(
+            addend + static_cast<uint64_t>(blockIdx.y) * residual_stride + 4 * t);
+        uint16_t sum[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint16_t xa = static_cast<uint16_t>(raw[i >> 1] >> ((i & 1) * 16));
+            const uint16_t xb = static_cast<uint16_t>(other[i >> 1] >> ((i & 1) * 16));
+            sum[i] = store16(widen(fz16(xa)) + widen(fz16(xb)));
+        }
+        raw = u32x2{sum[0] | (static_cast<uint32_t>(sum[1]) << 16),
+                    sum[2] | (static_cast<uint32_t>(sum[3]) << 16)};
+        *reinterpret_cast<u32x2*>(residual_out + static_cast<uint64_t>(blockIdx.y) * residual_stride +
+                                  4 * t) = raw;
+    }
     const float x0 = __uint_as_float(raw.x << 16), x1 = __uint_as_float(raw.x & 0xFFFF0000u);
     const float x2 = __uint_as_float(raw.y << 16), x3 = __uint_as_float(raw.y & 0xFFFF0000u);
     float sum = 0.0f;
@@ -143,8 +165,49 @@ int32_t launch_rms(const Bindings& b, const Grid& g, hipStream_t stream, bool va
         a.buffer<uint16_t>(2, (static_cast<uint64_t>(rows - 1) * out_stride + hidden) * 2);
     if (a.status != TT_OK || validate_only) return a.status;
     hipLaunchKernelGGL(rms_only_kernel, dim3(1, rows), dim3(hidden / 4), 0, stream, input, weight,
-                       output, hidden, in_stride, out_stride);
+                       output, hidden, in_stride, out_stride, static_cast<const uint16_t*>(nullptr),
+                       static_cast<uint16_t*>(nullptr), 0u);
     return TT_OK;
+}
+
+// residual_rms: b0 a, b1 b, b2 residual out (may alias b), b3 weight, b4 normed out;
+// grid 1 x hidden/4 (decode_step.cpp:735-742).  residual_rms_ms: + c5 row stride of a,
+// c6 row stride of b and of the residual, c7 row stride of the normed output
+// (elements); grid (1, rows) x hidden/4 (decode_step.cpp:1298-1308).
+int32_t launch_residual_rms(const Bindings& b, const Grid& g, hipStream_t stream,
+                            bool validate_only, bool strided) {
+    Args a(b);
+    a.require(g.gx == 1 && g.gz == 1 && g.ty == 1 && g.tz == 1 && g.tx >= 32 && g.tx <= 1024 &&
+                  g.tx % 32 == 0 && g.gy >= 1 && g.gy <= 65535 && (strided || g.gy == 1),
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    const uint32_t hidden = static_cast<uint32_t>(g.tx) * 4;
+    const uint32_t rows = static_cast<uint32_t>(g.gy);
+    const uint32_t a_stride = strided ? a.constant(5) : hidden;
+    const uint32_t lane_stride = strided ? a.constant(6) : hidden;
+    const uint32_t normed_stride = strided ? a.constant(7) : hidden;
+    a.require(a_stride >= hidden && lane_stride >= hidden && normed_stride >= hidden,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK) return a.status;
+    const auto extent = [&](uint32_t stride) {
+        return (static_cast<uint64_t>(rows - 1) * stride + hidden) * 2;
+    };
+    const uint16_t* first = a.buffer<const uint16_t>(0, extent(a_stride));
+    const uint16_t* second = a.buffer<const uint16_t>(1, extent(lane_stride));
+    uint16_t* residual = a.buffer<uint16_t>(2, extent(lane_stride));
+    const uint16_t* weight = a.buffer<const uint16_t>(3, static_cast<uint64_t>(hidden) * 2);
+    uint16_t* normed = a.buffer<uint16_t>(4, extent(normed_stride));
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(rms_only_kernel, dim3(1, rows), dim3(hidden / 4), 0, stream, first, weight,
+                       normed, hidden, a_stride, normed_stride, second, residual, lane_stride);
+    return TT_OK;
+}
+int32_t op_residual_rms(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only) {
+    return launch_residual_rms(b, g, stream, validate_only, false);
+}
+int32_t op_residual_rms_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                           bool validate_only) {
+    return launch_residual_rms(b, g, stream, validate_only, true);
 }
 
 // rms_only: b0 input, b1 weight, b2 output; grid 1 x hidden/4.
@@ -200,6 +263,8 @@ int32_t op_add_bf16(const Bindings& b, const Grid& g, hipStream_t stream, bool v
 const KernelDesc kStackStepKernels[] = {
     {"rms_only", op_rms_only},
     {"rms_only_ms", op_rms_only_ms},
+    {"residual_rms", op_residual_rms},
+    {"residual_rms_ms", op_residual_rms_ms},
     {"dense_bf16", op_dense_bf16},
     {"add_bf16", op_add_bf16},
 };

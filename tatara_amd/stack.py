@@ -7,7 +7,10 @@ does model-shaped work.  Per layer:
     n = rms_only(x, input_norm);  p = dense(n, W_in)
     a = GatedDeltaNet(p) | FullAttention(p);  x = x + dense(a, W_out)
 
-and after the last layer  logits = dense(rms_only(x, final_norm), W_vocab).
+and after the last layer  logits = dense(rms_only(x, final_norm), W_vocab).  The
+residual sum of a layer and the norm that follows it (the next layer's input norm or
+the final norm) are one dispatch, residual_rms_ms, as in the reference's layer loop
+(decode_step.cpp:1298-1308).
 
 The walk mirrors the reference's layer loop (src/runtime/decode_step.cpp:1008-1293
 for a token wave over pooled lanes, prefill_step.cpp:1386-2081 for a block of one
@@ -145,14 +148,18 @@ class StubStack:
                   (1, rows), (HIDDEN // 4,))
         cb.barrier()
 
-    def _residual(self, cb, rows):
-        n = rows * HIDDEN
-        cb.encode(self.lib.pipeline("add_bf16"), {0: self.x, 1: self.delta, 2: self.x}, {3: n},
-                  ((n + 255) // 256,), (256,))
+    def _residual_and_norm(self, cb, rows, index):
+        """x = bf16(x + delta) in place and normed = the norm layer `index + 1` (or the
+        head) starts from."""
+        following = (self.layers[index + 1]["input_norm"] if index + 1 < len(self.layers)
+                     else self.final_norm)
+        cb.encode(self.lib.pipeline("residual_rms_ms"),
+                  {0: self.x, 1: self.delta, 2: self.x, 3: following, 4: self.normed},
+                  {5: HIDDEN, 6: HIDDEN, 7: HIDDEN}, (1, rows), (HIDDEN // 4,))
         cb.barrier()
 
     def _head(self, cb, rows):
-        self._rms(cb, self.x, self.final_norm, self.normed, rows)
+        """The final norm has been applied by the last layer's residual step."""
         self._dense(cb, self.normed, self.w_vocab, self.logits, rows, HIDDEN, self.vocab)
 
     # ---- one token for every lane ----
@@ -160,8 +167,8 @@ class StubStack:
         """Records one decode step of all lanes; the lanes' inputs are rows of self.x.
         Call advance_token_wave() after the recording has been committed."""
         P, rows = self.lib.pipeline, self.lanes
-        for layer in self.layers:
-            self._rms(cb, self.x, layer["input_norm"], self.normed, rows)
+        self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
+        for index, layer in enumerate(self.layers):
             if layer["kind"] == "G":
                 self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
                 cb.encode(P("gdn_decode_fused_ms"),
@@ -186,7 +193,7 @@ class StubStack:
                           {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
             cb.barrier()
             self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
-            self._residual(cb, rows)
+            self._residual_and_norm(cb, rows, index)
         if with_head:
             self._head(cb, rows)
 
@@ -207,8 +214,8 @@ class StubStack:
         base = self.context[lane]
         stripe_bytes = 2 * self.capacity * 256 * 2
         plane_in, plane_out = self._gdn_planes(lane)
-        for layer in self.layers:
-            self._rms(cb, self.x, layer["input_norm"], self.normed, rows)
+        self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
+        for index, layer in enumerate(self.layers):
             if layer["kind"] == "G":
                 self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
                 conv_in = (layer["conv"], plane_in * CONV_ELEMS * 2)
@@ -247,7 +254,7 @@ class StubStack:
                           (16, (rows + 15) // 16), (256,))
             cb.barrier()
             self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
-            self._residual(cb, rows)
+            self._residual_and_norm(cb, rows, index)
         if with_head:
             self._head(cb, rows)
 

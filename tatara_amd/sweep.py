@@ -14,7 +14,7 @@ import numpy as np
 from . import backend as B
 from . import stack as S
 
-STUB_KERNELS = {"rms_only", "rms_only_ms", "dense_bf16", "add_bf16"}
+STUB_KERNELS = {"rms_only", "rms_only_ms", "residual_rms_ms", "dense_bf16", "add_bf16"}
 
 
 def _family_ms(times):

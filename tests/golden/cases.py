@@ -12,6 +12,7 @@ ATTN_CAPACITY = 512
 ATTN_CHAIN_POSITIONS = 5
 ATTN_CONTEXTS = (4, 300, 200)
 GDN_SEED = 0x6D46EED5
+RESIDUAL_SEED = 0x2E51D0A1
 GDN_CHAIN_STEPS = 4
 STATE_SAMPLE_STRIDE = 997
 

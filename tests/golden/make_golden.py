@@ -99,6 +99,21 @@ def main():
         if step == cases.GDN_CHAIN_STEPS - 1:
             out["gdn_conv_state_final"] = ncs.copy()
         st_in, cs = st_out, ncs
+    # residual sum and row norm either side of the family (hidden 2048, two rows)
+    hidden = 2048
+    res_a = ref_fill(cases.RESIDUAL_SEED, 2 * hidden)
+    res_b = ref_fill(cases.RESIDUAL_SEED + 1, 2 * hidden)
+    norm_w = ref_fill(cases.RESIDUAL_SEED + 2, hidden)
+    sums = np.zeros(2 * hidden, np.uint16)
+    r.ref_residual_sums(res_a, res_b, 2 * hidden, sums)
+    normed = np.zeros(2 * hidden, np.uint16)
+    for row in range(2):
+        part = np.zeros(hidden, np.uint16)
+        r.ref_rms_only(np.ascontiguousarray(sums[row * hidden:(row + 1) * hidden]), norm_w, hidden,
+                       1, 0, part)
+        normed[row * hidden:(row + 1) * hidden] = part
+    out["residual_sums"] = sums
+    out["residual_normed"] = normed
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

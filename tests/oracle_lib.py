@@ -97,6 +97,7 @@ def _load_ref():
         "ref_fill_banded_bf16": (None, [u64, _u16p, u64]),
         "ref_tree_sum": (f32, [_f32p, u32, u32]),
         "ref_rms_only": (None, [_u16p, _u16p, u32, u32, u32, _u16p]),
+        "ref_residual_sums": (None, [_u16p, _u16p, u64, _u16p]),
         "ref_attn_qk_rope": (None, [_u16p, _u16p, _u16p, u32, u32, _u16p, _u16p, _u16p, _u16p]),
         "ref_attention_decode": (None, [_u16p, _u16p, _u16p, _u16p, u32, u32, _u16p]),
         "ref_attention_decode_split": (None, [_u16p, _u16p, _u16p, _u16p, u32, u32, u32, _f32n,

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
-from gpu_util import gpu
+from gpu_util import gpu, run
 
 pytestmark = pytest.mark.gpu
 o = ol.oracle
@@ -117,3 +117,38 @@ def test_stacked_prefill_and_greedy_decode_match_the_checker():
             _compare(f"decode step {step} lane {lane}", got[lane], want[0])
             tokens[lane] = int(want[0].argmax())
     assert gpu_stack.context == [24 + 3, 9 + 3]
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 2048), (5, 2048), (3, 256), (2, 4096)])
+def test_residual_rms_operators(rows, hidden):
+    """residual = bf16(a + b) and the row norm of the rounded sums, single row and
+    strided rows, bit for bit against the checker (add, then rms_only)."""
+    print(f"[case] residual_rms rows={rows} hidden={hidden}", flush=True)
+    B, dev, queue, lib = gpu()
+    a = ol.gaussian_bf16(0xA1 + rows, rows * hidden, 0.0, 2.0)
+    b = ol.gaussian_bf16(0xB1 + rows, rows * hidden, 0.0, 0.5)
+    w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0xC1, hidden))
+    sums = np.zeros(rows * hidden, np.uint16)
+    o.tto_add_bf16(a, b, rows * hidden, sums)
+    normed = np.zeros(rows * hidden, np.uint16)
+    o.tto_rms_only(sums, w, rows, hidden, normed)
+    b_a, b_b, b_w = dev.buffer_from(a), dev.buffer_from(b), dev.buffer_from(w)
+    b_res, b_norm = dev.create_buffer(rows * hidden * 2), dev.create_buffer(rows * hidden * 2)
+
+    def rec(cb):
+        if rows == 1:
+            cb.encode(lib.pipeline("residual_rms"), {0: b_a, 1: b_b, 2: b_res, 3: b_w, 4: b_norm}, {},
+                      (1,), (hidden // 4,))
+        else:
+            cb.encode(lib.pipeline("residual_rms_ms"), {0: b_a, 1: b_b, 2: b_res, 3: b_w, 4: b_norm},
+                      {5: hidden, 6: hidden, 7: hidden}, (1, rows), (hidden // 4,))
+    run(rec)
+    assert np.array_equal(b_res.read(np.uint16), sums)
+    assert np.array_equal(b_norm.read(np.uint16), normed)
+    # in place on the second operand, as the layer loop uses it
+    def rec2(cb):
+        cb.encode(lib.pipeline("residual_rms_ms"), {0: b_a, 1: b_b, 2: b_b, 3: b_w, 4: b_norm},
+                  {5: hidden, 6: hidden, 7: hidden}, (1, rows), (hidden // 4,))
+    run(rec2)
+    assert np.array_equal(b_b.read(np.uint16), sums)
+    assert np.array_equal(b_norm.read(np.uint16), normed)

@@ -129,3 +129,17 @@ def test_gdn_fused_step_and_prefill_equal_chain():
     assert np.array_equal(gated_blk.reshape(T, 4096), np.stack(gated_steps))
     assert np.array_equal(st_blk.view(np.uint32), st_in.view(np.uint32))
     assert np.array_equal(ncs, cs)
+
+
+def test_residual_sum_and_row_norm():
+    """bf16(a + b) and the row norm of the rounded sums (residual_rms, moe.metal:1-46)."""
+    hidden = 2048
+    a = fill(cases.RESIDUAL_SEED, 2 * hidden)
+    b = fill(cases.RESIDUAL_SEED + 1, 2 * hidden)
+    w = fill(cases.RESIDUAL_SEED + 2, hidden)
+    sums = np.zeros(2 * hidden, np.uint16)
+    o.tto_add_bf16(a, b, 2 * hidden, sums)
+    assert np.array_equal(sums, G["residual_sums"])
+    normed = np.zeros(2 * hidden, np.uint16)
+    o.tto_rms_only(sums, w, 2, hidden, normed)
+    assert np.array_equal(normed, G["residual_normed"])

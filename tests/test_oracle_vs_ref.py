@@ -92,3 +92,18 @@ def test_rms_only_rows(hidden, kind):
         want = np.zeros(hidden, np.uint16)
         r.ref_rms_only(np.ascontiguousarray(x[row * hidden:(row + 1) * hidden]), w, hidden, 1, 0, want)
         assert np.array_equal(got[row * hidden:(row + 1) * hidden], want)
+
+
+@pytest.mark.parametrize("kind", ["banded", "gauss"])
+def test_residual_sums(kind):
+    """tto_add_bf16 against residual_rms_rounded_sums (kernel_reference.cpp:1160-1165)."""
+    n = 3 * 2048
+    if kind == "banded":
+        a, b = ol.banded_bf16(0x7E5, n), ol.banded_bf16(0x7E6, n)
+    else:
+        a, b = ol.gaussian_bf16(0x7E7, n, 0.0, 2.0), ol.gaussian_bf16(0x7E8, n, 0.0, 1e-3)
+    got = np.zeros(n, np.uint16)
+    want = np.zeros(n, np.uint16)
+    o.tto_add_bf16(a, b, n, got)
+    r.ref_residual_sums(a, b, n, want)
+    assert np.array_equal(got, want)
