@@ -884,6 +884,8 @@ PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan
     const std::uint64_t capacity = policy.context_capacity;
     g.attention_partitions =
         (policy.context_capacity + policy.attention_partition - 1u) / policy.attention_partition;
+    g.key_value_heads = plan.key_value_heads;
+    g.attention_head_dimension = plan.head_dimension;
     g.gdn_projection_rows = rows.gdn_projection;
     g.gdn_qk_values = rows.gdn_qk;
     g.gdn_value_values = rows.gdn_values;
@@ -1135,6 +1137,554 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
     walk.buffer(scratch.gdn_gated, 0, 3);
     walk.dispatch(32, 128, rows);
     return walk.error;
+}
+
+// ---- lane state record (Q36BRS01) ------------------------------------------
+
+namespace {
+
+constexpr std::uint64_t kRecordKvHeads = 2;                 // decode_harness.cpp:26
+constexpr std::uint64_t kRecordHeadRowBytes = 256 * 2;      // decode_harness.cpp:27
+
+bool fetch(const HipBuffer& buffer, std::uint64_t offset, std::byte* destination,
+           std::uint64_t length) {
+    return tt_buffer_read(buffer.native(), offset, destination, length) == TT_OK;
+}
+bool store(const HipBuffer& buffer, std::uint64_t offset, const std::byte* source,
+           std::uint64_t length) {
+    return tt_buffer_write(buffer.native(), offset, source, length) == TT_OK;
+}
+
+}  // namespace
+
+std::uint64_t state_record_bytes(const DecodeStep& step, std::uint32_t positions) noexcept {
+    if (positions == 0 || positions > step.capacity) return 0;
+    std::uint64_t bytes = kStateRecordHeaderBytes;
+    for (const LayerKind kind : step.schedule) {
+        bytes += is_gated(kind)
+                     ? step.geometry.gdn_conv_state_bytes + step.geometry.gdn_recurrent_state_bytes
+                     : 2 * kRecordKvHeads * positions * kRecordHeadRowBytes;
+    }
+    return bytes;
+}
+
+StateRecordError write_state_record(const DecodeStep& step, const DecodeStateSlot& state,
+                                    std::uint32_t positions, std::vector<std::byte>& record) {
+    if (!decode_state_slot_ready(step, state)) return StateRecordError::InvalidState;
+    const std::uint64_t total = state_record_bytes(step, positions);
+    if (total == 0) return StateRecordError::InvalidPositions;
+    record.assign(total, std::byte{0});
+    std::memcpy(record.data(), kStateRecordMagic, 8);
+    std::memcpy(record.data() + 8, &positions, 4);
+    std::uint64_t cursor = kStateRecordHeaderBytes;
+    const std::uint64_t head_bytes = positions * kRecordHeadRowBytes;
+    const std::uint64_t cache_head_stride = std::uint64_t{step.capacity} * kRecordHeadRowBytes;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        const DecodeLayerState& s = state.layers[layer];
+        if (is_gated(step.schedule[layer])) {
+            const bool live_out = gated_delta_live_is_out(s.swapped);
+            const HipBuffer& conv = live_out ? s.first_out : s.first;
+            const HipBuffer& recurrent = live_out ? s.second_out : s.second;
+            if (!fetch(conv, 0, record.data() + cursor, step.geometry.gdn_conv_state_bytes)) {
+                return StateRecordError::TransferFailed;
+            }
+            cursor += step.geometry.gdn_conv_state_bytes;
+            if (!fetch(recurrent, 0, record.data() + cursor,
+                       step.geometry.gdn_recurrent_state_bytes)) {
+                return StateRecordError::TransferFailed;
+            }
+            cursor += step.geometry.gdn_recurrent_state_bytes;
+        } else {
+            for (const HipBuffer* plane : {&s.first, &s.second}) {
+                for (std::uint64_t head = 0; head < kRecordKvHeads; ++head) {
+                    if (!fetch(*plane, head * cache_head_stride, record.data() + cursor, head_bytes)) {
+                        return StateRecordError::TransferFailed;
+                    }
+                    cursor += head_bytes;
+                }
+            }
+        }
+    }
+    return cursor == total ? StateRecordError::None : StateRecordError::TransferFailed;
+}
+
+StateRecordError load_state_record(std::span<const std::byte> record, const DecodeStep& step,
+                                   DecodeStateSlot& state, std::uint32_t& positions) {
+    if (!decode_state_slot_ready(step, state)) return StateRecordError::InvalidState;
+    if (record.size() < kStateRecordHeaderBytes) return StateRecordError::Truncated;
+    if (std::memcmp(record.data(), kStateRecordMagic, 8) != 0) return StateRecordError::MagicMismatch;
+    std::uint32_t count = 0;
+    std::memcpy(&count, record.data() + 8, 4);
+    const std::uint64_t total = state_record_bytes(step, count);
+    if (total == 0) return StateRecordError::InvalidPositions;
+    if (record.size() < total) return StateRecordError::Truncated;
+    if (record.size() > total) return StateRecordError::TrailingBytes;
+    std::uint64_t cursor = kStateRecordHeaderBytes;
+    const std::uint64_t head_bytes = count * kRecordHeadRowBytes;
+    const std::uint64_t cache_head_stride = std::uint64_t{step.capacity} * kRecordHeadRowBytes;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        DecodeLayerState& s = state.layers[layer];
+        if (is_gated(step.schedule[layer])) {
+            if (!store(s.first, 0, record.data() + cursor, step.geometry.gdn_conv_state_bytes)) {
+                return StateRecordError::TransferFailed;
+            }
+            cursor += step.geometry.gdn_conv_state_bytes;
+            if (!store(s.second, 0, record.data() + cursor,
+                       step.geometry.gdn_recurrent_state_bytes)) {
+                return StateRecordError::TransferFailed;
+            }
+            cursor += step.geometry.gdn_recurrent_state_bytes;
+            s.swapped = false;  // the installed planes are the ones the next step reads
+        } else {
+            for (const HipBuffer* plane : {&s.first, &s.second}) {
+                for (std::uint64_t head = 0; head < kRecordKvHeads; ++head) {
+                    if (!store(*plane, head * cache_head_stride, record.data() + cursor, head_bytes)) {
+                        return StateRecordError::TransferFailed;
+                    }
+                    cursor += head_bytes;
+                }
+            }
+        }
+    }
+    positions = count;
+    return StateRecordError::None;
+}
+
+// ---- prefix state snapshot / restore ---------------------------------------
+namespace {
+
+// 64-bit products and sums that report wrap-around instead of hiding it
+bool product(std::uint64_t a, std::uint64_t b, std::uint64_t& out) noexcept {
+    return !__builtin_mul_overflow(a, b, &out);
+}
+bool total(std::uint64_t a, std::uint64_t b, std::uint64_t& out) noexcept {
+    return !__builtin_add_overflow(a, b, &out);
+}
+bool extent_holds(std::uint64_t offset, std::uint64_t length, std::uint64_t extent) noexcept {
+    return offset <= extent && length <= extent - offset;
+}
+bool known_kind(LayerKind kind) noexcept {
+    return kind == LayerKind::GatedDelta || kind == LayerKind::FullAttention;
+}
+
+constexpr std::uint32_t kNoLayer = std::numeric_limits<std::uint32_t>::max();
+
+// schedule index of the `ordinal`-th layer of one family
+std::uint32_t nth_of_family(std::span<const LayerKind> schedule, bool gated,
+                            std::uint32_t ordinal) noexcept {
+    for (std::uint32_t layer = 0; layer < schedule.size(); ++layer) {
+        if (is_gated(schedule[layer]) != gated) continue;
+        if (ordinal == 0) return layer;
+        --ordinal;
+    }
+    return kNoLayer;
+}
+
+const HipBuffer* plane_of(const DecodeLayerState& layer, PrefixStateBufferPlane plane) noexcept {
+    switch (plane) {
+    case PrefixStateBufferPlane::First: return &layer.first;
+    case PrefixStateBufferPlane::FirstOutput: return &layer.first_out;
+    case PrefixStateBufferPlane::Second: return &layer.second;
+    case PrefixStateBufferPlane::SecondOutput: return &layer.second_out;
+    case PrefixStateBufferPlane::Arena: break;
+    }
+    return nullptr;
+}
+
+void forget_transfer(DecodeStateSlot& state) noexcept {
+    state.active_transfer_generation = 0;
+    state.active_transfer_arena = nullptr;
+    state.active_transfer_positions = 0;
+    state.active_transfer_offset_bytes = 0;
+    state.active_transfer_state_bytes = 0;
+}
+
+PrefixStateTransferResult refused(PrefixStateTransferError error,
+                                  PrefixStateLayoutError layout = PrefixStateLayoutError::None,
+                                  HipCommandError command = HipCommandError::None) noexcept {
+    PrefixStateTransferResult r;
+    r.error = error;
+    r.layout_error = layout;
+    r.command_error = command;
+    return r;
+}
+
+bool ticket_current(const PrefixStateTransferTicket& ticket, const DecodeStep& decode,
+                    const DecodeStateSlot& state, const HipBuffer& arena) noexcept {
+    const DecodeStateSlotStatus pending =
+        ticket.direction == PrefixStateTransferDirection::Snapshot
+            ? DecodeStateSlotStatus::SnapshotPending
+            : DecodeStateSlotStatus::RestorePending;
+    return ticket.generation != 0 && ticket.owner == &decode && ticket.state_owner == &state &&
+           ticket.arena_owner == &arena && state.status == pending &&
+           decode_state_slot_compatible(decode, state) &&
+           state.active_transfer_generation == ticket.generation &&
+           state.active_transfer_arena == &arena &&
+           state.active_transfer_positions == ticket.positions &&
+           state.active_transfer_offset_bytes == ticket.arena_offset_bytes &&
+           state.active_transfer_state_bytes == ticket.state_bytes;
+}
+
+// One copy of a transfer: the slot-side buffer and both offsets.
+struct PlannedCopy {
+    const HipBuffer* slot_buffer{nullptr};
+    std::uint64_t slot_offset{0};
+    std::uint64_t arena_offset{0};
+    std::uint64_t length{0};
+};
+
+bool plan_copy(const PrefixStateLayout& layout, std::uint32_t index,
+               PrefixStateTransferDirection direction, const DecodeStateSlot& state,
+               const HipBuffer& arena, std::uint64_t arena_base, PlannedCopy& copy,
+               PrefixStateLayoutError& layout_error) noexcept {
+    const PrefixStateSegmentResult found = prefix_state_segment(layout, index);
+    layout_error = found.error;
+    if (!found || found.segment.layer_index >= state.layers.size()) return false;
+    const DecodeLayerState& layer = state.layers[found.segment.layer_index];
+    const PrefixStateCopyRoute route = prefix_state_copy_route(found.segment, direction, layer.swapped);
+    copy.slot_buffer = plane_of(layer, direction == PrefixStateTransferDirection::Snapshot
+                                           ? route.source
+                                           : route.destination);
+    copy.slot_offset = found.segment.slot_offset_bytes;
+    copy.length = found.segment.length_bytes;
+    return copy.slot_buffer != nullptr && copy.slot_buffer != &arena &&
+           extent_holds(copy.slot_offset, copy.length, copy.slot_buffer->size_bytes()) &&
+           total(arena_base, found.segment.snapshot_offset_bytes, copy.arena_offset) &&
+           extent_holds(copy.arena_offset, copy.length, arena.size_bytes());
+}
+
+PrefixStateTransferResult encode_prefix_transfer(PrefixStateTransferDirection direction,
+                                                 const DecodeStep& decode, DecodeStateSlot& state,
+                                                 const PrefillGeometry& geometry,
+                                                 HipBlitPass& blit_pass, HipBuffer& arena,
+                                                 std::uint64_t arena_base, std::uint32_t positions,
+                                                 std::span<std::byte> evidence) noexcept {
+    const bool snapshot = direction == PrefixStateTransferDirection::Snapshot;
+    if (state.status == DecodeStateSlotStatus::Poisoned) {
+        return refused(PrefixStateTransferError::PoisonedStateSlot);
+    }
+    if (!decode_state_slot_compatible(decode, state) || !decode_state_slot_complete(decode, state)) {
+        return refused(PrefixStateTransferError::InvalidStateSlot);
+    }
+    if (!decode_state_slot_ready(decode, state)) {
+        return refused(PrefixStateTransferError::StateSlotNotReady);
+    }
+    if (!arena) return refused(PrefixStateTransferError::InvalidArena);
+    const std::size_t evidence_bytes =
+        snapshot ? prefix_state_phase_evidence_bytes(decode.schedule) : 0;
+    if (evidence.size() < evidence_bytes) {
+        return refused(PrefixStateTransferError::PhaseEvidenceTooSmall);
+    }
+    const PrefixStateLayoutResult made = make_prefix_state_layout(decode, geometry, positions);
+    if (!made) return refused(PrefixStateTransferError::InvalidLayout, made.error);
+    const PrefixStateLayout& layout = made.layout;
+    if (validate_prefix_state_arena_extent(layout, arena_base, arena.size_bytes()) !=
+        PrefixStateTransferError::None) {
+        return refused(PrefixStateTransferError::ArenaOutOfRange);
+    }
+    if (state.next_transfer_generation == 0) {
+        return refused(PrefixStateTransferError::GenerationExhausted);
+    }
+    if (!blit_pass) {
+        return refused(PrefixStateTransferError::CommandEncodingFailed, PrefixStateLayoutError::None,
+                       HipCommandError::InvalidBlitPass);
+    }
+    // every copy is checked before the first one is issued, so a refusal leaves
+    // both the slot and the arena untouched
+    for (std::uint32_t index = 0; index < layout.segment_count; ++index) {
+        PlannedCopy copy;
+        PrefixStateLayoutError layout_error = PrefixStateLayoutError::None;
+        if (!plan_copy(layout, index, direction, state, arena, arena_base, copy, layout_error)) {
+            return layout_error != PrefixStateLayoutError::None
+                       ? refused(PrefixStateTransferError::InvalidLayout, layout_error)
+                       : refused(PrefixStateTransferError::InvalidStateSlot);
+        }
+    }
+    for (std::uint32_t index = 0; index < layout.segment_count; ++index) {
+        PlannedCopy copy;
+        PrefixStateLayoutError layout_error = PrefixStateLayoutError::None;
+        (void)plan_copy(layout, index, direction, state, arena, arena_base, copy, layout_error);
+        const HipCommandError command =
+            snapshot ? copy_buffer(blit_pass, *copy.slot_buffer, copy.slot_offset, arena,
+                                   copy.arena_offset, copy.length)
+                     : copy_buffer(blit_pass, arena, copy.arena_offset,
+                                   const_cast<HipBuffer&>(*copy.slot_buffer), copy.slot_offset,
+                                   copy.length);
+        if (command != HipCommandError::None) {
+            state.status = DecodeStateSlotStatus::Poisoned;
+            forget_transfer(state);
+            return refused(PrefixStateTransferError::CommandEncodingFailed,
+                           PrefixStateLayoutError::None, command);
+        }
+    }
+    if (snapshot) {
+        const PrefixStateTransferError captured =
+            capture_prefix_state_phase_evidence(decode, state, evidence.first(evidence_bytes));
+        if (captured != PrefixStateTransferError::None) return refused(captured);
+    }
+    const std::uint64_t generation = state.next_transfer_generation;
+    state.next_transfer_generation =
+        generation == std::numeric_limits<std::uint64_t>::max() ? 0 : generation + 1u;
+    state.active_transfer_generation = generation;
+    state.active_transfer_arena = &arena;
+    state.active_transfer_positions = positions;
+    state.active_transfer_offset_bytes = arena_base;
+    state.active_transfer_state_bytes = layout.total_bytes;
+    state.status = snapshot ? DecodeStateSlotStatus::SnapshotPending
+                            : DecodeStateSlotStatus::RestorePending;
+    PrefixStateTransferResult done;
+    done.error = PrefixStateTransferError::None;
+    done.segment_count = layout.segment_count;
+    done.state_bytes = layout.total_bytes;
+    done.source_phase_evidence_bytes = evidence_bytes;
+    done.ticket = PrefixStateTransferTicket{direction,  &decode,          &state,
+                                            &arena,     positions,        arena_base,
+                                            layout.total_bytes, generation, true};
+    return done;
+}
+
+}  // namespace
+
+PrefixStateLayoutResult make_prefix_state_layout(const PrefixStateLayoutSpec& spec) noexcept {
+    const auto fail = [](PrefixStateLayoutError error) {
+        return PrefixStateLayoutResult{error, {}};
+    };
+    if (spec.schedule.empty() || spec.schedule.size() > std::numeric_limits<std::uint32_t>::max()) {
+        return fail(PrefixStateLayoutError::InvalidSchedule);
+    }
+    if (spec.capacity == 0 || spec.key_value_heads == 0 || spec.head_dimension == 0 ||
+        spec.expected_gated_delta_layers == 0 || spec.expected_attention_layers == 0 ||
+        spec.gated_delta_convolution_bytes == 0 || spec.gated_delta_recurrent_bytes == 0 ||
+        spec.expected_total_bytes == 0) {
+        return fail(PrefixStateLayoutError::InvalidGeometry);
+    }
+    if (spec.positions == 0 || spec.positions > spec.capacity) {
+        return fail(PrefixStateLayoutError::PositionOutOfRange);
+    }
+    PrefixStateLayout layout;
+    layout.specification = spec;
+    for (const LayerKind kind : spec.schedule) {
+        if (!known_kind(kind)) return fail(PrefixStateLayoutError::InvalidSchedule);
+        (is_gated(kind) ? layout.gated_delta_layers : layout.attention_layers) += 1;
+    }
+    if (layout.gated_delta_layers != spec.expected_gated_delta_layers ||
+        layout.attention_layers != spec.expected_attention_layers) {
+        return fail(PrefixStateLayoutError::FamilyCountMismatch);
+    }
+    // payload = G x (conv + recurrent) + A x 2 x kv_heads x positions x head_dimension bf16
+    const std::uint64_t row_bytes = std::uint64_t{spec.head_dimension} * kBf16Bytes;
+    std::uint64_t live_pair = 0, head_segments = 0, segments = 0;
+    const bool fits =
+        total(spec.gated_delta_convolution_bytes, spec.gated_delta_recurrent_bytes, live_pair) &&
+        product(live_pair, layout.gated_delta_layers, layout.gated_delta_bytes) &&
+        product(spec.positions, row_bytes, layout.attention_segment_bytes) &&
+        product(spec.capacity, row_bytes, layout.attention_slot_head_stride_bytes) &&
+        product(std::uint64_t{layout.attention_layers} * 2u, spec.key_value_heads, head_segments) &&
+        product(head_segments, layout.attention_segment_bytes, layout.attention_bytes) &&
+        total(layout.gated_delta_bytes, layout.attention_bytes, layout.total_bytes) &&
+        total(std::uint64_t{layout.gated_delta_layers} * 2u, head_segments, segments) &&
+        segments <= std::numeric_limits<std::uint32_t>::max();
+    if (!fits) return fail(PrefixStateLayoutError::Overflow);
+    if (layout.total_bytes != spec.expected_total_bytes) {
+        return fail(PrefixStateLayoutError::TotalMismatch);
+    }
+    layout.segment_count = static_cast<std::uint32_t>(segments);
+    return {PrefixStateLayoutError::None, layout};
+}
+
+PrefixStateLayoutResult make_prefix_state_layout(const DecodeStep& decode,
+                                                 const PrefillGeometry& geometry,
+                                                 std::uint32_t positions) noexcept {
+    const auto fail = [](PrefixStateLayoutError error) {
+        return PrefixStateLayoutResult{error, {}};
+    };
+    if (decode.capacity == 0 || geometry.policy.context_capacity != decode.capacity ||
+        geometry.key_value_heads == 0 || geometry.attention_head_dimension == 0 ||
+        geometry.gated_delta_layers == 0 || geometry.attention_layers == 0) {
+        return fail(PrefixStateLayoutError::InvalidGeometry);
+    }
+    // the prefill extents must describe the very buffers this step allocated
+    const std::uint64_t live_pair =
+        decode.geometry.gdn_conv_state_bytes + decode.geometry.gdn_recurrent_state_bytes;
+    const std::uint64_t per_position = 2ull * geometry.key_value_heads *
+                                       geometry.attention_head_dimension * kBf16Bytes;
+    if (live_pair != geometry.gdn_live_state_bytes_per_layer ||
+        per_position != geometry.attention_state_bytes_per_position_per_layer ||
+        2u * decode.geometry.attn_cache_bytes != geometry.attention_slot_state_bytes_per_layer) {
+        return fail(PrefixStateLayoutError::InvalidGeometry);
+    }
+    if (positions == 0 || positions > decode.capacity) {
+        return fail(PrefixStateLayoutError::PositionOutOfRange);
+    }
+    const PrefixStateSnapshotGeometry sized = make_prefix_state_snapshot_geometry(geometry, positions);
+    if (!sized.valid) return fail(PrefixStateLayoutError::InvalidGeometry);
+    PrefixStateLayoutSpec spec;
+    spec.schedule = decode.schedule;
+    spec.capacity = decode.capacity;
+    spec.positions = positions;
+    spec.key_value_heads = geometry.key_value_heads;
+    spec.head_dimension = geometry.attention_head_dimension;
+    spec.expected_gated_delta_layers = geometry.gated_delta_layers;
+    spec.expected_attention_layers = geometry.attention_layers;
+    spec.gated_delta_convolution_bytes = decode.geometry.gdn_conv_state_bytes;
+    spec.gated_delta_recurrent_bytes = decode.geometry.gdn_recurrent_state_bytes;
+    spec.expected_total_bytes = sized.total_bytes;
+    return make_prefix_state_layout(spec);
+}
+
+PrefixStateSegmentResult prefix_state_segment(const PrefixStateLayout& layout,
+                                              std::uint32_t index) noexcept {
+    if (index >= layout.segment_count) return {PrefixStateLayoutError::SegmentOutOfRange, {}};
+    const PrefixStateLayoutSpec& spec = layout.specification;
+    PrefixStateSegment segment;
+    const std::uint32_t gated_segments = 2u * layout.gated_delta_layers;
+    if (index < gated_segments) {
+        // (conv, recurrent) pairs, one pair per gated-delta layer
+        const std::uint32_t ordinal = index >> 1;
+        const bool recurrent = (index & 1u) != 0;
+        segment.layer_index = nth_of_family(spec.schedule, true, ordinal);
+        segment.kind = recurrent ? PrefixStateSegmentKind::GatedDeltaRecurrent
+                                 : PrefixStateSegmentKind::GatedDeltaConvolution;
+        segment.length_bytes =
+            recurrent ? spec.gated_delta_recurrent_bytes : spec.gated_delta_convolution_bytes;
+        segment.snapshot_offset_bytes =
+            ordinal * (spec.gated_delta_convolution_bytes + spec.gated_delta_recurrent_bytes) +
+            (recurrent ? spec.gated_delta_convolution_bytes : 0);
+    } else {
+        // per attention layer: keys of head 0..H-1, then values of head 0..H-1
+        const std::uint32_t packed = index - gated_segments;
+        const std::uint32_t per_layer = 2u * spec.key_value_heads;
+        const std::uint32_t within = packed % per_layer;
+        const bool value = within >= spec.key_value_heads;
+        segment.layer_index = nth_of_family(spec.schedule, false, packed / per_layer);
+        segment.kind =
+            value ? PrefixStateSegmentKind::AttentionValue : PrefixStateSegmentKind::AttentionKey;
+        segment.head_index = value ? within - spec.key_value_heads : within;
+        segment.slot_offset_bytes = segment.head_index * layout.attention_slot_head_stride_bytes;
+        segment.length_bytes = layout.attention_segment_bytes;
+        segment.snapshot_offset_bytes =
+            layout.gated_delta_bytes + packed * layout.attention_segment_bytes;
+    }
+    if (segment.layer_index == kNoLayer) return {PrefixStateLayoutError::FamilyCountMismatch, {}};
+    return {PrefixStateLayoutError::None, segment};
+}
+
+PrefixStateCopyRoute prefix_state_copy_route(const PrefixStateSegment& segment,
+                                             PrefixStateTransferDirection direction,
+                                             bool gated_delta_swapped) noexcept {
+    // the slot-side plane: a snapshot reads the live plane, a restore always
+    // writes the in plane (completion then clears `swapped`)
+    const bool out_plane =
+        direction == PrefixStateTransferDirection::Snapshot && gated_delta_swapped;
+    PrefixStateBufferPlane slot = PrefixStateBufferPlane::First;
+    switch (segment.kind) {
+    case PrefixStateSegmentKind::GatedDeltaConvolution:
+        slot = out_plane ? PrefixStateBufferPlane::FirstOutput : PrefixStateBufferPlane::First;
+        break;
+    case PrefixStateSegmentKind::GatedDeltaRecurrent:
+        slot = out_plane ? PrefixStateBufferPlane::SecondOutput : PrefixStateBufferPlane::Second;
+        break;
+    case PrefixStateSegmentKind::AttentionKey: slot = PrefixStateBufferPlane::First; break;
+    case PrefixStateSegmentKind::AttentionValue: slot = PrefixStateBufferPlane::Second; break;
+    }
+    return direction == PrefixStateTransferDirection::Snapshot
+               ? PrefixStateCopyRoute{slot, PrefixStateBufferPlane::Arena}
+               : PrefixStateCopyRoute{PrefixStateBufferPlane::Arena, slot};
+}
+
+PrefixStateTransferError validate_prefix_state_arena_extent(const PrefixStateLayout& layout,
+                                                            std::uint64_t arena_offset_bytes,
+                                                            std::uint64_t arena_capacity_bytes) noexcept {
+    if (layout.total_bytes == 0 || layout.segment_count == 0) {
+        return PrefixStateTransferError::InvalidLayout;
+    }
+    return extent_holds(arena_offset_bytes, layout.total_bytes, arena_capacity_bytes)
+               ? PrefixStateTransferError::None
+               : PrefixStateTransferError::ArenaOutOfRange;
+}
+
+std::size_t prefix_state_phase_evidence_bytes(std::span<const LayerKind> schedule) noexcept {
+    return (schedule.size() + 7u) / 8u;
+}
+
+PrefixStateTransferError capture_prefix_state_phase_evidence(const DecodeStep& decode,
+                                                             const DecodeStateSlot& state,
+                                                             std::span<std::byte> phase_evidence) noexcept {
+    if (phase_evidence.size() < prefix_state_phase_evidence_bytes(decode.schedule)) {
+        return PrefixStateTransferError::PhaseEvidenceTooSmall;
+    }
+    if (!decode_state_slot_compatible(decode, state)) {
+        return PrefixStateTransferError::InvalidStateSlot;
+    }
+    for (std::byte& b : phase_evidence) b = std::byte{0};
+    for (std::size_t layer = 0; layer < decode.schedule.size(); ++layer) {
+        if (is_gated(decode.schedule[layer]) && state.layers[layer].swapped) {
+            phase_evidence[layer >> 3] |= std::byte(1u << (layer & 7u));
+        }
+    }
+    return PrefixStateTransferError::None;
+}
+
+PrefixStateTransferResult encode_prefix_state_snapshot(const DecodeStep& decode,
+                                                       DecodeStateSlot& state,
+                                                       const PrefillGeometry& geometry,
+                                                       HipBlitPass& blit_pass, HipBuffer& state_arena,
+                                                       std::uint64_t arena_offset_bytes,
+                                                       std::uint32_t positions,
+                                                       std::span<std::byte> source_phase_evidence) noexcept {
+    return encode_prefix_transfer(PrefixStateTransferDirection::Snapshot, decode, state, geometry,
+                                  blit_pass, state_arena, arena_offset_bytes, positions,
+                                  source_phase_evidence);
+}
+
+PrefixStateTransferResult encode_prefix_state_restore(const DecodeStep& decode, DecodeStateSlot& state,
+                                                      const PrefillGeometry& geometry,
+                                                      HipBlitPass& blit_pass, HipBuffer& state_arena,
+                                                      std::uint64_t arena_offset_bytes,
+                                                      std::uint32_t positions) noexcept {
+    return encode_prefix_transfer(PrefixStateTransferDirection::Restore, decode, state, geometry,
+                                  blit_pass, state_arena, arena_offset_bytes, positions, {});
+}
+
+PrefixStateTransferError complete_prefix_state_transfer(PrefixStateTransferTicket& ticket,
+                                                        const DecodeStep& decode,
+                                                        DecodeStateSlot& state,
+                                                        const HipBuffer& state_arena) noexcept {
+    if (!ticket.pending) return PrefixStateTransferError::AlreadyCompleted;
+    if (state.status == DecodeStateSlotStatus::Poisoned) {
+        return PrefixStateTransferError::PoisonedStateSlot;
+    }
+    if (!ticket_current(ticket, decode, state, state_arena)) {
+        return PrefixStateTransferError::StaleTicket;
+    }
+    if (ticket.direction == PrefixStateTransferDirection::Restore) {
+        for (std::size_t layer = 0; layer < decode.schedule.size(); ++layer) {
+            if (is_gated(decode.schedule[layer])) state.layers[layer].swapped = false;
+        }
+    }
+    forget_transfer(state);
+    state.status = DecodeStateSlotStatus::Ready;
+    ticket.pending = false;
+    return PrefixStateTransferError::None;
+}
+
+PrefixStateTransferError abort_prefix_state_transfer(PrefixStateTransferTicket& ticket,
+                                                     const DecodeStep& decode, DecodeStateSlot& state,
+                                                     const HipBuffer& state_arena) noexcept {
+    if (!ticket.pending) return PrefixStateTransferError::AlreadyCompleted;
+    if (state.status == DecodeStateSlotStatus::Poisoned) {
+        forget_transfer(state);
+        ticket.pending = false;
+        return PrefixStateTransferError::PoisonedStateSlot;
+    }
+    if (!ticket_current(ticket, decode, state, state_arena)) {
+        return PrefixStateTransferError::StaleTicket;
+    }
+    // the copies may have landed partly: the slot is kept but never trusted again
+    forget_transfer(state);
+    state.status = DecodeStateSlotStatus::Poisoned;
+    ticket.pending = false;
+    return PrefixStateTransferError::None;
 }
 
 }  // namespace tatara::runtime

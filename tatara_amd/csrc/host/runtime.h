@@ -141,6 +141,10 @@ struct DecodeStateSlot {
     DecodeStateSlotStatus status{DecodeStateSlotStatus::Ready};
     std::uint64_t next_transfer_generation{1};
     std::uint64_t active_transfer_generation{0};
+    const HipBuffer* active_transfer_arena{nullptr};
+    std::uint32_t active_transfer_positions{0};
+    std::uint64_t active_transfer_offset_bytes{0};
+    std::uint64_t active_transfer_state_bytes{0};
     std::uint64_t next_reset_generation{1};
     std::uint64_t active_reset_generation{0};
     std::uint32_t active_reset_segments{0};
@@ -405,6 +409,8 @@ struct PrefillGeometry {
     std::uint32_t gated_delta_layers{0};
     std::uint32_t attention_layers{0};
     std::uint32_t attention_partitions{0};
+    std::uint32_t key_value_heads{0};
+    std::uint32_t attention_head_dimension{0};
     std::uint32_t gdn_projection_rows{0};
     std::uint32_t gdn_qk_values{0};
     std::uint32_t gdn_value_values{0};
@@ -502,5 +508,207 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
                                            const DecodeLayerState& state,
                                            const LayerWeights& weights, const PrefillChunk& chunk,
                                            std::uint32_t recurrence_ordinal, HipComputePass& pass);
+
+// ---- lane state record (Q36BRS01) ------------------------------------------
+// The file / wire form of exactly the buffers a lane owns on this path
+// (tools/native/decode_harness.cpp:25-27, 339-460; decode_harness.h:112-125):
+//   8 bytes magic "Q36BRS01", u32 positions, then per layer in schedule order
+//   gated delta: conv window [3][8192] bf16, recurrent state [32][128][128] f32 of
+//                the LIVE plane of each ping-pong pair;
+//   attention:   keys of kv head 0, keys of kv head 1, values of head 0, values of
+//                head 1, each `positions` rows of 256 bf16, packed (the caches are
+//                capacity-strided, the record is not).
+// The live plane is the one the last step wrote: advance_decode_state toggles
+// `swapped` after the write, so live is first_out / second_out exactly when
+// `swapped` is set (decode_harness.h:100-114).
+inline constexpr char kStateRecordMagic[8] = {'Q', '3', '6', 'B', 'R', 'S', '0', '1'};
+inline constexpr std::uint64_t kStateRecordHeaderBytes = 12;
+constexpr bool gated_delta_live_is_out(bool swapped) { return swapped; }
+
+enum class StateRecordError : std::uint8_t {
+    None,
+    InvalidState,       // slot not compatible with the step, or not Ready
+    InvalidPositions,   // zero, or more than the capacity
+    MagicMismatch,
+    Truncated,
+    TrailingBytes,
+    TransferFailed,
+};
+// Size of the record of `positions` cached tokens; 0 when positions is out of range.
+std::uint64_t state_record_bytes(const DecodeStep& step, std::uint32_t positions) noexcept;
+// Reads the lane's live planes and the first `positions` cache rows back from the
+// device into `record` (resized).  The slot is not modified.
+StateRecordError write_state_record(const DecodeStep& step, const DecodeStateSlot& state,
+                                    std::uint32_t positions, std::vector<std::byte>& record);
+// Installs a record into a Ready slot: gated-delta planes go to first / second and
+// `swapped` is cleared (the next step reads exactly those), attention rows go to
+// cache rows [0, positions).  On success `positions` is the context the lane
+// continues from.  Nothing is written unless the whole record parses.
+StateRecordError load_state_record(std::span<const std::byte> record, const DecodeStep& step,
+                                   DecodeStateSlot& state, std::uint32_t& positions);
+
+// ---- prefix state snapshot / restore ---------------------------------------
+// The device-resident form of the same state: one lane's live planes and its
+// first `positions` cache rows packed into a byte range of an arena buffer, and
+// back (prefix_state_transfer.h:13-186, prefix_state_transfer.cpp:311-575).
+// Unlike the record above the payload is family-major: every gated-delta layer
+// in schedule order (conv window, then recurrent state), then every attention
+// layer in schedule order (keys of each kv head, then values of each kv head,
+// `positions` rows each).  Restore always installs gated-delta bytes into
+// first / second and completion clears `swapped`.
+inline constexpr std::uint32_t kPrefixStateLayoutSchemaVersion = 1;
+inline constexpr std::uint32_t kPrefixStateTransferSchemaVersion = 1;
+
+enum class PrefixStateLayoutError : std::uint8_t {
+    None,
+    InvalidSchedule,
+    InvalidGeometry,
+    PositionOutOfRange,
+    FamilyCountMismatch,
+    TotalMismatch,
+    Overflow,
+    SegmentOutOfRange,
+};
+enum class PrefixStateSegmentKind : std::uint8_t {
+    GatedDeltaConvolution,
+    GatedDeltaRecurrent,
+    AttentionKey,
+    AttentionValue,
+};
+enum class PrefixStateBufferPlane : std::uint8_t { First, FirstOutput, Second, SecondOutput, Arena };
+enum class PrefixStateTransferDirection : std::uint8_t { Snapshot, Restore };
+
+struct PrefixStateLayoutSpec {
+    std::span<const LayerKind> schedule;
+    std::uint32_t capacity{0};
+    std::uint32_t positions{0};
+    std::uint32_t key_value_heads{0};
+    std::uint32_t head_dimension{0};
+    std::uint32_t expected_gated_delta_layers{0};
+    std::uint32_t expected_attention_layers{0};
+    std::uint64_t gated_delta_convolution_bytes{0};
+    std::uint64_t gated_delta_recurrent_bytes{0};
+    std::uint64_t expected_total_bytes{0};
+};
+struct PrefixStateLayout {
+    PrefixStateLayoutSpec specification;
+    std::uint32_t gated_delta_layers{0};
+    std::uint32_t attention_layers{0};
+    std::uint32_t segment_count{0};
+    std::uint64_t attention_segment_bytes{0};           // positions x head_dimension bf16
+    std::uint64_t attention_slot_head_stride_bytes{0};  // capacity x head_dimension bf16
+    std::uint64_t gated_delta_bytes{0};
+    std::uint64_t attention_bytes{0};
+    std::uint64_t total_bytes{0};
+};
+struct PrefixStateLayoutResult {
+    PrefixStateLayoutError error{PrefixStateLayoutError::InvalidGeometry};
+    PrefixStateLayout layout;
+    explicit constexpr operator bool() const noexcept {
+        return error == PrefixStateLayoutError::None;
+    }
+};
+struct PrefixStateSegment {
+    PrefixStateSegmentKind kind{PrefixStateSegmentKind::GatedDeltaConvolution};
+    std::uint32_t layer_index{0};
+    std::uint32_t head_index{0};
+    std::uint64_t slot_offset_bytes{0};
+    std::uint64_t snapshot_offset_bytes{0};
+    std::uint64_t length_bytes{0};
+};
+struct PrefixStateSegmentResult {
+    PrefixStateLayoutError error{PrefixStateLayoutError::SegmentOutOfRange};
+    PrefixStateSegment segment;
+    explicit constexpr operator bool() const noexcept {
+        return error == PrefixStateLayoutError::None;
+    }
+};
+struct PrefixStateCopyRoute {
+    PrefixStateBufferPlane source{PrefixStateBufferPlane::First};
+    PrefixStateBufferPlane destination{PrefixStateBufferPlane::Arena};
+};
+
+PrefixStateLayoutResult make_prefix_state_layout(const PrefixStateLayoutSpec& specification) noexcept;
+PrefixStateLayoutResult make_prefix_state_layout(const DecodeStep& decode,
+                                                 const PrefillGeometry& geometry,
+                                                 std::uint32_t positions) noexcept;
+// Segment `segment_index` of the payload, in payload order; allocates nothing.
+PrefixStateSegmentResult prefix_state_segment(const PrefixStateLayout& layout,
+                                              std::uint32_t segment_index) noexcept;
+PrefixStateCopyRoute prefix_state_copy_route(const PrefixStateSegment& segment,
+                                             PrefixStateTransferDirection direction,
+                                             bool gated_delta_swapped) noexcept;
+
+enum class PrefixStateTransferError : std::uint8_t {
+    None,
+    InvalidLayout,
+    InvalidStateSlot,
+    StateSlotNotReady,
+    InvalidArena,
+    ArenaOutOfRange,
+    GenerationExhausted,
+    PhaseEvidenceTooSmall,
+    CommandEncodingFailed,
+    StaleTicket,
+    AlreadyCompleted,
+    PoisonedStateSlot,
+};
+
+PrefixStateTransferError validate_prefix_state_arena_extent(const PrefixStateLayout& layout,
+                                                            std::uint64_t arena_offset_bytes,
+                                                            std::uint64_t arena_capacity_bytes) noexcept;
+// One bit per schedule entry, set for a gated-delta layer whose live planes were
+// the out planes when the snapshot was taken.
+std::size_t prefix_state_phase_evidence_bytes(std::span<const LayerKind> schedule) noexcept;
+PrefixStateTransferError capture_prefix_state_phase_evidence(const DecodeStep& decode,
+                                                             const DecodeStateSlot& state,
+                                                             std::span<std::byte> phase_evidence) noexcept;
+
+struct PrefixStateTransferTicket {
+    PrefixStateTransferDirection direction{PrefixStateTransferDirection::Snapshot};
+    const DecodeStep* owner{nullptr};
+    DecodeStateSlot* state_owner{nullptr};
+    const HipBuffer* arena_owner{nullptr};
+    std::uint32_t positions{0};
+    std::uint64_t arena_offset_bytes{0};
+    std::uint64_t state_bytes{0};
+    std::uint64_t generation{0};
+    bool pending{false};
+};
+struct PrefixStateTransferResult {
+    PrefixStateTransferError error{PrefixStateTransferError::InvalidLayout};
+    PrefixStateLayoutError layout_error{PrefixStateLayoutError::None};
+    HipCommandError command_error{HipCommandError::None};
+    std::uint32_t segment_count{0};
+    std::uint64_t state_bytes{0};
+    std::size_t source_phase_evidence_bytes{0};
+    std::optional<PrefixStateTransferTicket> ticket;
+    explicit operator bool() const noexcept {
+        return error == PrefixStateTransferError::None && ticket.has_value();
+    }
+};
+
+// Both encode device-to-device copies on the blit pass's queue and leave the slot
+// SnapshotPending / RestorePending until the ticket is completed after the
+// command buffer finished.  A copy that fails to encode poisons the slot.
+PrefixStateTransferResult encode_prefix_state_snapshot(const DecodeStep& decode,
+                                                       DecodeStateSlot& state,
+                                                       const PrefillGeometry& geometry,
+                                                       HipBlitPass& blit_pass, HipBuffer& state_arena,
+                                                       std::uint64_t arena_offset_bytes,
+                                                       std::uint32_t positions,
+                                                       std::span<std::byte> source_phase_evidence) noexcept;
+PrefixStateTransferResult encode_prefix_state_restore(const DecodeStep& decode, DecodeStateSlot& state,
+                                                      const PrefillGeometry& geometry,
+                                                      HipBlitPass& blit_pass, HipBuffer& state_arena,
+                                                      std::uint64_t arena_offset_bytes,
+                                                      std::uint32_t positions) noexcept;
+PrefixStateTransferError complete_prefix_state_transfer(PrefixStateTransferTicket& ticket,
+                                                        const DecodeStep& decode,
+                                                        DecodeStateSlot& state,
+                                                        const HipBuffer& state_arena) noexcept;
+PrefixStateTransferError abort_prefix_state_transfer(PrefixStateTransferTicket& ticket,
+                                                     const DecodeStep& decode, DecodeStateSlot& state,
+                                                     const HipBuffer& state_arena) noexcept;
 
 }  // namespace tatara::runtime

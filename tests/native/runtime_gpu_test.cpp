@@ -4,6 +4,7 @@
 // reset.  Returns a distinct non-zero code per failed check and prints the
 // error figures it accepts (max-abs <= 2e-2, mean-abs <= 2e-3 on bf16 outputs;
 // cache/state slot placement exact).
+#include <array>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -268,7 +269,7 @@ int main() {
     auto slot_made = create_decode_state_slot(*device.device, step);
     if (!slot_made) return 50;
     DecodeStateSlot& slot = *slot_made.slot;
-    std::vector<std::uint16_t> final_values;
+    std::vector<std::uint16_t> final_values, conv0_final;
     for (const bool chunked : {false, true}) {
     if (chunked) {  // fresh planes for the second pass
         auto again = create_decode_state_slot(*device.device, step);
@@ -347,6 +348,203 @@ int main() {
     if (slot.layers[0].swapped) return 75;
     if (download<std::uint16_t>(slot.layers[0].first, 3 * 8192) != conv0) return 76;
     final_values = values;
+    conv0_final = conv0;
+    }
+
+    // ---- lane state record (Q36BRS01): write, install into a fresh slot, round trip --
+    {
+        std::printf("[case] lane state record\n");
+        const std::uint32_t positions = 100;
+        // a second gated-delta layer whose live planes are the out planes
+        const auto marker_conv = gauss16(9100, 3 * 8192, 0.5);
+        std::vector<float> marker_rec(32 * 128 * 128);
+        for (std::size_t i = 0; i < marker_rec.size(); ++i) marker_rec[i] = 1e-3f * float(i % 977);
+        if (!upload(slot.layers[1].first_out, marker_conv)) return 100;
+        if (tt_buffer_write(slot.layers[1].second_out.native(), 0, marker_rec.data(),
+                            marker_rec.size() * 4) != TT_OK) {
+            return 100;
+        }
+        slot.layers[1].swapped = true;
+        std::vector<std::byte> record;
+        if (write_state_record(step, slot, positions, record) != StateRecordError::None) return 101;
+        const std::uint64_t gdn_bytes = 3 * 8192 * 2 + 32ull * 128 * 128 * 4;
+        const std::uint64_t expect = 12 + 3 * gdn_bytes + 4ull * positions * 512;
+        if (record.size() != expect || state_record_bytes(step, positions) != expect) return 102;
+        if (state_record_bytes(step, 0) != 0 || state_record_bytes(step, kCapacity + 1) != 0) return 103;
+        std::uint32_t stored = 0;
+        std::memcpy(&stored, record.data() + 8, 4);
+        if (std::memcmp(record.data(), "Q36BRS01", 8) != 0 || stored != positions) return 104;
+        // layer 0: the in planes are live; layer 1: the out planes
+        if (std::memcmp(record.data() + 12, conv0_final.data(), 3 * 8192 * 2) != 0) return 105;
+        if (std::memcmp(record.data() + 12 + gdn_bytes, marker_conv.data(), 3 * 8192 * 2) != 0) return 106;
+        if (std::memcmp(record.data() + 12 + gdn_bytes + 3 * 8192 * 2, marker_rec.data(),
+                        marker_rec.size() * 4) != 0) {
+            return 107;
+        }
+        // attention layer 3: keys head 0, keys head 1, values head 0, values head 1, packed
+        const std::byte* values0 = record.data() + 12 + 3 * gdn_bytes + 2ull * positions * 512;
+        if (std::memcmp(values0, final_values.data(), positions * 512) != 0) return 108;
+        if (std::memcmp(values0 + positions * 512, final_values.data() + std::size_t{kCapacity} * 256,
+                        positions * 512) != 0) {
+            return 109;
+        }
+
+        auto fresh_made = create_decode_state_slot(*device.device, step);
+        if (!fresh_made) return 110;
+        DecodeStateSlot& fresh = *fresh_made.slot;
+        std::uint32_t context = 0;
+        if (load_state_record(record, step, fresh, context) != StateRecordError::None) return 111;
+        if (context != positions) return 112;
+        if (download<std::uint16_t>(fresh.layers[0].first, 3 * 8192) != conv0_final) return 113;
+        if (download<std::uint16_t>(fresh.layers[1].first, 3 * 8192) != marker_conv) return 114;
+        if (fresh.layers[1].swapped) return 115;
+        if (download<float>(fresh.layers[1].second, marker_rec.size()) != marker_rec) return 116;
+        const auto loaded_values = download<std::uint16_t>(fresh.layers[3].second, final_values.size());
+        for (std::size_t head = 0; head < 2; ++head) {
+            for (std::size_t i = 0; i < std::size_t{kCapacity} * 256; ++i) {
+                const std::size_t at = head * kCapacity * 256 + i;
+                const std::uint16_t want = i < positions * 256 ? final_values[at] : 0;
+                if (loaded_values[at] != want) return 117;
+            }
+        }
+        std::vector<std::byte> again;
+        if (write_state_record(step, fresh, positions, again) != StateRecordError::None) return 118;
+        if (again != record) return 119;
+
+        // malformed records leave the slot untouched and name the defect
+        auto other_made = create_decode_state_slot(*device.device, step);
+        if (!other_made) return 120;
+        DecodeStateSlot& other = *other_made.slot;
+        std::vector<std::byte> bad = record;
+        bad[0] = std::byte{'X'};
+        if (load_state_record(bad, step, other, context) != StateRecordError::MagicMismatch) return 121;
+        bad = record;
+        bad.pop_back();
+        if (load_state_record(bad, step, other, context) != StateRecordError::Truncated) return 122;
+        bad = record;
+        bad.push_back(std::byte{0});
+        if (load_state_record(bad, step, other, context) != StateRecordError::TrailingBytes) return 123;
+        bad = record;
+        const std::uint32_t zero = 0, beyond = kCapacity + 1;
+        std::memcpy(bad.data() + 8, &zero, 4);
+        if (load_state_record(bad, step, other, context) != StateRecordError::InvalidPositions) return 124;
+        std::memcpy(bad.data() + 8, &beyond, 4);
+        if (load_state_record(bad, step, other, context) != StateRecordError::InvalidPositions) return 125;
+        if (load_state_record(std::span<const std::byte>(record.data(), 5), step, other, context) !=
+            StateRecordError::Truncated) {
+            return 126;
+        }
+        if (write_state_record(step, slot, 0, again) != StateRecordError::InvalidPositions) return 127;
+        for (const float v : download<float>(other.layers[0].second, 64)) {
+            if (v != 0.0f) return 128;
+        }
+
+        // ---- the same state as a device-resident prefix payload --------------------
+        std::printf("[case] prefix snapshot / restore\n");
+        const PrefillPolicy policy{.schedule = PrefillSchedule::ChunkMajor,
+                                   .context_capacity = kCapacity,
+                                   .maximum_block_rows = 64,
+                                   .first_chunk_rows = 64,
+                                   .query_tile_rows = 64,
+                                   .attention_partition = 256,
+                                   .gdn_gate_hoist = true,
+                                   .gdn_chunked = true};
+        const auto pg = make_prefill_geometry(plan, policy);
+        if (!pg) return 130;
+        const auto made = make_prefix_state_layout(step, pg.geometry, positions);
+        if (!made || made.layout.segment_count != 3 * 2 + 4 ||
+            made.layout.total_bytes != expect - 12) {
+            return 130;
+        }
+        const std::uint64_t arena_base = 256;
+        auto arena_made = tatara::backend::hip::create_shared_buffer(
+            *device.device, arena_base + made.layout.total_bytes + 64);
+        if (!arena_made) return 131;
+        HipBuffer& arena = *arena_made.buffer;
+        std::vector<std::uint8_t> guard(arena.size_bytes(), 0xa5);
+        if (tt_buffer_write(arena.native(), 0, guard.data(), guard.size()) != TT_OK) return 131;
+        std::array<std::byte, 1> evidence{};
+        {
+            auto cb = create_command_buffer(*queue.command_queue);
+            if (!cb) return 132;
+            auto blit = begin_blit_pass(std::move(*cb.command_buffer));
+            if (!blit) return 132;
+            // one byte short of the payload is refused before any copy
+            if (encode_prefix_state_snapshot(step, slot, pg.geometry, *blit.blit_pass, arena,
+                                             arena_base + 65, positions, evidence)
+                        .error != PrefixStateTransferError::ArenaOutOfRange ||
+                slot.status != DecodeStateSlotStatus::Ready) {
+                return 133;
+            }
+            PrefixStateTransferResult taken = encode_prefix_state_snapshot(
+                step, slot, pg.geometry, *blit.blit_pass, arena, arena_base, positions, evidence);
+            if (!taken || taken.segment_count != 10 || taken.state_bytes != made.layout.total_bytes ||
+                taken.source_phase_evidence_bytes != 1 || evidence[0] != std::byte{0b010}) {
+                return 134;
+            }
+            if (slot.status != DecodeStateSlotStatus::SnapshotPending ||
+                decode_state_slot_ready(step, slot)) {
+                return 135;
+            }
+            auto ended = end_blit_pass(std::move(*blit.blit_pass));
+            auto pending = commit(std::move(*ended.command_buffer));
+            if (!pending || !wait_until_completed(std::move(*pending.pending_execution))) return 136;
+            if (complete_prefix_state_transfer(*taken.ticket, step, slot, arena) !=
+                    PrefixStateTransferError::None ||
+                slot.status != DecodeStateSlotStatus::Ready || !slot.layers[1].swapped) {
+                return 137;
+            }
+        }
+        // payload == the record's pieces, family-major; the guard bytes either side survive
+        const auto image = download<std::uint8_t>(arena, arena.size_bytes());
+        for (std::size_t i = 0; i < arena_base; ++i) {
+            if (image[i] != 0xa5) return 138;
+        }
+        for (std::size_t i = arena_base + made.layout.total_bytes; i < image.size(); ++i) {
+            if (image[i] != 0xa5) return 138;
+        }
+        // schedule is G G G A, so the record body and the payload coincide byte for byte
+        if (std::memcmp(image.data() + arena_base, record.data() + 12, made.layout.total_bytes) != 0) {
+            return 139;
+        }
+        {
+            auto target_made = create_decode_state_slot(*device.device, step);
+            if (!target_made) return 140;
+            DecodeStateSlot& target = *target_made.slot;
+            target.layers[0].swapped = true;  // the recipient's own phase does not matter
+            auto cb = create_command_buffer(*queue.command_queue);
+            if (!cb) return 141;
+            auto blit = begin_blit_pass(std::move(*cb.command_buffer));
+            if (!blit) return 141;
+            PrefixStateTransferResult put = encode_prefix_state_restore(
+                step, target, pg.geometry, *blit.blit_pass, arena, arena_base, positions);
+            if (!put || target.status != DecodeStateSlotStatus::RestorePending) return 142;
+            // a lane with a transfer in flight admits no second one
+            if (encode_prefix_state_restore(step, target, pg.geometry, *blit.blit_pass, arena,
+                                            arena_base, positions)
+                    .error != PrefixStateTransferError::StateSlotNotReady) {
+                return 143;
+            }
+            auto ended = end_blit_pass(std::move(*blit.blit_pass));
+            auto pending = commit(std::move(*ended.command_buffer));
+            if (!pending || !wait_until_completed(std::move(*pending.pending_execution))) return 144;
+            if (complete_prefix_state_transfer(*put.ticket, step, target, arena) !=
+                    PrefixStateTransferError::None ||
+                target.layers[0].swapped || target.layers[1].swapped) {
+                return 145;
+            }
+            std::vector<std::byte> from_target;
+            if (write_state_record(step, target, positions, from_target) != StateRecordError::None ||
+                from_target != record) {
+                return 146;
+            }
+            // rows past the prefix were not touched
+            const auto target_keys = download<std::uint16_t>(target.layers[3].first, 2 * kCapacity * 256);
+            for (std::size_t i = positions * 256; i < std::size_t{kCapacity} * 256; ++i) {
+                if (target_keys[i] != 0) return 147;
+            }
+        }
+        slot.layers[1].swapped = false;
     }
 
     // ---- lane reset -----------------------------------------------------------

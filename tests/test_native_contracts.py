@@ -19,7 +19,7 @@ def _binary(name):
 
 
 @pytest.mark.parametrize("name", ["geometry_contract_test", "state_slot_contract_test",
-                                  "backend_contract_test"])
+                                  "backend_contract_test", "prefix_state_contract_test"])
 def test_host_contract(name):
     result = subprocess.run([_binary(name)], capture_output=True, text=True, timeout=120)
     assert result.returncode == 0, f"{name} failed check {result.returncode}\n{result.stdout}"
