@@ -336,7 +336,8 @@ void normalize_qk_heads(const uint16_t* activated, uint16_t* qk) {
 
 // delta-rule update of one (value head, value dim) state row
 inline uint16_t recurrence_row(const float* row_in, float* row_out, const uint16_t* q,
-                               const uint16_t* k, float v, float decay, float beta) {
+                               const uint16_t* k, float v, float decay, float beta,
+                               float* delta_out = nullptr) {
     float st[kGD];
     float part[32];
     for (uint32_t l = 0; l < 32; ++l) {
@@ -350,6 +351,7 @@ inline uint16_t recurrence_row(const float* row_in, float* row_out, const uint16
     }
     const float key_value = adjacent32(part);
     const float delta = fz32(fz32(v - key_value) * beta);
+    if (delta_out) *delta_out = delta;
     for (uint32_t l = 0; l < 32; ++l) {
         float o = 0.0f;
         for (uint32_t i = 0; i < 4; ++i) {
@@ -633,6 +635,84 @@ void tto_gdn_scan(const uint16_t* qk, const uint16_t* value, const float* decay,
         }
         std::memcpy(state_out + static_cast<size_t>(h) * kGD * kGD, st.data(),
                     st.size() * sizeof(float));
+    });
+}
+
+void tto_gdn_conv_tape(const uint16_t* projection, uint32_t rows, const uint16_t* conv_state,
+                       uint16_t* conv_tape, uint32_t tape_layer) {
+    if (rows > TTO_GDN_TAPE_ROWS) return;
+    const size_t P = TTO_GDN_PROJECTION_ROWS;
+    for (uint32_t r = 0; r < rows; ++r) {
+        uint16_t* window =
+            conv_tape + (static_cast<size_t>(tape_layer) * TTO_GDN_TAPE_ROWS + r) * 3 * kCh;
+        for (uint32_t tap = 0; tap < 3; ++tap) {
+            const uint32_t logical = r + tap + 1;  // taps 1..3 of row r
+            for (uint32_t c = 0; c < kCh; ++c) {
+                window[tap * kCh + c] = logical < 3 ? conv_state[logical * kCh + c]
+                                                    : projection[(logical - 3) * P + c];
+            }
+        }
+    }
+}
+
+void tto_gdn_scan_tape(const uint16_t* qk, const uint16_t* value, const float* decay,
+                       const float* beta, uint32_t steps, const float* state_in, uint16_t* y,
+                       float* state_out, float* tape, uint32_t tape_layer, uint32_t threads) {
+    const bool taped = steps <= TTO_GDN_TAPE_ROWS;
+    parallel_for(kVH, threads, [=](uint32_t h) {
+        const uint32_t kh = h >> 1;
+        std::vector<float> st(static_cast<size_t>(kGD) * kGD);
+        std::memcpy(st.data(), state_in + static_cast<size_t>(h) * kGD * kGD,
+                    st.size() * sizeof(float));
+        for (uint32_t t = 0; t < steps; ++t) {
+            const uint16_t* q = qk + static_cast<size_t>(t) * TTO_GDN_QK_VALUES + kh * kGD;
+            const uint16_t* k = q + TTO_GDN_K_OFFSET;
+            const uint16_t* v = value + static_cast<size_t>(t) * TTO_GDN_VALUE_VALUES + h * kGD;
+            uint16_t* yo = y + static_cast<size_t>(t) * TTO_GDN_VALUE_VALUES + h * kGD;
+            const size_t tape_row = static_cast<size_t>(tape_layer) * TTO_GDN_TAPE_ROWS + t;
+            for (uint32_t j = 0; j < kGD; ++j) {
+                float* row = st.data() + static_cast<size_t>(j) * kGD;
+                float delta = 0.0f;
+                yo[j] = recurrence_row(row, row, q, k, widen(v[j]), decay[t * kVH + h],
+                                       beta[t * kVH + h], &delta);
+                if (taped) tape[(tape_row * kVH + h) * kGD + j] = delta;
+            }
+            if (!taped) continue;
+            if ((h & 1) == 0) {
+                float* keys = tape + TTO_GDN_TAPE_KEY_OFFSET +
+                              (tape_row * TTO_GDN_KEY_HEADS + kh) * kGD;
+                for (uint32_t e = 0; e < kGD; ++e) keys[e] = widen(k[e]);
+            }
+            float* gates = tape + TTO_GDN_TAPE_GATE_OFFSET + (tape_row * kVH + h) * 2;
+            gates[0] = decay[t * kVH + h];
+            gates[1] = beta[t * kVH + h];
+        }
+        std::memcpy(state_out + static_cast<size_t>(h) * kGD * kGD, st.data(),
+                    st.size() * sizeof(float));
+    });
+}
+
+void tto_gdn_tape_replay(const float* tape, const float* state_in, float* state_out,
+                         uint32_t steps, uint32_t tape_layer, uint32_t threads) {
+    parallel_for(kVH, threads, [=](uint32_t h) {
+        const uint32_t kh = h >> 1;
+        for (uint32_t j = 0; j < kGD; ++j) {
+            const size_t base = (static_cast<size_t>(h) * kGD + j) * kGD;
+            float st[kGD];
+            std::memcpy(st, state_in + base, sizeof(st));
+            for (uint32_t t = 0; t < steps; ++t) {
+                const size_t tape_row = static_cast<size_t>(tape_layer) * TTO_GDN_TAPE_ROWS + t;
+                const float step_decay = tape[TTO_GDN_TAPE_GATE_OFFSET + (tape_row * kVH + h) * 2];
+                const float delta = tape[(tape_row * kVH + h) * kGD + j];
+                const float* keys =
+                    tape + TTO_GDN_TAPE_KEY_OFFSET + (tape_row * TTO_GDN_KEY_HEADS + kh) * kGD;
+                for (uint32_t e = 0; e < kGD; ++e) {
+                    st[e] = fz32(st[e] * step_decay);
+                    st[e] = std::fma(keys[e], delta, st[e]);
+                }
+            }
+            std::memcpy(state_out + base, st, sizeof(st));
+        }
     });
 }
 

@@ -29,6 +29,13 @@
  *     against an fp64 textbook evaluation.
  *   - tto_gdn_chunked_f64: brute-force equality with the sequential fp64
  *     recurrence on small shapes.
+ *   - tto_gdn_conv_tape / tto_gdn_scan_tape / tto_gdn_tape_replay: the
+ *     reference holds no test or fixture for the tape; pinned by what the
+ *     definition fixes: replaying c rows equals, bit for bit, the state the
+ *     pinned tto_gdn_scan stores after exactly c rows (every c in 0..16), the
+ *     taped scan equals the plain scan, tape rows equal the scan's operands,
+ *     one step from a zero state tapes delta = v * beta, and conv tape row c-1
+ *     equals the conv state tto_gdn_prefill commits after c rows.
  */
 #pragma once
 
@@ -60,7 +67,14 @@ enum {
     TTO_GDN_B_OFFSET = 12288,
     TTO_GDN_A_OFFSET = 12320,
     TTO_GDN_PROJECTION_ROWS = 12352,
-    TTO_GDN_CONV_WIDTH = 4
+    TTO_GDN_CONV_WIDTH = 4,
+    /* rollback tape (tools/generate_kernel_library.py:2045-2049) */
+    TTO_GDN_TAPE_ROWS = 16,
+    TTO_GDN_TAPE_LAYERS = 40,
+    TTO_GDN_TAPE_KEY_OFFSET = 40 * 16 * 32 * 128,
+    TTO_GDN_TAPE_GATE_OFFSET = 40 * 16 * 32 * 128 + 40 * 16 * 16 * 128,
+    TTO_GDN_TAPE_FLOATS = 40 * 16 * (32 * 128 + 16 * 128 + 64),
+    TTO_GDN_CONV_TAPE_VALUES = 40 * 16 * 3 * 8192
 };
 
 /* ---- numeric primitives (kernel_reference.cpp:77-103) ---- */
@@ -189,6 +203,29 @@ void tto_gdn_prefill(const uint16_t* projection, uint32_t rows, const uint16_t* 
 void tto_gdn_scan(const uint16_t* qk, const uint16_t* value, const float* decay,
                   const float* beta, uint32_t steps, const float* state_in, uint16_t* y,
                   float* state_out, uint32_t threads);
+
+/* Rollback tape of a block of at most 16 rows and its replay
+ * (prefill_gdn.metal:322-400, 432-511, 520-569).
+ * tto_gdn_conv_tape: conv_tape[layer][row][tap][8192] = the conv window as it
+ * stands after `row` (taps 1..3 of that row); rows > 16 writes nothing.
+ * tto_gdn_scan_tape: tto_gdn_scan that also records, per step, delta[32][128],
+ * the keys widened to fp32 [16][128] and {decay, beta}[32] into the three
+ * regions of `tape` (TTO_GDN_TAPE_* offsets, in floats); steps > 16 records
+ * nothing.
+ * tto_gdn_tape_replay: state_out = state_in advanced by the first `steps` taped
+ * rows with the scan's own two update statements (state *= decay;
+ * state = fma(key, delta, state)).
+ * Parity pins (no reference test covers the tape): replay(steps = c) equals the
+ * state tto_gdn_scan stores after exactly c rows, bit for bit, for every c; the
+ * conv tape row c-1 equals the new_conv_state of tto_gdn_prefill over c rows;
+ * from a zero state one step tapes delta = v * beta exactly. */
+void tto_gdn_conv_tape(const uint16_t* projection, uint32_t rows, const uint16_t* conv_state,
+                       uint16_t* conv_tape, uint32_t tape_layer);
+void tto_gdn_scan_tape(const uint16_t* qk, const uint16_t* value, const float* decay,
+                       const float* beta, uint32_t steps, const float* state_in, uint16_t* y,
+                       float* state_out, float* tape, uint32_t tape_layer, uint32_t threads);
+void tto_gdn_tape_replay(const float* tape, const float* state_in, float* state_out,
+                         uint32_t steps, uint32_t tape_layer, uint32_t threads);
 
 /* The steps either side of the path in a stacked run.
  * tto_rms_only: row RMS norm with the double rounding bf16(w * bf16(x * inv))

@@ -84,6 +84,8 @@ struct PrepareArgs {
     uint32_t projection_stride, qk_stride, value_stride, z_stride;
     uint32_t block_mode;          // 1: rows are consecutive tokens of one lane
     uint32_t rows;
+    uint16_t* conv_tape;          // [40][16][3][8192] window after each row, or null
+    uint32_t tape_layer;
 };
 
 constexpr uint32_t kBlockRowsPerGroup = 16;  // block mode: rows one workgroup walks
@@ -231,6 +233,15 @@ __global__ __launch_bounds__(256) void gdn_prepare_block_kernel(PrepareArgs a) {
             *reinterpret_cast<u32x4*>(a.conv_out + kCh + c) = t2;
             *reinterpret_cast<u32x4*>(a.conv_out + 2 * kCh + c) = t3;
         }
+        // what conv_out would hold had the block ended at this row
+        // (prefill_gdn.metal:376-386): a block no longer than the tape records it
+        if (a.conv_tape != nullptr && a.rows <= kGdnTapeRows) {
+            uint16_t* tape =
+                a.conv_tape + (static_cast<uint64_t>(a.tape_layer) * kGdnTapeRows + row) * 3 * kCh + c;
+            *reinterpret_cast<u32x4*>(tape) = t1;
+            *reinterpret_cast<u32x4*>(tape + kCh) = t2;
+            *reinterpret_cast<u32x4*>(tape + 2 * kCh) = t3;
+        }
         u32x4 packed;
         if (normalised) {
             const float run0 = ((act[0] * act[0] + act[1] * act[1]) + act[2] * act[2]) + act[3] * act[3];
@@ -272,12 +283,19 @@ struct RecurrenceArgs {
     const uint32_t* table;       // per row {.., .., rec_in, rec_out} element offsets
     uint32_t qk_stride, value_stride, projection_stride, y_stride;
     uint32_t steps;              // tokens walked per state row (1 for decode)
+    float* tape;                 // rollback tape (kTape instantiation only)
+    uint32_t tape_layer;
 };
 
 // One half wave per state row; a 256-thread workgroup covers 8 rows of one
 // (row-of-batch, value head).  grid (16, 32, rows).  The token loop serves the
 // block-prefill register scan: state stays in registers across steps
 // (prefill_gdn.metal:204-281).
+//
+// kTape (prefill_gdn.metal:432-511): a block of at most 16 steps also records, per
+// step, what a later replay needs to rebuild the state up to any row: the delta of
+// every state row, the keys as fp32, and {decay, beta} per value head.
+template <bool kTape>
 __global__ __launch_bounds__(256) void gdn_recurrence_kernel(RecurrenceArgs a) {
     const uint32_t half = threadIdx.x >> 5;              // 0..7
     const uint32_t lane = threadIdx.x & 31;
@@ -325,6 +343,24 @@ __global__ __launch_bounds__(256) void gdn_recurrence_kernel(RecurrenceArgs a) {
         const float v = widen(a.value[row_v + static_cast<uint64_t>(step) * a.value_stride +
                                       h * kGD + j]);
         const float delta = (v - kv) * beta;
+        if constexpr (kTape) {
+            if (a.steps <= kGdnTapeRows) {
+                const uint64_t tape_row = static_cast<uint64_t>(a.tape_layer) * kGdnTapeRows + step;
+                if (lane == 0) a.tape[(tape_row * kGdnValueHeads + h) * kGD + j] = delta;
+                if (j == 0) {
+                    if ((h & 1) == 0) {
+                        *reinterpret_cast<f32x4*>(a.tape + kGdnTapeKeyOffset +
+                                                  (tape_row * kGdnKeyHeads + kh) * kGD + lane * 4) =
+                            f32x4{k4[0], k4[1], k4[2], k4[3]};
+                    }
+                    if (lane == 0) {
+                        float* gates = a.tape + kGdnTapeGateOffset + (tape_row * kGdnValueHeads + h) * 2;
+                        gates[0] = decay;
+                        gates[1] = beta;
+                    }
+                }
+            }
+        }
         float out = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
@@ -334,6 +370,37 @@ __global__ __launch_bounds__(256) void gdn_recurrence_kernel(RecurrenceArgs a) {
         out = half_wave_sum(out);
         if (lane == 0) {
             a.y[row_y + static_cast<uint64_t>(step) * a.y_stride + h * kGD + j] = narrow(out);
+        }
+    }
+    *reinterpret_cast<f32x4*>(state_out + base) = st;
+}
+
+// gdn_tape_replay_blk (prefill_gdn.metal:520-569): the state after `steps` rows of
+// a taped block, rebuilt from the state before the block.  The two update
+// statements are the forward scan's own, so the result equals, bit for bit, what a
+// forward scan of exactly `steps` rows would have stored.  Same state-row mapping as
+// the forward kernel: grid (16, 32) x 256.
+__global__ __launch_bounds__(256) void gdn_tape_replay_kernel(const float* tape,
+                                                              const float* state_in,
+                                                              float* state_out, uint32_t steps,
+                                                              uint32_t tape_layer) {
+    const uint32_t half = threadIdx.x >> 5;
+    const uint32_t lane = threadIdx.x & 31;
+    const uint32_t j = blockIdx.x * 8 + half;
+    const uint32_t h = blockIdx.y;
+    const uint32_t kh = h >> 1;
+    const uint64_t base = (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4;
+    f32x4 st = *reinterpret_cast<const f32x4*>(state_in + base);
+    for (uint32_t step = 0; step < steps; ++step) {
+        const uint64_t tape_row = static_cast<uint64_t>(tape_layer) * kGdnTapeRows + step;
+        const float decay = tape[kGdnTapeGateOffset + (tape_row * kGdnValueHeads + h) * 2];
+        const float delta = tape[(tape_row * kGdnValueHeads + h) * kGD + j];
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(
+            tape + kGdnTapeKeyOffset + (tape_row * kGdnKeyHeads + kh) * kGD + lane * 4);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            st[i] *= decay;
+            st[i] = fmaf(k4[i], delta, st[i]);
         }
     }
     *reinterpret_cast<f32x4*>(state_out + base) = st;
@@ -1328,10 +1395,16 @@ int32_t op_gdn_prepare_ms(const Bindings& b, const Grid& g, hipStream_t stream,
 // gdn_conv_blk: b0 projection[rows][12352], b1 conv_in, b2 conv_w, b3 qk[rows][4096],
 // b4 value, b5 gate, b6 conv_out, c7 rows; grid (96, rows) x 128
 // (prefill_step.cpp:1934-1955).
-int32_t op_gdn_conv_blk(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only) {
+int32_t conv_blk_common(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only,
+                        bool taped) {
     Args a(b);
     PrepareArgs p{};
     p.rows = a.constant(7);
+    if (taped) {
+        p.conv_tape = a.buffer<uint16_t>(8, static_cast<uint64_t>(kGdnConvTapeElements) * 2);
+        p.tape_layer = a.constant(9);
+        a.require(p.tape_layer < kLayers, TT_CMD_INVALID_BUFFER);
+    }
     a.require(p.rows >= 1 && g.gx == 96 && g.gy == p.rows && g.gz == 1 && g.tx == 128 &&
                   g.ty == 1 && g.tz == 1,
               TT_CMD_INVALID_DISPATCH_EXTENT);
@@ -1350,10 +1423,24 @@ int32_t op_gdn_conv_blk(const Bindings& b, const Grid& g, hipStream_t stream, bo
     if (a.status != TT_OK || validate_only) return a.status;
     return launch_prepare(p, stream);
 }
+int32_t op_gdn_conv_blk(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only) {
+    return conv_blk_common(b, g, stream, validate_only, false);
+}
+// gdn_conv_tape_blk: gdn_conv_blk + b8 conv tape [40][16][3][8192] bf16, c9 layer; a
+// block of more than 16 rows leaves the tape untouched (prefill_step.cpp:1931-1947).
+int32_t op_gdn_conv_tape_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                             bool validate_only) {
+    return conv_blk_common(b, g, stream, validate_only, true);
+}
 
 int32_t launch_recurrence(const RecurrenceArgs& r, uint32_t rows, hipStream_t stream) {
-    hipLaunchKernelGGL(gdn_recurrence_kernel, dim3(kGD / 8, kGdnValueHeads, rows), dim3(256), 0,
-                       stream, r);
+    if (r.tape != nullptr) {
+        hipLaunchKernelGGL(gdn_recurrence_kernel<true>, dim3(kGD / 8, kGdnValueHeads, rows),
+                           dim3(256), 0, stream, r);
+        return TT_OK;
+    }
+    hipLaunchKernelGGL(gdn_recurrence_kernel<false>, dim3(kGD / 8, kGdnValueHeads, rows), dim3(256),
+                       0, stream, r);
     return TT_OK;
 }
 
@@ -1486,10 +1573,15 @@ int32_t op_gdn_gates_blk(const Bindings& b, const Grid& g, hipStream_t stream,
 // gdn_recurrence_blk: b2 projection, b3 a_log, b4 dt_bias instead.
 // grid (1,32,32) x (32,4,1) (prefill_step.cpp:2003-2036).
 int32_t op_gdn_scan(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only,
-                    bool hoisted_gates) {
+                    bool hoisted_gates, bool taped = false) {
     Args a(b);
     RecurrenceArgs r{};
     r.steps = a.constant(8);
+    if (taped) {
+        r.tape = a.buffer<float>(9, static_cast<uint64_t>(kGdnTapeFloats) * 4);
+        r.tape_layer = a.constant(10);
+        a.require(r.tape_layer < kLayers, TT_CMD_INVALID_BUFFER);
+    }
     a.require(r.steps >= 1, TT_CMD_INVALID_BUFFER);
     const uint64_t steps = r.steps;
     r.qk = a.buffer<const uint16_t>(0, steps * kGdnQkValues * 2);
@@ -1519,6 +1611,30 @@ int32_t op_gdn_recurrence_gates_blk(const Bindings& b, const Grid& g, hipStream_
 int32_t op_gdn_recurrence_blk(const Bindings& b, const Grid& g, hipStream_t stream,
                               bool validate_only) {
     return op_gdn_scan(b, g, stream, validate_only, false);
+}
+// gdn_recurrence_gates_tape_blk: gdn_recurrence_gates_blk + b9 tape (fp32, three
+// regions), c10 layer; more than 16 steps leave the tape untouched
+// (prefill_step.cpp:2003-2028).
+int32_t op_gdn_recurrence_gates_tape_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                                         bool validate_only) {
+    return op_gdn_scan(b, g, stream, validate_only, true, true);
+}
+// gdn_tape_replay_blk: b0 tape, b1 state_in, b2 state_out, c3 steps (0..16), c4 layer;
+// grid (1,32,32) x (32,4,1) (speculative_decode.cpp:546-556).
+int32_t op_gdn_tape_replay_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                               bool validate_only) {
+    Args a(b);
+    const float* tape = a.buffer<const float>(0, static_cast<uint64_t>(kGdnTapeFloats) * 4);
+    const float* state_in = a.buffer<const float>(1, kStateBytes);
+    float* state_out = a.buffer<float>(2, kStateBytes);
+    const uint32_t steps = a.constant(3);
+    const uint32_t layer = a.constant(4);
+    a.require(steps <= kGdnTapeRows && layer < kLayers, TT_CMD_INVALID_BUFFER);
+    a.require(grid_is(g, 1, 32, 32, 32, 4, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(gdn_tape_replay_kernel, dim3(kGD / 8, kGdnValueHeads), dim3(256), 0, stream,
+                       tape, state_in, state_out, steps, layer);
+    return TT_OK;
 }
 
 int32_t gate_norm_common(Args& a, const Grid& g, uint32_t rows, uint32_t stride,
@@ -1690,6 +1806,9 @@ const KernelDesc kGdnPrefillKernels[] = {
     {"gdn_recurrence_gates_blk", op_gdn_recurrence_gates_blk},
     {"gdn_recurrence_blk", op_gdn_recurrence_blk},
     {"gdn_gate_norm_blk", op_gdn_gate_norm_blk},
+    {"gdn_conv_tape_blk", op_gdn_conv_tape_blk},
+    {"gdn_recurrence_gates_tape_blk", op_gdn_recurrence_gates_tape_blk},
+    {"gdn_tape_replay_blk", op_gdn_tape_replay_blk},
     {"gdn_chunk_prepare_blk", op_gdn_chunk_prepare},
     {"gdn_chunk_scan_blk", op_gdn_chunk_scan},
     {"gdn_chunk_recurrence_blk", op_gdn_chunk_recurrence},

@@ -41,8 +41,23 @@ constexpr uint16_t kGdnQueryScaleBits = 0x3C00;  // bf16(1/128)
 constexpr uint16_t kGdnKeyScaleBits = 0x3DB5;    // bf16(1/sqrt(128)) = 0.08837890625
 constexpr float kRmsNormEpsilon = 1.0e-6f;
 
+// Rollback tape of a short verified block (tools/generate_kernel_library.py:2045-2049):
+// per layer and block row the 32x128 delta values, then the 16x128 keys, then
+// {decay, beta} per value head, each region sized for all 40 layers; the conv tape
+// holds the conv window as it stands after each row.
+constexpr uint32_t kGdnTapeRows = 16;
+constexpr uint32_t kGdnTapeKeyOffset = kLayers * kGdnTapeRows * kGdnValueHeads * kGdnHeadDim;
+constexpr uint32_t kGdnTapeGateOffset =
+    kGdnTapeKeyOffset + kLayers * kGdnTapeRows * kGdnKeyHeads * kGdnHeadDim;
+constexpr uint32_t kGdnTapeFloats = kGdnTapeGateOffset + kLayers * kGdnTapeRows * kGdnValueHeads * 2;
+constexpr uint32_t kGdnConvTapeElements =
+    kLayers * kGdnTapeRows * (kGdnConvWidth - 1) * kGdnConvChannels;
+
 static_assert(kAttnProjectionRows == 9216 && kAttnQGateRows == 8192 && kAttnVRowOffset == 8704);
 static_assert(kGdnProjectionRows == 12352 && kGdnBRowOffset == 12288 && kGdnARowOffset == 12320);
+static_assert(kGdnTapeKeyOffset == 40u * 16u * 32u * 128u &&
+              kGdnTapeGateOffset == 40u * 16u * 32u * 128u + 40u * 16u * 16u * 128u &&
+              kGdnTapeFloats == 40u * 16u * (32u * 128u + 16u * 128u + 64u));
 static_assert(kGdnConvChannels == 8192 && kGdnKOffset == 2048 && kAttnRopePairs == 32);
 
 }  // namespace tt

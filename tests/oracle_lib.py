@@ -68,6 +68,10 @@ def _load_oracle():
         "tto_gdn_prefill": (None, [_u16p, u32, _u16p, _u16p, _u16p, _u16p, _u16p, _f32p, _u16p,
                                    _f32p, _u16p, _u16n, _u16n, _u16n, u32]),
         "tto_gdn_scan": (None, [_u16p, _u16p, _f32p, _f32p, u32, _f32p, _u16p, _f32p, u32]),
+        "tto_gdn_conv_tape": (None, [_u16p, u32, _u16p, _u16p, u32]),
+        "tto_gdn_scan_tape": (None, [_u16p, _u16p, _f32p, _f32p, u32, _f32p, _u16p, _f32p, _f32p,
+                                     u32, u32]),
+        "tto_gdn_tape_replay": (None, [_f32p, _f32p, _f32p, u32, u32, u32]),
         "tto_rms_only": (None, [_u16p, _u16p, u32, u32, _u16p]),
         "tto_dense_bf16": (None, [_u16p, _u16p, u32, u32, u32, _u16p, u32]),
         "tto_add_bf16": (None, [_u16p, _u16p, C.c_uint64, _u16p]),

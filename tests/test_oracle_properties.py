@@ -349,6 +349,117 @@ def test_scan_matches_fp64_sequential_within_tolerance():
     assert np.abs(s1.reshape(32, 128, 128)[h] - st).max() < 1e-4
 
 
+TAPE_FLOATS = 40 * 16 * (32 * 128 + 16 * 128 + 64)
+TAPE_KEYS = 40 * 16 * 32 * 128
+TAPE_GATES = TAPE_KEYS + 40 * 16 * 16 * 128
+
+
+def _scan_inputs(steps, seed):
+    rng = np.random.default_rng(seed)
+    qn = rng.standard_normal((steps, 16, 128)); kn = rng.standard_normal((steps, 16, 128))
+    qn /= np.linalg.norm(qn, axis=2, keepdims=True) * np.sqrt(128.0)
+    kn /= np.linalg.norm(kn, axis=2, keepdims=True)
+    qk = np.concatenate([qn.reshape(steps, -1), kn.reshape(steps, -1)], axis=1).astype(np.float32)
+    qkb = BF(qk.reshape(-1))
+    vb = BF(rng.standard_normal(steps * 4096).astype(np.float32))
+    decay = np.exp(rng.uniform(-0.1, 0.0, (steps, 32))).astype(np.float32).reshape(-1)
+    beta = (1 / (1 + np.exp(-rng.standard_normal((steps, 32))))).astype(np.float32).reshape(-1)
+    s0 = (rng.standard_normal(32 * 128 * 128) * 0.02).astype(np.float32)
+    return qkb, vb, decay, beta, s0
+
+
+def test_tape_replay_rebuilds_every_prefix_of_the_scan():
+    """The tape has no reference test.  What fixes it: replaying c taped rows must give,
+    bit for bit, the state a scan of exactly c rows stores; the taped scan itself must
+    not differ from the plain one; and the tape rows are the scan's own operands."""
+    steps, layer = 16, 29
+    qkb, vb, decay, beta, s0 = _scan_inputs(steps, 4242)
+    y0 = np.zeros(steps * 4096, np.uint16); s_plain = np.zeros_like(s0)
+    o.tto_gdn_scan(qkb, vb, decay, beta, steps, s0, y0, s_plain, 4)
+    tape = np.full(TAPE_FLOATS, np.float32(-77.0))
+    y1 = np.zeros_like(y0); s_taped = np.zeros_like(s0)
+    o.tto_gdn_scan_tape(qkb, vb, decay, beta, steps, s0, y1, s_taped, tape, layer, 4)
+    assert np.array_equal(y0, y1) and np.array_equal(s_plain.view(np.uint32), s_taped.view(np.uint32))
+    # only this layer's rows were written
+    deltas = tape[:TAPE_KEYS].reshape(40, 16, 32, 128)
+    keys = tape[TAPE_KEYS:TAPE_GATES].reshape(40, 16, 16, 128)
+    gates = tape[TAPE_GATES:].reshape(40, 16, 32, 2)
+    for region in (deltas, keys, gates):
+        others = np.delete(region, layer, axis=0)
+        assert np.all(others == np.float32(-77.0))
+    assert np.array_equal(keys[layer].reshape(steps, 2048),
+                          F(qkb).reshape(steps, 4096)[:, 2048:])
+    assert np.array_equal(gates[layer, :, :, 0].reshape(-1), decay)
+    assert np.array_equal(gates[layer, :, :, 1].reshape(-1), beta)
+    for committed in (0, 1, 2, 7, 15, 16):
+        want = np.zeros_like(s0)
+        if committed:
+            yc = np.zeros(committed * 4096, np.uint16)
+            o.tto_gdn_scan(qkb[:committed * 4096], vb[:committed * 4096], decay[:committed * 32],
+                           beta[:committed * 32], committed, s0, yc, want, 4)
+        else:
+            want = s0.copy()
+        got = np.zeros_like(s0)
+        o.tto_gdn_tape_replay(tape, s0, got, committed, layer, 4)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), committed
+
+
+def test_tape_delta_closed_form_and_long_blocks():
+    """From a zero state the first key-value product is zero, so delta = v * beta exactly
+    and the replayed state is the outer product k (x) delta; a block longer than the tape
+    records nothing."""
+    qkb, vb, decay, beta, _ = _scan_inputs(1, 99)
+    zero = np.zeros(32 * 128 * 128, np.float32)
+    tape = np.zeros(TAPE_FLOATS, np.float32)
+    y = np.zeros(4096, np.uint16); s1 = np.zeros_like(zero)
+    o.tto_gdn_scan_tape(qkb, vb, decay, beta, 1, zero, y, s1, tape, 0, 2)
+    v = F(vb).reshape(32, 128)
+    want = v * beta.reshape(32, 1)
+    assert np.array_equal(tape[:32 * 128].reshape(32, 128), want.astype(np.float32))
+    k = F(qkb)[2048:].reshape(16, 128)
+    outer = want[:, :, None] * np.repeat(k, 2, axis=0)[:, None, :]
+    assert np.array_equal(s1.reshape(32, 128, 128), outer.astype(np.float32))
+    rebuilt = np.zeros_like(zero)
+    o.tto_gdn_tape_replay(tape, zero, rebuilt, 1, 0, 2)
+    assert np.array_equal(rebuilt, s1)
+
+    steps = 17
+    qkb, vb, decay, beta, s0 = _scan_inputs(steps, 100)
+    tape = np.full(TAPE_FLOATS, np.float32(3.0))
+    y = np.zeros(steps * 4096, np.uint16); s1 = np.zeros_like(s0)
+    o.tto_gdn_scan_tape(qkb, vb, decay, beta, steps, s0, y, s1, tape, 5, 4)
+    assert np.all(tape == np.float32(3.0))
+    y2 = np.zeros_like(y); s2 = np.zeros_like(s0)
+    o.tto_gdn_scan(qkb, vb, decay, beta, steps, s0, y2, s2, 4)
+    assert np.array_equal(y, y2) and np.array_equal(s1, s2)
+
+
+def test_conv_tape_rows_are_the_conv_state_of_each_prefix():
+    """conv_tape[row] must equal the new conv state of a block that ends at that row
+    (computed by the block prefill, an independent path)."""
+    rows, layer = 9, 13
+    proj = np.zeros(rows * 12352, np.uint16); o.tto_fill_gaussian_bf16(51, 0.0, 0.5, proj, proj.size)
+    conv = np.zeros(3 * 8192, np.uint16); o.tto_fill_gaussian_bf16(52, 0.0, 0.5, conv, conv.size)
+    cw = np.zeros(4 * 8192, np.uint16); o.tto_fill_gaussian_bf16(53, 0.0, 0.3, cw, cw.size)
+    small = np.zeros(32, np.uint16); nw = np.full(128, 0x3F80, np.uint16)
+    s0 = np.zeros(32 * 128 * 128, np.float32)
+    tape = np.full(40 * 16 * 3 * 8192, 0x7FC0, np.uint16)
+    o.tto_gdn_conv_tape(proj, rows, conv, tape, layer)
+    windows = tape.reshape(40, 16, 3 * 8192)
+    assert np.all(np.delete(windows, layer, axis=0) == 0x7FC0)
+    assert np.all(windows[layer, rows:] == 0x7FC0)
+    for ending in (1, 2, 3, 4, 9):
+        ncs = np.zeros_like(conv); s1 = np.zeros_like(s0)
+        gated = np.zeros(ending * 4096, np.uint16)
+        o.tto_gdn_prefill(proj[:ending * 12352], ending, conv, cw, small, small, nw, s0, ncs, s1,
+                          gated, None, None, None, 4)
+        assert np.array_equal(windows[layer, ending - 1], ncs), ending
+    untouched = np.full(40 * 16 * 3 * 8192, 0x7FC0, np.uint16)
+    big = np.zeros(17 * 12352, np.uint16)
+    o.tto_gdn_conv_tape(big, 17, conv, untouched, 0)
+    assert np.all(untouched == 0x7FC0)
+
+
 def test_dense_and_add_against_float64():
     """The stand-in projection is a plain dot product rounded once to bf16 and the
     residual sum is one bf16 addition: both against float64 numpy."""
