@@ -868,7 +868,9 @@ PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan
         policy.first_chunk_rows == 0 || policy.first_chunk_rows > policy.maximum_block_rows ||
         policy.query_tile_rows == 0 || policy.query_tile_rows > policy.maximum_block_rows ||
         policy.query_tile_rows % kPrefillQueryTileMultiple != 0 ||
-        policy.attention_partition != kAttentionPartition) {
+        policy.attention_partition != kAttentionPartition ||
+        (policy.gdn_tape && (!policy.gdn_gate_hoist || policy.gdn_chunked ||
+                             plan.layers.size() > kGdnTapeLayers))) {
         return {PrefillGeometryError::InvalidPolicy, {}};
     }
     PrefillGeometry g;
@@ -901,6 +903,8 @@ PrefillGeometryResult make_prefill_geometry(const model::qwen36::ModelPlan& plan
                                                kGdnChunkRows - 1u) / kGdnChunkRows) *
                                                  plan.recurrent_heads * kGdnChunkRecordBytes
                                            : 0;
+    g.gdn_tape_bytes = policy.gdn_tape ? kGdnTapeBytes : 0;
+    g.gdn_conv_tape_bytes = policy.gdn_tape ? kGdnConvTapeBytes : 0;
     g.attention_projection_bytes = block * rows.attn_projection * kBf16Bytes;
     g.attention_vector_bytes = block * rows.attn_query * kBf16Bytes;
     std::uint64_t records = 0;
@@ -977,7 +981,11 @@ PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::gdn_recurrence_gates_blk, "gdn_recurrence_gates_blk", error) &&
         resolve(library, p, &P::gdn_recurrence_blk, "gdn_recurrence_blk", error) &&
         resolve(library, p, &P::gdn_gate_norm_blk, "gdn_gate_norm_blk", error) &&
-        resolve(library, p, &P::gdn_chunk_recurrence_blk, "gdn_chunk_recurrence_blk", error);
+        resolve(library, p, &P::gdn_chunk_recurrence_blk, "gdn_chunk_recurrence_blk", error) &&
+        resolve(library, p, &P::gdn_conv_tape_blk, "gdn_conv_tape_blk", error) &&
+        resolve(library, p, &P::gdn_recurrence_gates_tape_blk, "gdn_recurrence_gates_tape_blk",
+                error) &&
+        resolve(library, p, &P::gdn_tape_replay_blk, "gdn_tape_replay_blk", error);
     if (!ok) return {error, std::nullopt};
     return {HipPipelineError::None, std::move(p)};
 }
@@ -999,6 +1007,9 @@ PrefillScratchResult create_prefill_scratch(const HipDevice& device,
         !allocate_zeroed(device, parameter_bytes, s.gdn_beta) ||
         (geometry.gdn_chunk_bytes != 0 &&
          !allocate_zeroed(device, geometry.gdn_chunk_bytes, s.gdn_chunk)) ||
+        (geometry.gdn_tape_bytes != 0 &&
+         (!allocate_zeroed(device, geometry.gdn_tape_bytes, s.gdn_tape) ||
+          !allocate_zeroed(device, geometry.gdn_conv_tape_bytes, s.gdn_conv_tape))) ||
         !allocate_zeroed(device, geometry.attention_projection_bytes, s.attn_projection) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_query) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_gate) ||
@@ -1049,16 +1060,21 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
                                            const PrefillGeometry& geometry, PrefillScratch& scratch,
                                            const DecodeLayerState& state,
                                            const LayerWeights& weights, const PrefillChunk& chunk,
-                                           std::uint32_t recurrence_ordinal, HipComputePass& pass) {
+                                           std::uint32_t recurrence_ordinal, HipComputePass& pass,
+                                           std::uint32_t layer_index) {
     const std::uint32_t rows = chunk.rows;
     if (rows == 0 || rows > scratch.block_rows) return HipCommandError::InvalidDispatchExtent;
+    const bool taped = geometry.policy.gdn_tape;
+    if (taped && (!scratch.gdn_tape || !scratch.gdn_conv_tape || layer_index >= kGdnTapeLayers)) {
+        return HipCommandError::InvalidBuffer;
+    }
     const bool phase = state.swapped ^ ((recurrence_ordinal & 1u) != 0u);
     const HipBuffer& conv_in = phase ? state.first_out : state.first;
     const HipBuffer& conv_out = phase ? state.first : state.first_out;
     const HipBuffer& recurrent_in = phase ? state.second_out : state.second;
     const HipBuffer& recurrent_out = phase ? state.second : state.second_out;
     Walk walk{pass};
-    walk.pipeline(pipelines.gdn_conv_blk);
+    walk.pipeline(taped ? pipelines.gdn_conv_tape_blk : pipelines.gdn_conv_blk);
     walk.buffer(scratch.gdn_projection, 0, 0);
     walk.buffer(conv_in, 0, 1);
     walk.weight(weights.conv_weight, 2);
@@ -1067,6 +1083,10 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
     walk.buffer(scratch.gdn_gate, 0, 5);
     walk.buffer(conv_out, 0, 6);
     walk.constant(rows, 7);
+    if (taped) {
+        walk.buffer(scratch.gdn_conv_tape, 0, 8);
+        walk.constant(layer_index, 9);
+    }
     walk.dispatch(96, 128, rows);
     walk.barrier();
     if (geometry.policy.gdn_chunked) {
@@ -1110,12 +1130,17 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
         walk.constant(rows, 5);
         walk.dispatch(HipSize{1, (rows + 3u) / 4u, 1}, HipSize{32, 4, 1});
         walk.barrier();
-        walk.pipeline(pipelines.gdn_recurrence_gates_blk);
+        walk.pipeline(taped ? pipelines.gdn_recurrence_gates_tape_blk
+                            : pipelines.gdn_recurrence_gates_blk);
         walk.buffer(scratch.gdn_qk, 0, 0);
         walk.buffer(scratch.gdn_value, 0, 1);
         walk.buffer(scratch.gdn_decay, 0, 2);
         walk.weight(weights.a_log, 3);
         walk.buffer(scratch.gdn_beta, 0, 4);
+        if (taped) {
+            walk.buffer(scratch.gdn_tape, 0, 9);
+            walk.constant(layer_index, 10);
+        }
     } else {
         walk.pipeline(pipelines.gdn_recurrence_blk);
         walk.buffer(scratch.gdn_qk, 0, 0);
@@ -1137,6 +1162,58 @@ HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
     walk.buffer(scratch.gdn_gated, 0, 3);
     walk.dispatch(32, 128, rows);
     return walk.error;
+}
+
+HipCommandError encode_gdn_tape_replay(const PrefillPipelines& pipelines, const DecodeStep& step,
+                                       const DecodeStateSlot& state, const PrefillScratch& scratch,
+                                       std::uint32_t committed, HipComputePass& pass) {
+    if (!decode_state_slot_compatible(step, state) || !decode_state_slot_ready(step, state)) {
+        return HipCommandError::StateSlotMismatch;
+    }
+    if (!scratch.gdn_tape || step.schedule.size() > kGdnTapeLayers) {
+        return HipCommandError::InvalidBuffer;
+    }
+    if (committed == 0 || committed > kGdnTapeRows) return HipCommandError::InvalidDispatchExtent;
+    Walk walk{pass};
+    for (std::uint32_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (!is_gated(step.schedule[layer])) continue;
+        const DecodeLayerState& s = state.layers[layer];
+        walk.pipeline(pipelines.gdn_tape_replay_blk);
+        walk.buffer(scratch.gdn_tape, 0, 0);
+        walk.buffer(s.swapped ? s.second_out : s.second, 0, 1);
+        walk.buffer(s.swapped ? s.second : s.second_out, 0, 2);
+        walk.constant(committed, 3);
+        walk.constant(layer, 4);
+        walk.dispatch(HipSize{1, 32, 32}, HipSize{32, 4, 1});
+    }
+    return walk.error;
+}
+
+HipCommandError encode_gdn_tape_windows(const DecodeStep& step, DecodeStateSlot& state,
+                                        const PrefillScratch& scratch, std::uint32_t committed,
+                                        HipBlitPass& blit_pass) {
+    if (!decode_state_slot_compatible(step, state) || !decode_state_slot_ready(step, state)) {
+        return HipCommandError::StateSlotMismatch;
+    }
+    if (!scratch.gdn_conv_tape || step.schedule.size() > kGdnTapeLayers) {
+        return HipCommandError::InvalidBuffer;
+    }
+    if (committed == 0 || committed > kGdnTapeRows) return HipCommandError::InvalidCopyExtent;
+    const std::uint64_t window = step.geometry.gdn_conv_state_bytes;
+    for (std::uint32_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (!is_gated(step.schedule[layer])) continue;
+        DecodeLayerState& s = state.layers[layer];
+        const HipCommandError copied = copy_buffer(
+            blit_pass, scratch.gdn_conv_tape,
+            (std::uint64_t{layer} * kGdnTapeRows + (committed - 1u)) * window,
+            s.swapped ? s.first : s.first_out, 0, window);
+        if (copied != HipCommandError::None) return copied;
+    }
+    return HipCommandError::None;
+}
+
+void complete_gdn_tape_rollback(const DecodeStep& step, DecodeStateSlot& state) {
+    advance_prefill_state(step, state, 1);
 }
 
 // ---- lane state record (Q36BRS01) ------------------------------------------

@@ -62,6 +62,12 @@ inline constexpr std::uint32_t kConvShiftSteps = 3;
 inline constexpr std::uint32_t kGdnChunkRows = 64;             // tokens per chunk of the MFMA recurrence
 inline constexpr std::uint32_t kGdnChunkRecordBytes = 115712;  // scratch per (chunk, value head)
 inline constexpr std::uint32_t kGdnChunkGroupRows = 2048;      // rows whose records are live at once
+inline constexpr std::uint32_t kGdnTapeRows = 16;              // rows a rollback tape holds
+inline constexpr std::uint32_t kGdnTapeLayers = 40;            // layers the tape is laid out for
+inline constexpr std::uint64_t kGdnTapeBytes =                 // prefill_step.cpp:3231-3233
+    std::uint64_t{40} * 16u * (32u * 128u + 16u * 128u + 64u) * 4u;
+inline constexpr std::uint64_t kGdnConvTapeBytes =             // prefill_step.cpp:3235-3237
+    std::uint64_t{40} * 16u * 3u * 8192u * 2u;
 inline constexpr std::uint32_t kBf16Bytes = 2;
 inline constexpr std::uint32_t kF32Bytes = 4;
 inline constexpr std::uint32_t kMaximumBatchRows = 16;         // decode_step.cpp:554, 1008
@@ -371,6 +377,10 @@ struct PrefillPolicy {
     // instead of the reference's token-by-token register loop.
     // Implies hoisted gates.  The reference has no such switch.
     bool gdn_chunked{false};
+    // Record the rollback tape while a block of at most kGdnTapeRows rows runs through
+    // the register loop (PrefillGdnRecurrence::RegisterLoopTape, prefill_step.cpp:1931-1933).
+    // Needs hoisted gates, excludes gdn_chunked, and at most kGdnTapeLayers layers.
+    bool gdn_tape{false};
 };
 
 enum class PrefillRequestError : std::uint8_t {
@@ -426,6 +436,8 @@ struct PrefillGeometry {
     std::uint64_t gdn_value_bytes{0};
     std::uint64_t gdn_parameter_bytes{0};
     std::uint64_t gdn_chunk_bytes{0};  // chunk records of the MFMA recurrence; 0 when unused
+    std::uint64_t gdn_tape_bytes{0};       // rollback tape (fp32 regions); 0 when unused
+    std::uint64_t gdn_conv_tape_bytes{0};  // conv windows after each taped row; 0 when unused
     std::uint64_t attention_projection_bytes{0};
     std::uint64_t attention_vector_bytes{0};
     std::uint64_t attention_partial_bytes{0};
@@ -464,6 +476,7 @@ struct PrefillPipelines {
     HipComputePipeline attn_qk_rope_blk, attention_flash_blk;
     HipComputePipeline gdn_conv_blk, gdn_gates_blk, gdn_recurrence_gates_blk, gdn_recurrence_blk,
         gdn_gate_norm_blk, gdn_chunk_recurrence_blk;
+    HipComputePipeline gdn_conv_tape_blk, gdn_recurrence_gates_tape_blk, gdn_tape_replay_blk;
 };
 struct PrefillPipelinesResult {
     backend::hip::HipPipelineError error;
@@ -479,6 +492,7 @@ struct PrefillScratch {
     std::uint32_t block_rows{0};
     HipBuffer gdn_projection, gdn_qk, gdn_value, gdn_gate, gdn_recurrence, gdn_gated;
     HipBuffer gdn_decay, gdn_beta, gdn_chunk;
+    HipBuffer gdn_tape, gdn_conv_tape;
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended;
 };
 struct PrefillScratchResult {
@@ -502,12 +516,30 @@ HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
 // encode_gated_delta (prefill_step.cpp:1854-2081): phase = swapped ^ (ordinal & 1)
 // selects the ping-pong planes; conv over the block, gates (hoisted or inline),
 // register-loop scan or, with policy.gdn_chunked, the chunked MFMA recurrence,
-// gate-norm.
+// gate-norm.  With policy.gdn_tape the conv and the scan also record the rollback
+// tape of `layer_index` (rows beyond kGdnTapeRows record nothing).
 HipCommandError encode_prefill_gated_delta(const PrefillPipelines& pipelines,
                                            const PrefillGeometry& geometry, PrefillScratch& scratch,
                                            const DecodeLayerState& state,
                                            const LayerWeights& weights, const PrefillChunk& chunk,
-                                           std::uint32_t recurrence_ordinal, HipComputePass& pass);
+                                           std::uint32_t recurrence_ordinal, HipComputePass& pass,
+                                           std::uint32_t layer_index = 0);
+
+// Rollback of a taped block to its first `committed` rows (tape_rollback,
+// speculative_decode.cpp:517-600).  Call while the slot's flags still name the planes
+// the block READ (that is, instead of advance_prefill_state for the block): every
+// gated-delta layer's recurrent state is replayed from that plane into the opposite
+// one, the conv window after row committed-1 is copied from the conv tape into the
+// opposite conv plane, and completion toggles `swapped` exactly as a block of
+// `committed` rows would have.  Attention caches need nothing: rows past the
+// committed context are never read.
+HipCommandError encode_gdn_tape_replay(const PrefillPipelines& pipelines, const DecodeStep& step,
+                                       const DecodeStateSlot& state, const PrefillScratch& scratch,
+                                       std::uint32_t committed, HipComputePass& pass);
+HipCommandError encode_gdn_tape_windows(const DecodeStep& step, DecodeStateSlot& state,
+                                        const PrefillScratch& scratch, std::uint32_t committed,
+                                        HipBlitPass& blit_pass);
+void complete_gdn_tape_rollback(const DecodeStep& step, DecodeStateSlot& state);
 
 // ---- lane state record (Q36BRS01) ------------------------------------------
 // The file / wire form of exactly the buffers a lane owns on this path

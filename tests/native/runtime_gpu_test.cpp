@@ -544,6 +544,114 @@ int main() {
                 if (target_keys[i] != 0) return 147;
             }
         }
+
+        // ---- a taped block of 12 rows rolled back to its first 5 -------------------
+        std::printf("[case] taped block, rollback to a prefix\n");
+        PrefillPolicy tape_policy = policy;
+        tape_policy.maximum_block_rows = tape_policy.first_chunk_rows =
+            tape_policy.query_tile_rows = 16;
+        tape_policy.gdn_chunked = false;
+        PrefillPolicy plain_policy = tape_policy;
+        tape_policy.gdn_tape = true;
+        {
+            PrefillPolicy refused = tape_policy;
+            refused.gdn_chunked = true;
+            if (make_prefill_geometry(plan, refused).error != PrefillGeometryError::InvalidPolicy) {
+                return 150;
+            }
+            refused = tape_policy;
+            refused.gdn_gate_hoist = false;
+            if (make_prefill_geometry(plan, refused).error != PrefillGeometryError::InvalidPolicy) {
+                return 150;
+            }
+        }
+        const auto taped_geometry = make_prefill_geometry(plan, tape_policy);
+        const auto plain_geometry = make_prefill_geometry(plan, plain_policy);
+        if (!taped_geometry || !plain_geometry) return 151;
+        if (taped_geometry.geometry.gdn_tape_bytes != 15'892'480ull ||
+            taped_geometry.geometry.gdn_conv_tape_bytes != 31'457'280ull ||
+            plain_geometry.geometry.gdn_tape_bytes != 0) {
+            return 152;
+        }
+        auto taped_scratch_made = create_prefill_scratch(*device.device, taped_geometry.geometry);
+        auto plain_scratch_made = create_prefill_scratch(*device.device, plain_geometry.geometry);
+        if (!taped_scratch_made || !plain_scratch_made) return 153;
+        PrefillScratch& taped_scratch = *taped_scratch_made.scratch;
+        PrefillScratch& plain_scratch = *plain_scratch_made.scratch;
+        const std::uint32_t block_rows = 12, committed = 5;
+        const auto block = gauss16(7100, block_rows * 12352, 0.5);
+        const std::vector<std::uint16_t> prefix(block.begin(), block.begin() + committed * 12352);
+        auto lane_a_made = create_decode_state_slot(*device.device, step);
+        auto lane_b_made = create_decode_state_slot(*device.device, step);
+        if (!lane_a_made || !lane_b_made) return 154;
+        DecodeStateSlot& lane_a = *lane_a_made.slot;
+        DecodeStateSlot& lane_b = *lane_b_made.slot;
+        std::uint32_t base_a = 0, base_b = 0;
+        if (load_state_record(record, step, lane_a, base_a) != StateRecordError::None ||
+            load_state_record(record, step, lane_b, base_b) != StateRecordError::None) {
+            return 155;
+        }
+        const auto run_block = [&](const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                   DecodeStateSlot& lane, std::uint32_t rows) {
+            const PrefillChunk chunk{0, rows, 0};
+            return submit.run([&](HipComputePass& pass) {
+                for (std::uint32_t layer = 0; layer < 3; ++layer) {
+                    HipCommandError e = encode_prefill_gated_delta(
+                        *prefill_pipes.pipelines, geometry, scratch, lane.layers[layer],
+                        bound[layer], chunk, 0, pass, layer);
+                    if (e != HipCommandError::None) return e;
+                    e = memory_barrier(pass);
+                    if (e != HipCommandError::None) return e;
+                }
+                return HipCommandError::None;
+            });
+        };
+        // lane A: the whole block with the tape on, then back to `committed` rows
+        if (!upload(taped_scratch.gdn_projection, block)) return 156;
+        if (run_block(taped_geometry.geometry, taped_scratch, lane_a, block_rows) != 0) return 157;
+        {
+            HipComputePass no_pass;
+            if (encode_gdn_tape_replay(*prefill_pipes.pipelines, step, lane_a, taped_scratch, 0,
+                                       no_pass) != HipCommandError::InvalidDispatchExtent ||
+                encode_gdn_tape_replay(*prefill_pipes.pipelines, step, lane_a, taped_scratch, 17,
+                                       no_pass) != HipCommandError::InvalidDispatchExtent ||
+                encode_gdn_tape_replay(*prefill_pipes.pipelines, step, lane_a, plain_scratch,
+                                       committed, no_pass) != HipCommandError::InvalidBuffer) {
+                return 158;
+            }
+        }
+        if (submit.run([&](HipComputePass& pass) {
+                return encode_gdn_tape_replay(*prefill_pipes.pipelines, step, lane_a, taped_scratch,
+                                              committed, pass);
+            }) != 0) {
+            return 159;
+        }
+        {
+            auto cb = create_command_buffer(*queue.command_queue);
+            if (!cb) return 160;
+            auto blit = begin_blit_pass(std::move(*cb.command_buffer));
+            if (!blit) return 160;
+            if (encode_gdn_tape_windows(step, lane_a, taped_scratch, committed, *blit.blit_pass) !=
+                HipCommandError::None) {
+                return 161;
+            }
+            auto ended = end_blit_pass(std::move(*blit.blit_pass));
+            auto pending = commit(std::move(*ended.command_buffer));
+            if (!pending || !wait_until_completed(std::move(*pending.pending_execution))) return 162;
+        }
+        complete_gdn_tape_rollback(step, lane_a);
+        // lane B: only the committed rows, no tape
+        if (!upload(plain_scratch.gdn_projection, prefix)) return 163;
+        if (run_block(plain_geometry.geometry, plain_scratch, lane_b, committed) != 0) return 164;
+        advance_prefill_state(step, lane_b, 1);
+        if (!lane_a.layers[0].swapped || !lane_b.layers[0].swapped) return 165;
+        std::vector<std::byte> record_a, record_b;
+        if (write_state_record(step, lane_a, positions, record_a) != StateRecordError::None ||
+            write_state_record(step, lane_b, positions, record_b) != StateRecordError::None) {
+            return 166;
+        }
+        if (record_a == record) return 167;  // the block did change the state
+        if (record_a != record_b) return 168;
         slot.layers[1].swapped = false;
     }
 
