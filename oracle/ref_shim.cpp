@@ -51,6 +51,15 @@ void ref_rms_only(const std::uint16_t* in, const std::uint16_t* w, std::uint32_t
                        std::span<std::uint16_t>(out, hidden));
 }
 
+float ref_q4_dot(const std::uint16_t* x, const std::uint32_t* words, const std::uint16_t* scales,
+                 const std::uint16_t* biases, std::uint32_t k_size) {
+    return q4_dot_reference(std::span<const std::uint16_t>(x, k_size),
+                            std::span<const std::uint32_t>(words, k_size / 8),
+                            std::span<const std::uint16_t>(scales, k_size / 64),
+                            std::span<const std::uint16_t>(biases, k_size / 64), k_size,
+                            SimdTreeShape::AdjacentPairs, ChainOrder::Fused);
+}
+
 void ref_residual_sums(const std::uint16_t* a, const std::uint16_t* b, std::uint64_t count,
                        std::uint16_t* out) {
     residual_rms_rounded_sums(std::span<const std::uint16_t>(a, count),

@@ -764,6 +764,55 @@ void tto_gdn_prefill(const uint16_t* projection, uint32_t rows, const uint16_t* 
     if (y_out) std::memcpy(y_out, y.data(), y.size() * 2);
 }
 
+float tto_q4_dot(const uint16_t* x, const uint32_t* words, const uint16_t* scales,
+                 const uint16_t* biases, uint32_t k_size) {
+    const uint16_t* packed = reinterpret_cast<const uint16_t*>(words);
+    float lanes[32];
+    for (uint32_t lane = 0; lane < 32; ++lane) {
+        float result = 0.0f;
+        for (uint32_t k = 0; k < k_size; k += 512) {
+            const uint16_t* xs = x + k + lane * 16;
+            float scaled[16];
+            float sum = 0.0f;
+            for (uint32_t i = 0; i < 16; i += 4) {
+                const float a0 = widen(xs[i]), a1 = widen(xs[i + 1]), a2 = widen(xs[i + 2]),
+                            a3 = widen(xs[i + 3]);
+                sum = fz32(sum + fz32((fz32(a0 + a1) + a2) + a3));
+                scaled[i] = a0;
+                scaled[i + 1] = a1 / 16.0f;
+                scaled[i + 2] = a2 / 256.0f;
+                scaled[i + 3] = a3 / 4096.0f;
+            }
+            float quant = 0.0f;
+            const uint16_t* w = packed + (k >> 2) + lane * 4;
+            for (uint32_t i = 0; i < 4; ++i) {
+                // masked, unshifted nibbles: 0..15, 0..240, 0..3840, 0..61440
+                quant = std::fma(scaled[i * 4], static_cast<float>(w[i] & 0x000Fu), quant);
+                quant = std::fma(scaled[i * 4 + 1], static_cast<float>(w[i] & 0x00F0u), quant);
+                quant = std::fma(scaled[i * 4 + 2], static_cast<float>(w[i] & 0x0F00u), quant);
+                quant = std::fma(scaled[i * 4 + 3], static_cast<float>(w[i] & 0xF000u), quant);
+            }
+            const uint32_t group = (k >> 6) + (lane >> 2);
+            result = std::fma(sum, widen(biases[group]), std::fma(widen(scales[group]), quant, result));
+        }
+        lanes[lane] = result;
+    }
+    return adjacent32(lanes);
+}
+
+void tto_q4_project(const uint16_t* x, uint64_t x_stride, uint32_t rows, const uint32_t* words,
+                    const uint16_t* scales, const uint16_t* biases, uint32_t k_size,
+                    uint32_t out_rows, uint16_t* out, uint64_t out_stride, uint32_t threads) {
+    parallel_for(out_rows, threads, [=](uint32_t n) {
+        const uint32_t* w = words + static_cast<size_t>(n) * (k_size / 8);
+        const uint16_t* s = scales + static_cast<size_t>(n) * (k_size / 64);
+        const uint16_t* b = biases + static_cast<size_t>(n) * (k_size / 64);
+        for (uint32_t r = 0; r < rows; ++r) {
+            out[r * out_stride + n] = store16(tto_q4_dot(x + r * x_stride, w, s, b, k_size));
+        }
+    });
+}
+
 void tto_rms_only(const uint16_t* input, const uint16_t* weight, uint32_t rows, uint32_t hidden,
                   uint16_t* output) {
     // hidden / 4 threads of 4 values, simdgroup trees over 32 lanes, then a tree over

@@ -29,6 +29,10 @@
  *     against an fp64 textbook evaluation.
  *   - tto_gdn_chunked_f64: brute-force equality with the sequential fp64
  *     recurrence on small shapes.
+ *   - tto_q4_dot / tto_q4_project: bit-equality with the reference's
+ *     q4_dot_reference (oracle/_ref), the packed-nibble addressing and affine
+ *     known answers of kernel_reference_test.cpp:327-345 restated for this
+ *     layout, and an fp64 dequantised dot product.
  *   - tto_gdn_conv_tape / tto_gdn_scan_tape / tto_gdn_tape_replay: the
  *     reference holds no test or fixture for the tape; pinned by what the
  *     definition fixes: replaying c rows equals, bit for bit, the state the
@@ -226,6 +230,22 @@ void tto_gdn_scan_tape(const uint16_t* qk, const uint16_t* value, const float* d
                        float* state_out, float* tape, uint32_t tape_layer, uint32_t threads);
 void tto_gdn_tape_replay(const float* tape, const float* state_in, float* state_out,
                          uint32_t steps, uint32_t tape_layer, uint32_t threads);
+
+/* Affine 4-bit projections (group 64): w[n][k] = scale[n][k/64] * nibble + bias[n][k/64],
+ * eight nibbles to a 32-bit word, low nibble first (q4_dot.metal:9-41;
+ * q4_dot_reference kernel_reference.cpp:388-443 in the fused order with the
+ * adjacent-pairs tree).  One lane of 32 owns 16 consecutive inputs of every 512
+ * block; the place value of a masked nibble is undone by exact power-of-two
+ * pre-scaling of the input.  k_size is a multiple of 512.
+ * tto_q4_project: out[r][n] = bf16(q4_dot(x[r], row n)) for n < out_rows, the
+ * arithmetic of attn_project / gdn_project / gdn_outproj and their _ms / _blk
+ * forms (attention.metal:1-41, gdn.metal:1-47, 209-230; prefill_dense.metal:120-260),
+ * whose batching never changes a row's sequence of operations. */
+float tto_q4_dot(const uint16_t* x, const uint32_t* words, const uint16_t* scales,
+                 const uint16_t* biases, uint32_t k_size);
+void tto_q4_project(const uint16_t* x, uint64_t x_stride, uint32_t rows, const uint32_t* words,
+                    const uint16_t* scales, const uint16_t* biases, uint32_t k_size,
+                    uint32_t out_rows, uint16_t* out, uint64_t out_stride, uint32_t threads);
 
 /* The steps either side of the path in a stacked run.
  * tto_rms_only: row RMS norm with the double rounding bf16(w * bf16(x * inv))

@@ -439,6 +439,7 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
         {tt::kAttentionPrefillKernels, tt::kAttentionPrefillKernelCount},
         {tt::kAttentionFamilyKernels, tt::kAttentionFamilyKernelCount},
         {tt::kStackStepKernels, tt::kStackStepKernelCount},
+        {tt::kQ4ProjectKernels, tt::kQ4ProjectKernelCount},
         {tt::kGdnDecodeKernels, tt::kGdnDecodeKernelCount},
         {tt::kGdnPrefillKernels, tt::kGdnPrefillKernelCount},
     };

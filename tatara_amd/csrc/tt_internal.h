@@ -98,6 +98,8 @@ extern const KernelDesc kAttentionPrefillKernels[];
 extern const uint32_t kAttentionPrefillKernelCount;
 extern const KernelDesc kAttentionFamilyKernels[];
 extern const uint32_t kAttentionFamilyKernelCount;
+extern const KernelDesc kQ4ProjectKernels[];
+extern const uint32_t kQ4ProjectKernelCount;
 extern const KernelDesc kStackStepKernels[];
 extern const uint32_t kStackStepKernelCount;
 extern const KernelDesc kGdnDecodeKernels[];

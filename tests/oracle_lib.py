@@ -72,6 +72,8 @@ def _load_oracle():
         "tto_gdn_scan_tape": (None, [_u16p, _u16p, _f32p, _f32p, u32, _f32p, _u16p, _f32p, _f32p,
                                      u32, u32]),
         "tto_gdn_tape_replay": (None, [_f32p, _f32p, _f32p, u32, u32, u32]),
+        "tto_q4_dot": (f32, [_u16p, _u32p, _u16p, _u16p, u32]),
+        "tto_q4_project": (None, [_u16p, u64, u32, _u32p, _u16p, _u16p, u32, u32, _u16p, u64, u32]),
         "tto_rms_only": (None, [_u16p, _u16p, u32, u32, _u16p]),
         "tto_dense_bf16": (None, [_u16p, _u16p, u32, u32, u32, _u16p, u32]),
         "tto_add_bf16": (None, [_u16p, _u16p, C.c_uint64, _u16p]),
@@ -102,6 +104,7 @@ def _load_ref():
         "ref_tree_sum": (f32, [_f32p, u32, u32]),
         "ref_rms_only": (None, [_u16p, _u16p, u32, u32, u32, _u16p]),
         "ref_residual_sums": (None, [_u16p, _u16p, u64, _u16p]),
+        "ref_q4_dot": (f32, [_u16p, _u32p, _u16p, _u16p, u32]),
         "ref_attn_qk_rope": (None, [_u16p, _u16p, _u16p, u32, u32, _u16p, _u16p, _u16p, _u16p]),
         "ref_attention_decode": (None, [_u16p, _u16p, _u16p, _u16p, u32, u32, _u16p]),
         "ref_attention_decode_split": (None, [_u16p, _u16p, _u16p, _u16p, u32, u32, u32, _f32n,

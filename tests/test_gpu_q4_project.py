@@ -1,0 +1,154 @@
+"""Affine 4-bit projections either side of the attention family on the GPU, through
+the C ABI, against the CPU checker (itself bit-equal to the reference's
+q4_dot_reference).
+
+Decode operators (`*_project`, `*_project_ms{,_v2}`, `gdn_outproj{,_ms,_ms_v2}`) keep the
+reference's sequence of operations, so every bf16 output must be the checker's bit
+pattern.  The block operators (`*_blk`) are held to the path's bar (max-abs 2e-2,
+mean-abs 2e-3) with a 2-step allowance on large values: their sums run in another
+order."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from gpu_util import check_bf16, gpu, run
+
+pytestmark = pytest.mark.gpu
+o = ol.oracle
+
+ATTN = {"name": "attn_project", "segments": [8192, 512, 512], "k": 2048, "out": 10, "threads": 128}
+GDN = {"name": "gdn_project", "segments": [8192, 4096, 32, 32], "k": 2048, "out": 13, "threads": 128}
+OUT = {"name": "gdn_outproj", "segments": [2048], "k": 4096, "out": 4, "threads": 64}
+
+
+def _matrix(seed, rows, k):
+    rng = np.random.default_rng(seed)
+    words = rng.integers(0, 2 ** 32, rows * k // 8, dtype=np.uint64).astype(np.uint32)
+    scales = ol.f32_to_bf16(rng.uniform(0.002, 0.01, rows * k // 64).astype(np.float32))
+    biases = ol.f32_to_bf16((-7.5 * ol.bf16_to_f32(scales) +
+                             rng.normal(0.0, 1e-3, scales.size)).astype(np.float32))
+    return words, scales, biases
+
+
+def _family(dev, family, seed):
+    host, device = [], {}
+    for index, rows in enumerate(family["segments"]):
+        w, s, b = _matrix(seed + index, rows, family["k"])
+        host.append((w, s, b))
+        slot = 1 + 3 * index
+        device[slot], device[slot + 1], device[slot + 2] = (dev.buffer_from(w), dev.buffer_from(s),
+                                                            dev.buffer_from(b))
+    return host, device
+
+
+def _groups(family):
+    per = family["threads"] // 32
+    return (sum(family["segments"]) + per - 1) // per
+
+
+def _expected(family, host, x, rows, out_stride=None):
+    total = sum(family["segments"])
+    stride = out_stride or total
+    want = np.zeros(rows * stride, np.uint16)
+    first = 0
+    for (w, s, b), n in zip(host, family["segments"]):
+        o.tto_q4_project(x, family["k"], rows, w, s, b, family["k"], n, want[first:], stride, 8)
+        first += n
+    return want
+
+
+@pytest.mark.parametrize("family", [ATTN, GDN, OUT], ids=lambda f: f["name"])
+def test_single_row_projection_bit_for_bit(family):
+    print(f"[case] {family['name']} one row", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9000)
+    x = ol.gaussian_bf16(0x9100, family["k"], 0.0, 1.0)
+    total = sum(family["segments"])
+    out = dev.create_buffer(total * 2)
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    ms = run(lambda cb: cb.encode(lib.pipeline(family["name"]), bindings, {}, (_groups(family), 1, 1),
+                                  (family["threads"], 1, 1)))
+    assert np.array_equal(out.read(np.uint16), _expected(family, host, x, 1))
+    print(f"[time] {family['name']}: {ms * 1e3:.1f} us", flush=True)
+
+
+@pytest.mark.parametrize("rows,tile", [(1, 16), (3, 2), (16, 16), (13, 5)])
+@pytest.mark.parametrize("family,suffix", [(ATTN, "_ms"), (GDN, "_ms_v2"), (OUT, "_ms")],
+                         ids=["attn", "gdn_v2", "out"])
+def test_wave_projection_bit_for_bit(family, suffix, rows, tile):
+    name = family["name"] + suffix
+    print(f"[case] {name} rows={rows} tile={tile}", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9200)
+    x = ol.gaussian_bf16(0x9300 + rows, rows * family["k"], 0.0, 1.0)
+    total = sum(family["segments"])
+    strided = family is OUT
+    stride = total + 64 if strided else total
+    out = dev.buffer_from(np.full(rows * stride, 0x7FC0, np.uint16))
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    slot = family["out"] + 1
+    constants = {slot: rows, slot + 1: stride, slot + 2: tile} if strided else {slot: rows, slot + 1: tile}
+    tiles = (rows + tile - 1) // tile
+    ms = run(lambda cb: cb.encode(lib.pipeline(name), bindings, constants, (_groups(family), tiles, 1),
+                                  (family["threads"], 1, 1)))
+    got = out.read(np.uint16).reshape(rows, stride)
+    want = _expected(family, host, x, rows, stride).reshape(rows, stride)
+    assert np.array_equal(got[:, :total], want[:, :total])
+    assert np.all(got[:, total:] == 0x7FC0)
+    print(f"[time] {name} rows={rows} tile={tile}: {ms * 1e3:.1f} us", flush=True)
+
+
+@pytest.mark.parametrize("family,name", [(ATTN, "attn_project_blk"), (GDN, "gdn_project_blk"),
+                                         (OUT, "outproj_blk")], ids=["attn", "gdn", "out"])
+@pytest.mark.parametrize("rows", [1, 37, 130])
+def test_block_projection(family, name, rows):
+    print(f"[case] {name} rows={rows}", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9400)
+    x = ol.gaussian_bf16(0x9500 + rows, rows * family["k"], 0.0, 1.0)
+    total = sum(family["segments"])
+    out = dev.create_buffer(rows * total * 2)
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    slot = family["out"] + 1
+    constants = {slot: rows, slot + 1: family["k"]} if family is OUT else {slot: rows}
+    ms = run(lambda cb: cb.encode(lib.pipeline(name), bindings, constants, (_groups(family), 1, 1),
+                                  (family["threads"], 1, 1)))
+    check_bf16(out.read(np.uint16), _expected(family, host, x, rows), name, ulps=2)
+    print(f"[time] {name} rows={rows}: {ms * 1e3:.1f} us", flush=True)
+
+
+def test_projection_validation():
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, ATTN, 0x9600)
+    bindings[0] = dev.create_buffer(16 * 2048 * 2)
+    bindings[10] = dev.create_buffer(16 * 9216 * 2)
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    ms = lib.pipeline("attn_project_ms")
+    cases = [
+        (bindings, {11: 17, 12: 16}, (2304, 2, 1), 15),     # more rows than a wave holds
+        (bindings, {11: 16, 12: 17}, (2304, 1, 1), 15),     # tile beyond the batch maximum
+        (bindings, {11: 16, 12: 4}, (2304, 3, 1), 15),      # tiles do not cover the rows
+        (bindings, {11: 16, 12: 4}, (2303, 4, 1), 15),      # groups do not cover the output rows
+        ({**bindings, 4: dev.create_buffer(512 * 256 * 4 - 4)}, {11: 4, 12: 4}, (2304, 1, 1), 10),
+        ({**bindings, 10: dev.create_buffer(4 * 9216 * 2 - 2)}, {11: 4, 12: 4}, (2304, 1, 1), 10),
+        ({**bindings, 0: dev.create_buffer(4 * 2048 * 2 - 2)}, {11: 4, 12: 4}, (2304, 1, 1), 10),
+    ]
+    for buffers, constants, grid, status in cases:
+        with pytest.raises(B.BackendError) as e:
+            cb.encode(ms, buffers, constants, grid, (128, 1, 1))
+        assert e.value.status == status, (constants, grid)
+    host, out_bindings = _family(dev, OUT, 0x9700)
+    out_bindings[0] = dev.create_buffer(4 * 4096 * 2)
+    out_bindings[4] = dev.create_buffer(4 * 2048 * 2)
+    with pytest.raises(B.BackendError) as e:   # output stride below the hidden width
+        cb.encode(lib.pipeline("gdn_outproj_ms"), out_bindings, {5: 4, 6: 2047, 7: 4}, (1024, 1, 1),
+                  (64, 1, 1))
+    assert e.value.status == 8
+    with pytest.raises(B.BackendError) as e:   # input width not a multiple of 512
+        cb.encode(lib.pipeline("outproj_blk"), out_bindings, {5: 4, 6: 4000}, (1024, 1, 1), (64, 1, 1))
+    assert e.value.status == 15
+    assert cb.command_count == 0

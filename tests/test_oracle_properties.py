@@ -486,3 +486,47 @@ def test_rms_only_closed_forms():
     twos = np.full(2048, 0x4000, np.uint16)
     o.tto_rms_only(twos, ones, 1, 2048, out)
     assert (out == 0x3F80).all()
+
+
+def _q4_dequantised(words, scales, biases, k_size):
+    """Plain reading of the format: nibble j of word i is column 8 i + j."""
+    w = np.asarray(words, np.uint32)
+    nib = np.stack([(w >> (4 * j)) & 0xF for j in range(8)], axis=-1).reshape(-1).astype(np.float64)
+    s = np.repeat(F(scales).astype(np.float64), 64)
+    b = np.repeat(F(biases).astype(np.float64), 64)
+    return s * nib + b
+
+
+def test_q4_addressing_and_affine_known_answers():
+    """The packed-nibble known answers of kernel_reference_test.cpp:327-345: all inputs 1.0 but
+    element 1 = 2.0, nibble 10 in the high half of byte 0 (column 1): 20 with unit scale, and
+    2 * 20 + 513 * 0.5 with scale 2 and bias 0.5."""
+    x = np.full(512, 0x3F80, np.uint16); x[1] = 0x4000
+    words = np.zeros(64, np.uint32); words[0] = 0x000000A0
+    ones = np.full(8, 0x3F80, np.uint16); zeros = np.zeros(8, np.uint16)
+    assert o.tto_q4_dot(x, words, ones, zeros, 512) == 20.0
+    twos = np.full(8, 0x4000, np.uint16); halves = np.full(8, 0x3F00, np.uint16)
+    assert o.tto_q4_dot(x, words, twos, halves, 512) == 2.0 * 20.0 + 513.0 * 0.5
+    # every column in turn: only that column's nibble is set, the input is one-hot there
+    for column in (0, 7, 8, 63, 64, 300, 511):
+        x = np.zeros(512, np.uint16); x[column] = 0x4040           # 3.0
+        words = np.zeros(64, np.uint32); words[column // 8] = np.uint32(13 << (4 * (column % 8)))
+        scales = np.zeros(8, np.uint16); scales[column // 64] = 0x3F00   # 0.5 for that group only
+        assert o.tto_q4_dot(x, words, scales, zeros, 512) == 0.5 * 13 * 3.0, column
+
+
+def test_q4_projection_matches_fp64_dequantised_product():
+    rng = np.random.default_rng(2718)
+    rows, k_size, out_rows = 3, 2048, 40
+    x = ol.gaussian_bf16(0x51, rows * k_size, 0.0, 1.0)
+    words = rng.integers(0, 2 ** 32, out_rows * k_size // 8, dtype=np.uint64).astype(np.uint32)
+    scales = BF(rng.uniform(0.002, 0.01, out_rows * k_size // 64).astype(np.float32))
+    biases = BF((-7.5 * F(scales) + rng.normal(0, 1e-3, scales.size)).astype(np.float32))
+    out = np.zeros(rows * 48, np.uint16)
+    o.tto_q4_project(x, k_size, rows, words, scales, biases, k_size, out_rows, out, 48, 4)
+    w = _q4_dequantised(words, scales, biases, k_size).reshape(out_rows, k_size)
+    want = F(x).reshape(rows, k_size).astype(np.float64) @ w.T
+    got = F(out).reshape(rows, 48)[:, :out_rows]
+    assert np.all(out.reshape(rows, 48)[:, out_rows:] == 0)
+    # bf16 output rounding dominates: half a step of the result's magnitude
+    assert np.all(np.abs(got - want) <= np.maximum(np.abs(want) * 2.0 ** -8, 1e-4))

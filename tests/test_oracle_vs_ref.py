@@ -107,3 +107,24 @@ def test_residual_sums(kind):
     o.tto_add_bf16(a, b, n, got)
     r.ref_residual_sums(a, b, n, want)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("k_size", [512, 2048, 4096])
+def test_q4_dot(k_size):
+    """tto_q4_dot against q4_dot_reference in the fused order (kernel_reference.cpp:388-443),
+    with the operands of the reference's own trial loop (banded bf16, raw generator words;
+    kernel_reference_test.cpp:163-183) and with realistic magnitudes."""
+    rng = np.random.default_rng(k_size)
+    for trial in range(40):
+        if trial % 2 == 0:
+            x = ol.banded_bf16(0x4D00 + trial, k_size)
+            scales = ol.banded_bf16(0x4E00 + trial, k_size // 64)
+            biases = ol.banded_bf16(0x4F00 + trial, k_size // 64)
+        else:
+            x = ol.gaussian_bf16(0x4D00 + trial, k_size, 0.0, 1.0)
+            scales = ol.f32_to_bf16(rng.uniform(0.001, 0.02, k_size // 64).astype(np.float32))
+            biases = ol.f32_to_bf16((-8.0 * rng.uniform(0.001, 0.02, k_size // 64)).astype(np.float32))
+        words = rng.integers(0, 2 ** 32, k_size // 8, dtype=np.uint64).astype(np.uint32)
+        got = np.float32(o.tto_q4_dot(x, words, scales, biases, k_size))
+        want = np.float32(r.ref_q4_dot(x, words, scales, biases, k_size))
+        assert got.view(np.uint32) == want.view(np.uint32) or (np.isnan(got) and np.isnan(want)), trial
