@@ -70,7 +70,10 @@ struct Q4Projection {
 };
 
 // grid (ceil(out_rows / 8), ceil(rows / row_tile)) x 256: half wave h of a workgroup
-// owns output row 8 * blockIdx.x + h for the tile's input rows.
+// owns output row 8 * blockIdx.x + h for the tile's input rows.  kBlocks = k_size / 512:
+// all of the row's nibbles, scales and biases are requested before the first is used, so
+// one row keeps kBlocks loads per lane in flight instead of one.
+template <uint32_t kBlocks>
 __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
     const uint32_t lane = threadIdx.x & 31;
     const uint32_t n = blockIdx.x * 8 + (threadIdx.x >> 5);
@@ -78,32 +81,39 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
     uint32_t segment = 0;
     while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
     const uint32_t local = n - p.first_row[segment];
-    const uint32_t* words = p.words[segment] + static_cast<uint64_t>(local) * (p.k_size / 8);
-    const uint16_t* scales = p.scales[segment] + static_cast<uint64_t>(local) * (p.k_size / kQ4Group);
-    const uint16_t* biases = p.biases[segment] + static_cast<uint64_t>(local) * (p.k_size / kQ4Group);
+    const uint32_t* words = p.words[segment] + static_cast<uint64_t>(local) * (kBlocks * 64);
+    const uint16_t* scales = p.scales[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
+    const uint16_t* biases = p.biases[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
     const uint32_t row_base = blockIdx.y * p.row_tile;
     const uint32_t tile_rows = min(p.row_tile, p.rows - row_base);
-    const uint16_t* x0 = p.input + static_cast<uint64_t>(row_base) * p.input_stride;
+    const uint16_t* x0 = p.input + static_cast<uint64_t>(row_base) * p.input_stride + lane * 16;
 
+    u32x2 packed[kBlocks];
+    uint16_t scale_bits[kBlocks], bias_bits[kBlocks];
+#pragma unroll
+    for (uint32_t b = 0; b < kBlocks; ++b) {
+        // four 16-bit words = this lane's 16 nibbles of block b
+        packed[b] = *reinterpret_cast<const u32x2*>(words + b * 64 + lane * 2);
+        scale_bits[b] = scales[b * 8 + (lane >> 2)];
+        bias_bits[b] = biases[b * 8 + (lane >> 2)];
+    }
     float acc[kQ4BatchRowsMax];
 #pragma unroll
     for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) acc[r] = 0.0f;
-    for (uint32_t k = 0; k < p.k_size; k += kQ4Block) {
-        // four 16-bit words = this lane's 16 nibbles; masked, never shifted
-        const u32x2 packed = *reinterpret_cast<const u32x2*>(words + (k >> 3) + lane * 2);
-        float wq[16];
+#pragma unroll
+    for (uint32_t b = 0; b < kBlocks; ++b) {
+        float wq[16];   // masked, never shifted
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
-            const uint32_t word = (i & 1) ? (packed[i >> 1] >> 16) : (packed[i >> 1] & 0xFFFFu);
+            const uint32_t word = (i & 1) ? (packed[b][i >> 1] >> 16) : (packed[b][i >> 1] & 0xFFFFu);
             wq[i * 4] = static_cast<float>(word & 0x000Fu);
             wq[i * 4 + 1] = static_cast<float>(word & 0x00F0u);
             wq[i * 4 + 2] = static_cast<float>(word & 0x0F00u);
             wq[i * 4 + 3] = static_cast<float>(word & 0xF000u);
         }
-        const uint32_t group = (k >> 6) + (lane >> 2);
-        const float scale = widen(scales[group]);
-        const float bias = widen(biases[group]);
-        const uint16_t* xk = x0 + k + lane * 16;
+        const float scale = widen(scale_bits[b]);
+        const float bias = widen(bias_bits[b]);
+        const uint16_t* xk = x0 + b * kQ4Block;
 #pragma unroll
         for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
             if (r < tile_rows) {
@@ -137,10 +147,304 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
     }
 }
 
+// 0 when the width has no instantiation
 int32_t launch_rows(const Q4Projection& p, hipStream_t stream) {
     const uint32_t out_rows = p.first_row[p.segments];
-    hipLaunchKernelGGL(q4_rows_kernel, dim3((out_rows + 7) / 8, (p.rows + p.row_tile - 1) / p.row_tile),
-                       dim3(256), 0, stream, p);
+    const dim3 grid((out_rows + 7) / 8, (p.rows + p.row_tile - 1) / p.row_tile);
+    switch (p.k_size / kQ4Block) {
+    case 4: hipLaunchKernelGGL(q4_rows_kernel<4>, grid, dim3(256), 0, stream, p); break;
+    case 8: hipLaunchKernelGGL(q4_rows_kernel<8>, grid, dim3(256), 0, stream, p); break;
+    default: return TT_CMD_INVALID_DISPATCH_EXTENT;
+    }
+    return TT_OK;
+}
+
+// ------------------------------------------------------------ block kernel ---
+//
+// out[m][n] = sum_g scale[n][g] * (sum_{k in g} x[m][k] q[n][k]) + bias[n][g] * xs[m][g],
+// xs[m][g] = sum_{k in g} x[m][k].  A workgroup of eight waves owns 128 output rows (n) x
+// 256 input rows (m) and walks K one group (64 columns) at a time through three stages:
+//   * x goes from global memory straight into LDS (no registers), requested two groups
+//     ahead; the nibbles are requested two groups ahead into registers, unpacked to exact
+//     bf16 integers 0..15 and written beside it with the group's 128 scales.  Rows are 128
+//     B without padding; 16-byte piece p of row r sits in slot p ^ (r & 7), which keeps the
+//     16-byte fragment reads of sixteen consecutive rows free of bank conflicts.
+//   * each wave multiplies a 64 x 64 part as 4 x 4 tiles of v_mfma_f32_16x16x32_bf16 (n
+//     along the rows of the result, so a lane ends up with four consecutive n of one m:
+//     8-byte stores), two MFMAs per tile and group from a zero accumulator, then
+//     acc += scale[n] * partial in fp32.
+//   * xs comes from the same MFMA unit (a ones operand against the x fragments), is split
+//     into bf16 hi + lo and, once every eight groups, multiplied with the eight biases by
+//     one v_mfma_f32_16x16x16_bf16 per tile (slots: 8 x hi, 8 x lo against the biases twice).
+constexpr uint32_t kBlockN = 128;                    // output rows of a workgroup tile
+constexpr uint32_t kBlockM = 256;                    // input rows of a workgroup tile
+constexpr uint32_t kBlockThreads = 512;
+constexpr uint32_t kStages = 3;                      // of what arrives from global memory
+constexpr uint32_t kRowBytes = 128;                  // one group of one row: 64 bf16
+constexpr uint32_t kXStageBytes = kBlockM * kRowBytes;                   // 32768
+constexpr uint32_t kWordStageBytes = kBlockN * 32;                       // 8 words per row
+constexpr uint32_t kScaleStageBytes = kBlockN * 4;                       // a pair of groups per row
+constexpr uint32_t kArrivalBytes = kXStageBytes + kWordStageBytes + kScaleStageBytes;  // 37376
+constexpr uint32_t kQStageBytes = kBlockN * kRowBytes;                   // unpacked: 16384, two of them
+constexpr uint32_t kQBase = kStages * kArrivalBytes;
+constexpr uint32_t kGroupSumBase = kQBase + 2 * kQStageBytes;
+constexpr uint32_t kGroupSumBytes = kBlockM * 16 * 2;                    // [m][8 hi, 8 lo] bf16
+constexpr uint32_t kBlockLdsBytes = kGroupSumBase + kGroupSumBytes;      // 153088
+constexpr uint32_t kTransfersPerGroup = 7;           // per wave: 4 x, 2 words, 1 scales
+static_assert(kBlockLdsBytes <= 160 * 1024, "one workgroup per compute unit");
+
+typedef __attribute__((ext_vector_type(4))) short bf16x4_bits;
+
+// eight nibbles of `word` -> eight bf16 integers (exact), low nibble first
+__device__ __forceinline__ u32x4 unpack_nibbles(uint32_t word) {
+    const uint32_t even = word & 0x0F0F0F0Fu;         // nibbles 0, 2, 4, 6 in bytes 0..3
+    const uint32_t odd = (word >> 4) & 0x0F0F0F0Fu;   // nibbles 1, 3, 5, 7
+    u32x4 out;
+    // a small integer is exact in bf16: the upper half of its fp32 pattern
+    out[0] = (__float_as_uint(static_cast<float>(even & 0xFFu)) >> 16) |
+             (__float_as_uint(static_cast<float>(odd & 0xFFu)) & 0xFFFF0000u);
+    out[1] = (__float_as_uint(static_cast<float>((even >> 8) & 0xFFu)) >> 16) |
+             (__float_as_uint(static_cast<float>((odd >> 8) & 0xFFu)) & 0xFFFF0000u);
+    out[2] = (__float_as_uint(static_cast<float>((even >> 16) & 0xFFu)) >> 16) |
+             (__float_as_uint(static_cast<float>((odd >> 16) & 0xFFu)) & 0xFFFF0000u);
+    out[3] = (__float_as_uint(static_cast<float>(even >> 24)) >> 16) |
+             (__float_as_uint(static_cast<float>(odd >> 24)) & 0xFFFF0000u);
+    return out;
+}
+
+__device__ __forceinline__ uint16_t truncate16(float v) {
+    return static_cast<uint16_t>(__float_as_uint(v) >> 16);
+}
+
+// Global memory -> LDS without passing through registers: lane l's 16 bytes land at
+// lds_address + 16 l.  Issued as assembly so that the only waits are the ones written
+// below; M0 is used for nothing else in this kernel.
+__device__ __forceinline__ void transfer_to_lds(const uint8_t* base, uint32_t offset,
+                                                uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(offset), "s"(base)
+                 : "memory");
+}
+
+// the same for 4 bytes per lane at an address of the lane's own: lands at lds_address + 4 l
+__device__ __forceinline__ void transfer_dword_to_lds(const void* address, uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(address)
+                 : "memory");
+}
+
+__global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t t = threadIdx.x;
+    const uint32_t lane = t & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t i16 = lane & 15, g = lane >> 4;
+    const uint32_t out_rows = p.first_row[p.segments];
+    const uint32_t n0 = blockIdx.x * kBlockN, m0 = blockIdx.y * kBlockM;
+    const uint32_t groups = p.k_size / kQ4Group;
+    const uint32_t lds_base = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
+
+    // which weight matrix a global output row lives in
+    auto locate = [&](uint32_t n, const uint32_t*& words, const uint16_t*& scales,
+                      const uint16_t*& biases) {
+        uint32_t segment = 0;
+        while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
+        const uint64_t local = n - p.first_row[segment];
+        words = p.words[segment] + local * (p.k_size / 8);
+        scales = p.scales[segment] + local * groups;
+        biases = p.biases[segment] + local * groups;
+    };
+
+    // ---- staging roles
+    // x: transfer j of wave w fills rows 32 w + 8 j .. + 7; lane l lands in row + (l >> 3),
+    // slot l & 7, so it fetches piece (l & 7) ^ (l >> 3) of that row
+    const uint8_t* x_base = reinterpret_cast<const uint8_t*>(p.input);
+    uint32_t x_offset[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t row = min(m0 + 32 * wave + 8 * j + (lane >> 3), p.rows - 1);
+        x_offset[j] = static_cast<uint32_t>(row * p.input_stride * 2) + (((lane & 7) ^ (lane >> 3)) * 16);
+    }
+    // words: transfer i of wave w fills rows 16 w + 8 i .. + 7, eight words each; the same
+    // wave unpacks them (thread t: words 2 (t & 3), 2 (t & 3) + 1 of row t >> 2), so its own
+    // wait covers them
+    const uint32_t* word_source[2];
+#pragma unroll
+    for (uint32_t i = 0; i < 2; ++i) {
+        const uint32_t* w_row;
+        const uint16_t *unused_scales, *unused_bias;
+        locate(min(n0 + 16 * wave + 8 * i + (lane >> 3), out_rows - 1), w_row, unused_scales,
+               unused_bias);
+        word_source[i] = w_row + (lane & 7);
+    }
+    // scales: one dword (an even group and the next) per row; waves of equal parity fetch the
+    // same 64 rows, which keeps every wave's transfer count the same
+    const uint16_t* scale_source;
+    {
+        const uint32_t* unused_words;
+        const uint16_t* unused_bias;
+        locate(min(n0 + 64 * (wave & 1) + lane, out_rows - 1), unused_words, scale_source, unused_bias);
+    }
+    const uint32_t q_row = t >> 2, q_quarter = t & 3;
+    const uint32_t q_slot0 = q_row * kRowBytes + (((2 * q_quarter) ^ (q_row & 7)) * 16);
+    const uint32_t q_slot1 = q_row * kRowBytes + (((2 * q_quarter + 1) ^ (q_row & 7)) * 16);
+
+    auto request = [&](uint32_t group) {
+        const uint32_t stage = lds_base + (group % kStages) * kArrivalBytes;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            transfer_to_lds(x_base, x_offset[j] + group * kRowBytes,
+                            stage + (32 * wave + 8 * j) * kRowBytes);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            transfer_dword_to_lds(word_source[i] + group * 8,
+                                  stage + kXStageBytes + (16 * wave + 8 * i) * 32);
+        }
+        transfer_dword_to_lds(scale_source + (group & ~1u),
+                              stage + kXStageBytes + kWordStageBytes + 64 * (wave & 1) * 4);
+    };
+    auto commit = [&](uint32_t group) {
+        const uint8_t* arrived = lds + (group % kStages) * kArrivalBytes + kXStageBytes;
+        const u32x2 words = *reinterpret_cast<const u32x2*>(arrived + q_row * 32 + q_quarter * 8);
+        uint8_t* stage = lds + kQBase + (group & 1) * kQStageBytes;
+        *reinterpret_cast<u32x4*>(stage + q_slot0) = unpack_nibbles(words[0]);
+        *reinterpret_cast<u32x4*>(stage + q_slot1) = unpack_nibbles(words[1]);
+    };
+
+    // ---- multiply role: wave (mq, nh) owns m in [64 mq, +64), n in [64 nh, +64) of the tile
+    const uint32_t nh = wave & 1, mq = wave >> 1;
+    // fragment of (row, 32-column step): piece 4 step + g, stored at slot piece ^ (row & 7)
+    const uint32_t piece_offset[2] = {((g ^ (i16 & 7)) * 16), (((4 + g) ^ (i16 & 7)) * 16)};
+    const uint32_t x_frag = (64 * mq + i16) * kRowBytes;
+    const uint32_t q_frag = (64 * nh + i16) * kRowBytes;
+    uint16_t* group_sums = reinterpret_cast<uint16_t*>(lds + kGroupSumBase);
+    f32x4 acc[4][4];
+#pragma unroll
+    for (uint32_t tn = 0; tn < 4; ++tn) {
+#pragma unroll
+        for (uint32_t tm = 0; tm < 4; ++tm) acc[tn][tm] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    bf16x8 ones;
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
+    const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto add_bias_terms = [&](uint32_t first_group) {
+        // slots 0..7 pair with hi, 8..15 with lo: lanes g and g + 2 hold the same biases
+        bf16x4_bits biases[4];
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+            const uint32_t* unused_words;
+            const uint16_t *unused_scales, *bias_row;
+            locate(min(n0 + 64 * nh + 16 * tn + i16, out_rows - 1), unused_words, unused_scales,
+                   bias_row);
+            biases[tn] = *reinterpret_cast<const bf16x4_bits*>(bias_row + first_group + 4 * (g & 1));
+        }
+#pragma unroll
+        for (uint32_t tm = 0; tm < 4; ++tm) {
+            const bf16x4_bits sums = *reinterpret_cast<const bf16x4_bits*>(
+                group_sums + (64 * mq + 16 * tm + i16) * 16 + 4 * g);
+#pragma unroll
+            for (uint32_t tn = 0; tn < 4; ++tn) {
+                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(biases[tn], sums,
+                                                                        acc[tn][tm], 0, 0, 0);
+            }
+        }
+    };
+
+    request(0);
+    request(1);   // the group count is a multiple of 8
+    for (uint32_t group = 0; group < groups; ++group) {
+        // this group's transfers have landed once at most the next group's are in flight
+        if (group + 1 < groups) {
+            __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        commit(group);
+        __syncthreads();
+        if (group + 2 < groups) request(group + 2);
+        const uint8_t* stage = lds + (group % kStages) * kArrivalBytes;
+        const uint8_t* q_stage = lds + kQBase + (group & 1) * kQStageBytes;
+        bf16x8 xf[4][2], qf[4][2];
+#pragma unroll
+        for (uint32_t tile = 0; tile < 4; ++tile) {
+#pragma unroll
+            for (uint32_t step = 0; step < 2; ++step) {
+                xf[tile][step] = *reinterpret_cast<const bf16x8*>(
+                    stage + x_frag + tile * 16 * kRowBytes + piece_offset[step]);
+                qf[tile][step] = *reinterpret_cast<const bf16x8*>(
+                    q_stage + q_frag + tile * 16 * kRowBytes + piece_offset[step]);
+            }
+        }
+        // group sums of two of this wave's four m tiles (the other n half takes the others)
+#pragma unroll
+        for (uint32_t tm = 0; tm < 4; ++tm) {
+            if ((tm >> 1) != nh) continue;   // wave-uniform; keeps the fragment index static
+            f32x4 sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xf[tm][0], zero, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xf[tm][1], sum, 0, 0, 0);
+            if (g == 0) {
+                const uint16_t hi = truncate16(sum[0]);
+                const uint16_t lo = truncate16(sum[0] - widen(hi));
+                uint16_t* slot = group_sums + (64 * mq + 16 * tm + i16) * 16 + (group & 7);
+                slot[0] = hi;
+                slot[8] = lo;
+            }
+        }
+        const uint32_t* scale_pairs =
+            reinterpret_cast<const uint32_t*>(stage + kXStageBytes + kWordStageBytes);
+        const bool odd_group = (group & 1) != 0;
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+            const u32x4 pairs = *reinterpret_cast<const u32x4*>(scale_pairs + 64 * nh + 16 * tn + 4 * g);
+            f32x4 scale;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                scale[j] = __uint_as_float(odd_group ? (pairs[j] & 0xFFFF0000u) : (pairs[j] << 16));
+            }
+#pragma unroll
+            for (uint32_t tm = 0; tm < 4; ++tm) {
+                f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[tn][0], xf[tm][0], zero, 0, 0, 0);
+                part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[tn][1], xf[tm][1], part, 0, 0, 0);
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) acc[tn][tm][j] = fmaf(scale[j], part[j], acc[tn][tm][j]);
+            }
+        }
+        if ((group & 7) == 7) {
+            __syncthreads();   // all eight groups' sums are in place
+            add_bias_terms(group - 7);
+        }
+    }
+
+    // ---- store: lane holds n = 4 g .. 4 g + 3 of column m = i16 of every tile
+#pragma unroll
+    for (uint32_t tm = 0; tm < 4; ++tm) {
+        const uint32_t m = m0 + 64 * mq + 16 * tm + i16;
+        if (m >= p.rows) continue;
+        uint16_t* out_row = p.output + static_cast<uint64_t>(m) * p.output_stride;
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+            const uint32_t n = n0 + 64 * nh + 16 * tn + 4 * g;
+            if (n >= out_rows) continue;
+            u32x2 packed;
+            packed[0] = static_cast<uint32_t>(store16(acc[tn][tm][0])) |
+                        (static_cast<uint32_t>(store16(acc[tn][tm][1])) << 16);
+            packed[1] = static_cast<uint32_t>(store16(acc[tn][tm][2])) |
+                        (static_cast<uint32_t>(store16(acc[tn][tm][3])) << 16);
+            *reinterpret_cast<u32x2*>(out_row + n) = packed;
+        }
+    }
+}
+
+int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
+    const uint32_t out_rows = p.first_row[p.segments];
+    hipLaunchKernelGGL(q4_block_kernel,
+                       dim3((out_rows + kBlockN - 1) / kBlockN, (p.rows + kBlockM - 1) / kBlockM),
+                       dim3(kBlockThreads), kBlockLdsBytes, stream, p);
     return TT_OK;
 }
 
@@ -209,6 +513,15 @@ int32_t finish(Args& a, const Grid& g, hipStream_t stream, bool validate_only, c
     p.output = a.buffer<uint16_t>(
         f.out_slot, (static_cast<uint64_t>(p.rows - 1) * p.output_stride + out_rows) * 2);
     if (a.status != TT_OK || validate_only) return a.status;
+    // a handful of rows is a weight-streaming problem: the exact rows kernel; a block
+    // is a matrix product: MFMA
+    if (p.rows > kQ4BatchRowsMax) {
+        // the block kernel addresses x with 32-bit byte offsets
+        if (static_cast<uint64_t>(p.rows) * p.input_stride * 2 >= (1ull << 32)) {
+            return TT_CMD_INVALID_DISPATCH_EXTENT;
+        }
+        return launch_block(p, stream);
+    }
     return launch_rows(p, stream);
 }
 
@@ -247,7 +560,8 @@ int32_t project_block(const Bindings& b, const Grid& g, hipStream_t stream, bool
     Q4Projection p{};
     p.rows = a.constant(f.out_slot + 1);
     const uint32_t k_size = variable_width ? a.constant(f.out_slot + 2) : f.k_size;
-    a.require(p.rows >= 1 && k_size >= kQ4Block && k_size % kQ4Block == 0 && k_size <= 8192,
+    // the two input widths of the model: hidden (2048) and the attention / value width (4096)
+    a.require(p.rows >= 1 && (k_size == kHidden || k_size == kGdnValueValues),
               TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK) return a.status;
     p.row_tile = kQ4BatchRowsMax;
@@ -299,6 +613,12 @@ int32_t op_outproj_blk(const Bindings& b, const Grid& g, hipStream_t s, bool v) 
 }  // namespace
 
 #if !defined(__HIP_DEVICE_COMPILE__)  // host-side table of launchers
+bool prepare_q4_kernels() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(q4_block_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kBlockLdsBytes) == hipSuccess;
+}
+
 const KernelDesc kQ4ProjectKernels[] = {
     {"attn_project", op_attn_project},
     {"attn_project_ms", op_attn_project_ms},

@@ -91,6 +91,7 @@ int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream
 // library is created, so it never runs inside a stream capture.
 bool prepare_decode_kernels();
 bool prepare_prefill_kernels();
+bool prepare_q4_kernels();
 
 extern const KernelDesc kAttentionDecodeKernels[];
 extern const uint32_t kAttentionDecodeKernelCount;
