@@ -1,8 +1,9 @@
 """A stubbed hybrid stack around the attention family, for stacked parity runs and
 context sweeps: `layers` layers in the G,G,G,A pattern at hidden 2048, with the
-reference's Q4/MoE arithmetic replaced by random bf16 dense projections
-(hidden -> 12352 / 9216 in, 4096 -> hidden out) so that only the attention family
-does model-shaped work.  Per layer:
+reference's MoE block left out and its projections (hidden -> 12352 / 9216 in,
+4096 -> hidden out) either as random bf16 dense matrices or, with quantized weights,
+as the reference's affine 4-bit projections (attn_project / gdn_project / gdn_outproj
+and their _ms / _blk forms).  Per layer:
 
     n = rms_only(x, input_norm);  p = dense(n, W_in)
     a = GatedDeltaNet(p) | FullAttention(p);  x = x + dense(a, W_out)
@@ -37,8 +38,23 @@ def _bf16(a):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-def make_weights(layers, vocab, seed):
-    """Host-side weights as uint16 bf16 arrays; scales keep the residual stream O(1)."""
+ATTN_SEGMENTS = (8192, 512, 512)        # query + gate, key, value rows of the in-projection
+GDN_SEGMENTS = (8192, 4096, 32, 32)     # qkv, z, b, a rows
+
+
+def quantize_random(rng, rows, k, sigma):
+    """A random affine 4-bit matrix (group 64) whose entries have standard deviation
+    about `sigma`: nibbles uniform in 0..15 (standard deviation 4.61 around 7.5), one
+    bf16 scale and bias per 64 columns.  Returns (words u32, scales bf16, biases bf16)."""
+    words = rng.integers(0, 2 ** 32, rows * k // 8, dtype=np.uint64).astype(np.uint32)
+    scale = (sigma / 4.61) * rng.uniform(0.8, 1.2, rows * k // 64).astype(np.float32)
+    return words, _bf16(scale), _bf16(-7.5 * scale)
+
+
+def make_weights(layers, vocab, seed, quantized=False):
+    """Host-side weights as uint16 bf16 arrays; scales keep the residual stream O(1).
+    With `quantized`, the in- and out-projections are affine 4-bit: w["in_q4"] holds one
+    (words, scales, biases) triple per matrix of the projection, w["out_q4"] one triple."""
     rng = np.random.default_rng(seed)
 
     def normal(n, sigma):
@@ -60,6 +76,11 @@ def make_weights(layers, vocab, seed):
             w["w_in"] = normal(ATTN_PROJ * HIDDEN, HIDDEN ** -0.5)
             w["q_norm"] = _bf16(1.0 + 0.1 * rng.standard_normal(256))
             w["k_norm"] = _bf16(1.0 + 0.1 * rng.standard_normal(256))
+        if quantized:
+            segments = GDN_SEGMENTS if kind == "G" else ATTN_SEGMENTS
+            w["in_q4"] = [quantize_random(rng, rows, HIDDEN, HIDDEN ** -0.5) for rows in segments]
+            w["out_q4"] = quantize_random(rng, HIDDEN, 4096, 0.5 * 4096 ** -0.5)
+            del w["w_in"], w["w_out"]
         out["layers"].append(w)
     return out
 
@@ -93,8 +114,13 @@ class StubStack:
         self.swapped = [False] * lanes      # GDN ping-pong phase per lane
         stripe = 2 * capacity * 256
         for w in weights["layers"]:
-            layer = {"kind": w["kind"], "input_norm": up(w["input_norm"]), "w_in": up(w["w_in"]),
-                     "w_out": up(w["w_out"]), "table": dev.create_buffer(256)}
+            layer = {"kind": w["kind"], "input_norm": up(w["input_norm"]),
+                     "table": dev.create_buffer(256)}
+            if "in_q4" in w:
+                layer["in_q4"] = [tuple(up(part) for part in matrix) for matrix in w["in_q4"]]
+                layer["out_q4"] = tuple(up(part) for part in w["out_q4"])
+            else:
+                layer["w_in"], layer["w_out"] = up(w["w_in"]), up(w["w_out"])
             if w["kind"] == "G":
                 for name in ("conv_w", "a_log", "dt_bias", "norm_w"):
                     layer[name] = up(w[name])
@@ -143,6 +169,43 @@ class StubStack:
                   ((n + 63) // 64, (rows + 15) // 16), (256,))
         cb.barrier()
 
+    def _project_in(self, cb, layer, rows, block):
+        """normed -> proj: the layer's input projection (a decode wave or a block)."""
+        gated = layer["kind"] == "G"
+        width = GDN_PROJ if gated else ATTN_PROJ
+        if "in_q4" not in layer:
+            self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, width)
+            return
+        name = "gdn_project" if gated else "attn_project"
+        bindings = {0: self.normed}
+        for index, matrix in enumerate(layer["in_q4"]):
+            for part in range(3):
+                bindings[1 + 3 * index + part] = matrix[part]
+        out = 1 + 3 * len(layer["in_q4"])
+        bindings[out] = self.proj
+        if block:
+            cb.encode(self.lib.pipeline(name + "_blk"), bindings, {out + 1: rows},
+                      ((width + 3) // 4,), (128,))
+        else:
+            cb.encode(self.lib.pipeline(name + "_ms"), bindings, {out + 1: rows, out + 2: 16},
+                      ((width + 3) // 4, 1), (128,))
+        cb.barrier()
+
+    def _project_out(self, cb, layer, rows, block):
+        """mixed -> delta: the projection back to the hidden width."""
+        if "out_q4" not in layer:
+            self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
+            return
+        words, scales, biases = layer["out_q4"]
+        bindings = {0: self.mixed, 1: words, 2: scales, 3: biases, 4: self.delta}
+        if block:
+            cb.encode(self.lib.pipeline("outproj_blk"), bindings, {5: rows, 6: 4096},
+                      (HIDDEN // 2,), (64,))
+        else:
+            cb.encode(self.lib.pipeline("gdn_outproj_ms"), bindings, {5: rows, 6: HIDDEN, 7: 16},
+                      (HIDDEN // 2, 1), (64,))
+        cb.barrier()
+
     def _rms(self, cb, x, w, out, rows):
         cb.encode(self.lib.pipeline("rms_only_ms"), {0: x, 1: w, 2: out}, {3: HIDDEN, 4: HIDDEN},
                   (1, rows), (HIDDEN // 4,))
@@ -169,14 +232,13 @@ class StubStack:
         P, rows = self.lib.pipeline, self.lanes
         self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
         for index, layer in enumerate(self.layers):
+            self._project_in(cb, layer, rows, block=False)
             if layer["kind"] == "G":
-                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
                 cb.encode(P("gdn_decode_fused_ms"),
                           {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
                            4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: self.mixed,
                            8: layer["table"]}, {9: GDN_PROJ, 10: 4096}, (32, rows), (512,))
             else:
-                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, ATTN_PROJ)
                 cb.encode(P("attn_qk_rope_ms"),
                           {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,
                            5: layer["keys"], 6: layer["values"], 8: layer["table"]},
@@ -192,7 +254,7 @@ class StubStack:
                           {0: self.partials, 1: self.gate, 2: layer["table"], 3: self.mixed},
                           {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
             cb.barrier()
-            self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
+            self._project_out(cb, layer, rows, block=False)
             self._residual_and_norm(cb, rows, index)
         if with_head:
             self._head(cb, rows)
@@ -216,8 +278,8 @@ class StubStack:
         plane_in, plane_out = self._gdn_planes(lane)
         self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
         for index, layer in enumerate(self.layers):
+            self._project_in(cb, layer, rows, block=True)
             if layer["kind"] == "G":
-                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, GDN_PROJ)
                 conv_in = (layer["conv"], plane_in * CONV_ELEMS * 2)
                 conv_out = (layer["conv"], plane_out * CONV_ELEMS * 2)
                 rec_in = (layer["rec"], plane_in * REC_ELEMS * 4)
@@ -241,7 +303,6 @@ class StubStack:
                 cb.encode(P("gdn_gate_norm_blk"), {0: self.y, 1: self.z, 2: layer["norm_w"], 3: self.mixed},
                           {}, (32, rows), (128,))
             else:
-                self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, ATTN_PROJ)
                 keys = (layer["keys"], lane * stripe_bytes)
                 values = (layer["values"], lane * stripe_bytes)
                 cb.encode(P("attn_qk_rope_blk"),
@@ -253,7 +314,7 @@ class StubStack:
                           {5: base + rows, 6: self.capacity, 7: rows, 8: base},
                           (16, (rows + 15) // 16), (256,))
             cb.barrier()
-            self._dense(cb, self.mixed, layer["w_out"], self.delta, rows, 4096, HIDDEN)
+            self._project_out(cb, layer, rows, block=True)
             self._residual_and_norm(cb, rows, index)
         if with_head:
             self._head(cb, rows)

@@ -4,6 +4,7 @@ the attention-family kernels are counted (per-command device time); the stand-in
 projections, norms and residual sums run but are reported separately.
 
     python -m tatara_amd.sweep [--layers 40] [--decode 1024,4096,...] [--prefill 4096,32768]
+                               [--quantized]   (4-bit projections instead of dense bf16)
 prints one JSON line per measured point and a closing summary line."""
 import argparse
 import json
@@ -14,7 +15,9 @@ import numpy as np
 from . import backend as B
 from . import stack as S
 
-STUB_KERNELS = {"rms_only", "rms_only_ms", "residual_rms_ms", "dense_bf16", "add_bf16"}
+STUB_KERNELS = {"rms_only", "rms_only_ms", "residual_rms_ms", "dense_bf16", "add_bf16",
+                "attn_project_ms", "gdn_project_ms", "gdn_outproj_ms", "attn_project_blk",
+                "gdn_project_blk", "outproj_blk"}
 
 
 def _family_ms(times):
@@ -81,11 +84,12 @@ def main(argv=None):
     ap.add_argument("--decode", default="1024,4096,16384,32768,65536,100000")
     ap.add_argument("--prefill", default="4096,32768")
     ap.add_argument("--lanes", default="1,4")
+    ap.add_argument("--quantized", action="store_true")
     args = ap.parse_args(argv)
     dev = B.Device()
     queue = dev.create_queue()
     lib = dev.create_library()
-    weights = S.make_weights(args.layers, 1024, 0x5EE9)
+    weights = S.make_weights(args.layers, 1024, 0x5EE9, quantized=args.quantized)
     points = []
     for lanes in [int(v) for v in args.lanes.split(",") if v]:
         for context in [int(v) for v in args.decode.split(",") if v]:

@@ -3,7 +3,8 @@ hidden 2048, random bf16 dense projections in place of the Q4/MoE arithmetic) on
 the GPU against the same stack evaluated with the CPU checker: block prefill of two
 lanes with ragged lengths, then greedy decode waves of both lanes through the
 pooled-state operators.  Judged by greedy argmax agreement on the final logits at
-every step.  The per-operator tolerance (max-abs 2e-2, mean-abs 2e-3) is held by
+every step (where the checker's own top two are closer than two bf16 steps, the GPU may
+pick the other of the two; the run continues with the checker's token).  The per-operator tolerance (max-abs 2e-2, mean-abs 2e-3) is held by
 the single-layer tests; forty layers of bf16 re-rounding put the two evaluations of
 the final logits (bf16, one step = 1.6e-2 at |x| in [2, 4)) a step or two apart, so
 here the logits only have to stay within a loose sanity band."""
@@ -33,6 +34,18 @@ class OracleLane:
                 self.state.append({"keys": np.zeros(2 * capacity * 256, np.uint16),
                                    "values": np.zeros(2 * capacity * 256, np.uint16)})
 
+    @staticmethod
+    def _project_in(lw, n, rows, width, p):
+        if "in_q4" not in lw:
+            o.tto_dense_bf16(n, lw["w_in"], rows, 2048, width, p, THREADS)
+            return
+        first = 0
+        for words, scales, biases in lw["in_q4"]:
+            out_rows = scales.size // 32
+            o.tto_q4_project(n, 2048, rows, words, scales, biases, 2048, out_rows, p[first:], width,
+                             THREADS)
+            first += out_rows
+
     def block(self, x, rows):
         """Runs `rows` tokens (x: [rows*2048] bf16); returns logits of every row."""
         x = x.copy()
@@ -41,7 +54,7 @@ class OracleLane:
             o.tto_rms_only(x, lw["input_norm"], rows, 2048, n)
             if lw["kind"] == "G":
                 p = np.zeros(rows * 12352, np.uint16)
-                o.tto_dense_bf16(n, lw["w_in"], rows, 2048, 12352, p, THREADS)
+                self._project_in(lw, n, rows, 12352, p)
                 conv = np.zeros_like(st["conv"]); rec = np.zeros_like(st["rec"])
                 a = np.zeros(rows * 4096, np.uint16)
                 scratch = [np.zeros(rows * 4096, np.uint16) for _ in range(3)]
@@ -50,13 +63,17 @@ class OracleLane:
                 st["conv"], st["rec"] = conv, rec
             else:
                 p = np.zeros(rows * 9216, np.uint16)
-                o.tto_dense_bf16(n, lw["w_in"], rows, 2048, 9216, p, THREADS)
+                self._project_in(lw, n, rows, 9216, p)
                 q = np.zeros(rows * 4096, np.uint16); g = np.zeros_like(q); a = np.zeros_like(q)
                 sel = np.arange(rows, dtype=np.uint32)
                 o.tto_attention_prefill(p, lw["q_norm"], lw["k_norm"], rows, self.context, self.cap,
                                         q, g, st["keys"], st["values"], sel, rows, a, THREADS)
             d = np.zeros(rows * 2048, np.uint16)
-            o.tto_dense_bf16(a, lw["w_out"], rows, 4096, 2048, d, THREADS)
+            if "out_q4" in lw:
+                words, scales, biases = lw["out_q4"]
+                o.tto_q4_project(a, 4096, rows, words, scales, biases, 4096, 2048, d, 2048, THREADS)
+            else:
+                o.tto_dense_bf16(a, lw["w_out"], rows, 4096, 2048, d, THREADS)
             o.tto_add_bf16(x, d, rows * 2048, x)
         self.context += rows
         n = np.zeros(rows * 2048, np.uint16)
@@ -73,15 +90,26 @@ def _compare(step, got, want):
           f"argmax {got.argmax()} / {want.argmax()} top-2 gap {top2[1] - top2[0]:.3e}", flush=True)
     assert np.isfinite(got).all()
     assert err.mean() <= 2e-2 * max(1.0, np.abs(want).max())
-    assert got.argmax() == want.argmax(), step
+    if got.argmax() != want.argmax():
+        # a tie within the noise of the run: the checker itself ranks the GPU's choice no more
+        # than two bf16 steps of the winning logit below its own
+        step16 = 2.0 ** (np.floor(np.log2(max(abs(want.max()), 1e-30))) - 7)
+        margin = want.max() - want[got.argmax()]
+        print(f"[parity] {step}: argmax differs on a margin of {margin:.3e} (bf16 step {step16:.3e})",
+              flush=True)
+        assert margin <= 2 * step16, step
 
 
-def test_stacked_prefill_and_greedy_decode_match_the_checker():
-    print("[case] 40-layer stub stack: prefill 2 lanes + 3 greedy decode waves", flush=True)
+@pytest.mark.parametrize("layers,quantized", [(40, False), (12, True)], ids=["dense40", "q4x12"])
+def test_stacked_prefill_and_greedy_decode_match_the_checker(layers, quantized):
+    """quantized: the projections are the affine 4-bit operators (block forms in the
+    prefill, wave forms in the decode)."""
+    print(f"[case] {layers}-layer stub stack (quantized={quantized}): prefill 2 lanes + 3 greedy "
+          "decode waves", flush=True)
     from tatara_amd import stack as S
     B, dev, queue, lib = gpu()
-    layers, vocab, capacity, lanes = 40, 4096, 128, 2
-    weights = S.make_weights(layers, vocab, 0x57AC)
+    vocab, capacity, lanes = 4096, 128, 2
+    weights = S.make_weights(layers, vocab, 0x57AC, quantized=quantized)
     embed = weights["embed"].reshape(vocab, 2048)
     gpu_stack = S.StubStack(dev, lib, weights, lanes, capacity, vocab, block_rows=64, split_keys=64)
     cpu_lanes = [OracleLane(weights, capacity, vocab) for _ in range(lanes)]
