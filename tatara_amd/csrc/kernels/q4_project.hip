@@ -448,6 +448,101 @@ int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
     return TT_OK;
 }
 
+// ------------------------------------------------------- decode-wave kernel ---
+//
+// The same mathematics as the block kernel for 2..16 input rows (a decode wave), sized for
+// latency: a workgroup owns 16 output rows and all input rows, its waves split K in slices
+// of 512 columns (eight groups each), every operand of a slice is requested before the
+// first is used, and the slices are summed through LDS in a fixed order.  Per group four
+// v_mfma_f32_16x16x16_bf16 multiply the x rows with the unpacked nibbles (lane g of a row
+// owns the group's columns 16 g .. 16 g + 15) and four more, against a ones operand, give
+// the group sums of x; then acc += scale[n] * products + bias[n] * sums in fp32.  The
+// result has n along its columns, so a lane needs one scale and one bias per group, and
+// reads all eight of a slice with two 16-byte loads.
+
+// nibbles 0..3 of the low 16 bits of `half_word` -> four bf16 integers (exact)
+__device__ __forceinline__ bf16x4_bits unpack_four(uint32_t half_word) {
+    const uint32_t even = half_word & 0x0F0Fu;         // nibbles 0, 2 in bytes 0, 1
+    const uint32_t odd = (half_word >> 4) & 0x0F0Fu;   // nibbles 1, 3
+    u32x2 out;
+    out[0] = (__float_as_uint(static_cast<float>(even & 0xFFu)) >> 16) |
+             (__float_as_uint(static_cast<float>(odd & 0xFFu)) & 0xFFFF0000u);
+    out[1] = (__float_as_uint(static_cast<float>(even >> 8)) >> 16) |
+             (__float_as_uint(static_cast<float>(odd >> 8)) & 0xFFFF0000u);
+    return __builtin_bit_cast(bf16x4_bits, out);
+}
+
+template <uint32_t kWaves>   // k_size / 512
+__global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
+    __shared__ float partial[kWaves][4][64];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t i16 = lane & 15, g = lane >> 4;
+    const uint32_t n = blockIdx.x * 16 + i16;   // every matrix has a multiple of 16 rows
+    uint32_t segment = 0;
+    while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
+    const uint64_t local = n - p.first_row[segment];
+    const uint32_t first_group = wave * 8;
+    const uint32_t* words = p.words[segment] + local * (kWaves * 64) + first_group * 8 + 2 * g;
+    const uint16_t* scales = p.scales[segment] + local * (kWaves * 8) + first_group;
+    const uint16_t* biases = p.biases[segment] + local * (kWaves * 8) + first_group;
+    const uint16_t* x_row = p.input + static_cast<uint64_t>(min(i16, p.rows - 1)) * p.input_stride +
+                            first_group * kQ4Group + 16 * g;
+
+    u32x2 q[8];
+    u32x4 x[8][2];
+#pragma unroll
+    for (uint32_t group = 0; group < 8; ++group) {
+        q[group] = *reinterpret_cast<const u32x2*>(words + group * 8);
+        x[group][0] = *reinterpret_cast<const u32x4*>(x_row + group * kQ4Group);
+        x[group][1] = *reinterpret_cast<const u32x4*>(x_row + group * kQ4Group + 8);
+    }
+    const u32x4 scale_bits = *reinterpret_cast<const u32x4*>(scales);
+    const u32x4 bias_bits = *reinterpret_cast<const u32x4*>(biases);
+
+    const bf16x4_bits ones = {0x3F80, 0x3F80, 0x3F80, 0x3F80};
+    const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4 acc = zero;
+#pragma unroll
+    for (uint32_t group = 0; group < 8; ++group) {
+        f32x4 products = zero, sums = zero;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const u32x2 x_bits = {x[group][j >> 1][2 * (j & 1)], x[group][j >> 1][2 * (j & 1) + 1]};
+            const bf16x4_bits xf = __builtin_bit_cast(bf16x4_bits, x_bits);
+            const uint32_t word = q[group][j >> 1];
+            const bf16x4_bits qf = unpack_four((j & 1) ? (word >> 16) : word);
+            products = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xf, qf, products, 0, 0, 0);
+            sums = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xf, ones, sums, 0, 0, 0);
+        }
+        const float scale = widen_half(scale_bits[group >> 1], group & 1);
+        const float bias = widen_half(bias_bits[group >> 1], group & 1);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) acc[i] = fmaf(bias, sums[i], fmaf(scale, products[i], acc[i]));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) partial[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        float total = partial[0][i][lane];
+#pragma unroll
+        for (uint32_t w = 1; w < kWaves; ++w) total += partial[w][i][lane];
+        const uint32_t m = 4 * g + i;   // the result has the input rows along its rows
+        if (m < p.rows) p.output[static_cast<uint64_t>(m) * p.output_stride + n] = store16(total);
+    }
+}
+
+int32_t launch_wave(const Q4Projection& p, hipStream_t stream) {
+    const uint32_t out_rows = p.first_row[p.segments];
+    switch (p.k_size / kQ4Block) {
+    case 4: hipLaunchKernelGGL(q4_wave_kernel<4>, dim3(out_rows / 16), dim3(256), 0, stream, p); break;
+    case 8: hipLaunchKernelGGL(q4_wave_kernel<8>, dim3(out_rows / 16), dim3(512), 0, stream, p); break;
+    default: return TT_CMD_INVALID_DISPATCH_EXTENT;
+    }
+    return TT_OK;
+}
+
 // Binds `count` weight matrices from buffer slots first, first+3, ...: words, scales,
 // biases of each, sized for its rows.
 void bind_segments(Args& a, Q4Projection& p, uint32_t first_slot, const uint32_t* rows,
@@ -502,7 +597,7 @@ static_assert(kOutProject.out_rows() == kHidden && kOutProject.groups() == 1024)
 // Binds input, weights and output once rows / strides / tiling are known, checks the
 // reference's grid (groups, tiles) x threads, and launches.
 int32_t finish(Args& a, const Grid& g, hipStream_t stream, bool validate_only, const Family& f,
-               Q4Projection& p, uint32_t k_size, uint64_t tiles) {
+               Q4Projection& p, uint32_t k_size, uint64_t tiles, bool wave_kernel = false) {
     const uint32_t out_rows = f.out_rows();
     a.require(p.output_stride >= out_rows, TT_CMD_INVALID_BUFFER);
     a.require(grid_is(g, f.groups(), tiles, 1, f.threads, 1, 1), TT_CMD_INVALID_DISPATCH_EXTENT);
@@ -513,6 +608,7 @@ int32_t finish(Args& a, const Grid& g, hipStream_t stream, bool validate_only, c
     p.output = a.buffer<uint16_t>(
         f.out_slot, (static_cast<uint64_t>(p.rows - 1) * p.output_stride + out_rows) * 2);
     if (a.status != TT_OK || validate_only) return a.status;
+    if (wave_kernel) return launch_wave(p, stream);
     // a handful of rows is a weight-streaming problem: the exact rows kernel; a block
     // is a matrix product: MFMA
     if (p.rows > kQ4BatchRowsMax) {
@@ -538,7 +634,7 @@ int32_t project_single(const Bindings& b, const Grid& g, hipStream_t stream, boo
 // rows of a decode wave: c[out+1] rows (1..16), then the output row stride where the
 // operator has one, then the row tile; grid (groups, ceil(rows / tile)) x threads
 int32_t project_tiled(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only,
-                      const Family& f, bool strided_output) {
+                      const Family& f, bool strided_output, bool wave_kernel = false) {
     Args a(b);
     Q4Projection p{};
     p.rows = a.constant(f.out_slot + 1);
@@ -549,7 +645,7 @@ int32_t project_tiled(const Bindings& b, const Grid& g, hipStream_t stream, bool
               TT_CMD_INVALID_DISPATCH_EXTENT);
     if (a.status != TT_OK) return a.status;
     return finish(a, g, stream, validate_only, f, p, f.k_size,
-                  (p.rows + p.row_tile - 1) / p.row_tile);
+                  (p.rows + p.row_tile - 1) / p.row_tile, wave_kernel);
 }
 
 // a block of consecutive tokens: c[out+1] rows, then the input width where the
@@ -605,6 +701,18 @@ int32_t op_gdn_outproj(const Bindings& b, const Grid& g, hipStream_t s, bool v) 
 int32_t op_gdn_outproj_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
     return project_tiled(b, g, s, v, kOutProject, true);
 }
+// attn_project_mfma_ms, gdn_project_mfma_ms, gdn_outproj_mfma_ms (no reference counterpart):
+// the bindings and grids of the _ms forms, evaluated on the matrix unit by q4_wave_kernel -
+// the same mathematics in another summation order, for decode waves of several lanes.
+int32_t op_attn_project_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kAttnProject, false, true);
+}
+int32_t op_gdn_project_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kGdnProject, false, true);
+}
+int32_t op_gdn_outproj_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kOutProject, true, true);
+}
 // outproj_blk: + c5 block rows, c6 input width (prefill_step.cpp:2063-2078).
 int32_t op_outproj_blk(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
     return project_block(b, g, s, v, kOutProject, true);
@@ -632,6 +740,9 @@ const KernelDesc kQ4ProjectKernels[] = {
     {"gdn_outproj_ms", op_gdn_outproj_ms},
     {"gdn_outproj_ms_v2", op_gdn_outproj_ms},
     {"outproj_blk", op_outproj_blk},
+    {"attn_project_mfma_ms", op_attn_project_mfma_ms},
+    {"gdn_project_mfma_ms", op_gdn_project_mfma_ms},
+    {"gdn_outproj_mfma_ms", op_gdn_outproj_mfma_ms},
 };
 const uint32_t kQ4ProjectKernelCount = sizeof(kQ4ProjectKernels) / sizeof(kQ4ProjectKernels[0]);
 #endif

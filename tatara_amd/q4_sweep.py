@@ -1,7 +1,7 @@
 """Timing of the affine 4-bit projections on one GPU: the three projections of the
 attention family (attention in-projection 2048 -> 9216, Gated DeltaNet in-projection
-2048 -> 12352, output projection 4096 -> 2048) at decode-wave row counts (`_ms`
-operators) and at block row counts (`_blk` operators), random weights.
+2048 -> 12352, output projection 4096 -> 2048) at decode-wave row counts (`_ms` and
+`_mfma_ms` operators) and at block row counts (`_blk` operators), random weights.
 
     python -m tatara_amd.q4_sweep [--decode 1,4,16] [--block 256,2048,16384] [--repeats 5]
 prints one JSON line per point: device microseconds per dispatch (best of the repeats,
@@ -40,7 +40,7 @@ def _bind(dev, family, rng):
     return bindings
 
 
-def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5):
+def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5, matrix_unit=False):
     family = FAMILIES[name]
     rng = np.random.default_rng(rows)
     total, k = sum(family["segments"]), family["k"]
@@ -54,7 +54,7 @@ def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5):
         constants = {slot: rows, slot + 1: k} if name == "gdn_outproj" else {slot: rows}
         grid = (groups, 1, 1)
     else:
-        operator = name + "_ms"
+        operator = name + ("_mfma_ms" if matrix_unit else "_ms")
         tile = 16
         constants = ({slot: rows, slot + 1: total, slot + 2: tile} if name == "gdn_outproj"
                      else {slot: rows, slot + 1: tile})
@@ -90,6 +90,9 @@ def main():
             for name in FAMILIES:
                 print(json.dumps(measure(dev, queue, lib, name, rows, block, args.repeats)),
                       flush=True)
+                if not block:   # the same wave on the matrix unit
+                    print(json.dumps(measure(dev, queue, lib, name, rows, block, args.repeats,
+                                             matrix_unit=True)), flush=True)
 
 
 if __name__ == "__main__":

@@ -187,7 +187,9 @@ class StubStack:
             cb.encode(self.lib.pipeline(name + "_blk"), bindings, {out + 1: rows},
                       ((width + 3) // 4,), (128,))
         else:
-            cb.encode(self.lib.pipeline(name + "_ms"), bindings, {out + 1: rows, out + 2: 16},
+            # several lanes: the matrix-unit form; one lane: the reference's own order
+            suffix = "_mfma_ms" if rows >= 2 else "_ms"
+            cb.encode(self.lib.pipeline(name + suffix), bindings, {out + 1: rows, out + 2: 16},
                       ((width + 3) // 4, 1), (128,))
         cb.barrier()
 
@@ -202,7 +204,8 @@ class StubStack:
             cb.encode(self.lib.pipeline("outproj_blk"), bindings, {5: rows, 6: 4096},
                       (HIDDEN // 2,), (64,))
         else:
-            cb.encode(self.lib.pipeline("gdn_outproj_ms"), bindings, {5: rows, 6: HIDDEN, 7: 16},
+            name = "gdn_outproj_mfma_ms" if rows >= 2 else "gdn_outproj_ms"
+            cb.encode(self.lib.pipeline(name), bindings, {5: rows, 6: HIDDEN, 7: 16},
                       (HIDDEN // 2, 1), (64,))
         cb.barrier()
 

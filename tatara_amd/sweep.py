@@ -16,7 +16,8 @@ from . import backend as B
 from . import stack as S
 
 STUB_KERNELS = {"rms_only", "rms_only_ms", "residual_rms_ms", "dense_bf16", "add_bf16",
-                "attn_project_ms", "gdn_project_ms", "gdn_outproj_ms", "attn_project_blk",
+                "attn_project_ms", "gdn_project_ms", "gdn_outproj_ms", "attn_project_mfma_ms",
+                "gdn_project_mfma_ms", "gdn_outproj_mfma_ms", "attn_project_blk",
                 "gdn_project_blk", "outproj_blk"}
 
 

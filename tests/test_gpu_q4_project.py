@@ -100,6 +100,34 @@ def test_wave_projection_bit_for_bit(family, suffix, rows, tile):
     print(f"[time] {name} rows={rows} tile={tile}: {ms * 1e3:.1f} us", flush=True)
 
 
+@pytest.mark.parametrize("rows", [1, 2, 4, 13, 16])
+@pytest.mark.parametrize("family", [ATTN, GDN, OUT], ids=lambda f: f["name"])
+def test_wave_projection_on_the_matrix_unit(family, rows):
+    """The _mfma_ms forms (no reference counterpart): the bindings and grids of the _ms forms,
+    sums in another order - held to the path's bar, with the share of bit-identical outputs
+    printed."""
+    name = family["name"] + "_mfma_ms"
+    print(f"[case] {name} rows={rows}", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9800)
+    x = ol.gaussian_bf16(0x9900 + rows, rows * family["k"], 0.0, 1.0)
+    total = sum(family["segments"])
+    strided = family is OUT
+    stride = total + 64 if strided else total
+    out = dev.buffer_from(np.full(rows * stride, 0x7FC0, np.uint16))
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    slot = family["out"] + 1
+    constants = {slot: rows, slot + 1: stride, slot + 2: 16} if strided else {slot: rows, slot + 1: 16}
+    ms = run(lambda cb: cb.encode(lib.pipeline(name), bindings, constants, (_groups(family), 1, 1),
+                                  (family["threads"], 1, 1)))
+    got = out.read(np.uint16).reshape(rows, stride)
+    want = _expected(family, host, x, rows, stride).reshape(rows, stride)
+    check_bf16(got[:, :total], want[:, :total], name, ulps=2)
+    assert np.all(got[:, total:] == 0x7FC0)
+    print(f"[time] {name} rows={rows}: {ms * 1e3:.1f} us", flush=True)
+
+
 @pytest.mark.parametrize("family,name", [(ATTN, "attn_project_blk"), (GDN, "gdn_project_blk"),
                                          (OUT, "outproj_blk")], ids=["attn", "gdn", "out"])
 @pytest.mark.parametrize("rows", [1, 37, 130])
