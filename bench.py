@@ -16,6 +16,10 @@ the stream.  The step is compiled into a HIP graph and replayed.
 one lane through a full-attention layer (causal flash attention on MFMA) and a
 Gated DeltaNet layer (chunk-64 recurrence on MFMA), tok/s and fraction of MFMA peak.
 
+`detail.q4_projections` adds the affine 4-bit projections either side of the family
+(attention / GDN in-projection, output projection) for the same 4-lane wave and the same
+16384-row block, device microseconds per dispatch (tatara_amd.q4_sweep).
+
 Prints ONE JSON line: `value` = microseconds per layer over the period,
 `roofline` for the dominant kernel (the split-K flash-decode), `cpu_baseline` =
 the CPU checker timed on this box's host cores on the same period."""
@@ -391,6 +395,12 @@ def main():
     }
     if not args.no_prefill:
         line["detail"]["prefill_16k"] = prefill_figures(B, dev, queue, lib, torch)
+    if not args.no_prefill:
+        from tatara_amd import q4_sweep
+        line["detail"]["q4_projections"] = (
+            [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)
+             for name in q4_sweep.FAMILIES] +
+            [q4_sweep.measure(dev, queue, lib, name, 16384, True, 2) for name in q4_sweep.FAMILIES])
     if not args.no_cpu_baseline:
         threads = min(16, os.cpu_count() or 1)
         line["cpu_baseline"] = cpu_baseline(threads)
