@@ -397,14 +397,15 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         }
         const uint32_t* scale_pairs =
             reinterpret_cast<const uint32_t*>(stage + kXStageBytes + kWordStageBytes);
-        const bool odd_group = (group & 1) != 0;
+        // bytes {0, 1} (even group) or {2, 3} (odd group) of a pair into the upper half, zeros below
+        const uint32_t pick = (group & 1) ? 0x03020C0Cu : 0x01000C0Cu;
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
             const u32x4 pairs = *reinterpret_cast<const u32x4*>(scale_pairs + 64 * nh + 16 * tn + 4 * g);
             f32x4 scale;
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
-                scale[j] = __uint_as_float(odd_group ? (pairs[j] & 0xFFFF0000u) : (pairs[j] << 16));
+                scale[j] = __uint_as_float(__builtin_amdgcn_perm(0u, pairs[j], pick));
             }
 #pragma unroll
             for (uint32_t tm = 0; tm < 4; ++tm) {
