@@ -711,6 +711,270 @@ HipCommandError encode_token(DecodeStep& step, DecodeStateSlot& state, DecodeBat
     return walk.error;
 }
 
+// ---- the stages either side of the family, from the model's 4-bit weights ----
+StagePipelinesResult resolve_stage_pipelines(const HipLibrary& library) {
+    StagePipelines p;
+    HipPipelineError error = HipPipelineError::None;
+    using P = StagePipelines;
+    const bool ok =
+        resolve(library, p, &P::rms_ms, "rms_only_ms", error) &&
+        resolve(library, p, &P::residual_rms_ms, "residual_rms_ms", error) &&
+        resolve(library, p, &P::gdn_project_ms, "gdn_project_ms", error) &&
+        resolve(library, p, &P::attn_project_ms, "attn_project_ms", error) &&
+        resolve(library, p, &P::gdn_outproj_ms, "gdn_outproj_ms", error) &&
+        resolve(library, p, &P::gdn_project_mfma_ms, "gdn_project_mfma_ms", error) &&
+        resolve(library, p, &P::attn_project_mfma_ms, "attn_project_mfma_ms", error) &&
+        resolve(library, p, &P::gdn_outproj_mfma_ms, "gdn_outproj_mfma_ms", error);
+    if (!ok) return {error, std::nullopt};
+    return {HipPipelineError::None, std::move(p)};
+}
+
+HiddenStreamsResult create_hidden_streams(const HipDevice& device, const DecodeGeometry& geometry,
+                                          std::uint32_t rows) {
+    if (rows == 0 || rows > kMaximumBatchRows) {
+        return {DecodeStepError::OffsetCountMismatch, std::nullopt};
+    }
+    HiddenStreams h;
+    h.rows = rows;
+    const std::uint64_t bytes = rows * geometry.hidden_bytes;
+    if (!allocate_zeroed(device, bytes, h.input) || !allocate_zeroed(device, bytes, h.normed) ||
+        !allocate_zeroed(device, bytes, h.branch) || !allocate_zeroed(device, bytes, h.residual)) {
+        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+    }
+    return {DecodeStepError::None, std::move(h)};
+}
+
+namespace {
+
+// decode_geometry.h:147-148: one 32-lane group per output row, four (two) groups
+// to a workgroup of the input (output) projections.
+constexpr std::uint32_t kProjectionThreads = 128;
+constexpr std::uint32_t kOutProjectionThreads = 64;
+
+void bind_quantized(Walk& walk, const QuantizedBinding& q, std::uint32_t first) {
+    walk.weight(q.weight, first);
+    walk.weight(q.scales, first + 1);
+    walk.weight(q.biases, first + 2);
+}
+
+bool stages_usable(const QuantizedLayerStages& s, std::size_t layer, LayerKind kind,
+                   std::uint32_t rows) {
+    return s.pipelines != nullptr && s.geometry != nullptr && s.scratch != nullptr &&
+           s.streams != nullptr && layer < s.layers.size() && layer < s.schedule.size() &&
+           s.schedule[layer] == kind && rows >= 1 && rows <= s.scratch->rows &&
+           rows <= s.streams->rows && s.row_tile >= 1 && s.row_tile <= kMaximumBatchRows;
+}
+
+const HipBuffer& layer_input(const QuantizedLayerStages& s, std::size_t layer) {
+    return layer != 0 && s.residual_feeds_next ? s.streams->residual : s.streams->input;
+}
+
+HipCommandError project_hook(void* user, HipComputePass& pass, std::size_t layer, LayerKind kind,
+                             std::uint32_t rows) {
+    return static_cast<const QuantizedLayerStages*>(user)->encode_project(pass, layer, kind, rows);
+}
+HipCommandError finish_hook(void* user, HipComputePass& pass, std::size_t layer, LayerKind kind,
+                            std::uint32_t rows) {
+    return static_cast<const QuantizedLayerStages*>(user)->encode_finish(pass, layer, kind, rows);
+}
+
+}  // namespace
+
+LayerStageHooks QuantizedLayerStages::hooks() { return {this, &project_hook, &finish_hook}; }
+
+HipCommandError QuantizedLayerStages::encode_project(HipComputePass& pass, std::size_t layer,
+                                                     LayerKind kind, std::uint32_t rows) const {
+    if (!stages_usable(*this, layer, kind, rows)) return HipCommandError::InvalidStreamGroup;
+    const DecodeGeometry& g = *geometry;
+    const StagePipelines& k = *pipelines;
+    const LayerBindings& bound = layers[layer];
+    const std::uint32_t hidden = static_cast<std::uint32_t>(g.hidden_bytes / 2);
+    const std::uint32_t tiles = (rows + row_tile - 1) / row_tile;
+    const bool wide = matrix_unit && rows >= 2;
+    Walk walk{pass};
+    walk.pipeline(k.rms_ms);
+    walk.buffer(layer_input(*this, layer), 0, 0);
+    walk.weight(bound.input_norm, 1);
+    walk.buffer(streams->normed, 0, 2);
+    walk.constant(hidden, 3);
+    walk.constant(hidden, 4);
+    walk.dispatch(HipSize{g.rms.groups, rows, 1}, HipSize{g.rms.threads, 1, 1});
+    walk.barrier();
+    if (is_gated(kind)) {
+        const std::uint32_t out_rows = static_cast<std::uint32_t>(g.gdn_projection_bytes / 2);
+        walk.pipeline(wide ? k.gdn_project_mfma_ms : k.gdn_project_ms);
+        walk.buffer(streams->normed, 0, 0);
+        bind_quantized(walk, bound.gated_delta.qkv, 1);
+        bind_quantized(walk, bound.gated_delta.z, 4);
+        bind_quantized(walk, bound.gated_delta.b, 7);
+        bind_quantized(walk, bound.gated_delta.a, 10);
+        walk.buffer(scratch->gdn_projection, 0, 13);
+        walk.constant(rows, 14);
+        walk.constant(row_tile, 15);
+        walk.dispatch(HipSize{(out_rows + 3) / 4, tiles, 1}, HipSize{kProjectionThreads, 1, 1});
+    } else {
+        const std::uint32_t out_rows = static_cast<std::uint32_t>(g.attn_projection_bytes / 2);
+        walk.pipeline(wide ? k.attn_project_mfma_ms : k.attn_project_ms);
+        walk.buffer(streams->normed, 0, 0);
+        bind_quantized(walk, bound.attention.query, 1);
+        bind_quantized(walk, bound.attention.key, 4);
+        bind_quantized(walk, bound.attention.value, 7);
+        walk.buffer(scratch->attn_projection, 0, 10);
+        walk.constant(rows, 11);
+        walk.constant(row_tile, 12);
+        walk.dispatch(HipSize{(out_rows + 3) / 4, tiles, 1}, HipSize{kProjectionThreads, 1, 1});
+    }
+    return walk.error;
+}
+
+HipCommandError QuantizedLayerStages::encode_finish(HipComputePass& pass, std::size_t layer,
+                                                    LayerKind kind, std::uint32_t rows) const {
+    if (!stages_usable(*this, layer, kind, rows)) return HipCommandError::InvalidStreamGroup;
+    const DecodeGeometry& g = *geometry;
+    const StagePipelines& k = *pipelines;
+    const LayerBindings& bound = layers[layer];
+    const std::uint32_t hidden = static_cast<std::uint32_t>(g.hidden_bytes / 2);
+    const std::uint32_t tiles = (rows + row_tile - 1) / row_tile;
+    const bool wide = matrix_unit && rows >= 2;
+    Walk walk{pass};
+    walk.barrier();
+    walk.pipeline(wide ? k.gdn_outproj_mfma_ms : k.gdn_outproj_ms);
+    walk.buffer(is_gated(kind) ? scratch->gdn_gated : scratch->attn_attended, 0, 0);
+    bind_quantized(walk, is_gated(kind) ? bound.gated_delta.out : bound.attention.out, 1);
+    walk.buffer(streams->branch, 0, 4);
+    walk.constant(rows, 5);
+    walk.constant(hidden, 6);
+    walk.constant(row_tile, 7);
+    walk.dispatch(HipSize{hidden / 2, tiles, 1}, HipSize{kOutProjectionThreads, 1, 1});
+    walk.barrier();
+    walk.pipeline(k.residual_rms_ms);
+    walk.buffer(layer_input(*this, layer), 0, 0);
+    walk.buffer(streams->branch, 0, 1);
+    walk.buffer(streams->residual, 0, 2);
+    walk.weight(bound.post_norm, 3);
+    walk.buffer(streams->normed, 0, 4);
+    walk.constant(hidden, 5);
+    walk.constant(hidden, 6);
+    walk.constant(hidden, 7);
+    walk.dispatch(HipSize{g.rms.groups, rows, 1}, HipSize{g.rms.threads, 1, 1});
+    return walk.error;
+}
+
+BlockStagePipelinesResult resolve_block_stage_pipelines(const HipLibrary& library) {
+    BlockStagePipelines p;
+    HipPipelineError error = HipPipelineError::None;
+    using P = BlockStagePipelines;
+    const bool ok = resolve(library, p, &P::rms, "rms_only_ms", error) &&
+                    resolve(library, p, &P::residual_rms, "residual_rms_ms", error) &&
+                    resolve(library, p, &P::gdn_project, "gdn_project_blk", error) &&
+                    resolve(library, p, &P::attn_project, "attn_project_blk", error) &&
+                    resolve(library, p, &P::out_projection, "outproj_blk", error);
+    if (!ok) return {error, std::nullopt};
+    return {HipPipelineError::None, std::move(p)};
+}
+
+BlockStreamsResult create_block_streams(const HipDevice& device, const PrefillGeometry& geometry,
+                                        std::uint32_t hidden) {
+    const std::uint32_t rows = geometry.policy.maximum_block_rows;
+    // the norm kernels hold four values per thread of one workgroup
+    if (rows == 0 || hidden == 0 || hidden % 128 != 0 || hidden > 4096) {
+        return {DecodeStepError::OffsetCountMismatch, std::nullopt};
+    }
+    BlockStreams b;
+    b.block_rows = rows;
+    b.hidden = hidden;
+    const std::uint64_t bytes = std::uint64_t{rows} * hidden * kBf16Bytes;
+    if (!allocate_zeroed(device, bytes, b.normalized) || !allocate_zeroed(device, bytes, b.branch) ||
+        !allocate_zeroed(device, bytes, b.block_hidden)) {
+        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+    }
+    return {DecodeStepError::None, std::move(b)};
+}
+
+namespace {
+
+bool block_stage_usable(const PrefillScratch& scratch, const BlockStreams& streams,
+                        const PrefillChunk& chunk) {
+    return chunk.rows >= 1 && chunk.rows <= scratch.block_rows && chunk.rows <= streams.block_rows &&
+           streams.hidden != 0;
+}
+
+}  // namespace
+
+HipCommandError encode_prefill_layer_input(const BlockStagePipelines& pipelines,
+                                           const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                           BlockStreams& streams, const LayerBindings& bindings,
+                                           LayerKind kind, const PrefillChunk& chunk,
+                                           const HipBuffer& input, std::uint64_t input_offset,
+                                           HipComputePass& pass) {
+    if (!block_stage_usable(scratch, streams, chunk)) return HipCommandError::InvalidDispatchExtent;
+    Walk walk{pass};
+    walk.barrier();
+    walk.pipeline(pipelines.rms);
+    walk.buffer(input, input_offset, 0);
+    walk.weight(bindings.input_norm, 1);
+    walk.buffer(streams.normalized, 0, 2);
+    walk.constant(streams.hidden, 3);
+    walk.constant(streams.hidden, 4);
+    walk.dispatch(HipSize{1, chunk.rows, 1}, HipSize{streams.hidden / 4, 1, 1});
+    walk.barrier();
+    if (is_gated(kind)) {
+        walk.pipeline(pipelines.gdn_project);
+        walk.buffer(streams.normalized, 0, 0);
+        bind_quantized(walk, bindings.gated_delta.qkv, 1);
+        bind_quantized(walk, bindings.gated_delta.z, 4);
+        bind_quantized(walk, bindings.gated_delta.b, 7);
+        bind_quantized(walk, bindings.gated_delta.a, 10);
+        walk.buffer(scratch.gdn_projection, 0, 13);
+        walk.constant(chunk.rows, 14);
+        walk.dispatch(HipSize{(geometry.gdn_projection_rows + 3) / 4, 1, 1},
+                      HipSize{kProjectionThreads, 1, 1});
+    } else {
+        walk.pipeline(pipelines.attn_project);
+        walk.buffer(streams.normalized, 0, 0);
+        bind_quantized(walk, bindings.attention.query, 1);
+        bind_quantized(walk, bindings.attention.key, 4);
+        bind_quantized(walk, bindings.attention.value, 7);
+        walk.buffer(scratch.attn_projection, 0, 10);
+        walk.constant(chunk.rows, 11);
+        walk.dispatch(HipSize{(geometry.attention_projection_rows + 3) / 4, 1, 1},
+                      HipSize{kProjectionThreads, 1, 1});
+    }
+    walk.barrier();
+    return walk.error;
+}
+
+HipCommandError encode_prefill_layer_output(const BlockStagePipelines& pipelines,
+                                            const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                            BlockStreams& streams, const LayerBindings& bindings,
+                                            LayerKind kind, const PrefillChunk& chunk,
+                                            const HipBuffer& input, std::uint64_t input_offset,
+                                            HipComputePass& pass) {
+    if (!block_stage_usable(scratch, streams, chunk)) return HipCommandError::InvalidDispatchExtent;
+    Walk walk{pass};
+    walk.barrier();
+    walk.pipeline(pipelines.out_projection);
+    walk.buffer(is_gated(kind) ? scratch.gdn_gated : scratch.attn_attended, 0, 0);
+    bind_quantized(walk, is_gated(kind) ? bindings.gated_delta.out : bindings.attention.out, 1);
+    walk.buffer(streams.branch, 0, 4);
+    walk.constant(chunk.rows, 5);
+    walk.constant(is_gated(kind) ? geometry.gdn_value_values : geometry.attention_vector_values, 6);
+    walk.dispatch(HipSize{streams.hidden / 2, 1, 1}, HipSize{kOutProjectionThreads, 1, 1});
+    walk.barrier();
+    walk.pipeline(pipelines.residual_rms);
+    walk.buffer(input, input_offset, 0);
+    walk.buffer(streams.branch, 0, 1);
+    walk.buffer(streams.block_hidden, 0, 2);
+    walk.weight(bindings.post_norm, 3);
+    walk.buffer(streams.normalized, 0, 4);
+    walk.constant(streams.hidden, 5);
+    walk.constant(streams.hidden, 6);
+    walk.constant(streams.hidden, 7);
+    walk.dispatch(HipSize{1, chunk.rows, 1}, HipSize{streams.hidden / 4, 1, 1});
+    walk.barrier();
+    return walk.error;
+}
+
 void advance_decode_state(const DecodeStep& step, DecodeStateSlot& state) {
     if (!decode_state_slot_available(step, state)) return;
     for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {

@@ -321,6 +321,89 @@ HipCommandError encode_token(DecodeStep& step, DecodeStateSlot& state, DecodeBat
                              std::span<const LayerWeights> weights, const LayerStageHooks& hooks,
                              HipComputePass& pass, std::uint32_t context);
 
+// ---- the stages either side of the family, from the model's 4-bit weights ----
+// An affine 4-bit matrix, group 64 (decode_bindings.h:17-24): weight [rows][k/8]
+// u32, scales and biases [rows][k/64] bf16.
+struct QuantizedBinding {
+    const HipBuffer* weight{nullptr};
+    const HipBuffer* scales{nullptr};
+    const HipBuffer* biases{nullptr};
+};
+// decode_bindings.h:27-48
+struct GatedDeltaBindings {
+    QuantizedBinding qkv, z, b, a, out;
+};
+struct AttentionBindings {
+    QuantizedBinding query, key, value, out;
+};
+// The attention-family members of LayerBindings (decode_bindings.h:50-64);
+// input_norm and post_norm are [hidden] bf16.
+struct LayerBindings {
+    const HipBuffer* input_norm{nullptr};
+    const HipBuffer* post_norm{nullptr};
+    GatedDeltaBindings gated_delta;
+    AttentionBindings attention;
+};
+struct StagePipelines {
+    HipComputePipeline rms_ms, residual_rms_ms;
+    HipComputePipeline gdn_project_ms, attn_project_ms, gdn_outproj_ms;
+    // the same bindings evaluated on the matrix unit (another summation order)
+    HipComputePipeline gdn_project_mfma_ms, attn_project_mfma_ms, gdn_outproj_mfma_ms;
+};
+struct StagePipelinesResult {
+    backend::hip::HipPipelineError error;
+    std::optional<StagePipelines> pipelines;
+    explicit operator bool() const noexcept {
+        return error == backend::hip::HipPipelineError::None && pipelines.has_value();
+    }
+};
+StagePipelinesResult resolve_stage_pipelines(const HipLibrary& library);
+
+// The hidden-width rows of one wave (decode_step.h:202-231: input, normed,
+// branch_stream, residual_stream), each [rows][hidden] bf16.
+struct HiddenStreams {
+    std::uint32_t rows{0};
+    HipBuffer input, normed, branch, residual;
+};
+struct HiddenStreamsResult {
+    DecodeStepError error;
+    std::optional<HiddenStreams> streams;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && streams.has_value();
+    }
+};
+HiddenStreamsResult create_hidden_streams(const HipDevice& device, const DecodeGeometry& geometry,
+                                          std::uint32_t rows);
+
+// LayerStageHooks that run the reference's own stages around the family
+// (decode_step.cpp:1102-1135, 1196-1211, 1280-1310):
+//   project: normed = rms(layer input, input_norm); projection slab = Q4(normed)
+//   finish:  branch = Q4 out-projection(gated / attended);
+//            residual = bf16(layer input + branch); normed = rms(residual, post_norm)
+// The layer input is streams.input for layer 0.  For later layers it is what
+// the expert stage (outside this path) left in streams.input, or, with
+// residual_feeds_next, the previous layer's residual.  The object must outlive
+// the encoding; scratch and streams must hold at least the wave's rows.
+struct QuantizedLayerStages {
+    const StagePipelines* pipelines{nullptr};
+    const DecodeGeometry* geometry{nullptr};
+    std::span<const LayerKind> schedule;
+    std::span<const LayerBindings> layers;
+    DecodeBatchScratch* scratch{nullptr};
+    HiddenStreams* streams{nullptr};
+    bool residual_feeds_next{true};
+    // waves of two or more rows on the matrix unit; one row always runs the
+    // reference's summation order
+    bool matrix_unit{true};
+    std::uint32_t row_tile{16};          // rows per tile of the _ms operators (decode_step.cpp:1080-1093)
+
+    LayerStageHooks hooks();
+    HipCommandError encode_project(HipComputePass& pass, std::size_t layer, LayerKind kind,
+                                   std::uint32_t rows) const;
+    HipCommandError encode_finish(HipComputePass& pass, std::size_t layer, LayerKind kind,
+                                  std::uint32_t rows) const;
+};
+
 // decode_step.cpp:1432-1441: toggles `swapped` on Gated DeltaNet layers of an
 // available, compatible slot; anything else is left untouched.
 void advance_decode_state(const DecodeStep& step, DecodeStateSlot& state);
@@ -540,6 +623,57 @@ HipCommandError encode_gdn_tape_windows(const DecodeStep& step, DecodeStateSlot&
                                         const PrefillScratch& scratch, std::uint32_t committed,
                                         HipBlitPass& blit_pass);
 void complete_gdn_tape_rollback(const DecodeStep& step, DecodeStateSlot& state);
+
+// ---- the block's stages either side of the family, from 4-bit weights ---------
+// encode_layer / encode_moe's head (prefill_step.cpp:2535-2567, 2236-2267) with
+// the projections of encode_gated_delta / encode_attention (1428-1446, 1909-1926,
+// 2063-2078):
+//   input:  normalized = rms(input rows, input_norm); projection slab = Q4(normalized)
+//   output: branch = Q4 out-projection(gated / attended);
+//           block_hidden = bf16(input + branch); normalized = rms(block_hidden, post_norm)
+// Blocks of more than 16 rows run on the matrix unit (another summation order
+// than the reference's), shorter ones in the reference's order.
+struct BlockStagePipelines {
+    HipComputePipeline rms, residual_rms, gdn_project, attn_project, out_projection;
+};
+struct BlockStagePipelinesResult {
+    backend::hip::HipPipelineError error;
+    std::optional<BlockStagePipelines> pipelines;
+    explicit operator bool() const noexcept {
+        return error == backend::hip::HipPipelineError::None && pipelines.has_value();
+    }
+};
+BlockStagePipelinesResult resolve_block_stage_pipelines(const HipLibrary& library);
+
+// [maximum_block_rows][hidden] bf16 each (prefill_step.h: normalized, branch, block_hidden).
+struct BlockStreams {
+    std::uint32_t block_rows{0};
+    std::uint32_t hidden{0};
+    HipBuffer normalized, branch, block_hidden;
+};
+struct BlockStreamsResult {
+    DecodeStepError error;
+    std::optional<BlockStreams> streams;
+    explicit operator bool() const noexcept {
+        return error == DecodeStepError::None && streams.has_value();
+    }
+};
+BlockStreamsResult create_block_streams(const HipDevice& device, const PrefillGeometry& geometry,
+                                        std::uint32_t hidden);
+
+// `input` holds the chunk's rows ([rows][hidden] bf16) from input_offset bytes on.
+HipCommandError encode_prefill_layer_input(const BlockStagePipelines& pipelines,
+                                           const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                           BlockStreams& streams, const LayerBindings& bindings,
+                                           LayerKind kind, const PrefillChunk& chunk,
+                                           const HipBuffer& input, std::uint64_t input_offset,
+                                           HipComputePass& pass);
+HipCommandError encode_prefill_layer_output(const BlockStagePipelines& pipelines,
+                                            const PrefillGeometry& geometry, PrefillScratch& scratch,
+                                            BlockStreams& streams, const LayerBindings& bindings,
+                                            LayerKind kind, const PrefillChunk& chunk,
+                                            const HipBuffer& input, std::uint64_t input_offset,
+                                            HipComputePass& pass);
 
 // ---- lane state record (Q36BRS01) ------------------------------------------
 // The file / wire form of exactly the buffers a lane owns on this path

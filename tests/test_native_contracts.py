@@ -27,8 +27,9 @@ def test_host_contract(name):
 
 @pytest.mark.gpu
 def test_runtime_on_gpu():
-    """Layer walk, state pool, block prefill and lane reset of the C++ host layer
-    against the CPU checker."""
+    """Layer walk, state pool, the norm and 4-bit projection stages either side of the
+    family, block prefill, state record, prefix snapshot, tape rollback and lane reset of
+    the C++ host layer against the CPU checker."""
     result = subprocess.run([_binary("runtime_gpu_test")], capture_output=True, text=True,
                             timeout=300)
     print(result.stdout, flush=True)
