@@ -808,7 +808,15 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
 
     // Keys and values of the chunk into LDS with 16-byte loads: 16 lanes per row, 16
     // rows per pass; rows past the block repeat the last one (their scales are zero).
+    // The wave's query rows (token rows 16w .. 16w+15) are requested with them.
     const bool is_k = wave < 2;
+    bf16x8 aq[4];
+    {
+        const uint16_t* qrow = a.qk + static_cast<uint64_t>(t0 + min(wave * 16 + m, valid - 1)) * kGdnQkValues +
+                               kh * kGD;
+#pragma unroll
+        for (uint32_t kk = 0; kk < 4; ++kk) aq[kk] = operand(qrow + kk * 32 + g * 8);
+    }
     {
         const uint16_t* ksrc = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kGdnKOffset + kh * kGD;
         const uint16_t* vsrc = a.value + static_cast<uint64_t>(t0) * kGdnValueValues + h * kGD;
@@ -850,15 +858,12 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
     }
     __syncthreads();
 
-    const uint16_t* qrows = a.qk + static_cast<uint64_t>(t0) * kGdnQkValues + kh * kGD;
     {
         // wave w owns token rows 16w..16w+15 against all 64 columns
-        const uint32_t trow = min(wave * 16 + m, valid - 1);
-        bf16x8 ak[4], aq[4];
+        bf16x8 ak[4];
 #pragma unroll
         for (uint32_t kk = 0; kk < 4; ++kk) {
             ak[kk] = operand(&ktile[wave * 16 + m][kk * 32 + g * 8]);
-            aq[kk] = operand(qrows + static_cast<uint64_t>(trow) * kGdnQkValues + kk * 32 + g * 8);
             *reinterpret_cast<u32x4*>(rec + kRecQ + ((wave * 4 + kk) * 64 + lane) * 16) =
                 __builtin_bit_cast(u32x4, aq[kk]);
         }
@@ -961,47 +966,22 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
         hi = __builtin_bit_cast(bf16x8, h);
         lo = __builtin_bit_cast(bf16x8, l);
     };
-    const uint16_t (*source)[kTileLd] = is_k ? ktile : vtile;
-    const float* scale = is_k ? scale_k : scale_v;
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t ct = 0; ct < 4; ++ct) {
-        const uint32_t col0 = (wave & 1) * 64 + ct * 16;
-        // right-hand side tiles, this lane: tokens 16i + 4g + r of column col0 + m.  One
-        // transposing read per tile: 16 lanes hand in 4 token rows x 16 columns (4
-        // lanes per row) and lane m receives column m of the 4 rows.
+    // every wave holds its left operands: `lower` and `tdiag` are free from here on
+    __syncthreads();
+
+    // Block column `wave` of T = (I + L)^-1 by block forward substitution on the
+    // identity: X_i = T_ii (E_i - sum_{j<i} L_ij X_j).  All products on MFMA with hi/lo
+    // operand pairs; a finished block goes, as bf16 hi/lo, into the wave's strip in LDS,
+    // from where it is read back as the right operand of the next products (rows
+    // contiguous: one 16-byte read per lane).  The four waves run the four columns side
+    // by side; the finished fp32 blocks overwrite `lower`.
+    {
         f32x4 rhs[4];
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
-            const s16x4 bits = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) s16x4*)(&source[16 * i + 4 * g + (m >> 2)]
-                                                                  [col0 + (m & 3) * 4]));
-            const f32x4 sc = *reinterpret_cast<const f32x4*>(&scale[16 * i + 4 * g]);
 #pragma unroll
-            for (uint32_t r = 0; r < 4; ++r) {
-                rhs[i][r] = 16 * i + 4 * g + r < valid
-                                ? widen(static_cast<uint16_t>(bits[r])) * sc[r] : 0.0f;
-            }
-        }
-        if (is_k) {
-            // the exact keys, token-contiguous: fragment (key tile, token step ks), lane =
-            // key col0 + m, tokens 32 ks + 8 g .. +7
-#pragma unroll
-            for (uint32_t ks = 0; ks < 2; ++ks) {
-                const uint16_t* at = &ktile[ks * 32 + g * 8 + (m >> 2)][col0 + (m & 3) * 4];
-                const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(at));
-                const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(at + 4 * kTileLd));
-                uint32_t bits[8];
-#pragma unroll
-                for (uint32_t e = 0; e < 4; ++e) {
-                    bits[e] = ks * 32 + g * 8 + e < valid ? static_cast<uint16_t>(first[e]) : 0u;
-                    bits[4 + e] = ks * 32 + g * 8 + 4 + e < valid ? static_cast<uint16_t>(second[e]) : 0u;
-                }
-                *reinterpret_cast<u32x4*>(rec + kRecKt + (((col0 >> 4) * 2 + ks) * 64 + lane) * 16) =
-                    u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
-                          bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
-            }
+            for (uint32_t r = 0; r < 4; ++r) rhs[i][r] = (i == wave && g * 4 + r == m) ? 1.0f : 0.0f;
         }
         bf16x8 b_hi, b_lo;
         f32x4 w[4];
@@ -1028,6 +1008,73 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkPrepareArgs
         put(x, 48);
         get(48, true, b_hi, b_lo);
         w[3] = product(t_hi[3], t_lo[3], b_hi, b_lo, zero);
+#pragma unroll
+        for (uint32_t mt = 0; mt < 4; ++mt) {
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) lower[16 * mt + 4 * g + r][16 * wave + m] = w[mt][r];
+        }
+    }
+    __syncthreads();
+
+    // [Wk | Wv] = T (beta o [g o K | V]) = (T o scale) [K | V]: the scales go into the
+    // columns of T (fp32, then hi/lo), which leaves the exact bf16 keys and values as the
+    // other operand - two products per step and no chain between them.  Every wave takes
+    // its own 64 columns (waves 0,1 the keys, 2,3 the values).  Block (mt, ks) of T,
+    // token rows 16 mt .., token columns 32 ks ..; T is lower triangular: ks <= mt / 2.
+    const uint16_t (*source)[kTileLd] = is_k ? ktile : vtile;
+    const float* scale = is_k ? scale_k : scale_v;
+    bf16x8 ts_hi[4][2], ts_lo[4][2];
+#pragma unroll
+    for (uint32_t mt = 0; mt < 4; ++mt) {
+#pragma unroll
+        for (uint32_t ks = 0; ks < 2; ++ks) {
+            if (2 * ks > mt) continue;
+            float x[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                x[e] = lower[16 * mt + m][32 * ks + 8 * g + e] * scale[32 * ks + 8 * g + e];
+            }
+            split8(x, ts_hi[mt][ks], ts_lo[mt][ks]);
+        }
+    }
+    for (uint32_t ct = 0; ct < 4; ++ct) {
+        const uint32_t col0 = (wave & 1) * 64 + ct * 16;
+        // the exact rows, token-contiguous: lane = column col0 + m, tokens 32 ks + 8 g .. +7,
+        // by transposing reads (16 lanes hand in 4 token rows x 16 columns, lane m
+        // receives column m of the 4 rows)
+        bf16x8 rows8[2];
+#pragma unroll
+        for (uint32_t ks = 0; ks < 2; ++ks) {
+            const uint16_t* at = &source[ks * 32 + g * 8 + (m >> 2)][col0 + (m & 3) * 4];
+            const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(at));
+            const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(at + 4 * kTileLd));
+            uint32_t bits[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 4; ++e) {
+                bits[e] = ks * 32 + g * 8 + e < valid ? static_cast<uint16_t>(first[e]) : 0u;
+                bits[4 + e] = ks * 32 + g * 8 + 4 + e < valid ? static_cast<uint16_t>(second[e]) : 0u;
+            }
+            const u32x4 packed = u32x4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                       bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
+            rows8[ks] = __builtin_bit_cast(bf16x8, packed);
+            if (is_k) {
+                // fragment (key tile, token step ks) of the record
+                *reinterpret_cast<u32x4*>(rec + kRecKt + (((col0 >> 4) * 2 + ks) * 64 + lane) * 16) = packed;
+            }
+        }
+        f32x4 w[4];
+#pragma unroll
+        for (uint32_t mt = 0; mt < 4; ++mt) {
+            f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ts_lo[mt][0], rows8[0], zero, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ts_hi[mt][0], rows8[0], acc, 0, 0, 0);
+            if (mt >= 2) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ts_lo[mt][1], rows8[1], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ts_hi[mt][1], rows8[1], acc, 0, 0, 0);
+            }
+            w[mt] = acc;
+        }
         // lane holds tokens 16mt+4g+i of column col0 + m
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; ++mt) {
