@@ -180,6 +180,14 @@ std::uint32_t attention_partitions(std::uint32_t context) {
                                         : (count + kAttentionPartition - 1) / kAttentionPartition;
 }
 
+std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
+                                std::uint32_t compute_units) noexcept {
+    const std::uint64_t units = std::max<std::uint32_t>(compute_units, 1);
+    const std::uint64_t per_group = (std::uint64_t{keys} * 2 * std::max<std::uint32_t>(rows, 1) + units - 1) / units;
+    const std::uint64_t rounded = (per_group + 31) / 32 * 32;
+    return static_cast<std::uint32_t>(std::clamp<std::uint64_t>(rounded, 128, 1024));
+}
+
 DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
     DecodePipelines p;
     HipPipelineError error = HipPipelineError::None;
@@ -337,8 +345,12 @@ DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
     DecodeBatchScratch b;
     b.rows = rows;
     const std::uint64_t table_bytes = step.schedule.size() * 16 * 4 * 4 + 64;
-    // split records: capacity / 32 partitions is the finest split the kernels take
-    const std::uint64_t record_bytes = std::uint64_t{rows} * g.attn_record_scratch_bytes;
+    // split records down to the finest split choose_split_keys picks (128 keys); the
+    // geometry's own figure is for the reference's 256-key partitions
+    const std::uint64_t finest_splits = (std::uint64_t{step.capacity} + 127) / 128;
+    const std::uint64_t record_bytes =
+        std::max<std::uint64_t>(g.attn_record_scratch_bytes,
+                                16 * finest_splits * kAttentionRecordFloats * kF32Bytes) * rows;
     if (!allocate_zeroed(device, rows * g.gdn_projection_bytes, b.gdn_projection) ||
         !allocate_zeroed(device, rows * g.gdn_qk_bytes, b.gdn_qk) ||
         !allocate_zeroed(device, rows * g.gdn_value_bytes, b.gdn_value) ||
@@ -446,8 +458,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
     const std::uint32_t rows = static_cast<std::uint32_t>(streams.size());
     if (rows == 0 || rows > batch.rows || rows > kMaximumBatchRows ||
         pool.layers.size() != step.schedule.size() || pool.stripes == 0 || !batch.state_offsets ||
-        weights.size() != step.schedule.size() || batch.split_keys == 0 ||
-        batch.split_keys % 32u != 0) {
+        weights.size() != step.schedule.size() || batch.split_keys % 32u != 0) {
         return HipCommandError::InvalidStreamGroup;
     }
     for (std::size_t index = 0; index < streams.size(); ++index) {
@@ -479,7 +490,21 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
     const std::uint64_t bucket_offset = step.schedule.size() * 256;
     bool any_long = false;
     for (const DecodeStream& s : streams) any_long |= attention_partitions(s.context) != 1;
-    const std::uint32_t max_splits = (step.capacity + batch.split_keys - 1) / batch.split_keys;
+    std::uint32_t longest = 1;
+    for (const DecodeStream& s : streams) longest = std::max(longest, s.context + 1);
+    // The grid always covers the capacity (the operator reads the contexts on the device
+    // and refuses a grid that could miss keys); a chosen split fits the longest lane of
+    // this wave, but no finer than 4096 workgroups over the capacity, most of which exit
+    // at once.
+    std::uint32_t split_keys = batch.split_keys;
+    if (split_keys == 0) {
+        const std::uint64_t coarsest =
+            (std::uint64_t{step.capacity} * 2 * rows + 4095) / 4096;
+        split_keys = std::max(choose_split_keys(rows, longest),
+                              static_cast<std::uint32_t>(std::min<std::uint64_t>(
+                                  (coarsest + 31) / 32 * 32, 1024)));
+    }
+    const std::uint32_t max_splits = (step.capacity + split_keys - 1) / split_keys;
     if (any_long && batch.attn_partials.size_bytes() <
                         std::uint64_t{rows} * 16 * max_splits * kAttentionRecordFloats * kF32Bytes) {
         return HipCommandError::InvalidBuffer;
@@ -572,7 +597,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                 walk.buffer(batch.attn_partials, 0, 4);
                 walk.constant(step.capacity, 5);
                 walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
-                walk.constant(batch.split_keys, 7);
+                walk.constant(split_keys, 7);
                 walk.constant(max_splits, 8);
                 walk.constant(1u, 9);
                 walk.dispatch(HipSize{max_splits, 2, rows}, HipSize{256, 1, 1});
@@ -582,7 +607,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                 walk.buffer(batch.attn_gate, 0, 1);
                 walk.buffer(batch.state_offsets, layer * 256, 2);
                 walk.buffer(batch.attn_attended, 0, 3);
-                walk.constant(batch.split_keys, 4);
+                walk.constant(split_keys, 4);
                 walk.constant(max_splits, 5);
                 walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
                 walk.constant(1u, 7);

@@ -193,11 +193,19 @@ struct DecodeBatchScratch {
     HipBuffer gdn_projection, gdn_qk, gdn_value, gdn_z, gdn_y, gdn_gated;
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended, attn_partials;
     HipBuffer state_offsets;
-    std::uint32_t split_keys{1024};      // keys per split-K workgroup of the batched path
+    // keys per split-K workgroup of the batched path (a multiple of 32); 0: chosen for
+    // every wave from its longest context by choose_split_keys
+    std::uint32_t split_keys{0};
     // One dispatch per Gated DeltaNet layer (gdn_decode_fused_ms) instead of the
     // reference's prepare / recurrence / gate-norm triple; same results bit for bit.
     bool gdn_fused{true};
 };
+
+// Keys per split-K workgroup with which one attention layer of a wave of `rows` lanes
+// fills the compute units about once (splits x 2 kv heads x rows ~ compute_units):
+// between 128 and 1024 keys, a multiple of 32.
+std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
+                                std::uint32_t compute_units = 256) noexcept;
 
 // The step: geometry, schedule and pipelines; its own primary slot (decode_step.h:115-153).
 struct DecodeStep {

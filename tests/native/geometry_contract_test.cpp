@@ -52,6 +52,13 @@ int main() {
         attention_partitions(512) != 3 || attention_partitions(32767) != 128) {
         return 18;
     }
+    // split choice: splits x 2 kv heads x lanes ~ 256 compute units, 128..1024 keys, x32
+    if (choose_split_keys(4, 32768) != 1024 || choose_split_keys(1, 32768) != 256 ||
+        choose_split_keys(1, 100000) != 800 || choose_split_keys(4, 16384) != 512 ||
+        choose_split_keys(1, 1) != 128 || choose_split_keys(16, 262144) != 1024 ||
+        choose_split_keys(0, 0, 0) != 128 || choose_split_keys(1, 20000) % 32 != 0) {
+        return 19;
+    }
 
     const PrefillPolicy policy{.schedule = PrefillSchedule::LayerMajor,
                                .context_capacity = 16384,

@@ -380,6 +380,7 @@ int main() {
         stages.streams = &hidden;
         for (int wave = 0; wave < 2; ++wave) {
             stages.matrix_unit = wave == 0;
+            batch.split_keys = wave == 0 ? 256 : 0;   // the second wave chooses its own split
             std::vector<std::uint16_t> x = gauss16(7400 + wave, kLanes * 2048);
             if (!upload(hidden.input, x)) return 206;
             std::vector<DecodeStream> streams;
