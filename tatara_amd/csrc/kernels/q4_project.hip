@@ -455,23 +455,32 @@ int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
 // latency: a workgroup owns 16 output rows and all input rows, its waves split K in slices
 // of 512 columns (eight groups each), every operand of a slice is requested before the
 // first is used, and the slices are summed through LDS in a fixed order.  Per group four
-// v_mfma_f32_16x16x16_bf16 multiply the x rows with the unpacked nibbles (lane g of a row
-// owns the group's columns 16 g .. 16 g + 15) and four more, against a ones operand, give
+// v_mfma_f32_16x16x16_bf16 multiply the x rows with the nibbles as bf16 128 + nibble (lane g
+// of a row owns the group's columns 16 g .. 16 g + 15) and four more, against a ones operand, give
 // the group sums of x; then acc += scale[n] * products + bias[n] * sums in fp32.  The
 // result has n along its columns, so a lane needs one scale and one bias per group, and
 // reads all eight of a slice with two 16-byte loads.
 
-// nibbles 0..3 of the low 16 bits of `half_word` -> four bf16 integers (exact)
-__device__ __forceinline__ bf16x4_bits unpack_four(uint32_t half_word) {
-    const uint32_t even = half_word & 0x0F0Fu;         // nibbles 0, 2 in bytes 0, 1
-    const uint32_t odd = (half_word >> 4) & 0x0F0Fu;   // nibbles 1, 3
+// nibbles 0..3 (upper = false) or 4..7 of `word` -> the four bf16 numbers 128 + nibble:
+// a nibble dropped into the low mantissa bits of bf16 128.0 (0x4300), whose unit in the
+// last place is one.  The offset leaves the products as 128 * (sum of x) too much, which
+// the caller takes out of the bias term.
+template <bool upper>
+__device__ __forceinline__ bf16x4_bits offset_four(uint32_t word) {
+    constexpr uint32_t kBase = 0x43004300u, kLow = 0x0000000Fu, kHigh = 0x000F0000u;
+    // nibble i sits at bits 4 i .. 4 i + 3; the even one of a pair goes to bits 0..3, the
+    // odd one to bits 16..19
     u32x2 out;
-    out[0] = (__float_as_uint(static_cast<float>(even & 0xFFu)) >> 16) |
-             (__float_as_uint(static_cast<float>(odd & 0xFFu)) & 0xFFFF0000u);
-    out[1] = (__float_as_uint(static_cast<float>(even >> 8)) >> 16) |
-             (__float_as_uint(static_cast<float>(odd >> 8)) & 0xFFFF0000u);
+    if (!upper) {
+        out[0] = ((word << 12) & kHigh) | ((word & kLow) | kBase);          // nibbles 0, 1
+        out[1] = ((word << 4) & kHigh) | (((word >> 8) & kLow) | kBase);    // nibbles 2, 3
+    } else {
+        out[0] = ((word >> 4) & kHigh) | (((word >> 16) & kLow) | kBase);   // nibbles 4, 5
+        out[1] = ((word >> 12) & kHigh) | (((word >> 24) & kLow) | kBase);  // nibbles 6, 7
+    }
     return __builtin_bit_cast(bf16x4_bits, out);
 }
+constexpr float kNibbleOffset = 128.0f;
 
 template <uint32_t kWaves>   // k_size / 512
 __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
@@ -511,12 +520,13 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
             const u32x2 x_bits = {x[group][j >> 1][2 * (j & 1)], x[group][j >> 1][2 * (j & 1) + 1]};
             const bf16x4_bits xf = __builtin_bit_cast(bf16x4_bits, x_bits);
             const uint32_t word = q[group][j >> 1];
-            const bf16x4_bits qf = unpack_four((j & 1) ? (word >> 16) : word);
+            const bf16x4_bits qf = (j & 1) ? offset_four<true>(word) : offset_four<false>(word);
             products = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xf, qf, products, 0, 0, 0);
             sums = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xf, ones, sums, 0, 0, 0);
         }
         const float scale = widen_half(scale_bits[group >> 1], group & 1);
-        const float bias = widen_half(bias_bits[group >> 1], group & 1);
+        // scale * (products - 128 sums) + bias * sums
+        const float bias = fmaf(-kNibbleOffset, scale, widen_half(bias_bits[group >> 1], group & 1));
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) acc[i] = fmaf(bias, sums[i], fmaf(scale, products[i], acc[i]));
     }

@@ -4,6 +4,7 @@ attention family (attention in-projection 2048 -> 9216, Gated DeltaNet in-projec
 `_mfma_ms` operators) and at block row counts (`_blk` operators), random weights.
 
     python -m tatara_amd.q4_sweep [--decode 1,4,16] [--block 256,2048,16384] [--repeats 5]
+                                  [--weight-sets 24]
 prints one JSON line per point: device microseconds per dispatch (best of the repeats,
 several dispatches per command buffer), MFMA-rate and weight-stream equivalents."""
 import argparse
@@ -40,13 +41,18 @@ def _bind(dev, family, rng):
     return bindings
 
 
-def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5, matrix_unit=False):
+def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5, matrix_unit=False,
+            weight_sets=1):
+    """weight_sets > 1 rotates that many distinct weight sets through the dispatches of a
+    command buffer: with more than 256 MB of them (the last-level cache) every dispatch
+    streams its weights from HBM, as the layers of a model do."""
     family = FAMILIES[name]
     rng = np.random.default_rng(rows)
     total, k = sum(family["segments"]), family["k"]
-    bindings = _bind(dev, family, rng)
-    bindings[0] = dev.buffer_from(_bf16(rng.standard_normal(rows * k)))
-    bindings[family["out"]] = dev.create_buffer(rows * total * 2)
+    weights = [_bind(dev, family, rng) for _ in range(weight_sets)]
+    shared = {0: dev.buffer_from(_bf16(rng.standard_normal(rows * k))),
+              family["out"]: dev.create_buffer(rows * total * 2)}
+    dispatches = max(dispatches, weight_sets)
     groups = (total + family["threads"] // 32 - 1) // (family["threads"] // 32)
     slot = family["out"] + 1
     if block:
@@ -64,14 +70,16 @@ def measure(dev, queue, lib, name, rows, block, repeats, dispatches=5, matrix_un
     for _ in range(repeats + 1):
         cb = queue.create_command_buffer()
         cb.begin_compute_pass()
-        for _ in range(dispatches):
-            cb.encode(pipeline, bindings, constants, grid, (family["threads"], 1, 1))
+        for index in range(dispatches):
+            cb.encode(pipeline, {**weights[index % weight_sets], **shared}, constants, grid,
+                      (family["threads"], 1, 1))
             cb.barrier()
         cb.end_compute_pass()
         ms = cb.commit().wait() / dispatches
         best = ms if best is None else min(best, ms)
     weight_bytes = total * k * (0.5 + 4.0 / 64.0)
-    return {"operator": operator, "rows": rows, "us": round(best * 1e3, 1),
+    return {"operator": operator, "rows": rows, "weight_sets": weight_sets,
+            "us": round(best * 1e3, 1),
             "tflops": round(2.0 * rows * total * k / best / 1e9, 1),
             "weight_gb_per_s": round(weight_bytes / best / 1e6, 1)}
 
@@ -81,6 +89,9 @@ def main():
     parser.add_argument("--decode", default="1,4,16")
     parser.add_argument("--block", default="256,2048,16384")
     parser.add_argument("--repeats", type=int, default=5)
+    parser.add_argument("--weight-sets", type=int, default=1,
+                        help="distinct weight sets rotated through a command buffer (24 keeps "
+                             "the decode forms out of the last-level cache)")
     args = parser.parse_args()
     dev = B.Device()
     queue = dev.create_queue()
@@ -88,11 +99,12 @@ def main():
     for block, rows_list in ((False, args.decode), (True, args.block)):
         for rows in [int(r) for r in rows_list.split(",") if r]:
             for name in FAMILIES:
-                print(json.dumps(measure(dev, queue, lib, name, rows, block, args.repeats)),
-                      flush=True)
+                sets = 1 if block else args.weight_sets
+                print(json.dumps(measure(dev, queue, lib, name, rows, block, args.repeats,
+                                         weight_sets=sets)), flush=True)
                 if not block:   # the same wave on the matrix unit
                     print(json.dumps(measure(dev, queue, lib, name, rows, block, args.repeats,
-                                             matrix_unit=True)), flush=True)
+                                             matrix_unit=True, weight_sets=sets)), flush=True)
 
 
 if __name__ == "__main__":
