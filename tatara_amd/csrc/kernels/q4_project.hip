@@ -482,9 +482,17 @@ __device__ __forceinline__ bf16x4_bits offset_four(uint32_t word) {
 }
 constexpr float kNibbleOffset = 128.0f;
 
+// bytes between the x rows staged in LDS: 16 more than a row, so that the sixteen lanes of
+// a fragment read (one row each, the same columns) fall on different banks
+template <uint32_t kWaves>
+constexpr uint32_t kWaveRowBytes = kWaves * 1024 + 16;
+
 template <uint32_t kWaves>   // k_size / 512
 __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
-    __shared__ float partial[kWaves][4][64];
+    // [rows][kWaveRowBytes] of x, then the waves' partial results
+    extern __shared__ __align__(16) uint8_t wave_lds[];
+    constexpr uint32_t kThreads = 64 * kWaves;
+    constexpr uint32_t kPiecesPerRow = kWaves * 64;          // 16-byte pieces of an x row
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t i16 = lane & 15, g = lane >> 4;
     const uint32_t n = blockIdx.x * 16 + i16;   // every matrix has a multiple of 16 rows
@@ -495,29 +503,51 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
     const uint32_t* words = p.words[segment] + local * (kWaves * 64) + first_group * 8 + 2 * g;
     const uint16_t* scales = p.scales[segment] + local * (kWaves * 8) + first_group;
     const uint16_t* biases = p.biases[segment] + local * (kWaves * 8) + first_group;
-    const uint16_t* x_row = p.input + static_cast<uint64_t>(min(i16, p.rows - 1)) * p.input_stride +
-                            first_group * kQ4Group + 16 * g;
 
+    // The x rows are the same for every workgroup: they come in once with coalesced 16-byte
+    // loads (requested first, so that storing them does not wait for the weights) and are
+    // read back from LDS as fragments; each lane loading its own 32 bytes per group from
+    // global memory cost as much as streaming the weights.
+    float* partial = reinterpret_cast<float*>(wave_lds + p.rows * kWaveRowBytes<kWaves>);
+    for (uint32_t piece = threadIdx.x; piece < p.rows * kPiecesPerRow; piece += 4 * kThreads) {
+        u32x4 staged[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
+            staged[j] = *reinterpret_cast<const u32x4*>(
+                p.input + static_cast<uint64_t>(at / kPiecesPerRow) * p.input_stride +
+                (at % kPiecesPerRow) * 8);
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
+            *reinterpret_cast<u32x4*>(wave_lds + (at / kPiecesPerRow) * kWaveRowBytes<kWaves> +
+                                      (at % kPiecesPerRow) * 16) = staged[j];
+        }
+    }
     u32x2 q[8];
-    u32x4 x[8][2];
 #pragma unroll
     for (uint32_t group = 0; group < 8; ++group) {
         q[group] = *reinterpret_cast<const u32x2*>(words + group * 8);
-        x[group][0] = *reinterpret_cast<const u32x4*>(x_row + group * kQ4Group);
-        x[group][1] = *reinterpret_cast<const u32x4*>(x_row + group * kQ4Group + 8);
     }
     const u32x4 scale_bits = *reinterpret_cast<const u32x4*>(scales);
     const u32x4 bias_bits = *reinterpret_cast<const u32x4*>(biases);
+    __syncthreads();
 
+    const uint8_t* x_row = wave_lds + min(i16, p.rows - 1) * kWaveRowBytes<kWaves> +
+                           first_group * (kQ4Group * 2) + 32 * g;
     const bf16x4_bits ones = {0x3F80, 0x3F80, 0x3F80, 0x3F80};
     const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     f32x4 acc = zero;
 #pragma unroll
     for (uint32_t group = 0; group < 8; ++group) {
+        const u32x4 x_low = *reinterpret_cast<const u32x4*>(x_row + group * (kQ4Group * 2));
+        const u32x4 x_high = *reinterpret_cast<const u32x4*>(x_row + group * (kQ4Group * 2) + 16);
         f32x4 products = zero, sums = zero;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            const u32x2 x_bits = {x[group][j >> 1][2 * (j & 1)], x[group][j >> 1][2 * (j & 1) + 1]};
+            const u32x4 half = j < 2 ? x_low : x_high;
+            const u32x2 x_bits = {half[2 * (j & 1)], half[2 * (j & 1) + 1]};
             const bf16x4_bits xf = __builtin_bit_cast(bf16x4_bits, x_bits);
             const uint32_t word = q[group][j >> 1];
             const bf16x4_bits qf = (j & 1) ? offset_four<true>(word) : offset_four<false>(word);
@@ -531,24 +561,35 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
         for (uint32_t i = 0; i < 4; ++i) acc[i] = fmaf(bias, sums[i], fmaf(scale, products[i], acc[i]));
     }
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) partial[wave][i][lane] = acc[i];
+    for (uint32_t i = 0; i < 4; ++i) partial[(wave * 4 + i) * 64 + lane] = acc[i];
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
     for (uint32_t i = 0; i < 4; ++i) {
-        float total = partial[0][i][lane];
+        float total = partial[i * 64 + lane];
 #pragma unroll
-        for (uint32_t w = 1; w < kWaves; ++w) total += partial[w][i][lane];
+        for (uint32_t w = 1; w < kWaves; ++w) total += partial[(w * 4 + i) * 64 + lane];
         const uint32_t m = 4 * g + i;   // the result has the input rows along its rows
         if (m < p.rows) p.output[static_cast<uint64_t>(m) * p.output_stride + n] = store16(total);
     }
 }
 
+template <uint32_t kWaves>
+constexpr uint32_t wave_lds_bytes(uint32_t rows) {
+    return rows * kWaveRowBytes<kWaves> + kWaves * 4 * 64 * 4;
+}
+
 int32_t launch_wave(const Q4Projection& p, hipStream_t stream) {
     const uint32_t out_rows = p.first_row[p.segments];
     switch (p.k_size / kQ4Block) {
-    case 4: hipLaunchKernelGGL(q4_wave_kernel<4>, dim3(out_rows / 16), dim3(256), 0, stream, p); break;
-    case 8: hipLaunchKernelGGL(q4_wave_kernel<8>, dim3(out_rows / 16), dim3(512), 0, stream, p); break;
+    case 4:
+        hipLaunchKernelGGL(q4_wave_kernel<4>, dim3(out_rows / 16), dim3(256),
+                           wave_lds_bytes<4>(p.rows), stream, p);
+        break;
+    case 8:
+        hipLaunchKernelGGL(q4_wave_kernel<8>, dim3(out_rows / 16), dim3(512),
+                           wave_lds_bytes<8>(p.rows), stream, p);
+        break;
     default: return TT_CMD_INVALID_DISPATCH_EXTENT;
     }
     return TT_OK;
@@ -735,7 +776,13 @@ int32_t op_outproj_blk(const Bindings& b, const Grid& g, hipStream_t s, bool v) 
 bool prepare_q4_kernels() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(q4_block_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kBlockLdsBytes) == hipSuccess;
+                               kBlockLdsBytes) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<4>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               wave_lds_bytes<4>(kQ4BatchRowsMax)) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<8>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               wave_lds_bytes<8>(kQ4BatchRowsMax)) == hipSuccess;
 }
 
 const KernelDesc kQ4ProjectKernels[] = {
