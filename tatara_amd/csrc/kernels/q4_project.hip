@@ -72,21 +72,37 @@ struct Q4Projection {
 // grid (ceil(out_rows / 8), ceil(rows / row_tile)) x 256: half wave h of a workgroup
 // owns output row 8 * blockIdx.x + h for the tile's input rows.  kBlocks = k_size / 512:
 // all of the row's nibbles, scales and biases are requested before the first is used, so
-// one row keeps kBlocks loads per lane in flight instead of one.
-template <uint32_t kBlocks>
+// one row keeps kBlocks loads per lane in flight instead of one.  The tile's x rows are
+// the same for all eight output rows: they come in once with coalesced 16-byte loads,
+// requested first, and are read back from LDS (every half wave fetching its own copy from
+// global memory cost as much as streaming the weights).  LDS layout of one 512-column
+// block of a row: the even 16-byte pieces, then the odd ones, so that the 32 lanes of a
+// half wave read 512 contiguous bytes twice.  Where the tiles of the workgroups that share
+// a compute unit do not fit its LDS (kStaged = false) x is read from global memory: there
+// the workgroups per compute unit matter more than the x traffic.
+template <uint32_t kBlocks, bool kStaged>
 __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
+    extern __shared__ __align__(16) uint8_t rows_lds[];   // [tile rows][kBlocks][1024]
+    constexpr uint32_t kPiecesPerRow = kBlocks * 64;
     const uint32_t lane = threadIdx.x & 31;
-    const uint32_t n = blockIdx.x * 8 + (threadIdx.x >> 5);
-    if (n >= p.first_row[p.segments]) return;
+    const uint32_t row_base = blockIdx.y * p.row_tile;
+    const uint32_t tile_rows = min(p.row_tile, p.rows - row_base);
+    for (uint32_t piece = threadIdx.x; kStaged && piece < tile_rows * kPiecesPerRow; piece += 256) {
+        const uint32_t r = piece / kPiecesPerRow, c = piece % kPiecesPerRow;
+        const u32x4 staged = *reinterpret_cast<const u32x4*>(
+            p.input + static_cast<uint64_t>(row_base + r) * p.input_stride + c * 8);
+        const uint32_t slot = (c & ~63u) + ((c & 63u) >> 1) + (c & 1u) * 32;
+        *reinterpret_cast<u32x4*>(rows_lds + (r * kPiecesPerRow + slot) * 16) = staged;
+    }
+    // rows past the last one compute on the last row and store nothing
+    const uint32_t n = min(blockIdx.x * 8 + (threadIdx.x >> 5), p.first_row[p.segments] - 1);
+    const bool stores = blockIdx.x * 8 + (threadIdx.x >> 5) < p.first_row[p.segments];
     uint32_t segment = 0;
     while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
     const uint32_t local = n - p.first_row[segment];
     const uint32_t* words = p.words[segment] + static_cast<uint64_t>(local) * (kBlocks * 64);
     const uint16_t* scales = p.scales[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
     const uint16_t* biases = p.biases[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
-    const uint32_t row_base = blockIdx.y * p.row_tile;
-    const uint32_t tile_rows = min(p.row_tile, p.rows - row_base);
-    const uint16_t* x0 = p.input + static_cast<uint64_t>(row_base) * p.input_stride + lane * 16;
 
     u32x2 packed[kBlocks];
     uint16_t scale_bits[kBlocks], bias_bits[kBlocks];
@@ -97,6 +113,8 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
         scale_bits[b] = scales[b * 8 + (lane >> 2)];
         bias_bits[b] = biases[b * 8 + (lane >> 2)];
     }
+    if (kStaged) __syncthreads();
+    const uint16_t* x0 = p.input + static_cast<uint64_t>(row_base) * p.input_stride + lane * 16;
     float acc[kQ4BatchRowsMax];
 #pragma unroll
     for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) acc[r] = 0.0f;
@@ -113,12 +131,20 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
         }
         const float scale = widen(scale_bits[b]);
         const float bias = widen(bias_bits[b]);
-        const uint16_t* xk = x0 + b * kQ4Block;
+        const uint8_t* xk = rows_lds + b * 1024 + lane * 16;
 #pragma unroll
         for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
             if (r < tile_rows) {
-                const u32x4* xr = reinterpret_cast<const u32x4*>(xk + r * p.input_stride);
-                const u32x4 lo = xr[0], hi = xr[1];
+                u32x4 lo, hi;
+                if (kStaged) {
+                    lo = *reinterpret_cast<const u32x4*>(xk + r * (kPiecesPerRow * 16));
+                    hi = *reinterpret_cast<const u32x4*>(xk + r * (kPiecesPerRow * 16) + 512);
+                } else {
+                    const u32x4* xr =
+                        reinterpret_cast<const u32x4*>(x0 + b * kQ4Block + r * p.input_stride);
+                    lo = xr[0];
+                    hi = xr[1];
+                }
                 float sum = 0.0f, quant = 0.0f;
 #pragma unroll
                 for (uint32_t i = 0; i < 4; ++i) {
@@ -140,20 +166,41 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
     for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
         if (r < tile_rows) {
             const float total = half_wave_sum(acc[r]);
-            if (lane == 0) {
+            if (lane == 0 && stores) {
                 p.output[static_cast<uint64_t>(row_base + r) * p.output_stride + n] = store16(total);
             }
         }
     }
 }
 
+constexpr uint32_t kRowsStagedBytes = 128 * 1024;   // of the 160 KB of a compute unit
+
 // 0 when the width has no instantiation
 int32_t launch_rows(const Q4Projection& p, hipStream_t stream) {
     const uint32_t out_rows = p.first_row[p.segments];
     const dim3 grid((out_rows + 7) / 8, (p.rows + p.row_tile - 1) / p.row_tile);
+    const uint32_t tile_rows = min(p.rows, p.row_tile);
+    // as many workgroups as the grid puts on a compute unit (up to eight) must still fit
+    const uint32_t resident = min(8u, (grid.x * grid.y + 255) / 256);
+    const auto staged = [&](uint32_t row_bytes) {
+        return tile_rows * row_bytes * resident <= kRowsStagedBytes;
+    };
     switch (p.k_size / kQ4Block) {
-    case 4: hipLaunchKernelGGL(q4_rows_kernel<4>, grid, dim3(256), 0, stream, p); break;
-    case 8: hipLaunchKernelGGL(q4_rows_kernel<8>, grid, dim3(256), 0, stream, p); break;
+    // LDS: the tile's x rows where they fit kRowsStagedBytes
+    case 4:
+        if (staged(4096)) {
+            hipLaunchKernelGGL((q4_rows_kernel<4, true>), grid, dim3(256), tile_rows * 4096, stream, p);
+        } else {
+            hipLaunchKernelGGL((q4_rows_kernel<4, false>), grid, dim3(256), 0, stream, p);
+        }
+        break;
+    case 8:
+        if (staged(8192)) {
+            hipLaunchKernelGGL((q4_rows_kernel<8, true>), grid, dim3(256), tile_rows * 8192, stream, p);
+        } else {
+            hipLaunchKernelGGL((q4_rows_kernel<8, false>), grid, dim3(256), 0, stream, p);
+        }
+        break;
     default: return TT_CMD_INVALID_DISPATCH_EXTENT;
     }
     return TT_OK;
@@ -777,6 +824,12 @@ bool prepare_q4_kernels() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(q4_block_kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                kBlockLdsBytes) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_rows_kernel<4, true>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kRowsStagedBytes) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_rows_kernel<8, true>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kRowsStagedBytes) == hipSuccess &&
            hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<4>),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                wave_lds_bytes<4>(kQ4BatchRowsMax)) == hipSuccess &&
