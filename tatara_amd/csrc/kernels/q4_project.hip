@@ -502,32 +502,33 @@ int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
 // latency: a workgroup owns 16 output rows and all input rows, its waves split K in slices
 // of 512 columns (eight groups each), every operand of a slice is requested before the
 // first is used, and the slices are summed through LDS in a fixed order.  Per group four
-// v_mfma_f32_16x16x16_bf16 multiply the x rows with the nibbles as bf16 128 + nibble (lane g
+// v_mfma_f32_16x16x16_bf16 multiply the x rows with the nibbles as bf16 16 + nibble (lane g
 // of a row owns the group's columns 16 g .. 16 g + 15) and four more, against a ones operand, give
 // the group sums of x; then acc += scale[n] * products + bias[n] * sums in fp32.  The
 // result has n along its columns, so a lane needs one scale and one bias per group, and
 // reads all eight of a slice with two 16-byte loads.
 
-// nibbles 0..3 (upper = false) or 4..7 of `word` -> the four bf16 numbers 128 + nibble:
-// a nibble dropped into the low mantissa bits of bf16 128.0 (0x4300), whose unit in the
-// last place is one.  The offset leaves the products as 128 * (sum of x) too much, which
-// the caller takes out of the bias term.
+// nibbles 0..3 (upper = false) or 4..7 of `word` -> the four bf16 numbers 16 + nibble: a
+// nibble dropped into mantissa bits 3..6 of bf16 16.0 (0x4180), where it counts units.  The
+// offset leaves the products as 16 * (sum of x) too much, which the caller takes out of the
+// bias term; 16 is the smallest offset that keeps all sixteen values in one binade, and
+// keeps the fp32 partial sums about three times as large as the plain ones.
 template <bool upper>
 __device__ __forceinline__ bf16x4_bits offset_four(uint32_t word) {
-    constexpr uint32_t kBase = 0x43004300u, kLow = 0x0000000Fu, kHigh = 0x000F0000u;
-    // nibble i sits at bits 4 i .. 4 i + 3; the even one of a pair goes to bits 0..3, the
-    // odd one to bits 16..19
+    constexpr uint32_t kBase = 0x41804180u, kLow = 0x00000078u, kHigh = 0x00780000u;
+    // nibble i sits at bits 4 i .. 4 i + 3; the even one of a pair goes to bits 3..6, the
+    // odd one to bits 19..22
     u32x2 out;
     if (!upper) {
-        out[0] = ((word << 12) & kHigh) | ((word & kLow) | kBase);          // nibbles 0, 1
-        out[1] = ((word << 4) & kHigh) | (((word >> 8) & kLow) | kBase);    // nibbles 2, 3
+        out[0] = ((word << 15) & kHigh) | (((word << 3) & kLow) | kBase);   // nibbles 0, 1
+        out[1] = ((word << 7) & kHigh) | (((word >> 5) & kLow) | kBase);    // nibbles 2, 3
     } else {
-        out[0] = ((word >> 4) & kHigh) | (((word >> 16) & kLow) | kBase);   // nibbles 4, 5
-        out[1] = ((word >> 12) & kHigh) | (((word >> 24) & kLow) | kBase);  // nibbles 6, 7
+        out[0] = ((word >> 1) & kHigh) | (((word >> 13) & kLow) | kBase);   // nibbles 4, 5
+        out[1] = ((word >> 9) & kHigh) | (((word >> 21) & kLow) | kBase);   // nibbles 6, 7
     }
     return __builtin_bit_cast(bf16x4_bits, out);
 }
-constexpr float kNibbleOffset = 128.0f;
+constexpr float kNibbleOffset = 16.0f;
 
 // bytes between the x rows staged in LDS: 16 more than a row, so that the sixteen lanes of
 // a fragment read (one row each, the same columns) fall on different banks
@@ -602,7 +603,7 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
             sums = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(xf, ones, sums, 0, 0, 0);
         }
         const float scale = widen_half(scale_bits[group >> 1], group & 1);
-        // scale * (products - 128 sums) + bias * sums
+        // scale * (products - 16 sums) + bias * sums
         const float bias = fmaf(-kNibbleOffset, scale, widen_half(bias_bits[group >> 1], group & 1));
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) acc[i] = fmaf(bias, sums[i], fmaf(scale, products[i], acc[i]));
