@@ -482,6 +482,35 @@ int main() {
                                *pass.compute_pass) != HipCommandError::InvalidStreamGroup) {
             return 228;
         }
+        // one fresh lane through encode_token (the un-batched operators) and through a
+        // batch of one: the stages hand both the same rows, bit for bit
+        auto lone = create_decode_state_slot(*device.device, step);
+        auto lone_pool = create_decode_state_slot_pool(*device.device, step, 1);
+        auto lone_scratch = create_decode_batch_scratch(*device.device, step, 1);
+        auto lone_hidden = create_hidden_streams(*device.device, geometry, 1);
+        if (!lone || !lone_pool || !lone_scratch || !lone_hidden) return 229;
+        QuantizedLayerStages single = stages;
+        single.scratch = &*lone_scratch.scratch;
+        single.streams = &*lone_hidden.streams;
+        if (!upload(lone_hidden.streams->input, gauss16(7600, 2048))) return 229;
+        int rc = submit.run([&](HipComputePass& p) {
+            return encode_token(step, *lone.slot, *lone_scratch.scratch, bound, single.hooks(), p, 0);
+        });
+        if (rc != 0) return 229;
+        const auto lone_residual = download<std::uint16_t>(lone_hidden.streams->residual, 2048);
+        const auto lone_normed = download<std::uint16_t>(lone_hidden.streams->normed, 2048);
+        std::vector<DecodeStream> one{{&lone_pool.slots[0], 0, 0}};
+        rc = submit.run([&](HipComputePass& p) {
+            return encode_token_batch(step, one, *lone_pool.pool, *lone_scratch.scratch, bound,
+                                      single.hooks(), p);
+        });
+        if (rc != 0) return 229;
+        if (lone_residual.empty() ||
+            download<std::uint16_t>(lone_hidden.streams->residual, 2048) != lone_residual ||
+            download<std::uint16_t>(lone_hidden.streams->normed, 2048) != lone_normed) {
+            return 229;
+        }
+        std::printf("[case] one lane: encode_token and a batch of one agree bit for bit\n");
     }
 
     // ---- block prefill on a private slot: 100 rows in chunks of 64, with the
