@@ -18,6 +18,8 @@
 // instruction moves two rows = 1 KiB contiguous.  The 32-lane sums are xor
 // butterflies (1,2,4,8,16), which is the adjacent-pairs tree of the reference
 // bit for bit.
+#include <type_traits>
+
 #include "../tt_internal.h"
 
 namespace tt {
@@ -49,9 +51,44 @@ __device__ __forceinline__ float sigmoid_bf16(float x) {
     return x < 0.0f ? low : rb(1.0f - low);
 }
 
+// Sum over the 32 lanes of a half wave, every lane receiving it, as the xor butterfly
+// (1, 2, 4, 8, 16) - the adjacent-pairs tree.  The partner of the first two steps comes
+// through quad permutes; after them a quad holds one value, so the mirror of a half row
+// (lane 7 - i) and of a row (lane 15 - i) deliver what lanes i ^ 4 and i ^ 8 hold; the
+// last step swaps the two rows of the half wave with a bit-mask swizzle.  Same sums bit
+// for bit as five __shfl_xor steps (fp addition commutes), without their LDS-permute
+// round trips.
 __device__ __forceinline__ float half_wave_sum(float v) {
-    for (uint32_t off = 1; off < 32; off <<= 1) v += __shfl_xor(v, off, 64);
+    const auto dpp = [](float x, auto ctrl) {
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
+                                                          0xF, 0xF, false));
+    };
+    v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
+    v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
+    v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
+    v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
+    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));  // lane ^ 16
     return v;
+}
+
+// The same butterfly over the 16 lanes of a row (xor 1, 2, 4, 8).
+__device__ __forceinline__ float row_sum(float v) {
+    const auto dpp = [](float x, auto ctrl) {
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
+                                                          0xF, 0xF, false));
+    };
+    v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
+    v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
+    v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
+    v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
+    return v;
+}
+// The value quad lane kLane holds, in every lane of its quad: on lane 4k that is what
+// __shfl_down by kLane delivers.
+template <int kLane>
+__device__ __forceinline__ float quad_lane(float v) {
+    return __int_as_float(
+        __builtin_amdgcn_update_dpp(0, __float_as_int(v), kLane * 0x55, 0xF, 0xF, false));
 }
 
 // decay and beta of one value head from the a / b projection rows
@@ -140,16 +177,16 @@ __global__ __launch_bounds__(128) void gdn_prepare_kernel(PrepareArgs a) {
             // RMS over the head: lane l (< 32) sums values 4l..4l+3, then the tree
             float sq = act * act;
             // gather 4 consecutive squares in ascending order onto lane 4k
-            const float s1 = __shfl_down(sq, 1, 64);
-            const float s2 = __shfl_down(sq, 2, 64);
-            const float s3 = __shfl_down(sq, 3, 64);
+            const float s1 = quad_lane<1>(sq);
+            const float s2 = quad_lane<2>(sq);
+            const float s3 = quad_lane<3>(sq);
             const float neighbour_sum = ((sq + s1) + s2) + s3;
             // lanes 4k hold thread-k partials; bring them to lanes 0..15 of each wave
             const uint32_t wave = lane >> 6;
             const uint32_t wl = lane & 63;
             float v = __shfl(neighbour_sum, (wl & 15) * 4, 64);  // 16 partials per wave
             // adjacent-pairs over 32 partials = pairs within each wave, then across
-            for (uint32_t off = 1; off < 16; off <<= 1) v += __shfl_xor(v, off, 64);
+            v = row_sum(v);
             __syncthreads();  // the previous row's readers are done with `partial`
             if (wl == 0) partial[wave] = v;
             __syncthreads();
@@ -247,7 +284,7 @@ __global__ __launch_bounds__(256) void gdn_prepare_block_kernel(PrepareArgs a) {
             const float run0 = ((act[0] * act[0] + act[1] * act[1]) + act[2] * act[2]) + act[3] * act[3];
             const float run1 = ((act[4] * act[4] + act[5] * act[5]) + act[6] * act[6]) + act[7] * act[7];
             float total = run0 + run1;
-            for (uint32_t off = 1; off < 16; off <<= 1) total += __shfl_xor(total, off, 64);
+            total = row_sum(total);
             const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
@@ -438,13 +475,13 @@ __global__ __launch_bounds__(128) void gdn_gate_norm_kernel(const uint16_t* y, c
         const uint64_t at = static_cast<uint64_t>(row) * stride + head * kGD + lane;
         const float v = widen(y[at]);
         const float sq = v * v;
-        const float s1 = __shfl_down(sq, 1, 64);
-        const float s2 = __shfl_down(sq, 2, 64);
-        const float s3 = __shfl_down(sq, 3, 64);
+        const float s1 = quad_lane<1>(sq);
+        const float s2 = quad_lane<2>(sq);
+        const float s3 = quad_lane<3>(sq);
         const float four = ((sq + s1) + s2) + s3;
         const uint32_t wl = lane & 63;
         float t = __shfl(four, (wl & 15) * 4, 64);
-        for (uint32_t off = 1; off < 16; off <<= 1) t += __shfl_xor(t, off, 64);
+        t = row_sum(t);
         __syncthreads();  // the previous row's readers are done with `partial`
         if (wl == 0) partial[lane >> 6] = t;
         __syncthreads();
@@ -482,7 +519,7 @@ __global__ __launch_bounds__(256) void gdn_gate_norm_block_kernel(
         const float run0 = ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3];
         const float run1 = ((v[4] * v[4] + v[5] * v[5]) + v[6] * v[6]) + v[7] * v[7];
         float total = run0 + run1;
-        for (uint32_t off = 1; off < 16; off <<= 1) total += __shfl_xor(total, off, 64);
+        total = row_sum(total);
         const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
         float r[8];
 #pragma unroll
@@ -583,7 +620,7 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     if (tid < 64) {  // lanes 0..31: q head, 32..63: k head; lane l sums squares 4l..4l+3
         const float* v = act + (tid >> 5) * kGD + (tid & 31) * 4;
         float sum = ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3];
-        for (uint32_t off = 1; off < 32; off <<= 1) sum += __shfl_xor(sum, off, 64);
+        sum = half_wave_sum(sum);
         if ((tid & 31) == 0) {
             inverse[tid >> 5] = 1.0f / sqrtf(sum / static_cast<float>(kGD) + kRmsNormEpsilon);
         }
@@ -629,13 +666,13 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     if (tid < kGD) {
         const float v = y_head[tid];
         const float sq = v * v;
-        const float s1 = __shfl_down(sq, 1, 64);
-        const float s2 = __shfl_down(sq, 2, 64);
-        const float s3 = __shfl_down(sq, 3, 64);
+        const float s1 = quad_lane<1>(sq);
+        const float s2 = quad_lane<2>(sq);
+        const float s3 = quad_lane<3>(sq);
         const float four = ((sq + s1) + s2) + s3;
         const uint32_t wl = tid & 63;
         float t = __shfl(four, (wl & 15) * 4, 64);
-        for (uint32_t off = 1; off < 16; off <<= 1) t += __shfl_xor(t, off, 64);
+        t = row_sum(t);
         if (wl == 0) partial[tid >> 6] = t;
     }
     __syncthreads();
