@@ -31,6 +31,7 @@
 // arithmetic runs at a few percent of MFMA peak, so the kernel is bound by how
 // many loads are in flight, not by compute.
 #include "../tt_internal.h"
+#include "lane_sums.h"
 
 namespace tt {
 namespace {
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
                 const float v = bf16_bits_to_f32(proj[base + d * 4 + j]);
                 acc += v * v;
             }
-            for (uint32_t off = 1; off < 32; off <<= 1) acc += __shfl_xor(acc, off, 64);
+            acc = half_wave_sum(acc);
             const float total = acc + __shfl_xor(acc, 32, 64);
             if (d == 0) {
                 inverse_shared = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(192) void attn_qk_rope_block_kernel(RopeArgs a) {
             run1 += x[4 + j] * x[4 + j];
         }
         float acc = run0 + run1;
-        for (uint32_t off = 1; off < 16; off <<= 1) acc += __shfl_xor(acc, off, 64);
+        acc = row_sum(acc);
         const float total = acc + __shfl_xor(acc, 16, 64);
         const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
         float n[8];

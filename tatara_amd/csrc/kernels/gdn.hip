@@ -18,9 +18,8 @@
 // instruction moves two rows = 1 KiB contiguous.  The 32-lane sums are xor
 // butterflies (1,2,4,8,16), which is the adjacent-pairs tree of the reference
 // bit for bit.
-#include <type_traits>
-
 #include "../tt_internal.h"
+#include "lane_sums.h"
 
 namespace tt {
 namespace {
@@ -49,46 +48,6 @@ __device__ __forceinline__ float sigmoid_bf16(float x) {
     const float e = rb(expf(fabsf(x)));
     const float low = rb(1.0f / rb(1.0f + e));
     return x < 0.0f ? low : rb(1.0f - low);
-}
-
-// Sum over the 32 lanes of a half wave, every lane receiving it, as the xor butterfly
-// (1, 2, 4, 8, 16) - the adjacent-pairs tree.  The partner of the first two steps comes
-// through quad permutes; after them a quad holds one value, so the mirror of a half row
-// (lane 7 - i) and of a row (lane 15 - i) deliver what lanes i ^ 4 and i ^ 8 hold; the
-// last step swaps the two rows of the half wave with a bit-mask swizzle.  Same sums bit
-// for bit as five __shfl_xor steps (fp addition commutes), without their LDS-permute
-// round trips.
-__device__ __forceinline__ float half_wave_sum(float v) {
-    const auto dpp = [](float x, auto ctrl) {
-        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
-                                                          0xF, 0xF, false));
-    };
-    v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
-    v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
-    v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
-    v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
-    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));  // lane ^ 16
-    return v;
-}
-
-// The same butterfly over the 16 lanes of a row (xor 1, 2, 4, 8).
-__device__ __forceinline__ float row_sum(float v) {
-    const auto dpp = [](float x, auto ctrl) {
-        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
-                                                          0xF, 0xF, false));
-    };
-    v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
-    v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
-    v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
-    v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
-    return v;
-}
-// The value quad lane kLane holds, in every lane of its quad: on lane 4k that is what
-// __shfl_down by kLane delivers.
-template <int kLane>
-__device__ __forceinline__ float quad_lane(float v) {
-    return __int_as_float(
-        __builtin_amdgcn_update_dpp(0, __float_as_int(v), kLane * 0x55, 0xF, 0xF, false));
 }
 
 // decay and beta of one value head from the a / b projection rows

@@ -20,9 +20,8 @@
 //    sum_k x q per 64-column group runs on MFMA with fp32 accumulation and the affine
 //    terms (scale per group and output row, bias against the group sums of x) are
 //    applied in fp32 - the same mathematics in another summation order.
-#include <type_traits>
-
 #include "../tt_internal.h"
+#include "lane_sums.h"
 
 namespace tt {
 namespace {
@@ -50,25 +49,6 @@ __device__ __forceinline__ uint16_t store16(float v) {
     if ((b & 0x7F800000u) == 0x7F800000u) return static_cast<uint16_t>(b >> 16);
     const uint16_t h = static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
     return (h & 0x7F80u) ? h : static_cast<uint16_t>(h & 0x8000u);
-}
-// Sum over the 32 lanes of a half wave, every lane receiving it, as the xor butterfly
-// (1, 2, 4, 8, 16) - the adjacent-pairs tree.  The partner of the first two steps comes
-// through quad permutes; after them a quad holds one value, so the mirror of a half row
-// (lane 7 - i) and of a row (lane 15 - i) deliver what lanes i ^ 4 and i ^ 8 hold; the
-// last step swaps the two rows of the half wave with a bit-mask swizzle.  Same sums bit
-// for bit as five __shfl_xor steps (fp addition commutes), without their LDS-permute
-// round trips.
-__device__ __forceinline__ float half_wave_sum(float v) {
-    const auto dpp = [](float x, auto ctrl) {
-        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
-                                                          0xF, 0xF, false));
-    };
-    v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
-    v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
-    v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
-    v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
-    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));  // lane ^ 16
-    return v;
 }
 
 // A projection = up to four weight matrices stacked along the output rows.

@@ -12,6 +12,7 @@
 //   dense_bf16, add_bf16   no reference counterpart: the reference projects with
 //       4-bit weights (q4_dot.metal); here the weights are plain bf16.
 #include "../tt_internal.h"
+#include "lane_sums.h"
 
 namespace tt {
 namespace {
@@ -75,14 +76,14 @@ __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, c
     sum += x1 * x1;
     sum += x2 * x2;
     sum += x3 * x3;
-    for (uint32_t off = 1; off < 32; off <<= 1) sum += __shfl_xor(sum, off, 64);
+    sum = half_wave_sum(sum);
     if (t < 32) stage[t] = 0.0f;
     __syncthreads();
     if ((t & 31) == 0) stage[t >> 5] = sum;
     __syncthreads();
     if (t < 32) {
         float total = stage[t];
-        for (uint32_t off = 1; off < 32; off <<= 1) total += __shfl_xor(total, off, 64);
+        total = half_wave_sum(total);
         if (t == 0) inverse_norm = 1.0f / sqrtf(total / static_cast<float>(hidden) + kRmsNormEpsilon);
     }
     __syncthreads();
