@@ -564,6 +564,53 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
     }
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                         static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
+    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+    // Up to 32 partitions (a 32k context in splits of 1024 keys): every load is requested
+    // before the first is used - the numerators of all partitions by the lane that owns
+    // dimension d, their maxima and sums through uniform loads - so the kernel is one
+    // round trip to memory deep instead of one per stage; same operations in the same
+    // order as the general path below.
+    constexpr uint32_t kFastParts = 32;
+    if (nparts <= kFastParts) {
+        __shared__ __attribute__((aligned(16))) float part_max[kFastParts];
+        __shared__ __attribute__((aligned(16))) float part_sum[kFastParts];
+        float numerator[kFastParts];
+#pragma unroll
+        for (uint32_t p = 0; p < kFastParts; ++p) {
+            numerator[p] = base[static_cast<uint64_t>(min(p, nparts - 1)) * kAttnRecordFloats + d];
+        }
+        if (d < kFastParts) {
+            const float* rec = base + static_cast<uint64_t>(min(d, nparts - 1)) * kAttnRecordFloats;
+            part_max[d] = d < nparts ? rec[kD] : -INFINITY;
+            part_sum[d] = rec[kD + 1];
+        }
+        __syncthreads();
+        float pmax[kFastParts], psum[kFastParts];
+#pragma unroll
+        for (uint32_t p = 0; p < kFastParts; p += 4) {
+            const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
+            const f32x4 s4 = *reinterpret_cast<const f32x4*>(part_sum + p);
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u) {
+                pmax[p + u] = m4[u];
+                psum[p + u] = s4[u];
+            }
+        }
+        float gmax = -INFINITY;
+#pragma unroll
+        for (uint32_t p = 0; p < kFastParts; ++p) gmax = fmaxf(gmax, pmax[p]);
+        float acc = 0.0f, denom = 0.0f;
+#pragma unroll
+        for (uint32_t p = 0; p < kFastParts; ++p) {
+            if (p < nparts) {
+                const float w = pmax[p] == -INFINITY ? 0.0f : __expf(pmax[p] - gmax);
+                acc = fmaf(w, numerator[p], acc);
+                denom += w * psum[p];
+            }
+        }
+        a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
+        return;
+    }
     __shared__ float red[256];
     __shared__ float weight[256];
     __shared__ float wsum[256];
@@ -611,7 +658,6 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
             denom += wsum[p];
         }
     }
-    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
     a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
 }
 
