@@ -113,6 +113,10 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         if (position >= a.capacity) continue;  // a bad table row must not write outside the cache
         const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
         const float x = bf16_bits_to_f32(proj[base + d]);
+        // the gate (query heads) or value (kv heads) element this thread copies through:
+        // requested with x, not after the rotation
+        const uint16_t copied =
+            proj[is_query ? head * 2 * kD + kD + d : kAttnVRowOffset + local * kD + d];
         __syncthreads();  // the previous row's readers are done with the shared values
         if (d < 64) {
             float acc = 0.0f;
@@ -144,12 +148,12 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         if (is_query) {
             const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
             a.q_out[at] = stored;
-            a.gate_out[at] = proj[head * 2 * kD + kD + d];
+            a.gate_out[at] = copied;
         } else {
             const uint64_t at =
                 kv_offset + (static_cast<uint64_t>(local) * a.capacity + position) * kD + d;
             a.keys[at] = stored;
-            a.values[at] = proj[kAttnVRowOffset + local * kD + d];
+            a.values[at] = copied;
         }
     }
 }
