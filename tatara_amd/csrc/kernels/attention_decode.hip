@@ -117,6 +117,14 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         // requested with x, not after the rotation
         const uint16_t copied =
             proj[is_query ? head * 2 * kD + kD + d : kAttnVRowOffset + local * kD + d];
+        // the rotation's cosine and sine depend on the position only: evaluated while the
+        // loads above are in flight, not after the norm
+        float c = 1.0f, s = 0.0f;
+        if (d < 2 * kAttnRopePairs) {
+            const float theta = static_cast<float>(position) / inverse_frequency;
+            c = cosf(theta);
+            s = sinf(theta);
+        }
         __syncthreads();  // the previous row's readers are done with the shared values
         if (d < 64) {
             float acc = 0.0f;
@@ -138,9 +146,6 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         __syncthreads();
         float rotated = n;
         if (d < 2 * kAttnRopePairs) {
-            const float theta = static_cast<float>(position) / inverse_frequency;
-            const float c = cosf(theta);
-            const float s = sinf(theta);
             rotated = d < kAttnRopePairs ? fmaf(-normed[d + kAttnRopePairs], s, n * c)
                                          : fmaf(normed[d - kAttnRopePairs], s, n * c);
         }
