@@ -271,6 +271,7 @@ struct FlashArgs {
     uint32_t final_mode;        // 1: one workgroup sees every key, writes bf16 output
     uint32_t long_rows_only;    // 1: rows with a single partition are skipped
     uint32_t single_partition;  // keys of one reference partition (256)
+    uint32_t row_limit;         // rows the q / gate / out / table operands hold
 };
 
 // value of lane (l ^ 8) within each row of 16 lanes
@@ -293,7 +294,10 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     const uint32_t split = blockIdx.x;
     const uint32_t kvh = blockIdx.y;
     uint32_t row = blockIdx.z;
-    if (a.row_list != nullptr) row = a.row_list[row];
+    if (a.row_list != nullptr) {
+        row = a.row_list[row];
+        if (row >= a.row_limit) return;  // a bad list entry must not index outside the slabs
+    }
     uint64_t kv_offset = 0;
     uint32_t context = a.context;
     if (a.table != nullptr) {
@@ -570,6 +574,9 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
         const uint32_t n = a.table[row * 4 + 1] + 1;
         if (a.long_rows_only && n <= a.single_partition) return;
         nparts = (n + a.part - 1) / a.part;
+        // a table row the split kernel refused (context past the capacity the records were
+        // sized for) has no records: leave its output alone rather than read past them
+        if (nparts > a.record_splits) return;
     }
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                         static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
@@ -922,6 +929,17 @@ int32_t op_attention_decode_ms(const Bindings& b, const Grid& g, hipStream_t str
     f.out = a.buffer<uint16_t>(5, kQueryBytes);
     f.row_list = a.buffer<const uint32_t>(7, rows * 4);
     f.final_mode = 1;
+    // The row indices come from device memory: the kernel skips any that the smallest of
+    // the three slabs does not hold, so a stale list entry cannot reach outside them.
+    if (a.status == TT_OK) {
+        uint64_t held = kMaxBatchRows;
+        for (uint32_t index : {0u, 1u, 5u}) {
+            const uint64_t values = a.buffer_bytes(index) / 2;
+            held = std::min<uint64_t>(held, (values - kAttnQueryValues) / f.query_stride + 1);
+        }
+        f.row_limit = static_cast<uint32_t>(held);
+        a.require(rows <= f.row_limit, TT_CMD_INVALID_BUFFER_OFFSET);
+    }
     if (a.status != TT_OK || validate_only) return a.status;
     return launch_flash(f, 1, rows, stream);
 }

@@ -186,9 +186,12 @@ def test_decode_context_edges(ctx):
         check_bf16(b_o2.read(np.uint16), want, f"split part {part} ctx {ctx}")
 
 
-def _lane_batch(contexts, cap, part, seed):
+def _lane_batch(contexts, cap, part, seed, replays=0):
     """Lane-batched decode over a striped pool with a state table, long rows
-    through attention_decode_split_ms and short rows through attention_decode_ms."""
+    through attention_decode_split_ms and short rows through attention_decode_ms.
+    replays > 0: the recording is also compiled into a HIP graph and replayed that
+    many times with the outputs and records cleared in between; every replay must
+    reproduce the eager bits."""
     B, dev, queue, lib = gpu()
     rows = len(contexts)
     stripe = 2 * cap * 256          # elements per lane cache
@@ -239,6 +242,15 @@ def _lane_batch(contexts, cap, part, seed):
     got = b_o.read(np.uint16).reshape(rows, 4096)
     for r, ctx in enumerate(contexts):
         check_bf16(got[r], want[r], f"lane {r} ctx {ctx} (stripe {stripes[r]}, part {part})")
+    if replays:
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass(); rec(cb); cb.end_compute_pass()
+        cb.compile()
+        for replay in range(replays):
+            b_o.write(np.zeros(rows * 4096, np.uint16))
+            b_part.write(np.full(rows * 16 * max_splits * 258, np.nan, np.float32))
+            cb.commit().wait()
+            assert np.array_equal(b_o.read(np.uint16).reshape(rows, 4096), got), f"replay {replay}"
     return ms
 
 
@@ -252,6 +264,21 @@ def test_config3_four_ragged_lanes_at_depth():
     capacity-32768 pool."""
     print("[case] config 3: 4 ragged lanes 32768/30000/24576/8192", flush=True)
     _lane_batch([32767, 29999, 24575, 8191], 32768, 512, 0xC0F3)
+
+
+def test_headline_shape_four_lanes_32768_split_1024_graph_replay():
+    """The benchmark's own configuration: 4 lanes x 32768 visible keys, 1024 keys per
+    split (32 records per head: the all-loads-up-front combine), eager and as a
+    compiled walk."""
+    print("[case] headline shape: 4 x 32768, split 1024, graph replay", flush=True)
+    _lane_batch([32767] * 4, 32768, 1024, 0xBE7C, replays=3)
+
+
+def test_lane_batch_record_counts_straddle_32():
+    """Rows with 64, 33, 32, 31 and 1 records per head in one dispatch: both combine
+    paths (up to 32 records with every load up front, more than 32 staged) side by side."""
+    print("[case] lane batch, records per head 64/33/32/31/1", flush=True)
+    _lane_batch([8191, 4096, 4095, 3967, 100], 8192, 128, 0x5732, replays=2)
 
 
 def test_config3_single_lane_100k():

@@ -268,3 +268,42 @@ def test_grouped_chunk_recurrence_equals_the_two_stages():
                    4: dev.create_buffer(1024), 5: bufs["state_in"], 6: y2, 7: state2}, {8: rows},
                   (8, 32, 1), (256, 1, 1))
     assert e.value.status == 10
+
+
+def test_config4_gdn_prefill_16384_rows_against_token_loop():
+    """Config 4, Gated DeltaNet half at full size: 16384 tokens of one lane through conv,
+    gates, the chunk-64 recurrence (grouped operator, scratch for one 2048-row group as
+    the benchmark binds it) and the gate-norm, against the checker's token-by-token
+    scan.  The drift of y is reported per 2048-row group; the bar does not move."""
+    rows, group = 16384, 2048
+    print(f"[case] config 4: gdn block prefill, {rows} rows", flush=True)
+    B, dev, queue, lib = gpu()
+    weights = _weights()
+    proj, conv_state, state = _block(rows, 0xC0F4)
+    ref = _oracle_block(proj, conv_state, state, weights, rows)
+    bufs = _buffers(dev, proj, conv_state, state, weights, min(rows, group))
+    for name in ("qk", "value", "z", "y", "gated"):
+        bufs[name] = dev.create_buffer(rows * 8192)
+    bufs["decay"], bufs["beta"] = dev.create_buffer(rows * 128), dev.create_buffer(rows * 128)
+    bufs["proj"] = dev.buffer_from(proj.reshape(-1))
+
+    def rec(cb):
+        _encode_front(cb, lib, bufs, rows)
+        cb.encode(lib.pipeline("gdn_chunk_recurrence_blk"),
+                  {0: bufs["qk"], 1: bufs["value"], 2: bufs["decay"], 3: bufs["beta"],
+                   4: bufs["chunk"], 5: bufs["state_in"], 6: bufs["y"], 7: bufs["state_out"]},
+                  {8: rows}, (8, 32, 1), (256, 1, 1))
+        _encode_gate_norm(cb, lib, bufs, rows)
+    run(rec)
+    assert np.array_equal(bufs["conv_out"].read(np.uint16), ref["conv"])      # conv state: exact
+    y = bufs["y"].read(np.uint16).reshape(rows, 4096)
+    want_y = ref["y"].reshape(rows, 4096)
+    for first in range(0, rows, group):
+        g = ol.bf16_to_f32(y[first:first + group].reshape(-1))
+        w = ol.bf16_to_f32(want_y[first:first + group].reshape(-1))
+        err = np.abs(g - w)
+        print(f"[drift] y rows {first}..{first + group - 1}: max-abs {err.max():.3e} "
+              f"mean-abs {err.mean():.3e}", flush=True)
+    check_bf16(y, want_y, "config 4 chunked y, 16384 rows")
+    check_f32(bufs["state_out"].read(np.float32), ref["state"], "config 4 final state", 2e-3, 2e-4)
+    check_bf16(bufs["gated"].read(np.uint16), ref["gated"], "config 4 gated", ulps=4)

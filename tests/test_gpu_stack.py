@@ -180,3 +180,69 @@ def test_residual_rms_operators(rows, hidden):
     run(rec2)
     assert np.array_equal(b_b.read(np.uint16), sums)
     assert np.array_equal(b_norm.read(np.uint16), normed)
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 2048), (4, 2048), (7, 256), (2, 4096)])
+def test_rms_only_operators_bit_for_bit(rows, hidden):
+    """rms_only (one row) and rms_only_ms (strided rows, strides wider than the row):
+    every bf16 output is the checker's bit pattern."""
+    print(f"[case] rms_only rows={rows} hidden={hidden}", flush=True)
+    B, dev, queue, lib = gpu()
+    x = ol.gaussian_bf16(0xD1 + rows, rows * hidden, 0.0, 3.0)
+    w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0xD2, hidden))
+    want = np.zeros(rows * hidden, np.uint16)
+    o.tto_rms_only(x, w, rows, hidden, want)
+    b_w = dev.buffer_from(w)
+    if rows == 1:
+        b_x, b_o = dev.buffer_from(x), dev.create_buffer(hidden * 2)
+        run(lambda cb: cb.encode(lib.pipeline("rms_only"), {0: b_x, 1: b_w, 2: b_o}, {}, (1,),
+                                 (hidden // 4,)))
+        assert np.array_equal(b_o.read(np.uint16), want)
+        return
+    in_stride, out_stride = hidden + 64, hidden + 128
+    slab = np.full((rows, in_stride), 0x7FC0, np.uint16)        # NaN between the rows
+    slab[:, :hidden] = x.reshape(rows, hidden)
+    b_x = dev.buffer_from(slab.reshape(-1))
+    b_o = dev.create_buffer(rows * out_stride * 2)
+    run(lambda cb: cb.encode(lib.pipeline("rms_only_ms"), {0: b_x, 1: b_w, 2: b_o},
+                             {3: in_stride, 4: out_stride}, (1, rows), (hidden // 4,)))
+    got = b_o.read(np.uint16).reshape(rows, out_stride)
+    assert np.array_equal(got[:, :hidden].reshape(-1), want)
+    assert not got[:, hidden:].any()                             # nothing written past a row
+
+
+@pytest.mark.parametrize("rows,in_dim,out_dim", [(1, 2048, 9216), (4, 2048, 12352), (16, 4096, 2048),
+                                                 (37, 2048, 4096), (3, 64, 70)])
+def test_dense_bf16_operator(rows, in_dim, out_dim):
+    """The stub stack's dense projection against the checker (fp32 dot in ascending
+    order, one bf16 rounding); the matrix unit sums in another order, so the bar is the
+    path's output tolerance scaled to the magnitude of the sums, and most outputs are
+    the checker's bit pattern."""
+    print(f"[case] dense_bf16 rows={rows} in={in_dim} out={out_dim}", flush=True)
+    B, dev, queue, lib = gpu()
+    x = ol.gaussian_bf16(0xE1 + rows, rows * in_dim)
+    w = ol.gaussian_bf16(0xE2 + rows, out_dim * in_dim, 0.0, 1.0 / np.sqrt(in_dim))
+    want = np.zeros(rows * out_dim, np.uint16)
+    o.tto_dense_bf16(x, w, rows, in_dim, out_dim, want, THREADS)
+    b_x, b_w = dev.buffer_from(x), dev.buffer_from(w)
+    b_o = dev.create_buffer(rows * out_dim * 2)
+    run(lambda cb: cb.encode(lib.pipeline("dense_bf16"), {0: b_x, 1: b_w, 2: b_o},
+                             {3: rows, 4: in_dim, 5: out_dim},
+                             ((out_dim + 63) // 64, (rows + 15) // 16), (256,)))
+    got = b_o.read(np.uint16)
+    from gpu_util import check_bf16
+    check_bf16(got, want, f"dense_bf16 {rows}x{in_dim}x{out_dim}", ulps=1)
+    assert np.mean(got == want) > 0.97
+
+
+def test_add_bf16_operator_bit_for_bit():
+    print("[case] add_bf16", flush=True)
+    B, dev, queue, lib = gpu()
+    n = 5 * 2048 + 3
+    a = ol.gaussian_bf16(0xF1, n, 0.0, 2.0); b = ol.gaussian_bf16(0xF2, n)
+    want = np.zeros(n, np.uint16)
+    o.tto_add_bf16(a, b, n, want)
+    b_a, b_b = dev.buffer_from(a), dev.buffer_from(b)
+    run(lambda cb: cb.encode(lib.pipeline("add_bf16"), {0: b_a, 1: b_b, 2: b_a}, {3: n},
+                             ((n + 255) // 256,), (256,)))
+    assert np.array_equal(b_a.read(np.uint16), want)
