@@ -79,6 +79,9 @@ typedef enum tt_status {
     TT_CMD_ENCODER_CREATION_FAILED = 20,
     TT_CMD_INVALID_DEVICE = 27,
     TT_CMD_INVALID_STREAM_GROUP = 28,
+    /* no counterpart in MetalCommandError: a request needs more of the library's fixed
+     * device scratch than TT_STATIC_SCRATCH_BYTES (tt_attention_decode_lanes_static) */
+    TT_CMD_STATIC_SCRATCH_EXCEEDED = 40,
     TT_RES_INVALID_DEVICE = 101,
     TT_RES_SYSTEM_DEVICE_UNAVAILABLE = 102,
     TT_RES_COMMAND_QUEUE_CREATION_FAILED = 103,
@@ -232,6 +235,43 @@ const char* tt_command_name(const tt_command_buffer* command_buffer, uint32_t in
 int32_t tt_command_gpu_ms(tt_command_buffer* command_buffer, uint32_t index, double* ms_out);
 /* Discards the recording so the command buffer can be encoded afresh. */
 int32_t tt_command_buffer_reset(tt_command_buffer* command_buffer);
+
+/* ---- entry point that allocates nothing ---- */
+/* Has no counterpart in the reference.  It is for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It is the lane-batched split-K decode attention that a recording of
+ * `attention_decode_split_ms` followed by `attention_decode_combine_ms` runs (same
+ * kernels, same operands, same results bit for bit), launched directly on the queue's
+ * stream, with the split records - the scratch those two dispatches otherwise take as a
+ * caller-bound buffer - in a fixed array of TT_STATIC_SCRATCH_BYTES that the library's
+ * code object holds on every GPU it is loaded on until the process ends.  It calls no
+ * hipMalloc / hipFree and no allocating library routine.
+ *
+ *   q, gate, out     [rows][query_stride] bf16 slabs, 16 x 256 values used per row
+ *   keys_pool, values_pool   bf16 caches, row r's at element offset table[4r]
+ *   state_table      rows x {kv element offset, context, 0, 0} u32 in device memory
+ *   *_bytes          bytes readable / writable behind each pointer (validated like bound
+ *                    buffers: TT_CMD_INVALID_BUFFER for a null pointer,
+ *                    TT_CMD_INVALID_BUFFER_OFFSET for an extent too small)
+ *   rows 1..16, query_stride >= 4096, split_keys a positive multiple of 32
+ *
+ * Every row is processed (short contexts take one split).  The records need
+ * rows * 16 * ceil(capacity / split_keys) * 1032 bytes; a request beyond
+ * TT_STATIC_SCRATCH_BYTES returns TT_CMD_STATIC_SCRATCH_EXCEEDED and launches nothing
+ * (raise split_keys or lower rows).  All calls on one GPU share that GPU's array, which
+ * keeps the last call's records: every record a call reads was written by that call, so
+ * nothing needs clearing, but two calls that overlap in time on one GPU (different
+ * queues, or a replayed capture next to a direct call) race on it.  The call only
+ * enqueues; completion is the stream's (hipStreamSynchronize on
+ * tt_queue_native_stream, or a later tt_commit / tt_wait on the same queue). */
+#define TT_STATIC_SCRATCH_BYTES (8u << 20)
+int32_t tt_attention_decode_lanes_static(tt_queue* queue, const void* q, uint64_t q_bytes,
+                                         const void* gate, uint64_t gate_bytes,
+                                         const void* keys_pool, uint64_t keys_bytes,
+                                         const void* values_pool, uint64_t values_bytes,
+                                         const void* state_table, uint64_t table_bytes, void* out,
+                                         uint64_t out_bytes, uint32_t rows, uint32_t capacity,
+                                         uint32_t query_stride, uint32_t split_keys);
 
 #ifdef __cplusplus
 }

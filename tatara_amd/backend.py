@@ -28,7 +28,7 @@ EXPORTED_SYMBOLS = [
     "tt_pass_set_buffer", "tt_pass_set_bytes", "tt_pass_dispatch", "tt_pass_barrier",
     "tt_blit_copy", "tt_blit_fill", "tt_command_count", "tt_commit", "tt_wait",
     "tt_command_buffer_reset", "tt_command_buffer_compile", "tt_command_buffer_set_profiling",
-    "tt_command_name", "tt_command_gpu_ms",
+    "tt_command_name", "tt_command_gpu_ms", "tt_attention_decode_lanes_static",
 ]
 
 
@@ -100,6 +100,7 @@ def lib():
         "tt_command_buffer_set_profiling": (i32, [vp, i32]),
         "tt_command_name": (C.c_char_p, [vp, u32]),
         "tt_command_gpu_ms": (i32, [vp, u32, C.POINTER(C.c_double)]),
+        "tt_attention_decode_lanes_static": (i32, [vp] + [vp, u64] * 6 + [u32] * 4),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -182,6 +183,26 @@ class CommandQueue:
 
     def create_command_buffer(self):
         return CommandBuffer(self)
+
+    def attention_decode_lanes_static(self, q, gate, keys_pool, values_pool, state_table, out,
+                                      rows, capacity, query_stride, split_keys):
+        """tt_attention_decode_lanes_static: the lane-batched split-K decode launched directly
+        on this queue with its split records in the library's fixed device scratch (no
+        allocation).  Operands are Buffers or (Buffer, byte offset) pairs; only enqueues."""
+        args = []
+        for operand in (q, gate, keys_pool, values_pool, state_table, out):
+            buffer, offset = operand if isinstance(operand, tuple) else (operand, 0)
+            args += [C.c_void_p(buffer.device_pointer + offset),
+                     C.c_uint64(buffer.size_bytes - offset)]
+        _check(lib().tt_attention_decode_lanes_static(self.handle, *args, rows, capacity,
+                                                      query_stride, split_keys),
+               "attention_decode_lanes_static")
+
+    def synchronize(self):
+        """Blocks until everything enqueued on the queue's stream has completed (an empty
+        recording committed and waited on the same in-order stream)."""
+        cb = self.create_command_buffer()
+        cb.commit().wait()
 
     def __del__(self, _release=_release):
         _release(self, "tt_queue_destroy")

@@ -33,6 +33,12 @@
 #include "../tt_internal.h"
 #include "lane_sums.h"
 
+// Split records of tt_attention_decode_lanes_static: device memory that belongs to the
+// code object, one copy per GPU the library is loaded on, held until the process ends.
+// In host code this name is only a handle for hipGetSymbolAddress; the device address a
+// kernel may use is the one static_scratch() returns.
+static __device__ __align__(256) unsigned char scratch[TT_STATIC_SCRATCH_BYTES];
+
 namespace tt {
 namespace {
 
@@ -1108,13 +1114,57 @@ int32_t op_attention_values(const Bindings& b, const Grid& g, hipStream_t stream
 
 }  // namespace
 
-#if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
-bool prepare_decode_kernels() {
+// Host code that names `scratch` stays visible to the device pass of the compiler: that
+// is how it learns that the host refers to the static device variable and gives it a
+// symbol the runtime can resolve.
+namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};   // device address of `scratch`, per GPU
+bool g_decode_ready[kMaxDevices] = {};
+
+// Set-up of the current device, once per device: the large dynamic LDS opt-in of the
+// split kernel and the device address of this GPU's copy of `scratch`.  Neither call
+// allocates.  Called when a library is created and, for a caller that never created
+// one, by the first direct launch on the device.
+bool prepare_current_device() {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (g_decode_ready[device]) return true;
     // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kWaves * kWaveLdsBytes) == hipSuccess;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kWaves * kWaveLdsBytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    void* address = nullptr;
+    if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess || address == nullptr) {
+        (void)hipGetLastError();
+        return false;
+    }
+    g_static_scratch[device] = address;
+    g_decode_ready[device] = true;
+    return true;
 }
+
+// Device address of the current GPU's `scratch`; null before prepare_current_device().
+void* static_scratch() {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return g_static_scratch[device];
+}
+
+}  // namespace
+
+#if !defined(__HIP_DEVICE_COMPILE__)  // host-side tables of launchers
+bool prepare_decode_kernels() { return prepare_current_device(); }
 
 const KernelDesc kAttentionDecodeKernels[] = {
     {"attn_qk_rope", op_attn_qk_rope},
@@ -1134,3 +1184,67 @@ const uint32_t kAttentionDecodeKernelCount =
 #endif
 
 }  // namespace tt
+
+#if !defined(__HIP_DEVICE_COMPILE__)
+// Direct launch of the lane-batched split-K decode with its records in `scratch`: the
+// operand checks of op_attention_split_ms / op_attention_combine_ms on plain pointers,
+// then the same two kernels.  No allocation on any path.
+extern "C" int32_t tt_attention_decode_lanes_static(
+    tt_queue* queue, const void* q, uint64_t q_bytes, const void* gate, uint64_t gate_bytes,
+    const void* keys_pool, uint64_t keys_bytes, const void* values_pool, uint64_t values_bytes,
+    const void* state_table, uint64_t table_bytes, void* out, uint64_t out_bytes, uint32_t rows,
+    uint32_t capacity, uint32_t query_stride, uint32_t split_keys) {
+    using namespace tt;
+    hipStream_t stream = queue_stream(queue);
+    if (queue == nullptr || stream == nullptr) return TT_CMD_INVALID_COMMAND_QUEUE;
+    if (q == nullptr || gate == nullptr || keys_pool == nullptr || values_pool == nullptr ||
+        state_table == nullptr || out == nullptr) {
+        return TT_CMD_INVALID_BUFFER;
+    }
+    if (rows < 1 || rows > kMaxBatchRows || capacity == 0 || query_stride < kAttnQueryValues ||
+        split_keys == 0 || split_keys % kBlockKeys != 0) {
+        return TT_CMD_INVALID_DISPATCH_EXTENT;
+    }
+    const uint64_t slab_bytes =
+        (static_cast<uint64_t>(rows - 1) * query_stride + kAttnQueryValues) * 2;
+    if (q_bytes < slab_bytes || gate_bytes < slab_bytes || out_bytes < slab_bytes ||
+        keys_bytes < cache_bytes(capacity) || values_bytes < cache_bytes(capacity) ||
+        table_bytes < static_cast<uint64_t>(rows) * 16) {
+        return TT_CMD_INVALID_BUFFER_OFFSET;
+    }
+    const uint32_t splits = (capacity + split_keys - 1) / split_keys;
+    const uint64_t row_floats = static_cast<uint64_t>(kAttnQueryHeads) * splits * kAttnRecordFloats;
+    if (row_floats * rows * 4 > TT_STATIC_SCRATCH_BYTES) return TT_CMD_STATIC_SCRATCH_EXCEEDED;
+    if (!prepare_current_device()) return TT_CMD_INVALID_DEVICE;
+    float* records = static_cast<float*>(static_scratch());
+    if (records == nullptr) return TT_CMD_INVALID_DEVICE;
+
+    FlashArgs f{};
+    f.q = static_cast<const uint16_t*>(q);
+    f.keys = static_cast<const uint16_t*>(keys_pool);
+    f.values = static_cast<const uint16_t*>(values_pool);
+    f.table = static_cast<const uint32_t*>(state_table);
+    f.partials = records;
+    f.capacity = capacity;
+    f.part = split_keys;
+    f.record_splits = splits;
+    f.query_stride = query_stride;
+    f.partial_row_floats = row_floats;
+    f.single_partition = kAttnPartition;
+    launch_flash(f, splits, rows, stream);
+
+    CombineArgs c{};
+    c.partials = records;
+    c.gate = static_cast<const uint16_t*>(gate);
+    c.out = static_cast<uint16_t*>(out);
+    c.table = f.table;
+    c.part = split_keys;
+    c.record_splits = splits;
+    c.query_stride = query_stride;
+    c.partial_row_floats = row_floats;
+    c.single_partition = kAttnPartition;
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
+                       c);
+    return hipGetLastError() == hipSuccess ? TT_OK : TT_CMD_INVALID_PENDING_EXECUTION;
+}
+#endif

@@ -47,6 +47,12 @@ struct tt_pipeline {
     KernelDesc desc{};
 };
 
+namespace tt {
+hipStream_t queue_stream(const tt_queue* queue) {
+    return queue != nullptr ? queue->stream : nullptr;
+}
+}  // namespace tt
+
 namespace {
 
 enum class CommandKind : uint8_t { Dispatch, Copy, Fill };
@@ -174,6 +180,7 @@ const char* tt_status_name(int32_t status) {
     case TT_CMD_ENCODER_CREATION_FAILED: return "EncoderCreationFailed";
     case TT_CMD_INVALID_DEVICE: return "InvalidDevice";
     case TT_CMD_INVALID_STREAM_GROUP: return "InvalidStreamGroup";
+    case TT_CMD_STATIC_SCRATCH_EXCEEDED: return "StaticScratchExceeded";
     case TT_RES_INVALID_DEVICE: return "Resource.InvalidDevice";
     case TT_RES_SYSTEM_DEVICE_UNAVAILABLE: return "Resource.SystemDeviceUnavailable";
     case TT_RES_COMMAND_QUEUE_CREATION_FAILED: return "Resource.CommandQueueCreationFailed";

@@ -87,6 +87,10 @@ inline bool grid_is(const Grid& g, uint64_t gx, uint64_t gy, uint64_t gz, uint64
 int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream,
                             bool validate_only);
 
+// The HIP stream of a queue (tt_queue is defined by the C-ABI core), for entry points
+// that launch directly instead of recording.
+hipStream_t queue_stream(const tt_queue* queue);
+
 // One-time kernel attribute set-up (large dynamic LDS opt-in); called when a
 // library is created, so it never runs inside a stream capture.
 bool prepare_decode_kernels();
