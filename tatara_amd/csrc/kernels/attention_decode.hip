@@ -53,6 +53,9 @@ constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16640
 constexpr uint32_t kWaves = 4;
 constexpr uint32_t kMergeTileFloats = 20;   // 16 accumulator words of one MFMA + 4 pad
 constexpr uint32_t kMergeHeadFloats = 16 * kMergeTileFloats + 4;  // 324: head stride of the merge
+// Bound of the rows a state table may carry (decode_step.cpp:1007-1009).
+constexpr uint32_t kMaxBatchRows = 16;
+constexpr uint32_t kMaxStreams = kMaxBatchRows * kAttnKvHeads;  // (row, kv head) key streams
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -553,6 +556,532 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     }
 }
 
+// ------------------------------------------------- whole decode layer -------
+//
+// attention_decode_layer_ms: the attention layer of a token wave in one dispatch - qk-norm
+// and rotation of the new token, its K / V append, split-K attention over every lane's
+// cache and the gated combine (attn_qk_rope_ms + the split path + the combine of
+// decode_step.cpp:1231-1259 folded together).
+//
+// Work is dealt by keys, not by lane: a (row, kv head) pair is a stream of
+// ceil(context / 32) units of 32 cached keys (one empty unit when the cache is empty), the
+// streams are laid end to end, and workgroup g of G takes units [g U / G, (g + 1) U / G) of
+// the U in total - ragged lanes and deep single lanes load every workgroup alike.  A
+// workgroup's range may cross stream boundaries; each piece inside one stream is a
+// segment, processed like a split of flash_decode_kernel and stored as one record per
+// head.  Everything is derived from the contexts in the state table, so one compiled walk
+// serves every token.
+//
+// The new token never goes through the cache: whoever finishes a stream folds it in as
+// one more record {numerator = V row, max = its score, sum = 1} from the projection row,
+// and appends its K / V rows for later tokens.
+//
+// Finishing.  finish_in_kernel = 0: a second dispatch (attention_layer_finish_kernel, one
+// wave per head and row).  finish_in_kernel = 1: the workgroups of a stream count their
+// arrivals on a ticket and the last to arrive finishes the stream, so the layer is a single
+// dispatch.  Records then travel between compute units that do not share an L2: they are
+// written with agent-scope atomic stores (write-through, no cache-wide write-back), the
+// ticket is taken after those stores have been acknowledged, and the finisher invalidates
+// its caches (acquire fence) before it reads them.  No workgroup ever waits for another.
+
+struct LayerArgs {
+    const uint16_t* projection;   // [rows][projection_stride]: {q | gate} x 16, K x 2, V x 2
+    const uint16_t* q_weight;
+    const uint16_t* k_weight;
+    uint16_t* keys;               // pools; row r's cache at + table[4 r] elements
+    uint16_t* values;
+    const uint32_t* table;        // per row {kv element offset, context, -, -}
+    float* records;               // [groups + streams - 1][8][258]
+    uint32_t* tickets;            // [streams] arrivals, zero between launches
+    uint16_t* out;                // [rows][query_stride]
+    uint32_t capacity;
+    uint32_t projection_stride;
+    uint32_t query_stride;
+    uint32_t rows;
+    uint32_t groups;              // G: workgroups the units are dealt to
+    uint32_t finish_in_kernel;
+};
+
+// Units of stream `stream` (lanes beyond the streams and rows whose context lies outside
+// the cache hold none, so such a row is skipped by every workgroup alike).
+__device__ __forceinline__ uint32_t stream_units(const LayerArgs& a, uint32_t stream) {
+    if (stream >= a.rows * kAttnKvHeads) return 0;
+    const uint32_t context = a.table[(stream >> 1) * 4 + 1];
+    if (context >= a.capacity) return 0;
+    return max(1u, (context + kBlockKeys - 1) / kBlockKeys);
+}
+
+// Workgroup that holds unit u when U units are dealt to G workgroups in ranges
+// [g U / G, (g + 1) U / G): the largest g with g U / G <= u.
+__device__ __forceinline__ uint32_t group_of_unit(uint32_t u, uint32_t total, uint32_t groups) {
+    return static_cast<uint32_t>(((static_cast<uint64_t>(u) + 1) * groups - 1) / total);
+}
+
+// One head of 256 values through RMS norm, weight and rotation by one wave; lane l
+// receives dims l, l + 64, l + 128, l + 192 as the fp32 of the stored bf16.  Operation for
+// operation attn_qk_rope_kernel: lane l's four squares are thread l's there, the same
+// half-wave tree, the same rounding points, the same cosine and sine.
+struct HeadLoads {
+    uint32_t run[2];      // values 4 l .. 4 l + 3 (sum of squares)
+    uint16_t x[4];        // values l + 64 c
+    uint16_t w[4];
+};
+__device__ __forceinline__ HeadLoads load_head(const uint16_t* x, const uint16_t* weight,
+                                               uint32_t lane) {
+    HeadLoads h;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(x + lane * 4);
+    h.run[0] = words[0];
+    h.run[1] = words[1];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        h.x[c] = x[lane + 64 * c];
+        h.w[c] = weight[lane + 64 * c];
+    }
+    return h;
+}
+__device__ __forceinline__ void norm_rope_head(const HeadLoads& h, uint32_t position, uint32_t lane,
+                                               float (&out)[4]) {
+    float acc = 0.0f;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const float v = __uint_as_float((j & 1) ? (h.run[j >> 1] & 0xFFFF0000u)
+                                                : (h.run[j >> 1] << 16));
+        acc += v * v;
+    }
+    acc = half_wave_sum(acc);
+    const float total = acc + __shfl_xor(acc, 32, 64);
+    const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        out[c] = round_bf16(bf16_bits_to_f32(h.w[c]) * round_bf16(bf16_bits_to_f32(h.x[c]) * inverse));
+    }
+    // dims below 64 rotate: lane l holds dim l, its partner (l ^ 32) the other half of the pair
+    const uint32_t pair = lane & (kAttnRopePairs - 1);
+    const float inverse_frequency =
+        powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs));
+    const float theta = static_cast<float>(position) / inverse_frequency;
+    const float c = cosf(theta);
+    const float sn = sinf(theta);
+    const float n = out[0];
+    const float partner = __shfl_xor(n, kAttnRopePairs, 64);
+    const float rotated = lane < kAttnRopePairs ? fmaf(-partner, sn, n * c) : fmaf(partner, sn, n * c);
+    out[0] = round_bf16(rotated);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v = half_wave_sum(v);
+    return v + __shfl_xor(v, 32, 64);
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (uint32_t off = 32; off; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// One wave finishes one head of one row: merges the stream's `count` records (slots
+// first_slot ..), folds in the new token, applies the gate and writes the output row;
+// with write_kv it also appends the token's K and V rows.  q: dims lane + 64 c of the
+// roped query head (fp32 of bf16).
+__device__ __forceinline__ void finish_head(const LayerArgs& a, uint32_t row, uint32_t head,
+                                            uint32_t context, uint64_t kv_offset,
+                                            uint32_t first_slot, uint32_t count,
+                                            const float (&q)[4], bool write_kv, uint32_t lane) {
+    const uint32_t kvh = head / kAttnHeadsPerKv;
+    const uint32_t hl = head % kAttnHeadsPerKv;
+    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const HeadLoads kl = load_head(proj + kAttnQGateRows + kvh * kD, a.k_weight, lane);
+    uint16_t vraw[4], gate[4];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        vraw[c] = proj[kAttnVRowOffset + kvh * kD + lane + 64 * c];
+        gate[c] = proj[head * 2 * kD + kD + lane + 64 * c];
+    }
+    float kn[4];
+    norm_rope_head(kl, context, lane, kn);
+    if (write_kv) {
+        const uint64_t at = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            a.keys[at + 64 * c] = f32_to_bf16_bits(kn[c]);
+            a.values[at + 64 * c] = vraw[c];
+        }
+    }
+    float dot = 0.0f;
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) dot = fmaf(q[c], kn[c], dot);
+    const float s_new = wave_sum(dot) * kAttnScale;
+
+    const float* base = a.records + (static_cast<uint64_t>(first_slot) * kAttnHeadsPerKv + hl) *
+                                        kAttnRecordFloats;
+    constexpr uint64_t kSlotFloats = static_cast<uint64_t>(kAttnHeadsPerKv) * kAttnRecordFloats;
+    float lmax = -INFINITY;
+    for (uint32_t p = lane; p < count; p += 64) lmax = fmaxf(lmax, base[p * kSlotFloats + kD]);
+    const float gmax = fmaxf(wave_max(lmax), s_new);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float denom = 0.0f;
+    for (uint32_t p0 = 0; p0 < count; p0 += 64) {
+        float my_w = 0.0f, my_ws = 0.0f;
+        if (p0 + lane < count) {
+            const float* rec = base + (p0 + lane) * kSlotFloats;
+            const float pm = rec[kD];
+            my_w = pm == -INFINITY ? 0.0f : __expf(pm - gmax);
+            my_ws = my_w * rec[kD + 1];
+        }
+        const uint32_t batch = min(64u, count - p0);
+        for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
+            float num[8][4];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                const float* rec = base + (p0 + min(j0 + u, batch - 1)) * kSlotFloats + lane;
+#pragma unroll
+                for (uint32_t c = 0; c < 4; ++c) num[u][c] = rec[64 * c];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                const bool live = j0 + u < batch;
+                const float w = live ? __shfl(my_w, j0 + u, 64) : 0.0f;
+                const float ws = live ? __shfl(my_ws, j0 + u, 64) : 0.0f;
+#pragma unroll
+                for (uint32_t c = 0; c < 4; ++c) acc[c] = fmaf(w, num[u][c], acc[c]);
+                denom += ws;
+            }
+        }
+    }
+    const float w_new = __expf(s_new - gmax);
+    denom += w_new;
+    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + lane;
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        const float value = fmaf(w_new, bf16_bits_to_f32(vraw[c]), acc[c]);
+        a.out[at + 64 * c] = f32_to_bf16_bits((value / denom) * sigmoid_gate(gate[c]));
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // after the four K stages: the roped query heads of the segment's kv group (bf16),
+    // the stream offsets and the ticket broadcast
+    uint16_t* qs = reinterpret_cast<uint16_t*>(lds + kWaves * kWaveLdsBytes);
+    uint32_t* s_off = reinterpret_cast<uint32_t*>(lds + kWaves * kWaveLdsBytes +
+                                                  kAttnHeadsPerKv * kD * 2);
+    uint32_t* s_ticket = s_off + kMaxStreams + 1;
+
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t group = blockIdx.x;
+    const uint32_t streams = a.rows * kAttnKvHeads;
+
+    if (wave == 0) {
+        uint32_t inclusive = stream_units(a, lane);
+#pragma unroll
+        for (uint32_t off = 1; off < kMaxStreams; off <<= 1) {
+            const uint32_t below = __shfl_up(inclusive, off, 64);
+            if (lane >= off) inclusive += below;
+        }
+        if (lane < kMaxStreams) s_off[lane + 1] = inclusive;
+        if (lane == 0) s_off[0] = 0;
+    }
+    __syncthreads();
+    const uint32_t total = s_off[streams];
+    // with fewer units than workgroups the first `total` workgroups take one unit each, so
+    // the workgroups of a stream are always consecutive and none of them is empty
+    const uint32_t groups = min(a.groups, total);
+    if (group >= groups) return;
+    uint32_t unit = static_cast<uint32_t>(static_cast<uint64_t>(group) * total / groups);
+    const uint32_t unit_end =
+        static_cast<uint32_t>((static_cast<uint64_t>(group) + 1) * total / groups);
+    uint8_t* stage = lds + wave * kWaveLdsBytes;
+    uint32_t stream = 0;
+
+    while (unit < unit_end) {
+        while (s_off[stream + 1] <= unit) ++stream;
+        const uint32_t stream_first = s_off[stream];
+        const uint32_t stream_last = s_off[stream + 1];
+        const uint32_t segment_end = min(unit_end, stream_last);
+        const uint32_t row = stream >> 1;
+        const uint32_t kvh = stream & 1;
+        const uint64_t kv_offset = a.table[row * 4];
+        const uint32_t context = a.table[row * 4 + 1];
+        const uint32_t k0 = (unit - stream_first) * kBlockKeys;
+        const uint32_t k1 = min(context, (segment_end - stream_first) * kBlockKeys);
+        const uint32_t nblocks = k1 > k0 ? (k1 - k0 + kBlockKeys - 1) / kBlockKeys : 0u;
+        const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+        const uint16_t* kbase = a.keys + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
+        const uint16_t* vbase = a.values + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
+
+        // the wave's two query heads: their loads go out first, then the first block of
+        // keys and values, and the norm / rotation runs while that block is in flight
+        HeadLoads ql[2];
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            ql[i] = load_head(proj + (kvh * kAttnHeadsPerKv + wave * 2 + i) * 2 * kD, a.q_weight, lane);
+        }
+
+        auto stage_keys = [&](uint32_t blk) {
+            const uint32_t key0 = k0 + blk * kBlockKeys;
+            const uint32_t valid = min(kBlockKeys, k1 - key0);
+#pragma unroll
+            for (uint32_t i = 0; i < 16; ++i) {
+                const uint32_t key = min(i + (lane >> 5) * 16, valid - 1);
+                const uint16_t* src = kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(src),
+                    (__attribute__((address_space(3))) void*)(stage + i * kLdsPairBytes),
+                    16, 0, 0);
+            }
+        };
+        auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
+            const uint32_t key0 = k0 + blk * kBlockKeys;
+            const uint32_t valid = min(kBlockKeys, k1 - key0);
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
+                vhalf[e] = *reinterpret_cast<const u32x4*>(
+                    vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8);
+            }
+        };
+
+        u32x4 vreg[2][8];
+        if (wave < nblocks) {
+            stage_keys(wave);
+            load_values(vreg[0], wave, 0);
+            load_values(vreg[1], wave, 1);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            float n[4];
+            norm_rope_head(ql[i], context, lane, n);
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                qs[(wave * 2 + i) * kD + lane + 64 * c] = f32_to_bf16_bits(n[c]);
+            }
+        }
+        __syncthreads();
+        // B operand of S^T: Q^T, column m holds head (m & 7)
+        bf16x8 qreg[8];
+#pragma unroll
+        for (uint32_t kb = 0; kb < 8; ++kb) {
+            qreg[kb] = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(qs + (m & 7) * kD + kb * 32 + g * 8));
+        }
+
+        f32x4 o[16];
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) o[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        float m_run = -INFINITY;
+        float l_run = 0.0f;
+
+        for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
+            const uint32_t valid = min(kBlockKeys, k1 - (k0 + blk * kBlockKeys));
+            const bool more = blk + kWaves < nblocks;
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __builtin_amdgcn_wave_barrier();
+            f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f};
+            f32x4 s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t kb = 0; kb < 8; ++kb) {
+                const bf16x8 a0 = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes +
+                                                            (kb * 4 + g) * 16));
+                const bf16x8 a1 = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes + 512 +
+                                                            (kb * 4 + g) * 16));
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[kb], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[kb], s1, 0, 0, 0);
+            }
+            float sc[8];
+            float block_max = -INFINITY;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                sc[i] = (g * 4 + i) < valid ? s0[i] * kAttnScale : -INFINITY;
+                sc[4 + i] = (16 + g * 4 + i) < valid ? s1[i] * kAttnScale : -INFINITY;
+                block_max = fmaxf(block_max, fmaxf(sc[i], sc[4 + i]));
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (more) stage_keys(blk + kWaves);
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
+            const float m_new = fmaxf(m_run, block_max);
+            const float alpha = __expf(m_run - m_new);
+            float p[8];
+            float block_sum = 0.0f;
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                p[e] = __expf(sc[e] - m_new);
+                block_sum += p[e];
+            }
+            block_sum += __shfl_xor(block_sum, 16, 64);
+            block_sum += __shfl_xor(block_sum, 32, 64);
+            l_run = l_run * alpha + block_sum;
+            m_run = m_new;
+            uint32_t pw[4];
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                float x0 = p[2 * c];
+                float x1 = p[2 * c + 1];
+                if (m >= 8) {
+                    x0 -= round_bf16(x0);
+                    x1 -= round_bf16(x1);
+                }
+                pw[c] = static_cast<uint32_t>(f32_to_bf16_bits(x0)) |
+                        (static_cast<uint32_t>(f32_to_bf16_bits(x1)) << 16);
+            }
+            const bf16x8 pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                for (uint32_t j = 0; j < 16; ++j) o[j] *= alpha;
+            }
+#pragma unroll
+            for (uint32_t hh = 0; hh < 2; ++hh) {
+#pragma unroll
+                for (uint32_t dw = 0; dw < 4; ++dw) {
+                    u32x4 lo, hi;
+                    lo.x = pack_low(vreg[hh][0][dw], vreg[hh][1][dw]);
+                    lo.y = pack_low(vreg[hh][2][dw], vreg[hh][3][dw]);
+                    lo.z = pack_low(vreg[hh][4][dw], vreg[hh][5][dw]);
+                    lo.w = pack_low(vreg[hh][6][dw], vreg[hh][7][dw]);
+                    hi.x = pack_high(vreg[hh][0][dw], vreg[hh][1][dw]);
+                    hi.y = pack_high(vreg[hh][2][dw], vreg[hh][3][dw]);
+                    hi.z = pack_high(vreg[hh][4][dw], vreg[hh][5][dw]);
+                    hi.w = pack_high(vreg[hh][6][dw], vreg[hh][7][dw]);
+                    o[hh * 8 + 2 * dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, lo), pb, o[hh * 8 + 2 * dw], 0, 0, 0);
+                    o[hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, hi), pb, o[hh * 8 + 2 * dw + 1], 0, 0, 0);
+                }
+                if (more) load_values(vreg[hh], blk + kWaves, hh);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+
+        // the wave's {O[8][256], max, sum} into its own stage (layout as in flash_decode_kernel)
+        float* merge = reinterpret_cast<float*>(stage);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            f32x4 sum4;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) sum4[i] = o[j][i] + dpp_row_ror8(o[j][i]);
+            if (m < 8) {
+                *reinterpret_cast<f32x4*>(merge + m * kMergeHeadFloats + j * kMergeTileFloats +
+                                          g * 4) = sum4;
+            }
+        }
+        if (lane < 8) {
+            merge[8 * kMergeHeadFloats + lane * 2] = m_run;
+            merge[8 * kMergeHeadFloats + lane * 2 + 1] = l_run;
+        }
+        __syncthreads();
+
+        // cross-wave merge into the segment's record: slot = workgroup + stream
+        const uint32_t slot = group + stream;
+#pragma unroll
+        for (uint32_t hl = 0; hl < 2; ++hl) {
+            const uint32_t h = wave * 2 + hl;
+            float scale[kWaves];
+            float gmax = -INFINITY;
+            float lsum[kWaves];
+#pragma unroll
+            for (uint32_t w = 0; w < kWaves; ++w) {
+                const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
+                scale[w] = wm[8 * kMergeHeadFloats + h * 2];
+                lsum[w] = wm[8 * kMergeHeadFloats + h * 2 + 1];
+                gmax = fmaxf(gmax, scale[w]);
+            }
+            float denom = 0.0f;
+#pragma unroll
+            for (uint32_t w = 0; w < kWaves; ++w) {
+                scale[w] = scale[w] == -INFINITY ? 0.0f : __expf(scale[w] - gmax);
+                denom = fmaf(scale[w], lsum[w], denom);
+            }
+            float* record = a.records + (static_cast<uint64_t>(slot) * kAttnHeadsPerKv + h) *
+                                            kAttnRecordFloats;
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                const uint32_t d = lane + 64 * c;
+                const uint32_t at = ((d >> 7) * 8 + (d & 7)) * kMergeTileFloats + ((d & 127) >> 3);
+                float acc = 0.0f;
+#pragma unroll
+                for (uint32_t w = 0; w < kWaves; ++w) {
+                    const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
+                    acc = fmaf(scale[w], wm[h * kMergeHeadFloats + at], acc);
+                }
+                __hip_atomic_store(record + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (lane == 0) {
+                __hip_atomic_store(record + kD, gmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(record + kD + 1, denom, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+
+        if (a.finish_in_kernel) {
+            // the record stores have been acknowledged before the ticket is taken
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            const uint32_t first_group = group_of_unit(stream_first, total, groups);
+            const uint32_t count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
+            if (threadIdx.x == 0) {
+                *s_ticket = __hip_atomic_fetch_add(a.tickets + stream, 1u, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            if (*s_ticket == count - 1) {
+                // last to arrive: every record of the stream is in memory; drop what this
+                // compute unit's caches may hold of that memory, then finish two heads a wave
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll 1
+                for (uint32_t hl = 0; hl < 2; ++hl) {
+                    const uint32_t h = wave * 2 + hl;
+                    float q[4];
+#pragma unroll
+                    for (uint32_t c = 0; c < 4; ++c) q[c] = bf16_bits_to_f32(qs[h * kD + lane + 64 * c]);
+                    finish_head(a, row, kvh * kAttnHeadsPerKv + h, context, kv_offset,
+                                first_group + stream, count, q, h == 0, lane);
+                }
+                if (threadIdx.x == 0) {
+                    __hip_atomic_store(a.tickets + stream, 0u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        __syncthreads();  // the stages and the query heads are free for the next segment
+        unit = segment_end;
+    }
+}
+
+// Second dispatch of the two-dispatch form: grid (16 heads, rows) x 64, one wave per head.
+__global__ __launch_bounds__(64) void attention_layer_finish_kernel(LayerArgs a) {
+    const uint32_t head = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t stream = row * kAttnKvHeads + head / kAttnHeadsPerKv;
+    uint32_t inclusive = stream_units(a, lane);
+#pragma unroll
+    for (uint32_t off = 1; off < kMaxStreams; off <<= 1) {
+        const uint32_t below = __shfl_up(inclusive, off, 64);
+        if (lane >= off) inclusive += below;
+    }
+    const uint32_t total = __shfl(inclusive, a.rows * kAttnKvHeads - 1, 64);
+    const uint32_t stream_last = __shfl(inclusive, stream, 64);
+    const uint32_t below = __shfl(inclusive, stream == 0 ? 0 : stream - 1, 64);
+    const uint32_t stream_first = stream == 0 ? 0u : below;
+    if (stream_last == stream_first) return;   // a row the table places outside its cache
+    const uint32_t groups = min(a.groups, total);
+    const uint32_t first_group = group_of_unit(stream_first, total, groups);
+    const uint32_t count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
+    const uint64_t kv_offset = a.table[row * 4];
+    const uint32_t context = a.table[row * 4 + 1];
+    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const HeadLoads ql = load_head(proj + head * 2 * kD, a.q_weight, lane);
+    float q[4];
+    norm_rope_head(ql, context, lane, q);
+    finish_head(a, row, head, context, kv_offset, first_group + stream, count, q,
+                head % kAttnHeadsPerKv == 0, lane);
+}
+
 // ----------------------------------------------------------------- combine ---
 
 struct CombineArgs {
@@ -817,9 +1346,6 @@ int32_t op_attn_qk_rope(const Bindings& b, const Grid& g, hipStream_t stream, bo
     return launch_rope(r, 1, stream);
 }
 
-// Host-side bound of the rows a state table may carry (decode_step.cpp:1007-1009).
-constexpr uint32_t kMaxBatchRows = 16;
-
 // attn_qk_rope_ms: b0 projection slab, b1 q_w, b2 k_w, b3 q slab, b4 gate slab,
 // b5 keys_pool, b6 values_pool, c7 capacity, b8 state_table, c9 projection
 // stride, c10 query stride; grid (18, rows) x 256 (decode_step.cpp:1231-1243).
@@ -1065,6 +1591,84 @@ int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t st
     return TT_OK;
 }
 
+constexpr uint32_t kLayerLdsBytes =
+    kWaves * kWaveLdsBytes + kAttnHeadsPerKv * kD * 2 + (kMaxStreams + 2) * 4;
+constexpr uint32_t kLayerTicketBytes = 256;   // tickets lead the scratch, records follow
+constexpr uint32_t kMaxLayerGroups = 4096;
+
+uint64_t layer_scratch_bytes(uint32_t groups, uint32_t rows) {
+    return kLayerTicketBytes + static_cast<uint64_t>(groups + rows * kAttnKvHeads - 1) *
+                                   kAttnHeadsPerKv * kAttnRecordFloats * 4;
+}
+
+// Bindings shared by the two dispatches of the whole-layer decode: b0 projection slab
+// [rows][projection stride], b1 q_w, b2 k_w, b3 keys_pool, b4 values_pool, b5 state_table,
+// b6 scratch (256 B of tickets, then (groups + 2 rows - 1) x 8 records of 258 floats; zero
+// before the first use, left zeroed by every launch), b7 out slab [rows][query stride],
+// c8 capacity, c9 projection stride, c10 query stride.
+LayerArgs layer_args(Args& a, uint32_t rows, uint32_t groups) {
+    LayerArgs l{};
+    l.capacity = a.constant(8);
+    l.projection_stride = a.constant(9);
+    l.query_stride = a.constant(10);
+    l.rows = rows;
+    l.groups = groups;
+    a.require(rows >= 1 && rows <= kMaxBatchRows && groups >= 1 && groups <= kMaxLayerGroups,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(l.capacity != 0 && l.projection_stride >= kAttnProjectionRows &&
+                  l.projection_stride % 4 == 0 && l.query_stride >= kAttnQueryValues,
+              TT_CMD_INVALID_BUFFER);
+    if (a.status != TT_OK) return l;
+    const uint64_t last = rows - 1;
+    l.projection =
+        a.buffer<const uint16_t>(0, (last * l.projection_stride + kAttnProjectionRows) * 2);
+    l.q_weight = a.buffer<const uint16_t>(1, kD * 2);
+    l.k_weight = a.buffer<const uint16_t>(2, kD * 2);
+    l.keys = a.buffer<uint16_t>(3, cache_bytes(l.capacity));
+    l.values = a.buffer<uint16_t>(4, cache_bytes(l.capacity));
+    l.table = a.buffer<const uint32_t>(5, rows * 16);
+    uint8_t* scratch_base = a.buffer<uint8_t>(6, layer_scratch_bytes(groups, rows));
+    l.out = a.buffer<uint16_t>(7, (last * l.query_stride + kAttnQueryValues) * 2);
+    if (scratch_base != nullptr) {
+        l.tickets = reinterpret_cast<uint32_t*>(scratch_base);
+        l.records = reinterpret_cast<float*>(scratch_base + kLayerTicketBytes);
+    }
+    return l;
+}
+
+// attention_decode_layer_ms (no reference counterpart; attn_qk_rope_ms, the split path of
+// every row and the combine of decode_step.cpp:1231-1259 in one dispatch): bindings as
+// above, c11 finish mode (1: finished inside the dispatch by the last workgroup of each
+// stream; 0: attention_decode_layer_finish_ms follows); grid (groups, rows) x 256 -
+// `groups` workgroups are launched, the keys of all rows are dealt evenly among them.
+int32_t op_attention_layer_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                              bool validate_only) {
+    Args a(b);
+    a.require(g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1, TT_CMD_INVALID_DISPATCH_EXTENT);
+    LayerArgs l = layer_args(a, static_cast<uint32_t>(std::min<uint64_t>(g.gy, 0xFFFF)),
+                             static_cast<uint32_t>(std::min<uint64_t>(g.gx, 0xFFFF)));
+    l.finish_in_kernel = a.constant(11) != 0 ? 1u : 0u;
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_decode_layer_kernel, dim3(l.groups), dim3(256), kLayerLdsBytes,
+                       stream, l);
+    return TT_OK;
+}
+
+// attention_decode_layer_finish_ms: bindings as above, c11 groups of the dispatch whose
+// records it merges; grid (16, rows) x 64.
+int32_t op_attention_layer_finish_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                                     bool validate_only) {
+    Args a(b);
+    a.require(g.gx == kAttnQueryHeads && g.gz == 1 && g.tx == 64 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    LayerArgs l = layer_args(a, static_cast<uint32_t>(std::min<uint64_t>(g.gy, 0xFFFF)),
+                             a.constant(11));
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_layer_finish_kernel, dim3(kAttnQueryHeads, l.rows), dim3(64), 0,
+                       stream, l);
+    return TT_OK;
+}
+
 // attention_decode_scores_gqa4: b0 q, b1 keys, c2 context, c3 capacity, c4 part,
 // b5 weights[16][nparts][258], c6 nparts; grid (4, nparts) x (256, 4)
 // (decode_step.cpp:309-318).
@@ -1137,7 +1741,10 @@ bool prepare_current_device() {
     // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kWaves * kWaveLdsBytes) != hipSuccess) {
+                            kWaves * kWaveLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLayerLdsBytes) != hipSuccess) {
         (void)hipGetLastError();
         return false;
     }
@@ -1177,6 +1784,8 @@ const KernelDesc kAttentionDecodeKernels[] = {
     {"attention_decode_values_gqa8", op_attention_values},
     {"attention_decode_split_ms", op_attention_split_ms},
     {"attention_decode_combine_ms", op_attention_combine_ms},
+    {"attention_decode_layer_ms", op_attention_layer_ms},
+    {"attention_decode_layer_finish_ms", op_attention_layer_finish_ms},
 };
 const uint32_t kAttentionDecodeKernelCount =
     sizeof(kAttentionDecodeKernels) / sizeof(kAttentionDecodeKernels[0]);
