@@ -145,6 +145,89 @@ def build_workload(B, dev, lib, torch, PART):
     return record, record_split_only, keep
 
 
+def build_period(dev, lib, torch, variant, cus, part=DEFAULT_SPLIT_KEYS):
+    """Recorder of one decode period for the timing variants: `three` = rope, split and
+    combine dispatches; `layer0` / `layer1` = the whole-layer dispatch finished by a second
+    dispatch / inside the first; `gdn_only`, `attn_three`, `attn_layer0`, `attn_layer1` =
+    parts of the period."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x7A7A)
+
+    def rand_bf16(n, sigma=1.0):
+        t = (torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma).to(
+            torch.bfloat16)
+        return dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t)
+
+    def rand_f32(n, sigma):
+        t = torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma
+        return dev.wrap(t.data_ptr(), t.numel() * 4, keepalive=t)
+
+    rows, context = LANES, VISIBLE - 1
+    stripe_elems = 2 * CAPACITY * 256
+    max_splits = (CAPACITY + part - 1) // part
+    kv = [(rand_bf16(rows * stripe_elems), rand_bf16(rows * stripe_elems)) for _ in range(2)]
+    attn_table = np.zeros(64, np.uint32)
+    for r in range(rows):
+        attn_table[r * 4] = r * stripe_elems
+        attn_table[r * 4 + 1] = context
+    b_attn_table = dev.buffer_from(attn_table)
+    attn_proj = rand_bf16(rows * 9216)
+    q_w = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
+    b_q, b_gate, b_att = (dev.create_buffer(rows * 8192) for _ in range(3))
+    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
+    groups = cus
+    b_scratch = dev.create_buffer(256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4)
+    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
+    gdn_layers = []
+    for i in range(3):
+        table = np.zeros(64, np.uint32)
+        for r in range(rows):
+            table[r * 4 + 0] = (2 * r) * conv_elems
+            table[r * 4 + 1] = (2 * r + 1) * conv_elems
+            table[r * 4 + 2] = (2 * r) * rec_elems
+            table[r * 4 + 3] = (2 * r + 1) * rec_elems
+        rng = np.random.default_rng(i + 1)
+        a_log = (rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        dt_bias = (rng.normal(0, 0.3, 32).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        gdn_layers.append(dict(conv=rand_bf16(2 * rows * conv_elems, 0.5),
+                               rec=rand_f32(2 * rows * rec_elems, 0.02), table=dev.buffer_from(table),
+                               proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
+                               a_log=dev.buffer_from(a_log), dt_bias=dev.buffer_from(dt_bias),
+                               norm_w=dev.buffer_from(np.full(128, 0x3F80, np.uint16))))
+    g_out = dev.create_buffer(rows * 8192)
+    P = lib.pipeline
+
+    def record(cb, copy):
+        if not variant.startswith("attn_"):
+            for layer in gdn_layers:
+                cb.encode(P("gdn_decode_fused_ms"),
+                          {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
+                           4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: g_out,
+                           8: layer["table"]}, {9: 12352, 10: 4096}, (32, rows), (512,))
+        if variant == "gdn_only":
+            return
+        keys, values = kv[copy]
+        if variant.endswith("three"):
+            cb.encode(P("attn_qk_rope_ms"),
+                      {0: attn_proj, 1: q_w, 2: q_w, 3: b_q, 4: b_gate, 5: keys, 6: values,
+                       8: b_attn_table}, {7: CAPACITY, 9: 9216, 10: 4096}, (18, rows), (256,))
+            cb.encode(P("attention_decode_split_ms"),
+                      {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
+                      {5: CAPACITY, 6: 4096, 7: part, 8: max_splits, 9: 0}, (max_splits, 2, rows), (256,))
+            cb.encode(P("attention_decode_combine_ms"),
+                      {0: b_part, 1: b_gate, 2: b_attn_table, 3: b_att},
+                      {4: part, 5: max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
+            return
+        mode = 1 if variant.endswith("1") else 0
+        bind = {0: attn_proj, 1: q_w, 2: q_w, 3: keys, 4: values, 5: b_attn_table, 6: b_scratch, 7: b_att}
+        const = {8: CAPACITY, 9: 9216, 10: 4096}
+        cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: mode}, (groups, rows), (256,))
+        if mode == 0:
+            cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: groups}, (16, rows), (64,))
+
+    return record
+
+
 def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
     """Block prefill of `rows` new tokens into an empty cache, one lane, resident
     random inputs: the causal flash attention kernel (rope stage timed beside it) and

@@ -593,6 +593,7 @@ struct LayerArgs {
     const uint32_t* table;        // per row {kv element offset, context, -, -}
     float* records;               // [groups + streams - 1][8][258]
     uint32_t* tickets;            // [streams] arrivals, zero between launches
+    uint16_t* queries;            // [streams][8][256] roped query heads (two-dispatch form)
     uint16_t* out;                // [rows][query_stride]
     uint32_t capacity;
     uint32_t projection_stride;
@@ -602,13 +603,65 @@ struct LayerArgs {
     uint32_t finish_in_kernel;
 };
 
-// Units of stream `stream` (lanes beyond the streams and rows whose context lies outside
-// the cache hold none, so such a row is skipped by every workgroup alike).
-__device__ __forceinline__ uint32_t stream_units(const LayerArgs& a, uint32_t stream) {
-    if (stream >= a.rows * kAttnKvHeads) return 0;
-    const uint32_t context = a.table[(stream >> 1) * 4 + 1];
-    if (context >= a.capacity) return 0;
-    return max(1u, (context + kBlockKeys - 1) / kBlockKeys);
+// How the key streams are dealt to the G workgroups, evaluated by one wave (lane s =
+// stream s) from the contexts in the state table.  A stream holds ceil(context / 32) units
+// (one empty unit for an empty cache; none when the table places the row outside its
+// cache, which every workgroup then skips alike).
+//   * G at least the number of streams that hold units: whole workgroups per stream.
+//     Stream s starts at workgroup b_s = the boundary g U / G nearest to its first unit,
+//     moved where needed so that every such stream keeps at least one workgroup; its
+//     units are split evenly among min(b_{s+1} - b_s, units) workgroups.  One segment per
+//     workgroup - none pays a second prologue at a stream boundary - and the loads differ by
+//     less than one part in the stream's workgroup count.
+//   * fewer workgroups than streams (`flat`): the streams are laid end to end and
+//     workgroup g takes units [g U / G', (g + 1) U / G'), G' = min(G, U), crossing stream
+//     boundaries as they come.
+struct StreamDeal {
+    uint32_t units;        // units of stream `lane`
+    uint32_t inclusive;    // units of streams 0 .. lane
+    uint32_t first_group;  // b_lane (G for lanes past the last stream); unused when flat
+    uint32_t total;        // U
+    bool flat;
+    uint32_t context;      // of the lane's row, as the table holds it
+};
+__device__ __forceinline__ StreamDeal deal_streams(const LayerArgs& a, uint32_t lane) {
+    StreamDeal d;
+    uint32_t units = 0;
+    d.context = 0;
+    if (lane < a.rows * kAttnKvHeads) {
+        d.context = a.table[(lane >> 1) * 4 + 1];
+        if (d.context < a.capacity) units = max(1u, (d.context + kBlockKeys - 1) / kBlockKeys);
+    }
+    uint32_t inclusive = units;
+#pragma unroll
+    for (uint32_t off = 1; off < 64; off <<= 1) {   // lane 32 must see the total as well
+        const uint32_t below = __shfl_up(inclusive, off, 64);
+        if (lane >= off) inclusive += below;
+    }
+    d.units = units;
+    d.inclusive = inclusive;
+    d.total = __shfl(inclusive, kMaxStreams - 1, 64);
+    const uint64_t holding = __builtin_amdgcn_ballot_w64(units != 0);
+    const uint32_t holders = __builtin_popcountll(holding);
+    d.flat = a.groups < holders;
+    const uint32_t before = __builtin_amdgcn_mbcnt_hi(
+        static_cast<uint32_t>(holding >> 32),
+        __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(holding), 0u));
+    d.first_group = 0;
+    if (!d.flat && d.total != 0) {
+        // 32-bit arithmetic: units x workgroups stays below 2^30 (layer_args bounds both)
+        const uint32_t first_unit = inclusive - units;
+        int32_t slack = static_cast<int32_t>((2 * first_unit * a.groups + d.total) / (2 * d.total)) -
+                        static_cast<int32_t>(before);
+#pragma unroll
+        for (uint32_t off = 1; off < 64; off <<= 1) {
+            const int32_t below = __shfl_up(slack, off, 64);
+            if (lane >= off) slack = max(slack, below);
+        }
+        slack = min(slack, static_cast<int32_t>(a.groups - holders));
+        d.first_group = static_cast<uint32_t>(slack) + before;
+    }
+    return d;
 }
 
 // Workgroup that holds unit u when U units are dealt to G workgroups in ranges
@@ -668,6 +721,27 @@ __device__ __forceinline__ void norm_rope_head(const HeadLoads& h, uint32_t posi
     out[0] = round_bf16(rotated);
 }
 
+// The new token's key (normed, rotated; fp32 of the stored bf16) and raw value for dims
+// lane + 64 c, from the projection row; with `append` the wave also writes both rows into
+// the cache at position `context`.
+__device__ __forceinline__ void new_token_rows(const LayerArgs& a, const uint16_t* proj,
+                                               uint32_t kvh, uint32_t context, uint64_t kv_offset,
+                                               bool append, uint32_t lane, float (&kn)[4],
+                                               uint16_t (&vraw)[4]) {
+    const HeadLoads kl = load_head(proj + kAttnQGateRows + kvh * kD, a.k_weight, lane);
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) vraw[c] = proj[kAttnVRowOffset + kvh * kD + lane + 64 * c];
+    norm_rope_head(kl, context, lane, kn);
+    if (append) {
+        const uint64_t at = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            a.keys[at + 64 * c] = f32_to_bf16_bits(kn[c]);
+            a.values[at + 64 * c] = vraw[c];
+        }
+    }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
     v = half_wave_sum(v);
     return v + __shfl_xor(v, 32, 64);
@@ -679,72 +753,83 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // One wave finishes one head of one row: merges the stream's `count` records (slots
-// first_slot ..), folds in the new token, applies the gate and writes the output row;
-// with write_kv it also appends the token's K and V rows.  q: dims lane + 64 c of the
-// roped query head (fp32 of bf16).
+// first_slot ..), folds in the new token, applies the gate and writes the output row.
+// q: dims lane + 64 c of the roped query head (fp32 of bf16).  new_token(kn, vraw) delivers
+// the token's roped key (fp32 of bf16) and raw value row for the same dims; it is called
+// after the records have been requested, so whatever it loads or computes runs while they
+// are under way.
+template <uint32_t kFinishBatch, typename NewToken>   // kFinishBatch: records requested at once
 __device__ __forceinline__ void finish_head(const LayerArgs& a, uint32_t row, uint32_t head,
-                                            uint32_t context, uint64_t kv_offset,
                                             uint32_t first_slot, uint32_t count,
-                                            const float (&q)[4], bool write_kv, uint32_t lane) {
-    const uint32_t kvh = head / kAttnHeadsPerKv;
+                                            const float (&q)[4], NewToken&& new_token,
+                                            uint32_t lane) {
     const uint32_t hl = head % kAttnHeadsPerKv;
     const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
-    const HeadLoads kl = load_head(proj + kAttnQGateRows + kvh * kD, a.k_weight, lane);
-    uint16_t vraw[4], gate[4];
+    uint16_t gate[4];
 #pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        vraw[c] = proj[kAttnVRowOffset + kvh * kD + lane + 64 * c];
-        gate[c] = proj[head * 2 * kD + kD + lane + 64 * c];
+    for (uint32_t c = 0; c < 4; ++c) gate[c] = proj[head * 2 * kD + kD + lane + 64 * c];
+    // The first 64 maxima and sums one per lane, the numerators of the first batch of
+    // records by the lane that owns the dimension: with a batch of 32, one trip to memory
+    // for a stream of up to 32 records.
+    const float* base = a.records + (static_cast<uint64_t>(first_slot) * kAttnHeadsPerKv + hl) *
+                                        kAttnRecordFloats;
+    constexpr uint64_t kSlotFloats = static_cast<uint64_t>(kAttnHeadsPerKv) * kAttnRecordFloats;
+    float first_max = -INFINITY, first_sum = 0.0f;
+    if (lane < count) {
+        first_max = base[lane * kSlotFloats + kD];
+        first_sum = base[lane * kSlotFloats + kD + 1];
+    }
+    float num[kFinishBatch][4];
+#pragma unroll
+    for (uint32_t u = 0; u < kFinishBatch; ++u) {
+        const float* rec = base + min(u, count - 1) * kSlotFloats + lane;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) num[u][c] = rec[64 * c];
     }
     float kn[4];
-    norm_rope_head(kl, context, lane, kn);
-    if (write_kv) {
-        const uint64_t at = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
-#pragma unroll
-        for (uint32_t c = 0; c < 4; ++c) {
-            a.keys[at + 64 * c] = f32_to_bf16_bits(kn[c]);
-            a.values[at + 64 * c] = vraw[c];
-        }
-    }
+    uint16_t vraw[4];
+    new_token(kn, vraw);
     float dot = 0.0f;
 #pragma unroll
     for (uint32_t c = 0; c < 4; ++c) dot = fmaf(q[c], kn[c], dot);
     const float s_new = wave_sum(dot) * kAttnScale;
 
-    const float* base = a.records + (static_cast<uint64_t>(first_slot) * kAttnHeadsPerKv + hl) *
-                                        kAttnRecordFloats;
-    constexpr uint64_t kSlotFloats = static_cast<uint64_t>(kAttnHeadsPerKv) * kAttnRecordFloats;
-    float lmax = -INFINITY;
-    for (uint32_t p = lane; p < count; p += 64) lmax = fmaxf(lmax, base[p * kSlotFloats + kD]);
+    // maxima beyond the first 64 records (only streams spread over more than 64 workgroups)
+    float lmax = first_max;
+    for (uint32_t p = lane + 64; p < count; p += 64) lmax = fmaxf(lmax, base[p * kSlotFloats + kD]);
     const float gmax = fmaxf(wave_max(lmax), s_new);
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     float denom = 0.0f;
-    for (uint32_t p0 = 0; p0 < count; p0 += 64) {
-        float my_w = 0.0f, my_ws = 0.0f;
-        if (p0 + lane < count) {
-            const float* rec = base + (p0 + lane) * kSlotFloats;
-            const float pm = rec[kD];
-            my_w = pm == -INFINITY ? 0.0f : __expf(pm - gmax);
-            my_ws = my_w * rec[kD + 1];
-        }
-        const uint32_t batch = min(64u, count - p0);
-        for (uint32_t j0 = 0; j0 < batch; j0 += 8) {
-            float num[8][4];
+    for (uint32_t p0 = 0; p0 < count; p0 += kFinishBatch) {
+        if (p0 != 0) {
 #pragma unroll
-            for (uint32_t u = 0; u < 8; ++u) {
-                const float* rec = base + (p0 + min(j0 + u, batch - 1)) * kSlotFloats + lane;
+            for (uint32_t u = 0; u < kFinishBatch; ++u) {
+                const float* rec = base + min(p0 + u, count - 1) * kSlotFloats + lane;
 #pragma unroll
                 for (uint32_t c = 0; c < 4; ++c) num[u][c] = rec[64 * c];
             }
+        }
+        // lane j (and the lanes that repeat it) weighs record p0 + j
+        const uint32_t mine = p0 + (lane & (kFinishBatch - 1));
+        float record_max, record_sum;
+        if (p0 < 64) {
+            record_max = __shfl(first_max, mine & 63, 64);
+            record_sum = __shfl(first_sum, mine & 63, 64);
+        } else {
+            const float* rec = base + min(mine, count - 1) * kSlotFloats;
+            record_max = rec[kD];
+            record_sum = rec[kD + 1];
+        }
+        const float my_w =
+            (mine < count && record_max != -INFINITY) ? __expf(record_max - gmax) : 0.0f;
+        const float my_ws = my_w * record_sum;
 #pragma unroll
-            for (uint32_t u = 0; u < 8; ++u) {
-                const bool live = j0 + u < batch;
-                const float w = live ? __shfl(my_w, j0 + u, 64) : 0.0f;
-                const float ws = live ? __shfl(my_ws, j0 + u, 64) : 0.0f;
+        for (uint32_t u = 0; u < kFinishBatch; ++u) {
+            const float w = __shfl(my_w, u, 64);
+            const float ws = __shfl(my_ws, u, 64);
 #pragma unroll
-                for (uint32_t c = 0; c < 4; ++c) acc[c] = fmaf(w, num[u][c], acc[c]);
-                denom += ws;
-            }
+            for (uint32_t c = 0; c < 4; ++c) acc[c] = fmaf(w, num[u][c], acc[c]);
+            denom += ws;
         }
     }
     const float w_new = __expf(s_new - gmax);
@@ -757,6 +842,7 @@ __device__ __forceinline__ void finish_head(const LayerArgs& a, uint32_t row, ui
     }
 }
 
+template <bool kFinishInKernel>
 __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // after the four K stages: the roped query heads of the segment's kv group (bf16),
@@ -765,45 +851,87 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
     uint32_t* s_off = reinterpret_cast<uint32_t*>(lds + kWaves * kWaveLdsBytes +
                                                   kAttnHeadsPerKv * kD * 2);
     uint32_t* s_ticket = s_off + kMaxStreams + 1;
+    uint32_t* s_context = s_ticket + 1;            // per row, as the table holds them
+    uint32_t* s_kv_offset = s_context + kMaxBatchRows;
+    uint32_t* s_group = s_kv_offset + kMaxBatchRows;   // first workgroup per stream, then G
+    uint32_t* s_flat = s_group + kMaxStreams + 1;
+    uint32_t* s_range = s_flat + 1;                    // this workgroup's {first unit, end, stream}
 
-    const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t m = lane & 15;
-    const uint32_t g = lane >> 4;
     const uint32_t group = blockIdx.x;
     const uint32_t streams = a.rows * kAttnKvHeads;
 
-    if (wave == 0) {
-        uint32_t inclusive = stream_units(a, lane);
-#pragma unroll
-        for (uint32_t off = 1; off < kMaxStreams; off <<= 1) {
-            const uint32_t below = __shfl_up(inclusive, off, 64);
-            if (lane >= off) inclusive += below;
+    if (threadIdx.x < 64) {
+        // one read of the state table: the contexts size the streams, and both words of a
+        // row are kept in LDS for the segments (no second trip to memory per segment)
+        const uint32_t lane = threadIdx.x;
+        const StreamDeal deal = deal_streams(a, lane);
+        if (lane < streams && (lane & 1) == 0) {
+            s_context[lane >> 1] = deal.context;
+            s_kv_offset[lane >> 1] = a.table[(lane >> 1) * 4];
         }
-        if (lane < kMaxStreams) s_off[lane + 1] = inclusive;
-        if (lane == 0) s_off[0] = 0;
+        if (lane < kMaxStreams) s_off[lane + 1] = deal.inclusive;
+        if (lane <= kMaxStreams) s_group[lane] = deal.first_group;
+        if (lane == 0) {
+            s_off[0] = 0;
+            *s_flat = deal.flat ? 1u : 0u;
+        }
+        // this workgroup's own units {first, end, stream of the first}: found by the lane of
+        // the stream whose workgroups include it
+        const uint32_t total = deal.total;
+        if (deal.flat) {
+            if (lane == 0) {
+                const uint32_t flat_groups = min(a.groups, total);
+                const bool idle = total == 0 || group >= flat_groups;
+                s_range[0] = idle ? 0u : static_cast<uint32_t>(static_cast<uint64_t>(group) * total / flat_groups);
+                s_range[1] = idle ? 0u : static_cast<uint32_t>((static_cast<uint64_t>(group) + 1) * total / flat_groups);
+                s_range[2] = 0;
+            }
+        } else {
+            const uint32_t next_group = __shfl_down(deal.first_group, 1, 64);
+            if (lane == 0) s_range[0] = s_range[1] = s_range[2] = 0;   // idle unless a stream claims it
+            if (lane < streams && deal.units != 0 && deal.first_group <= group && group < next_group) {
+                const uint32_t sharers = min(next_group - deal.first_group, deal.units);
+                const uint32_t place = group - deal.first_group;
+                const uint32_t first_unit = deal.inclusive - deal.units;
+                if (place < sharers) {                                 // else more workgroups than units
+                    s_range[0] = first_unit + place * deal.units / sharers;
+                    s_range[1] = first_unit + (place + 1) * deal.units / sharers;
+                    s_range[2] = lane;
+                }
+            }
+        }
     }
     __syncthreads();
-    const uint32_t total = s_off[streams];
-    // with fewer units than workgroups the first `total` workgroups take one unit each, so
-    // the workgroups of a stream are always consecutive and none of them is empty
-    const uint32_t groups = min(a.groups, total);
-    if (group >= groups) return;
-    uint32_t unit = static_cast<uint32_t>(static_cast<uint64_t>(group) * total / groups);
-    const uint32_t unit_end =
-        static_cast<uint32_t>((static_cast<uint64_t>(group) + 1) * total / groups);
-    uint8_t* stage = lds + wave * kWaveLdsBytes;
-    uint32_t stream = 0;
+    // values read back from LDS are the same in every lane: moved to scalar registers so
+    // that the segment walk, the key ranges and the row's table entries stay scalar
+    const auto uniform = [](uint32_t v) { return __builtin_amdgcn_readfirstlane(v); };
+    uint32_t unit = uniform(s_range[0]);
+    const uint32_t unit_end = uniform(s_range[1]);
+    if (unit >= unit_end) return;
+    const uint32_t total = uniform(s_off[streams]);
+    const bool flat = uniform(*s_flat) != 0;
+    const uint32_t flat_groups = min(a.groups, total);
+    uint32_t stream = uniform(s_range[2]);
 
     while (unit < unit_end) {
-        while (s_off[stream + 1] <= unit) ++stream;
-        const uint32_t stream_first = s_off[stream];
-        const uint32_t stream_last = s_off[stream + 1];
+        // Everything derived from the thread index is derived inside the segment, from an
+        // opaque copy: hoisted out of this loop it would be carried in registers across
+        // the key walk (which has none to spare) and spilled.
+        uint32_t thread_early = threadIdx.x;
+        asm volatile("" : "+v"(thread_early));
+        const uint32_t wave = thread_early >> 6;
+        const uint32_t lane = thread_early & 63;
+        const uint32_t m = lane & 15;
+        const uint32_t g = lane >> 4;
+        uint8_t* stage = lds + wave * kWaveLdsBytes;
+        while (uniform(s_off[stream + 1]) <= unit) ++stream;
+        const uint32_t stream_first = uniform(s_off[stream]);
+        const uint32_t stream_last = uniform(s_off[stream + 1]);
         const uint32_t segment_end = min(unit_end, stream_last);
         const uint32_t row = stream >> 1;
         const uint32_t kvh = stream & 1;
-        const uint64_t kv_offset = a.table[row * 4];
-        const uint32_t context = a.table[row * 4 + 1];
+        const uint64_t kv_offset = uniform(s_kv_offset[row]);
+        const uint32_t context = uniform(s_context[row]);
         const uint32_t k0 = (unit - stream_first) * kBlockKeys;
         const uint32_t k1 = min(context, (segment_end - stream_first) * kBlockKeys);
         const uint32_t nblocks = k1 > k0 ? (k1 - k0 + kBlockKeys - 1) / kBlockKeys : 0u;
@@ -849,14 +977,28 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
             load_values(vreg[0], wave, 0);
             load_values(vreg[1], wave, 1);
         }
+        // two-dispatch form: the workgroup that holds a stream's first unit leaves the roped
+        // query heads in the scratch and appends the token's key and value rows (no key walk
+        // reads position `context`), so the finishing dispatch only loads them
+        const bool publishes = !kFinishInKernel && unit == stream_first;
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             float n[4];
             norm_rope_head(ql[i], context, lane, n);
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
-                qs[(wave * 2 + i) * kD + lane + 64 * c] = f32_to_bf16_bits(n[c]);
+                const uint16_t bits = f32_to_bf16_bits(n[c]);
+                qs[(wave * 2 + i) * kD + lane + 64 * c] = bits;
+                if (publishes) {
+                    a.queries[(static_cast<uint64_t>(stream) * kAttnHeadsPerKv + wave * 2 + i) * kD +
+                              lane + 64 * c] = bits;
+                }
             }
+        }
+        if (publishes && wave == 0) {
+            float kn[4];
+            uint16_t vraw[4];
+            new_token_rows(a, proj, kvh, context, kv_offset, true, lane, kn, vraw);
         }
         __syncthreads();
         // B operand of S^T: Q^T, column m holds head (m & 7)
@@ -956,22 +1098,30 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);
 
+        // the same for the addresses of the merge below
+        uint32_t thread_late = threadIdx.x;
+        asm volatile("" : "+v"(thread_late));
+        const uint32_t wave_l = thread_late >> 6;
+        const uint32_t lane_l = thread_late & 63;
+        const uint32_t m_l = lane_l & 15;
+        const uint32_t g_l = lane_l >> 4;
+
         // the wave's {O[8][256], max, sum} into its own stage (layout as in flash_decode_kernel)
-        float* merge = reinterpret_cast<float*>(stage);
+        float* merge = reinterpret_cast<float*>(lds + wave_l * kWaveLdsBytes);
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             f32x4 sum4;
 #pragma unroll
             for (uint32_t i = 0; i < 4; ++i) sum4[i] = o[j][i] + dpp_row_ror8(o[j][i]);
-            if (m < 8) {
-                *reinterpret_cast<f32x4*>(merge + m * kMergeHeadFloats + j * kMergeTileFloats +
-                                          g * 4) = sum4;
+            if (m_l < 8) {
+                *reinterpret_cast<f32x4*>(merge + m_l * kMergeHeadFloats + j * kMergeTileFloats +
+                                          g_l * 4) = sum4;
             }
         }
-        if (lane < 8) {
-            merge[8 * kMergeHeadFloats + lane * 2] = m_run;
-            merge[8 * kMergeHeadFloats + lane * 2 + 1] = l_run;
+        if (lane_l < 8) {
+            merge[8 * kMergeHeadFloats + lane_l * 2] = m_run;
+            merge[8 * kMergeHeadFloats + lane_l * 2 + 1] = l_run;
         }
         __syncthreads();
 
@@ -979,7 +1129,7 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
         const uint32_t slot = group + stream;
 #pragma unroll
         for (uint32_t hl = 0; hl < 2; ++hl) {
-            const uint32_t h = wave * 2 + hl;
+            const uint32_t h = wave_l * 2 + hl;
             float scale[kWaves];
             float gmax = -INFINITY;
             float lsum[kWaves];
@@ -1000,7 +1150,7 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
                                             kAttnRecordFloats;
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
-                const uint32_t d = lane + 64 * c;
+                const uint32_t d = lane_l + 64 * c;
                 const uint32_t at = ((d >> 7) * 8 + (d & 7)) * kMergeTileFloats + ((d & 127) >> 3);
                 float acc = 0.0f;
 #pragma unroll
@@ -1010,25 +1160,31 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
                 }
                 __hip_atomic_store(record + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            if (lane == 0) {
+            if (lane_l == 0) {
                 __hip_atomic_store(record + kD, gmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(record + kD + 1, denom, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
             }
         }
 
-        if (a.finish_in_kernel) {
+        if constexpr (kFinishInKernel) {
             // the record stores have been acknowledged before the ticket is taken
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            const uint32_t first_group = group_of_unit(stream_first, total, groups);
-            const uint32_t count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
+            uint32_t first_group, count;
+            if (flat) {
+                first_group = group_of_unit(stream_first, total, flat_groups);
+                count = group_of_unit(stream_last - 1, total, flat_groups) - first_group + 1;
+            } else {
+                first_group = uniform(s_group[stream]);
+                count = min(uniform(s_group[stream + 1]) - first_group, stream_last - stream_first);
+            }
             if (threadIdx.x == 0) {
                 *s_ticket = __hip_atomic_fetch_add(a.tickets + stream, 1u, __ATOMIC_RELAXED,
                                                    __HIP_MEMORY_SCOPE_AGENT);
             }
             __syncthreads();
-            if (*s_ticket == count - 1) {
+            if (uniform(*s_ticket) == count - 1) {
                 // last to arrive: every record of the stream is in memory; drop what this
                 // compute unit's caches may hold of that memory, then finish two heads a wave
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -1038,8 +1194,13 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
                     float q[4];
 #pragma unroll
                     for (uint32_t c = 0; c < 4; ++c) q[c] = bf16_bits_to_f32(qs[h * kD + lane + 64 * c]);
-                    finish_head(a, row, kvh * kAttnHeadsPerKv + h, context, kv_offset,
-                                first_group + stream, count, q, h == 0, lane);
+                    // eight records at a time: the key walk above leaves no registers for more
+                    finish_head<8>(a, row, kvh * kAttnHeadsPerKv + h, first_group + stream, count, q,
+                                   [&](float (&kn)[4], uint16_t (&vraw)[4]) {
+                                       new_token_rows(a, proj, kvh, context, kv_offset, h == 0,
+                                                      lane, kn, vraw);
+                                   },
+                                   lane);
                 }
                 if (threadIdx.x == 0) {
                     __hip_atomic_store(a.tickets + stream, 0u, __ATOMIC_RELAXED,
@@ -1058,28 +1219,45 @@ __global__ __launch_bounds__(64) void attention_layer_finish_kernel(LayerArgs a)
     const uint32_t row = blockIdx.y;
     const uint32_t lane = threadIdx.x;
     const uint32_t stream = row * kAttnKvHeads + head / kAttnHeadsPerKv;
-    uint32_t inclusive = stream_units(a, lane);
-#pragma unroll
-    for (uint32_t off = 1; off < kMaxStreams; off <<= 1) {
-        const uint32_t below = __shfl_up(inclusive, off, 64);
-        if (lane >= off) inclusive += below;
-    }
-    const uint32_t total = __shfl(inclusive, a.rows * kAttnKvHeads - 1, 64);
-    const uint32_t stream_last = __shfl(inclusive, stream, 64);
-    const uint32_t below = __shfl(inclusive, stream == 0 ? 0 : stream - 1, 64);
+    const StreamDeal deal = deal_streams(a, lane);
+    const uint32_t total = deal.total;
+    const uint32_t stream_last = __shfl(deal.inclusive, stream, 64);
+    const uint32_t below = __shfl(deal.inclusive, stream == 0 ? 0 : stream - 1, 64);
     const uint32_t stream_first = stream == 0 ? 0u : below;
     if (stream_last == stream_first) return;   // a row the table places outside its cache
-    const uint32_t groups = min(a.groups, total);
-    const uint32_t first_group = group_of_unit(stream_first, total, groups);
-    const uint32_t count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
+    uint32_t first_group, count;
+    if (deal.flat) {
+        const uint32_t groups = min(a.groups, total);
+        first_group = group_of_unit(stream_first, total, groups);
+        count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
+    } else {
+        first_group = __shfl(deal.first_group, stream, 64);
+        count = min(__shfl(deal.first_group, stream + 1, 64) - first_group,
+                    stream_last - stream_first);
+    }
+    // The first dispatch left the roped query heads in the scratch and the token's key and
+    // value rows in the cache: nothing is normed or rotated again here.
     const uint64_t kv_offset = a.table[row * 4];
     const uint32_t context = a.table[row * 4 + 1];
-    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
-    const HeadLoads ql = load_head(proj + head * 2 * kD, a.q_weight, lane);
+    const uint32_t kvh = head / kAttnHeadsPerKv;
     float q[4];
-    norm_rope_head(ql, context, lane, q);
-    finish_head(a, row, head, context, kv_offset, first_group + stream, count, q,
-                head % kAttnHeadsPerKv == 0, lane);
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        q[c] = bf16_bits_to_f32(
+            a.queries[(static_cast<uint64_t>(stream) * kAttnHeadsPerKv + head % kAttnHeadsPerKv) * kD +
+                      lane + 64 * c]);
+    }
+    finish_head<32>(a, row, head, first_group + stream, count, q,
+                    [&](float (&kn)[4], uint16_t (&vraw)[4]) {
+                        const uint64_t at =
+                            kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
+#pragma unroll
+                        for (uint32_t c = 0; c < 4; ++c) {
+                            kn[c] = bf16_bits_to_f32(a.keys[at + 64 * c]);
+                            vraw[c] = a.values[at + 64 * c];
+                        }
+                    },
+                    lane);
 }
 
 // ----------------------------------------------------------------- combine ---
@@ -1591,20 +1769,22 @@ int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t st
     return TT_OK;
 }
 
-constexpr uint32_t kLayerLdsBytes =
-    kWaves * kWaveLdsBytes + kAttnHeadsPerKv * kD * 2 + (kMaxStreams + 2) * 4;
-constexpr uint32_t kLayerTicketBytes = 256;   // tickets lead the scratch, records follow
-constexpr uint32_t kMaxLayerGroups = 4096;
+constexpr uint32_t kLayerLdsBytes = kWaves * kWaveLdsBytes + kAttnHeadsPerKv * kD * 2 +
+                                    (2 * kMaxStreams + 8 + 2 * kMaxBatchRows) * 4;
+constexpr uint32_t kLayerTicketBytes = 256;   // tickets lead the scratch
+constexpr uint32_t kLayerQueryBytes = kMaxStreams * kAttnHeadsPerKv * kD * 2;  // then the queries
+constexpr uint32_t kMaxLayerGroups = 2048;   // keeps units x workgroups in 32 bits
 
 uint64_t layer_scratch_bytes(uint32_t groups, uint32_t rows) {
-    return kLayerTicketBytes + static_cast<uint64_t>(groups + rows * kAttnKvHeads - 1) *
-                                   kAttnHeadsPerKv * kAttnRecordFloats * 4;
+    return kLayerTicketBytes + kLayerQueryBytes +
+           static_cast<uint64_t>(groups + rows * kAttnKvHeads - 1) * kAttnHeadsPerKv *
+               kAttnRecordFloats * 4;
 }
 
 // Bindings shared by the two dispatches of the whole-layer decode: b0 projection slab
 // [rows][projection stride], b1 q_w, b2 k_w, b3 keys_pool, b4 values_pool, b5 state_table,
-// b6 scratch (256 B of tickets, then (groups + 2 rows - 1) x 8 records of 258 floats; zero
-// before the first use, left zeroed by every launch), b7 out slab [rows][query stride],
+// b6 scratch (256 B of tickets, 128 KiB of query heads, then (groups + 2 rows - 1) x 8
+// records of 258 floats; zero before the first use, tickets left zeroed by every launch), b7 out slab [rows][query stride],
 // c8 capacity, c9 projection stride, c10 query stride.
 LayerArgs layer_args(Args& a, uint32_t rows, uint32_t groups) {
     LayerArgs l{};
@@ -1631,7 +1811,8 @@ LayerArgs layer_args(Args& a, uint32_t rows, uint32_t groups) {
     l.out = a.buffer<uint16_t>(7, (last * l.query_stride + kAttnQueryValues) * 2);
     if (scratch_base != nullptr) {
         l.tickets = reinterpret_cast<uint32_t*>(scratch_base);
-        l.records = reinterpret_cast<float*>(scratch_base + kLayerTicketBytes);
+        l.queries = reinterpret_cast<uint16_t*>(scratch_base + kLayerTicketBytes);
+        l.records = reinterpret_cast<float*>(scratch_base + kLayerTicketBytes + kLayerQueryBytes);
     }
     return l;
 }
@@ -1649,8 +1830,13 @@ int32_t op_attention_layer_ms(const Bindings& b, const Grid& g, hipStream_t stre
                              static_cast<uint32_t>(std::min<uint64_t>(g.gx, 0xFFFF)));
     l.finish_in_kernel = a.constant(11) != 0 ? 1u : 0u;
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(attention_decode_layer_kernel, dim3(l.groups), dim3(256), kLayerLdsBytes,
-                       stream, l);
+    if (l.finish_in_kernel) {
+        hipLaunchKernelGGL(attention_decode_layer_kernel<true>, dim3(l.groups), dim3(256),
+                           kLayerLdsBytes, stream, l);
+    } else {
+        hipLaunchKernelGGL(attention_decode_layer_kernel<false>, dim3(l.groups), dim3(256),
+                           kLayerLdsBytes, stream, l);
+    }
     return TT_OK;
 }
 
@@ -1742,7 +1928,10 @@ bool prepare_current_device() {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWaves * kWaveLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel<true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLayerLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel<false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLayerLdsBytes) != hipSuccess) {
         (void)hipGetLastError();

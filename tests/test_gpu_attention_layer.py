@@ -60,7 +60,7 @@ def _layer_batch(contexts, cap, groups_list, seed, replays=0, projection_stride=
     b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
     outs = {}
     for groups in groups_list:
-        b_scratch = dev.create_buffer(256 + (groups + 2 * rows - 1) * 8 * 258 * 4)
+        b_scratch = dev.create_buffer(256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4)
         for mode in (0, 1):
             for r, (k, v, _, _) in enumerate(caches):   # caches back to their state before the token
                 k_pool.write(k, stripes[r] * stride)
@@ -124,6 +124,15 @@ def test_layer_single_lane_context_edges(ctx):
     _layer_batch([ctx], 1100, [3, 32], 0x2B00 + ctx)
 
 
+@pytest.mark.parametrize("groups", [10, 11, 40, 300])
+def test_layer_tiny_streams_between_deep_ones(groups):
+    """Lanes of 3, 0 and 40 cached keys beside lanes of thousands: every stream that holds
+    keys keeps a workgroup of its own however small its share (10 workgroups for 10
+    streams), and more workgroups than a short stream has 32-key units leave some idle."""
+    print(f"[case] decode layer, tiny streams between deep ones, {groups} workgroups", flush=True)
+    _layer_batch([5000, 3, 0, 4000, 40], 5120, [groups], 0x5E03, replays=1)
+
+
 def test_layer_wide_strides():
     print("[case] decode layer, slab strides wider than the rows", flush=True)
     _layer_batch([500, 37], 512, [16], 0x3C01, projection_stride=9216 + 64, query_stride=4096 + 256)
@@ -159,7 +168,7 @@ def test_layer_validation():
     pool = dev.create_buffer(2 * cap * 512 * rows)
     tab = dev.create_buffer(256)
     out = dev.create_buffer(rows * 8192)
-    need = 256 + (groups + 2 * rows - 1) * 8 * 258 * 4
+    need = 256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4
     cb = queue.create_command_buffer()
     cb.begin_compute_pass()
     bind = {0: ok, 1: w, 2: w, 3: pool, 4: pool, 5: tab, 7: out}
