@@ -1,28 +1,37 @@
 #!/usr/bin/env python3
 """Benchmark of the attention-family hot path on one MI355X.
 
-A step is one decode token wave of 4 lanes at 32768 visible keys through one
-hybrid period of the layer stack, G,G,G,A (three Gated DeltaNet layers, one
-full-attention layer), with the lane-batched operators:
+A step is one decode token wave of 4 lanes at 32768 visible keys through the attention
+family of the whole 40-layer hybrid stack, G,G,G,A x 10 (30 Gated DeltaNet layers, 10
+full-attention layers), with the lane-batched operators:
     GDN:       gdn_decode_fused_ms (prepare + recurrence + gate-norm in one dispatch)
-    attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms
-Projections (the reference's Q4 GEMVs) are not on the path: their outputs are
-resident random bf16 slabs.  KV caches, GDN state and all scratch are in HBM
-before the timed region; two copies of the attention layer's KV pools (537 MB in
-total) alternate from step to step so the 256 MB last-level cache cannot serve
-the stream.  The step is compiled into a HIP graph and replayed.
+    attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms, or
+               with --attention layer attention_decode_layer_ms +
+               attention_decode_layer_finish_ms (qk-norm, rotation, K / V append, split-K
+               attention over keys dealt evenly to the workgroups and the gated combine in
+               two dispatches; same layer time, slower key walk)
+Projections (the reference's Q4 GEMVs) are not on the path: their outputs are resident
+random bf16 slabs.  Every layer has its own KV pools, recurrent state and inputs, all in
+HBM before the timed region (2.7 GB of keys and values: the 256 MB last-level cache cannot
+serve the stream).  The wave is compiled into one HIP graph and replayed, one launch per
+token as a serving loop would issue it.  `value` = microseconds per layer = step / 40.
 
-`detail.prefill_16k` adds the block-prefill side of the metric: 16384 new tokens of
-one lane through a full-attention layer (causal flash attention on MFMA) and a
-Gated DeltaNet layer (chunk-64 recurrence on MFMA), tok/s and fraction of MFMA peak.
+`roofline` is for the dominant kernel, the key walk of the attention layer
+(flash_decode_kernel): algorithmic bytes (2048 B per visible key and lane) over its
+launch duration, measured with HIP events on the queue's stream around a graph that holds
+that kernel once per attention layer (10 launches on 10 different KV sets per replay; median
+and p10 / p90 over the replays).  `detail.config3` repeats the figure for the ragged lanes and
+the single deep lane, next to the duration of all dispatches of the layer.
 
-`detail.q4_projections` adds the affine 4-bit projections either side of the family
-(attention / GDN in-projection, output projection) for the same 4-lane wave and the same
-16384-row block, device microseconds per dispatch (tatara_amd.q4_sweep).
+`detail.prefill_16k` adds the block-prefill side of the metric: 16384 new tokens of one lane
+through a full-attention layer (causal flash attention on MFMA) and a Gated DeltaNet layer
+(chunk-64 recurrence on MFMA), tok/s and fraction of MFMA peak, with the CPU checker timed on
+a strided subset of the rows beside it.
 
-Prints ONE JSON line: `value` = microseconds per layer over the period,
-`roofline` for the dominant kernel (the split-K flash-decode), `cpu_baseline` =
-the CPU checker timed on this box's host cores on the same period."""
+`cpu_baseline` = the CPU checker (the reference's scalar arithmetic restated) timed on this
+box's host cores on one G,G,G,A period of the same wave, one thread and all threads.
+
+Prints ONE JSON line."""
 import argparse
 import ctypes as C
 import json
@@ -39,193 +48,183 @@ sys.path.insert(0, ROOT)
 LANES = 4
 VISIBLE = 32768
 CAPACITY = 32768
-DEFAULT_SPLIT_KEYS = 1024       # keys per split-K workgroup
+LAYERS = 40
+PERIOD = 4                      # G,G,G,A
+DEFAULT_SPLIT_KEYS = 1024       # keys per split-K workgroup of the three-dispatch form
 HBM_PEAK_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
-# HBM traffic of one launch of the split-K kernel at this workload, from two
-# rocprofv3 counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
-# scaled by what the same counter read for a plain 256 MiB copy of known size.
-FLASH_FETCH_KIB, FETCH_SCALE = 131297.0, 262144.0 / 131083.3
-FLASH_WRITE_KIB, WRITE_SCALE = 2112.0, 262144.0 / 262144.0
+# HBM traffic of one launch of the key-walk kernel at 4 lanes x 32768 keys, from two rocprofv3
+# counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
+# counter read for a plain 256 MiB copy of known size; see the file named here.
+TRAFFIC_SOURCE = "profiles/decode_layer_4x32768_hbm_counters.md"
+TRAFFIC_BYTES = None            # filled from the counter runs; None until they exist
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
+CONFIG3 = {
+    "uniform": ([VISIBLE - 1] * 4, CAPACITY),
+    "ragged": ([32767, 29999, 24575, 8191], CAPACITY),
+    "lane100k": ([99999], 100096),
+}
 
 
-def build_workload(B, dev, lib, torch, PART):
-    """Allocates and fills every buffer of the period; returns the two step
-    recorders (even/odd KV copy) and bookkeeping."""
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x7A7A)
-    keep = []
+def layer_scratch_bytes(groups, rows):
+    return 256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4
 
-    def rand_bf16(n, sigma=1.0):
-        t = (torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma).to(
-            torch.bfloat16)
-        keep.append(t)
-        return dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t)
 
-    def rand_f32(n, sigma):
-        t = torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma
-        keep.append(t)
-        return dev.wrap(t.data_ptr(), t.numel() * 4, keepalive=t)
+class Wave:
+    """Buffers and recorders of the attention family of one token wave."""
 
-    def from_np(a):
-        return dev.buffer_from(a)
+    def __init__(self, dev, lib, torch, attention, split_keys, attention_layers, gdn_layers,
+                 contexts, capacity, seed=0x7A7A):
+        self.dev, self.lib, self.attention, self.part = dev, lib, attention, split_keys
+        self.contexts, self.capacity = list(contexts), capacity
+        self.rows = len(contexts)
+        self.groups = dev.compute_units
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
 
-    rows = LANES
-    context = VISIBLE - 1
-    stripe_elems = 2 * CAPACITY * 256
-    max_splits = (CAPACITY + PART - 1) // PART
-    # attention layer: two alternating KV copies, 4 stripes each
-    kv = [(rand_bf16(rows * stripe_elems), rand_bf16(rows * stripe_elems)) for _ in range(2)]
-    attn_table = np.zeros(64, np.uint32)
-    for r in range(rows):
-        attn_table[r * 4] = r * stripe_elems
-        attn_table[r * 4 + 1] = context
-    b_attn_table = from_np(attn_table)
-    attn_proj = rand_bf16(rows * 9216)
-    q_w = from_np(np.full(256, 0x3F80, np.uint16))
-    k_w = from_np(np.full(256, 0x3F80, np.uint16))
-    b_q, b_gate, b_att = (dev.create_buffer(rows * 8192) for _ in range(3))
-    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
+        def rand_bf16(n, sigma=1.0):
+            t = (torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma).to(
+                torch.bfloat16)
+            return dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t)
 
-    # three GDN layers, each with its own pooled state and weights
-    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
-    gdn_layers = []
-    for _ in range(3):
-        conv_pool = rand_bf16(2 * rows * conv_elems, 0.5)
-        rec_pool = rand_f32(2 * rows * rec_elems, 0.02)
+        def rand_f32(n, sigma):
+            t = torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma
+            return dev.wrap(t.data_ptr(), t.numel() * 4, keepalive=t)
+
+        rows = self.rows
+        stripe = 2 * capacity * 256
+        self.max_splits = (capacity + split_keys - 1) // split_keys
+        ones = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
+        self.set_contexts(contexts)
+        self.attn = []
+        for _ in range(attention_layers):
+            self.attn.append(dict(keys=rand_bf16(rows * stripe), values=rand_bf16(rows * stripe),
+                                  proj=rand_bf16(rows * 9216), q_w=ones, k_w=ones))
+        self.b_q, self.b_gate, self.b_out = (dev.create_buffer(rows * 8192) for _ in range(3))
+        self.b_part = dev.create_buffer(rows * 16 * self.max_splits * 258 * 4)
+        self.b_scratch = dev.create_buffer(layer_scratch_bytes(self.groups, rows))
+        conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
         table = np.zeros(64, np.uint32)
         for r in range(rows):
             table[r * 4 + 0] = (2 * r) * conv_elems
             table[r * 4 + 1] = (2 * r + 1) * conv_elems
             table[r * 4 + 2] = (2 * r) * rec_elems
             table[r * 4 + 3] = (2 * r + 1) * rec_elems
-        rng = np.random.default_rng(len(gdn_layers) + 1)
-        a_log = (rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16).astype(
-            np.uint16)
-        dt_bias = (rng.normal(0, 0.3, 32).astype(np.float32).view(np.uint32) >> 16).astype(
-            np.uint16)
-        gdn_layers.append(dict(conv=conv_pool, rec=rec_pool, table=from_np(table),
-                               proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
-                               a_log=from_np(a_log), dt_bias=from_np(dt_bias),
-                               norm_w=from_np(np.full(128, 0x3F80, np.uint16))))
-    g_out = dev.create_buffer(rows * 8192)
+        gdn_table = dev.buffer_from(table)
+        self.gdn = []
+        for i in range(gdn_layers):
+            rng = np.random.default_rng(i + 1)
+            a_log = (rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16).astype(
+                np.uint16)
+            dt_bias = (rng.normal(0, 0.3, 32).astype(np.float32).view(np.uint32) >> 16).astype(
+                np.uint16)
+            self.gdn.append(dict(conv=rand_bf16(2 * rows * conv_elems, 0.5),
+                                 rec=rand_f32(2 * rows * rec_elems, 0.02), table=gdn_table,
+                                 proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
+                                 a_log=dev.buffer_from(a_log), dt_bias=dev.buffer_from(dt_bias),
+                                 norm_w=dev.buffer_from(np.full(128, 0x3F80, np.uint16))))
+        self.g_out = dev.create_buffer(rows * 8192)
 
-    P = lib.pipeline
-
-    def record(cb, copy):
-        for layer in gdn_layers:
-            cb.encode(P("gdn_decode_fused_ms"),
-                      {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
-                       4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: g_out,
-                       8: layer["table"]}, {9: 12352, 10: 4096}, (32, rows), (512,))
-            cb.barrier()
-        keys, values = kv[copy]
-        cb.encode(P("attn_qk_rope_ms"),
-                  {0: attn_proj, 1: q_w, 2: k_w, 3: b_q, 4: b_gate, 5: keys, 6: values,
-                   8: b_attn_table}, {7: CAPACITY, 9: 9216, 10: 4096}, (18, rows), (256,))
-        cb.barrier()
-        cb.encode(P("attention_decode_split_ms"),
-                  {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
-                  {5: CAPACITY, 6: 4096, 7: PART, 8: max_splits, 9: 0}, (max_splits, 2, rows),
-                  (256,))
-        cb.barrier()
-        cb.encode(P("attention_decode_combine_ms"),
-                  {0: b_part, 1: b_gate, 2: b_attn_table, 3: b_att},
-                  {4: PART, 5: max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
-
-    def record_split_only(cb, copy):
-        keys, values = kv[copy]
-        cb.encode(P("attention_decode_split_ms"),
-                  {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
-                  {5: CAPACITY, 6: 4096, 7: PART, 8: max_splits, 9: 0}, (max_splits, 2, rows),
-                  (256,))
-
-    return record, record_split_only, keep
-
-
-def build_period(dev, lib, torch, variant, cus, part=DEFAULT_SPLIT_KEYS):
-    """Recorder of one decode period for the timing variants: `three` = rope, split and
-    combine dispatches; `layer0` / `layer1` = the whole-layer dispatch finished by a second
-    dispatch / inside the first; `gdn_only`, `attn_three`, `attn_layer0`, `attn_layer1` =
-    parts of the period."""
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x7A7A)
-
-    def rand_bf16(n, sigma=1.0):
-        t = (torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma).to(
-            torch.bfloat16)
-        return dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t)
-
-    def rand_f32(n, sigma):
-        t = torch.randn(n, generator=gen, device="cuda", dtype=torch.float32) * sigma
-        return dev.wrap(t.data_ptr(), t.numel() * 4, keepalive=t)
-
-    rows, context = LANES, VISIBLE - 1
-    stripe_elems = 2 * CAPACITY * 256
-    max_splits = (CAPACITY + part - 1) // part
-    kv = [(rand_bf16(rows * stripe_elems), rand_bf16(rows * stripe_elems)) for _ in range(2)]
-    attn_table = np.zeros(64, np.uint32)
-    for r in range(rows):
-        attn_table[r * 4] = r * stripe_elems
-        attn_table[r * 4 + 1] = context
-    b_attn_table = dev.buffer_from(attn_table)
-    attn_proj = rand_bf16(rows * 9216)
-    q_w = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
-    b_q, b_gate, b_att = (dev.create_buffer(rows * 8192) for _ in range(3))
-    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
-    groups = cus
-    b_scratch = dev.create_buffer(256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4)
-    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
-    gdn_layers = []
-    for i in range(3):
+    def set_contexts(self, contexts):
+        """A new state table (same pools): other lane depths over the same caches."""
+        assert len(contexts) == self.rows and max(contexts) < self.capacity
+        stripe = 2 * self.capacity * 256
         table = np.zeros(64, np.uint32)
-        for r in range(rows):
-            table[r * 4 + 0] = (2 * r) * conv_elems
-            table[r * 4 + 1] = (2 * r + 1) * conv_elems
-            table[r * 4 + 2] = (2 * r) * rec_elems
-            table[r * 4 + 3] = (2 * r + 1) * rec_elems
-        rng = np.random.default_rng(i + 1)
-        a_log = (rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-        dt_bias = (rng.normal(0, 0.3, 32).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-        gdn_layers.append(dict(conv=rand_bf16(2 * rows * conv_elems, 0.5),
-                               rec=rand_f32(2 * rows * rec_elems, 0.02), table=dev.buffer_from(table),
-                               proj=rand_bf16(rows * 12352, 0.5), conv_w=rand_bf16(4 * 8192, 0.5),
-                               a_log=dev.buffer_from(a_log), dt_bias=dev.buffer_from(dt_bias),
-                               norm_w=dev.buffer_from(np.full(128, 0x3F80, np.uint16))))
-    g_out = dev.create_buffer(rows * 8192)
-    P = lib.pipeline
+        for r, context in enumerate(contexts):
+            table[r * 4] = r * stripe
+            table[r * 4 + 1] = context
+        self.contexts = list(contexts)
+        self.attn_table = self.dev.buffer_from(table)
 
-    def record(cb, copy):
-        if not variant.startswith("attn_"):
-            for layer in gdn_layers:
-                cb.encode(P("gdn_decode_fused_ms"),
-                          {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
-                           4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: g_out,
-                           8: layer["table"]}, {9: 12352, 10: 4096}, (32, rows), (512,))
-        if variant == "gdn_only":
+    def visible_keys(self):
+        return sum(c + 1 for c in self.contexts)
+
+    def record_gdn(self, cb, index):
+        layer = self.gdn[index]
+        cb.encode(self.lib.pipeline("gdn_decode_fused_ms"),
+                  {0: layer["proj"], 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
+                   4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: self.g_out,
+                   8: layer["table"]}, {9: 12352, 10: 4096}, (32, self.rows), (512,))
+
+    def record_attention(self, cb, index, walk_only=False):
+        """All dispatches of one attention layer; walk_only: the key-walk kernel alone."""
+        layer, rows, cap, P = self.attn[index], self.rows, self.capacity, self.lib.pipeline
+        if self.attention == "layer":
+            bind = {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: layer["keys"],
+                    4: layer["values"], 5: self.attn_table, 6: self.b_scratch, 7: self.b_out}
+            const = {8: cap, 9: 9216, 10: 4096}
+            cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: 0}, (self.groups, rows),
+                      (256,))
+            if not walk_only:
+                cb.barrier()
+                cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: self.groups},
+                          (16, rows), (64,))
             return
-        keys, values = kv[copy]
-        if variant.endswith("three"):
+        if not walk_only:
             cb.encode(P("attn_qk_rope_ms"),
-                      {0: attn_proj, 1: q_w, 2: q_w, 3: b_q, 4: b_gate, 5: keys, 6: values,
-                       8: b_attn_table}, {7: CAPACITY, 9: 9216, 10: 4096}, (18, rows), (256,))
-            cb.encode(P("attention_decode_split_ms"),
-                      {0: b_q, 1: keys, 2: values, 3: b_attn_table, 4: b_part},
-                      {5: CAPACITY, 6: 4096, 7: part, 8: max_splits, 9: 0}, (max_splits, 2, rows), (256,))
+                      {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: self.b_q,
+                       4: self.b_gate, 5: layer["keys"], 6: layer["values"], 8: self.attn_table},
+                      {7: cap, 9: 9216, 10: 4096}, (18, rows), (256,))
+            cb.barrier()
+        cb.encode(P("attention_decode_split_ms"),
+                  {0: self.b_q, 1: layer["keys"], 2: layer["values"], 3: self.attn_table,
+                   4: self.b_part}, {5: cap, 6: 4096, 7: self.part, 8: self.max_splits, 9: 0},
+                  (self.max_splits, 2, rows), (256,))
+        if not walk_only:
+            cb.barrier()
             cb.encode(P("attention_decode_combine_ms"),
-                      {0: b_part, 1: b_gate, 2: b_attn_table, 3: b_att},
-                      {4: part, 5: max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
-            return
-        mode = 1 if variant.endswith("1") else 0
-        bind = {0: attn_proj, 1: q_w, 2: q_w, 3: keys, 4: values, 5: b_attn_table, 6: b_scratch, 7: b_att}
-        const = {8: CAPACITY, 9: 9216, 10: 4096}
-        cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: mode}, (groups, rows), (256,))
-        if mode == 0:
-            cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: groups}, (16, rows), (64,))
+                      {0: self.b_part, 1: self.b_gate, 2: self.attn_table, 3: self.b_out},
+                      {4: self.part, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
 
-    return record
+    def record_wave(self, cb):
+        gdn = attn = 0
+        for layer in range(len(self.gdn) + len(self.attn)):
+            if layer % PERIOD == PERIOD - 1:
+                self.record_attention(cb, attn)
+                attn += 1
+            else:
+                self.record_gdn(cb, gdn)
+                gdn += 1
+            cb.barrier()
+
+
+def percentiles(samples_us):
+    s = sorted(samples_us)
+    pick = lambda f: s[min(len(s) - 1, int(round(f * (len(s) - 1))))]
+    return {"median_us": round(statistics.median(s), 2), "p10_us": round(pick(0.1), 2),
+            "p90_us": round(pick(0.9), 2), "mean_us": round(statistics.mean(s), 2)}
+
+
+def time_graph(queue, record, launches_per_replay, replays=12, warm=3):
+    """Compiles `record` into a graph; device time of each replay (events on the queue's
+    stream around the launch) divided by the launches it holds."""
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    record(cb)
+    cb.end_compute_pass()
+    cb.compile()
+    for _ in range(warm):
+        cb.commit().wait()
+    per_launch = [cb.commit().wait() * 1e3 / launches_per_replay for _ in range(replays)]
+    out = percentiles(per_launch)
+    out["launches"] = launches_per_replay * replays
+    return out
+
+
+def attention_figures(queue, wave):
+    """Key-walk kernel and whole attention layer of `wave` at its current contexts."""
+    n = len(wave.attn)
+    walk = time_graph(queue, lambda cb: [wave.record_attention(cb, i, walk_only=True)
+                                         for i in range(n)], n)
+    layer = time_graph(queue, lambda cb: [wave.record_attention(cb, i) for i in range(n)], n)
+    algo = wave.visible_keys() * ATTN_BYTES_PER_KEY
+    gbs = algo / (walk["median_us"] * 1e-6) / 1e9
+    return {"lanes_visible_keys": [c + 1 for c in wave.contexts], "algorithmic_bytes": algo,
+            "walk_kernel": walk, "walk_kernel_gbs": round(gbs, 1),
+            "walk_kernel_frac": round(gbs / HBM_PEAK_GBS, 4),
+            "layer_all_dispatches": layer,
+            "layer_frac": round(algo / (layer["median_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
@@ -291,6 +290,7 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
     attn_ms = flash_ms + best["attn_qk_rope_blk"]
     gdn_ms = sum(best[k] for k in ("gdn_conv_blk", "gdn_gates_blk", "gdn_chunk_recurrence_blk",
                                    "gdn_gate_norm_blk"))
+    gdn_flops = 32 * 7 * 128 * 128 * rows      # sequential-equivalent delta rule
     return {"rows": rows,
             "attention_layer_ms": round(attn_ms, 3),
             "attention_layer_tok_per_s": round(rows / (attn_ms * 1e-3)),
@@ -305,67 +305,147 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
                          "algorithmic_flops": flops},
             "gdn_layer_ms": round(gdn_ms, 3),
             "gdn_layer_tok_per_s": round(rows / (gdn_ms * 1e-3)),
+            "gdn_recurrence_note": "chunk-64 recurrence: bound by the serial chain over 256 chunks "
+                                   "and its chunk records, not by MFMA throughput",
+            "gdn_recurrence_frac_of_bf16_mfma_peak_sequential_equivalent": round(
+                gdn_flops / (best["gdn_chunk_recurrence_blk"] * 1e-3) / 2.5e15, 4),
             "kernel_ms": {k: round(v, 3) for k, v in best.items()}}
 
 
-def cpu_baseline(threads):
-    """The CPU checker (reference arithmetic restated, oracle/liboracle.so) on one
-    G,G,G,A period at the same shapes: 4 lanes x 32768 keys of attention decode and
-    3 x 4 lanes of GDN decode.  Baseline only; never part of the product path."""
+def _oracle():
     path = os.path.join(ROOT, "oracle", "liboracle.so")
     if not os.path.exists(path):
         return None
     L = C.CDLL(path)
     u16 = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
     f32 = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
-    L.tto_attention_decode_split.argtypes = [u16, u16, u16, u16, C.c_uint32, C.c_uint32,
-                                             C.c_uint32, C.c_void_p, u16, C.c_uint32]
+    u32 = np.ctypeslib.ndpointer(np.uint32, flags="C_CONTIGUOUS")
+    c32 = C.c_uint32
+    L.tto_attn_qk_rope.argtypes = [u16, u16, u16, c32, c32, u16, u16, u16, u16]
+    L.tto_attn_qk_rope.restype = None
+    L.tto_attention_decode_split.argtypes = [u16, u16, u16, u16, c32, c32, c32, C.c_void_p, u16, c32]
     L.tto_attention_decode_split.restype = None
-    L.tto_gdn_decode_step.argtypes = [u16] * 6 + [f32, u16, f32, u16, C.c_uint32]
+    L.tto_gdn_decode_step.argtypes = [u16] * 6 + [f32, u16, f32, u16, c32]
     L.tto_gdn_decode_step.restype = None
+    L.tto_attention_prefill.argtypes = [u16, u16, u16, c32, c32, c32, u16, u16, u16, u16, u32, c32,
+                                        u16, c32]
+    L.tto_attention_prefill.restype = None
+    L.tto_gdn_prefill.argtypes = [u16, c32, u16, u16, u16, u16, u16, f32, u16, f32, u16, u16, u16,
+                                  u16, c32]
+    L.tto_gdn_prefill.restype = None
+    return L
+
+
+def _bf16(rng, n, sigma=1.0):
+    x = rng.standard_normal(n, dtype=np.float32) * np.float32(sigma)
+    return (x.view(np.uint32) >> 16).astype(np.uint16)      # truncation is fine for random data
+
+
+def cpu_baseline(all_threads):
+    """The CPU checker (reference arithmetic restated, oracle/liboracle.so) on one G,G,G,A
+    period of the wave: per lane its own data, rope + append + 32768-key attention, and
+    3 x 4 lanes of GDN decode; timed with one thread and with all host threads.  Baseline
+    only; never part of the product path."""
+    L = _oracle()
+    if L is None:
+        return None
     rng = np.random.default_rng(7)
-
-    def bf16(n, sigma=1.0):
-        x = rng.standard_normal(n, dtype=np.float32) * np.float32(sigma)
-        return (x.view(np.uint32) >> 16).astype(np.uint16)   # truncation is fine for random data
-
-    keys = bf16(2 * CAPACITY * 256)
-    values = bf16(2 * CAPACITY * 256)
-    q, gate = bf16(4096), bf16(4096)
-    out = np.zeros(4096, np.uint16)
-    proj, cs, cw = bf16(12352, 0.5), bf16(3 * 8192, 0.5), bf16(4 * 8192, 0.5)
+    ones = np.full(256, 0x3F80, np.uint16)
+    lanes = []
+    for _ in range(LANES):
+        lanes.append(dict(keys=_bf16(rng, 2 * CAPACITY * 256), values=_bf16(rng, 2 * CAPACITY * 256),
+                          proj=_bf16(rng, 9216), gproj=_bf16(rng, 12352, 0.5),
+                          cs=_bf16(rng, 3 * 8192, 0.5),
+                          st=rng.standard_normal(32 * 128 * 128, dtype=np.float32) * np.float32(0.02)))
+    cw = _bf16(rng, 4 * 8192, 0.5)
     a_log = np.full(32, 0xC040, np.uint16)   # -3.0
     dtb = np.zeros(32, np.uint16)
     nw = np.full(128, 0x3F80, np.uint16)
-    st = (rng.standard_normal(32 * 128 * 128, dtype=np.float32) * 0.02)
-    ncs = np.zeros(3 * 8192, np.uint16)
-    so = np.zeros_like(st)
+    q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16); out = np.zeros(4096, np.uint16)
+    ncs = np.zeros(3 * 8192, np.uint16); so = np.zeros(32 * 128 * 128, np.float32)
     gated = np.zeros(4096, np.uint16)
+
+    def period(threads):
+        t0 = time.perf_counter()
+        for lane in lanes:
+            L.tto_attn_qk_rope(lane["proj"], ones, ones, VISIBLE - 1, CAPACITY, q, gate,
+                               lane["keys"], lane["values"])
+            L.tto_attention_decode_split(q, gate, lane["keys"], lane["values"], VISIBLE - 1,
+                                         CAPACITY, 256, None, out, threads)
+        t_attn = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        for _ in range(3):
+            for lane in lanes:
+                L.tto_gdn_decode_step(lane["gproj"], lane["cs"], cw, a_log, dtb, nw, lane["st"],
+                                      ncs, so, gated, threads)
+        return t_attn, time.perf_counter() - t0
+
+    a1, g1 = period(1)
+    an, gn = period(all_threads)
+    return {"value": round((an + gn) * 1e6 / 4.0, 1), "unit": "us/layer", "cores": all_threads,
+            "kind": "port", "host_cpu_count": os.cpu_count(),
+            "single_thread": {"value": round((a1 + g1) * 1e6 / 4.0, 1), "unit": "us/layer", "cores": 1,
+                              "attention_layer_us": round(a1 * 1e6), "gdn_layer_us": round(g1 * 1e6 / 3)},
+            "sample": "one full G,G,G,A period of the wave, 4 lanes x 32768 keys, distinct data per "
+                      f"lane, rope and append included (all threads: attention layer {an * 1e6:.0f} us, "
+                      f"GDN layer {gn * 1e6 / 3:.0f} us)"}
+
+
+def cpu_prefill_baseline(threads, rows=16384):
+    """The CPU checker beside the 16384-row block prefill: the attention layer on every 256th
+    query row (plus the rope of all rows), extrapolated by causal pair count; the GDN layer on
+    the first 2048 rows, extrapolated by rows."""
+    L = _oracle()
+    if L is None:
+        return None
+    rng = np.random.default_rng(11)
+    ones = np.full(256, 0x3F80, np.uint16)
+    proj = _bf16(rng, rows * 9216)
+    keys = np.zeros(2 * rows * 256, np.uint16); values = np.zeros_like(keys)
+    query = np.zeros(rows * 4096, np.uint16); gate = np.zeros_like(query); att = np.zeros_like(query)
+    sel = np.arange(255, rows, 256, dtype=np.uint32)
     t0 = time.perf_counter()
-    for _ in range(LANES):   # lanes are independent; same-shape data per lane
-        L.tto_attention_decode_split(q, gate, keys, values, VISIBLE - 1, CAPACITY, 256, None, out,
-                                     threads)
+    L.tto_attention_prefill(proj, ones, ones, rows, 0, rows, query, gate, keys, values, sel,
+                            len(sel), att, threads)
     t_attn = time.perf_counter() - t0
+    sampled_pairs = int(sum(int(r) + 1 for r in sel))
+    all_pairs = rows * (rows + 1) // 2
+    g_rows = 2048
+    gproj = _bf16(rng, g_rows * 12352, 0.5)
+    outs = [np.zeros(g_rows * 4096, np.uint16) for _ in range(4)]
+    conv = np.zeros(3 * 8192, np.uint16); state = np.zeros(32 * 128 * 128, np.float32)
     t0 = time.perf_counter()
-    for _ in range(3 * LANES):
-        L.tto_gdn_decode_step(proj, cs, cw, a_log, dtb, nw, st, ncs, so, gated, threads)
+    L.tto_gdn_prefill(gproj, g_rows, _bf16(rng, 3 * 8192, 0.5), _bf16(rng, 4 * 8192, 0.5),
+                      np.full(32, 0xC040, np.uint16), np.zeros(32, np.uint16),
+                      np.full(128, 0x3F80, np.uint16),
+                      rng.standard_normal(32 * 128 * 128, dtype=np.float32) * np.float32(0.02), conv,
+                      state, *outs, threads)
     t_gdn = time.perf_counter() - t0
-    return {"value": round((t_attn + t_gdn) * 1e6 / 4.0, 1), "unit": "us/layer",
-            "cores": threads, "kind": "port",
-            "sample": "one full G,G,G,A period, 4 lanes x 32768 keys (attention layer "
-                      f"{t_attn * 1e6:.0f} us, GDN layer {t_gdn * 1e6 / 3:.0f} us)"}
+    attn_full = t_attn * all_pairs / sampled_pairs
+    gdn_full = t_gdn * rows / g_rows
+    return {"kind": "port", "cores": threads, "extrapolated": True,
+            "attention_layer_tok_per_s": round(rows / attn_full, 1),
+            "gdn_layer_tok_per_s": round(rows / gdn_full, 1),
+            "sample": f"attention: {len(sel)} of {rows} query rows (every 256th) = {sampled_pairs} of "
+                      f"{all_pairs} causal pairs in {t_attn:.2f} s incl. the rope of all rows; GDN: first "
+                      f"{g_rows} of {rows} rows in {t_gdn:.2f} s"}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--attention", choices=("layer", "three"), default="three",
+                    help="three: rope, split and combine dispatches (the faster key walk); layer: one "
+                         "dispatch for the layer plus its finishing dispatch")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the 16384-row block prefill figures in detail.prefill_16k")
+    ap.add_argument("--no-config3", action="store_true",
+                    help="skip the ragged-lane and deep-lane figures in detail.config3")
     ap.add_argument("--split-keys", type=int, default=DEFAULT_SPLIT_KEYS,
-                    help="keys per split-K workgroup (multiple of 32)")
+                    help="keys per split-K workgroup of --attention three (multiple of 32)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device-to-device copies first, so a "
                          "counter run has a kernel of known traffic to scale its readings by")
@@ -383,7 +463,6 @@ def main():
     dev = B.Device()
     queue = dev.create_queue()
     lib = dev.create_library()
-    PART = args.split_keys
     if args.calibrate_copy:
         src = dev.create_buffer(CALIBRATION_COPY_BYTES)
         dst = dev.create_buffer(CALIBRATION_COPY_BYTES)
@@ -391,65 +470,37 @@ def main():
             cb = queue.create_command_buffer()
             cb.copy_buffer(src, 0, dst, 0, CALIBRATION_COPY_BYTES)
             cb.commit().wait()
-    record, record_split_only, keep = build_workload(B, dev, lib, torch, PART)
+    attention_layers = LAYERS // PERIOD
+    wave = Wave(dev, lib, torch, args.attention, args.split_keys, attention_layers,
+                LAYERS - attention_layers, CONFIG3["uniform"][0], CAPACITY)
 
-    steps = []
-    for copy in range(2):
-        cb = queue.create_command_buffer()
-        cb.begin_compute_pass()
-        record(cb, copy)
-        cb.end_compute_pass()
-        cb.compile()
-        steps.append(cb)
-
-    for k in range(args.warmup):
-        steps[k & 1].commit()
+    step = queue.create_command_buffer()
+    step.begin_compute_pass()
+    wave.record_wave(step)
+    step.end_compute_pass()
+    step.compile()
+    for _ in range(args.warmup):
+        step.commit()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for k in range(args.steps):
-        steps[k & 1].commit()
+    for _ in range(args.steps):
+        step.commit()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+    # the same step, device time of single replays (median and tails)
+    step_us = percentiles([step.commit().wait() * 1e3 for _ in range(max(20, min(args.steps, 100)))])
 
-    # per-kernel device time: eager commits with an event after every command
-    prof = []
-    for copy in range(2):
-        cb = queue.create_command_buffer()
-        cb.begin_compute_pass()
-        record(cb, copy)
-        cb.end_compute_pass()
-        cb.set_profiling(True)
-        prof.append(cb)
-    per_kernel = {}
-    reps = 30
-    for k in range(reps):
-        cb = prof[k & 1]
-        cb.commit().wait()
-        for name, ms in cb.command_times():
-            per_kernel.setdefault(name, []).append(ms)
-    # one list entry per launch: average launch duration of each kernel
-    kernel_us = {name: round(statistics.mean(v) * 1e3, 2) for name, v in per_kernel.items()}
-    # the dominant kernel alone, back to back between one pair of events on its
-    # stream, alternating the two KV copies: average launch duration
-    cb = queue.create_command_buffer()
-    cb.begin_compute_pass()
-    launches = 40
-    for k in range(launches):
-        record_split_only(cb, k & 1)
-    cb.end_compute_pass()
-    cb.commit().wait()
-    split_us = round(statistics.mean(cb.commit().wait() for _ in range(3)) * 1e3 / launches, 2)
-    algo_bytes = LANES * VISIBLE * ATTN_BYTES_PER_KEY
-    achieved = algo_bytes / (split_us * 1e-6) / 1e9
-    attn_layer_us = sum(kernel_us[k] for k in ("attn_qk_rope_ms", "attention_decode_split_ms",
-                                               "attention_decode_combine_ms"))
-    gdn_layer_us = kernel_us["gdn_decode_fused_ms"]
-    gdn_gbs = LANES * GDN_BYTES_PER_LANE_LAYER / (gdn_layer_us * 1e-6) / 1e9
-
+    uniform = attention_figures(queue, wave)
+    gdn = time_graph(queue, lambda cb: [wave.record_gdn(cb, i) for i in range(len(wave.gdn))],
+                     len(wave.gdn))
+    gdn_gbs = LANES * GDN_BYTES_PER_LANE_LAYER / (gdn["median_us"] * 1e-6) / 1e9
+    walk = uniform["walk_kernel"]
+    kernel_name = ("attention_decode_layer_ms (attention_decode_layer_kernel)"
+                   if args.attention == "layer" else "attention_decode_split_ms (flash_decode_kernel)")
     line = {
         "metric": "decode attn+GDN us/layer @32k ctx x4 lanes",
-        "value": round(ms_per_step * 1e3 / 4.0, 3),
+        "value": round(ms_per_step * 1e3 / LAYERS, 3),
         "unit": "us/layer",
         "n_gpus": 1,
         "steps": args.steps,
@@ -460,32 +511,58 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "decode wave, 4 lanes x 32768 visible keys, one G,G,G,A period "
-                               "(3 GDN layers + 1 full-attention layer), HIP-graph replay",
-                   "lanes": LANES, "visible_keys": VISIBLE, "capacity": CAPACITY,
-                   "split_keys": PART, "device": dev.name},
-        "roofline": {"bound": "hbm", "kernel": "attention_decode_split_ms (flash_decode_kernel)",
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (round((FLASH_FETCH_KIB * FETCH_SCALE +
-                                        FLASH_WRITE_KIB * WRITE_SCALE) * 1024)
-                                 if PART == DEFAULT_SPLIT_KEYS else None),
-                     "algorithmic_bytes": algo_bytes, "avg_launch_us": split_us},
-        "detail": {"attention_layer_us": round(attn_layer_us, 2),
-                   "gdn_layer_us": round(gdn_layer_us, 2),
-                   "gdn_layer_gbs": round(gdn_gbs, 1),
-                   "kernel_avg_us": kernel_us},
+        "config": {"workload": "decode token wave, 4 lanes x 32768 visible keys, attention family of "
+                               "the 40-layer stack (G,G,G,A x 10: 30 GDN + 10 full-attention layers, "
+                               "own KV / state per layer), one HIP-graph replay per wave",
+                   "lanes": LANES, "visible_keys": VISIBLE, "capacity": CAPACITY, "layers": LAYERS,
+                   "attention_form": args.attention, "workgroups": wave.groups,
+                   "split_keys": args.split_keys if args.attention == "three" else None,
+                   "device": dev.name},
+        "roofline": {"bound": "hbm", "kernel": kernel_name,
+                     "achieved": uniform["walk_kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": uniform["walk_kernel_frac"], "traffic": TRAFFIC_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE if TRAFFIC_BYTES else None,
+                     "algorithmic_bytes": uniform["algorithmic_bytes"],
+                     "avg_launch_us": walk["mean_us"], "median_launch_us": walk["median_us"],
+                     "p10_launch_us": walk["p10_us"], "p90_launch_us": walk["p90_us"],
+                     "launches": walk["launches"],
+                     "how": "graph of this kernel alone, once per attention layer (10 KV sets), "
+                            "HIP events on the queue's stream around each replay"},
+        "detail": {"step_device_us": step_us,
+                   "attention_layer_us": uniform["layer_all_dispatches"],
+                   "attention_layer_frac_of_hbm_peak": uniform["layer_frac"],
+                   "gdn_layer_us": gdn, "gdn_layer_gbs": round(gdn_gbs, 1),
+                   "gdn_layer_frac_of_hbm_peak": round(gdn_gbs / HBM_PEAK_GBS, 4)},
     }
+    if not args.no_config3:
+        config3 = {"uniform": uniform}
+        wave.set_contexts(CONFIG3["ragged"][0])
+        config3["ragged"] = attention_figures(queue, wave)
+        del wave, step
+        torch.cuda.empty_cache()
+        deep = Wave(dev, lib, torch, args.attention, args.split_keys, 4, 0, *CONFIG3["lane100k"])
+        config3["lane100k"] = attention_figures(queue, deep)
+        del deep
+        torch.cuda.empty_cache()
+        line["detail"]["config3"] = config3
+    else:
+        del wave, step
+        torch.cuda.empty_cache()
+    # host threads of the CPU legs: what this process may run on, bounded by the box's CPU
+    # share where the environment states one (OMP_NUM_THREADS)
+    threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        threads = max(1, min(threads, int(os.environ["OMP_NUM_THREADS"])))
     if not args.no_prefill:
         line["detail"]["prefill_16k"] = prefill_figures(B, dev, queue, lib, torch)
-    if not args.no_prefill:
+        if not args.no_cpu_baseline:
+            line["detail"]["prefill_16k"]["cpu_baseline"] = cpu_prefill_baseline(threads)
         from tatara_amd import q4_sweep
         line["detail"]["q4_projections"] = (
             [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)
              for name in q4_sweep.FAMILIES] +
             [q4_sweep.measure(dev, queue, lib, name, 16384, True, 2) for name in q4_sweep.FAMILIES])
     if not args.no_cpu_baseline:
-        threads = min(16, os.cpu_count() or 1)
         line["cpu_baseline"] = cpu_baseline(threads)
     print(json.dumps(line))
 

@@ -51,6 +51,11 @@ constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
 constexpr uint32_t kLdsPairBytes = 1040;    // key i row | key 16+i row | 16 B pad
 constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16640
 constexpr uint32_t kWaves = 4;
+// Cache policy of the K transfers and V loads: every key and value byte is used once per
+// dispatch, so it is requested nontemporal (the `nt` bit; V through
+// __builtin_nontemporal_load) and does not displace what the caches hold.  Measured on the
+// 4 x 32768 walk: 51.9 us with the default policy, 48.3 us with it.
+constexpr uint32_t kStreamOnce = 2;
 constexpr uint32_t kMergeTileFloats = 20;   // 16 accumulator words of one MFMA + 4 pad
 constexpr uint32_t kMergeHeadFloats = 16 * kMergeTileFloats + 4;  // 324: head stride of the merge
 // Bound of the rows a state table may carry (decode_step.cpp:1007-1009).
@@ -362,7 +367,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(src),
                 (__attribute__((address_space(3))) void*)(stage + i * kLdsPairBytes),
-                16, 0, 0);
+                16, 0, kStreamOnce);
         }
     };
 
@@ -374,8 +379,8 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) {
             const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
-            vhalf[e] = *reinterpret_cast<const u32x4*>(
-                vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8);
+            vhalf[e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8));
         }
     };
 
@@ -692,8 +697,23 @@ __device__ __forceinline__ HeadLoads load_head(const uint16_t* x, const uint16_t
     }
     return h;
 }
-__device__ __forceinline__ void norm_rope_head(const HeadLoads& h, uint32_t position, uint32_t lane,
-                                               float (&out)[4]) {
+// Cosine and sine of the rotation of pair (lane & 31) at `position`: the same for every
+// head of a row, so a wave evaluates them once (one shared argument reduction) for all the
+// heads it norms.
+struct RopeAngle {
+    float c, s;
+};
+__device__ __forceinline__ RopeAngle rope_angle(uint32_t position, uint32_t lane) {
+    const uint32_t pair = lane & (kAttnRopePairs - 1);
+    const float inverse_frequency =
+        powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs));
+    const float theta = static_cast<float>(position) / inverse_frequency;
+    RopeAngle a;
+    sincosf(theta, &a.s, &a.c);
+    return a;
+}
+__device__ __forceinline__ void norm_rope_head(const HeadLoads& h, const RopeAngle& angle,
+                                               uint32_t lane, float (&out)[4]) {
     float acc = 0.0f;
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
@@ -709,15 +729,10 @@ __device__ __forceinline__ void norm_rope_head(const HeadLoads& h, uint32_t posi
         out[c] = round_bf16(bf16_bits_to_f32(h.w[c]) * round_bf16(bf16_bits_to_f32(h.x[c]) * inverse));
     }
     // dims below 64 rotate: lane l holds dim l, its partner (l ^ 32) the other half of the pair
-    const uint32_t pair = lane & (kAttnRopePairs - 1);
-    const float inverse_frequency =
-        powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs));
-    const float theta = static_cast<float>(position) / inverse_frequency;
-    const float c = cosf(theta);
-    const float sn = sinf(theta);
     const float n = out[0];
     const float partner = __shfl_xor(n, kAttnRopePairs, 64);
-    const float rotated = lane < kAttnRopePairs ? fmaf(-partner, sn, n * c) : fmaf(partner, sn, n * c);
+    const float rotated = lane < kAttnRopePairs ? fmaf(-partner, angle.s, n * angle.c)
+                                                : fmaf(partner, angle.s, n * angle.c);
     out[0] = round_bf16(rotated);
 }
 
@@ -726,12 +741,12 @@ __device__ __forceinline__ void norm_rope_head(const HeadLoads& h, uint32_t posi
 // the cache at position `context`.
 __device__ __forceinline__ void new_token_rows(const LayerArgs& a, const uint16_t* proj,
                                                uint32_t kvh, uint32_t context, uint64_t kv_offset,
-                                               bool append, uint32_t lane, float (&kn)[4],
-                                               uint16_t (&vraw)[4]) {
+                                               const RopeAngle& angle, bool append, uint32_t lane,
+                                               float (&kn)[4], uint16_t (&vraw)[4]) {
     const HeadLoads kl = load_head(proj + kAttnQGateRows + kvh * kD, a.k_weight, lane);
 #pragma unroll
     for (uint32_t c = 0; c < 4; ++c) vraw[c] = proj[kAttnVRowOffset + kvh * kD + lane + 64 * c];
-    norm_rope_head(kl, context, lane, kn);
+    norm_rope_head(kl, angle, lane, kn);
     if (append) {
         const uint64_t at = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
 #pragma unroll
@@ -957,7 +972,7 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)(src),
                     (__attribute__((address_space(3))) void*)(stage + i * kLdsPairBytes),
-                    16, 0, 0);
+                    16, 0, kStreamOnce);
             }
         };
         auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
@@ -966,8 +981,8 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
 #pragma unroll
             for (uint32_t e = 0; e < 8; ++e) {
                 const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
-                vhalf[e] = *reinterpret_cast<const u32x4*>(
-                    vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8);
+                vhalf[e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                    vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8));
             }
         };
 
@@ -981,10 +996,11 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
         // query heads in the scratch and appends the token's key and value rows (no key walk
         // reads position `context`), so the finishing dispatch only loads them
         const bool publishes = !kFinishInKernel && unit == stream_first;
+        const RopeAngle angle = rope_angle(context, lane);
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             float n[4];
-            norm_rope_head(ql[i], context, lane, n);
+            norm_rope_head(ql[i], angle, lane, n);
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
                 const uint16_t bits = f32_to_bf16_bits(n[c]);
@@ -998,7 +1014,7 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
         if (publishes && wave == 0) {
             float kn[4];
             uint16_t vraw[4];
-            new_token_rows(a, proj, kvh, context, kv_offset, true, lane, kn, vraw);
+            new_token_rows(a, proj, kvh, context, kv_offset, angle, true, lane, kn, vraw);
         }
         __syncthreads();
         // B operand of S^T: Q^T, column m holds head (m & 7)
@@ -1197,8 +1213,8 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
                     // eight records at a time: the key walk above leaves no registers for more
                     finish_head<8>(a, row, kvh * kAttnHeadsPerKv + h, first_group + stream, count, q,
                                    [&](float (&kn)[4], uint16_t (&vraw)[4]) {
-                                       new_token_rows(a, proj, kvh, context, kv_offset, h == 0,
-                                                      lane, kn, vraw);
+                                       new_token_rows(a, proj, kvh, context, kv_offset, angle,
+                                                      h == 0, lane, kn, vraw);
                                    },
                                    lane);
                 }

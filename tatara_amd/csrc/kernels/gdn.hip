@@ -368,7 +368,7 @@ __global__ __launch_bounds__(256) void gdn_recurrence_kernel(RecurrenceArgs a) {
             a.y[row_y + static_cast<uint64_t>(step) * a.y_stride + h * kGD + j] = narrow(out);
         }
     }
-    *reinterpret_cast<f32x4*>(state_out + base) = st;
+    __builtin_nontemporal_store(st, reinterpret_cast<f32x4*>(state_out + base));  // read next by a later dispatch
 }
 
 // gdn_tape_replay_blk (prefill_gdn.metal:520-569): the state after `steps` rows of
@@ -527,7 +527,6 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     __shared__ float qk_n[2 * kGD];     // normalised, scaled q | k (bf16 values)
     __shared__ float y_head[kGD];       // bf16 values of the head's outputs
     __shared__ float inverse[2];
-    __shared__ float gates[2];
     __shared__ float partial[2];
     const uint32_t h = blockIdx.x;
     const uint32_t row = blockIdx.y;
@@ -540,8 +539,27 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     float* state_out = a.rec_pool_out + a.table[row * 4 + 3];
     const uint32_t half = tid >> 5;  // 0..15
     const uint32_t lane = tid & 31;
-    // the state rows this half wave walks are requested first: their 64 KiB per head
-    // arrive while the conv, norm and gate stages run
+    // Loads come back in the order they were requested.  The few bytes the conv, norm and
+    // gate stages need go out first, the head's 64 KiB of state right behind them: those
+    // stages then run while the state is still arriving instead of after it.
+    // Every thread issues every one of them (threads past the 384 channels repeat the value
+    // channels): a load inside a branch would be waited for before the branch ends, one
+    // round trip after the other.
+    const uint16_t z_bits = proj[kCh + h * kGD + (tid & 127)];
+    const uint16_t norm_bits = a.norm_weight[tid & 127];
+    const uint32_t part = min(tid >> 7, 2u);  // 0 q, 1 k, 2 v
+    const uint32_t c = (part == 0 ? kh * kGD : part == 1 ? kGdnKOffset + kh * kGD
+                                                         : kGdnQkValues + h * kGD) + (tid & 127);
+    const uint16_t t0 = conv_in[c];
+    const uint16_t t1 = conv_in[kCh + c];
+    const uint16_t t2 = conv_in[2 * kCh + c];
+    const uint16_t t3 = proj[c];
+    const uint16_t* w = a.conv_weights + static_cast<uint64_t>(c) * 4;
+    const uint16_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3];
+    const uint16_t gate_a = proj[kGdnARowOffset + h];
+    const uint16_t gate_b = proj[kGdnBRowOffset + h];
+    const uint16_t gate_log = a.a_log[h];
+    const uint16_t gate_bias = a.dt_bias[h];
     f32x4 st[8];
 #pragma unroll
     for (uint32_t it = 0; it < 8; ++it) {
@@ -549,31 +567,22 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
         st[it] = *reinterpret_cast<const f32x4*>(
             state_in + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4);
     }
-    const uint16_t z_bits = tid < kGD ? proj[kCh + h * kGD + tid] : uint16_t{0};
-    const uint16_t norm_bits = tid < kGD ? a.norm_weight[tid] : uint16_t{0};
 
+    // computed by every thread as well, so that the loads above cannot be moved into a
+    // branch behind the state loads; only the stores are conditional
+    const float convolved = widen(w0) * widen(t0) + widen(w1) * widen(t1) +
+                            widen(w2) * widen(t2) + widen(w3) * widen(t3);
+    const float conv_b = rb(convolved);
+    const float activated = rb(conv_b * sigmoid_bf16(conv_b));
+    float decay, beta;
+    head_gates(gate_a, gate_b, gate_log, gate_bias, decay, beta);
     if (tid < 3 * kGD) {
-        const uint32_t part = tid >> 7;  // 0 q, 1 k, 2 v
-        const uint32_t c = (part == 0 ? kh * kGD : part == 1 ? kGdnKOffset + kh * kGD
-                                                             : kGdnQkValues + h * kGD) + (tid & 127);
-        const uint16_t t0 = conv_in[c], t1 = conv_in[kCh + c], t2 = conv_in[2 * kCh + c];
-        const uint16_t t3 = proj[c];
-        const uint16_t* w = a.conv_weights + static_cast<uint64_t>(c) * 4;
-        const float convolved = widen(w[0]) * widen(t0) + widen(w[1]) * widen(t1) +
-                                widen(w[2]) * widen(t2) + widen(w[3]) * widen(t3);
-        const float conv_b = rb(convolved);
-        act[tid] = rb(conv_b * sigmoid_bf16(conv_b));
+        act[tid] = activated;
         if (part == 2 || (h & 1) == 0) {
             conv_out[c] = t1;
             conv_out[kCh + c] = t2;
             conv_out[2 * kCh + c] = t3;
         }
-    } else if (tid == 3 * kGD) {
-        float decay, beta;
-        head_gates(proj[kGdnARowOffset + h], proj[kGdnBRowOffset + h], a.a_log[h], a.dt_bias[h],
-                   decay, beta);
-        gates[0] = decay;
-        gates[1] = beta;
     }
     __syncthreads();
     if (tid < 64) {  // lanes 0..31: q head, 32..63: k head; lane l sums squares 4l..4l+3
@@ -591,8 +600,6 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     }
     __syncthreads();
 
-    const float decay = gates[0];
-    const float beta = gates[1];
     float q4[4], k4[4];
 #pragma unroll
     for (uint32_t i = 0; i < 4; ++i) {
@@ -617,8 +624,10 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
             out = fmaf(st[it][i], q4[i], out);
         }
         out = half_wave_sum(out);
-        *reinterpret_cast<f32x4*>(state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4) =
-            st[it];
+        // written once, read by the next token's dispatch at the earliest: stored past the
+        // cache (nontemporal), so the dispatch does not end on a write-back of the whole state
+        __builtin_nontemporal_store(st[it], reinterpret_cast<f32x4*>(
+            state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4));
         if (lane == 0) y_head[j] = rb(out);
     }
     __syncthreads();
