@@ -56,8 +56,8 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # HBM traffic of one launch of the key-walk kernel at 4 lanes x 32768 keys, from two rocprofv3
 # counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
 # counter read for a plain 256 MiB copy of known size; see the file named here.
-TRAFFIC_SOURCE = "profiles/decode_layer_4x32768_hbm_counters.md"
-TRAFFIC_BYTES = None            # filled from the counter runs; None until they exist
+TRAFFIC_SOURCE = "profiles/flash_decode_4x32768_hbm_counters.md"
+TRAFFIC_BYTES = round((131297.1 * 262144.0 / 131083.3 + 2112.0) * 1024)   # 271,035,969
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 CONFIG3 = {
@@ -520,8 +520,9 @@ def main():
                    "device": dev.name},
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": uniform["walk_kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": uniform["walk_kernel_frac"], "traffic": TRAFFIC_BYTES,
-                     "traffic_source": TRAFFIC_SOURCE if TRAFFIC_BYTES else None,
+                     "frac": uniform["walk_kernel_frac"],
+                     "traffic": TRAFFIC_BYTES if args.attention == "three" else None,
+                     "traffic_source": TRAFFIC_SOURCE if args.attention == "three" else None,
                      "algorithmic_bytes": uniform["algorithmic_bytes"],
                      "avg_launch_us": walk["mean_us"], "median_launch_us": walk["median_us"],
                      "p10_launch_us": walk["p10_us"], "p90_launch_us": walk["p90_us"],
