@@ -99,8 +99,15 @@ class StubStack:
     state and the scratch, and records token waves and prefill blocks."""
 
     def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
-                 split_keys=None):
+                 split_keys=None, attention_form="three"):
+        """attention_form: "three" records a token wave's attention layer as rope, split-K
+        and combine dispatches (split_keys keys per workgroup); "layer" as the whole-layer
+        dispatch plus its finishing dispatch (keys dealt evenly to one workgroup per compute
+        unit, whatever the lanes' depths)."""
+        assert attention_form in ("three", "layer")
         self.dev, self.lib = dev, lib
+        self.attention_form = attention_form
+        self.groups = dev.compute_units
         self.lanes, self.capacity, self.vocab = lanes, capacity, vocab
         self.block_rows = block_rows
         self.split_keys = split_keys or choose_split_keys(lanes, capacity)
@@ -142,6 +149,7 @@ class StubStack:
         self.q, self.gate = mk(rows * 8192), mk(rows * 8192)
         self.decay, self.beta = mk(rows * 128), mk(rows * 128)
         self.partials = mk(lanes * 16 * self.max_splits * 258 * 4)
+        self.layer_scratch = mk(256 + 131072 + (self.groups + 2 * lanes - 1) * 8 * 258 * 4)
         self.chunk = mk(((min(block_rows, 2048) + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
         self.logits = mk(rows * vocab * 2)
         self._write_tables()
@@ -241,6 +249,15 @@ class StubStack:
                           {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
                            4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: self.mixed,
                            8: layer["table"]}, {9: GDN_PROJ, 10: 4096}, (32, rows), (512,))
+            elif self.attention_form == "layer":
+                bind = {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: layer["keys"],
+                        4: layer["values"], 5: layer["table"], 6: self.layer_scratch, 7: self.mixed}
+                const = {8: self.capacity, 9: ATTN_PROJ, 10: 4096}
+                cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: 0},
+                          (self.groups, rows), (256,))
+                cb.barrier()
+                cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: self.groups},
+                          (16, rows), (64,))
             else:
                 cb.encode(P("attn_qk_rope_ms"),
                           {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,

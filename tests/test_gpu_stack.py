@@ -17,13 +17,19 @@ from gpu_util import gpu, run
 pytestmark = pytest.mark.gpu
 o = ol.oracle
 THREADS = 16
+_WIDE = {}
 
 
 class OracleLane:
     """One lane of the stack on the CPU checker."""
 
-    def __init__(self, weights, capacity, vocab):
+    def __init__(self, weights, capacity, vocab, fast_dense=False):
+        """fast_dense: the stub's dense projections (which have no reference counterpart; the
+        operator-level test holds the GPU kernel to tto_dense_bf16) are evaluated as a
+        float32 matrix product by numpy instead of the checker's scalar loop, so that a
+        stack of thousands of rows stays within a minute of CPU time."""
         self.w, self.cap, self.vocab = weights, capacity, vocab
+        self.fast_dense = fast_dense
         self.context = 0
         self.state = []
         for lw in weights["layers"]:
@@ -34,10 +40,19 @@ class OracleLane:
                 self.state.append({"keys": np.zeros(2 * capacity * 256, np.uint16),
                                    "values": np.zeros(2 * capacity * 256, np.uint16)})
 
-    @staticmethod
-    def _project_in(lw, n, rows, width, p):
+    def _dense(self, x, w, rows, k, n, out):
+        if not self.fast_dense:
+            o.tto_dense_bf16(x, w, rows, k, n, out, THREADS)
+            return
+        key = id(w)
+        if key not in _WIDE:          # float32 copies of the weights, shared by the lanes
+            _WIDE[key] = np.ascontiguousarray(ol.bf16_to_f32(w).reshape(n, k).T)
+        out[:rows * n] = ol.f32_to_bf16((ol.bf16_to_f32(x[:rows * k]).reshape(rows, k) @
+                                         _WIDE[key]).reshape(-1))
+
+    def _project_in(self, lw, n, rows, width, p):
         if "in_q4" not in lw:
-            o.tto_dense_bf16(n, lw["w_in"], rows, 2048, width, p, THREADS)
+            self._dense(n, lw["w_in"], rows, 2048, width, p)
             return
         first = 0
         for words, scales, biases in lw["in_q4"]:
@@ -73,13 +88,13 @@ class OracleLane:
                 words, scales, biases = lw["out_q4"]
                 o.tto_q4_project(a, 4096, rows, words, scales, biases, 4096, 2048, d, 2048, THREADS)
             else:
-                o.tto_dense_bf16(a, lw["w_out"], rows, 4096, 2048, d, THREADS)
+                self._dense(a, lw["w_out"], rows, 4096, 2048, d)
             o.tto_add_bf16(x, d, rows * 2048, x)
         self.context += rows
         n = np.zeros(rows * 2048, np.uint16)
         o.tto_rms_only(x, self.w["final_norm"], rows, 2048, n)
         logits = np.zeros(rows * self.vocab, np.uint16)
-        o.tto_dense_bf16(n, self.w["vocab"], rows, 2048, self.vocab, logits, THREADS)
+        self._dense(n, self.w["vocab"], rows, 2048, self.vocab, logits)
         return ol.bf16_to_f32(logits).reshape(rows, self.vocab)
 
 
@@ -246,3 +261,80 @@ def test_add_bf16_operator_bit_for_bit():
     run(lambda cb: cb.encode(lib.pipeline("add_bf16"), {0: b_a, 1: b_b, 2: b_a}, {3: n},
                              ((n + 255) // 256,), (256,)))
     assert np.array_equal(b_a.read(np.uint16), want)
+
+
+_DEPTH = {}
+
+
+def _depth_reference(layers, vocab, capacity, prompts, waves):
+    """The checker's side of the run at depth, evaluated once for both attention forms:
+    last-row logits of every lane's prefill and every lane's logits of each greedy wave."""
+    from tatara_amd import stack as S
+    key = (layers, vocab, capacity, tuple(len(p) for p in prompts), waves)
+    if key in _DEPTH:
+        return _DEPTH[key]
+    weights = S.make_weights(layers, vocab, 0xD3E9)
+    embed = weights["embed"].reshape(vocab, 2048)
+    lanes = [OracleLane(weights, capacity, vocab, fast_dense=True) for _ in prompts]
+    prefill, tokens = [], []
+    for lane, prompt in enumerate(prompts):
+        print(f"[checker] prefill lane {lane}: {len(prompt)} rows", flush=True)
+        want = lanes[lane].block(np.ascontiguousarray(embed[prompt]).reshape(-1), len(prompt))
+        prefill.append(want[-1])
+        tokens.append(int(want[-1].argmax()))
+    steps = []
+    for step in range(waves):
+        print(f"[checker] greedy wave {step}", flush=True)
+        row = [lanes[lane].block(np.ascontiguousarray(embed[tokens[lane]]), 1)[0]
+               for lane in range(len(prompts))]
+        steps.append((list(tokens), row))
+        tokens = [int(r.argmax()) for r in row]
+    _DEPTH[key] = (weights, prefill, steps)
+    return _DEPTH[key]
+
+
+@pytest.mark.parametrize("form", ["three", "layer"])
+def test_stacked_run_at_depth_four_ragged_lanes(form):
+    """Config 5 at depth: 12 layers (G,G,G,A x 3), four lanes with prompts of 1024, 640,
+    384 and 160 tokens prefilled in blocks of 512 rows (two blocks for the longer ones), then
+    three greedy token waves of all four lanes through the pooled-state operators, with the
+    split size the stack chooses for itself (form "three") or the whole-layer dispatch (form
+    "layer").  Every greedy token must be the checker's (ties within two bf16 steps of the
+    winning logit aside, as in the shallow run)."""
+    print(f"[case] stacked run at depth, attention form {form}", flush=True)
+    from tatara_amd import stack as S
+    B, dev, queue, lib = gpu()
+    layers, vocab, capacity, block_rows, waves = 12, 4096, 1280, 512, 3
+    rng = np.random.default_rng(17)
+    prompts = [rng.integers(0, vocab, n) for n in (1024, 640, 384, 160)]
+    weights, want_prefill, want_steps = _depth_reference(layers, vocab, capacity, prompts, waves)
+    embed = weights["embed"].reshape(vocab, 2048)
+    stack = S.StubStack(dev, lib, weights, len(prompts), capacity, vocab, block_rows=block_rows,
+                        attention_form=form)
+    assert stack.split_keys == S.choose_split_keys(len(prompts), capacity)
+    for lane, prompt in enumerate(prompts):
+        for first in range(0, len(prompt), block_rows):
+            rows = min(block_rows, len(prompt) - first)
+            stack.x.write(np.ascontiguousarray(embed[prompt[first:first + rows]]).reshape(-1))
+            cb = queue.create_command_buffer()
+            cb.begin_compute_pass()
+            stack.record_prefill_block(cb, lane, rows, chunked=True, with_head=True)
+            cb.end_compute_pass()
+            cb.commit().wait()
+            stack.advance_prefill_block(lane, rows)
+        got = ol.bf16_to_f32(stack.logits.read(np.uint16, rows * vocab)).reshape(rows, vocab)
+        _compare(f"depth prefill lane {lane} ({len(prompt)} rows) last row", got[-1],
+                 want_prefill[lane])
+    assert stack.context == [len(p) for p in prompts]
+    for step, (tokens, want_rows) in enumerate(want_steps):
+        stack.x.write(np.ascontiguousarray(embed[tokens]).reshape(-1))
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        stack.record_token_wave(cb)
+        cb.end_compute_pass()
+        cb.commit().wait()
+        stack.advance_token_wave()
+        got = ol.bf16_to_f32(stack.logits.read(np.uint16, len(prompts) * vocab)).reshape(-1, vocab)
+        for lane in range(len(prompts)):
+            _compare(f"depth wave {step} lane {lane} (context {stack.context[lane] - 1})",
+                     got[lane], want_rows[lane])
