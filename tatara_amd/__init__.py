@@ -9,4 +9,4 @@ There is no CPU or PyTorch fallback: importing `tatara_amd.backend` raises if th
 library has not been built (`python -c "import __graft_entry__ as g; g.build()"`
 or `make -C tatara_amd/csrc`)."""
 
-__all__ = ["backend", "layout"]
+__all__ = ["backend", "stack", "sweep", "q4_sweep"]
