@@ -267,6 +267,33 @@ DecodeStateSlotResult create_decode_state_slot(const HipDevice& device, const De
                                step.schedule.data());
 }
 
+namespace {
+
+// What one layer of one lane keeps on the device.  Both layer kinds hold two buffers: `first`
+// (conv history | keys) and `second` (recurrent state | values); a Gated DeltaNet layer holds
+// each as a ping-pong pair of planes, an attention layer as a single plane.  Everything that
+// walks a slot's buffers (pool carving, completeness) goes through this table.
+struct LayerFootprint {
+    std::uint64_t bytes[2];   // [0] first, [1] second
+    std::uint32_t planes;     // 1 or 2 planes of each
+};
+
+LayerFootprint footprint_of(const DecodeGeometry& g, LayerKind kind) noexcept {
+    if (is_gated(kind)) return {{g.gdn_conv_state_bytes, g.gdn_recurrent_state_bytes}, 2};
+    return {{g.attn_cache_bytes, g.attn_cache_bytes}, 1};
+}
+
+// plane p of buffer b of a layer's state: [b][p]
+HipBuffer DecodeLayerState::*const kPlaneOf[2][2] = {
+    {&DecodeLayerState::first, &DecodeLayerState::first_out},
+    {&DecodeLayerState::second, &DecodeLayerState::second_out},
+};
+
+}  // namespace
+
+// One striped pool per layer and buffer (decode_step.cpp:460-540): slot s owns stripes
+// planes * s .. planes * s + planes - 1, so a state table addresses a lane's planes as
+// (planes * stripe + plane) * stride.  The slots' buffers are windows into the pools.
 DecodeStateSlotPoolResult create_decode_state_slot_pool(const HipDevice& device,
                                                         const DecodeStep& step,
                                                         std::uint32_t count) {
@@ -279,60 +306,48 @@ DecodeStateSlotPoolResult create_decode_state_slot_pool(const HipDevice& device,
         result.error = DecodeStepError::OffsetCountMismatch;
         return result;
     }
+    // state-table offsets are u32 element counts of at least two bytes (decode_step.cpp:476)
+    constexpr std::uint64_t kAddressableBytes = 0xffffffffull * 2;
     DecodeStatePool pool;
     pool.stripes = count;
-    result.slots.resize(count);
-    for (DecodeStateSlot& slot : result.slots) {
+    std::vector<DecodeStateSlot> slots(count);
+    for (DecodeStateSlot& slot : slots) {
         slot.capacity = step.capacity;
         slot.schedule_identity = step.schedule.data();
-        slot.layers.reserve(step.schedule.size());
+        slot.layers.resize(step.schedule.size());
     }
-    const auto fail = [&result]() {
-        result.error = DecodeStepError::BufferAllocationFailed;
-        result.slots.clear();
-        return std::move(result);
-    };
-    for (const LayerKind kind : step.schedule) {
-        const bool gated = is_gated(kind);
-        const std::uint64_t first_bytes =
-            gated ? step.geometry.gdn_conv_state_bytes : step.geometry.attn_cache_bytes;
-        const std::uint64_t second_bytes =
-            gated ? step.geometry.gdn_recurrent_state_bytes : step.geometry.attn_cache_bytes;
-        const std::uint32_t stripes = gated ? 2u * count : count;
+    bool ok = true;
+    for (std::size_t index = 0; ok && index < step.schedule.size(); ++index) {
+        const LayerFootprint shape = footprint_of(step.geometry, step.schedule[index]);
         DecodeStatePoolLayer layer;
-        auto first = create_striped_pool_buffer(device, first_bytes, stripes);
-        auto second = create_striped_pool_buffer(device, second_bytes, stripes);
-        // offsets in the state table are u32 element counts (decode_step.cpp:476)
-        if (!first || !second || first.buffer->size_bytes() > 0xffffffffull * 2 ||
-            second.buffer->size_bytes() > 0xffffffffull * 2) {
-            return fail();
-        }
-        layer.first = std::move(*first.buffer);
-        layer.second = std::move(*second.buffer);
-        layer.first_stride = first.stripe_stride_bytes;
-        layer.second_stride = second.stripe_stride_bytes;
-        for (std::uint32_t slot = 0; slot < count; ++slot) {
-            DecodeLayerState state;
-            const std::uint64_t base = gated ? std::uint64_t{slot} * 2 : std::uint64_t{slot};
-            auto w0 = create_buffer_window(layer.first, base * layer.first_stride, first_bytes);
-            auto w1 = create_buffer_window(layer.second, base * layer.second_stride, second_bytes);
-            if (!w0 || !w1) return fail();
-            state.first = std::move(*w0.buffer);
-            state.second = std::move(*w1.buffer);
-            if (gated) {
-                auto o0 =
-                    create_buffer_window(layer.first, (base + 1) * layer.first_stride, first_bytes);
-                auto o1 = create_buffer_window(layer.second, (base + 1) * layer.second_stride,
-                                               second_bytes);
-                if (!o0 || !o1) return fail();
-                state.first_out = std::move(*o0.buffer);
-                state.second_out = std::move(*o1.buffer);
+        HipBuffer DecodeStatePoolLayer::*const pools[2] = {&DecodeStatePoolLayer::first,
+                                                           &DecodeStatePoolLayer::second};
+        std::uint64_t DecodeStatePoolLayer::*const strides[2] = {
+            &DecodeStatePoolLayer::first_stride, &DecodeStatePoolLayer::second_stride};
+        for (std::uint32_t b = 0; ok && b < 2; ++b) {
+            auto striped = create_striped_pool_buffer(device, shape.bytes[b], shape.planes * count);
+            ok = striped && striped.buffer->size_bytes() <= kAddressableBytes;
+            if (!ok) break;
+            layer.*pools[b] = std::move(*striped.buffer);
+            layer.*strides[b] = striped.stripe_stride_bytes;
+            for (std::uint32_t slot = 0; ok && slot < count; ++slot) {
+                for (std::uint32_t plane = 0; ok && plane < shape.planes; ++plane) {
+                    const std::uint64_t stripe = std::uint64_t{slot} * shape.planes + plane;
+                    auto window = create_buffer_window(layer.*pools[b], stripe * (layer.*strides[b]),
+                                                       shape.bytes[b]);
+                    ok = static_cast<bool>(window);
+                    if (ok) slots[slot].layers[index].*kPlaneOf[b][plane] = std::move(*window.buffer);
+                }
             }
-            result.slots[slot].layers.push_back(std::move(state));
         }
         pool.layers.push_back(std::move(layer));
     }
+    if (!ok) {
+        result.error = DecodeStepError::BufferAllocationFailed;
+        return result;
+    }
     result.pool = std::move(pool);
+    result.slots = std::move(slots);
     return result;
 }
 
@@ -368,39 +383,35 @@ DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
     return {DecodeStepError::None, std::move(b)};
 }
 
+// Slot predicates (decode_step.cpp:577-618), each the conjunction of the one before and one
+// more condition: compatible (same step, same shape) -> available (idle and Ready) -> ready
+// (every plane the schedule needs is there and large enough).
 bool decode_state_slot_compatible(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
-    return step.capacity != 0 && state.capacity == step.capacity &&
-           state.schedule_identity == step.schedule.data() &&
-           state.layers.size() == step.schedule.size();
+    const bool same_step = state.schedule_identity == step.schedule.data();
+    const bool same_shape =
+        state.capacity == step.capacity && state.layers.size() == step.schedule.size();
+    return step.capacity != 0 && same_step && same_shape;
 }
 
 bool decode_state_slot_complete(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
     if (!decode_state_slot_compatible(step, state)) return false;
-    const auto enough = [](const HipBuffer& buffer, std::uint64_t bytes) {
-        return buffer && buffer.size_bytes() >= bytes;
-    };
-    const DecodeGeometry& g = step.geometry;
-    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
-        const DecodeLayerState& s = state.layers[layer];
-        if (is_gated(step.schedule[layer])) {
-            if (!enough(s.first, g.gdn_conv_state_bytes) ||
-                !enough(s.first_out, g.gdn_conv_state_bytes) ||
-                !enough(s.second, g.gdn_recurrent_state_bytes) ||
-                !enough(s.second_out, g.gdn_recurrent_state_bytes)) {
-                return false;
+    for (std::size_t index = 0; index < step.schedule.size(); ++index) {
+        const LayerFootprint shape = footprint_of(step.geometry, step.schedule[index]);
+        for (std::uint32_t b = 0; b < 2; ++b) {
+            for (std::uint32_t plane = 0; plane < shape.planes; ++plane) {
+                const HipBuffer& buffer = state.layers[index].*kPlaneOf[b][plane];
+                if (!buffer || buffer.size_bytes() < shape.bytes[b]) return false;
             }
-        } else if (!enough(s.first, g.attn_cache_bytes) || !enough(s.second, g.attn_cache_bytes)) {
-            return false;
         }
     }
     return true;
 }
 
 bool decode_state_slot_available(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
+    const bool idle = state.active_transfer_generation == 0 && state.active_reset_generation == 0 &&
+                      state.active_reset_segments == 0 && state.active_reset_bytes == 0;
     return decode_state_slot_compatible(step, state) &&
-           state.status == DecodeStateSlotStatus::Ready && state.active_transfer_generation == 0 &&
-           state.active_reset_generation == 0 && state.active_reset_segments == 0 &&
-           state.active_reset_bytes == 0;
+           state.status == DecodeStateSlotStatus::Ready && idle;
 }
 
 bool decode_state_slot_ready(const DecodeStep& step, const DecodeStateSlot& state) noexcept {
@@ -1523,14 +1534,51 @@ bool store(const HipBuffer& buffer, std::uint64_t offset, const std::byte* sourc
 
 }  // namespace
 
+namespace {
+
+// The body of a record is a sequence of byte runs taken from (or installed into) a lane's
+// buffers, in schedule order: a Gated DeltaNet layer contributes its conv window and its
+// recurrent state whole, an attention layer the first `positions` rows of each kv head of the
+// keys, then of the values - packed, although the caches are capacity-strided
+// (decode_harness.cpp:339-460).  One walker produces the runs; sizing, writing and loading are
+// three visitors of it.
+struct RecordRun {
+    std::size_t layer;
+    std::uint32_t buffer;        // 0: first (conv | keys), 1: second (recurrent | values)
+    std::uint64_t slot_offset;   // byte offset inside the lane's buffer
+    std::uint64_t bytes;
+};
+
+template <typename Visit>   // bool visit(const RecordRun&): false stops the walk
+bool walk_state_record(const DecodeStep& step, std::uint32_t positions, Visit&& visit) {
+    const std::uint64_t packed_head = positions * kRecordHeadRowBytes;
+    const std::uint64_t cache_head = std::uint64_t{step.capacity} * kRecordHeadRowBytes;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        const bool gated = is_gated(step.schedule[layer]);
+        for (std::uint32_t buffer = 0; buffer < 2; ++buffer) {
+            if (gated) {
+                const std::uint64_t whole = buffer == 0 ? step.geometry.gdn_conv_state_bytes
+                                                        : step.geometry.gdn_recurrent_state_bytes;
+                if (!visit(RecordRun{layer, buffer, 0, whole})) return false;
+                continue;
+            }
+            for (std::uint64_t head = 0; head < kRecordKvHeads; ++head) {
+                if (!visit(RecordRun{layer, buffer, head * cache_head, packed_head})) return false;
+            }
+        }
+    }
+    return true;
+}
+
+}  // namespace
+
 std::uint64_t state_record_bytes(const DecodeStep& step, std::uint32_t positions) noexcept {
     if (positions == 0 || positions > step.capacity) return 0;
     std::uint64_t bytes = kStateRecordHeaderBytes;
-    for (const LayerKind kind : step.schedule) {
-        bytes += is_gated(kind)
-                     ? step.geometry.gdn_conv_state_bytes + step.geometry.gdn_recurrent_state_bytes
-                     : 2 * kRecordKvHeads * positions * kRecordHeadRowBytes;
-    }
+    walk_state_record(step, positions, [&bytes](const RecordRun& run) {
+        bytes += run.bytes;
+        return true;
+    });
     return bytes;
 }
 
@@ -1542,36 +1590,19 @@ StateRecordError write_state_record(const DecodeStep& step, const DecodeStateSlo
     record.assign(total, std::byte{0});
     std::memcpy(record.data(), kStateRecordMagic, 8);
     std::memcpy(record.data() + 8, &positions, 4);
-    std::uint64_t cursor = kStateRecordHeaderBytes;
-    const std::uint64_t head_bytes = positions * kRecordHeadRowBytes;
-    const std::uint64_t cache_head_stride = std::uint64_t{step.capacity} * kRecordHeadRowBytes;
-    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
-        const DecodeLayerState& s = state.layers[layer];
-        if (is_gated(step.schedule[layer])) {
-            const bool live_out = gated_delta_live_is_out(s.swapped);
-            const HipBuffer& conv = live_out ? s.first_out : s.first;
-            const HipBuffer& recurrent = live_out ? s.second_out : s.second;
-            if (!fetch(conv, 0, record.data() + cursor, step.geometry.gdn_conv_state_bytes)) {
-                return StateRecordError::TransferFailed;
-            }
-            cursor += step.geometry.gdn_conv_state_bytes;
-            if (!fetch(recurrent, 0, record.data() + cursor,
-                       step.geometry.gdn_recurrent_state_bytes)) {
-                return StateRecordError::TransferFailed;
-            }
-            cursor += step.geometry.gdn_recurrent_state_bytes;
-        } else {
-            for (const HipBuffer* plane : {&s.first, &s.second}) {
-                for (std::uint64_t head = 0; head < kRecordKvHeads; ++head) {
-                    if (!fetch(*plane, head * cache_head_stride, record.data() + cursor, head_bytes)) {
-                        return StateRecordError::TransferFailed;
-                    }
-                    cursor += head_bytes;
-                }
-            }
-        }
-    }
-    return cursor == total ? StateRecordError::None : StateRecordError::TransferFailed;
+    std::byte* cursor = record.data() + kStateRecordHeaderBytes;
+    // a record carries the LIVE plane of each ping-pong pair
+    const bool moved = walk_state_record(step, positions, [&](const RecordRun& run) {
+        const DecodeLayerState& s = state.layers[run.layer];
+        const bool out_plane = is_gated(step.schedule[run.layer]) && gated_delta_live_is_out(s.swapped);
+        const HipBuffer& source = run.buffer == 0 ? (out_plane ? s.first_out : s.first)
+                                                  : (out_plane ? s.second_out : s.second);
+        if (!fetch(source, run.slot_offset, cursor, run.bytes)) return false;
+        cursor += run.bytes;
+        return true;
+    });
+    if (!moved || cursor != record.data() + total) return StateRecordError::TransferFailed;
+    return StateRecordError::None;
 }
 
 StateRecordError load_state_record(std::span<const std::byte> record, const DecodeStep& step,
@@ -1585,32 +1616,20 @@ StateRecordError load_state_record(std::span<const std::byte> record, const Deco
     if (total == 0) return StateRecordError::InvalidPositions;
     if (record.size() < total) return StateRecordError::Truncated;
     if (record.size() > total) return StateRecordError::TrailingBytes;
-    std::uint64_t cursor = kStateRecordHeaderBytes;
-    const std::uint64_t head_bytes = count * kRecordHeadRowBytes;
-    const std::uint64_t cache_head_stride = std::uint64_t{step.capacity} * kRecordHeadRowBytes;
-    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
-        DecodeLayerState& s = state.layers[layer];
-        if (is_gated(step.schedule[layer])) {
-            if (!store(s.first, 0, record.data() + cursor, step.geometry.gdn_conv_state_bytes)) {
-                return StateRecordError::TransferFailed;
-            }
-            cursor += step.geometry.gdn_conv_state_bytes;
-            if (!store(s.second, 0, record.data() + cursor,
-                       step.geometry.gdn_recurrent_state_bytes)) {
-                return StateRecordError::TransferFailed;
-            }
-            cursor += step.geometry.gdn_recurrent_state_bytes;
-            s.swapped = false;  // the installed planes are the ones the next step reads
-        } else {
-            for (const HipBuffer* plane : {&s.first, &s.second}) {
-                for (std::uint64_t head = 0; head < kRecordKvHeads; ++head) {
-                    if (!store(*plane, head * cache_head_stride, record.data() + cursor, head_bytes)) {
-                        return StateRecordError::TransferFailed;
-                    }
-                    cursor += head_bytes;
-                }
-            }
+    // the whole record has been checked against the step before the first byte moves; it is
+    // installed into `first` / `second`, which the cleared phase below makes the live planes
+    const std::byte* cursor = record.data() + kStateRecordHeaderBytes;
+    const bool moved = walk_state_record(step, count, [&](const RecordRun& run) {
+        DecodeLayerState& s = state.layers[run.layer];
+        if (!store(run.buffer == 0 ? s.first : s.second, run.slot_offset, cursor, run.bytes)) {
+            return false;
         }
+        cursor += run.bytes;
+        return true;
+    });
+    if (!moved) return StateRecordError::TransferFailed;
+    for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
+        if (is_gated(step.schedule[layer])) state.layers[layer].swapped = false;
     }
     positions = count;
     return StateRecordError::None;
