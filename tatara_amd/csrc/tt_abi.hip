@@ -138,6 +138,12 @@ struct tt_command_buffer {
     bool pass_open = false;
     const tt_pipeline* pipeline = nullptr;
     Bindings table{};
+    const tt_buffer* bound[tt::kArgSlots] = {};   // the buffer behind each bound slot
+    // Every buffer a recorded command names is kept alive until the recording is reset or
+    // the command buffer destroyed (after its last submission has completed), as the
+    // reference's command buffers retain their resources: a caller may destroy its handle
+    // between encode and commit, or before a later replay.
+    std::vector<tt_buffer*> retained;
     hipEvent_t begin = nullptr;
     hipEvent_t end = nullptr;
     bool committed = false;
@@ -150,6 +156,18 @@ struct tt_command_buffer {
 };
 
 static void drop_graph(tt_command_buffer* cb);
+
+static void retain(tt_command_buffer* cb, const tt_buffer* buffer) {
+    if (buffer == nullptr) return;
+    if (!cb->retained.empty() && cb->retained.back() == buffer) return;   // same as the last one
+    tt_buffer* held = const_cast<tt_buffer*>(buffer);
+    held->refs.fetch_add(1);
+    cb->retained.push_back(held);
+}
+static void release_retained(tt_command_buffer* cb) {
+    for (tt_buffer* buffer : cb->retained) release_buffer(buffer);
+    cb->retained.clear();
+}
 
 extern "C" {
 
@@ -518,6 +536,7 @@ void tt_command_buffer_destroy(tt_command_buffer* cb) {
     if (cb->end != nullptr) (void)hipEventDestroy(cb->end);
     for (hipEvent_t event : cb->marks) (void)hipEventDestroy(event);
     drop_graph(cb);
+    release_retained(cb);
     delete cb;
 }
 
@@ -527,6 +546,7 @@ int32_t tt_pass_begin(tt_command_buffer* cb) {
     cb->pass_open = true;
     cb->pipeline = nullptr;
     std::memset(&cb->table, 0, sizeof(cb->table));
+    std::memset(cb->bound, 0, sizeof(cb->bound));
     return TT_OK;
 }
 
@@ -554,6 +574,7 @@ int32_t tt_pass_set_buffer(tt_command_buffer* cb, const tt_buffer* buffer, uint6
     cb->table.bytes[index] = buffer->size - offset_bytes;
     cb->table.has_buffer |= 1u << index;
     cb->table.clen[index] = 0;
+    cb->bound[index] = buffer;
     return TT_OK;
 }
 
@@ -569,6 +590,7 @@ int32_t tt_pass_set_bytes(tt_command_buffer* cb, const void* bytes, uint32_t len
     cb->table.cval[index] = word;
     cb->table.clen[index] = length_bytes;
     cb->table.has_buffer &= ~(1u << index);
+    cb->bound[index] = nullptr;
     return TT_OK;
 }
 
@@ -590,6 +612,9 @@ int32_t tt_pass_dispatch(tt_command_buffer* cb, uint64_t gx, uint64_t gy, uint64
     const int32_t status = command.launch(command.bindings, command.grid, nullptr, true);
     if (status != TT_OK) return status;
     cb->commands.push_back(command);
+    for (uint32_t index = 0; index < tt::kArgSlots; ++index) {
+        if (cb->table.has_buffer & (1u << index)) retain(cb, cb->bound[index]);
+    }
     return TT_OK;
 }
 
@@ -617,6 +642,8 @@ int32_t tt_blit_copy(tt_command_buffer* cb, const tt_buffer* source, uint64_t so
     command.b = destination->dptr + destination_offset;
     command.length = length;
     cb->commands.push_back(command);
+    retain(cb, source);
+    retain(cb, destination);
     return TT_OK;
 }
 
@@ -636,6 +663,7 @@ int32_t tt_blit_fill(tt_command_buffer* cb, tt_buffer* destination, uint64_t des
     command.length = length;
     command.value = value;
     cb->commands.push_back(command);
+    retain(cb, destination);
     return TT_OK;
 }
 
@@ -795,6 +823,7 @@ int32_t tt_command_buffer_reset(tt_command_buffer* cb) {
     cb->commands.clear();
     cb->marks_valid = false;
     drop_graph(cb);
+    release_retained(cb);
     cb->pass_open = false;
     cb->pipeline = nullptr;
     return TT_OK;

@@ -55,3 +55,30 @@ def test_staging_view_round_trip():
     buf.write(np.full(1 << 15, 9, np.uint16))
     buf.synchronize()
     assert (buf.contents(np.uint16) == 9).all()
+
+
+def test_recording_keeps_its_buffers_alive():
+    """A recording names buffers by device address; it holds a reference on each, so a
+    caller that destroys its handles between encode and commit (or before a later replay
+    of a compiled recording) does not leave the GPU working on freed memory."""
+    B, dev, queue, lib = gpu()
+    L = B.lib()
+    n = 1 << 16
+    data = np.arange(n, dtype=np.uint32)
+    src, mid = dev.buffer_from(data), dev.create_buffer(n * 4)
+    dst = dev.create_buffer(n * 4)
+    cb = queue.create_command_buffer()
+    cb.copy_buffer(src, 0, mid, 0, n * 4)
+    cb.copy_buffer(mid, 0, dst, 0, n * 4)
+    cb._refs.clear()                       # drop the Python wrapper's own references ...
+    for doomed in (src, mid):              # ... and the caller's handles
+        L.tt_buffer_destroy(doomed.handle)
+        doomed.handle = None
+    # other allocations may now land where freed memory would have been
+    noise = [dev.buffer_from(np.full(n, 0xDEAD, np.uint32)) for _ in range(4)]
+    cb.compile()
+    for _ in range(2):
+        dst.write(np.zeros(n, np.uint32))
+        cb.commit().wait()
+        assert np.array_equal(dst.read(np.uint32), data)
+    del noise
