@@ -208,7 +208,10 @@ DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::attn_qk_rope_ms, "attn_qk_rope_ms", error) &&
         resolve(library, p, &P::attention_decode_ms, "attention_decode_ms", error) &&
         resolve(library, p, &P::attention_split_ms, "attention_decode_split_ms", error) &&
-        resolve(library, p, &P::attention_combine_ms, "attention_decode_combine_ms", error);
+        resolve(library, p, &P::attention_combine_ms, "attention_decode_combine_ms", error) &&
+        resolve(library, p, &P::attention_layer_ms, "attention_decode_layer_ms", error) &&
+        resolve(library, p, &P::attention_layer_finish_ms, "attention_decode_layer_finish_ms",
+                error);
     if (!ok) return {error, std::nullopt};
     return {HipPipelineError::None, std::move(p)};
 }
@@ -380,6 +383,15 @@ DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
         !allocate_zeroed(device, table_bytes, b.state_offsets)) {
         return {DecodeStepError::BufferAllocationFailed, std::nullopt};
     }
+    // whole-layer attention: one workgroup per compute unit; 256 B of tickets, 128 KiB of
+    // query heads, then one record of 8 x 258 floats per workgroup and stream boundary
+    b.layer_groups = std::max<std::uint32_t>(device.compute_units(), 1);
+    const std::uint64_t layer_scratch_bytes =
+        256 + 131072 +
+        (std::uint64_t{b.layer_groups} + 2 * rows - 1) * 8 * kAttentionRecordFloats * kF32Bytes;
+    if (!allocate_zeroed(device, layer_scratch_bytes, b.attn_layer_scratch)) {
+        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
+    }
     return {DecodeStepError::None, std::move(b)};
 }
 
@@ -469,7 +481,8 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
     const std::uint32_t rows = static_cast<std::uint32_t>(streams.size());
     if (rows == 0 || rows > batch.rows || rows > kMaximumBatchRows ||
         pool.layers.size() != step.schedule.size() || pool.stripes == 0 || !batch.state_offsets ||
-        weights.size() != step.schedule.size() || batch.split_keys % 32u != 0) {
+        weights.size() != step.schedule.size() || batch.split_keys % 32u != 0 ||
+        (batch.attention_whole_layer && (batch.layer_groups == 0 || !batch.attn_layer_scratch))) {
         return HipCommandError::InvalidStreamGroup;
     }
     for (std::size_t index = 0; index < streams.size(); ++index) {
@@ -583,6 +596,28 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
             walk.buffer(batch.gdn_gated, 0, 3);
             walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 4);
             walk.dispatch(g.gdn_gate_norm.groups, g.gdn_gate_norm.threads, rows);
+        } else if (batch.attention_whole_layer) {
+            for (const bool finishing : {false, true}) {
+                if (finishing) walk.barrier();
+                walk.pipeline(finishing ? k.attention_layer_finish_ms : k.attention_layer_ms);
+                walk.buffer(batch.attn_projection, 0, 0);
+                walk.weight(w.query_norm, 1);
+                walk.weight(w.key_norm, 2);
+                walk.buffer(pool.layers[layer].first, 0, 3);
+                walk.buffer(pool.layers[layer].second, 0, 4);
+                walk.buffer(batch.state_offsets, layer * 256, 5);
+                walk.buffer(batch.attn_layer_scratch, 0, 6);
+                walk.buffer(batch.attn_attended, 0, 7);
+                walk.constant(step.capacity, 8);
+                walk.constant(static_cast<std::uint32_t>(g.attn_projection_bytes / 2), 9);
+                walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 10);
+                walk.constant(finishing ? batch.layer_groups : 0u, 11);
+                if (finishing) {
+                    walk.dispatch(HipSize{16, rows, 1}, HipSize{64, 1, 1});
+                } else {
+                    walk.dispatch(HipSize{batch.layer_groups, rows, 1}, HipSize{256, 1, 1});
+                }
+            }
         } else {
             walk.pipeline(k.attn_qk_rope_ms);
             walk.buffer(batch.attn_projection, 0, 0);

@@ -176,6 +176,7 @@ struct DecodePipelines {
     HipComputePipeline gdn_prepare_ms, gdn_recurrence_ms, gate_norm_ms, gdn_decode_fused_ms;
     HipComputePipeline attn_qk_rope_ms, attention_decode_ms, attention_split_ms,
         attention_combine_ms;
+    HipComputePipeline attention_layer_ms, attention_layer_finish_ms;
 };
 struct DecodePipelinesResult {
     backend::hip::HipPipelineError error;
@@ -199,6 +200,14 @@ struct DecodeBatchScratch {
     // One dispatch per Gated DeltaNet layer (gdn_decode_fused_ms) instead of the
     // reference's prepare / recurrence / gate-norm triple; same results bit for bit.
     bool gdn_fused{true};
+    // The attention layer of a wave as attention_decode_layer_ms +
+    // attention_decode_layer_finish_ms (norm, rotation, append, split-K over keys dealt evenly
+    // to `layer_groups` workgroups, gated combine) instead of rope, split path, combine and
+    // the short-row bucket: no split size to choose, every row through the same two
+    // dispatches.  `attn_layer_scratch` holds its tickets, query heads and records.
+    bool attention_whole_layer{false};
+    std::uint32_t layer_groups{0};
+    HipBuffer attn_layer_scratch;
 };
 
 // Keys per split-K workgroup with which one attention layer of a wave of `rows` lanes

@@ -275,9 +275,13 @@ int main() {
         for (std::uint32_t r = 0; r < kLanes; ++r) {
             streams.push_back({&pooled.slots[stripes[r]], contexts[r], stripes[r]});
         }
+        // first wave: rope, split path, combine and the short-row bucket; second wave: the
+        // whole-layer dispatch and its finishing dispatch - both held to the same checker rows
+        batch.attention_whole_layer = token == 1;
         const int rc = submit.run([&](HipComputePass& pass) {
             return encode_token_batch(step, streams, *pooled.pool, batch, bound, no_hooks, pass);
         });
+        batch.attention_whole_layer = false;
         if (rc != 0) return 20 + rc;
         const auto gated = download<std::uint16_t>(batch.gdn_gated, kLanes * 4096);
         const auto attended = download<std::uint16_t>(batch.attn_attended, kLanes * 4096);
