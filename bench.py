@@ -50,7 +50,6 @@ VISIBLE = 32768
 CAPACITY = 32768
 LAYERS = 40
 PERIOD = 4                      # G,G,G,A
-DEFAULT_SPLIT_KEYS = 1024       # keys per split-K workgroup of the three-dispatch form
 HBM_PEAK_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
 # HBM traffic of one launch of the key-walk kernel at 4 lanes x 32768 keys, from two rocprofv3
@@ -76,6 +75,11 @@ class Wave:
 
     def __init__(self, dev, lib, torch, attention, split_keys, attention_layers, gdn_layers,
                  contexts, capacity, seed=0x7A7A):
+        if not split_keys:
+            # the host's own choice (runtime.cpp choose_split_keys): splits x 2 kv heads x lanes
+            # about one workgroup per compute unit, 128..1024 keys, a multiple of 32
+            per_group = -(-(max(contexts) + 1) * 2 * len(contexts) // dev.compute_units)
+            split_keys = max(128, min(1024, -(-per_group // 32) * 32))
         self.dev, self.lib, self.attention, self.part = dev, lib, attention, split_keys
         self.contexts, self.capacity = list(contexts), capacity
         self.rows = len(contexts)
@@ -221,6 +225,7 @@ def attention_figures(queue, wave):
     algo = wave.visible_keys() * ATTN_BYTES_PER_KEY
     gbs = algo / (walk["median_us"] * 1e-6) / 1e9
     return {"lanes_visible_keys": [c + 1 for c in wave.contexts], "algorithmic_bytes": algo,
+            "split_keys": wave.part if wave.attention == "three" else None,
             "walk_kernel": walk, "walk_kernel_gbs": round(gbs, 1),
             "walk_kernel_frac": round(gbs / HBM_PEAK_GBS, 4),
             "layer_all_dispatches": layer,
@@ -444,8 +449,9 @@ def main():
                     help="skip the 16384-row block prefill figures in detail.prefill_16k")
     ap.add_argument("--no-config3", action="store_true",
                     help="skip the ragged-lane and deep-lane figures in detail.config3")
-    ap.add_argument("--split-keys", type=int, default=DEFAULT_SPLIT_KEYS,
-                    help="keys per split-K workgroup of --attention three (multiple of 32)")
+    ap.add_argument("--split-keys", type=int, default=0,
+                    help="keys per split-K workgroup of --attention three (multiple of 32); 0: what "
+                         "the host runtime picks for the wave (1024 at 4 x 32768, 800 at 1 x 100000)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device-to-device copies first, so a "
                          "counter run has a kernel of known traffic to scale its readings by")
@@ -516,7 +522,7 @@ def main():
                                "own KV / state per layer), one HIP-graph replay per wave",
                    "lanes": LANES, "visible_keys": VISIBLE, "capacity": CAPACITY, "layers": LAYERS,
                    "attention_form": args.attention, "workgroups": wave.groups,
-                   "split_keys": args.split_keys if args.attention == "three" else None,
+                   "split_keys": wave.part if args.attention == "three" else None,
                    "device": dev.name},
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": uniform["walk_kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

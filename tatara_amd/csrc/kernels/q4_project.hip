@@ -208,18 +208,23 @@ int32_t launch_rows(const Q4Projection& p, hipStream_t stream) {
 // out[m][n] = sum_g scale[n][g] * (sum_{k in g} x[m][k] q[n][k]) + bias[n][g] * xs[m][g],
 // xs[m][g] = sum_{k in g} x[m][k].  A workgroup of eight waves owns 128 output rows (n) x
 // 256 input rows (m) and walks K one group (64 columns) at a time through three stages:
-//   * x goes from global memory straight into LDS (no registers), requested two groups
-//     ahead; the nibbles are requested two groups ahead into registers, unpacked to exact
-//     bf16 integers 0..15 and written beside it with the group's 128 scales.  Rows are 128
-//     B without padding; 16-byte piece p of row r sits in slot p ^ (r & 7), which keeps the
-//     16-byte fragment reads of sixteen consecutive rows free of bank conflicts.
-//   * each wave multiplies a 64 x 64 part as 4 x 4 tiles of v_mfma_f32_16x16x32_bf16 (n
-//     along the rows of the result, so a lane ends up with four consecutive n of one m:
-//     8-byte stores), two MFMAs per tile and group from a zero accumulator, then
+//   * x, the nibble words and the groups' scales and biases go from global memory straight
+//     into LDS (no registers), requested two groups ahead.  A nibble becomes the bf16
+//     number 16 + nibble (dropped into mantissa bits 3..6 of 0x4180, three instructions a
+//     pair) and is written beside x.  Rows are 128 B without padding; 16-byte piece p of
+//     row r sits in slot p ^ (r & 7), which keeps the 16-byte fragment reads of sixteen
+//     consecutive rows free of bank conflicts.
+//   * each wave multiplies a 64 x 64 part as 4 x 4 tiles of v_mfma_f32_16x16x32_bf16 with m
+//     along the rows of the result, so a lane holds one n per tile and needs one scale per
+//     tile and group: two MFMAs per tile and group from a zero accumulator, then
 //     acc += scale[n] * partial in fp32.
 //   * xs comes from the same MFMA unit (a ones operand against the x fragments), is split
-//     into bf16 hi + lo and, once every eight groups, multiplied with the eight biases by
-//     one v_mfma_f32_16x16x16_bf16 per tile (slots: 8 x hi, 8 x lo against the biases twice).
+//     into bf16 hi + lo and, once every eight groups, multiplied by one
+//     v_mfma_f32_16x16x16_bf16 per tile with the eight biases (slots: 8 x hi, 8 x lo against
+//     the biases twice) and by a second one with -16 * scale, which takes the nibble offset
+//     back out.
+//   * the result leaves through LDS, so that a row of 64 outputs is stored as 128
+//     contiguous bytes.
 constexpr uint32_t kBlockN = 128;                    // output rows of a workgroup tile
 constexpr uint32_t kBlockM = 256;                    // input rows of a workgroup tile
 constexpr uint32_t kBlockThreads = 512;
@@ -227,32 +232,37 @@ constexpr uint32_t kStages = 3;                      // of what arrives from glo
 constexpr uint32_t kRowBytes = 128;                  // one group of one row: 64 bf16
 constexpr uint32_t kXStageBytes = kBlockM * kRowBytes;                   // 32768
 constexpr uint32_t kWordStageBytes = kBlockN * 32;                       // 8 words per row
-constexpr uint32_t kScaleStageBytes = kBlockN * 4;                       // a pair of groups per row
-constexpr uint32_t kArrivalBytes = kXStageBytes + kWordStageBytes + kScaleStageBytes;  // 37376
+constexpr uint32_t kArrivalBytes = kXStageBytes + kWordStageBytes;       // 36864
 constexpr uint32_t kQStageBytes = kBlockN * kRowBytes;                   // unpacked: 16384, two of them
 constexpr uint32_t kQBase = kStages * kArrivalBytes;
 constexpr uint32_t kGroupSumBase = kQBase + 2 * kQStageBytes;
-constexpr uint32_t kGroupSumBytes = kBlockM * 16 * 2;                    // [m][8 hi, 8 lo] bf16
-constexpr uint32_t kBlockLdsBytes = kGroupSumBase + kGroupSumBytes;      // 153088
-constexpr uint32_t kTransfersPerGroup = 7;           // per wave: 4 x, 2 words, 1 scales
+constexpr uint32_t kGroupSumBytes = 2 * kBlockM * 8 * 2;                 // [window of 4 groups][m][4 hi, 4 lo] bf16
+// scales and biases of a window of eight groups, two windows: [window][scales, biases]
+// [pair of groups][n] dwords (a dword = the bf16 of an even group and of the next)
+constexpr uint32_t kMetaBase = kGroupSumBase + kGroupSumBytes;
+constexpr uint32_t kMetaPairBytes = kBlockN * 4;
+constexpr uint32_t kMetaKindBytes = 4 * kMetaPairBytes;
+constexpr uint32_t kMetaWindowBytes = 2 * kMetaKindBytes;
+constexpr uint32_t kBlockLdsBytes = kMetaBase + 2 * kMetaWindowBytes;    // 159744
+constexpr uint32_t kTransfersPerGroup = 7;           // per wave: 4 x, 2 words, 1 scales or biases
+constexpr uint32_t kOutRowBytes = 144;               // a wave's 64 results of one m on the way out
 static_assert(kBlockLdsBytes <= 160 * 1024, "one workgroup per compute unit");
+static_assert(8 * 64 * kOutRowBytes <= kQBase, "the results leave through the idle stages");
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4_bits;
+constexpr float kNibbleOffset = 16.0f;   // nibbles enter the matrix unit as 16 + nibble
 
-// eight nibbles of `word` -> eight bf16 integers (exact), low nibble first
-__device__ __forceinline__ u32x4 unpack_nibbles(uint32_t word) {
-    const uint32_t even = word & 0x0F0F0F0Fu;         // nibbles 0, 2, 4, 6 in bytes 0..3
-    const uint32_t odd = (word >> 4) & 0x0F0F0F0Fu;   // nibbles 1, 3, 5, 7
+// eight nibbles of `word` -> the eight bf16 numbers 16 + nibble, low nibble first
+__device__ __forceinline__ u32x4 offset_nibbles(uint32_t word) {
+    // byte i of `even` = 0x80 | nibble 2 i << 3, of `odd` the same for nibble 2 i + 1: the
+    // low byte of the bf16 pattern 0x4180 | nibble << 3
+    const uint32_t even = ((word << 3) & 0x78787878u) | 0x80808080u;
+    const uint32_t odd = ((word >> 1) & 0x78787878u) | 0x80808080u;
     u32x4 out;
-    // a small integer is exact in bf16: the upper half of its fp32 pattern
-    out[0] = (__float_as_uint(static_cast<float>(even & 0xFFu)) >> 16) |
-             (__float_as_uint(static_cast<float>(odd & 0xFFu)) & 0xFFFF0000u);
-    out[1] = (__float_as_uint(static_cast<float>((even >> 8) & 0xFFu)) >> 16) |
-             (__float_as_uint(static_cast<float>((odd >> 8) & 0xFFu)) & 0xFFFF0000u);
-    out[2] = (__float_as_uint(static_cast<float>((even >> 16) & 0xFFu)) >> 16) |
-             (__float_as_uint(static_cast<float>((odd >> 16) & 0xFFu)) & 0xFFFF0000u);
-    out[3] = (__float_as_uint(static_cast<float>(even >> 24)) >> 16) |
-             (__float_as_uint(static_cast<float>(odd >> 24)) & 0xFFFF0000u);
+    out[0] = __builtin_amdgcn_perm(odd, even, 0x0C040C00u) | 0x41004100u;
+    out[1] = __builtin_amdgcn_perm(odd, even, 0x0C050C01u) | 0x41004100u;
+    out[2] = __builtin_amdgcn_perm(odd, even, 0x0C060C02u) | 0x41004100u;
+    out[3] = __builtin_amdgcn_perm(odd, even, 0x0C070C03u) | 0x41004100u;
     return out;
 }
 
@@ -260,9 +270,9 @@ __device__ __forceinline__ uint16_t truncate16(float v) {
     return static_cast<uint16_t>(__float_as_uint(v) >> 16);
 }
 
-// Global memory -> LDS without passing through registers: lane l's 16 bytes land at
-// lds_address + 16 l.  Issued as assembly so that the only waits are the ones written
-// below; M0 is used for nothing else in this kernel.
+// Global memory -> LDS without passing through registers: lane l's 16 bytes at base +
+// offset land at lds_address + 16 l.  Issued as assembly so that the only waits are the
+// ones written below; M0 is used for nothing else in this kernel.
 __device__ __forceinline__ void transfer_to_lds(const uint8_t* base, uint32_t offset,
                                                 uint32_t lds_address) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -324,13 +334,13 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
                unused_bias);
         word_source[i] = w_row + (lane & 7);
     }
-    // scales: one dword (an even group and the next) per row; waves of equal parity fetch the
-    // same 64 rows, which keeps every wave's transfer count the same
-    const uint16_t* scale_source;
+    // scales (with an even group) and biases (with the odd one that follows): one dword,
+    // the pair of groups, per row; waves of equal parity fetch the same 64 rows, which keeps
+    // every wave's transfer count the same
+    const uint16_t *scale_source, *bias_source;
     {
         const uint32_t* unused_words;
-        const uint16_t* unused_bias;
-        locate(min(n0 + 64 * (wave & 1) + lane, out_rows - 1), unused_words, scale_source, unused_bias);
+        locate(min(n0 + 64 * (wave & 1) + lane, out_rows - 1), unused_words, scale_source, bias_source);
     }
     const uint32_t q_row = t >> 2, q_quarter = t & 3;
     const uint32_t q_slot0 = q_row * kRowBytes + (((2 * q_quarter) ^ (q_row & 7)) * 16);
@@ -338,28 +348,32 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
 
     auto request = [&](uint32_t group) {
         const uint32_t stage = lds_base + (group % kStages) * kArrivalBytes;
+        const uint8_t* x_group = x_base + group * kRowBytes;   // uniform: scalar arithmetic
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            transfer_to_lds(x_base, x_offset[j] + group * kRowBytes,
-                            stage + (32 * wave + 8 * j) * kRowBytes);
+            transfer_to_lds(x_group, x_offset[j], stage + (32 * wave + 8 * j) * kRowBytes);
         }
 #pragma unroll
         for (uint32_t i = 0; i < 2; ++i) {
             transfer_dword_to_lds(word_source[i] + group * 8,
                                   stage + kXStageBytes + (16 * wave + 8 * i) * 32);
         }
-        transfer_dword_to_lds(scale_source + (group & ~1u),
-                              stage + kXStageBytes + kWordStageBytes + 64 * (wave & 1) * 4);
+        const uint32_t kind = group & 1;
+        transfer_dword_to_lds((kind ? bias_source : scale_source) + (group & ~1u),
+                              lds_base + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
+                                  kind * kMetaKindBytes + ((group >> 1) & 3) * kMetaPairBytes +
+                                  64 * (wave & 1) * 4);
     };
     auto commit = [&](uint32_t group) {
         const uint8_t* arrived = lds + (group % kStages) * kArrivalBytes + kXStageBytes;
         const u32x2 words = *reinterpret_cast<const u32x2*>(arrived + q_row * 32 + q_quarter * 8);
         uint8_t* stage = lds + kQBase + (group & 1) * kQStageBytes;
-        *reinterpret_cast<u32x4*>(stage + q_slot0) = unpack_nibbles(words[0]);
-        *reinterpret_cast<u32x4*>(stage + q_slot1) = unpack_nibbles(words[1]);
+        *reinterpret_cast<u32x4*>(stage + q_slot0) = offset_nibbles(words[0]);
+        *reinterpret_cast<u32x4*>(stage + q_slot1) = offset_nibbles(words[1]);
     };
 
-    // ---- multiply role: wave (mq, nh) owns m in [64 mq, +64), n in [64 nh, +64) of the tile
+    // ---- multiply role: wave (mq, nh) owns m in [64 mq, +64), n in [64 nh, +64) of the tile;
+    // in a 16 x 16 result the lane holds m = 4 g .. 4 g + 3 of column n = i16
     const uint32_t nh = wave & 1, mq = wave >> 1;
     // fragment of (row, 32-column step): piece 4 step + g, stored at slot piece ^ (row & 7)
     const uint32_t piece_offset[2] = {((g ^ (i16 & 7)) * 16), (((4 + g) ^ (i16 & 7)) * 16)};
@@ -377,40 +391,54 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     for (uint32_t e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(1.0f);
     const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto add_bias_terms = [&](uint32_t first_group) {
-        // slots 0..7 pair with hi, 8..15 with lo: lanes g and g + 2 hold the same biases
-        bf16x4_bits biases[4];
+    // sum_g (bias[n][g] - 16 scale[n][g]) xs[m][g] over the four groups that start at
+    // `first_group`: one MFMA per tile with the sixteen slots {hi, lo, hi, lo} of the sums
+    // against {bias, bias, -16 scale, -16 scale}
+    auto add_affine_terms = [&](uint32_t first_group) {
+        const uint32_t* meta = reinterpret_cast<const uint32_t*>(
+            lds + kMetaBase + ((first_group >> 3) & 1) * kMetaWindowBytes +
+            (1 - (g >> 1)) * kMetaKindBytes + ((first_group >> 1) & 3) * kMetaPairBytes);
+        // lanes g = 0, 1 carry the biases (which sit after the scales), g = 2, 3 the scales
+        const float factor = (g >> 1) ? -kNibbleOffset : 1.0f;
+        bf16x4_bits weights[4];
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
-            const uint32_t* unused_words;
-            const uint16_t *unused_scales, *bias_row;
-            locate(min(n0 + 64 * nh + 16 * tn + i16, out_rows - 1), unused_words, unused_scales,
-                   bias_row);
-            biases[tn] = *reinterpret_cast<const bf16x4_bits*>(bias_row + first_group + 4 * (g & 1));
+            const uint32_t row = 64 * nh + 16 * tn + i16;
+            u32x2 bits;
+#pragma unroll
+            for (uint32_t j = 0; j < 2; ++j) {
+                const uint32_t pair = meta[j * kBlockN + row];
+                // times 1 or times -16: exact in bf16
+                const float low = factor * __uint_as_float(pair << 16);
+                const float high = factor * __uint_as_float(pair & 0xFFFF0000u);
+                bits[j] = (__float_as_uint(low) >> 16) | (__float_as_uint(high) & 0xFFFF0000u);
+            }
+            weights[tn] = __builtin_bit_cast(bf16x4_bits, bits);
         }
+        const uint16_t* sums_window = group_sums + ((first_group >> 2) & 1) * (kBlockM * 8);
 #pragma unroll
         for (uint32_t tm = 0; tm < 4; ++tm) {
             const bf16x4_bits sums = *reinterpret_cast<const bf16x4_bits*>(
-                group_sums + (64 * mq + 16 * tm + i16) * 16 + 4 * g);
+                sums_window + (64 * mq + 16 * tm + i16) * 8 + 4 * (g & 1));
 #pragma unroll
             for (uint32_t tn = 0; tn < 4; ++tn) {
-                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(biases[tn], sums,
+                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sums, weights[tn],
                                                                         acc[tn][tm], 0, 0, 0);
             }
         }
     };
 
+    // One barrier per group.  Between the barrier that ends group g - 1 and the one that ends
+    // group g a wave requests group g + 2 (into the stage group g - 1 was read from), multiplies
+    // group g and, in the shadow of the multiply, unpacks the nibbles of group g + 1 into the
+    // other unpacked stage; before the barrier it has waited for its own transfers of group
+    // g + 1, so after the barrier all of x (g + 1) and all unpacked nibbles are in place.
     request(0);
     request(1);   // the group count is a multiple of 8
+    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
+    commit(0);
+    __syncthreads();
     for (uint32_t group = 0; group < groups; ++group) {
-        // this group's transfers have landed once at most the next group's are in flight
-        if (group + 1 < groups) {
-            __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        commit(group);
-        __syncthreads();
         if (group + 2 < groups) request(group + 2);
         const uint8_t* stage = lds + (group % kStages) * kArrivalBytes;
         const uint8_t* q_stage = lds + kQBase + (group & 1) * kQStageBytes;
@@ -425,62 +453,80 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
                     q_stage + q_frag + tile * 16 * kRowBytes + piece_offset[step]);
             }
         }
-        // group sums of two of this wave's four m tiles (the other n half takes the others)
+        // the four groups before this one are complete since the last barrier
+        if ((group & 3) == 0 && group != 0) add_affine_terms(group - 4);
+        const uint32_t* scale_pairs = reinterpret_cast<const uint32_t*>(
+            lds + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
+            ((group >> 1) & 3) * kMetaPairBytes);
+        // bytes {0, 1} (even group) or {2, 3} (odd group) of a pair into the upper half, zeros below
+        const uint32_t pick = (group & 1) ? 0x03020C0Cu : 0x01000C0Cu;
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+            if (tn == 2 && group + 1 < groups) {
+                // the next group's transfers have landed once at most this iteration's are in flight
+                if (group + 2 < groups) {
+                    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
+                } else {
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
+                }
+                commit(group + 1);
+            }
+            const float scale = __uint_as_float(
+                __builtin_amdgcn_perm(0u, scale_pairs[64 * nh + 16 * tn + i16], pick));
+#pragma unroll
+            for (uint32_t tm = 0; tm < 4; ++tm) {
+                f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[tm][0], qf[tn][0], zero, 0, 0, 0);
+                part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[tm][1], qf[tn][1], part, 0, 0, 0);
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) acc[tn][tm][j] = fmaf(scale, part[j], acc[tn][tm][j]);
+            }
+        }
+        // group sums of two of this wave's four m tiles (the other n half takes the others):
+        // every row of the result is the sum; lanes g = 0, 2 store hi, lanes g = 1, 3 lo (the
+        // same value to the same place twice, so that no lane has to be switched off)
+        uint16_t* sum_slot = group_sums + ((group >> 2) & 1) * (kBlockM * 8) + (64 * mq + i16) * 8 +
+                             4 * (g & 1) + (group & 3);
 #pragma unroll
         for (uint32_t tm = 0; tm < 4; ++tm) {
             if ((tm >> 1) != nh) continue;   // wave-uniform; keeps the fragment index static
             f32x4 sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xf[tm][0], zero, 0, 0, 0);
             sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, xf[tm][1], sum, 0, 0, 0);
-            if (g == 0) {
-                const uint16_t hi = truncate16(sum[0]);
-                const uint16_t lo = truncate16(sum[0] - widen(hi));
-                uint16_t* slot = group_sums + (64 * mq + 16 * tm + i16) * 16 + (group & 7);
-                slot[0] = hi;
-                slot[8] = lo;
-            }
+            const float hi = __uint_as_float(__float_as_uint(sum[0]) & 0xFFFF0000u);
+            sum_slot[16 * tm * 8] = truncate16((g & 1) ? sum[0] - hi : hi);
         }
-        const uint32_t* scale_pairs =
-            reinterpret_cast<const uint32_t*>(stage + kXStageBytes + kWordStageBytes);
-        // bytes {0, 1} (even group) or {2, 3} (odd group) of a pair into the upper half, zeros below
-        const uint32_t pick = (group & 1) ? 0x03020C0Cu : 0x01000C0Cu;
-#pragma unroll
-        for (uint32_t tn = 0; tn < 4; ++tn) {
-            const u32x4 pairs = *reinterpret_cast<const u32x4*>(scale_pairs + 64 * nh + 16 * tn + 4 * g);
-            f32x4 scale;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                scale[j] = __uint_as_float(__builtin_amdgcn_perm(0u, pairs[j], pick));
-            }
-#pragma unroll
-            for (uint32_t tm = 0; tm < 4; ++tm) {
-                f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[tn][0], xf[tm][0], zero, 0, 0, 0);
-                part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[tn][1], xf[tm][1], part, 0, 0, 0);
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) acc[tn][tm][j] = fmaf(scale[j], part[j], acc[tn][tm][j]);
-            }
-        }
-        if ((group & 7) == 7) {
-            __syncthreads();   // all eight groups' sums are in place
-            add_bias_terms(group - 7);
-        }
+        __syncthreads();
     }
+    add_affine_terms(groups - 4);
 
-    // ---- store: lane holds n = 4 g .. 4 g + 3 of column m = i16 of every tile
+    // ---- store: through a tile of the wave's own in LDS ([m][n], rows 16 B apart from a
+    // multiple of 128), read back as 16-byte pieces: 128 contiguous bytes per m
+    __syncthreads();   // nobody reads the stages any more (nor the sums, which the tiles do not reach)
+    uint8_t* tile = lds + wave * 64 * kOutRowBytes;
 #pragma unroll
     for (uint32_t tm = 0; tm < 4; ++tm) {
-        const uint32_t m = m0 + 64 * mq + 16 * tm + i16;
-        if (m >= p.rows) continue;
-        uint16_t* out_row = p.output + static_cast<uint64_t>(m) * p.output_stride;
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
-            const uint32_t n = n0 + 64 * nh + 16 * tn + 4 * g;
-            if (n >= out_rows) continue;
-            u32x2 packed;
-            packed[0] = static_cast<uint32_t>(store16(acc[tn][tm][0])) |
-                        (static_cast<uint32_t>(store16(acc[tn][tm][1])) << 16);
-            packed[1] = static_cast<uint32_t>(store16(acc[tn][tm][2])) |
-                        (static_cast<uint32_t>(store16(acc[tn][tm][3])) << 16);
-            *reinterpret_cast<u32x2*>(out_row + n) = packed;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint16_t*>(tile + (16 * tm + 4 * g + j) * kOutRowBytes +
+                                             (16 * tn + i16) * 2) = store16(acc[tn][tm][j]);
+            }
+        }
+    }
+    const bool wide = ((reinterpret_cast<uintptr_t>(p.output) | (p.output_stride * 2)) & 15) == 0;
+#pragma unroll
+    for (uint32_t piece = lane; piece < 64 * 8; piece += 64) {
+        const uint32_t row = piece >> 3, m = m0 + 64 * mq + row;
+        const uint32_t n = n0 + 64 * nh + 8 * (piece & 7);
+        if (m >= p.rows || n >= out_rows) continue;
+        const u32x4 eight = *reinterpret_cast<const u32x4*>(tile + row * kOutRowBytes + (piece & 7) * 16);
+        uint16_t* out = p.output + static_cast<uint64_t>(m) * p.output_stride + n;
+        if (wide && n + 8 <= out_rows) {
+            *reinterpret_cast<u32x4*>(out) = eight;
+        } else {
+            for (uint32_t e = 0; e < 8 && n + e < out_rows; ++e) {
+                out[e] = static_cast<uint16_t>(eight[e >> 1] >> (16 * (e & 1)));
+            }
         }
     }
 }
@@ -525,7 +571,6 @@ __device__ __forceinline__ bf16x4_bits offset_four(uint32_t word) {
     }
     return __builtin_bit_cast(bf16x4_bits, out);
 }
-constexpr float kNibbleOffset = 16.0f;
 
 // bytes between the x rows staged in LDS: 16 more than a row, so that the sixteen lanes of
 // a fragment read (one row each, the same columns) fall on different banks
