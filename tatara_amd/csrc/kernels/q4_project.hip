@@ -300,6 +300,11 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     const uint32_t groups = p.k_size / kQ4Group;
     const uint32_t lds_base = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
+    // multiply role: the waves form two sets of four, the two waves that share a SIMD in
+    // different sets (waves w and w + 4, as a workgroup's waves are dealt to the SIMDs in
+    // turn); wave (mq, nh) owns m in [64 mq, +64), n in [64 nh, +64) of the tile
+    const uint32_t second_set = wave >> 2;
+    const uint32_t nh = wave & 1, mq = 2 * second_set + ((wave >> 1) & 1);
 
     // which weight matrix a global output row lives in
     auto locate = [&](uint32_t n, const uint32_t*& words, const uint16_t*& scales,
@@ -335,12 +340,13 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         word_source[i] = w_row + (lane & 7);
     }
     // scales (with an even group) and biases (with the odd one that follows): one dword,
-    // the pair of groups, per row; waves of equal parity fetch the same 64 rows, which keeps
-    // every wave's transfer count the same
+    // the pair of groups, per row; a wave fetches the 64 rows of its own n half (as do the
+    // three others of that half, which keeps every wave's transfer count the same and makes
+    // its own wait enough before it reads them)
     const uint16_t *scale_source, *bias_source;
     {
         const uint32_t* unused_words;
-        locate(min(n0 + 64 * (wave & 1) + lane, out_rows - 1), unused_words, scale_source, bias_source);
+        locate(min(n0 + 64 * nh + lane, out_rows - 1), unused_words, scale_source, bias_source);
     }
     const uint32_t q_row = t >> 2, q_quarter = t & 3;
     const uint32_t q_slot0 = q_row * kRowBytes + (((2 * q_quarter) ^ (q_row & 7)) * 16);
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         transfer_dword_to_lds((kind ? bias_source : scale_source) + (group & ~1u),
                               lds_base + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
                                   kind * kMetaKindBytes + ((group >> 1) & 3) * kMetaPairBytes +
-                                  64 * (wave & 1) * 4);
+                                  64 * nh * 4);
     };
     auto commit = [&](uint32_t group) {
         const uint8_t* arrived = lds + (group % kStages) * kArrivalBytes + kXStageBytes;
@@ -372,9 +378,7 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         *reinterpret_cast<u32x4*>(stage + q_slot1) = offset_nibbles(words[1]);
     };
 
-    // ---- multiply role: wave (mq, nh) owns m in [64 mq, +64), n in [64 nh, +64) of the tile;
-    // in a 16 x 16 result the lane holds m = 4 g .. 4 g + 3 of column n = i16
-    const uint32_t nh = wave & 1, mq = wave >> 1;
+    // ---- multiply role: in a 16 x 16 result the lane holds m = 4 g .. 4 g + 3 of column n = i16
     // fragment of (row, 32-column step): piece 4 step + g, stored at slot piece ^ (row & 7)
     const uint32_t piece_offset[2] = {((g ^ (i16 & 7)) * 16), (((4 + g) ^ (i16 & 7)) * 16)};
     const uint32_t x_frag = (64 * mq + i16) * kRowBytes;
@@ -394,13 +398,13 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     // sum_g (bias[n][g] - 16 scale[n][g]) xs[m][g] over the four groups that start at
     // `first_group`: one MFMA per tile with the sixteen slots {hi, lo, hi, lo} of the sums
     // against {bias, bias, -16 scale, -16 scale}
-    auto add_affine_terms = [&](uint32_t first_group) {
+    bf16x4_bits affine_weights[4], affine_sums[4];
+    auto read_affine_terms = [&](uint32_t first_group) __attribute__((always_inline)) {
         const uint32_t* meta = reinterpret_cast<const uint32_t*>(
             lds + kMetaBase + ((first_group >> 3) & 1) * kMetaWindowBytes +
             (1 - (g >> 1)) * kMetaKindBytes + ((first_group >> 1) & 3) * kMetaPairBytes);
         // lanes g = 0, 1 carry the biases (which sit after the scales), g = 2, 3 the scales
         const float factor = (g >> 1) ? -kNibbleOffset : 1.0f;
-        bf16x4_bits weights[4];
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
             const uint32_t row = 64 * nh + 16 * tn + i16;
@@ -413,36 +417,45 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
                 const float high = factor * __uint_as_float(pair & 0xFFFF0000u);
                 bits[j] = (__float_as_uint(low) >> 16) | (__float_as_uint(high) & 0xFFFF0000u);
             }
-            weights[tn] = __builtin_bit_cast(bf16x4_bits, bits);
+            affine_weights[tn] = __builtin_bit_cast(bf16x4_bits, bits);
         }
         const uint16_t* sums_window = group_sums + ((first_group >> 2) & 1) * (kBlockM * 8);
 #pragma unroll
         for (uint32_t tm = 0; tm < 4; ++tm) {
-            const bf16x4_bits sums = *reinterpret_cast<const bf16x4_bits*>(
+            affine_sums[tm] = *reinterpret_cast<const bf16x4_bits*>(
                 sums_window + (64 * mq + 16 * tm + i16) * 8 + 4 * (g & 1));
+        }
+    };
+    auto add_affine_terms = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t tm = 0; tm < 4; ++tm) {
 #pragma unroll
             for (uint32_t tn = 0; tn < 4; ++tn) {
-                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sums, weights[tn],
-                                                                        acc[tn][tm], 0, 0, 0);
+                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                    affine_sums[tm], affine_weights[tn], acc[tn][tm], 0, 0, 0);
             }
         }
     };
 
-    // One barrier per group.  Between the barrier that ends group g - 1 and the one that ends
-    // group g a wave requests group g + 2 (into the stage group g - 1 was read from), multiplies
-    // group g and, in the shadow of the multiply, unpacks the nibbles of group g + 1 into the
-    // other unpacked stage; before the barrier it has waited for its own transfers of group
-    // g + 1, so after the barrier all of x (g + 1) and all unpacked nibbles are in place.
-    request(0);
-    request(1);   // the group count is a multiple of 8
-    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
-    commit(0);
-    __syncthreads();
-    for (uint32_t group = 0; group < groups; ++group) {
+    // The two sets alternate: while one multiplies group g from registers (the matrix
+    // unit), the other does everything else of its group - requests the transfers of two
+    // groups ahead, reads its fragments from LDS, unpacks its share of the next group's
+    // nibbles - and a barrier separates the slots.  The second set runs one slot behind the
+    // first.  In the slot of its `fetch (g)` a wave
+    //   * requests group g + 2 into the stage that both sets read in their fetch (g - 1),
+    //   * reads the fragments of group g: x (g) has landed and the nibbles of g are unpacked,
+    //     because every wave waited for its transfers of g and unpacked its share in its
+    //     fetch (g - 1), one or two slots ago,
+    //   * waits for its own transfers of group g + 1 and unpacks its share into the unpacked
+    //     stage that both sets read in their fetch (g - 1).
+    // The group sums are exchanged between the two waves of an m quarter, which belong to
+    // the same set, and a wave reads only the scales and biases that it transferred itself.
+    bf16x8 xf[4][2], qf[4][2];
+    float scale[4];
+    auto fetch = [&](uint32_t group) __attribute__((always_inline)) {
         if (group + 2 < groups) request(group + 2);
         const uint8_t* stage = lds + (group % kStages) * kArrivalBytes;
         const uint8_t* q_stage = lds + kQBase + (group & 1) * kQStageBytes;
-        bf16x8 xf[4][2], qf[4][2];
 #pragma unroll
         for (uint32_t tile = 0; tile < 4; ++tile) {
 #pragma unroll
@@ -453,8 +466,8 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
                     q_stage + q_frag + tile * 16 * kRowBytes + piece_offset[step]);
             }
         }
-        // the four groups before this one are complete since the last barrier
-        if ((group & 3) == 0 && group != 0) add_affine_terms(group - 4);
+        // everything else the multiply reads from LDS, so that the multiply reads nothing:
+        // the group's scales and, every fourth group, the affine terms of the four before
         const uint32_t* scale_pairs = reinterpret_cast<const uint32_t*>(
             lds + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
             ((group >> 1) & 3) * kMetaPairBytes);
@@ -462,24 +475,48 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         const uint32_t pick = (group & 1) ? 0x03020C0Cu : 0x01000C0Cu;
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
-            if (tn == 2 && group + 1 < groups) {
-                // the next group's transfers have landed once at most this iteration's are in flight
-                if (group + 2 < groups) {
-                    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
-                } else {
-                    __builtin_amdgcn_s_waitcnt(0x0F70);
-                }
-                commit(group + 1);
-            }
-            const float scale = __uint_as_float(
+            scale[tn] = __uint_as_float(
                 __builtin_amdgcn_perm(0u, scale_pairs[64 * nh + 16 * tn + i16], pick));
+        }
+        if ((group & 3) == 0 && group != 0) read_affine_terms(group - 4);
+        if (group + 1 < groups) {
+            // the next group's transfers have landed once at most this slot's are in flight
+            if (group + 2 < groups) {
+                __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
+            } else {
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
+            commit(group + 1);
+        }
+    };
+    auto multiply = [&](uint32_t group) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_setprio(1);
+        // the four groups before this one are complete since this set's last multiply
+        if ((group & 3) == 0 && group != 0) add_affine_terms();
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
 #pragma unroll
             for (uint32_t tm = 0; tm < 4; ++tm) {
                 f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[tm][0], qf[tn][0], zero, 0, 0, 0);
                 part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[tm][1], qf[tn][1], part, 0, 0, 0);
 #pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) acc[tn][tm][j] = fmaf(scale, part[j], acc[tn][tm][j]);
+                for (uint32_t j = 0; j < 4; ++j) acc[tn][tm][j] = fmaf(scale[tn], part[j], acc[tn][tm][j]);
             }
+        }
+        // issue order: the scale FMAs of a tile go into the shadow of the MFMAs two tiles on
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+#pragma unroll
+        for (uint32_t tile = 0; tile < 14; ++tile) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        // the FMAs belong to this block: left to itself the compiler sinks all 64 behind the
+        // group sums, where nothing overlaps them
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+#pragma unroll
+            for (uint32_t tm = 0; tm < 4; ++tm) asm volatile("" : "+v"(acc[tn][tm]));
         }
         // group sums of two of this wave's four m tiles (the other n half takes the others):
         // every row of the result is the sum; lanes g = 0, 2 store hi, lanes g = 1, 3 lo (the
@@ -494,9 +531,26 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
             const float hi = __uint_as_float(__float_as_uint(sum[0]) & 0xFFFF0000u);
             sum_slot[16 * tm * 8] = truncate16((g & 1) ? sum[0] - hi : hi);
         }
+        __builtin_amdgcn_s_setprio(0);
+    };
+
+    request(0);
+    request(1);   // the group count is a multiple of 8
+    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
+    commit(0);
+    __syncthreads();
+    // every wave passes 2 * groups + 1 barriers: the second set one before its first slot,
+    // the first set one after its last
+    if (second_set) __syncthreads();
+    for (uint32_t group = 0; group < groups; ++group) {
+        fetch(group);
+        __syncthreads();
+        multiply(group);
         __syncthreads();
     }
-    add_affine_terms(groups - 4);
+    if (!second_set) __syncthreads();
+    read_affine_terms(groups - 4);
+    add_affine_terms();
 
     // ---- store: through a tile of the wave's own in LDS ([m][n], rows 16 B apart from a
     // multiple of 128), read back as 16-byte pieces: 128 contiguous bytes per m
