@@ -207,22 +207,25 @@ int32_t launch_rows(const Q4Projection& p, hipStream_t stream) {
 //
 // out[m][n] = sum_g scale[n][g] * (sum_{k in g} x[m][k] q[n][k]) + bias[n][g] * xs[m][g],
 // xs[m][g] = sum_{k in g} x[m][k].  A workgroup of eight waves owns 128 output rows (n) x
-// 256 input rows (m) and walks K one group (64 columns) at a time through three stages:
-//   * x, the nibble words and the groups' scales and biases go from global memory straight
-//     into LDS (no registers), requested two groups ahead.  A nibble becomes the bf16
-//     number 16 + nibble (dropped into mantissa bits 3..6 of 0x4180, three instructions a
-//     pair) and is written beside x.  Rows are 128 B without padding; 16-byte piece p of
-//     row r sits in slot p ^ (r & 7), which keeps the 16-byte fragment reads of sixteen
-//     consecutive rows free of bank conflicts.
+// 256 input rows (m) and walks K one group (64 columns) at a time:
+//   * x (three stages), the nibble words (a pair of groups per transfer, two stages) and
+//     the scales and biases (a window of eight groups per transfer, two stages) go from
+//     global memory straight into LDS (no registers), x two groups ahead.  A nibble becomes
+//     the bf16 number 16 + nibble (dropped into mantissa bits 3..6 of 0x4180, three
+//     instructions a pair) and is written to one of two unpacked stages.  Rows are 128 B
+//     without padding; 16-byte piece p of row r sits in slot p ^ (r & 7), which keeps the
+//     16-byte fragment reads of sixteen consecutive rows free of bank conflicts.
 //   * each wave multiplies a 64 x 64 part as 4 x 4 tiles of v_mfma_f32_16x16x32_bf16 with m
 //     along the rows of the result, so a lane holds one n per tile and needs one scale per
 //     tile and group: two MFMAs per tile and group from a zero accumulator, then
 //     acc += scale[n] * partial in fp32.
 //   * xs comes from the same MFMA unit (a ones operand against the x fragments), is split
-//     into bf16 hi + lo and, once every eight groups, multiplied by one
-//     v_mfma_f32_16x16x16_bf16 per tile with the eight biases (slots: 8 x hi, 8 x lo against
-//     the biases twice) and by a second one with -16 * scale, which takes the nibble offset
-//     back out.
+//     into bf16 hi + lo and, once every four groups, multiplied by one
+//     v_mfma_f32_16x16x16_bf16 per tile: slots {hi, lo, hi, lo} of four groups against
+//     {bias, bias, -16 scale, -16 scale}, the latter taking the nibble offset back out.
+//   * the eight waves work as two sets of four that alternate between the matrix unit and
+//     everything else of a group, so that the two waves of a SIMD are never in the same
+//     phase (see the schedule before the main loop).
 //   * the result leaves through LDS, so that a row of 64 outputs is stored as 128
 //     contiguous bytes.
 constexpr uint32_t kBlockN = 128;                    // output rows of a workgroup tile
@@ -230,24 +233,23 @@ constexpr uint32_t kBlockM = 256;                    // input rows of a workgrou
 constexpr uint32_t kBlockThreads = 512;
 constexpr uint32_t kStages = 3;                      // of what arrives from global memory
 constexpr uint32_t kRowBytes = 128;                  // one group of one row: 64 bf16
-constexpr uint32_t kXStageBytes = kBlockM * kRowBytes;                   // 32768
-constexpr uint32_t kWordStageBytes = kBlockN * 32;                       // 8 words per row
-constexpr uint32_t kArrivalBytes = kXStageBytes + kWordStageBytes;       // 36864
+constexpr uint32_t kXStageBytes = kBlockM * kRowBytes;                   // 32768, three of them
+// the nibble words of a pair of groups (an even one and the next): [n][16 words], two of them
+constexpr uint32_t kWordBase = kStages * kXStageBytes;
+constexpr uint32_t kWordPairBytes = kBlockN * 64;
 constexpr uint32_t kQStageBytes = kBlockN * kRowBytes;                   // unpacked: 16384, two of them
-constexpr uint32_t kQBase = kStages * kArrivalBytes;
+constexpr uint32_t kQBase = kWordBase + 2 * kWordPairBytes;
 constexpr uint32_t kGroupSumBase = kQBase + 2 * kQStageBytes;
 constexpr uint32_t kGroupSumBytes = 2 * kBlockM * 8 * 2;                 // [window of 4 groups][m][4 hi, 4 lo] bf16
-// scales and biases of a window of eight groups, two windows: [window][scales, biases]
-// [pair of groups][n] dwords (a dword = the bf16 of an even group and of the next)
+// scales and biases of a window of eight groups, two windows: [window][scales, biases][n]
+// [8 bf16]
 constexpr uint32_t kMetaBase = kGroupSumBase + kGroupSumBytes;
-constexpr uint32_t kMetaPairBytes = kBlockN * 4;
-constexpr uint32_t kMetaKindBytes = 4 * kMetaPairBytes;
+constexpr uint32_t kMetaKindBytes = kBlockN * 16;
 constexpr uint32_t kMetaWindowBytes = 2 * kMetaKindBytes;
-constexpr uint32_t kBlockLdsBytes = kMetaBase + 2 * kMetaWindowBytes;    // 159744
-constexpr uint32_t kTransfersPerGroup = 7;           // per wave: 4 x, 2 words, 1 scales or biases
+constexpr uint32_t kBlockLdsBytes = kMetaBase + 2 * kMetaWindowBytes;    // 163840
 constexpr uint32_t kOutRowBytes = 144;               // a wave's 64 results of one m on the way out
 static_assert(kBlockLdsBytes <= 160 * 1024, "one workgroup per compute unit");
-static_assert(8 * 64 * kOutRowBytes <= kQBase, "the results leave through the idle stages");
+static_assert(8 * 64 * kOutRowBytes <= kWordBase, "the results leave through the idle x stages");
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4_bits;
 constexpr float kNibbleOffset = 16.0f;   // nibbles enter the matrix unit as 16 + nibble
@@ -278,6 +280,14 @@ __device__ __forceinline__ void transfer_to_lds(const uint8_t* base, uint32_t of
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(offset), "s"(base)
+                 : "memory");
+}
+
+// the same at an address of the lane's own
+__device__ __forceinline__ void transfer_piece_to_lds(const void* address, uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(address)
                  : "memory");
 }
 
@@ -327,52 +337,57 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         const uint32_t row = min(m0 + 32 * wave + 8 * j + (lane >> 3), p.rows - 1);
         x_offset[j] = static_cast<uint32_t>(row * p.input_stride * 2) + (((lane & 7) ^ (lane >> 3)) * 16);
     }
-    // words: transfer i of wave w fills rows 16 w + 8 i .. + 7, eight words each; the same
-    // wave unpacks them (thread t: words 2 (t & 3), 2 (t & 3) + 1 of row t >> 2), so its own
-    // wait covers them
-    const uint32_t* word_source[2];
-#pragma unroll
-    for (uint32_t i = 0; i < 2; ++i) {
-        const uint32_t* w_row;
+    // words: one transfer of wave w per pair of groups fills rows 16 w .. 16 w + 15 with the
+    // sixteen words of the pair (lane l: piece l & 3 of row l >> 2); the same wave unpacks
+    // them (lane l: words 2 (l & 3), 2 (l & 3) + 1 of a group of row l >> 2), so its own wait
+    // covers them
+    const uint32_t* word_source;
+    {
         const uint16_t *unused_scales, *unused_bias;
-        locate(min(n0 + 16 * wave + 8 * i + (lane >> 3), out_rows - 1), w_row, unused_scales,
-               unused_bias);
-        word_source[i] = w_row + (lane & 7);
+        locate(min(n0 + 16 * wave + (lane >> 2), out_rows - 1), word_source, unused_scales, unused_bias);
+        word_source += 4 * (lane & 3);
     }
-    // scales (with an even group) and biases (with the odd one that follows): one dword,
-    // the pair of groups, per row; a wave fetches the 64 rows of its own n half (as do the
-    // three others of that half, which keeps every wave's transfer count the same and makes
-    // its own wait enough before it reads them)
+    // scales and biases: one 4-byte transfer each per window of eight groups and wave, for a
+    // quarter of the rows of the wave's n half (lane l: groups 2 (l & 3), 2 (l & 3) + 1 of
+    // the window, row l >> 2 of the quarter); the other quarters come from the other three
+    // waves of the half, and two barriers pass between a window's arrival and its first use
     const uint16_t *scale_source, *bias_source;
     {
         const uint32_t* unused_words;
-        locate(min(n0 + 64 * nh + lane, out_rows - 1), unused_words, scale_source, bias_source);
+        locate(min(n0 + 64 * nh + 16 * (wave >> 1) + (lane >> 2), out_rows - 1), unused_words,
+               scale_source, bias_source);
+        scale_source += 2 * (lane & 3);
+        bias_source += 2 * (lane & 3);
     }
     const uint32_t q_row = t >> 2, q_quarter = t & 3;
     const uint32_t q_slot0 = q_row * kRowBytes + (((2 * q_quarter) ^ (q_row & 7)) * 16);
     const uint32_t q_slot1 = q_row * kRowBytes + (((2 * q_quarter + 1) ^ (q_row & 7)) * 16);
 
     auto request = [&](uint32_t group) {
-        const uint32_t stage = lds_base + (group % kStages) * kArrivalBytes;
+        const uint32_t stage = lds_base + (group % kStages) * kXStageBytes;
         const uint8_t* x_group = x_base + group * kRowBytes;   // uniform: scalar arithmetic
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
             transfer_to_lds(x_group, x_offset[j], stage + (32 * wave + 8 * j) * kRowBytes);
         }
-#pragma unroll
-        for (uint32_t i = 0; i < 2; ++i) {
-            transfer_dword_to_lds(word_source[i] + group * 8,
-                                  stage + kXStageBytes + (16 * wave + 8 * i) * 32);
+        if ((group & 1) == 0) {
+            transfer_piece_to_lds(word_source + group * 8,
+                                  lds_base + kWordBase + ((group >> 1) & 1) * kWordPairBytes +
+                                      16 * wave * 64);
         }
-        const uint32_t kind = group & 1;
-        transfer_dword_to_lds((kind ? bias_source : scale_source) + (group & ~1u),
-                              lds_base + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
-                                  kind * kMetaKindBytes + ((group >> 1) & 3) * kMetaPairBytes +
-                                  64 * nh * 4);
+        if ((group & 7) == 0) {
+            const uint32_t window = lds_base + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
+                                    (64 * nh + 16 * (wave >> 1)) * 16;
+            transfer_dword_to_lds(scale_source + group, window);
+            transfer_dword_to_lds(bias_source + group, window + kMetaKindBytes);
+        }
     };
-    auto commit = [&](uint32_t group) {
-        const uint8_t* arrived = lds + (group % kStages) * kArrivalBytes + kXStageBytes;
-        const u32x2 words = *reinterpret_cast<const u32x2*>(arrived + q_row * 32 + q_quarter * 8);
+    // the nibble words of `group` that this lane unpacks
+    auto read_words = [&](uint32_t group) {
+        return *reinterpret_cast<const u32x2*>(lds + kWordBase + ((group >> 1) & 1) * kWordPairBytes +
+                                               q_row * 64 + (group & 1) * 32 + q_quarter * 8);
+    };
+    auto commit = [&](uint32_t group, u32x2 words) {
         uint8_t* stage = lds + kQBase + (group & 1) * kQStageBytes;
         *reinterpret_cast<u32x4*>(stage + q_slot0) = offset_nibbles(words[0]);
         *reinterpret_cast<u32x4*>(stage + q_slot1) = offset_nibbles(words[1]);
@@ -400,18 +415,18 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     // against {bias, bias, -16 scale, -16 scale}
     bf16x4_bits affine_weights[4], affine_sums[4];
     auto read_affine_terms = [&](uint32_t first_group) __attribute__((always_inline)) {
-        const uint32_t* meta = reinterpret_cast<const uint32_t*>(
-            lds + kMetaBase + ((first_group >> 3) & 1) * kMetaWindowBytes +
-            (1 - (g >> 1)) * kMetaKindBytes + ((first_group >> 1) & 3) * kMetaPairBytes);
+        const uint8_t* meta = lds + kMetaBase + ((first_group >> 3) & 1) * kMetaWindowBytes +
+                              (1 - (g >> 1)) * kMetaKindBytes + (first_group & 4) * 2;
         // lanes g = 0, 1 carry the biases (which sit after the scales), g = 2, 3 the scales
         const float factor = (g >> 1) ? -kNibbleOffset : 1.0f;
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
             const uint32_t row = 64 * nh + 16 * tn + i16;
+            const u32x2 pairs = *reinterpret_cast<const u32x2*>(meta + row * 16);
             u32x2 bits;
 #pragma unroll
             for (uint32_t j = 0; j < 2; ++j) {
-                const uint32_t pair = meta[j * kBlockN + row];
+                const uint32_t pair = pairs[j];
                 // times 1 or times -16: exact in bf16
                 const float low = factor * __uint_as_float(pair << 16);
                 const float high = factor * __uint_as_float(pair & 0xFFFF0000u);
@@ -442,19 +457,23 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     // groups ahead, reads its fragments from LDS, unpacks its share of the next group's
     // nibbles - and a barrier separates the slots.  The second set runs one slot behind the
     // first.  In the slot of its `fetch (g)` a wave
-    //   * requests group g + 2 into the stage that both sets read in their fetch (g - 1),
+    //   * waits for the transfers it requested in its fetch (g - 1): group g + 1,
     //   * reads the fragments of group g: x (g) has landed and the nibbles of g are unpacked,
     //     because every wave waited for its transfers of g and unpacked its share in its
     //     fetch (g - 1), one or two slots ago,
-    //   * waits for its own transfers of group g + 1 and unpacks its share into the unpacked
-    //     stage that both sets read in their fetch (g - 1).
+    //   * requests group g + 2 into the x stage that both sets read in their fetch (g - 1),
+    //   * unpacks its share of the nibbles of group g + 1 into the unpacked stage that both
+    //     sets read in their fetch (g - 1).
     // The group sums are exchanged between the two waves of an m quarter, which belong to
-    // the same set, and a wave reads only the scales and biases that it transferred itself.
+    // the same set; a window of scales and biases arrives two barriers before its first use.
     bf16x8 xf[4][2], qf[4][2];
     float scale[4];
     auto fetch = [&](uint32_t group) __attribute__((always_inline)) {
-        if (group + 2 < groups) request(group + 2);
-        const uint8_t* stage = lds + (group % kStages) * kArrivalBytes;
+        // the transfers this wave requested in its last fetch (group g + 1) have landed
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        u32x2 words;
+        if (group + 1 < groups) words = read_words(group + 1);   // first, to have them first
+        const uint8_t* stage = lds + (group % kStages) * kXStageBytes;
         const uint8_t* q_stage = lds + kQBase + (group & 1) * kQStageBytes;
 #pragma unroll
         for (uint32_t tile = 0; tile < 4; ++tile) {
@@ -468,26 +487,20 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         }
         // everything else the multiply reads from LDS, so that the multiply reads nothing:
         // the group's scales and, every fourth group, the affine terms of the four before
-        const uint32_t* scale_pairs = reinterpret_cast<const uint32_t*>(
-            lds + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
-            ((group >> 1) & 3) * kMetaPairBytes);
+        const uint8_t* scale_pairs = lds + kMetaBase + ((group >> 3) & 1) * kMetaWindowBytes +
+                                     ((group >> 1) & 3) * 4;
         // bytes {0, 1} (even group) or {2, 3} (odd group) of a pair into the upper half, zeros below
         const uint32_t pick = (group & 1) ? 0x03020C0Cu : 0x01000C0Cu;
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
-            scale[tn] = __uint_as_float(
-                __builtin_amdgcn_perm(0u, scale_pairs[64 * nh + 16 * tn + i16], pick));
+            scale[tn] = __uint_as_float(__builtin_amdgcn_perm(
+                0u, *reinterpret_cast<const uint32_t*>(scale_pairs + (64 * nh + 16 * tn + i16) * 16), pick));
         }
         if ((group & 3) == 0 && group != 0) read_affine_terms(group - 4);
-        if (group + 1 < groups) {
-            // the next group's transfers have landed once at most this slot's are in flight
-            if (group + 2 < groups) {
-                __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
-            } else {
-                __builtin_amdgcn_s_waitcnt(0x0F70);
-            }
-            commit(group + 1);
-        }
+        // the transfers overlap the reads above; they go into the x stage that both sets read
+        // in their fetch (g - 1)
+        if (group + 2 < groups) request(group + 2);
+        if (group + 1 < groups) commit(group + 1, words);
     };
     auto multiply = [&](uint32_t group) __attribute__((always_inline)) {
         __builtin_amdgcn_s_setprio(1);
@@ -536,8 +549,8 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
 
     request(0);
     request(1);   // the group count is a multiple of 8
-    __builtin_amdgcn_s_waitcnt(0x0F70 | kTransfersPerGroup);
-    commit(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    commit(0, read_words(0));
     __syncthreads();
     // every wave passes 2 * groups + 1 barriers: the second set one before its first slot,
     // the first set one after its last
@@ -587,6 +600,16 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
 
 int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
     const uint32_t out_rows = p.first_row[p.segments];
+    // the transfers move 16-byte pieces of x and of the nibble words and 4-byte pairs of
+    // scales and biases
+    uintptr_t wide = reinterpret_cast<uintptr_t>(p.input), narrow = 0;
+    for (uint32_t s = 0; s < p.segments; ++s) {
+        wide |= reinterpret_cast<uintptr_t>(p.words[s]);
+        narrow |= reinterpret_cast<uintptr_t>(p.scales[s]) | reinterpret_cast<uintptr_t>(p.biases[s]);
+    }
+    if ((wide & 15) != 0 || (narrow & 3) != 0 || ((p.input_stride * 2) & 15) != 0) {
+        return TT_CMD_INVALID_BUFFER_OFFSET;
+    }
     hipLaunchKernelGGL(q4_block_kernel,
                        dim3((out_rows + kBlockN - 1) / kBlockN, (p.rows + kBlockM - 1) / kBlockM),
                        dim3(kBlockThreads), kBlockLdsBytes, stream, p);
