@@ -81,6 +81,9 @@ class Wave:
             per_group = -(-(max(contexts) + 1) * 2 * len(contexts) // dev.compute_units)
             split_keys = max(128, min(1024, -(-per_group // 32) * 32))
         self.dev, self.lib, self.attention, self.part = dev, lib, attention, split_keys
+        # as the host runtime records it: waves of one or two lanes deal a lane's 32-key blocks
+        # to its workgroups in turn
+        self.interleave = 1 if len(contexts) <= 2 else 0
         self.contexts, self.capacity = list(contexts), capacity
         self.rows = len(contexts)
         self.groups = dev.compute_units
@@ -173,7 +176,8 @@ class Wave:
             cb.barrier()
         cb.encode(P("attention_decode_split_ms"),
                   {0: self.b_q, 1: layer["keys"], 2: layer["values"], 3: self.attn_table,
-                   4: self.b_part}, {5: cap, 6: 4096, 7: self.part, 8: self.max_splits, 9: 0},
+                   4: self.b_part}, {5: cap, 6: 4096, 7: self.part, 8: self.max_splits,
+                   9: 2 * self.interleave},
                   (self.max_splits, 2, rows), (256,))
         if not walk_only:
             cb.barrier()

@@ -286,6 +286,7 @@ struct FlashArgs {
     uint32_t long_rows_only;    // 1: rows with a single partition are skipped
     uint32_t single_partition;  // keys of one reference partition (256)
     uint32_t row_limit;         // rows the q / gate / out / table operands hold
+    uint32_t interleave;        // 1: a row's workgroups take its 32-key blocks in turn
 };
 
 // value of lane (l ^ 8) within each row of 16 lanes
@@ -322,9 +323,17 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     const uint32_t n = context + 1;
     if (a.long_rows_only && n <= a.single_partition) return;
     const uint32_t part = a.final_mode ? n : a.part;
-    const uint32_t k0 = split * part;
-    if (k0 >= n) return;
-    const uint32_t k1 = min(n, k0 + part);
+    if (split * part >= n) return;
+    // The workgroup's blocks of 32 keys: block b of its own is block first_block + b *
+    // block_stride of the row.  Contiguous: the keys [split * part, + part).  Interleaved: the
+    // row's ceil(n / part) workgroups take the row's blocks in turn, so that at any moment
+    // they read one contiguous window of the cache and all get the same number of blocks.
+    const uint32_t row_blocks = (n + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t row_splits = (n + part - 1) / part;
+    const bool interleave = a.interleave != 0 && a.final_mode == 0;
+    const uint32_t first_block = interleave ? split : split * (part / kBlockKeys);
+    const uint32_t block_stride = interleave ? row_splits : 1;
+    const uint32_t key_end = interleave ? n : min(n, split * part + part);
 
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t lane = threadIdx.x & 63;
@@ -351,15 +360,17 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     float m_run = -INFINITY;
     float l_run = 0.0f;
 
-    const uint32_t nblocks = (k1 - k0 + kBlockKeys - 1) / kBlockKeys;
+    const uint32_t nblocks =
+        interleave ? (row_blocks - split + row_splits - 1) / row_splits
+                   : (key_end - first_block * kBlockKeys + kBlockKeys - 1) / kBlockKeys;
 
     // K rows go from HBM straight into the wave's LDS stage (no registers): one
     // instruction lands 1 KiB contiguous in LDS, lanes 0..31 fetching key i
     // (tile 0) and lanes 32..63 key 16+i (tile 1), so the two rows sharing LDS
     // banks are never read by the same operand load.
     auto stage_keys = [&](uint32_t blk) {
-        const uint32_t key0 = k0 + blk * kBlockKeys;
-        const uint32_t valid = min(kBlockKeys, k1 - key0);
+        const uint32_t key0 = (first_block + blk * block_stride) * kBlockKeys;
+        const uint32_t valid = min(kBlockKeys, key_end - key0);
 #pragma unroll
         for (uint32_t i = 0; i < 16; ++i) {
             const uint32_t key = min(i + (lane >> 5) * 16, valid - 1);
@@ -374,8 +385,8 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // V rows: contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3);
     // one call fetches one 128-dim half (8 x 16 B per lane)
     auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
-        const uint32_t key0 = k0 + blk * kBlockKeys;
-        const uint32_t valid = min(kBlockKeys, k1 - key0);
+        const uint32_t key0 = (first_block + blk * block_stride) * kBlockKeys;
+        const uint32_t valid = min(kBlockKeys, key_end - key0);
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) {
             const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
@@ -395,7 +406,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
         load_values(vreg[1], wave, 1);
     }
     for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
-        const uint32_t valid = min(kBlockKeys, k1 - (k0 + blk * kBlockKeys));
+        const uint32_t valid = min(kBlockKeys, key_end - (first_block + blk * block_stride) * kBlockKeys);
         const bool more = blk + kWaves < nblocks;
         // every transfer issued so far (this block's K and V) has landed
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1722,8 +1733,9 @@ int32_t op_attention_combine(const Bindings& b, const Grid& g, hipStream_t strea
 // a lane batch into one split-K grid): b0 q slab, b1 keys_pool, b2 values_pool,
 // b3 state_table, b4 partials [rows][16][max_splits][258], c5 capacity,
 // c6 query stride, c7 part (keys per workgroup, multiple of 32), c8 max_splits,
-// c9 long_rows_only (1: rows whose context fits one 256-key partition are left
-// to attention_decode_ms); grid (max_splits, 2, rows) x 256.
+// c9 bit 0 long_rows_only (1: rows whose context fits one 256-key partition are left
+// to attention_decode_ms), bit 1 interleave (1: a row's workgroups take its blocks of
+// 32 keys in turn instead of `part` consecutive keys each); grid (max_splits, 2, rows) x 256.
 int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stream,
                               bool validate_only) {
     Args a(b);
@@ -1732,7 +1744,8 @@ int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stre
     f.query_stride = a.constant(6);
     f.part = a.constant(7);
     f.record_splits = a.constant(8);
-    f.long_rows_only = a.constant(9);
+    f.long_rows_only = a.constant(9) & 1;
+    f.interleave = (a.constant(9) >> 1) & 1;
     f.single_partition = kAttnPartition;
     const uint32_t rows = static_cast<uint32_t>(g.gz);
     a.require(f.capacity != 0 && f.query_stride >= kAttnQueryValues && f.part != 0 &&

@@ -186,9 +186,10 @@ def test_decode_context_edges(ctx):
         check_bf16(b_o2.read(np.uint16), want, f"split part {part} ctx {ctx}")
 
 
-def _lane_batch(contexts, cap, part, seed, replays=0):
+def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False):
     """Lane-batched decode over a striped pool with a state table, long rows
     through attention_decode_split_ms and short rows through attention_decode_ms.
+    interleave: a lane's workgroups take its 32-key blocks in turn (bit 1 of c9).
     replays > 0: the recording is also compiled into a HIP graph and replayed that
     many times with the outputs and records cleared in between; every replay must
     reproduce the eager bits."""
@@ -229,7 +230,8 @@ def _lane_batch(contexts, cap, part, seed, replays=0):
     def rec(cb):
         cb.encode(lib.pipeline("attention_decode_split_ms"),
                   {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
-                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1}, (max_splits, 2, rows), (256,))
+                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1 + 2 * int(interleave)},
+                  (max_splits, 2, rows), (256,))
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
                   {0: b_part, 1: b_g, 2: b_tab, 3: b_o},
@@ -257,6 +259,18 @@ def _lane_batch(contexts, cap, part, seed, replays=0):
 def test_lane_batch_small_ragged():
     print("[case] lane batch ragged small", flush=True)
     _lane_batch([2000, 1499, 700, 100, 255, 256, 0], 2048, 128, 0xBEEF)
+
+
+@pytest.mark.parametrize("contexts,cap,part", [
+    ([2000, 1499, 700, 100, 255, 256, 0, 287, 288, 319], 2048, 128),   # blocks not a multiple of the splits
+    ([5000, 4999, 31], 5120, 1024),                                    # a partial last block, one split short
+    ([99999], 100000, 800),                                            # the single deep lane of config 3
+], ids=["ragged-128", "partial-1024", "lane100k-800"])
+def test_lane_batch_interleaved_blocks(contexts, cap, part):
+    """The same rows with a lane's workgroups taking its blocks of 32 keys in turn: the
+    records cover interleaved key sets, the combined output is held to the same bar."""
+    print(f"[case] lane batch interleaved {contexts} part {part}", flush=True)
+    _lane_batch(contexts, cap, part, 0x1E7E, replays=2, interleave=True)
 
 
 def test_config3_four_ragged_lanes_at_depth():
