@@ -22,6 +22,7 @@
 //    applied in fp32 - the same mathematics in another summation order.
 #include "../tt_internal.h"
 #include "lane_sums.h"
+#include "rms_row.h"
 
 namespace tt {
 namespace {
@@ -64,6 +65,10 @@ struct Q4Projection {
     uint64_t input_stride, output_stride;
     uint32_t rows;                         // input rows in this dispatch
     uint32_t row_tile;                     // input rows one workgroup carries (<= 16)
+    // the decode-wave kernel only:
+    const uint16_t* norm_weight;           // not null: the input rows go through the RMS norm first
+    const uint16_t* residual;              // not null: output = bf16(residual + bf16(projection)),
+    uint64_t residual_stride;              //   [rows][residual_stride]; may be the output itself
 };
 
 // grid (ceil(out_rows / 8), ceil(rows / row_tile)) x 256: half wave h of a workgroup
@@ -654,7 +659,7 @@ __device__ __forceinline__ bf16x4_bits offset_four(uint32_t word) {
 template <uint32_t kWaves>
 constexpr uint32_t kWaveRowBytes = kWaves * 1024 + 16;
 
-template <uint32_t kWaves>   // k_size / 512
+template <uint32_t kWaves, bool kNorm = false, bool kResidual = false>   // kWaves = k_size / 512
 __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
     // [rows][kWaveRowBytes] of x, then the waves' partial results
     extern __shared__ __align__(16) uint8_t wave_lds[];
@@ -676,29 +681,82 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
     // read back from LDS as fragments; each lane loading its own 32 bytes per group from
     // global memory cost as much as streaming the weights.
     float* partial = reinterpret_cast<float*>(wave_lds + p.rows * kWaveRowBytes<kWaves>);
-    for (uint32_t piece = threadIdx.x; piece < p.rows * kPiecesPerRow; piece += 4 * kThreads) {
-        u32x4 staged[4];
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
-            staged[j] = *reinterpret_cast<const u32x4*>(
-                p.input + static_cast<uint64_t>(at / kPiecesPerRow) * p.input_stride +
-                (at % kPiecesPerRow) * 8);
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
-            *reinterpret_cast<u32x4*>(wave_lds + (at / kPiecesPerRow) * kWaveRowBytes<kWaves> +
-                                      (at % kPiecesPerRow) * 16) = staged[j];
-        }
-    }
     u32x2 q[8];
+    u32x4 scale_bits, bias_bits;
+    auto request_weights = [&]() {
 #pragma unroll
-    for (uint32_t group = 0; group < 8; ++group) {
-        q[group] = *reinterpret_cast<const u32x2*>(words + group * 8);
+        for (uint32_t group = 0; group < 8; ++group) {
+            q[group] = *reinterpret_cast<const u32x2*>(words + group * 8);
+        }
+        scale_bits = *reinterpret_cast<const u32x4*>(scales);
+        bias_bits = *reinterpret_cast<const u32x4*>(biases);
+    };
+    if constexpr (kNorm) {
+        // The rows go through the RMS norm on their way into LDS, bit for bit as the norm
+        // operator does it with one thread per four values: a thread here holds eight
+        // values of a row, the slices of that operator's threads 2 t and 2 t + 1, whose
+        // sum is the first step of its 32-lane tree; the other four steps run over the 16
+        // lanes of a row of this wave, and the sixteen sums of a row of x meet in the same
+        // zero-padded 32-slot tree.
+        static_assert(kWaves == 4, "one 16-byte piece of a 2048-wide row per thread");
+        float* stage = partial;   // [rows][16], before the partial results need the space
+        u32x4 raw[kQ4BatchRowsMax];
+#pragma unroll
+        for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
+            if (r < p.rows) {
+                raw[r] = *reinterpret_cast<const u32x4*>(
+                    p.input + static_cast<uint64_t>(r) * p.input_stride + threadIdx.x * 8);
+            }
+        }
+        const u32x4 weight = *reinterpret_cast<const u32x4*>(p.norm_weight + threadIdx.x * 8);
+        request_weights();   // in flight while the rows are normed
+#pragma unroll
+        for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
+            if (r < p.rows) {
+                const float slices = rms_slice_squares(raw[r][0], raw[r][1]) +
+                                     rms_slice_squares(raw[r][2], raw[r][3]);
+                const float sixteen = row_sum(slices);
+                if ((threadIdx.x & 15) == 0) stage[r * 16 + (threadIdx.x >> 4)] = sixteen;
+            }
+        }
+        __syncthreads();
+        float inverse[kQ4BatchRowsMax];
+#pragma unroll
+        for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
+            if (r < p.rows) {
+                const float slot = (lane & 31) < 16 ? stage[r * 16 + (lane & 15)] : 0.0f;
+                inverse[r] = rms_inverse(half_wave_sum(slot), kWaves * kQ4Block);
+            }
+        }
+        __syncthreads();   // the stage is read before the partial results overwrite it
+#pragma unroll
+        for (uint32_t r = 0; r < kQ4BatchRowsMax; ++r) {
+            if (r < p.rows) {
+                u32x4 normed;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) normed[j] = rms_scale_pair(raw[r][j], weight[j], inverse[r]);
+                *reinterpret_cast<u32x4*>(wave_lds + r * kWaveRowBytes<kWaves> + threadIdx.x * 16) = normed;
+            }
+        }
+    } else {
+        for (uint32_t piece = threadIdx.x; piece < p.rows * kPiecesPerRow; piece += 4 * kThreads) {
+            u32x4 staged[4];
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
+                staged[j] = *reinterpret_cast<const u32x4*>(
+                    p.input + static_cast<uint64_t>(at / kPiecesPerRow) * p.input_stride +
+                    (at % kPiecesPerRow) * 8);
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const uint32_t at = min(piece + j * kThreads, p.rows * kPiecesPerRow - 1);
+                *reinterpret_cast<u32x4*>(wave_lds + (at / kPiecesPerRow) * kWaveRowBytes<kWaves> +
+                                          (at % kPiecesPerRow) * 16) = staged[j];
+            }
+        }
+        request_weights();
     }
-    const u32x4 scale_bits = *reinterpret_cast<const u32x4*>(scales);
-    const u32x4 bias_bits = *reinterpret_cast<const u32x4*>(biases);
     __syncthreads();
 
     const uint8_t* x_row = wave_lds + min(i16, p.rows - 1) * kWaveRowBytes<kWaves> +
@@ -737,7 +795,15 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
 #pragma unroll
         for (uint32_t w = 1; w < kWaves; ++w) total += partial[(w * 4 + i) * 64 + lane];
         const uint32_t m = 4 * g + i;   // the result has the input rows along its rows
-        if (m < p.rows) p.output[static_cast<uint64_t>(m) * p.output_stride + n] = store16(total);
+        if (m < p.rows) {
+            uint16_t result = store16(total);
+            if constexpr (kResidual) {
+                // the residual sum of the step that follows (moe.metal:1-46), on the rounded projection
+                const uint16_t before = p.residual[static_cast<uint64_t>(m) * p.residual_stride + n];
+                result = rms_store16(rms_widen(rms_fz16(before)) + rms_widen(rms_fz16(result)));
+            }
+            p.output[static_cast<uint64_t>(m) * p.output_stride + n] = result;
+        }
     }
 }
 
@@ -750,12 +816,24 @@ int32_t launch_wave(const Q4Projection& p, hipStream_t stream) {
     const uint32_t out_rows = p.first_row[p.segments];
     switch (p.k_size / kQ4Block) {
     case 4:
-        hipLaunchKernelGGL(q4_wave_kernel<4>, dim3(out_rows / 16), dim3(256),
-                           wave_lds_bytes<4>(p.rows), stream, p);
+        if (p.residual != nullptr) return TT_CMD_INVALID_DISPATCH_EXTENT;
+        if (p.norm_weight != nullptr) {
+            hipLaunchKernelGGL((q4_wave_kernel<4, true, false>), dim3(out_rows / 16), dim3(256),
+                               wave_lds_bytes<4>(p.rows), stream, p);
+        } else {
+            hipLaunchKernelGGL((q4_wave_kernel<4>), dim3(out_rows / 16), dim3(256),
+                               wave_lds_bytes<4>(p.rows), stream, p);
+        }
         break;
     case 8:
-        hipLaunchKernelGGL(q4_wave_kernel<8>, dim3(out_rows / 16), dim3(512),
-                           wave_lds_bytes<8>(p.rows), stream, p);
+        if (p.norm_weight != nullptr) return TT_CMD_INVALID_DISPATCH_EXTENT;
+        if (p.residual != nullptr) {
+            hipLaunchKernelGGL((q4_wave_kernel<8, false, true>), dim3(out_rows / 16), dim3(512),
+                               wave_lds_bytes<8>(p.rows), stream, p);
+        } else {
+            hipLaunchKernelGGL((q4_wave_kernel<8>), dim3(out_rows / 16), dim3(512),
+                               wave_lds_bytes<8>(p.rows), stream, p);
+        }
         break;
     default: return TT_CMD_INVALID_DISPATCH_EXTENT;
     }
@@ -852,8 +930,11 @@ int32_t project_single(const Bindings& b, const Grid& g, hipStream_t stream, boo
 
 // rows of a decode wave: c[out+1] rows (1..16), then the output row stride where the
 // operator has one, then the row tile; grid (groups, ceil(rows / tile)) x threads
+enum class WaveExtra { None, NormedInput, ResidualOutput };
+
 int32_t project_tiled(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only,
-                      const Family& f, bool strided_output, bool wave_kernel = false) {
+                      const Family& f, bool strided_output, bool wave_kernel = false,
+                      WaveExtra extra = WaveExtra::None) {
     Args a(b);
     Q4Projection p{};
     p.rows = a.constant(f.out_slot + 1);
@@ -862,6 +943,16 @@ int32_t project_tiled(const Bindings& b, const Grid& g, hipStream_t stream, bool
     a.require(p.rows >= 1 && p.rows <= kMaxBatchRows && p.row_tile >= 1 &&
                   p.row_tile <= kQ4BatchRowsMax,
               TT_CMD_INVALID_DISPATCH_EXTENT);
+    // the buffer after the operator's last constant: the norm weight of the input rows, or
+    // the rows the projection is added to (same row stride as the output)
+    const uint32_t extra_slot = f.out_slot + (strided_output ? 4 : 3);
+    if (extra == WaveExtra::NormedInput) {
+        p.norm_weight = a.buffer<const uint16_t>(extra_slot, static_cast<uint64_t>(f.k_size) * 2);
+    } else if (extra == WaveExtra::ResidualOutput && a.status == TT_OK) {
+        p.residual_stride = p.output_stride;
+        p.residual = a.buffer<const uint16_t>(
+            extra_slot, (static_cast<uint64_t>(p.rows - 1) * p.residual_stride + f.out_rows()) * 2);
+    }
     if (a.status != TT_OK) return a.status;
     return finish(a, g, stream, validate_only, f, p, f.k_size,
                   (p.rows + p.row_tile - 1) / p.row_tile, wave_kernel);
@@ -932,6 +1023,22 @@ int32_t op_gdn_project_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, 
 int32_t op_gdn_outproj_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
     return project_tiled(b, g, s, v, kOutProject, true, true);
 }
+// attn_project_rms_mfma_ms, gdn_project_rms_mfma_ms (no reference counterpart): the _mfma_ms
+// forms on rows that have not been normed yet, + b13 / b16 the norm weight [2048]: every
+// workgroup norms the rows while it stages them (rms_only_ms's bits), which takes the norm
+// dispatch out of a decode layer.
+int32_t op_attn_project_rms_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kAttnProject, false, true, WaveExtra::NormedInput);
+}
+int32_t op_gdn_project_rms_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kGdnProject, false, true, WaveExtra::NormedInput);
+}
+// gdn_outproj_residual_mfma_ms (no reference counterpart): gdn_outproj_mfma_ms + b8 the rows
+// the projection is added to, [rows][c6]: output = bf16(residual + bf16(projection)), the sum
+// residual_rms would form next (moe.metal:1-46); the output may be the residual buffer itself.
+int32_t op_gdn_outproj_residual_mfma_ms(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
+    return project_tiled(b, g, s, v, kOutProject, true, true, WaveExtra::ResidualOutput);
+}
 // outproj_blk: + c5 block rows, c6 input width (prefill_step.cpp:2063-2078).
 int32_t op_outproj_blk(const Bindings& b, const Grid& g, hipStream_t s, bool v) {
     return project_block(b, g, s, v, kOutProject, true);
@@ -955,6 +1062,12 @@ bool prepare_q4_kernels() {
                                wave_lds_bytes<4>(kQ4BatchRowsMax)) == hipSuccess &&
            hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<8>),
                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                               wave_lds_bytes<8>(kQ4BatchRowsMax)) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<4, true, false>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               wave_lds_bytes<4>(kQ4BatchRowsMax)) == hipSuccess &&
+           hipFuncSetAttribute(reinterpret_cast<const void*>(q4_wave_kernel<8, false, true>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
                                wave_lds_bytes<8>(kQ4BatchRowsMax)) == hipSuccess;
 }
 
@@ -974,6 +1087,9 @@ const KernelDesc kQ4ProjectKernels[] = {
     {"attn_project_mfma_ms", op_attn_project_mfma_ms},
     {"gdn_project_mfma_ms", op_gdn_project_mfma_ms},
     {"gdn_outproj_mfma_ms", op_gdn_outproj_mfma_ms},
+    {"attn_project_rms_mfma_ms", op_attn_project_rms_mfma_ms},
+    {"gdn_project_rms_mfma_ms", op_gdn_project_rms_mfma_ms},
+    {"gdn_outproj_residual_mfma_ms", op_gdn_outproj_residual_mfma_ms},
 };
 const uint32_t kQ4ProjectKernelCount = sizeof(kQ4ProjectKernels) / sizeof(kQ4ProjectKernels[0]);
 #endif

@@ -13,6 +13,7 @@
 //       4-bit weights (q4_dot.metal); here the weights are plain bf16.
 #include "../tt_internal.h"
 #include "lane_sums.h"
+#include "rms_row.h"
 
 namespace tt {
 namespace {
@@ -69,13 +70,7 @@ __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, c
         *reinterpret_cast<u32x2*>(residual_out + static_cast<uint64_t>(blockIdx.y) * residual_stride +
                                   4 * t) = raw;
     }
-    const float x0 = __uint_as_float(raw.x << 16), x1 = __uint_as_float(raw.x & 0xFFFF0000u);
-    const float x2 = __uint_as_float(raw.y << 16), x3 = __uint_as_float(raw.y & 0xFFFF0000u);
-    float sum = 0.0f;
-    sum += x0 * x0;
-    sum += x1 * x1;
-    sum += x2 * x2;
-    sum += x3 * x3;
+    float sum = rms_slice_squares(raw.x, raw.y);
     sum = half_wave_sum(sum);
     if (t < 32) stage[t] = 0.0f;
     __syncthreads();
@@ -84,22 +79,13 @@ __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, c
     if (t < 32) {
         float total = stage[t];
         total = half_wave_sum(total);
-        if (t == 0) inverse_norm = 1.0f / sqrtf(total / static_cast<float>(hidden) + kRmsNormEpsilon);
+        if (t == 0) inverse_norm = rms_inverse(total, hidden);
     }
     __syncthreads();
     const float inverse = inverse_norm;
     const u32x2 wraw = *reinterpret_cast<const u32x2*>(weight + 4 * t);
-    const float xs[4] = {x0, x1, x2, x3};
-    const uint16_t ws[4] = {static_cast<uint16_t>(wraw.x), static_cast<uint16_t>(wraw.x >> 16),
-                            static_cast<uint16_t>(wraw.y), static_cast<uint16_t>(wraw.y >> 16)};
-    uint16_t r[4];
-#pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) {
-        const uint16_t scaled = store16(xs[i] * inverse);
-        r[i] = store16(widen(fz16(ws[i])) * widen(scaled));
-    }
     *reinterpret_cast<u32x2*>(out + 4 * t) =
-        u32x2{r[0] | (static_cast<uint32_t>(r[1]) << 16), r[2] | (static_cast<uint32_t>(r[3]) << 16)};
+        u32x2{rms_scale_pair(raw.x, wraw.x, inverse), rms_scale_pair(raw.y, wraw.y, inverse)};
 }
 
 // out[r][n] = bf16(sum_k x[r][k] w[n][k]).  grid (ceil(N/64), ceil(rows/16)) x 256:

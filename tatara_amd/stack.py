@@ -99,14 +99,19 @@ class StubStack:
     state and the scratch, and records token waves and prefill blocks."""
 
     def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
-                 split_keys=None, attention_form="three"):
+                 split_keys=None, attention_form="three", fused_wave_steps=False):
         """attention_form: "three" records a token wave's attention layer as rope, split-K
         and combine dispatches (split_keys keys per workgroup); "layer" as the whole-layer
         dispatch plus its finishing dispatch (keys dealt evenly to one workgroup per compute
-        unit, whatever the lanes' depths)."""
+        unit, whatever the lanes' depths).
+        fused_wave_steps: decode waves of several lanes over 4-bit weights take the norm in
+        the prologue of the input projection and the residual sum in the epilogue of the
+        output projection (same bits, one dispatch less per layer; measured slower, because
+        every workgroup of the projection norms the rows again)."""
         assert attention_form in ("three", "layer")
         self.dev, self.lib = dev, lib
         self.attention_form = attention_form
+        self.fused_wave_steps = fused_wave_steps
         self.groups = dev.compute_units
         self.lanes, self.capacity, self.vocab = lanes, capacity, vocab
         self.block_rows = block_rows
@@ -177,15 +182,23 @@ class StubStack:
                   ((n + 63) // 64, (rows + 15) // 16), (256,))
         cb.barrier()
 
+    def _fused_wave(self, layer, rows):
+        """Decode waves of several lanes over 4-bit weights take the norm in the prologue of
+        the input projection and the residual sum in the epilogue of the output projection:
+        two dispatches of a layer instead of three outside the attention family."""
+        return self.fused_wave_steps and "in_q4" in layer and "out_q4" in layer and rows >= 2
+
     def _project_in(self, cb, layer, rows, block):
-        """normed -> proj: the layer's input projection (a decode wave or a block)."""
+        """normed -> proj: the layer's input projection (a decode wave or a block); with
+        _fused_wave x -> proj through the layer's input norm."""
         gated = layer["kind"] == "G"
         width = GDN_PROJ if gated else ATTN_PROJ
         if "in_q4" not in layer:
             self._dense(cb, self.normed, layer["w_in"], self.proj, rows, HIDDEN, width)
             return
         name = "gdn_project" if gated else "attn_project"
-        bindings = {0: self.normed}
+        fused = not block and self._fused_wave(layer, rows)
+        bindings = {0: self.x if fused else self.normed}
         for index, matrix in enumerate(layer["in_q4"]):
             for part in range(3):
                 bindings[1 + 3 * index + part] = matrix[part]
@@ -196,7 +209,9 @@ class StubStack:
                       ((width + 3) // 4,), (128,))
         else:
             # several lanes: the matrix-unit form; one lane: the reference's own order
-            suffix = "_mfma_ms" if rows >= 2 else "_ms"
+            suffix = "_rms_mfma_ms" if fused else "_mfma_ms" if rows >= 2 else "_ms"
+            if fused:
+                bindings[out + 3] = layer["input_norm"]
             cb.encode(self.lib.pipeline(name + suffix), bindings, {out + 1: rows, out + 2: 16},
                       ((width + 3) // 4, 1), (128,))
         cb.barrier()
@@ -211,6 +226,11 @@ class StubStack:
         if block:
             cb.encode(self.lib.pipeline("outproj_blk"), bindings, {5: rows, 6: 4096},
                       (HIDDEN // 2,), (64,))
+        elif self._fused_wave(layer, rows):
+            # x = bf16(x + bf16(projection)) in place
+            cb.encode(self.lib.pipeline("gdn_outproj_residual_mfma_ms"),
+                      {**bindings, 4: self.x, 8: self.x}, {5: rows, 6: HIDDEN, 7: 16},
+                      (HIDDEN // 2, 1), (64,))
         else:
             name = "gdn_outproj_mfma_ms" if rows >= 2 else "gdn_outproj_ms"
             cb.encode(self.lib.pipeline(name), bindings, {5: rows, 6: HIDDEN, 7: 16},
@@ -241,7 +261,8 @@ class StubStack:
         """Records one decode step of all lanes; the lanes' inputs are rows of self.x.
         Call advance_token_wave() after the recording has been committed."""
         P, rows = self.lib.pipeline, self.lanes
-        self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
+        if not self._fused_wave(self.layers[0], rows):
+            self._rms(cb, self.x, self.layers[0]["input_norm"], self.normed, rows)
         for index, layer in enumerate(self.layers):
             self._project_in(cb, layer, rows, block=False)
             if layer["kind"] == "G":
@@ -275,7 +296,12 @@ class StubStack:
                           {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
             cb.barrier()
             self._project_out(cb, layer, rows, block=False)
-            self._residual_and_norm(cb, rows, index)
+            if not self._fused_wave(layer, rows):
+                self._residual_and_norm(cb, rows, index)
+            elif index + 1 == len(self.layers):
+                self._rms(cb, self.x, self.final_norm, self.normed, rows)   # for the head
+            elif not self._fused_wave(self.layers[index + 1], rows):
+                self._rms(cb, self.x, self.layers[index + 1]["input_norm"], self.normed, rows)
         if with_head:
             self._head(cb, rows)
 

@@ -148,6 +148,76 @@ def test_block_projection(family, name, rows):
     print(f"[time] {name} rows={rows}: {ms * 1e3:.1f} us", flush=True)
 
 
+@pytest.mark.parametrize("rows", [2, 4, 13, 16])
+@pytest.mark.parametrize("family", [ATTN, GDN], ids=lambda f: f["name"])
+def test_wave_projection_with_the_norm_in_its_prologue(family, rows):
+    """`*_project_rms_mfma_ms` (no reference counterpart) on rows that have not been normed
+    against `rms_only_ms` followed by `*_project_mfma_ms`: the same bits, and the norm the
+    fused form applies is the checker's."""
+    name = family["name"]
+    print(f"[case] {name}_rms_mfma_ms rows={rows}", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9A00)
+    x = ol.gaussian_bf16(0x9B00 + rows, rows * 2048, 0.0, 1.5)
+    weight = ol.gaussian_bf16(0x9C00, 2048, 1.0, 0.25)
+    total = sum(family["segments"])
+    b_x, b_w = dev.buffer_from(x), dev.buffer_from(weight)
+    b_normed = dev.create_buffer(rows * 2048 * 2)
+    two_step = dev.buffer_from(np.full(rows * total, 0x7FC0, np.uint16))
+    fused = dev.buffer_from(np.full(rows * total, 0x7FC0, np.uint16))
+    out, slot = family["out"], family["out"] + 1
+    grid = (_groups(family), 1, 1)
+
+    def rec(cb):
+        cb.encode(lib.pipeline("rms_only_ms"), {0: b_x, 1: b_w, 2: b_normed}, {3: 2048, 4: 2048},
+                  (1, rows), (512,))
+        cb.barrier()
+        cb.encode(lib.pipeline(name + "_mfma_ms"), {**bindings, 0: b_normed, out: two_step},
+                  {slot: rows, slot + 1: 16}, grid, (family["threads"], 1, 1))
+        cb.encode(lib.pipeline(name + "_rms_mfma_ms"), {**bindings, 0: b_x, out: fused, out + 3: b_w},
+                  {slot: rows, slot + 1: 16}, grid, (family["threads"], 1, 1))
+    run(rec)
+    normed = np.zeros(rows * 2048, np.uint16)
+    o.tto_rms_only(x, weight, rows, 2048, normed)
+    assert np.array_equal(b_normed.read(np.uint16), normed)
+    assert np.array_equal(fused.read(np.uint16), two_step.read(np.uint16))
+    check_bf16(fused.read(np.uint16), _expected(family, host, normed, rows), name + "_rms_mfma_ms", ulps=2)
+
+
+@pytest.mark.parametrize("in_place", [False, True], ids=["apart", "in-place"])
+@pytest.mark.parametrize("rows", [2, 4, 16])
+def test_wave_out_projection_with_the_residual_in_its_epilogue(rows, in_place):
+    """`gdn_outproj_residual_mfma_ms` (no reference counterpart) against `gdn_outproj_mfma_ms`
+    followed by the residual sum of `residual_rms_ms`: the same bits, with the output in a
+    buffer of its own and in the residual buffer itself."""
+    print(f"[case] gdn_outproj_residual_mfma_ms rows={rows} in_place={in_place}", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, OUT, 0x9D00)
+    mixed = ol.gaussian_bf16(0x9E00 + rows, rows * 4096, 0.0, 1.0)
+    x = ol.gaussian_bf16(0x9F00 + rows, rows * 2048, 0.0, 1.0)
+    weight = ol.gaussian_bf16(0xA000, 2048, 1.0, 0.25)
+    b_mixed, b_x, b_w = dev.buffer_from(mixed), dev.buffer_from(x), dev.buffer_from(weight)
+    b_delta = dev.create_buffer(rows * 2048 * 2)
+    b_sum, b_normed = dev.create_buffer(rows * 2048 * 2), dev.create_buffer(rows * 2048 * 2)
+    b_fused = dev.buffer_from(x) if in_place else dev.create_buffer(rows * 2048 * 2)
+    b_before = b_fused if in_place else b_x
+
+    def rec(cb):
+        cb.encode(lib.pipeline("gdn_outproj_mfma_ms"), {**bindings, 0: b_mixed, 4: b_delta},
+                  {5: rows, 6: 2048, 7: 16}, (1024, 1, 1), (64, 1, 1))
+        cb.barrier()
+        cb.encode(lib.pipeline("residual_rms_ms"), {0: b_x, 1: b_delta, 2: b_sum, 3: b_w, 4: b_normed},
+                  {5: 2048, 6: 2048, 7: 2048}, (1, rows), (512,))
+        cb.encode(lib.pipeline("gdn_outproj_residual_mfma_ms"),
+                  {**bindings, 0: b_mixed, 4: b_fused, 8: b_before}, {5: rows, 6: 2048, 7: 16},
+                  (1024, 1, 1), (64, 1, 1))
+    run(rec)
+    assert np.array_equal(b_fused.read(np.uint16), b_sum.read(np.uint16))
+    delta = ol.bf16_to_f32(b_delta.read(np.uint16))
+    want = ol.f32_to_bf16(ol.bf16_to_f32(x) + delta)
+    assert np.array_equal(b_fused.read(np.uint16), want)
+
+
 def test_projection_validation():
     B, dev, queue, lib = gpu()
     host, bindings = _family(dev, ATTN, 0x9600)

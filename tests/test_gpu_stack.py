@@ -115,10 +115,12 @@ def _compare(step, got, want):
         assert margin <= 2 * step16, step
 
 
-@pytest.mark.parametrize("layers,quantized", [(40, False), (12, True)], ids=["dense40", "q4x12"])
-def test_stacked_prefill_and_greedy_decode_match_the_checker(layers, quantized):
+@pytest.mark.parametrize("layers,quantized,fused", [(40, False, False), (12, True, False), (12, True, True)],
+                         ids=["dense40", "q4x12", "q4x12-fused-steps"])
+def test_stacked_prefill_and_greedy_decode_match_the_checker(layers, quantized, fused):
     """quantized: the projections are the affine 4-bit operators (block forms in the
-    prefill, wave forms in the decode)."""
+    prefill, wave forms in the decode); fused: the decode waves take the norm in the
+    prologue of the input projection and the residual sum in the output projection."""
     print(f"[case] {layers}-layer stub stack (quantized={quantized}): prefill 2 lanes + 3 greedy "
           "decode waves", flush=True)
     from tatara_amd import stack as S
@@ -126,7 +128,8 @@ def test_stacked_prefill_and_greedy_decode_match_the_checker(layers, quantized):
     vocab, capacity, lanes = 4096, 128, 2
     weights = S.make_weights(layers, vocab, 0x57AC, quantized=quantized)
     embed = weights["embed"].reshape(vocab, 2048)
-    gpu_stack = S.StubStack(dev, lib, weights, lanes, capacity, vocab, block_rows=64, split_keys=64)
+    gpu_stack = S.StubStack(dev, lib, weights, lanes, capacity, vocab, block_rows=64, split_keys=64,
+                            fused_wave_steps=fused)
     cpu_lanes = [OracleLane(weights, capacity, vocab) for _ in range(lanes)]
     rng = np.random.default_rng(5)
     prompts = [rng.integers(0, vocab, 24), rng.integers(0, vocab, 9)]
