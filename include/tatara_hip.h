@@ -50,6 +50,7 @@ typedef struct tt_buffer tt_buffer;
 typedef struct tt_library tt_library;
 typedef struct tt_pipeline tt_pipeline;
 typedef struct tt_command_buffer tt_command_buffer;
+typedef struct tt_event tt_event;
 
 /* Status codes.  0 is success in every family.  Command errors keep the
  * numbering of MetalCommandError (commands.h:232-262); resource errors are
@@ -85,6 +86,7 @@ typedef enum tt_status {
     TT_RES_INVALID_DEVICE = 101,
     TT_RES_SYSTEM_DEVICE_UNAVAILABLE = 102,
     TT_RES_COMMAND_QUEUE_CREATION_FAILED = 103,
+    TT_RES_EVENT_CREATION_FAILED = 104,
     TT_RES_INVALID_BUFFER_SIZE = 105,
     TT_RES_BUFFER_CREATION_FAILED = 106,
     TT_RES_OWNERSHIP_FAILURE = 107,
@@ -141,6 +143,10 @@ int32_t tt_queue_create(tt_device* device, tt_queue** out);
 void tt_queue_destroy(tt_queue* queue);
 /* The HIP stream (hipStream_t) behind a queue, for event timing by the caller. */
 void* tt_queue_native_stream(tt_queue* queue);
+/* create_event (resources.h:240): a counter that command buffers of any queue of the
+ * device signal and wait for (tt_encode_signal_event / tt_encode_wait_for_event). */
+int32_t tt_event_create(tt_device* device, tt_event** out);
+void tt_event_destroy(tt_event* event);
 
 /* create_shared_buffer (resources.h:241) with the zeroed-allocation rule of
  * decode_step.cpp:49-57 built in: the HBM allocation is zero-filled. */
@@ -210,6 +216,17 @@ int32_t tt_blit_copy(tt_command_buffer* command_buffer, const tt_buffer* source,
                      uint64_t length);
 int32_t tt_blit_fill(tt_command_buffer* command_buffer, tt_buffer* destination,
                      uint64_t destination_offset, uint64_t length, uint8_t value);
+/* encode_signal_event / encode_wait_for_event (commands.h:421-426), recorded on the command
+ * buffer outside a pass.  A signal marks `value` reached once everything recorded before
+ * it has completed; a wait holds everything recorded after it until the event has reached
+ * `value` (a signal of `value` or more).  value 0 is TT_CMD_INVALID_EVENT_VALUE.  The
+ * signal that a wait depends on must have been committed before the waiting command
+ * buffer is committed (commits in dependency order, as the reference's lane queues do);
+ * otherwise the commit fails and tt_wait reports it.  A command buffer with event
+ * commands cannot be compiled into a graph. */
+int32_t tt_encode_signal_event(tt_command_buffer* command_buffer, tt_event* event, uint64_t value);
+int32_t tt_encode_wait_for_event(tt_command_buffer* command_buffer, tt_event* event,
+                                 uint64_t value);
 /* Number of commands recorded so far. */
 uint32_t tt_command_count(const tt_command_buffer* command_buffer);
 /* commit (commands.h:500): launches every recorded command on the queue's

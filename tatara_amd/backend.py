@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = [
     "tt_blit_copy", "tt_blit_fill", "tt_command_count", "tt_commit", "tt_wait",
     "tt_command_buffer_reset", "tt_command_buffer_compile", "tt_command_buffer_set_profiling",
     "tt_command_name", "tt_command_gpu_ms", "tt_attention_decode_lanes_static",
+    "tt_event_create", "tt_event_destroy", "tt_encode_signal_event", "tt_encode_wait_for_event",
 ]
 
 
@@ -101,6 +102,9 @@ def lib():
         "tt_command_name": (C.c_char_p, [vp, u32]),
         "tt_command_gpu_ms": (i32, [vp, u32, C.POINTER(C.c_double)]),
         "tt_attention_decode_lanes_static": (i32, [vp] + [vp, u64] * 6 + [u32] * 4),
+        "tt_event_create": (i32, [vp, pvp]), "tt_event_destroy": (None, [vp]),
+        "tt_encode_signal_event": (i32, [vp, vp, u64]),
+        "tt_encode_wait_for_event": (i32, [vp, vp, u64]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -169,6 +173,21 @@ class Device:
 
     def create_library(self):
         return Library(self)
+
+    def create_event(self):
+        return Event(self)
+
+
+class Event:
+    """create_event: a counter that command buffers of any queue signal and wait for."""
+
+    def __init__(self, device):
+        h = C.c_void_p()
+        _check(lib().tt_event_create(device.handle, C.byref(h)), "create_event")
+        self.handle, self.device = h, device
+
+    def __del__(self, _release=_release):
+        _release(self, "tt_event_destroy")
 
 
 class CommandQueue:
@@ -357,6 +376,19 @@ class CommandBuffer:
         _check(lib().tt_blit_copy(self.handle, source.handle, source_offset, destination.handle,
                                   destination_offset, length), "copy_buffer")
         self._refs += [source, destination]
+
+    def signal_event(self, event, value):
+        """encode_signal_event: `value` is reached once everything recorded so far completes."""
+        handle = event.handle if event is not None else None
+        _check(lib().tt_encode_signal_event(self.handle, handle, value), "encode_signal_event")
+        self._refs.append(event)
+
+    def wait_for_event(self, event, value):
+        """encode_wait_for_event: what is recorded after this waits for the event to reach
+        `value`; the signal must be committed before this command buffer is."""
+        handle = event.handle if event is not None else None
+        _check(lib().tt_encode_wait_for_event(self.handle, handle, value), "encode_wait_for_event")
+        self._refs.append(event)
 
     def fill_buffer(self, destination, offset, length, value):
         _check(lib().tt_blit_fill(self.handle, destination.handle, offset, length, value),

@@ -38,6 +38,8 @@ enum class HipCommandError : std::uint8_t {
     None = TT_OK,
     InvalidCommandQueue = TT_CMD_INVALID_COMMAND_QUEUE,
     InvalidCommandBuffer = TT_CMD_INVALID_COMMAND_BUFFER,
+    InvalidEvent = TT_CMD_INVALID_EVENT,
+    InvalidEventValue = TT_CMD_INVALID_EVENT_VALUE,
     InvalidComputePass = TT_CMD_INVALID_COMPUTE_PASS,
     InvalidBlitPass = TT_CMD_INVALID_BLIT_PASS,
     InvalidPipeline = TT_CMD_INVALID_PIPELINE,
@@ -64,6 +66,7 @@ enum class HipResourceError : std::uint8_t {
     InvalidDevice = TT_RES_INVALID_DEVICE,
     SystemDeviceUnavailable = TT_RES_SYSTEM_DEVICE_UNAVAILABLE,
     CommandQueueCreationFailed = TT_RES_COMMAND_QUEUE_CREATION_FAILED,
+    EventCreationFailed = TT_RES_EVENT_CREATION_FAILED,
     InvalidBufferSize = TT_RES_INVALID_BUFFER_SIZE,
     BufferCreationFailed = TT_RES_BUFFER_CREATION_FAILED,
     OwnershipFailure = TT_RES_OWNERSHIP_FAILURE,
@@ -152,6 +155,19 @@ class HipCommandQueue {
   private:
     friend struct HipCommandQueueResult create_command_queue(const HipDevice&);
     detail::Handle<tt_queue, tt_queue_destroy> h_;
+};
+
+// create_event (resources.h:95-118, 240): a counter that command buffers of any queue of
+// the device signal and wait for.
+class HipEvent {
+  public:
+    HipEvent() noexcept = default;
+    explicit operator bool() const noexcept { return static_cast<bool>(h_); }
+    tt_event* native() const noexcept { return h_.get(); }
+
+  private:
+    friend struct HipEventResult create_event(const HipDevice&);
+    detail::Handle<tt_event, tt_event_destroy> h_;
 };
 
 class HipBuffer {
@@ -263,6 +279,13 @@ struct HipCommandQueueResult {
     std::optional<HipCommandQueue> command_queue;
     explicit operator bool() const noexcept {
         return error == HipResourceError::None && command_queue.has_value();
+    }
+};
+struct HipEventResult {
+    HipResourceError error;
+    std::optional<HipEvent> event;
+    explicit operator bool() const noexcept {
+        return error == HipResourceError::None && event.has_value();
     }
 };
 struct HipBufferResult {
@@ -502,6 +525,31 @@ inline HipCommandBufferResult end_compute_pass(HipComputePass&& pass) {
     HipCommandBuffer cb;
     cb.h_ = std::move(pass.h_);
     return {HipCommandError::None, std::move(cb)};
+}
+
+inline HipEventResult create_event(const HipDevice& device) {
+    if (!device) return {HipResourceError::InvalidDevice, std::nullopt};
+    tt_event* raw = nullptr;
+    const std::int32_t status = tt_event_create(device.native(), &raw);
+    if (status != TT_OK) return {static_cast<HipResourceError>(status), std::nullopt};
+    HipEvent event;
+    event.h_ = detail::Handle<tt_event, tt_event_destroy>(raw);
+    return {HipResourceError::None, std::move(event)};
+}
+
+// encode_wait_for_event / encode_signal_event (commands.h:421-426): between passes.  The
+// command buffer that signals must be committed before the one that waits for it.
+inline HipCommandError encode_wait_for_event(HipCommandBuffer& command_buffer, const HipEvent& event,
+                                             std::uint64_t value) {
+    if (!command_buffer) return HipCommandError::InvalidCommandBuffer;
+    return static_cast<HipCommandError>(
+        tt_encode_wait_for_event(command_buffer.native(), event.native(), value));
+}
+inline HipCommandError encode_signal_event(HipCommandBuffer& command_buffer, const HipEvent& event,
+                                           std::uint64_t value) {
+    if (!command_buffer) return HipCommandError::InvalidCommandBuffer;
+    return static_cast<HipCommandError>(
+        tt_encode_signal_event(command_buffer.native(), event.native(), value));
 }
 
 inline HipBlitPassResult begin_blit_pass(HipCommandBuffer&& command_buffer) {

@@ -6,6 +6,8 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -38,6 +40,14 @@ struct tt_buffer {
     std::atomic<int> refs{1};
 };
 
+// A counter command buffers signal and wait for: every signalled value owns a HIP event
+// recorded where the signal was committed; a wait takes the smallest value that reaches it.
+struct tt_event {
+    std::mutex mutex;
+    std::map<uint64_t, hipEvent_t> reached;
+    std::atomic<int> refs{1};
+};
+
 struct tt_library {
     tt_device* device = nullptr;
     std::vector<KernelDesc> kernels;
@@ -55,7 +65,7 @@ hipStream_t queue_stream(const tt_queue* queue) {
 
 namespace {
 
-enum class CommandKind : uint8_t { Dispatch, Copy, Fill };
+enum class CommandKind : uint8_t { Dispatch, Copy, Fill, Signal, Wait };
 
 struct Command {
     CommandKind kind;
@@ -67,6 +77,8 @@ struct Command {
     uint8_t* b;
     uint64_t length;
     uint8_t value;
+    tt_event* event;        // Signal / Wait
+    uint64_t event_value;
 };
 
 __global__ void tt_fill_bytes(uint8_t* dst, uint64_t length, uint8_t value) {
@@ -104,6 +116,13 @@ void release_buffer(tt_buffer* buffer) {
         if (buffer->owns_device && buffer->dptr != nullptr) (void)hipFree(buffer->dptr);
     }
     delete buffer;
+}
+
+void release_event(tt_event* event) {
+    if (event == nullptr) return;
+    if (event->refs.fetch_sub(1) != 1) return;
+    for (auto& reached : event->reached) (void)hipEventDestroy(reached.second);
+    delete event;
 }
 
 int32_t classify(hipError_t error) {
@@ -144,6 +163,7 @@ struct tt_command_buffer {
     // reference's command buffers retain their resources: a caller may destroy its handle
     // between encode and commit, or before a later replay.
     std::vector<tt_buffer*> retained;
+    std::vector<tt_event*> retained_events;
     hipEvent_t begin = nullptr;
     hipEvent_t end = nullptr;
     bool committed = false;
@@ -167,6 +187,8 @@ static void retain(tt_command_buffer* cb, const tt_buffer* buffer) {
 static void release_retained(tt_command_buffer* cb) {
     for (tt_buffer* buffer : cb->retained) release_buffer(buffer);
     cb->retained.clear();
+    for (tt_event* event : cb->retained_events) release_event(event);
+    cb->retained_events.clear();
 }
 
 extern "C" {
@@ -202,6 +224,7 @@ const char* tt_status_name(int32_t status) {
     case TT_RES_INVALID_DEVICE: return "Resource.InvalidDevice";
     case TT_RES_SYSTEM_DEVICE_UNAVAILABLE: return "Resource.SystemDeviceUnavailable";
     case TT_RES_COMMAND_QUEUE_CREATION_FAILED: return "Resource.CommandQueueCreationFailed";
+    case TT_RES_EVENT_CREATION_FAILED: return "Resource.EventCreationFailed";
     case TT_RES_INVALID_BUFFER_SIZE: return "Resource.InvalidBufferSize";
     case TT_RES_BUFFER_CREATION_FAILED: return "Resource.BufferCreationFailed";
     case TT_RES_OWNERSHIP_FAILURE: return "Resource.OwnershipFailure";
@@ -696,6 +719,21 @@ static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool
             const int32_t status = command.launch(command.bindings, command.grid, stream, false);
             error = hipGetLastError();
             if (status != TT_OK && error == hipSuccess) error = hipErrorInvalidValue;
+        } else if (command.kind == CommandKind::Signal) {
+            // a fresh HIP event per signalled value, recorded behind everything issued so far
+            std::lock_guard<std::mutex> lock(command.event->mutex);
+            hipEvent_t& reached = command.event->reached[command.event_value];
+            if (reached == nullptr) {
+                error = hipEventCreateWithFlags(&reached, hipEventDisableTiming);
+            }
+            if (error == hipSuccess) error = hipEventRecord(reached, stream);
+        } else if (command.kind == CommandKind::Wait) {
+            // the smallest committed signal that reaches the value
+            std::lock_guard<std::mutex> lock(command.event->mutex);
+            const auto reached = command.event->reached.lower_bound(command.event_value);
+            error = reached == command.event->reached.end()
+                        ? hipErrorNotReady
+                        : hipStreamWaitEvent(stream, reached->second, 0);
         } else if (command.kind == CommandKind::Copy) {
             const bool wide = ((reinterpret_cast<uintptr_t>(command.a) |
                                 reinterpret_cast<uintptr_t>(command.b)) & 15u) == 0;
@@ -741,6 +779,11 @@ int32_t tt_command_buffer_compile(tt_command_buffer* cb) {
     if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
     if (cb->pass_open) return TT_CMD_INVALID_COMPUTE_PASS;
     if (cb->commands.empty()) return TT_CMD_INVALID_COMMAND_BUFFER;
+    for (const Command& command : cb->commands) {
+        if (command.kind == CommandKind::Signal || command.kind == CommandKind::Wait) {
+            return TT_CMD_COMMAND_BUFFER_CREATION_FAILED;
+        }
+    }
     if (cb->committed) (void)hipEventSynchronize(cb->end);
     drop_graph(cb);
     hipStream_t stream = cb->queue->stream;
@@ -815,6 +858,44 @@ int32_t tt_wait(tt_command_buffer* cb, tt_execution_result* result) {
     }
     return TT_OK;
 }
+
+static int32_t encode_event(tt_command_buffer* cb, tt_event* event, uint64_t value,
+                            CommandKind kind) {
+    if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;
+    if (cb->pass_open) return TT_CMD_INVALID_COMMAND_BUFFER;   // between passes only
+    if (event == nullptr) return TT_CMD_INVALID_EVENT;
+    if (value == 0) return TT_CMD_INVALID_EVENT_VALUE;
+    Command command{};
+    command.kind = kind;
+    command.name = kind == CommandKind::Signal ? "signal_event" : "wait_for_event";
+    command.event = event;
+    command.event_value = value;
+    event->refs.fetch_add(1);
+    cb->retained_events.push_back(event);
+    cb->commands.push_back(command);
+    drop_graph(cb);
+    return TT_OK;
+}
+
+int32_t tt_encode_signal_event(tt_command_buffer* cb, tt_event* event, uint64_t value) {
+    return encode_event(cb, event, value, CommandKind::Signal);
+}
+
+int32_t tt_encode_wait_for_event(tt_command_buffer* cb, tt_event* event, uint64_t value) {
+    return encode_event(cb, event, value, CommandKind::Wait);
+}
+
+int32_t tt_event_create(tt_device* device, tt_event** out) {
+    if (out == nullptr) return TT_RES_EVENT_CREATION_FAILED;
+    *out = nullptr;
+    if (device == nullptr) return TT_RES_INVALID_DEVICE;
+    tt_event* event = new (std::nothrow) tt_event;
+    if (event == nullptr) return TT_RES_EVENT_CREATION_FAILED;
+    *out = event;
+    return TT_OK;
+}
+
+void tt_event_destroy(tt_event* event) { release_event(event); }
 
 int32_t tt_command_buffer_reset(tt_command_buffer* cb) {
     if (cb == nullptr) return TT_CMD_INVALID_COMMAND_BUFFER;

@@ -46,6 +46,11 @@ int main() {
     const HipExecutionResult waited = wait_until_completed(std::move(pending));
     if (waited.error != HipCommandError::InvalidPendingExecution || waited) return 20;
     if (did_modify_range(buffer, 0, 1) != HipCommandError::InvalidBuffer) return 21;
+    if (create_event(device).error != HipResourceError::InvalidDevice) return 23;
+    HipEvent event;
+    HipCommandBuffer cb3;
+    if (encode_signal_event(cb3, event, 1) != HipCommandError::InvalidCommandBuffer) return 24;
+    if (encode_wait_for_event(cb3, event, 1) != HipCommandError::InvalidCommandBuffer) return 25;
     // system device: either a device or the typed "unavailable" error, never a crash
     const HipDeviceResult made = create_system_device();
     if (!made && made.error != HipResourceError::SystemDeviceUnavailable) return 22;

@@ -1083,6 +1083,47 @@ int main() {
             return 90;
         }
     }
+    // ---- events: a fill on one queue, a copy of it on another that waits for the fill ----
+    {
+        auto second = create_command_queue(*device.device);
+        auto event = create_event(*device.device);
+        auto source = create_shared_buffer(*device.device, 1 << 20);
+        auto copied = create_shared_buffer(*device.device, 1 << 20);
+        if (!second || !event || !source || !copied) return 91;
+        auto first_cb = create_command_buffer(*queue.command_queue);
+        auto blit = begin_blit_pass(std::move(*first_cb.command_buffer));
+        if (fill_buffer(*blit.blit_pass, *source.buffer, 0, 1 << 20, std::byte{0x5A}) !=
+            HipCommandError::None) {
+            return 92;
+        }
+        auto filled = end_blit_pass(std::move(*blit.blit_pass));
+        if (encode_signal_event(*filled.command_buffer, *event.event, 0) !=
+            HipCommandError::InvalidEventValue) {
+            return 93;
+        }
+        if (encode_signal_event(*filled.command_buffer, *event.event, 1) != HipCommandError::None) {
+            return 94;
+        }
+        auto second_cb = create_command_buffer(*second.command_queue);
+        if (encode_wait_for_event(*second_cb.command_buffer, *event.event, 1) !=
+            HipCommandError::None) {
+            return 95;
+        }
+        auto blit2 = begin_blit_pass(std::move(*second_cb.command_buffer));
+        if (copy_buffer(*blit2.blit_pass, *source.buffer, 0, *copied.buffer, 0, 1 << 20) !=
+            HipCommandError::None) {
+            return 96;
+        }
+        auto copying = end_blit_pass(std::move(*blit2.blit_pass));
+        auto pending_fill = commit(std::move(*filled.command_buffer));
+        auto pending_copy = commit(std::move(*copying.command_buffer));
+        if (!pending_fill || !pending_copy) return 97;
+        if (!wait_until_completed(std::move(*pending_copy.pending_execution))) return 98;
+        if (!wait_until_completed(std::move(*pending_fill.pending_execution))) return 99;
+        for (const std::uint8_t byte : download<std::uint8_t>(*copied.buffer, 1 << 20)) {
+            if (byte != 0x5A) return 100;
+        }
+    }
     std::printf("runtime gpu test ok\n");
     return 0;
 }

@@ -82,3 +82,63 @@ def test_recording_keeps_its_buffers_alive():
         cb.commit().wait()
         assert np.array_equal(dst.read(np.uint32), data)
     del noise
+
+
+def test_events_order_command_buffers_of_two_queues():
+    """encode_signal_event / encode_wait_for_event: a chain of copies alternating between two
+    queues, each step waiting for the value the step before it signals; without the waits the
+    two streams would run the copies in any order."""
+    B, dev, queue, lib = gpu()
+    other = dev.create_queue()
+    event = dev.create_event()
+    n = 1 << 22
+    data = np.arange(n, dtype=np.uint32)
+    stages = [dev.buffer_from(data)] + [dev.create_buffer(n * 4) for _ in range(6)]
+    buffers = []
+    for step in range(6):
+        cb = (queue if step % 2 == 0 else other).create_command_buffer()
+        if step > 0:
+            cb.wait_for_event(event, step)
+        cb.copy_buffer(stages[step], 0, stages[step + 1], 0, n * 4)
+        cb.signal_event(event, step + 1)
+        assert cb.command_count == (3 if step > 0 else 2)
+        buffers.append(cb.commit())            # committed in dependency order
+    for cb in buffers:
+        cb.wait()
+    assert np.array_equal(stages[6].read(np.uint32), data)
+    # a wait is satisfied by a signal of a larger value
+    cb = other.create_command_buffer()
+    cb.wait_for_event(event, 3)
+    cb.fill_buffer(stages[1], 0, 16, 0xAB)
+    cb.commit().wait()
+    assert (stages[1].read(np.uint8)[:16] == 0xAB).all()
+
+
+def test_event_encoding_errors():
+    B, dev, queue, lib = gpu()
+    event = dev.create_event()
+    cb = queue.create_command_buffer()
+    with pytest.raises(B.BackendError) as e:
+        cb.signal_event(event, 0)
+    assert e.value.status == 4                 # InvalidEventValue
+    with pytest.raises(B.BackendError) as e:
+        cb.wait_for_event(None, 1)
+    assert e.value.status == 3                 # InvalidEvent
+    cb.begin_compute_pass()
+    with pytest.raises(B.BackendError) as e:   # between passes only
+        cb.signal_event(event, 1)
+    assert e.value.status == 2
+    cb.end_compute_pass()
+    assert cb.command_count == 0
+    # a wait whose signal has not been committed cannot be submitted
+    cb.wait_for_event(event, 7)
+    with pytest.raises(RuntimeError):          # the submission is reported as failed
+        cb.commit().wait()
+    # event commands keep a recording out of a graph
+    cb2 = queue.create_command_buffer()
+    cb2.signal_event(event, 7)
+    with pytest.raises(B.BackendError) as e:
+        cb2.compile()
+    assert e.value.status == 19
+    cb2.commit().wait()
+    cb.commit().wait()                         # now the value has been signalled
