@@ -603,10 +603,10 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     }
 }
 
-int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
-    const uint32_t out_rows = p.first_row[p.segments];
-    // the transfers move 16-byte pieces of x and of the nibble words and 4-byte pairs of
-    // scales and biases
+// What the block kernel assumes of its operands beyond their sizes: its transfers move
+// 16-byte pieces of x and of the nibble words and 4-byte pairs of scales and biases, and it
+// addresses x with 32-bit byte offsets.
+int32_t check_block_operands(const Q4Projection& p) {
     uintptr_t wide = reinterpret_cast<uintptr_t>(p.input), narrow = 0;
     for (uint32_t s = 0; s < p.segments; ++s) {
         wide |= reinterpret_cast<uintptr_t>(p.words[s]);
@@ -615,6 +615,14 @@ int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
     if ((wide & 15) != 0 || (narrow & 3) != 0 || ((p.input_stride * 2) & 15) != 0) {
         return TT_CMD_INVALID_BUFFER_OFFSET;
     }
+    if (static_cast<uint64_t>(p.rows) * p.input_stride * 2 >= (1ull << 32)) {
+        return TT_CMD_INVALID_DISPATCH_EXTENT;
+    }
+    return TT_OK;
+}
+
+int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
+    const uint32_t out_rows = p.first_row[p.segments];
     hipLaunchKernelGGL(q4_block_kernel,
                        dim3((out_rows + kBlockN - 1) / kBlockN, (p.rows + kBlockM - 1) / kBlockM),
                        dim3(kBlockThreads), kBlockLdsBytes, stream, p);
@@ -904,18 +912,17 @@ int32_t finish(Args& a, const Grid& g, hipStream_t stream, bool validate_only, c
     bind_segments(a, p, 1, f.segment_rows, f.segments, k_size);
     p.output = a.buffer<uint16_t>(
         f.out_slot, (static_cast<uint64_t>(p.rows - 1) * p.output_stride + out_rows) * 2);
-    if (a.status != TT_OK || validate_only) return a.status;
-    if (wave_kernel) return launch_wave(p, stream);
+    if (a.status != TT_OK) return a.status;
     // a handful of rows is a weight-streaming problem: the exact rows kernel; a block
     // is a matrix product: MFMA
-    if (p.rows > kQ4BatchRowsMax) {
-        // the block kernel addresses x with 32-bit byte offsets
-        if (static_cast<uint64_t>(p.rows) * p.input_stride * 2 >= (1ull << 32)) {
-            return TT_CMD_INVALID_DISPATCH_EXTENT;
-        }
-        return launch_block(p, stream);
+    const bool block = !wave_kernel && p.rows > kQ4BatchRowsMax;
+    if (block) {
+        const int32_t status = check_block_operands(p);
+        if (status != TT_OK) return status;
     }
-    return launch_rows(p, stream);
+    if (validate_only) return TT_OK;
+    if (wave_kernel) return launch_wave(p, stream);
+    return block ? launch_block(p, stream) : launch_rows(p, stream);
 }
 
 // one input row; grid (groups) x threads

@@ -249,4 +249,11 @@ def test_projection_validation():
     with pytest.raises(B.BackendError) as e:   # input width not a multiple of 512
         cb.encode(lib.pipeline("outproj_blk"), out_bindings, {5: 4, 6: 4000}, (1024, 1, 1), (64, 1, 1))
     assert e.value.status == 15
+    # the block form moves 16-byte pieces: an input bound 2 bytes off is refused when encoded
+    blk_bindings = dict(bindings)
+    blk_bindings[0] = (dev.create_buffer(64 * 2048 * 2 + 16), 2)
+    blk_bindings[10] = dev.create_buffer(64 * 9216 * 2)
+    with pytest.raises(B.BackendError) as e:
+        cb.encode(lib.pipeline("attn_project_blk"), blk_bindings, {11: 64}, (2304, 1, 1), (128, 1, 1))
+    assert e.value.status == 10
     assert cb.command_count == 0
