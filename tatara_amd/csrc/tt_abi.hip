@@ -42,6 +42,8 @@ struct tt_buffer {
 
 // A counter command buffers signal and wait for: every signalled value owns a HIP event
 // recorded where the signal was committed; a wait takes the smallest value that reaches it.
+constexpr size_t kEventValuesKept = 64;
+
 struct tt_event {
     std::mutex mutex;
     std::map<uint64_t, hipEvent_t> reached;
@@ -727,6 +729,14 @@ static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool
                 error = hipEventCreateWithFlags(&reached, hipEventDisableTiming);
             }
             if (error == hipSuccess) error = hipEventRecord(reached, stream);
+            // A wait takes the smallest committed value that reaches the one it asks for, so
+            // the oldest values can go once there are many: a late wait for one of them is
+            // served by a newer signal, which the counter has passed as well.
+            while (error == hipSuccess && command.event->reached.size() > kEventValuesKept &&
+                   command.event->reached.begin()->first != command.event_value) {
+                (void)hipEventDestroy(command.event->reached.begin()->second);
+                command.event->reached.erase(command.event->reached.begin());
+            }
         } else if (command.kind == CommandKind::Wait) {
             // the smallest committed signal that reaches the value
             std::lock_guard<std::mutex> lock(command.event->mutex);

@@ -114,6 +114,28 @@ def test_events_order_command_buffers_of_two_queues():
     assert (stages[1].read(np.uint8)[:16] == 0xAB).all()
 
 
+def test_event_keeps_serving_old_values():
+    """Many signalled values: the library keeps a bounded number of them, and a wait for one
+    it has let go of is served by a newer signal."""
+    B, dev, queue, lib = gpu()
+    other = dev.create_queue()
+    event = dev.create_event()
+    buf = dev.create_buffer(4096)
+    for value in range(1, 101):
+        cb = queue.create_command_buffer()
+        cb.fill_buffer(buf, 0, 4096, value)
+        cb.signal_event(event, value)
+        cb.commit()
+    cb = other.create_command_buffer()
+    cb.wait_for_event(event, 1)
+    copied = dev.create_buffer(4096)
+    cb.copy_buffer(buf, 0, copied, 0, 4096)
+    cb.commit().wait()
+    queue.synchronize()
+    seen = copied.read(np.uint8)
+    assert (seen == seen[0]).all() and 1 <= int(seen[0]) <= 100
+
+
 def test_event_encoding_errors():
     B, dev, queue, lib = gpu()
     event = dev.create_event()
