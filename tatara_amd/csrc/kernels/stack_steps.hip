@@ -125,6 +125,61 @@ __global__ __launch_bounds__(256) void dense_bf16_kernel(const uint16_t* input,
     }
 }
 
+// The same for at most 16 rows (a decode wave), sized for latency: a workgroup owns 16
+// outputs, its kWaves waves split K = 512 kWaves in slices of 512 columns, and a lane
+// requests all 16 weight fragments and all 16 x fragments of its slice before the first
+// product (the kernel above walks K with one dependent load pair after the other, which
+// makes a 64 KB weight stream per wave a chain of 32 round trips).  The slices are summed
+// through LDS in wave order.  grid ceil(N / 16) x 64 kWaves.
+template <uint32_t kWaves>
+__global__ __launch_bounds__(64 * kWaves) void dense_rows_kernel(const uint16_t* input,
+                                                                 const uint16_t* weights,
+                                                                 uint16_t* output, uint32_t rows,
+                                                                 uint32_t out_dim) {
+    constexpr uint32_t kInDim = 512 * kWaves;
+    __shared__ float partial[kWaves][4][64];
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t m = lane & 15;
+    const uint32_t g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * 16;
+    const uint16_t* wp =
+        weights + static_cast<uint64_t>(min(n0 + m, out_dim - 1)) * kInDim + wave * 512 + g * 8;
+    const uint16_t* xp = input + static_cast<uint64_t>(min(m, rows - 1)) * kInDim + wave * 512 + g * 8;
+    u32x4 w[16], x[16];
+#pragma unroll
+    for (uint32_t s = 0; s < 16; ++s) w[s] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + s * 32));
+#pragma unroll
+    for (uint32_t s = 0; s < 16; ++s) x[s] = *reinterpret_cast<const u32x4*>(xp + s * 32);
+    f32x4 acc0 = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4 acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t s = 0; s < 16; s += 2) {
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w[s]),
+                                                       __builtin_bit_cast(bf16x8, x[s]), acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w[s + 1]),
+                                                       __builtin_bit_cast(bf16x8, x[s + 1]), acc1, 0, 0, 0);
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) partial[wave][i][lane] = acc0[i] + acc1[i];
+    __syncthreads();
+    if (wave != 0 || m >= rows) return;
+    // lane holds outputs n0 + 4g + i of row m
+    uint16_t result[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        float total = partial[0][i][lane];
+#pragma unroll
+        for (uint32_t v = 1; v < kWaves; ++v) total += partial[v][i][lane];
+        result[i] = store16(total);
+    }
+    uint16_t* out = output + static_cast<uint64_t>(m) * out_dim + n0 + g * 4;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        if (n0 + g * 4 + i < out_dim) out[i] = result[i];
+    }
+}
+
 __global__ __launch_bounds__(256) void add_bf16_kernel(const uint16_t* a, const uint16_t* b,
                                                        uint16_t* out, uint32_t count) {
     const uint32_t at = blockIdx.x * 256 + threadIdx.x;
@@ -222,8 +277,17 @@ int32_t op_dense_bf16(const Bindings& b, const Grid& g, hipStream_t stream, bool
     const uint16_t* weights = a.buffer<const uint16_t>(1, static_cast<uint64_t>(out_dim) * in_dim * 2);
     uint16_t* output = a.buffer<uint16_t>(2, static_cast<uint64_t>(rows) * out_dim * 2);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(dense_bf16_kernel, dim3((out_dim + 63) / 64, (rows + 15) / 16), dim3(256), 0,
-                       stream, input, weights, output, rows, in_dim, out_dim);
+    // a decode wave over one of the model's two widths: the latency-sized form
+    if (rows <= 16 && in_dim == 2048) {
+        hipLaunchKernelGGL(dense_rows_kernel<4>, dim3((out_dim + 15) / 16), dim3(256), 0, stream, input,
+                           weights, output, rows, out_dim);
+    } else if (rows <= 16 && in_dim == 4096) {
+        hipLaunchKernelGGL(dense_rows_kernel<8>, dim3((out_dim + 15) / 16), dim3(512), 0, stream, input,
+                           weights, output, rows, out_dim);
+    } else {
+        hipLaunchKernelGGL(dense_bf16_kernel, dim3((out_dim + 63) / 64, (rows + 15) / 16), dim3(256), 0,
+                           stream, input, weights, output, rows, in_dim, out_dim);
+    }
     return TT_OK;
 }
 

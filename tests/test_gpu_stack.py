@@ -106,13 +106,15 @@ def _compare(step, got, want):
     assert np.isfinite(got).all()
     assert err.mean() <= 2e-2 * max(1.0, np.abs(want).max())
     if got.argmax() != want.argmax():
-        # a tie within the noise of the run: the checker itself ranks the GPU's choice no more
-        # than two bf16 steps of the winning logit below its own
+        # a tie within the noise of the run: the checker itself ranks the GPU's choice below its
+        # own by no more than two bf16 steps of the winning logit, or by no more than the two
+        # vectors differ anywhere (a gap smaller than the error of a logit decides nothing; the
+        # error itself is held by the mean bar above)
         step16 = 2.0 ** (np.floor(np.log2(max(abs(want.max()), 1e-30))) - 7)
         margin = want.max() - want[got.argmax()]
-        print(f"[parity] {step}: argmax differs on a margin of {margin:.3e} (bf16 step {step16:.3e})",
-              flush=True)
-        assert margin <= 2 * step16, step
+        print(f"[parity] {step}: argmax differs on a margin of {margin:.3e} (bf16 step {step16:.3e}, "
+              f"largest logit error {err.max():.3e})", flush=True)
+        assert margin <= max(2 * step16, err.max()), step
 
 
 @pytest.mark.parametrize("layers,quantized,fused", [(40, False, False), (12, True, False), (12, True, True)],
@@ -230,7 +232,8 @@ def test_rms_only_operators_bit_for_bit(rows, hidden):
 
 
 @pytest.mark.parametrize("rows,in_dim,out_dim", [(1, 2048, 9216), (4, 2048, 12352), (16, 4096, 2048),
-                                                 (37, 2048, 4096), (3, 64, 70)])
+                                                 (37, 2048, 4096), (3, 64, 70), (2, 2048, 70),
+                                                 (13, 4096, 24)])
 def test_dense_bf16_operator(rows, in_dim, out_dim):
     """The stub stack's dense projection against the checker (fp32 dot in ascending
     order, one bf16 rounding); the matrix unit sums in another order, so the bar is the
