@@ -1303,6 +1303,50 @@ struct CombineArgs {
     uint32_t single_partition;
 };
 
+// Up to kParts partitions: every load is requested before the first is used - the
+// numerators of all partitions by the lane that owns dimension d, their maxima and sums
+// through uniform loads, the gate - so the kernel is one round trip to memory deep instead
+// of one per stage (and, on the general path, one per eight partitions).
+template <uint32_t kParts>
+__device__ __forceinline__ void combine_few_parts(const float* base, uint32_t nparts, uint32_t d,
+                                                  const uint16_t* gate_at, uint16_t* out_at) {
+    __shared__ __attribute__((aligned(16))) float part_max[kParts];
+    __shared__ __attribute__((aligned(16))) float part_sum[kParts];
+    float numerator[kParts];
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; ++p) {
+        numerator[p] = base[static_cast<uint64_t>(min(p, nparts - 1)) * kAttnRecordFloats + d];
+    }
+    if (d < kParts) {
+        const float* rec = base + static_cast<uint64_t>(min(d, nparts - 1)) * kAttnRecordFloats;
+        part_max[d] = d < nparts ? rec[kD] : -INFINITY;
+        part_sum[d] = rec[kD + 1];
+    }
+    const uint16_t gate = *gate_at;
+    __syncthreads();
+    float gmax = -INFINITY;
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; p += 4) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
+        gmax = fmaxf(fmaxf(gmax, m4[0]), fmaxf(fmaxf(m4[1], m4[2]), m4[3]));
+    }
+    float acc = 0.0f, denom = 0.0f;
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; p += 4) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(part_sum + p);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            if (p + u < nparts) {
+                const float w = m4[u] == -INFINITY ? 0.0f : __expf(m4[u] - gmax);
+                acc = fmaf(w, numerator[p + u], acc);
+                denom += w * s4[u];
+            }
+        }
+    }
+    *out_at = f32_to_bf16_bits((acc / denom) * sigmoid_gate(gate));
+}
+
 // grid (16, rows) x 256.  out = bf16((sum_p w_p num_p / sum_p w_p sum_p) * sigmoid(gate)),
 // w_p = exp(max_p - max) (attention.metal:1086-1108).
 __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
@@ -1321,52 +1365,11 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                         static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
     const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
-    // Up to 32 partitions (a 32k context in splits of 1024 keys): every load is requested
-    // before the first is used - the numerators of all partitions by the lane that owns
-    // dimension d, their maxima and sums through uniform loads - so the kernel is one
-    // round trip to memory deep instead of one per stage; same operations in the same
-    // order as the general path below.
-    constexpr uint32_t kFastParts = 32;
-    if (nparts <= kFastParts) {
-        __shared__ __attribute__((aligned(16))) float part_max[kFastParts];
-        __shared__ __attribute__((aligned(16))) float part_sum[kFastParts];
-        float numerator[kFastParts];
-#pragma unroll
-        for (uint32_t p = 0; p < kFastParts; ++p) {
-            numerator[p] = base[static_cast<uint64_t>(min(p, nparts - 1)) * kAttnRecordFloats + d];
-        }
-        if (d < kFastParts) {
-            const float* rec = base + static_cast<uint64_t>(min(d, nparts - 1)) * kAttnRecordFloats;
-            part_max[d] = d < nparts ? rec[kD] : -INFINITY;
-            part_sum[d] = rec[kD + 1];
-        }
-        __syncthreads();
-        float pmax[kFastParts], psum[kFastParts];
-#pragma unroll
-        for (uint32_t p = 0; p < kFastParts; p += 4) {
-            const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
-            const f32x4 s4 = *reinterpret_cast<const f32x4*>(part_sum + p);
-#pragma unroll
-            for (uint32_t u = 0; u < 4; ++u) {
-                pmax[p + u] = m4[u];
-                psum[p + u] = s4[u];
-            }
-        }
-        float gmax = -INFINITY;
-#pragma unroll
-        for (uint32_t p = 0; p < kFastParts; ++p) gmax = fmaxf(gmax, pmax[p]);
-        float acc = 0.0f, denom = 0.0f;
-#pragma unroll
-        for (uint32_t p = 0; p < kFastParts; ++p) {
-            if (p < nparts) {
-                const float w = pmax[p] == -INFINITY ? 0.0f : __expf(pmax[p] - gmax);
-                acc = fmaf(w, numerator[p], acc);
-                denom += w * psum[p];
-            }
-        }
-        a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
-        return;
-    }
+    // 32 partitions are a 32k context in splits of 1024 keys, 128 a 100k context in splits of
+    // 800; beyond that the general path below
+    if (nparts <= 32) return combine_few_parts<32>(base, nparts, d, a.gate + at, a.out + at);
+    if (nparts <= 64) return combine_few_parts<64>(base, nparts, d, a.gate + at, a.out + at);
+    if (nparts <= 128) return combine_few_parts<128>(base, nparts, d, a.gate + at, a.out + at);
     __shared__ float red[256];
     __shared__ float weight[256];
     __shared__ float wsum[256];
