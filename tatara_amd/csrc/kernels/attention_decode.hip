@@ -136,14 +136,15 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         float c = 1.0f, s = 0.0f;
         if (d < 2 * kAttnRopePairs) {
             const float theta = static_cast<float>(position) / inverse_frequency;
-            c = cosf(theta);
-            s = sinf(theta);
+            sincosf(theta, &s, &c);   // one argument reduction for both
         }
         __syncthreads();  // the previous row's readers are done with the shared values
+        normed[d] = x;    // the head's values pass through LDS: no second trip to memory
+        __syncthreads();
         if (d < 64) {
             float acc = 0.0f;
             for (uint32_t j = 0; j < 4; ++j) {
-                const float v = bf16_bits_to_f32(proj[base + d * 4 + j]);
+                const float v = normed[d * 4 + j];
                 acc += v * v;
             }
             acc = half_wave_sum(acc);
