@@ -55,6 +55,8 @@ __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, c
     const uint16_t* in = input + static_cast<uint64_t>(blockIdx.y) * in_stride;
     uint16_t* out = output + static_cast<uint64_t>(blockIdx.y) * out_stride;
     u32x2 raw = *reinterpret_cast<const u32x2*>(in + 4 * t);
+    // requested with the row, not after the reduction
+    const u32x2 wraw = *reinterpret_cast<const u32x2*>(weight + 4 * t);
     if (addend != nullptr) {
         const u32x2 other = *reinterpret_cast<const u32x2*>(
             addend + static_cast<uint64_t>(blockIdx.y) * residual_stride + 4 * t);
@@ -83,7 +85,6 @@ __global__ __launch_bounds__(1024) void rms_only_kernel(const uint16_t* input, c
     }
     __syncthreads();
     const float inverse = inverse_norm;
-    const u32x2 wraw = *reinterpret_cast<const u32x2*>(weight + 4 * t);
     *reinterpret_cast<u32x2*>(out + 4 * t) =
         u32x2{rms_scale_pair(raw.x, wraw.x, inverse), rms_scale_pair(raw.y, wraw.y, inverse)};
 }
