@@ -288,7 +288,8 @@ class StubStack:
                 cb.encode(P("attention_decode_split_ms"),
                           {0: self.q, 1: layer["keys"], 2: layer["values"], 3: layer["table"],
                            4: self.partials},
-                          {5: self.capacity, 6: 4096, 7: self.split_keys, 8: self.max_splits, 9: 0},
+                          {5: self.capacity, 6: 4096, 7: self.split_keys, 8: self.max_splits,
+                           9: 2 if rows <= 2 else 0},   # one or two lanes: blocks dealt in turn
                           (self.max_splits, 2, rows), (256,))
                 cb.barrier()
                 cb.encode(P("attention_decode_combine_ms"),

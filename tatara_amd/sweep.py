@@ -1,7 +1,9 @@
 """Context sweep of the stubbed hybrid stack on one GPU: decode waves at a list of
 contexts and block prefill of a list of prompt lengths, for 1 and 4 lanes.  Only
 the attention-family kernels are counted (per-command device time); the stand-in
-projections, norms and residual sums run but are reported separately.
+projections, norms and residual sums run but are reported separately.  A decode
+point also replays the whole wave as one compiled graph (`graph_us_per_wave`:
+family, projections and norms together, without the per-command events).
 
     python -m tatara_amd.sweep [--layers 40] [--decode 1024,4096,...] [--prefill 4096,32768]
                                [--quantized]   (4-bit projections instead of dense bf16)
@@ -44,11 +46,19 @@ def measure_decode(dev, queue, lib, weights, layers, lanes, context, repeats=5):
         fam, stub = _family_ms(cb.command_times())
         if best is None or fam < best[0]:
             best = (fam, stub)
+    # the same wave as one compiled graph: device time of whole replays, launch gaps and all
+    graph = queue.create_command_buffer()
+    graph.begin_compute_pass()
+    st.record_token_wave(graph, with_head=False)
+    graph.end_compute_pass()
+    graph.compile()
+    replays = sorted(graph.commit().wait() for _ in range(3 + 2 * repeats))[: 2 * repeats]
     attn_layers = sum(1 for k in S.layer_kinds(layers) if k == "A")
     return {"mode": "decode", "lanes": lanes, "context": context, "layers": layers,
             "family_us_per_layer": round(best[0] * 1e3 / layers, 3),
             "family_us_per_wave": round(best[0] * 1e3, 1),
             "stub_us_per_wave": round(best[1] * 1e3, 1), "split_keys": st.split_keys,
+            "graph_us_per_wave": round(replays[len(replays) // 2] * 1e3, 1),
             "kv_bytes_per_wave": attn_layers * lanes * (context + 1) * 2048}
 
 
