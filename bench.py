@@ -45,6 +45,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from tatara_amd import stack as stack_rules   # noqa: E402  (the host's split-K planning rule)
+
 LANES = 4
 VISIBLE = 32768
 CAPACITY = 32768
@@ -75,15 +77,8 @@ class Wave:
 
     def __init__(self, dev, lib, torch, attention, split_keys, attention_layers, gdn_layers,
                  contexts, capacity, seed=0x7A7A):
-        if not split_keys:
-            # the host's own choice (runtime.cpp choose_split_keys): splits x 2 kv heads x lanes
-            # about one workgroup per compute unit, 128..1024 keys, a multiple of 32
-            per_group = -(-(max(contexts) + 1) * 2 * len(contexts) // dev.compute_units)
-            split_keys = max(128, min(1024, -(-per_group // 32) * 32))
-        self.dev, self.lib, self.attention, self.part = dev, lib, attention, split_keys
-        # as the host runtime records it: waves of one or two lanes deal a lane's 32-key blocks
-        # to its workgroups in turn
-        self.interleave = 1 if len(contexts) <= 2 else 0
+        self.dev, self.lib, self.attention = dev, lib, attention
+        self.forced_split = split_keys
         self.contexts, self.capacity = list(contexts), capacity
         self.rows = len(contexts)
         self.groups = dev.compute_units
@@ -101,7 +96,6 @@ class Wave:
 
         rows = self.rows
         stripe = 2 * capacity * 256
-        self.max_splits = (capacity + split_keys - 1) // split_keys
         ones = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
         self.set_contexts(contexts)
         self.attn = []
@@ -109,7 +103,8 @@ class Wave:
             self.attn.append(dict(keys=rand_bf16(rows * stripe), values=rand_bf16(rows * stripe),
                                   proj=rand_bf16(rows * 9216), q_w=ones, k_w=ones))
         self.b_q, self.b_gate, self.b_out = (dev.create_buffer(rows * 8192) for _ in range(3))
-        self.b_part = dev.create_buffer(rows * 16 * self.max_splits * 258 * 4)
+        # records down to the finest split the rule picks (128 keys)
+        self.b_part = dev.create_buffer(rows * 16 * ((capacity + 127) // 128) * 258 * 4)
         self.b_scratch = dev.create_buffer(layer_scratch_bytes(self.groups, rows))
         conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
         table = np.zeros(64, np.uint32)
@@ -143,6 +138,19 @@ class Wave:
             table[r * 4 + 1] = context
         self.contexts = list(contexts)
         self.attn_table = self.dev.buffer_from(table)
+        # The split-K walk as the host runtime plans it for a wave (runtime.cpp
+        # choose_split_keys and the operator's c9): keys per workgroup so that the
+        # workgroups that hold keys come to about one per compute unit (at least 128 keys, a
+        # multiple of 32); waves of one or two lanes deal a lane's 32-key blocks to its
+        # workgroups in turn; where the grid is larger than the chip and part of it holds no
+        # keys, the workgroups that do are placed first in the dispatch order.
+        visible = [c + 1 for c in contexts]
+        self.part = self.forced_split or stack_rules.choose_split_keys(visible, self.dev.compute_units)
+        self.max_splits = (self.capacity + self.part - 1) // self.part
+        self.interleave = 1 if self.rows <= 2 else 0
+        live = stack_rules.split_workgroups(visible, self.part)
+        grid = self.max_splits * 2 * self.rows
+        self.compact = 1 if grid > live and grid > self.dev.compute_units else 0
 
     def visible_keys(self):
         return sum(c + 1 for c in self.contexts)
@@ -177,7 +185,7 @@ class Wave:
         cb.encode(P("attention_decode_split_ms"),
                   {0: self.b_q, 1: layer["keys"], 2: layer["values"], 3: self.attn_table,
                    4: self.b_part}, {5: cap, 6: 4096, 7: self.part, 8: self.max_splits,
-                   9: 2 * self.interleave},
+                   9: 2 * self.interleave + 4 * self.compact},
                   (self.max_splits, 2, rows), (256,))
         if not walk_only:
             cb.barrier()
@@ -230,6 +238,7 @@ def attention_figures(queue, wave):
     gbs = algo / (walk["median_us"] * 1e-6) / 1e9
     return {"lanes_visible_keys": [c + 1 for c in wave.contexts], "algorithmic_bytes": algo,
             "split_keys": wave.part if wave.attention == "three" else None,
+            "workgroups_with_keys_first": bool(wave.compact) if wave.attention == "three" else None,
             "walk_kernel": walk, "walk_kernel_gbs": round(gbs, 1),
             "walk_kernel_frac": round(gbs / HBM_PEAK_GBS, 4),
             "layer_all_dispatches": layer,

@@ -180,12 +180,40 @@ std::uint32_t attention_partitions(std::uint32_t context) {
                                         : (count + kAttentionPartition - 1) / kAttentionPartition;
 }
 
-std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
+std::uint32_t split_workgroups(std::span<const std::uint32_t> visible_keys,
+                               std::uint32_t split_keys) noexcept {
+    std::uint64_t groups = 0;
+    for (const std::uint32_t keys : visible_keys) {
+        groups += 2 * ((std::uint64_t{keys} + split_keys - 1) / split_keys);   // two kv heads
+    }
+    return static_cast<std::uint32_t>(std::min<std::uint64_t>(groups, UINT32_MAX));
+}
+
+std::uint32_t choose_split_keys(std::span<const std::uint32_t> visible_keys,
                                 std::uint32_t compute_units) noexcept {
     const std::uint64_t units = std::max<std::uint32_t>(compute_units, 1);
-    const std::uint64_t per_group = (std::uint64_t{keys} * 2 * std::max<std::uint32_t>(rows, 1) + units - 1) / units;
-    const std::uint64_t rounded = (per_group + 31) / 32 * 32;
-    return static_cast<std::uint32_t>(std::clamp<std::uint64_t>(rounded, 128, 1024));
+    std::uint64_t total = 0;
+    for (const std::uint32_t keys : visible_keys) total += keys;
+    // an even share of all keys, then coarser until the last, partly filled split of every
+    // row fits too: one workgroup more than compute units costs a third of the walk
+    std::uint64_t split = std::max<std::uint64_t>(((2 * total + units - 1) / units + 31) / 32 * 32, 128);
+    while (split < UINT32_MAX - 31 &&
+           split_workgroups(visible_keys, static_cast<std::uint32_t>(split)) > units &&
+           2 * visible_keys.size() <= units) {
+        split += 32;
+    }
+    return static_cast<std::uint32_t>(split);
+}
+
+std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
+                                std::uint32_t compute_units) noexcept {
+    const std::array<std::uint32_t, kMaximumBatchRows> same = [&] {
+        std::array<std::uint32_t, kMaximumBatchRows> v{};
+        v.fill(keys);
+        return v;
+    }();
+    const std::size_t count = std::clamp<std::size_t>(rows, 1, same.size());
+    return choose_split_keys(std::span<const std::uint32_t>(same.data(), count), compute_units);
 }
 
 DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
@@ -514,19 +542,26 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
     const std::uint64_t bucket_offset = step.schedule.size() * 256;
     bool any_long = false;
     for (const DecodeStream& s : streams) any_long |= attention_partitions(s.context) != 1;
-    std::uint32_t longest = 1;
-    for (const DecodeStream& s : streams) longest = std::max(longest, s.context + 1);
-    // The grid always covers the capacity (the operator reads the contexts on the device
-    // and refuses a grid that could miss keys); a chosen split fits the longest lane of
-    // this wave, but no finer than 4096 workgroups over the capacity, most of which exit
-    // at once.
+    // Keys per split-K workgroup: chosen from the depths of the rows that take the split
+    // path, but no finer than 4096 workgroups over the capacity.  The grid always covers the
+    // capacity (the operator reads the contexts on the device and refuses a grid that could
+    // miss keys); where that leaves workgroups without keys in a grid larger than the chip,
+    // the ones with keys are placed first in the dispatch order (bit 2 of the operator's c9).
+    std::array<std::uint32_t, kMaximumBatchRows> visible{};
+    std::size_t long_rows = 0;
+    for (const DecodeStream& s : streams) {
+        if (attention_partitions(s.context) != 1 && long_rows < visible.size()) {
+            visible[long_rows++] = s.context + 1;
+        }
+    }
+    const std::span<const std::uint32_t> long_keys(visible.data(), long_rows);
+    const std::uint32_t units = batch.layer_groups != 0 ? batch.layer_groups : 256;
     std::uint32_t split_keys = batch.split_keys;
     if (split_keys == 0) {
         const std::uint64_t coarsest =
-            (std::uint64_t{step.capacity} * 2 * rows + 4095) / 4096;
-        split_keys = std::max(choose_split_keys(rows, longest),
-                              static_cast<std::uint32_t>(std::min<std::uint64_t>(
-                                  (coarsest + 31) / 32 * 32, 1024)));
+            ((std::uint64_t{step.capacity} * 2 * rows + 4095) / 4096 + 31) / 32 * 32;
+        split_keys = std::max(choose_split_keys(long_keys, units),
+                              static_cast<std::uint32_t>(std::min<std::uint64_t>(coarsest, 1u << 30)));
     }
     const std::uint32_t max_splits = (step.capacity + split_keys - 1) / split_keys;
     if (any_long && batch.attn_partials.size_bytes() <
@@ -647,8 +682,17 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                 walk.constant(max_splits, 8);
                 // bit 0: short rows are left to the single-partition operator; bit 1: waves of
                 // one or two lanes deal a lane's 32-key blocks to its workgroups in turn
-                // (measured 1-3 % faster there, 3 % slower at four lanes)
-                walk.constant(1u | (rows <= 2 ? 2u : 0u), 9);
+                // (measured 1-3 % faster there, 3 % slower at four lanes); bit 2: the grid is
+                // larger than the chip and part of it holds no keys, so the workgroups that do
+                // go first (0.4 us dearer than the order by grid position where that is not so)
+                const std::uint64_t grid_groups = std::uint64_t{max_splits} * 2 * rows;
+                const bool keyless_between =
+                    grid_groups > units && grid_groups > split_workgroups(long_keys, split_keys);
+                const bool in_turn =
+                    batch.split_order == DecodeBatchScratch::SplitOrder::Automatic
+                        ? rows <= 2
+                        : batch.split_order == DecodeBatchScratch::SplitOrder::BlocksInTurn;
+                walk.constant(1u | (in_turn ? 2u : 0u) | (keyless_between ? 4u : 0u), 9);
                 walk.dispatch(HipSize{max_splits, 2, rows}, HipSize{256, 1, 1});
                 walk.barrier();
                 walk.pipeline(k.attention_combine_ms);

@@ -195,8 +195,16 @@ struct DecodeBatchScratch {
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended, attn_partials;
     HipBuffer state_offsets;
     // keys per split-K workgroup of the batched path (a multiple of 32); 0: chosen for
-    // every wave from its longest context by choose_split_keys
+    // every wave from the depths of its rows by choose_split_keys
     std::uint32_t split_keys{0};
+    // How a row's split-K workgroups share its keys: consecutive ranges of `split_keys`, or
+    // its 32-key blocks in turn.  Automatic: in turn for waves of one or two rows.  Ranges
+    // are the faster order at most depths, but their time depends on how the cache's strides
+    // fall on the memory channels (measured 47-77 us for the same 4 x 32768 keys over
+    // capacities 32768 ... 135168 at 1024 keys a workgroup), blocks in turn do not
+    // (48-49 us): a deployment whose capacity falls badly can pin the order here.
+    enum class SplitOrder : std::uint8_t { Automatic, Ranges, BlocksInTurn };
+    SplitOrder split_order{SplitOrder::Automatic};
     // One dispatch per Gated DeltaNet layer (gdn_decode_fused_ms) instead of the
     // reference's prepare / recurrence / gate-norm triple; same results bit for bit.
     bool gdn_fused{true};
@@ -210,11 +218,17 @@ struct DecodeBatchScratch {
     HipBuffer attn_layer_scratch;
 };
 
-// Keys per split-K workgroup with which one attention layer of a wave of `rows` lanes
-// fills the compute units about once (splits x 2 kv heads x rows ~ compute_units):
-// between 128 and 1024 keys, a multiple of 32.
+// Keys per split-K workgroup for one attention layer of a wave whose rows see
+// `visible_keys[r]` keys each: the finest multiple of 32, at least 128, with which the
+// workgroups that hold keys (two kv heads x the rows' ceil(keys / split)) fit the compute
+// units one each.  The second form: `rows` rows at the same depth.
+std::uint32_t choose_split_keys(std::span<const std::uint32_t> visible_keys,
+                                std::uint32_t compute_units = 256) noexcept;
 std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
                                 std::uint32_t compute_units = 256) noexcept;
+// Workgroups of that layer's split-K grid that hold keys.
+std::uint32_t split_workgroups(std::span<const std::uint32_t> visible_keys,
+                               std::uint32_t split_keys) noexcept;
 
 // The step: geometry, schedule and pipelines; its own primary slot (decode_step.h:115-153).
 struct DecodeStep {

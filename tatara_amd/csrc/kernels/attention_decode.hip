@@ -45,6 +45,7 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr uint32_t kD = kAttnHeadDim;
 constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
@@ -288,6 +289,7 @@ struct FlashArgs {
     uint32_t single_partition;  // keys of one reference partition (256)
     uint32_t row_limit;         // rows the q / gate / out / table operands hold
     uint32_t interleave;        // 1: a row's workgroups take its 32-key blocks in turn
+    uint32_t compact;           // 1: the splits that hold keys lead the dispatch order
 };
 
 // value of lane (l ^ 8) within each row of 16 lanes
@@ -307,18 +309,50 @@ __device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
 
 __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const uint32_t split = blockIdx.x;
-    const uint32_t kvh = blockIdx.y;
+    uint32_t split = blockIdx.x;
+    uint32_t kvh = blockIdx.y;
     uint32_t row = blockIdx.z;
-    if (a.row_list != nullptr) {
-        row = a.row_list[row];
-        if (row >= a.row_limit) return;  // a bad list entry must not index outside the slabs
-    }
     uint64_t kv_offset = 0;
     uint32_t context = a.context;
-    if (a.table != nullptr) {
-        kv_offset = a.table[row * 4];
-        context = a.table[row * 4 + 1];
+    if (a.compact) {
+        // The grid covers the capacity of every row, but only ceil(keys / part) splits of a row
+        // hold keys.  Taken by grid position, the empty ones lie between the others in the
+        // dispatch order and the ones that work end up two to a compute unit while other units
+        // hold none.  Here the workgroups that work are the first of the dispatch order, row
+        // after row, head after head, split after split, and the rest of the grid leaves at
+        // once: lane r counts the splits of row r, a prefix sum over the rows places this
+        // workgroup.  (Launched with a state table, without a row list, never in final mode.)
+        const uint32_t l = threadIdx.x & 63;
+        const u32x2 entry = *reinterpret_cast<const u32x2*>(a.table + min(l, gridDim.z - 1) * 4);
+        uint32_t mine = 0;
+        if (l < gridDim.z && entry[1] < a.capacity) {
+            const uint32_t keys = entry[1] + 1;
+            if (!(a.long_rows_only && keys <= a.single_partition)) mine = (keys + a.part - 1) / a.part;
+        }
+        uint32_t through = mine;   // splits of rows 0 .. l
+        through += __builtin_amdgcn_update_dpp(0, through, 0x111, 0xF, 0xF, true);   // row_shr:1
+        through += __builtin_amdgcn_update_dpp(0, through, 0x112, 0xF, 0xF, true);
+        through += __builtin_amdgcn_update_dpp(0, through, 0x114, 0xF, 0xF, true);
+        through += __builtin_amdgcn_update_dpp(0, through, 0x118, 0xF, 0xF, true);
+        const uint32_t linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const uint64_t passed = __ballot(l < kMaxBatchRows && kAttnKvHeads * through <= linear);
+        row = __builtin_popcountll(passed);
+        if (row >= gridDim.z) return;
+        const uint32_t row_splits = __builtin_amdgcn_readlane(mine, row);
+        const uint32_t place = linear - kAttnKvHeads * (__builtin_amdgcn_readlane(through, row) - row_splits);
+        kvh = place >= row_splits ? 1u : 0u;   // two kv heads
+        split = place - kvh * row_splits;
+        kv_offset = __builtin_amdgcn_readlane(entry[0], row);
+        context = __builtin_amdgcn_readlane(entry[1], row);
+    } else {
+        if (a.row_list != nullptr) {
+            row = a.row_list[row];
+            if (row >= a.row_limit) return;  // a bad list entry must not index outside the slabs
+        }
+        if (a.table != nullptr) {
+            kv_offset = a.table[row * 4];
+            context = a.table[row * 4 + 1];
+        }
     }
     if (context >= a.capacity) return;  // a bad table row must not read outside the cache
     const uint32_t n = context + 1;
@@ -1739,7 +1773,9 @@ int32_t op_attention_combine(const Bindings& b, const Grid& g, hipStream_t strea
 // c6 query stride, c7 part (keys per workgroup, multiple of 32), c8 max_splits,
 // c9 bit 0 long_rows_only (1: rows whose context fits one 256-key partition are left
 // to attention_decode_ms), bit 1 interleave (1: a row's workgroups take its blocks of
-// 32 keys in turn instead of `part` consecutive keys each); grid (max_splits, 2, rows) x 256.
+// 32 keys in turn instead of `part` consecutive keys each), bit 2 compact (1: the
+// workgroups whose splits hold keys are the first of the dispatch order, whatever the
+// contexts; same records); grid (max_splits, 2, rows) x 256.
 int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stream,
                               bool validate_only) {
     Args a(b);
@@ -1750,6 +1786,7 @@ int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stre
     f.record_splits = a.constant(8);
     f.long_rows_only = a.constant(9) & 1;
     f.interleave = (a.constant(9) >> 1) & 1;
+    f.compact = (a.constant(9) >> 2) & 1;
     f.single_partition = kAttnPartition;
     const uint32_t rows = static_cast<uint32_t>(g.gz);
     a.require(f.capacity != 0 && f.query_stride >= kAttnQueryValues && f.part != 0 &&
@@ -1767,6 +1804,8 @@ int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stre
     f.values = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
     f.table = a.buffer<const uint32_t>(3, rows * 16);
     f.partials = a.buffer<float>(4, f.partial_row_floats * rows * 4);
+    // the compact order reads a table row as one 8-byte load
+    a.require(!f.compact || reinterpret_cast<uintptr_t>(f.table) % 8 == 0, TT_CMD_INVALID_BUFFER_OFFSET);
     if (a.status != TT_OK || validate_only) return a.status;
     return launch_flash(f, f.record_splits, rows, stream);
 }

@@ -85,13 +85,21 @@ def make_weights(layers, vocab, seed, quantized=False):
     return out
 
 
-def choose_split_keys(lanes, capacity):
-    """Keys per split-K workgroup so that one attention layer of a token wave fills
-    the 256 compute units about once: splits * 2 kv heads * lanes ~ 256, between 128
-    and 1024 keys, a multiple of 32."""
-    keys = (capacity * 2 * lanes + 255) // 256
-    keys = ((keys + 31) // 32) * 32
-    return max(128, min(1024, keys))
+def split_workgroups(visible_keys, split_keys):
+    """Workgroups of one attention layer's split-K grid that hold keys (two kv heads)."""
+    return 2 * sum(-(-keys // split_keys) for keys in visible_keys)
+
+
+def choose_split_keys(visible_keys, compute_units=256):
+    """Keys per split-K workgroup for a token wave whose lanes see `visible_keys[r]` keys
+    each: the finest multiple of 32, at least 128, with which the workgroups that hold
+    keys fit the compute units one each (runtime.cpp choose_split_keys)."""
+    visible_keys = list(visible_keys)
+    share = -(-2 * sum(visible_keys) // compute_units)
+    split = max(128, -(-share // 32) * 32)
+    while split_workgroups(visible_keys, split) > compute_units and 2 * len(visible_keys) <= compute_units:
+        split += 32
+    return split
 
 
 class StubStack:
@@ -115,7 +123,7 @@ class StubStack:
         self.groups = dev.compute_units
         self.lanes, self.capacity, self.vocab = lanes, capacity, vocab
         self.block_rows = block_rows
-        self.split_keys = split_keys or choose_split_keys(lanes, capacity)
+        self.split_keys = split_keys or choose_split_keys([capacity] * lanes, dev.compute_units)
         split_keys = self.split_keys
         self.max_splits = (capacity + split_keys - 1) // split_keys
         up = dev.buffer_from
@@ -256,6 +264,14 @@ class StubStack:
         """The final norm has been applied by the last layer's residual step."""
         self._dense(cb, self.normed, self.w_vocab, self.logits, rows, HIDDEN, self.vocab)
 
+    def _split_flags(self, rows):
+        """c9 of attention_decode_split_ms as the host runtime sets it: one or two lanes take
+        their blocks in turn (bit 1); where the grid is larger than the chip and part of it
+        holds no keys, the workgroups that do go first (bit 2)."""
+        live = split_workgroups([c + 1 for c in self.context[:rows]], self.split_keys)
+        grid = self.max_splits * 2 * rows
+        return (2 if rows <= 2 else 0) | (4 if grid > live and grid > self.groups else 0)
+
     # ---- one token for every lane ----
     def record_token_wave(self, cb, with_head=True):
         """Records one decode step of all lanes; the lanes' inputs are rows of self.x.
@@ -289,7 +305,7 @@ class StubStack:
                           {0: self.q, 1: layer["keys"], 2: layer["values"], 3: layer["table"],
                            4: self.partials},
                           {5: self.capacity, 6: 4096, 7: self.split_keys, 8: self.max_splits,
-                           9: 2 if rows <= 2 else 0},   # one or two lanes: blocks dealt in turn
+                           9: self._split_flags(rows)},
                           (self.max_splits, 2, rows), (256,))
                 cb.barrier()
                 cb.encode(P("attention_decode_combine_ms"),

@@ -52,12 +52,24 @@ int main() {
         attention_partitions(512) != 3 || attention_partitions(32767) != 128) {
         return 18;
     }
-    // split choice: splits x 2 kv heads x lanes ~ 256 compute units, 128..1024 keys, x32
+    // split choice: the workgroups that hold keys (2 kv heads x splits of every row) fit 256
+    // compute units one each; at least 128 keys, a multiple of 32
     if (choose_split_keys(4, 32768) != 1024 || choose_split_keys(1, 32768) != 256 ||
         choose_split_keys(1, 100000) != 800 || choose_split_keys(4, 16384) != 512 ||
-        choose_split_keys(1, 1) != 128 || choose_split_keys(16, 262144) != 1024 ||
-        choose_split_keys(0, 0, 0) != 128 || choose_split_keys(1, 20000) % 32 != 0) {
+        choose_split_keys(1, 1) != 128 || choose_split_keys(16, 262144) != 32768 ||
+        choose_split_keys(0, 0, 0) != 128 || choose_split_keys(1, 20000) % 32 != 0 ||
+        choose_split_keys(4, 100000) != 3136 || choose_split_keys(3, 32768) != 800) {
         return 19;
+    }
+    {
+        const std::array<std::uint32_t, 4> ragged{32768, 30000, 24576, 8192};
+        const std::array<std::uint32_t, 8> wide{65536, 50001, 40001, 30001, 20001, 10001, 5001, 1001};
+        if (choose_split_keys(ragged) != 768 || split_workgroups(ragged, 768) != 252 ||
+            split_workgroups(ragged, 1024) != 188 || choose_split_keys(wide) != 1792 ||
+            split_workgroups(wide, 1792) != 254 ||
+            choose_split_keys(std::span<const std::uint32_t>{}) != 128) {
+            return 19;
+        }
     }
 
     const PrefillPolicy policy{.schedule = PrefillSchedule::LayerMajor,

@@ -398,7 +398,15 @@ int main() {
             // matrix-unit wave leaves by a rounding step here and there
             const bool reordered = wave == 1;
             stages.matrix_unit = reordered;
-            batch.split_keys = wave == 0 ? 256 : 0;   // the second wave chooses its own split
+            // the second wave chooses its own split, for a chip of four compute units: 704 keys
+            // (one workgroup per long row and head) in a grid of twelve, so the workgroups that
+            // hold keys are placed first in the dispatch order
+            batch.split_keys = wave == 0 ? 256 : 0;
+            const std::uint32_t chip_units = batch.layer_groups;
+            if (wave == 1) {
+                batch.layer_groups = 4;
+                batch.split_order = DecodeBatchScratch::SplitOrder::BlocksInTurn;   // pinned, three rows
+            }
             std::vector<std::uint16_t> x = gauss16(7400 + wave, kLanes * 2048);
             if (!upload(hidden.input, x)) return 206;
             std::vector<DecodeStream> streams;
@@ -409,6 +417,8 @@ int main() {
                 return encode_token_batch(step, streams, *pooled.pool, batch, bound, stages.hooks(),
                                           pass);
             });
+            batch.layer_groups = chip_units;
+            batch.split_order = DecodeBatchScratch::SplitOrder::Automatic;
             if (rc != 0) return 210 + rc;
             const auto got_residual = download<std::uint16_t>(hidden.residual, kLanes * 2048);
             const auto got_normed = download<std::uint16_t>(hidden.normed, kLanes * 2048);

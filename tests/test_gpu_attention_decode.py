@@ -186,10 +186,12 @@ def test_decode_context_edges(ctx):
         check_bf16(b_o2.read(np.uint16), want, f"split part {part} ctx {ctx}")
 
 
-def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False):
+def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=False):
     """Lane-batched decode over a striped pool with a state table, long rows
     through attention_decode_split_ms and short rows through attention_decode_ms.
     interleave: a lane's workgroups take its 32-key blocks in turn (bit 1 of c9).
+    compact: the workgroups whose splits hold keys lead the dispatch order (bit 2 of c9);
+    the records, and so the output bits, are those of the plain order.
     replays > 0: the recording is also compiled into a HIP graph and replayed that
     many times with the outputs and records cleared in between; every replay must
     reproduce the eager bits."""
@@ -230,7 +232,7 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False):
     def rec(cb):
         cb.encode(lib.pipeline("attention_decode_split_ms"),
                   {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
-                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1 + 2 * int(interleave)},
+                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1 + 2 * int(interleave) + 4 * int(compact)},
                   (max_splits, 2, rows), (256,))
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
@@ -240,7 +242,7 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False):
             cb.encode(lib.pipeline("attention_decode_ms"),
                       {0: b_q, 1: b_g, 2: k_pool, 3: v_pool, 4: b_tab, 5: b_o,
                        7: (b_tab, 256)}, {6: cap, 8: 4096}, (16, len(short)), (256,))
-    ms = run(rec)
+    run(rec)
     got = b_o.read(np.uint16).reshape(rows, 4096)
     for r, ctx in enumerate(contexts):
         check_bf16(got[r], want[r], f"lane {r} ctx {ctx} (stripe {stripes[r]}, part {part})")
@@ -253,7 +255,7 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False):
             b_part.write(np.full(rows * 16 * max_splits * 258, np.nan, np.float32))
             cb.commit().wait()
             assert np.array_equal(b_o.read(np.uint16).reshape(rows, 4096), got), f"replay {replay}"
-    return ms
+    return got
 
 
 def test_lane_batch_small_ragged():
@@ -271,6 +273,23 @@ def test_lane_batch_interleaved_blocks(contexts, cap, part):
     records cover interleaved key sets, the combined output is held to the same bar."""
     print(f"[case] lane batch interleaved {contexts} part {part}", flush=True)
     _lane_batch(contexts, cap, part, 0x1E7E, replays=2, interleave=True)
+
+
+@pytest.mark.parametrize("contexts,cap,part,interleave", [
+    ([2000, 1499, 700, 100, 255, 256, 0, 287, 288, 319], 2048, 128, False),  # short rows between long ones
+    ([300, 5000, 4999, 31, 2047], 8192, 1024, False),          # capacity well past every context
+    ([99999], 100000, 800, True),                               # the single deep lane, blocks in turn
+    ([32767, 29999, 24575, 8191], 32768, 768, False),           # config 3's ragged lanes, 252 live of 344
+    ([1000] * 16, 1024, 128, False),                            # every row of a full wave
+], ids=["ragged-128", "roomy-1024", "lane100k-800", "config3-ragged-768", "sixteen-lanes"])
+def test_lane_batch_compact_dispatch_order(contexts, cap, part, interleave):
+    """The workgroups that hold keys placed first in the dispatch order: same records as
+    the order by grid position, so the output must equal that order's bit for bit, and
+    the oracle's within the bar."""
+    print(f"[case] lane batch compact {contexts} part {part}", flush=True)
+    outputs = [_lane_batch(contexts, cap, part, 0xC0AC, replays=2 if compact else 0,
+                           interleave=interleave, compact=compact) for compact in (False, True)]
+    assert np.array_equal(outputs[0], outputs[1])
 
 
 def test_config3_four_ragged_lanes_at_depth():

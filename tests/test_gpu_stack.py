@@ -317,7 +317,7 @@ def test_stacked_run_at_depth_four_ragged_lanes(form):
     embed = weights["embed"].reshape(vocab, 2048)
     stack = S.StubStack(dev, lib, weights, len(prompts), capacity, vocab, block_rows=block_rows,
                         attention_form=form)
-    assert stack.split_keys == S.choose_split_keys(len(prompts), capacity)
+    assert stack.split_keys == S.choose_split_keys([capacity] * len(prompts))
     for lane, prompt in enumerate(prompts):
         for first in range(0, len(prompt), block_rows):
             rows = min(block_rows, len(prompt) - first)
