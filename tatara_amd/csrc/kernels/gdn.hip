@@ -606,29 +606,40 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
         q4[i] = qk_n[lane * 4 + i];
         k4[i] = qk_n[kGD + lane * 4 + i];
     }
+    // The eight rows of a half wave go through each step side by side, not row after row:
+    // a row's two cross-lane sums are chains of dependent lane exchanges (the last through the
+    // LDS crossbar), and eight independent chains fill each other's waits.
+    float kv[8], out[8];
 #pragma unroll
     for (uint32_t it = 0; it < 8; ++it) {
-        const uint32_t j = half * 8 + it;
-        float kv = 0.0f;
+        kv[it] = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
             st[it][i] *= decay;
-            kv = fmaf(st[it][i], k4[i], kv);
+            kv[it] = fmaf(st[it][i], k4[i], kv[it]);
         }
-        kv = half_wave_sum(kv);
-        const float delta = (act[2 * kGD + j] - kv) * beta;
-        float out = 0.0f;
+    }
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) kv[it] = half_wave_sum(kv[it]);
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) {
+        const float delta = (act[2 * kGD + half * 8 + it] - kv[it]) * beta;
+        out[it] = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
             st[it][i] = fmaf(k4[i], delta, st[it][i]);
-            out = fmaf(st[it][i], q4[i], out);
+            out[it] = fmaf(st[it][i], q4[i], out[it]);
         }
-        out = half_wave_sum(out);
         // written once, read by the next token's dispatch at the earliest: stored past the
         // cache (nontemporal), so the dispatch does not end on a write-back of the whole state
         __builtin_nontemporal_store(st[it], reinterpret_cast<f32x4*>(
-            state_out + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4));
-        if (lane == 0) y_head[j] = rb(out);
+            state_out + (static_cast<uint64_t>(h) * kGD + half * 8 + it) * kGD + lane * 4));
+    }
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) out[it] = half_wave_sum(out[it]);
+    if (lane == 0) {
+#pragma unroll
+        for (uint32_t it = 0; it < 8; ++it) y_head[half * 8 + it] = rb(out[it]);
     }
     __syncthreads();
     if (tid < kGD) {
