@@ -523,11 +523,11 @@ struct FusedDecodeArgs {
 // share a key head both evaluate its q/k channels; the even one writes their new
 // conv history.
 __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a) {
-    __shared__ float act[3 * kGD];      // activated q | k | v channels (bf16 values)
+    __shared__ float act_v[kGD];        // activated v channels (bf16 values)
     __shared__ float qk_n[2 * kGD];     // normalised, scaled q | k (bf16 values)
     __shared__ float y_head[kGD];       // bf16 values of the head's outputs
-    __shared__ float inverse[2];
-    __shared__ float partial[2];
+    __shared__ float wave_squares[8];   // per wave: sum of its 64 channels' squares
+    __shared__ float wave_outputs[8];   // per wave: sum of its 16 outputs' squares
     const uint32_t h = blockIdx.x;
     const uint32_t row = blockIdx.y;
     const uint32_t kh = h >> 1;
@@ -576,27 +576,36 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     const float activated = rb(conv_b * sigmoid_bf16(conv_b));
     float decay, beta;
     head_gates(gate_a, gate_b, gate_log, gate_bias, decay, beta);
+    // the output gate needs nothing but z: done here, while the state is in flight
+    const float gate_value = widen(z_bits);
+    const float gate_low = 1.0f / (1.0f + expf(fabsf(gate_value)));
+    const float gated = gate_value * (gate_value < 0.0f ? gate_low : 1.0f - gate_low);
     if (tid < 3 * kGD) {
-        act[tid] = activated;
+        if (part == 2) act_v[tid - 2 * kGD] = activated;
         if (part == 2 || (h & 1) == 0) {
             conv_out[c] = t1;
             conv_out[kCh + c] = t2;
             conv_out[2 * kCh + c] = t3;
         }
     }
-    __syncthreads();
-    if (tid < 64) {  // lanes 0..31: q head, 32..63: k head; lane l sums squares 4l..4l+3
-        const float* v = act + (tid >> 5) * kGD + (tid & 31) * 4;
-        float sum = ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3];
-        sum = half_wave_sum(sum);
-        if ((tid & 31) == 0) {
-            inverse[tid >> 5] = 1.0f / sqrtf(sum / static_cast<float>(kGD) + kRmsNormEpsilon);
-        }
-    }
+    // RMS over the q head (waves 0, 1) and the k head (waves 2, 3) without a trip through
+    // LDS per stage: a quad sums its four squares in order (slice l of gdn_prepare's lane l),
+    // then the adjacent-pairs tree over the 32 slices runs over quads (mirrors of a half row
+    // and a row: a quad holds one value), rows, the halves of the wave, and the two waves.
+    const float sq = activated * activated;
+    float slices = ((quad_lane<0>(sq) + quad_lane<1>(sq)) + quad_lane<2>(sq)) + quad_lane<3>(sq);
+    slices += lane_dpp<0x141>(slices);   // row_half_mirror: the neighbouring quad
+    slices += lane_dpp<0x140>(slices);   // row_mirror: the neighbouring pair of quads
+    slices += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(slices), 0x401F));  // lane ^ 16
+    const float wave_slices = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 0)) +
+                              __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 32));
+    if ((tid & 63) == 0) wave_squares[tid >> 6] = wave_slices;
     __syncthreads();
     if (tid < 2 * kGD) {
+        const float sum = wave_squares[(tid >> 7) * 2] + wave_squares[(tid >> 7) * 2 + 1];
+        const float inverse = 1.0f / sqrtf(sum / static_cast<float>(kGD) + kRmsNormEpsilon);
         const float scale = widen(tid < kGD ? kGdnQueryScaleBits : kGdnKeyScaleBits);
-        qk_n[tid] = rb(rb(act[tid] * inverse[tid >> 7]) * scale);
+        qk_n[tid] = rb(rb(activated * inverse) * scale);
     }
     __syncthreads();
 
@@ -623,7 +632,7 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     for (uint32_t it = 0; it < 8; ++it) kv[it] = half_wave_sum(kv[it]);
 #pragma unroll
     for (uint32_t it = 0; it < 8; ++it) {
-        const float delta = (act[2 * kGD + half * 8 + it] - kv[it]) * beta;
+        const float delta = (act_v[half * 8 + it] - kv[it]) * beta;
         out[it] = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
@@ -637,33 +646,33 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     }
 #pragma unroll
     for (uint32_t it = 0; it < 8; ++it) out[it] = half_wave_sum(out[it]);
+    // Gate-norm: every lane of a half wave holds its eight outputs, two slices of four of the
+    // RMS tree (gdn_gate_norm's lane sums four squares in order, then adjacent pairs over the
+    // 32 slices).  The first step of the tree is the half wave's own pair, the second the
+    // wave's two halves, the rest the eight waves - one value per wave through LDS.
+    float y8[8], squares[2];
+#pragma unroll
+    for (uint32_t it = 0; it < 8; ++it) y8[it] = rb(out[it]);
+#pragma unroll
+    for (uint32_t sl = 0; sl < 2; ++sl) {
+        squares[sl] = ((y8[4 * sl] * y8[4 * sl] + y8[4 * sl + 1] * y8[4 * sl + 1]) +
+                       y8[4 * sl + 2] * y8[4 * sl + 2]) + y8[4 * sl + 3] * y8[4 * sl + 3];
+    }
+    const float pair = squares[0] + squares[1];
+    const float wave_pair = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pair), 0)) +
+                            __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pair), 32));
     if (lane == 0) {
 #pragma unroll
-        for (uint32_t it = 0; it < 8; ++it) y_head[half * 8 + it] = rb(out[it]);
+        for (uint32_t it = 0; it < 8; ++it) y_head[half * 8 + it] = y8[it];
     }
+    if ((tid & 63) == 0) wave_outputs[tid >> 6] = wave_pair;
     __syncthreads();
     if (tid < kGD) {
-        const float v = y_head[tid];
-        const float sq = v * v;
-        const float s1 = quad_lane<1>(sq);
-        const float s2 = quad_lane<2>(sq);
-        const float s3 = quad_lane<3>(sq);
-        const float four = ((sq + s1) + s2) + s3;
-        const uint32_t wl = tid & 63;
-        float t = __shfl(four, (wl & 15) * 4, 64);
-        t = row_sum(t);
-        if (wl == 0) partial[tid >> 6] = t;
-    }
-    __syncthreads();
-    if (tid < kGD) {
-        const float v = y_head[tid];
-        const float inv =
-            1.0f / sqrtf((partial[0] + partial[1]) / static_cast<float>(kGD) + kRmsNormEpsilon);
-        const float normed = rb(widen(norm_bits) * rb(v * inv));
-        const float g = widen(z_bits);
-        const float low = 1.0f / (1.0f + expf(fabsf(g)));
-        const float sig = g < 0.0f ? low : 1.0f - low;
-        a.out[static_cast<uint64_t>(row) * a.out_stride + h * kGD + tid] = narrow((g * sig) * normed);
+        const float total = ((wave_outputs[0] + wave_outputs[1]) + (wave_outputs[2] + wave_outputs[3])) +
+                            ((wave_outputs[4] + wave_outputs[5]) + (wave_outputs[6] + wave_outputs[7]));
+        const float inv = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
+        const float normed = rb(widen(norm_bits) * rb(y_head[tid] * inv));
+        a.out[static_cast<uint64_t>(row) * a.out_stride + h * kGD + tid] = narrow(gated * normed);
     }
 }
 
