@@ -71,6 +71,30 @@ struct Q4Projection {
     uint64_t residual_stride;              //   [rows][residual_stride]; may be the output itself
 };
 
+// The weight matrix that holds output row `n`, with n the same for every lane (matrices have
+// multiples of 16 rows, so a workgroup's 8 or 16 rows share one): the operands are picked with
+// selects on scalar registers.  Indexing the argument arrays with a per-lane value instead
+// turns into vector loads from the argument block - a round trip to memory before the
+// first weight can be requested.
+struct Q4Matrix {
+    const uint32_t* words;
+    const uint16_t* scales;
+    const uint16_t* biases;
+    uint32_t first_row;
+};
+__device__ __forceinline__ Q4Matrix matrix_of_row(const Q4Projection& p, uint32_t n) {
+    Q4Matrix m{p.words[0], p.scales[0], p.biases[0], 0};
+#pragma unroll
+    for (uint32_t s = 1; s < kMaxSegments; ++s) {
+        const bool here = s < p.segments && n >= p.first_row[s];
+        m.words = here ? p.words[s] : m.words;
+        m.scales = here ? p.scales[s] : m.scales;
+        m.biases = here ? p.biases[s] : m.biases;
+        m.first_row = here ? p.first_row[s] : m.first_row;
+    }
+    return m;
+}
+
 // grid (ceil(out_rows / 8), ceil(rows / row_tile)) x 256: half wave h of a workgroup
 // owns output row 8 * blockIdx.x + h for the tile's input rows.  kBlocks = k_size / 512:
 // all of the row's nibbles, scales and biases are requested before the first is used, so
@@ -99,12 +123,11 @@ __global__ __launch_bounds__(256) void q4_rows_kernel(Q4Projection p) {
     // rows past the last one compute on the last row and store nothing
     const uint32_t n = min(blockIdx.x * 8 + (threadIdx.x >> 5), p.first_row[p.segments] - 1);
     const bool stores = blockIdx.x * 8 + (threadIdx.x >> 5) < p.first_row[p.segments];
-    uint32_t segment = 0;
-    while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
-    const uint32_t local = n - p.first_row[segment];
-    const uint32_t* words = p.words[segment] + static_cast<uint64_t>(local) * (kBlocks * 64);
-    const uint16_t* scales = p.scales[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
-    const uint16_t* biases = p.biases[segment] + static_cast<uint64_t>(local) * (kBlocks * 8);
+    const Q4Matrix matrix = matrix_of_row(p, min(blockIdx.x * 8, p.first_row[p.segments] - 1));
+    const uint32_t local = n - matrix.first_row;
+    const uint32_t* words = matrix.words + static_cast<uint64_t>(local) * (kBlocks * 64);
+    const uint16_t* scales = matrix.scales + static_cast<uint64_t>(local) * (kBlocks * 8);
+    const uint16_t* biases = matrix.biases + static_cast<uint64_t>(local) * (kBlocks * 8);
 
     u32x2 packed[kBlocks];
     uint16_t scale_bits[kBlocks], bias_bits[kBlocks];
@@ -676,13 +699,12 @@ __global__ __launch_bounds__(64 * kWaves) void q4_wave_kernel(Q4Projection p) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t i16 = lane & 15, g = lane >> 4;
     const uint32_t n = blockIdx.x * 16 + i16;   // every matrix has a multiple of 16 rows
-    uint32_t segment = 0;
-    while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
-    const uint64_t local = n - p.first_row[segment];
+    const Q4Matrix matrix = matrix_of_row(p, blockIdx.x * 16);
+    const uint64_t local = n - matrix.first_row;
     const uint32_t first_group = wave * 8;
-    const uint32_t* words = p.words[segment] + local * (kWaves * 64) + first_group * 8 + 2 * g;
-    const uint16_t* scales = p.scales[segment] + local * (kWaves * 8) + first_group;
-    const uint16_t* biases = p.biases[segment] + local * (kWaves * 8) + first_group;
+    const uint32_t* words = matrix.words + local * (kWaves * 64) + first_group * 8 + 2 * g;
+    const uint16_t* scales = matrix.scales + local * (kWaves * 8) + first_group;
+    const uint16_t* biases = matrix.biases + local * (kWaves * 8) + first_group;
 
     // The x rows are the same for every workgroup: they come in once with coalesced 16-byte
     // loads (requested first, so that storing them does not wait for the weights) and are
