@@ -2101,6 +2101,10 @@ extern "C" int32_t tt_attention_decode_lanes_static(
     f.query_stride = query_stride;
     f.partial_row_floats = row_floats;
     f.single_partition = kAttnPartition;
+    // a grid larger than the chip may hold workgroups without keys: the ones with keys first
+    // (the contexts are on the device, so this cannot be decided more finely here)
+    f.compact = static_cast<uint64_t>(splits) * kAttnKvHeads * rows > 256 &&
+                reinterpret_cast<uintptr_t>(state_table) % 8 == 0;
     launch_flash(f, splits, rows, stream);
 
     CombineArgs c{};

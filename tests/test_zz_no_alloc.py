@@ -79,6 +79,11 @@ def test_static_scratch_entry_point_two_calls_in_a_row():
     _call_and_check(queue, large, "first call")
     _call_and_check(queue, small, "second call (smaller)")
     _call_and_check(queue, large, "third call (large again)")
+    # a grid larger than the chip (128 splits x 2 x 3 workgroups, most of them without keys):
+    # the entry point then places the workgroups that hold keys first; same records, same bits
+    print("[case] no-alloc entry: 3 lanes cap 4096 part 32", flush=True)
+    fine = _case([4095, 2500, 100], 4096, 32, 0x2A04)
+    _call_and_check(queue, fine, "fourth call (grid larger than the chip)")
 
 
 def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
