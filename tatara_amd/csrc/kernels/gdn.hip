@@ -518,16 +518,24 @@ struct FusedDecodeArgs {
 // head's 128 x 128 state and the gate-norm of its 128 outputs, with the
 // arithmetic of gdn_prepare / gdn_recurrence / gdn_gate_norm operation for
 // operation (so the results are theirs bit for bit) and none of their
-// intermediates in memory.  grid (32 heads, rows) x 512: sixteen half waves, each
+// intermediates in memory.  grid (32 heads, rows) x kFusedThreads: sixteen half waves, each
 // walking 8 state rows with 4 key columns per lane.  The two value heads that
 // share a key head both evaluate its q/k channels; the even one writes their new
 // conv history.
-__global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a) {
+// 512 threads: sixteen half waves of eight state rows.  1024 (four rows each) measured 0.2 us
+// slower - more waves to start and to meet at the barriers than the shorter row loop wins.
+constexpr uint32_t kFusedThreads = 512;
+
+template <uint32_t kThreads>
+__global__ __launch_bounds__(kThreads) void gdn_decode_fused_kernel(FusedDecodeArgs a) {
+    constexpr uint32_t kWavesHere = kThreads / 64;
+    constexpr uint32_t kRowsEach = kGD / (kThreads / 32);   // state rows a half wave walks
+    static_assert(kThreads >= 3 * kGD && (kRowsEach == 4 || kRowsEach == 8), "one thread per q, k, v channel; whole slices per half wave");
     __shared__ float act_v[kGD];        // activated v channels (bf16 values)
     __shared__ float qk_n[2 * kGD];     // normalised, scaled q | k (bf16 values)
     __shared__ float y_head[kGD];       // bf16 values of the head's outputs
-    __shared__ float wave_squares[8];   // per wave: sum of its 64 channels' squares
-    __shared__ float wave_outputs[8];   // per wave: sum of its 16 outputs' squares
+    __shared__ float wave_squares[kWavesHere];   // per wave: sum of its 64 channels' squares
+    __shared__ float wave_outputs[kWavesHere];   // per wave: sum of its outputs' squares
     const uint32_t h = blockIdx.x;
     const uint32_t row = blockIdx.y;
     const uint32_t kh = h >> 1;
@@ -537,7 +545,7 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     uint16_t* conv_out = a.conv_pool_out + a.table[row * 4 + 1];
     const float* state_in = a.rec_pool + a.table[row * 4 + 2];
     float* state_out = a.rec_pool_out + a.table[row * 4 + 3];
-    const uint32_t half = tid >> 5;  // 0..15
+    const uint32_t half = tid >> 5;
     const uint32_t lane = tid & 31;
     // Loads come back in the order they were requested.  The few bytes the conv, norm and
     // gate stages need go out first, the head's 64 KiB of state right behind them: those
@@ -560,10 +568,10 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     const uint16_t gate_b = proj[kGdnBRowOffset + h];
     const uint16_t gate_log = a.a_log[h];
     const uint16_t gate_bias = a.dt_bias[h];
-    f32x4 st[8];
+    f32x4 st[kRowsEach];
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) {
-        const uint32_t j = half * 8 + it;
+    for (uint32_t it = 0; it < kRowsEach; ++it) {
+        const uint32_t j = half * kRowsEach + it;
         st[it] = *reinterpret_cast<const f32x4*>(
             state_in + (static_cast<uint64_t>(h) * kGD + j) * kGD + lane * 4);
     }
@@ -618,9 +626,9 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
     // The eight rows of a half wave go through each step side by side, not row after row:
     // a row's two cross-lane sums are chains of dependent lane exchanges (the last through the
     // LDS crossbar), and eight independent chains fill each other's waits.
-    float kv[8], out[8];
+    float kv[kRowsEach], out[kRowsEach];
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) {
+    for (uint32_t it = 0; it < kRowsEach; ++it) {
         kv[it] = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
@@ -629,10 +637,10 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
         }
     }
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) kv[it] = half_wave_sum(kv[it]);
+    for (uint32_t it = 0; it < kRowsEach; ++it) kv[it] = half_wave_sum(kv[it]);
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) {
-        const float delta = (act_v[half * 8 + it] - kv[it]) * beta;
+    for (uint32_t it = 0; it < kRowsEach; ++it) {
+        const float delta = (act_v[half * kRowsEach + it] - kv[it]) * beta;
         out[it] = 0.0f;
 #pragma unroll
         for (uint32_t i = 0; i < 4; ++i) {
@@ -642,34 +650,41 @@ __global__ __launch_bounds__(512) void gdn_decode_fused_kernel(FusedDecodeArgs a
         // written once, read by the next token's dispatch at the earliest: stored past the
         // cache (nontemporal), so the dispatch does not end on a write-back of the whole state
         __builtin_nontemporal_store(st[it], reinterpret_cast<f32x4*>(
-            state_out + (static_cast<uint64_t>(h) * kGD + half * 8 + it) * kGD + lane * 4));
+            state_out + (static_cast<uint64_t>(h) * kGD + half * kRowsEach + it) * kGD + lane * 4));
     }
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) out[it] = half_wave_sum(out[it]);
+    for (uint32_t it = 0; it < kRowsEach; ++it) out[it] = half_wave_sum(out[it]);
     // Gate-norm: every lane of a half wave holds its eight outputs, two slices of four of the
     // RMS tree (gdn_gate_norm's lane sums four squares in order, then adjacent pairs over the
     // 32 slices).  The first step of the tree is the half wave's own pair, the second the
     // wave's two halves, the rest the eight waves - one value per wave through LDS.
-    float y8[8], squares[2];
+    float y8[kRowsEach], squares[kRowsEach / 4];
 #pragma unroll
-    for (uint32_t it = 0; it < 8; ++it) y8[it] = rb(out[it]);
+    for (uint32_t it = 0; it < kRowsEach; ++it) y8[it] = rb(out[it]);
 #pragma unroll
-    for (uint32_t sl = 0; sl < 2; ++sl) {
+    for (uint32_t sl = 0; sl < kRowsEach / 4; ++sl) {
         squares[sl] = ((y8[4 * sl] * y8[4 * sl] + y8[4 * sl + 1] * y8[4 * sl + 1]) +
                        y8[4 * sl + 2] * y8[4 * sl + 2]) + y8[4 * sl + 3] * y8[4 * sl + 3];
     }
-    const float pair = squares[0] + squares[1];
+    const float pair = kRowsEach == 8 ? squares[0] + squares[kRowsEach / 4 - 1] : squares[0];
     const float wave_pair = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pair), 0)) +
                             __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pair), 32));
     if (lane == 0) {
 #pragma unroll
-        for (uint32_t it = 0; it < 8; ++it) y_head[half * 8 + it] = y8[it];
+        for (uint32_t it = 0; it < kRowsEach; ++it) y_head[half * kRowsEach + it] = y8[it];
     }
     if ((tid & 63) == 0) wave_outputs[tid >> 6] = wave_pair;
     __syncthreads();
     if (tid < kGD) {
-        const float total = ((wave_outputs[0] + wave_outputs[1]) + (wave_outputs[2] + wave_outputs[3])) +
-                            ((wave_outputs[4] + wave_outputs[5]) + (wave_outputs[6] + wave_outputs[7]));
+        float level[kWavesHere];
+#pragma unroll
+        for (uint32_t w = 0; w < kWavesHere; ++w) level[w] = wave_outputs[w];
+#pragma unroll
+        for (uint32_t width = kWavesHere; width > 1; width >>= 1) {   // adjacent pairs, level by level
+#pragma unroll
+            for (uint32_t w = 0; w < width / 2; ++w) level[w] = level[2 * w] + level[2 * w + 1];
+        }
+        const float total = level[0];
         const float inv = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
         const float normed = rb(widen(norm_bits) * rb(y_head[tid] * inv));
         a.out[static_cast<uint64_t>(row) * a.out_stride + h * kGD + tid] = narrow(gated * normed);
@@ -1614,7 +1629,7 @@ int32_t op_gdn_decode_fused_ms(const Bindings& b, const Grid& g, hipStream_t str
     f.out = a.buffer<uint16_t>(7, (last * f.out_stride + kGdnValueValues) * 2);
     f.table = a.buffer<const uint32_t>(8, rows * 16);
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(gdn_decode_fused_kernel, dim3(kGdnValueHeads, rows), dim3(512), 0, stream, f);
+    hipLaunchKernelGGL(gdn_decode_fused_kernel<kFusedThreads>, dim3(kGdnValueHeads, rows), dim3(kFusedThreads), 0, stream, f);
     return TT_OK;
 }
 
