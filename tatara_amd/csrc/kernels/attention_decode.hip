@@ -100,12 +100,11 @@ struct RopeArgs {
 };
 
 // grid (18, ceil(rows / rows_per_group)) x 256: one head per workgroup, one
-// dimension per thread.  Sum of squares: 64 threads x 4 values, a 32-lane
-// adjacent-pairs tree per half-wave, then the two halves added
-// (attention.metal:63-88).
+// dimension per thread.  Sum of squares as the reference takes it: 64 slices of 4
+// values summed in order, a 32-slice adjacent-pairs tree per half, then the two
+// halves added (attention.metal:63-88).
 __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
-    __shared__ float normed[kD];
-    __shared__ float inverse_shared;
+    __shared__ float wave_squares[4];
     const uint32_t head = blockIdx.x;
     const uint32_t d = threadIdx.x;
     const bool is_query = head < kAttnQueryHeads;
@@ -139,31 +138,29 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
             const float theta = static_cast<float>(position) / inverse_frequency;
             sincosf(theta, &s, &c);   // one argument reduction for both
         }
+        // Sum of squares in registers: a quad sums its four squares in order (thread q of the
+        // reference's 64), then the adjacent-pairs tree over the 64 slices runs over quads
+        // (mirrors of a half row and of a row: a quad holds one value), rows, the halves of
+        // the wave, and the four waves - one value per wave through LDS, one barrier.
+        const float sq = x * x;
+        float slices = ((quad_lane<0>(sq) + quad_lane<1>(sq)) + quad_lane<2>(sq)) + quad_lane<3>(sq);
+        slices += lane_dpp<0x141>(slices);   // row_half_mirror: the neighbouring quad
+        slices += lane_dpp<0x140>(slices);   // row_mirror: the neighbouring pair of quads
+        slices += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(slices), 0x401F));  // lane ^ 16
+        const float wave_slices = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 0)) +
+                                  __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 32));
         __syncthreads();  // the previous row's readers are done with the shared values
-        normed[d] = x;    // the head's values pass through LDS: no second trip to memory
+        if ((d & 63) == 0) wave_squares[d >> 6] = wave_slices;
         __syncthreads();
-        if (d < 64) {
-            float acc = 0.0f;
-            for (uint32_t j = 0; j < 4; ++j) {
-                const float v = normed[d * 4 + j];
-                acc += v * v;
-            }
-            acc = half_wave_sum(acc);
-            const float total = acc + __shfl_xor(acc, 32, 64);
-            if (d == 0) {
-                inverse_shared = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
-            }
-        }
-        __syncthreads();
-        const float inverse = inverse_shared;
+        const float total = (wave_squares[0] + wave_squares[1]) + (wave_squares[2] + wave_squares[3]);
+        const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
         // w * bf16(x * inv), the product rounded to bf16 again
         const float n = round_bf16(weight * round_bf16(x * inverse));
-        normed[d] = n;
-        __syncthreads();
+        // the rotation's partner dimension sits 32 lanes away in the same wave
+        const float partner = __shfl_xor(n, static_cast<int>(kAttnRopePairs), 64);
         float rotated = n;
         if (d < 2 * kAttnRopePairs) {
-            rotated = d < kAttnRopePairs ? fmaf(-normed[d + kAttnRopePairs], s, n * c)
-                                         : fmaf(normed[d - kAttnRopePairs], s, n * c);
+            rotated = d < kAttnRopePairs ? fmaf(-partner, s, n * c) : fmaf(partner, s, n * c);
         }
         const uint16_t stored = f32_to_bf16_bits(rotated);
         if (is_query) {
