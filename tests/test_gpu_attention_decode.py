@@ -292,6 +292,58 @@ def test_lane_batch_compact_dispatch_order(contexts, cap, part, interleave):
     assert np.array_equal(outputs[0], outputs[1])
 
 
+def test_compact_walk_compiled_once_replayed_while_contexts_grow():
+    """One compiled split + combine, replayed after the state table has moved on: the rows'
+    split counts change under the same grid (a row crosses a split boundary, a short row
+    becomes a split-path row, a row's split count shrinks to zero when its lane is reset), and
+    the workgroup placement has to follow from the table alone."""
+    print("[case] compact walk, one graph, moving contexts", flush=True)
+    B, dev, queue, lib = gpu()
+    cap, part, rows = 2048, 128, 4
+    stripe = 2 * cap * 256
+    k_pool, stride = dev.create_pool(stripe * 2, rows)
+    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    q = np.stack([ol.gaussian_bf16(0x6A01 + r, 4096) for r in range(rows)])
+    gate = np.stack([ol.gaussian_bf16(0x6B01 + r, 4096) for r in range(rows)])
+    keys = [ol.gaussian_bf16(0x6C01 + r, stripe).reshape(2, cap, 256) for r in range(rows)]
+    values = [ol.gaussian_bf16(0x6D01 + r, stripe).reshape(2, cap, 256) for r in range(rows)]
+    for r in range(rows):
+        k_pool.write(keys[r], r * stride)
+        v_pool.write(values[r], r * stride)
+    b_q, b_g = dev.buffer_from(q), dev.buffer_from(gate)
+    b_o = dev.create_buffer(rows * 8192)
+    max_splits = cap // part
+    b_part = dev.create_buffer(rows * 16 * max_splits * 258 * 4)
+    b_tab = dev.create_buffer(256)
+    cb = queue.create_command_buffer()
+    cb.begin_compute_pass()
+    cb.encode(lib.pipeline("attention_decode_split_ms"),
+              {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
+              {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 4}, (max_splits, 2, rows), (256,))
+    cb.barrier()
+    cb.encode(lib.pipeline("attention_decode_combine_ms"),
+              {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0},
+              (16, rows), (256,))
+    cb.end_compute_pass()
+    cb.compile()
+    for contexts in ([255, 126, 2047, 600], [256, 127, 2047, 601], [257, 128, 0, 602],
+                     [383, 1000, 1, 639], [384, 1001, 2, 640]):
+        table = np.zeros(64, np.uint32)
+        for r, ctx in enumerate(contexts):
+            table[r * 4] = r * (stride // 2)
+            table[r * 4 + 1] = ctx
+        b_tab.write(table)
+        b_o.write(np.zeros(rows * 4096, np.uint16))
+        b_part.write(np.full(rows * 16 * max_splits * 258, np.nan, np.float32))
+        cb.commit().wait()
+        got = b_o.read(np.uint16).reshape(rows, 4096)
+        for r, ctx in enumerate(contexts):
+            want = np.zeros(4096, np.uint16)
+            o.tto_attention_decode_split(q[r], gate[r], keys[r].reshape(-1), values[r].reshape(-1),
+                                         ctx, cap, 256, None, want, 4)
+            check_bf16(got[r], want, f"contexts {contexts} lane {r}")
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
