@@ -344,6 +344,115 @@ def test_compact_walk_compiled_once_replayed_while_contexts_grow():
             check_bf16(got[r], want, f"contexts {contexts} lane {r}")
 
 
+@pytest.mark.parametrize("compact", [False, True], ids=["grid-order", "keyed-first"])
+def test_table_rows_past_the_capacity_are_left_alone(compact):
+    """A state-table row whose context is not a cache position (the capacity itself, or far
+    past it) must neither be read nor written for: its output keeps what it held, the rows
+    around it come out as always."""
+    print(f"[case] lane batch with table rows past the capacity, compact={compact}", flush=True)
+    B, dev, queue, lib = gpu()
+    cap, part, rows = 1024, 128, 4
+    stripe = 2 * cap * 256
+    k_pool, stride = dev.create_pool(stripe * 2, rows)
+    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    contexts = [700, cap, 300, cap + 4000]          # rows 1 and 3 are not cache positions
+    q = np.stack([ol.gaussian_bf16(0x7A01 + r, 4096) for r in range(rows)])
+    gate = np.stack([ol.gaussian_bf16(0x7B01 + r, 4096) for r in range(rows)])
+    keys = [ol.gaussian_bf16(0x7C01 + r, stripe) for r in range(rows)]
+    values = [ol.gaussian_bf16(0x7D01 + r, stripe) for r in range(rows)]
+    table = np.zeros(64, np.uint32)
+    for r in range(rows):
+        k_pool.write(keys[r], r * stride)
+        v_pool.write(values[r], r * stride)
+        table[r * 4] = r * (stride // 2)
+        table[r * 4 + 1] = contexts[r]
+    b_tab, b_q, b_g = dev.buffer_from(table), dev.buffer_from(q), dev.buffer_from(gate)
+    sentinel = np.full(rows * 4096, 0x4321, np.uint16)
+    b_o = dev.buffer_from(sentinel)
+    max_splits = cap // part
+    b_part = dev.buffer_from(np.full(rows * 16 * max_splits * 258, np.nan, np.float32))
+
+    def rec(cb):
+        cb.encode(lib.pipeline("attention_decode_split_ms"),
+                  {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
+                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 4 * int(compact)},
+                  (max_splits, 2, rows), (256,))
+        cb.barrier()
+        cb.encode(lib.pipeline("attention_decode_combine_ms"),
+                  {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0},
+                  (16, rows), (256,))
+    run(rec)
+    got = b_o.read(np.uint16).reshape(rows, 4096)
+    records = b_part.read(np.float32).reshape(rows, -1)
+    for r, ctx in enumerate(contexts):
+        if ctx >= cap:
+            assert np.isnan(records[r]).all(), f"row {r}: records written for a context past the capacity"
+            if ctx >= max_splits * part:
+                assert (got[r] == 0x4321).all(), f"row {r}: output written"
+            continue
+        want = np.zeros(4096, np.uint16)
+        o.tto_attention_decode_split(q[r], gate[r], keys[r], values[r], ctx, cap, 256, None, want, 4)
+        check_bf16(got[r], want, f"lane {r} ctx {ctx} beside rows past the capacity")
+
+
+def test_qk_rope_of_a_token_wave_on_striped_pools():
+    """attn_qk_rope_ms: every row of a wave normed, rotated at its own position and appended
+    to its own lane's stripe; a row whose context is not a cache position is skipped whole."""
+    print("[case] attn_qk_rope_ms, 5 rows on reversed stripes, one row past the capacity", flush=True)
+    B, dev, queue, lib = gpu()
+    cap, rows = 512, 5
+    contexts = [0, 511, 17, cap, 300]               # row 3 is not a cache position
+    stripes = [4, 3, 2, 1, 0]
+    q_w, k_w = _weights()
+    stripe = 2 * cap * 256
+    k_pool, stride = dev.create_pool(stripe * 2, rows)
+    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    old_k = np.full(rows * (stride // 2), 0x1111, np.uint16)
+    old_v = np.full(rows * (stride // 2), 0x2222, np.uint16)
+    k_pool.write(old_k); v_pool.write(old_v)
+    proj = np.stack([ol.gaussian_bf16(0x8A01 + r, 9216) for r in range(rows)])
+    table = np.zeros(64, np.uint32)
+    for r in range(rows):
+        table[r * 4] = stripes[r] * (stride // 2)
+        table[r * 4 + 1] = contexts[r]
+    b_proj, b_tab = dev.buffer_from(proj), dev.buffer_from(table)
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q = dev.buffer_from(np.full(rows * 4096, 0x3333, np.uint16))
+    b_g = dev.buffer_from(np.full(rows * 4096, 0x4444, np.uint16))
+
+    def rec(cb):
+        cb.encode(lib.pipeline("attn_qk_rope_ms"),
+                  {0: b_proj, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: k_pool, 6: v_pool, 8: b_tab},
+                  {7: cap, 9: 9216, 10: 4096}, (18, rows), (256,))
+    run(rec)
+    got_q = b_q.read(np.uint16).reshape(rows, 4096)
+    got_g = b_g.read(np.uint16).reshape(rows, 4096)
+    got_k = k_pool.read(np.uint16).reshape(rows, stride // 2)
+    got_v = v_pool.read(np.uint16).reshape(rows, stride // 2)
+    want_k = old_k.reshape(rows, -1).copy(); want_v = old_v.reshape(rows, -1).copy()
+    for r, ctx in enumerate(contexts):
+        if ctx >= cap:
+            assert (got_q[r] == 0x3333).all() and (got_g[r] == 0x4444).all()
+            continue
+        q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16)
+        lane_k = want_k[stripes[r], :stripe].copy(); lane_v = want_v[stripes[r], :stripe].copy()
+        o.tto_attn_qk_rope(proj[r], q_w, k_w, ctx, cap, q, gate, lane_k, lane_v)
+        want_k[stripes[r], :stripe] = lane_k; want_v[stripes[r], :stripe] = lane_v
+        assert np.array_equal(got_g[r], gate)                              # raw copy: exact
+        check_bf16(got_q[r], q, f"row {r} q at position {ctx}", ulps=1)
+        assert np.mean(got_q[r] == q) > 0.99
+    assert np.array_equal(got_v, want_v)                                   # raw copies, slots: exact
+    # K: the appended rows within a bf16 step, every other element of every stripe untouched
+    changed = got_k != want_k
+    rope_rows = np.zeros_like(changed)
+    for r, ctx in enumerate(contexts):
+        if ctx < cap:
+            for head in range(2):
+                rope_rows[stripes[r], (head * cap + ctx) * 256:(head * cap + ctx + 1) * 256] = True
+    assert not (changed & ~rope_rows).any()
+    check_bf16(got_k[rope_rows], want_k[rope_rows], "appended K rows", ulps=1)
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
