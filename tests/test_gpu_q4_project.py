@@ -74,8 +74,9 @@ def test_single_row_projection_bit_for_bit(family):
 
 
 @pytest.mark.parametrize("rows,tile", [(1, 16), (3, 2), (16, 16), (13, 5)])
-@pytest.mark.parametrize("family,suffix", [(ATTN, "_ms"), (GDN, "_ms_v2"), (OUT, "_ms")],
-                         ids=["attn", "gdn_v2", "out"])
+@pytest.mark.parametrize("family,suffix", [(ATTN, "_ms"), (ATTN, "_ms_v2"), (GDN, "_ms"),
+                                           (GDN, "_ms_v2"), (OUT, "_ms"), (OUT, "_ms_v2")],
+                         ids=["attn", "attn_v2", "gdn", "gdn_v2", "out", "out_v2"])
 def test_wave_projection_bit_for_bit(family, suffix, rows, tile):
     name = family["name"] + suffix
     print(f"[case] {name} rows={rows} tile={tile}", flush=True)
