@@ -40,13 +40,31 @@ __device__ __forceinline__ uint16_t narrow(float v) {
     if ((b & 0x7F800000u) == 0x7F800000u) return static_cast<uint16_t>(b >> 16);
     return static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
 }
-// one bf16 arithmetic step: operate in fp32, round the result to bf16
-__device__ __forceinline__ float rb(float v) { return widen(narrow(v)); }
+// one bf16 arithmetic step: operate in fp32, round the result to bf16 (narrow, widened
+// again: the carry of the rounding add runs into the exponent as it should, infinities stay,
+// NaNs keep their upper bits)
+__device__ __forceinline__ float rb(float v) {
+    const uint32_t b = __float_as_uint(v);
+    const uint32_t rounded = (b + 0x7FFFu + ((b >> 16) & 1u)) & 0xFFFF0000u;
+    return __uint_as_float(v != v ? (b & 0xFFFF0000u) : rounded);
+}
+
+// bf16(1 / d) for a bf16 value d.  The reciprocal instruction is within one fp32 ulp of the
+// quotient, and that is enough to round like the quotient itself: with d = D 2^a (D an
+// 8-bit integer) and a midpoint between bf16 neighbours M = (2K + 1) 2^b, 1 - d M is a
+// multiple of 2^-17 and not zero unless d is a power of two (where the instruction is
+// exact), so 1 / d stays 2^-17 of its own size away from every midpoint.  Outside the range
+// where the instruction keeps full precision the division is taken.
+__device__ __forceinline__ float rb_reciprocal(float d) {
+    const float size = fabsf(d);
+    if (!(size >= 0x1p-100f && size <= 0x1p+100f)) return rb(1.0f / d);
+    return rb(__builtin_amdgcn_rcpf(d));
+}
 
 // sigmoid in bf16 steps with the |x| branch (gdn.metal:76-79)
 __device__ __forceinline__ float sigmoid_bf16(float x) {
     const float e = rb(expf(fabsf(x)));
-    const float low = rb(1.0f / rb(1.0f + e));
+    const float low = rb_reciprocal(rb(1.0f + e));
     return x < 0.0f ? low : rb(1.0f - low);
 }
 

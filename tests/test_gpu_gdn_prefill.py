@@ -145,6 +145,49 @@ def test_element_wise_block_kernels_bit_for_bit(rows):
     assert np.array_equal(bufs["gated"].read(np.uint16), ref["gated"])
 
 
+def test_activation_of_every_bf16_value_bit_for_bit():
+    """conv + SiLU of all 65536 bf16 bit patterns (the non-finite ones replaced by zero):
+    16 rows whose 4096 value channels carry the patterns, taps (0, 0, 0, 1) and an empty
+    window, so a channel's convolution is its input.  Pins the kernels' bf16 rounding step
+    and their reciprocal-instruction sigmoid to the checker's division over the whole
+    range, not only where random inputs fall."""
+    rows = 16
+    print("[case] gdn conv + SiLU over every bf16 value", flush=True)
+    B, dev, queue, lib = gpu()
+    _, a_log, dt_bias, norm_w = _weights()
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    patterns[(patterns & 0x7F80) == 0x7F80] = 0
+    proj = np.zeros((rows, 12352), np.uint16)
+    proj[:, 4096:8192] = patterns.reshape(rows, 4096)
+    conv_w = np.zeros((8192, 4), np.uint16)
+    conv_w[:, 3] = 0x3F80
+    weights = (conv_w.reshape(-1), a_log, dt_bias, norm_w)
+    conv_state = np.zeros(3 * 8192, np.uint16)
+    state = np.zeros(STATE, np.float32)
+    ref = _oracle_block(proj, conv_state, state, weights, rows)
+    bufs = _buffers(dev, proj, conv_state, state, weights, rows)
+    run(lambda cb: _encode_front(cb, lib, bufs, rows))
+    got = bufs["value"].read(np.uint16)
+    differ = np.flatnonzero(got != ref["value"])
+    assert differ.size == 0, (f"{differ.size} of 65536 activations differ, first: input "
+                              f"{patterns[differ[0]]:#06x} got {got[differ[0]]:#06x} "
+                              f"want {ref['value'][differ[0]]:#06x}")
+    assert np.array_equal(bufs["conv_out"].read(np.uint16), ref["conv"])
+    # the decode operator on the last row's window: the same activations bit for bit
+    last = rows - 1
+    b_qk, b_v, b_z = (dev.create_buffer(8192) for _ in range(3))
+    b_conv_in = dev.buffer_from(np.concatenate([proj[last - 3 + t, :8192] for t in range(3)]))
+    b_conv_out = dev.create_buffer(3 * 8192 * 2)
+    b_row = dev.buffer_from(proj[last])
+
+    def rec(cb):
+        cb.encode(lib.pipeline("gdn_prepare"),
+                  {0: b_row, 1: b_conv_in, 2: bufs["conv_w"], 3: b_qk, 4: b_v, 5: b_z,
+                   6: b_conv_out}, {}, (96,), (128,))
+    run(rec)
+    assert np.array_equal(b_v.read(np.uint16), ref["value"].reshape(rows, 4096)[last])
+
+
 def _encode_chunked(cb, lib, bufs, rows, state_in="state_in", state_out="state_out"):
     chunks = (rows + 63) // 64
     cb.encode(lib.pipeline("gdn_chunk_prepare_blk"),
