@@ -188,6 +188,38 @@ def test_activation_of_every_bf16_value_bit_for_bit():
     assert np.array_equal(b_v.read(np.uint16), ref["value"].reshape(rows, 4096)[last])
 
 
+def test_output_gate_of_every_bf16_value_bit_for_bit():
+    """The gate-norm's SiLU(z) over all 65536 bf16 bit patterns of z (non-finite ones replaced
+    by zero) on rows of seeded y: the fp32 sigmoid with its |z| branch, the product and the
+    final rounding against the checker, for the block operator and the decode operator."""
+    rows = 16
+    print("[case] gdn gate-norm over every bf16 gate value", flush=True)
+    B, dev, queue, lib = gpu()
+    _, _, _, norm_w = _weights()
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    patterns[(patterns & 0x7F80) == 0x7F80] = 0
+    z = patterns.reshape(rows, 4096)
+    y = ol.gaussian_bf16(0x6E01, rows * 4096).reshape(rows, 4096)
+    want = np.zeros((rows, 4096), np.uint16)
+    for r in range(rows):
+        o.tto_gdn_gate_norm(y[r], z[r], norm_w, 32, want[r])
+    b_y, b_z, b_w = dev.buffer_from(y), dev.buffer_from(z), dev.buffer_from(norm_w)
+    b_blk, b_one = dev.create_buffer(rows * 8192), dev.create_buffer(8192)
+
+    def rec(cb):
+        cb.encode(lib.pipeline("gdn_gate_norm_blk"), {0: b_y, 1: b_z, 2: b_w, 3: b_blk}, {},
+                  (32, rows, 1), (128, 1, 1))
+        cb.encode(lib.pipeline("gdn_gate_norm"), {0: (b_y, 5 * 8192), 1: (b_z, 5 * 8192), 2: b_w,
+                                                  3: b_one}, {}, (32,), (128,))
+    run(rec)
+    got = b_blk.read(np.uint16).reshape(rows, 4096)
+    differ = np.argwhere(got != want)
+    assert differ.size == 0, (f"{len(differ)} of 65536 gated outputs differ, first: z "
+                              f"{z[tuple(differ[0])]:#06x} got {got[tuple(differ[0])]:#06x} "
+                              f"want {want[tuple(differ[0])]:#06x}")
+    assert np.array_equal(b_one.read(np.uint16), want[5])
+
+
 def _encode_chunked(cb, lib, bufs, rows, state_in="state_in", state_out="state_out"):
     chunks = (rows + 63) // 64
     cb.encode(lib.pipeline("gdn_chunk_prepare_blk"),
