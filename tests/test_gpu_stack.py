@@ -231,6 +231,48 @@ def test_rms_only_operators_bit_for_bit(rows, hidden):
     assert not got[:, hidden:].any()                             # nothing written past a row
 
 
+def test_norm_and_residual_sum_over_every_bf16_value():
+    """rms_only_ms, residual_rms_ms and add_bf16 on all 65536 bf16 bit patterns (non-finite
+    ones replaced by zero), ordered by magnitude so that a row of 2048 holds neighbouring
+    binades: rows of subnormals (flushed on the way in), rows that round into and out of the
+    subnormal range, rows whose squares overflow."""
+    print("[case] rms_only_ms / residual_rms_ms / add_bf16 over every bf16 value", flush=True)
+    B, dev, queue, lib = gpu()
+    hidden, rows = 2048, 32
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    patterns[(patterns & 0x7F80) == 0x7F80] = 0
+    order = np.argsort(patterns & 0x7FFF, kind="stable")
+    x = np.ascontiguousarray(patterns[order])
+    # the second operand: the same magnitudes one binade away and in another order of signs
+    other = np.ascontiguousarray(np.roll(x, 193) ^ np.uint16(0x8000))
+    w = ol.f32_to_bf16(1.0 + 0.1 * ol.gaussian_f32(0xE2, hidden))
+    want_norm = np.zeros(rows * hidden, np.uint16)
+    o.tto_rms_only(x, w, rows, hidden, want_norm)
+    sums = np.zeros(rows * hidden, np.uint16)
+    o.tto_add_bf16(x, other, rows * hidden, sums)
+    want_sum_norm = np.zeros(rows * hidden, np.uint16)
+    o.tto_rms_only(sums, w, rows, hidden, want_sum_norm)
+    b_x, b_y, b_w = dev.buffer_from(x), dev.buffer_from(other), dev.buffer_from(w)
+    b_norm, b_res, b_res_norm, b_add = (dev.create_buffer(rows * hidden * 2) for _ in range(4))
+
+    def rec(cb):
+        cb.encode(lib.pipeline("rms_only_ms"), {0: b_x, 1: b_w, 2: b_norm}, {3: hidden, 4: hidden},
+                  (1, rows), (hidden // 4,))
+        cb.encode(lib.pipeline("residual_rms_ms"), {0: b_x, 1: b_y, 2: b_res, 3: b_w, 4: b_res_norm},
+                  {5: hidden, 6: hidden, 7: hidden}, (1, rows), (hidden // 4,))
+        cb.encode(lib.pipeline("add_bf16"), {0: b_x, 1: b_y, 2: b_add}, {3: rows * hidden},
+                  ((rows * hidden + 255) // 256,), (256,))
+    run(rec)
+    for what, got, want in (("rms_only_ms", b_norm, want_norm), ("residual", b_res, sums),
+                            ("residual_rms_ms norm", b_res_norm, want_sum_norm),
+                            ("add_bf16", b_add, sums)):
+        g = got.read(np.uint16)
+        differ = np.flatnonzero(g != want)
+        assert differ.size == 0, (f"{what}: {differ.size} of 65536 differ, first at input "
+                                  f"{x[differ[0]]:#06x}: got {g[differ[0]]:#06x} want "
+                                  f"{want[differ[0]]:#06x}")
+
+
 @pytest.mark.parametrize("rows,in_dim,out_dim", [(1, 2048, 9216), (4, 2048, 12352), (16, 4096, 2048),
                                                  (37, 2048, 4096), (3, 64, 70), (2, 2048, 70),
                                                  (13, 4096, 24)])
