@@ -453,6 +453,46 @@ def test_qk_rope_of_a_token_wave_on_striped_pools():
     check_bf16(got_k[rope_rows], want_k[rope_rows], "appended K rows", ulps=1)
 
 
+def test_qk_norm_over_every_bf16_value_bit_for_bit():
+    """The qk norm of attn_qk_rope_ms on all 65536 bf16 bit patterns (non-finite ones replaced
+    by zero; ordered by magnitude, so a head of 256 holds neighbouring binades) at position 0,
+    where the rotation is the identity: the square sums, the inverse, both roundings and the
+    flushes of the reference's model, bit for bit."""
+    print("[case] attn_qk_rope_ms over every bf16 value", flush=True)
+    B, dev, queue, lib = gpu()
+    cap, rows = 32, 16
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    patterns[(patterns & 0x7F80) == 0x7F80] = 0
+    x = patterns[np.argsort(patterns & 0x7FFF, kind="stable")].reshape(rows, 16, 256)
+    q_w, k_w = _weights()
+    proj = np.zeros((rows, 9216), np.uint16)
+    proj.reshape(rows, -1)[:, :8192].reshape(rows, 16, 2, 256)[:, :, 0, :] = x     # q halves
+    proj[:, 8192:8704] = x[:, 5:7, :].reshape(rows, 512)                            # two k heads
+    stripe = 2 * cap * 256
+    k_pool, stride = dev.create_pool(stripe * 2, rows)
+    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    table = np.zeros(64, np.uint32)
+    for r in range(rows):
+        table[r * 4] = r * (stride // 2)
+    b_proj, b_tab = dev.buffer_from(proj), dev.buffer_from(table)
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g = dev.create_buffer(rows * 8192), dev.create_buffer(rows * 8192)
+    run(lambda cb: cb.encode(lib.pipeline("attn_qk_rope_ms"),
+                             {0: b_proj, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: k_pool, 6: v_pool,
+                              8: b_tab}, {7: cap, 9: 9216, 10: 4096}, (18, rows), (256,)))
+    got_q = b_q.read(np.uint16).reshape(rows, 4096)
+    got_k = k_pool.read(np.uint16).reshape(rows, stride // 2)
+    for r in range(rows):
+        q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16)
+        keys = np.zeros(stripe, np.uint16); values = np.zeros(stripe, np.uint16)
+        o.tto_attn_qk_rope(proj[r], q_w, k_w, 0, cap, q, gate, keys, values)
+        differ = np.flatnonzero(got_q[r] != q)
+        assert differ.size == 0, (f"row {r}: {differ.size} q values differ, first: input "
+                                  f"{x[r].reshape(-1)[differ[0]]:#06x} got "
+                                  f"{got_q[r][differ[0]]:#06x} want {q[differ[0]]:#06x}")
+        assert np.array_equal(got_k[r, :stripe], keys), f"row {r}: K rows"
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
