@@ -101,6 +101,35 @@ def test_wave_projection_bit_for_bit(family, suffix, rows, tile):
     print(f"[time] {name} rows={rows} tile={tile}: {ms * 1e3:.1f} us", flush=True)
 
 
+def test_wave_projection_of_every_small_bf16_input_bit_for_bit():
+    """attn_project_ms on inputs that run through every bf16 bit pattern below 2^30 in
+    magnitude (the subnormals among them), ordered by magnitude so that a row of 2048 holds
+    neighbouring binades: what the reference's model does with subnormal inputs, products
+    and sums (q4_dot_reference), bit for bit."""
+    print("[case] attn_project_ms over every bf16 input below 2^30", flush=True)
+    B, dev, queue, lib = gpu()
+    family = ATTN
+    host, bindings = _family(dev, family, 0x9800)
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    small = patterns[(patterns & 0x7FFF) < 0x4E80]
+    small = small[np.argsort(small & 0x7FFF, kind="stable")]
+    rows = 16
+    x = np.resize(small, rows * family["k"])            # 32768 values: the 32768 smallest magnitudes
+    assert x.size <= small.size
+    total = sum(family["segments"])
+    out = dev.create_buffer(rows * total * 2)
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    slot = family["out"] + 1
+    run(lambda cb: cb.encode(lib.pipeline("attn_project_ms"), bindings, {slot: rows, slot + 1: 16},
+                             (_groups(family), 1, 1), (family["threads"], 1, 1)))
+    got = out.read(np.uint16)
+    want = _expected(family, host, x, rows)
+    differ = np.flatnonzero(got != want)
+    assert differ.size == 0, (f"{differ.size} of {got.size} outputs differ, first: row "
+                              f"{differ[0] // total} got {got[differ[0]]:#06x} want {want[differ[0]]:#06x}")
+
+
 @pytest.mark.parametrize("rows", [1, 2, 4, 13, 16])
 @pytest.mark.parametrize("family", [ATTN, GDN, OUT], ids=lambda f: f["name"])
 def test_wave_projection_on_the_matrix_unit(family, rows):
