@@ -220,6 +220,48 @@ def test_output_gate_of_every_bf16_value_bit_for_bit():
     assert np.array_equal(b_one.read(np.uint16), want[5])
 
 
+def test_gates_of_every_bf16_value():
+    """decay and beta (gdn_gates_blk) with the a and b rows running through all 65536 bf16
+    bit patterns (non-finite ones replaced by zero).  beta is a chain of bf16 steps: the
+    checker's bits.  decay = exp(y) ends in two fp32 exponentials of different libraries: within
+    a few ulps of y, i.e. 4e-7 (1 + |y|) of the result."""
+    rows = 2048
+    print("[case] gdn gates over every bf16 value", flush=True)
+    B, dev, queue, lib = gpu()
+    _, a_log, dt_bias, _ = _weights()
+    patterns = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    patterns[(patterns & 0x7F80) == 0x7F80] = 0
+    proj = np.zeros((rows, 12352), np.uint16)
+    proj[:, 12288:12320] = patterns.reshape(rows, 32)                   # b
+    proj[:, 12320:12352] = np.roll(patterns, 7).reshape(rows, 32)       # a
+    want_decay = np.zeros((rows, 32), np.float32); want_beta = np.zeros((rows, 32), np.float32)
+    for r in range(rows):
+        o.tto_gdn_gates(proj[r], a_log, dt_bias, want_decay[r], want_beta[r])
+    b_proj = dev.buffer_from(proj.reshape(-1))
+    b_al, b_dt = dev.buffer_from(a_log), dev.buffer_from(dt_bias)
+    b_decay, b_beta = dev.create_buffer(rows * 128), dev.create_buffer(rows * 128)
+    run(lambda cb: cb.encode(lib.pipeline("gdn_gates_blk"),
+                             {0: b_proj, 1: b_al, 2: b_dt, 3: b_decay, 4: b_beta}, {5: rows},
+                             (1, (rows + 3) // 4, 1), (32, 4, 1)))
+    beta = b_beta.read(np.float32).reshape(rows, 32)
+    decay = b_decay.read(np.float32).reshape(rows, 32)
+    assert np.array_equal(beta.view(np.uint32), want_beta.view(np.uint32)), \
+        f"{np.count_nonzero(beta.view(np.uint32) != want_beta.view(np.uint32))} betas differ"
+    assert np.isfinite(decay).all()
+    # decay = exp(y): an ulp of y is |y| 2^-23 of the result
+    exponent = np.abs(np.log(np.maximum(want_decay.astype(np.float64), 1e-300)))
+    # (a subnormal decay comes out as zero: the family's arithmetic flushes, and the checker's
+    # next step, state * decay, flushes the product as well)
+    bar = 4e-7 * (1.0 + np.minimum(exponent, 110.0)) * np.abs(want_decay) + 1.2e-38
+    close = np.abs(decay.astype(np.float64) - want_decay) <= bar
+    bad = np.argwhere(~close)
+    detail = [(hex(int(proj[r, 12320 + h])), hex(int(a_log[h])), hex(int(dt_bias[h])),
+               float(decay[r, h]), float(want_decay[r, h])) for r, h in bad[:6]]
+    assert close.all(), (f"{len(bad)} decays differ, worst relative "
+                         f"{np.max(np.abs(decay - want_decay) / np.maximum(np.abs(want_decay), 1e-30)):.3e}"
+                         f" (a, A_log, dt_bias, got, want): {detail}")
+
+
 def _encode_chunked(cb, lib, bufs, rows, state_in="state_in", state_out="state_out"):
     chunks = (rows + 63) // 64
     cb.encode(lib.pipeline("gdn_chunk_prepare_blk"),
