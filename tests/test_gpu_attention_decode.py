@@ -493,6 +493,46 @@ def test_qk_norm_over_every_bf16_value_bit_for_bit():
         assert np.array_equal(got_k[r, :stripe], keys), f"row {r}: K rows"
 
 
+@pytest.mark.parametrize("position", [100000, 65535, 262143])
+def test_qk_rope_far_positions(position):
+    """The rotation at the deep end of config 3 and beyond: angles up to 2.6e5 rad, where the
+    sine and cosine stand or fall with the argument reduction.  Against the golden q of the
+    reference's model at position 100000, and the checker within a bf16 step elsewhere."""
+    print(f"[case] attn_qk_rope at position {position}", flush=True)
+    B, dev, queue, lib = gpu()
+    proj, q_w, k_w = cases.attention_chain_inputs(ol.banded_bf16)
+    cap = position + 1
+    b_p, b_qw, b_kw = dev.buffer_from(proj[0]), dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g = dev.create_buffer(8192), dev.create_buffer(8192)
+    b_k, b_v = dev.create_buffer(2 * cap * 512), dev.create_buffer(2 * cap * 512)
+    run(lambda cb: cb.encode(lib.pipeline("attn_qk_rope"),
+                             {0: b_p, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: b_k, 6: b_v},
+                             {7: position, 8: cap}, (18,), (256,)))
+    q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16)
+    keys = np.zeros(2 * cap * 256, np.uint16); values = np.zeros_like(keys)
+    o.tto_attn_qk_rope(proj[0], q_w, k_w, position, cap, q, gate, keys, values)
+    if position == 100000:
+        G = np.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
+        assert np.array_equal(q, G["rope_far_q"])
+    got_q = b_q.read(np.uint16)
+    got_k = b_k.read(np.uint16).reshape(2, cap, 256)[:, position]
+    for what, got, want in (("q", got_q, q), ("k row", got_k.reshape(-1),
+                                              keys.reshape(2, cap, 256)[:, position].reshape(-1))):
+        g = ol.bf16_to_f32(got).reshape(-1, 256)
+        w = ol.bf16_to_f32(want).reshape(-1, 256)
+        # a rotated value may be the small difference of two large products: the step that
+        # counts is the one of the pair's size (the rotation keeps the pair's norm)
+        size = np.abs(w).copy()
+        pair = np.maximum(size[:, :32], size[:, 32:64])
+        size[:, :32] = pair; size[:, 32:64] = pair
+        rel = np.abs(g - w) / np.maximum(size, 1e-3)
+        print(f"[parity] far rope {what}: exact {np.mean(got == want):.4f} max-rel {rel.max():.3e}",
+              flush=True)
+        assert rel.max() <= 2 ** -7          # at most one bf16 step of the pair's size
+        assert np.mean(got == want) > 0.99
+    assert np.array_equal(b_g.read(np.uint16), gate)
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
