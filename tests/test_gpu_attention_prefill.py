@@ -96,6 +96,13 @@ def test_block_shapes(rows, base):
     _prefill_case(rows, base, 2048, 0x5EED + rows, control=rows <= 48)
 
 
+def test_block_at_the_deep_end_of_a_100k_cache():
+    """13 rows appended at positions 99987 .. 99999: the block rope's angles at the far end
+    (argument reduction), 32-bit offsets into a 102 MB cache, and a flash pass over 100k keys."""
+    print("[case] prefill 13 rows at context 99987, capacity 100000", flush=True)
+    _prefill_case(13, 99987, 100000, 0xFA12, control=False)
+
+
 def test_prefill_row_equals_decode_step_on_gpu():
     """Row r of a block at context c is the decode operator at context c + r over
     the same cache (prefill_attention.metal:117-119)."""
