@@ -339,8 +339,10 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
         const uint32_t place = linear - kAttnKvHeads * (__builtin_amdgcn_readlane(through, row) - row_splits);
         kvh = place >= row_splits ? 1u : 0u;   // two kv heads
         split = place - kvh * row_splits;
-        kv_offset = __builtin_amdgcn_readlane(entry[0], row);
-        context = __builtin_amdgcn_readlane(entry[1], row);
+        // (the builtin returns int: without the cast an offset past 2^31 elements would be
+        // sign-extended into the 64-bit address)
+        kv_offset = static_cast<uint32_t>(__builtin_amdgcn_readlane(entry[0], row));
+        context = static_cast<uint32_t>(__builtin_amdgcn_readlane(entry[1], row));
     } else {
         if (a.row_list != nullptr) {
             row = a.row_list[row];

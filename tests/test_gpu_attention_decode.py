@@ -186,25 +186,28 @@ def test_decode_context_edges(ctx):
         check_bf16(b_o2.read(np.uint16), want, f"split part {part} ctx {ctx}")
 
 
-def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=False):
+def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=False,
+                stripes=None, pool_stripes=None):
     """Lane-batched decode over a striped pool with a state table, long rows
     through attention_decode_split_ms and short rows through attention_decode_ms.
     interleave: a lane's workgroups take its 32-key blocks in turn (bit 1 of c9).
     compact: the workgroups whose splits hold keys lead the dispatch order (bit 2 of c9);
     the records, and so the output bits, are those of the plain order.
+    stripes / pool_stripes: which stripe of a pool of `pool_stripes` each lane lives on
+    (default: the lanes in reverse order on a pool of their number).
     replays > 0: the recording is also compiled into a HIP graph and replayed that
     many times with the outputs and records cleared in between; every replay must
     reproduce the eager bits."""
     B, dev, queue, lib = gpu()
     rows = len(contexts)
     stripe = 2 * cap * 256          # elements per lane cache
-    k_pool, stride = dev.create_pool(stripe * 2, rows)
-    v_pool, _ = dev.create_pool(stripe * 2, rows)
+    k_pool, stride = dev.create_pool(stripe * 2, pool_stripes or rows)
+    v_pool, _ = dev.create_pool(stripe * 2, pool_stripes or rows)
     assert stride == stripe * 2
     q = np.zeros((rows, 4096), np.uint16); gate = np.zeros_like(q)
     want = np.zeros_like(q)
     # lanes are placed on stripes in reverse order so row != stripe
-    stripes = list(range(rows))[::-1]
+    stripes = stripes or list(range(rows))[::-1]
     table = np.zeros(64, np.uint32)
     for r, ctx in enumerate(contexts):
         lane_seed = seed ^ (r * 0x9E3779B97F4A7C15 & 0xFFFFFFFFFFFFFFFF)
@@ -531,6 +534,48 @@ def test_qk_rope_far_positions(position):
         assert rel.max() <= 2 ** -7          # at most one bf16 step of the pair's size
         assert np.mean(got == want) > 0.99
     assert np.array_equal(b_g.read(np.uint16), gate)
+
+
+def test_lane_on_the_last_stripe_a_32_bit_offset_can_name():
+    """State-table offsets are 32-bit element counts (decode_step.cpp:476): a pool of 127
+    stripes of a 65536-key cache (8.5 GB) puts the last stripe 4.23e9 elements in, the first
+    one at zero.  Every address past the table entry has to be 64-bit arithmetic."""
+    print("[case] lane batch on stripes 126 and 0 of 127 x 65536 keys", flush=True)
+    cap, pool_stripes = 65536, 127
+    assert (pool_stripes - 1) * 2 * cap * 256 > 0.98 * 2 ** 32      # the last stripe's offset
+    assert (pool_stripes + 1) * 2 * cap * 512 > 2 * 0xFFFFFFFF      # one stripe more is refused
+    _lane_batch([65535, 40000], cap, 1024, 0x32B1, replays=1, compact=True, stripes=[126, 0],
+                pool_stripes=pool_stripes)
+    # order by grid position, blocks in turn, and a short row through attention_decode_ms
+    _lane_batch([100, 5000], cap, 512, 0x32B2, interleave=True, stripes=[126, 125],
+                pool_stripes=pool_stripes)
+    # the appending side: the rope of a token wave writes its K / V rows there
+    B, dev, queue, lib = gpu()
+    stripe = 2 * cap * 256
+    k_pool, stride = dev.create_pool(stripe * 2, pool_stripes)
+    v_pool, _ = dev.create_pool(stripe * 2, pool_stripes)
+    q_w, k_w = _weights()
+    proj = np.stack([ol.gaussian_bf16(0x32C1 + r, 9216) for r in range(2)])
+    positions, stripes = [65535, 7], [126, 0]
+    table = np.zeros(64, np.uint32)
+    for r in range(2):
+        table[r * 4] = stripes[r] * (stride // 2)
+        table[r * 4 + 1] = positions[r]
+    b_proj, b_tab = dev.buffer_from(proj), dev.buffer_from(table)
+    b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
+    b_q, b_g = dev.create_buffer(2 * 8192), dev.create_buffer(2 * 8192)
+    run(lambda cb: cb.encode(lib.pipeline("attn_qk_rope_ms"),
+                             {0: b_proj, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: k_pool, 6: v_pool,
+                              8: b_tab}, {7: cap, 9: 9216, 10: 4096}, (18, 2), (256,)))
+    for r in range(2):
+        q = np.zeros(4096, np.uint16); gate = np.zeros(4096, np.uint16)
+        keys = np.zeros(stripe, np.uint16); values = np.zeros(stripe, np.uint16)
+        o.tto_attn_qk_rope(proj[r], q_w, k_w, positions[r], cap, q, gate, keys, values)
+        got_v = v_pool.read(np.uint16, stripe, stripes[r] * stride)
+        got_k = k_pool.read(np.uint16, stripe, stripes[r] * stride)
+        assert np.array_equal(got_v, values), f"row {r}: V rows of stripe {stripes[r]}"
+        assert np.array_equal(got_k != 0, keys != 0), f"row {r}: which K elements were written"
+        check_bf16(got_k, keys, f"row {r} K row on stripe {stripes[r]}", ulps=1)
 
 
 def test_config3_four_ragged_lanes_at_depth():
