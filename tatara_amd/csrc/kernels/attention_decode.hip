@@ -964,7 +964,8 @@ __global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArg
     __syncthreads();
     // values read back from LDS are the same in every lane: moved to scalar registers so
     // that the segment walk, the key ranges and the row's table entries stay scalar
-    const auto uniform = [](uint32_t v) { return __builtin_amdgcn_readfirstlane(v); };
+    // (the builtin returns int: as uint32_t, so that a 32-bit offset widens without its sign)
+    const auto uniform = [](uint32_t v) -> uint32_t { return __builtin_amdgcn_readfirstlane(v); };
     uint32_t unit = uniform(s_range[0]);
     const uint32_t unit_end = uniform(s_range[1]);
     if (unit >= unit_end) return;

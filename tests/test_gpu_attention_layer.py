@@ -24,14 +24,14 @@ def _weights():
 
 
 def _layer_batch(contexts, cap, groups_list, seed, replays=0, projection_stride=9216,
-                 query_stride=4096):
+                 query_stride=4096, stripes=None, pool_stripes=None):
     B, dev, queue, lib = gpu()
     rows = len(contexts)
     q_w, k_w = _weights()
     stripe = 2 * cap * 256
-    k_pool, stride = dev.create_pool(stripe * 2, rows)
-    v_pool, _ = dev.create_pool(stripe * 2, rows)
-    stripes = list(range(rows))[::-1]          # row != stripe
+    k_pool, stride = dev.create_pool(stripe * 2, pool_stripes or rows)
+    v_pool, _ = dev.create_pool(stripe * 2, pool_stripes or rows)
+    stripes = stripes or list(range(rows))[::-1]          # row != stripe
     proj = np.zeros((rows, projection_stride), np.uint16)
     want = np.zeros((rows, 4096), np.uint16)
     table = np.zeros(64, np.uint32)
@@ -158,6 +158,13 @@ def test_layer_config3_single_lane_100k():
 def test_layer_sixteen_lanes():
     print("[case] decode layer, 16 lanes (32 streams)", flush=True)
     _layer_batch([100 + 61 * i for i in range(16)], 1280, [256], 0x4D02, replays=1)
+
+
+def test_layer_lane_on_the_last_stripe_a_32_bit_offset_can_name():
+    """A pool of 127 stripes of a 65536-key cache puts the last stripe 4.23e9 elements in:
+    state-table offsets are 32-bit element counts, every address beyond them 64-bit."""
+    print("[case] layer batch on stripes 126 and 0 of 127 x 65536 keys", flush=True)
+    _layer_batch([65534, 3000], 65536, [64], 0x32D1, stripes=[126, 0], pool_stripes=127)
 
 
 def test_layer_validation():
