@@ -578,6 +578,15 @@ def test_lane_on_the_last_stripe_a_32_bit_offset_can_name():
         check_bf16(got_k, keys, f"row {r} K row on stripe {stripes[r]}", ulps=1)
 
 
+def test_lane_at_the_longest_context_of_the_model():
+    """One lane at 262144 visible keys (the model's context length): 128 splits of 2048 keys
+    as the host picks them, blocks in turn, the 128-record combine."""
+    print("[case] lane batch, 1 lane at 262144 keys", flush=True)
+    from tatara_amd import stack as S
+    assert S.choose_split_keys([262144]) == 2048
+    _lane_batch([262143], 262144, 2048, 0x40000, interleave=True)
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
