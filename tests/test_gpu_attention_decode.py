@@ -587,6 +587,24 @@ def test_lane_at_the_longest_context_of_the_model():
     _lane_batch([262143], 262144, 2048, 0x40000, interleave=True)
 
 
+def test_lane_batch_drawn_shapes():
+    """Two dozen waves drawn from a fixed seed: 1 to 16 lanes, contexts anywhere in the cache
+    (empty and full ones among them), split sizes from one block up, every combination of the
+    dispatch order and the block order; half of them also compiled and replayed."""
+    import random
+    rng = random.Random(0xD1CE)
+    for case in range(24):
+        rows = rng.choice([1, 2, 3, 4, 5, 8, 11, 16])
+        cap = rng.choice([512, 1024, 2048, 4096])
+        part = 32 * rng.randint(1, 16)
+        contexts = [rng.choice([0, cap - 1, rng.randrange(cap), rng.randrange(cap)]) for _ in range(rows)]
+        interleave, compact = rng.random() < 0.5, rng.random() < 0.5
+        print(f"[case] drawn wave {case}: contexts {contexts} cap {cap} part {part} "
+              f"interleave {interleave} compact {compact}", flush=True)
+        _lane_batch(contexts, cap, part, 0xD1CE00 + case, replays=case % 2, interleave=interleave,
+                    compact=compact)
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
