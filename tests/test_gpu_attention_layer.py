@@ -167,6 +167,22 @@ def test_layer_lane_on_the_last_stripe_a_32_bit_offset_can_name():
     _layer_batch([65534, 3000], 65536, [64], 0x32D1, stripes=[126, 0], pool_stripes=127)
 
 
+def test_layer_drawn_shapes():
+    """A dozen waves drawn from a fixed seed through both forms of the whole-layer dispatch:
+    1 to 16 lanes, contexts anywhere short of the last position, 1 to 400 workgroups - fewer
+    than streams, more than units, and everything between."""
+    import random
+    rng = random.Random(0x1A7E)
+    for case in range(12):
+        rows = rng.choice([1, 2, 3, 4, 7, 16])
+        cap = rng.choice([512, 1024, 2048])
+        contexts = [rng.choice([0, cap - 2, rng.randrange(cap - 1), rng.randrange(cap - 1)])
+                    for _ in range(rows)]
+        groups = [rng.choice([1, 2, 3, 5, 8, 17, 32, 33, 64, 100, 256, 400]) for _ in range(2)]
+        print(f"[case] drawn layer wave {case}: contexts {contexts} cap {cap} groups {groups}", flush=True)
+        _layer_batch(contexts, cap, groups, 0x1A7E00 + case, replays=case % 2)
+
+
 def test_layer_validation():
     B, dev, queue, lib = gpu()
     rows, cap, groups = 2, 512, 8
