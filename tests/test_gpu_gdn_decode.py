@@ -235,3 +235,68 @@ def test_fused_decode_step_equals_the_three_operators():
                   {0: b_proj, 1: pools[0][0], 2: b_w, 3: b_al, 4: b_dt, 5: pools[0][1], 6: b_nw,
                    7: outs[1], 8: b_tab}, {9: 12352, 10: 4096}, (32, 17), (512,))
     assert e.value.status == 15
+
+
+@pytest.mark.parametrize("lanes", [1, 3, 16])
+def test_fused_decode_step_on_drawn_planes(lanes):
+    """The fused step against the three operators for 1, 3 and 16 lanes whose input and
+    output planes are drawn from a pool in any order (the state table names them): the
+    same output bits and the same state planes, every other plane untouched."""
+    import random
+    print(f"[case] gdn fused decode step, {lanes} lanes on drawn planes", flush=True)
+    B, dev, queue, lib = gpu()
+    rng = random.Random(0x6D00 + lanes)
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    b_w, b_al, b_dt, b_nw = (dev.buffer_from(x) for x in (conv_w, a_log, dt_bias, norm_w))
+    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
+    planes = 2 * lanes + 3
+    order = list(range(planes))
+    rng.shuffle(order)
+    proj = np.zeros((lanes, 12352), np.uint16)
+    conv0 = ol.gaussian_bf16(0x6D10, planes * conv_elems, 0.0, 0.5)
+    rec0 = ol.gaussian_f32(0x6D11, planes * rec_elems, 0.0, 0.02)
+    table = np.zeros(64, np.uint32)
+    for r in range(lanes):
+        p, cs, st = _lane_inputs(r % 4)
+        proj[r] = np.roll(p, r // 4)             # lanes beyond the four seeded ones: shifted rows
+        i, o_ = order[2 * r], order[2 * r + 1]
+        table[4 * r:4 * r + 4] = (i * conv_elems, o_ * conv_elems, i * rec_elems, o_ * rec_elems)
+    b_tab, b_proj = dev.buffer_from(table), dev.buffer_from(proj)
+    pools = [(dev.buffer_from(conv0), dev.buffer_from(rec0)) for _ in range(2)]
+    b_qk, b_v, b_z, b_y = (dev.create_buffer(lanes * 8192) for _ in range(4))
+    outs = [dev.create_buffer(lanes * 8192) for _ in range(2)]
+
+    def rec(cb):
+        conv, rec_ = pools[0]
+        cb.encode(lib.pipeline("gdn_prepare_ms"),
+                  {0: b_proj, 1: conv, 2: b_w, 3: b_qk, 4: b_v, 5: b_z, 6: b_tab},
+                  {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, lanes), (128,))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_recurrence_ms"),
+                  {0: b_qk, 1: b_v, 2: b_proj, 3: b_al, 4: b_dt, 5: rec_, 6: b_y, 7: b_tab},
+                  {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32 * lanes), (32, 4, 1))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_gate_norm_ms"), {0: b_y, 1: b_z, 2: b_nw, 3: outs[0]}, {4: 4096},
+                  (32, lanes), (128,))
+        conv, rec_ = pools[1]
+        cb.encode(lib.pipeline("gdn_decode_fused_ms"),
+                  {0: b_proj, 1: conv, 2: b_w, 3: b_al, 4: b_dt, 5: rec_, 6: b_nw, 7: outs[1],
+                   8: b_tab}, {9: 12352, 10: 4096}, (32, lanes), (512,))
+    run(rec)
+    assert np.array_equal(outs[0].read(np.uint16), outs[1].read(np.uint16))
+    conv_after = [pool[0].read(np.uint16).reshape(planes, conv_elems) for pool in pools]
+    rec_after = [pool[1].read(np.float32).reshape(planes, rec_elems) for pool in pools]
+    assert np.array_equal(conv_after[0], conv_after[1])
+    assert np.array_equal(rec_after[0].view(np.uint32), rec_after[1].view(np.uint32))
+    written = {order[2 * r + 1] for r in range(lanes)}
+    for plane in range(planes):
+        if plane not in written:
+            assert np.array_equal(conv_after[1][plane], conv0.reshape(planes, -1)[plane]), plane
+            assert np.array_equal(rec_after[1][plane], rec0.reshape(planes, -1)[plane]), plane
+    # lane 0 against the checker (the other lanes are held to it through the three operators)
+    p, cs, st = proj[0], conv0.reshape(planes, -1)[order[0]], rec0.reshape(planes, -1)[order[0]]
+    ncs = np.zeros(conv_elems, np.uint16); so = np.zeros(rec_elems, np.float32)
+    gated = np.zeros(4096, np.uint16)
+    o.tto_gdn_decode_step(p, cs, conv_w, a_log, dt_bias, norm_w, st, ncs, so, gated, 8)
+    check_bf16(outs[1].read(np.uint16)[:4096], gated, "fused lane 0 gated")
+    assert np.array_equal(conv_after[1][order[1]], ncs)
