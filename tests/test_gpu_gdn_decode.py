@@ -300,3 +300,60 @@ def test_fused_decode_step_on_drawn_planes(lanes):
     o.tto_gdn_decode_step(p, cs, conv_w, a_log, dt_bias, norm_w, st, ncs, so, gated, 8)
     check_bf16(outs[1].read(np.uint16)[:4096], gated, "fused lane 0 gated")
     assert np.array_equal(conv_after[1][order[1]], ncs)
+
+
+def test_conv_planes_at_the_far_end_of_a_32_bit_offset():
+    """State-table entries are 32-bit element offsets: conv planes 174000 and 174001 of an
+    8.55 GB pool sit 4.28e9 bf16 elements in, just short of 2^32.  The fused step and the
+    prepare operator have to reach them with 64-bit addresses."""
+    print("[case] gdn decode with conv planes 4.28e9 elements into the pool", flush=True)
+    B, dev, queue, lib = gpu()
+    conv_w, a_log, dt_bias, norm_w = _weights()
+    b_w, b_al, b_dt, b_nw = (dev.buffer_from(x) for x in (conv_w, a_log, dt_bias, norm_w))
+    conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
+    first = 174000
+    assert 0.99 * 2 ** 32 < (first + 3) * conv_elems < 2 ** 32
+    conv_pool, conv_stride = dev.create_pool(conv_elems * 2, first + 4)
+    assert conv_stride == conv_elems * 2
+    rec_pool, rec_stride = dev.create_pool(rec_elems * 4, 4)
+    p, cs, st = _lane_inputs(1)
+    table = np.zeros(64, np.uint32)
+    outs = []
+    for form in range(2):                        # planes (first, first + 1), then (first + 2, first + 3)
+        i, o_ = first + 2 * form, first + 2 * form + 1
+        conv_pool.write(cs, i * conv_stride)
+        rec_pool.write(st, 2 * form * rec_stride)
+        table[4 * form:4 * form + 4] = (i * conv_elems, o_ * conv_elems, 2 * form * rec_elems,
+                                        (2 * form + 1) * rec_elems)
+    b_tab = dev.buffer_from(table)
+    b_proj = dev.buffer_from(np.stack([p, p]))
+    b_qk, b_v, b_z, b_y = (dev.create_buffer(2 * 8192) for _ in range(4))
+    b_out = dev.create_buffer(2 * 8192)
+    b_fused = dev.create_buffer(2 * 8192)
+
+    def rec(cb):
+        # row 0 through the three operators, row 1 through the fused step (row 1's table entry)
+        cb.encode(lib.pipeline("gdn_prepare_ms"),
+                  {0: b_proj, 1: conv_pool, 2: b_w, 3: b_qk, 4: b_v, 5: b_z, 6: b_tab},
+                  {7: 12352, 8: 4096, 9: 4096, 10: 4096}, (96, 1), (128,))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_recurrence_ms"),
+                  {0: b_qk, 1: b_v, 2: b_proj, 3: b_al, 4: b_dt, 5: rec_pool, 6: b_y, 7: b_tab},
+                  {8: 4096, 9: 4096, 10: 12352, 11: 4096, 12: 32}, (1, 32, 32), (32, 4, 1))
+        cb.barrier()
+        cb.encode(lib.pipeline("gdn_gate_norm_ms"), {0: b_y, 1: b_z, 2: b_nw, 3: b_out}, {4: 4096},
+                  (32, 1), (128,))
+        cb.encode(lib.pipeline("gdn_decode_fused_ms"),
+                  {0: (b_proj, 12352 * 2), 1: conv_pool, 2: b_w, 3: b_al, 4: b_dt, 5: rec_pool,
+                   6: b_nw, 7: b_fused, 8: (b_tab, 16)}, {9: 12352, 10: 4096}, (32, 1), (512,))
+    run(rec)
+    ncs = np.zeros(conv_elems, np.uint16); so = np.zeros(rec_elems, np.float32)
+    gated = np.zeros(4096, np.uint16)
+    o.tto_gdn_decode_step(p, cs, conv_w, a_log, dt_bias, norm_w, st, ncs, so, gated, 8)
+    three, fused = b_out.read(np.uint16)[:4096], b_fused.read(np.uint16)[:4096]
+    assert np.array_equal(three, fused)
+    check_bf16(fused, gated, "gated, planes at the far end")
+    for form in range(2):
+        got = conv_pool.read(np.uint16, conv_elems, (first + 2 * form + 1) * conv_stride)
+        assert np.array_equal(got, ncs), f"conv plane written by form {form}"
+        assert np.array_equal(conv_pool.read(np.uint16, conv_elems, (first + 2 * form) * conv_stride), cs)
