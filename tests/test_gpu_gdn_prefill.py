@@ -294,6 +294,34 @@ def test_chunked_recurrence_matches_token_loop(rows):
     check_bf16(bufs["gated"].read(np.uint16), ref["gated"], "chunked gated", ulps=4)
 
 
+def test_chunked_recurrence_with_harsh_gates():
+    """Gates far from the seeded tests' mild ones: exp(A_log) from 0.4 to 16 and a wide a row,
+    so that decays run from 1 down to exp(-100) and underflow inside a chunk, betas from 0 to 1.
+    The chunked evaluation keeps its decay products in logarithms; the token loop is the bar."""
+    rows = 200
+    print("[case] gdn chunked recurrence with harsh gates", flush=True)
+    B, dev, queue, lib = gpu()
+    conv_w, _, dt_bias, norm_w = _weights()
+    a_log = ol.f32_to_bf16(ol.uniform_f32(0x7B, 32, -1.0, 2.8))
+    weights = (conv_w, a_log, dt_bias, norm_w)
+    proj, conv_state, state = _block(rows, 0x5400)
+    proj[:, 12320:12352] = ol.gaussian_bf16(0x5401, rows * 32, 0.0, 3.0).reshape(rows, 32)   # a
+    proj[:, 12288:12320] = ol.gaussian_bf16(0x5402, rows * 32, 0.0, 6.0).reshape(rows, 32)   # b
+    ref = _oracle_block(proj, conv_state, state, weights, rows)
+    assert ref["decay"].min() < 1e-30 and ref["decay"].max() > 0.99
+    assert ref["beta"].min() < 1e-3 and ref["beta"].max() > 0.999
+    bufs = _buffers(dev, proj, conv_state, state, weights, rows)
+
+    def rec(cb):
+        _encode_front(cb, lib, bufs, rows)
+        _encode_chunked(cb, lib, bufs, rows)
+        _encode_gate_norm(cb, lib, bufs, rows)
+    run(rec)
+    check_bf16(bufs["y"].read(np.uint16), ref["y"], "harsh gates: chunked y")
+    check_f32(bufs["state_out"].read(np.float32), ref["state"], "harsh gates: chunked state", 2e-3, 2e-4)
+    check_bf16(bufs["gated"].read(np.uint16), ref["gated"], "harsh gates: chunked gated", ulps=4)
+
+
 def test_chunked_recurrence_in_place_and_chained_blocks():
     """Two consecutive blocks (130 + 70 rows) with the state plane updated in
     place equal one 200-row token loop."""
