@@ -187,7 +187,7 @@ def test_decode_context_edges(ctx):
 
 
 def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=False,
-                stripes=None, pool_stripes=None):
+                stripes=None, pool_stripes=None, sharpen=0):
     """Lane-batched decode over a striped pool with a state table, long rows
     through attention_decode_split_ms and short rows through attention_decode_ms.
     interleave: a lane's workgroups take its 32-key blocks in turn (bit 1 of c9).
@@ -195,6 +195,7 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
     the records, and so the output bits, are those of the plain order.
     stripes / pool_stripes: which stripe of a pool of `pool_stripes` each lane lives on
     (default: the lanes in reverse order on a pool of their number).
+    sharpen: the queries are scaled by 2^sharpen (scores in the hundreds: a one-hot softmax).
     replays > 0: the recording is also compiled into a HIP graph and replayed that
     many times with the outputs and records cleared in between; every replay must
     reproduce the eager bits."""
@@ -212,6 +213,8 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
     for r, ctx in enumerate(contexts):
         lane_seed = seed ^ (r * 0x9E3779B97F4A7C15 & 0xFFFFFFFFFFFFFFFF)
         q[r] = ol.gaussian_bf16(lane_seed + 1, 4096)
+        if sharpen:
+            q[r] = np.where(q[r] & 0x7F80, q[r] + np.uint16(sharpen << 7), q[r])   # exponent + sharpen
         gate[r] = ol.gaussian_bf16(lane_seed + 2, 4096)
         n = ctx + 1
         k = np.zeros((2, cap, 256), np.uint16); v = np.zeros_like(k)
@@ -603,6 +606,14 @@ def test_lane_batch_drawn_shapes():
               f"interleave {interleave} compact {compact}", flush=True)
         _lane_batch(contexts, cap, part, 0xD1CE00 + case, replays=case % 2, interleave=interleave,
                     compact=compact)
+
+
+def test_lane_batch_with_scores_in_the_hundreds():
+    """Queries 32 times as large: scores of several hundred either way, a softmax that is one-hot
+    to working precision, records whose maxima differ by hundreds between splits."""
+    print("[case] lane batch, queries x 32", flush=True)
+    _lane_batch([5000, 4999, 31, 2047, 300], 8192, 512, 0x5A4B, replays=1, compact=True, sharpen=5)
+    _lane_batch([40000], 40960, 320, 0x5A4C, interleave=True, sharpen=5)
 
 
 def test_config3_four_ragged_lanes_at_depth():
