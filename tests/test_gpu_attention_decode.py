@@ -195,7 +195,8 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
     the records, and so the output bits, are those of the plain order.
     stripes / pool_stripes: which stripe of a pool of `pool_stripes` each lane lives on
     (default: the lanes in reverse order on a pool of their number).
-    sharpen: the queries are scaled by 2^sharpen (scores in the hundreds: a one-hot softmax).
+    sharpen: the queries are scaled by 2^sharpen (scores in the hundreds: a one-hot softmax);
+    negative: zero queries (a flat softmax).
     replays > 0: the recording is also compiled into a HIP graph and replayed that
     many times with the outputs and records cleared in between; every replay must
     reproduce the eager bits."""
@@ -213,8 +214,10 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
     for r, ctx in enumerate(contexts):
         lane_seed = seed ^ (r * 0x9E3779B97F4A7C15 & 0xFFFFFFFFFFFFFFFF)
         q[r] = ol.gaussian_bf16(lane_seed + 1, 4096)
-        if sharpen:
+        if sharpen > 0:
             q[r] = np.where(q[r] & 0x7F80, q[r] + np.uint16(sharpen << 7), q[r])   # exponent + sharpen
+        elif sharpen < 0:
+            q[r] = 0                                    # every score zero: the mean of the values
         gate[r] = ol.gaussian_bf16(lane_seed + 2, 4096)
         n = ctx + 1
         k = np.zeros((2, cap, 256), np.uint16); v = np.zeros_like(k)
@@ -614,6 +617,13 @@ def test_lane_batch_with_scores_in_the_hundreds():
     print("[case] lane batch, queries x 32", flush=True)
     _lane_batch([5000, 4999, 31, 2047, 300], 8192, 512, 0x5A4B, replays=1, compact=True, sharpen=5)
     _lane_batch([40000], 40960, 320, 0x5A4C, interleave=True, sharpen=5)
+
+
+def test_lane_batch_with_zero_queries():
+    """Every score zero: the output is the plain mean of the visible values times the gate,
+    each split's record a sum of `part` values with weight one."""
+    print("[case] lane batch, zero queries", flush=True)
+    _lane_batch([5000, 0, 255, 256, 8191], 8192, 1024, 0x5A4D, compact=True, sharpen=-1)
 
 
 def test_config3_four_ragged_lanes_at_depth():
