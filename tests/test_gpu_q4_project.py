@@ -178,6 +178,38 @@ def test_block_projection(family, name, rows):
     print(f"[time] {name} rows={rows}: {ms * 1e3:.1f} us", flush=True)
 
 
+@pytest.mark.parametrize("family,name", [(ATTN, "attn_project_blk"), (GDN, "gdn_project_blk"),
+                                         (OUT, "outproj_blk")], ids=["attn", "gdn", "out"])
+@pytest.mark.parametrize("rows", [256, 257, 700, 16384])
+def test_block_projection_over_several_row_tiles(family, name, rows):
+    """Blocks that span more than one 256-row tile of the block kernel, up to the 16384 rows
+    the benchmark times: every output row is produced, and a sample of rows - the first and
+    last of the block, the rows either side of each tile boundary sampled, a few inside -
+    is held to the checker."""
+    print(f"[case] {name} rows={rows} (sampled rows)", flush=True)
+    B, dev, queue, lib = gpu()
+    host, bindings = _family(dev, family, 0x9600)
+    k = family["k"]
+    x = ol.gaussian_bf16(0x9700 + rows, rows * k, 0.0, 1.0)
+    total = sum(family["segments"])
+    out = dev.buffer_from(np.full(rows * total, 0x7FC0, np.uint16))      # NaN until written
+    bindings[0] = dev.buffer_from(x)
+    bindings[family["out"]] = out
+    slot = family["out"] + 1
+    constants = {slot: rows, slot + 1: k} if family is OUT else {slot: rows}
+    run(lambda cb: cb.encode(lib.pipeline(name), bindings, constants, (_groups(family), 1, 1),
+                             (family["threads"], 1, 1)))
+    got = out.read(np.uint16).reshape(rows, total)
+    assert not np.any((got & 0x7FFF) > 0x7F80), "an output row was left unwritten"
+    sample = {0, rows - 1, rows // 2, rows // 3}
+    for edge in range(256, rows, 256 if rows <= 1024 else 4096):
+        sample.update({edge - 1, edge})
+    sample = sorted(r for r in sample if 0 <= r < rows)
+    xs = np.ascontiguousarray(x.reshape(rows, k)[sample]).reshape(-1)
+    want = _expected(family, host, xs, len(sample)).reshape(len(sample), total)
+    check_bf16(got[sample], want, f"{name} rows {sample[:4]}..{sample[-1]}", ulps=2)
+
+
 @pytest.mark.parametrize("rows", [2, 4, 13, 16])
 @pytest.mark.parametrize("family", [ATTN, GDN], ids=lambda f: f["name"])
 def test_wave_projection_with_the_norm_in_its_prologue(family, rows):
