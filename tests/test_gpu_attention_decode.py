@@ -626,6 +626,18 @@ def test_lane_batch_with_zero_queries():
     _lane_batch([5000, 0, 255, 256, 8191], 8192, 1024, 0x5A4D, compact=True, sharpen=-1)
 
 
+def test_four_deep_lanes_with_the_split_the_host_picks():
+    """Four lanes around 100k keys: the host's rule goes well past 1024 keys a workgroup here
+    (2656: 25 to 38 workgroups per lane and head, 256 in all), ranges in a grid that covers
+    the capacity."""
+    from tatara_amd import stack as S
+    contexts = [99999, 65535, 99999, 70000]
+    part = S.choose_split_keys([c + 1 for c in contexts])
+    print(f"[case] lane batch, 4 deep lanes, {part} keys per workgroup", flush=True)
+    assert part > 1024 and S.split_workgroups([c + 1 for c in contexts], part) <= 256
+    _lane_batch(contexts, 100000, part, 0xDEE9, replays=1, compact=True)
+
+
 def test_config3_four_ragged_lanes_at_depth():
     """Config 3: lanes at (32768, 30000, 24576, 8192) visible keys in a
     capacity-32768 pool."""
