@@ -413,7 +413,8 @@ DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
     }
     // whole-layer attention: one workgroup per compute unit; 256 B of tickets, 128 KiB of
     // query heads, then one record of 8 x 258 floats per workgroup and stream boundary
-    b.layer_groups = std::max<std::uint32_t>(device.compute_units(), 1);
+    b.compute_units = std::max<std::uint32_t>(device.compute_units(), 1);
+    b.layer_groups = b.compute_units;
     const std::uint64_t layer_scratch_bytes =
         256 + 131072 +
         (std::uint64_t{b.layer_groups} + 2 * rows - 1) * 8 * kAttentionRecordFloats * kF32Bytes;
@@ -555,7 +556,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
         }
     }
     const std::span<const std::uint32_t> long_keys(visible.data(), long_rows);
-    const std::uint32_t units = batch.layer_groups != 0 ? batch.layer_groups : 256;
+    const std::uint32_t units = std::max<std::uint32_t>(batch.compute_units, 1);
     std::uint32_t split_keys = batch.split_keys;
     if (split_keys == 0) {
         const std::uint64_t coarsest =

@@ -197,6 +197,8 @@ struct DecodeBatchScratch {
     // keys per split-K workgroup of the batched path (a multiple of 32); 0: chosen for
     // every wave from the depths of its rows by choose_split_keys
     std::uint32_t split_keys{0};
+    // compute units of the device the scratch was made on: what the automatic split fills
+    std::uint32_t compute_units{256};
     // How a row's split-K workgroups share its keys: consecutive ranges of `split_keys`, or
     // its 32-key blocks in turn.  Automatic: in turn for waves of one or two rows.  Ranges
     // are the faster order at most depths, but their time depends on how the cache's strides

@@ -402,9 +402,9 @@ int main() {
             // (one workgroup per long row and head) in a grid of twelve, so the workgroups that
             // hold keys are placed first in the dispatch order
             batch.split_keys = wave == 0 ? 256 : 0;
-            const std::uint32_t chip_units = batch.layer_groups;
+            const std::uint32_t chip_units = batch.compute_units;
             if (wave == 1) {
-                batch.layer_groups = 4;
+                batch.compute_units = 4;
                 batch.split_order = DecodeBatchScratch::SplitOrder::BlocksInTurn;   // pinned, three rows
             }
             std::vector<std::uint16_t> x = gauss16(7400 + wave, kLanes * 2048);
@@ -417,7 +417,7 @@ int main() {
                 return encode_token_batch(step, streams, *pooled.pool, batch, bound, stages.hooks(),
                                           pass);
             });
-            batch.layer_groups = chip_units;
+            batch.compute_units = chip_units;
             batch.split_order = DecodeBatchScratch::SplitOrder::Automatic;
             if (rc != 0) return 210 + rc;
             const auto got_residual = download<std::uint16_t>(hidden.residual, kLanes * 2048);
