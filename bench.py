@@ -148,9 +148,17 @@ class Wave:
         self.part = self.forced_split or stack_rules.choose_split_keys(visible, self.dev.compute_units)
         self.max_splits = (self.capacity + self.part - 1) // self.part
         self.interleave = 1 if self.rows <= 2 else 0
+        self.rotate = getattr(self, "rotate", 0)
         live = stack_rules.split_workgroups(visible, self.part)
         grid = self.max_splits * 2 * self.rows
         self.compact = 1 if grid > live and grid > self.dev.compute_units else 0
+        # the token form walks the cached keys only (the token itself is folded in afterwards)
+        cached = [max(c, 1) for c in contexts]
+        self.token_part = self.forced_split or stack_rules.choose_split_keys(cached, self.dev.compute_units)
+        token_splits = (self.capacity + self.token_part - 1) // self.token_part
+        grid = token_splits * 2 * self.rows
+        self.token_compact = 1 if (grid > stack_rules.split_workgroups(cached, self.token_part)
+                                   and grid > self.dev.compute_units) else 0
 
     def visible_keys(self):
         return sum(c + 1 for c in self.contexts)
@@ -176,6 +184,17 @@ class Wave:
                 cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: self.groups},
                           (16, rows), (64,))
             return
+        if self.attention == "token":
+            splits = (cap + self.token_part - 1) // self.token_part
+            bind = {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: layer["keys"],
+                    4: layer["values"], 5: self.attn_table, 6: self.b_part, 7: self.b_out}
+            const = {8: cap, 9: 9216, 10: 4096, 11: self.token_part, 12: splits,
+                     13: 2 * self.interleave + 4 * self.token_compact + 8 * self.rotate}
+            cb.encode(P("attention_decode_token_ms"), bind, const, (splits, 2, rows), (256,))
+            if not walk_only:
+                cb.barrier()
+                cb.encode(P("attention_decode_token_finish_ms"), bind, const, (16, rows), (256,))
+            return
         if not walk_only:
             cb.encode(P("attn_qk_rope_ms"),
                       {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: self.b_q,
@@ -185,7 +204,7 @@ class Wave:
         cb.encode(P("attention_decode_split_ms"),
                   {0: self.b_q, 1: layer["keys"], 2: layer["values"], 3: self.attn_table,
                    4: self.b_part}, {5: cap, 6: 4096, 7: self.part, 8: self.max_splits,
-                   9: 2 * self.interleave + 4 * self.compact},
+                   9: 2 * self.interleave + 4 * self.compact + 8 * self.rotate},
                   (self.max_splits, 2, rows), (256,))
         if not walk_only:
             cb.barrier()
@@ -454,7 +473,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--attention", choices=("layer", "three"), default="three",
+    ap.add_argument("--attention", choices=("layer", "three", "token"), default="three",
                     help="three: rope, split and combine dispatches (the faster key walk); layer: one "
                          "dispatch for the layer plus its finishing dispatch")
     ap.add_argument("--no-cpu-baseline", action="store_true")

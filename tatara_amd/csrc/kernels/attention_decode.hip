@@ -33,6 +33,8 @@
 #include "../tt_internal.h"
 #include "lane_sums.h"
 
+#include <utility>
+
 // Split records of tt_attention_decode_lanes_static: device memory that belongs to the
 // code object, one copy per GPU the library is loaded on, held until the process ends.
 // In host code this name is only a handle for hipGetSymbolAddress; the device address a
@@ -79,6 +81,62 @@ __device__ __forceinline__ float sigmoid_gate(uint16_t g) {
     return 1.0f / (1.0f + __expf(-bf16_bits_to_f32(g)));
 }
 
+// ------------------------------------------------------------ rotation angle ---
+
+// powf(1e7f, pair / 32.0f) for pair 0..31, the rotation's inverse frequencies as the
+// reference's scalar model takes them (tests/native/kernel_reference.cpp:636-676 receives the
+// cosines and sines its caller derived this way), written out so that every kernel uses
+// the correctly rounded values whatever the device's powf returns.
+// Selected with a tree of conditional moves on the bits of `pair`: a table in memory would
+// put a load from the code object's constant data at the head of every kernel that rotates.
+__device__ __forceinline__ float rope_inverse_frequency(uint32_t pair) {
+    float f[kAttnRopePairs] = {
+        0x1p+0f,        0x1.a7a218p+0f,  0x1.5e8488p+1f,  0x1.220578p+2f,  0x1.dfeeaap+2f,  0x1.8d19ap+3f,
+        0x1.489062p+4f, 0x1.0fdb4ep+5f,  0x1.c1df8p+5f,   0x1.743a94p+6f,  0x1.33fc3cp+7f,  0x1.fda8ccp+7f,
+        0x1.a5b24ep+8f, 0x1.5cea5p+9f,   0x1.20b20cp+10f, 0x1.ddbcfep+10f, 0x1.8b48e2p+11f, 0x1.470fdcp+12f,
+        0x1.0e9d26p+13f, 0x1.bfd102p+13f, 0x1.7286f2p+14f, 0x1.3293ccp+15f, 0x1.fb5454p+15f, 0x1.a3c4c8p+16f,
+        0x1.5b51f8p+17f, 0x1.1f602ep+18f, 0x1.db8de2p+18f, 0x1.897a46p+19f, 0x1.459116p+20f, 0x1.0d607p+21f,
+        0x1.bdc4eap+21f, 0x1.70d55p+22f,
+    };
+#pragma unroll
+    for (uint32_t level = 0; level < 5; ++level) {
+        const bool odd = (pair >> level) & 1u;
+#pragma unroll
+        for (uint32_t i = 0; i < (kAttnRopePairs >> (level + 1)); ++i) f[i] = odd ? f[2 * i + 1] : f[2 * i];
+    }
+    return f[0];
+}
+
+// Cosine and sine of theta = position / inverse_frequency (the fp32 quotient, as the model
+// forms it).  The quadrant reduction runs in fp64 - theta reaches 2.6e5 at the deepest
+// cache position, where an fp32 reduction would lose the angle - and the two polynomials on
+// [-pi/4, pi/4] in fp32, a few dozen instructions where the library's sincosf spends
+// hundreds on an argument of this size.  Within 2 ulp of the correctly rounded values; the
+// rotated values are rounded to bf16 next.
+struct RopeAngle {
+    float c, s;
+};
+__device__ __forceinline__ RopeAngle rope_angle_of(uint32_t position, float inverse_frequency) {
+    const float theta = static_cast<float>(position) / inverse_frequency;
+    const double t = static_cast<double>(theta);
+    const double k = rint(t * 0.63661977236758134308);
+    double r = fma(-k, 1.57079632679489655800e+00, t);
+    r = fma(-k, 6.12323399573676603587e-17, r);
+    const float x = static_cast<float>(r);
+    const float z = x * x;
+    const float sine = fmaf(((-1.9515295891e-4f * z + 8.3321608736e-3f) * z - 1.6666654611e-1f) * z, x, x);
+    const float cosine =
+        fmaf(((2.443315711809948e-5f * z - 1.388731625493765e-3f) * z + 4.166664568298827e-2f) * z, z,
+             fmaf(-0.5f, z, 1.0f));
+    const uint32_t quadrant = static_cast<uint32_t>(static_cast<int32_t>(k)) & 3u;
+    RopeAngle a;
+    a.s = (quadrant & 1u) ? cosine : sine;
+    a.c = (quadrant & 1u) ? sine : cosine;
+    if (quadrant == 1u || quadrant == 2u) a.c = -a.c;
+    if (quadrant >= 2u) a.s = -a.s;
+    return a;
+}
+
 // ---------------------------------------------------------------- qk rope ---
 
 struct RopeArgs {
@@ -99,6 +157,19 @@ struct RopeArgs {
     uint32_t rows_per_group;    // rows one workgroup walks (1 for decode)
 };
 
+// The squares of the 64 consecutive values a wave holds (one per lane), summed as the
+// reference sums them: a quad sums its four squares in order (thread q of the reference's
+// 64), then the adjacent-pairs tree over the slices runs over quads (mirrors of a half row
+// and of a row: a quad holds one value), rows and the halves of the wave.
+__device__ __forceinline__ float wave_square_slices(float sq) {
+    float slices = ((quad_lane<0>(sq) + quad_lane<1>(sq)) + quad_lane<2>(sq)) + quad_lane<3>(sq);
+    slices += lane_dpp<0x141>(slices);   // row_half_mirror: the neighbouring quad
+    slices += lane_dpp<0x140>(slices);   // row_mirror: the neighbouring pair of quads
+    slices += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(slices), 0x401F));  // lane ^ 16
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 0)) +
+           __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 32));
+}
+
 // grid (18, ceil(rows / rows_per_group)) x 256: one head per workgroup, one
 // dimension per thread.  Sum of squares as the reference takes it: 64 slices of 4
 // values summed in order, a 32-slice adjacent-pairs tree per half, then the two
@@ -112,10 +183,7 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
     const uint32_t base = is_query ? head * 2 * kD : kAttnQGateRows + local * kD;
     const float weight = bf16_bits_to_f32(is_query ? a.q_weight[d] : a.k_weight[d]);
     const uint32_t pair = d & (kAttnRopePairs - 1);
-    const float inverse_frequency =
-        d < 2 * kAttnRopePairs
-            ? powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs))
-            : 1.0f;
+    const float inverse_frequency = rope_inverse_frequency(pair);
     const uint32_t row_end = min(a.rows, (blockIdx.y + 1) * a.rows_per_group);
     for (uint32_t row = blockIdx.y * a.rows_per_group; row < row_end; ++row) {
         uint32_t position = a.context + (a.position_per_row ? row : 0u);
@@ -135,20 +203,15 @@ __global__ __launch_bounds__(256) void attn_qk_rope_kernel(RopeArgs a) {
         // loads above are in flight, not after the norm
         float c = 1.0f, s = 0.0f;
         if (d < 2 * kAttnRopePairs) {
-            const float theta = static_cast<float>(position) / inverse_frequency;
-            sincosf(theta, &s, &c);   // one argument reduction for both
+            const RopeAngle angle = rope_angle_of(position, inverse_frequency);
+            c = angle.c;
+            s = angle.s;
         }
         // Sum of squares in registers: a quad sums its four squares in order (thread q of the
         // reference's 64), then the adjacent-pairs tree over the 64 slices runs over quads
         // (mirrors of a half row and of a row: a quad holds one value), rows, the halves of
         // the wave, and the four waves - one value per wave through LDS, one barrier.
-        const float sq = x * x;
-        float slices = ((quad_lane<0>(sq) + quad_lane<1>(sq)) + quad_lane<2>(sq)) + quad_lane<3>(sq);
-        slices += lane_dpp<0x141>(slices);   // row_half_mirror: the neighbouring quad
-        slices += lane_dpp<0x140>(slices);   // row_mirror: the neighbouring pair of quads
-        slices += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(slices), 0x401F));  // lane ^ 16
-        const float wave_slices = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 0)) +
-                                  __int_as_float(__builtin_amdgcn_readlane(__float_as_int(slices), 32));
+        const float wave_slices = wave_square_slices(x * x);
         __syncthreads();  // the previous row's readers are done with the shared values
         if ((d & 63) == 0) wave_squares[d >> 6] = wave_slices;
         __syncthreads();
@@ -200,8 +263,7 @@ __global__ __launch_bounds__(192) void attn_qk_rope_block_kernel(RopeArgs a) {
             weight[j] = __uint_as_float((j & 1) ? (bits[j >> 1] & 0xFFFF0000u) : (bits[j >> 1] << 16));
         }
     }
-    const float inverse_frequency = powf(
-        kAttnRopeBase, static_cast<float>(lane & (kAttnRopePairs - 1)) / static_cast<float>(kAttnRopePairs));
+    const float inverse_frequency = rope_inverse_frequency(lane & (kAttnRopePairs - 1));
     const bool rotates = l < 2 * kAttnRopePairs / 8;
     const uint32_t row_end = min(a.rows, (blockIdx.y + 1) * a.rows_per_group);
     for (uint32_t row = blockIdx.y * a.rows_per_group; row < row_end; ++row) {
@@ -229,9 +291,9 @@ __global__ __launch_bounds__(192) void attn_qk_rope_block_kernel(RopeArgs a) {
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) n[j] = round_bf16(weight[j] * round_bf16(x[j] * inverse));
         // pair p = lane & 31 of this row, shared by the wave's two heads
-        const float theta = static_cast<float>(position) / inverse_frequency;
-        const float c = cosf(theta);
-        const float sn = sinf(theta);
+        const RopeAngle angle = rope_angle_of(position, inverse_frequency);
+        const float c = angle.c;
+        const float sn = angle.s;
         u32x4 packed;
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
@@ -264,6 +326,101 @@ __global__ __launch_bounds__(192) void attn_qk_rope_block_kernel(RopeArgs a) {
     }
 }
 
+// ------------------------------------------- norm and rotation by one wave ---
+
+// One head of 256 values through RMS norm, weight and rotation by one wave; lane l
+// receives dims l, l + 64, l + 128, l + 192 as the fp32 of the stored bf16.  Operation for
+// operation attn_qk_rope_kernel: lane l's four squares are thread l's there, the same
+// half-wave tree, the same rounding points, the same cosine and sine.
+struct HeadLoads {
+    uint32_t run[2];      // values 4 l .. 4 l + 3 (sum of squares)
+    uint16_t x[4];        // values l + 64 c
+    uint16_t w[4];
+    uint32_t x32[4];      // the registers of load_head_untracked, narrowed by heads_landed
+    uint32_t w32[4];
+};
+__device__ __forceinline__ HeadLoads load_head(const uint16_t* x, const uint16_t* weight,
+                                               uint32_t lane) {
+    HeadLoads h;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(x + lane * 4);
+    h.run[0] = words[0];
+    h.run[1] = words[1];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        h.x[c] = x[lane + 64 * c];
+        h.w[c] = weight[lane + 64 * c];
+    }
+    return h;
+}
+// The same loads issued as assembly, which the compiler does not count, for a caller that
+// places them itself among the requests of a kernel's first microsecond and waits for
+// them with heads_landed() (left to the compiler, a wait for these values would also wait
+// for every request issued behind them: it does not wait for part of a queue that holds
+// LDS transfers).
+__device__ __forceinline__ HeadLoads load_head_untracked(const uint16_t* x, const uint16_t* weight,
+                                                         uint32_t lane) {
+    HeadLoads h;
+    const uint16_t* words = x + lane * 4;
+    u32x2 run;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(run) : "v"(words));
+    h.run[0] = run[0];
+    h.run[1] = run[1];
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        uint32_t xv, wv;
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(xv) : "v"(x + lane + 64 * c));
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(wv) : "v"(weight + lane + 64 * c));
+        h.x32[c] = xv;
+        h.w32[c] = wv;
+    }
+    return h;
+}
+// Waits for every vector memory request of the wave and ties the registers of two
+// load_head_untracked to the wait.
+__device__ __forceinline__ void heads_landed(HeadLoads& a, HeadLoads& b) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(a.run[0]), "+v"(a.run[1]), "+v"(a.x32[0]), "+v"(a.x32[1]), "+v"(a.x32[2]),
+                   "+v"(a.x32[3]), "+v"(a.w32[0]), "+v"(a.w32[1]), "+v"(a.w32[2]), "+v"(a.w32[3]),
+                   "+v"(b.run[0]), "+v"(b.run[1]), "+v"(b.x32[0]), "+v"(b.x32[1]), "+v"(b.x32[2]),
+                   "+v"(b.x32[3]), "+v"(b.w32[0]), "+v"(b.w32[1]), "+v"(b.w32[2]), "+v"(b.w32[3]));
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        a.x[c] = static_cast<uint16_t>(a.x32[c]);
+        a.w[c] = static_cast<uint16_t>(a.w32[c]);
+        b.x[c] = static_cast<uint16_t>(b.x32[c]);
+        b.w[c] = static_cast<uint16_t>(b.w32[c]);
+    }
+}
+// Cosine and sine of the rotation of pair (lane & 31) at `position`: the same for every
+// head of a row, so a wave evaluates them once (one shared argument reduction) for all the
+// heads it norms.
+__device__ __forceinline__ RopeAngle rope_angle(uint32_t position, uint32_t lane) {
+    return rope_angle_of(position, rope_inverse_frequency(lane & (kAttnRopePairs - 1)));
+}
+__device__ __forceinline__ void norm_rope_head(const HeadLoads& h, const RopeAngle& angle,
+                                               uint32_t lane, float (&out)[4]) {
+    float acc = 0.0f;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const float v = __uint_as_float((j & 1) ? (h.run[j >> 1] & 0xFFFF0000u)
+                                                : (h.run[j >> 1] << 16));
+        acc += v * v;
+    }
+    acc = half_wave_sum(acc);
+    const float total = acc + __shfl_xor(acc, 32, 64);
+    const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
+#pragma unroll
+    for (uint32_t c = 0; c < 4; ++c) {
+        out[c] = round_bf16(bf16_bits_to_f32(h.w[c]) * round_bf16(bf16_bits_to_f32(h.x[c]) * inverse));
+    }
+    // dims below 64 rotate: lane l holds dim l, its partner (l ^ 32) the other half of the pair
+    const float n = out[0];
+    const float partner = __shfl_xor(n, kAttnRopePairs, 64);
+    const float rotated = lane < kAttnRopePairs ? fmaf(-partner, angle.s, n * angle.c)
+                                                : fmaf(partner, angle.s, n * angle.c);
+    out[0] = round_bf16(rotated);
+}
+
 // ------------------------------------------------------------ flash decode ---
 
 struct FlashArgs {
@@ -287,6 +444,12 @@ struct FlashArgs {
     uint32_t row_limit;         // rows the q / gate / out / table operands hold
     uint32_t interleave;        // 1: a row's workgroups take its 32-key blocks in turn
     uint32_t compact;           // 1: the splits that hold keys lead the dispatch order
+    uint32_t rotate;            // != 0: a workgroup starts (its place x rotate) blocks into its range
+    // rope form (flash_decode_kernel<true>): q is null, the query heads come from the
+    // projection rows and are normed and rotated by the workgroup itself
+    const uint16_t* projection; // [rows][projection_stride]: {q | gate} x 16, K x 2, V x 2
+    const uint16_t* q_weight;
+    uint32_t projection_stride;
 };
 
 // value of lane (l ^ 8) within each row of 16 lanes
@@ -304,8 +467,59 @@ __device__ __forceinline__ uint32_t pack_high(uint32_t a, uint32_t b) {
     return __builtin_amdgcn_perm(b, a, 0x07060302u);
 }
 
+// kRope: the token's query heads are taken from its projection row - normed and rotated by
+// the workgroup while its first blocks of keys and values are in flight - and the walk
+// covers the `context` cached keys only; the token's own key and value never pass through
+// the cache here, attention_finish_kernel folds them in and appends them.
+// Transfer kI of the 16 that bring a block of 32 key rows into a wave's LDS stage: rows kI
+// and 16 + kI (the lanes' halves), 1 KiB.  `from` = the block's first row + the lane's place.
+// The row's offset travels as the instruction's immediate (at most 4095, so two bases 4 KiB
+// apart); the hardware adds the immediate to the LDS address as well, so the destination is
+// given less that much.
+template <uint32_t kI>
+__device__ __forceinline__ void key_row_transfer(const uint8_t* from, uint8_t* stage) {
+    constexpr uint32_t kImmediate = (kI & 7) * kD * 2;
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(from + (kI >> 3) * 8 * kD * 2),
+        (__attribute__((address_space(3))) void*)(stage + kI * kLdsPairBytes - kImmediate), 16,
+        kImmediate, kStreamOnce);
+}
+template <uint32_t... kI>
+__device__ __forceinline__ void key_block_transfers(const uint8_t* from, uint8_t* stage,
+                                                    std::integer_sequence<uint32_t, kI...>) {
+    (key_row_transfer<kI>(from, stage), ...);
+}
+
+template <bool kRope>
 __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // (rope form) the rotation's inverse frequency of pair lane & 31
+    float inverse_frequency = 1.0f;
+    if constexpr (kRope) {
+        inverse_frequency = rope_inverse_frequency(threadIdx.x & (kAttnRopePairs - 1));
+        // The arguments of the rope form are fetched here, with the others: left to the
+        // compiler they are fetched where they are first used, behind the state table, one
+        // more trip to memory before the first block of keys can be requested.
+        asm volatile("" ::"s"(a.projection), "s"(a.q_weight), "s"(a.projection_stride));
+    }
+    // (rope form) The wave's two query heads as the projection holds them.  Requested at
+    // once where the grid position names the row, next to the state table; in the compact
+    // order, where the table names it, right behind the table.  Either way they are here
+    // before the walk's first requests go out: requested among those, they would wait in
+    // the memory system's queues behind the first blocks of every workgroup.
+    HeadLoads ql[2];
+    auto request_heads = [&](uint32_t of_row, uint32_t of_kvh) {
+        const uint16_t* proj = a.projection + static_cast<uint64_t>(of_row) * a.projection_stride;
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            ql[i] = load_head_untracked(
+                proj + (of_kvh * kAttnHeadsPerKv + (threadIdx.x >> 6) * 2 + i) * 2 * kD, a.q_weight,
+                threadIdx.x & 63);
+        }
+    };
+    if constexpr (kRope) {
+        if (!a.compact) request_heads(blockIdx.z, blockIdx.y);
+    }
     uint32_t split = blockIdx.x;
     uint32_t kvh = blockIdx.y;
     uint32_t row = blockIdx.z;
@@ -323,7 +537,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
         const u32x2 entry = *reinterpret_cast<const u32x2*>(a.table + min(l, gridDim.z - 1) * 4);
         uint32_t mine = 0;
         if (l < gridDim.z && entry[1] < a.capacity) {
-            const uint32_t keys = entry[1] + 1;
+            const uint32_t keys = kRope ? entry[1] : entry[1] + 1;
             if (!(a.long_rows_only && keys <= a.single_partition)) mine = (keys + a.part - 1) / a.part;
         }
         uint32_t through = mine;   // splits of rows 0 .. l
@@ -354,7 +568,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
         }
     }
     if (context >= a.capacity) return;  // a bad table row must not read outside the cache
-    const uint32_t n = context + 1;
+    const uint32_t n = kRope ? context : context + 1;
     if (a.long_rows_only && n <= a.single_partition) return;
     const uint32_t part = a.final_mode ? n : a.part;
     if (split * part >= n) return;
@@ -369,19 +583,27 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     const uint32_t block_stride = interleave ? row_splits : 1;
     const uint32_t key_end = interleave ? n : min(n, split * part + part);
 
-    const uint32_t wave = threadIdx.x >> 6;
+    // the wave index as a scalar: block numbers, key ranges and base addresses then stay in
+    // scalar registers, and a request is one instruction (scalar base + lane offset +
+    // immediate) instead of a 64-bit vector address computed per request
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t m = lane & 15;
     const uint32_t g = lane >> 4;
 
     // B operand of S^T: Q^T, column m holds head (m & 7)
-    const uint16_t* qh = a.q + static_cast<uint64_t>(row) * a.query_stride +
-                         (kvh * kAttnHeadsPerKv + (m & 7)) * kD;
     bf16x8 qreg[8];
+    if constexpr (kRope) {
+        if (a.compact) request_heads(row, kvh);
+        heads_landed(ql[0], ql[1]);
+    } else {
+        const uint16_t* qh = a.q + static_cast<uint64_t>(row) * a.query_stride +
+                             (kvh * kAttnHeadsPerKv + (m & 7)) * kD;
 #pragma unroll
-    for (uint32_t kb = 0; kb < 8; ++kb) {
-        qreg[kb] = __builtin_bit_cast(
-            bf16x8, *reinterpret_cast<const u32x4*>(qh + kb * 32 + g * 8));
+        for (uint32_t kb = 0; kb < 8; ++kb) {
+            qreg[kb] = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(qh + kb * 32 + g * 8));
+        }
     }
 
     const uint16_t* kbase = a.keys + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
@@ -397,15 +619,40 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     const uint32_t nblocks =
         interleave ? (row_blocks - split + row_splits - 1) / row_splits
                    : (key_end - first_block * kBlockKeys + kBlockKeys - 1) / kBlockKeys;
+    // Rotation: the workgroup walks its own blocks starting `turn` blocks in and wraps around
+    // (the online softmax does not care about the order).  Workgroups that advance in step
+    // through ranges a fixed stride apart then sit at different offsets of their ranges at any
+    // moment, so how the stride between ranges falls on the memory channels no longer decides
+    // whether their requests of the moment spread out or pile up.
+    const uint32_t turn =
+        (split + kvh * 5u + row * 11u) * a.rotate % nblocks;
+    auto own_block = [&](uint32_t blk) {
+        const uint32_t turned = blk + turn;
+        return first_block + (turned >= nblocks ? turned - nblocks : turned) * block_stride;
+    };
 
     // K rows go from HBM straight into the wave's LDS stage (no registers): one
     // instruction lands 1 KiB contiguous in LDS, lanes 0..31 fetching key i
     // (tile 0) and lanes 32..63 key 16+i (tile 1), so the two rows sharing LDS
     // banks are never read by the same operand load.
+    // A whole block of 32 keys is requested from one scalar base per eight transfers, the
+    // lane's place as a 32-bit offset and the row as the instruction's immediate (which the
+    // hardware adds to the LDS address as well: the destination is given less that much).
+    // Only a row's last, partial block takes the path that clamps every row to the last key.
+    constexpr uint32_t kRowBytes = kD * 2;
+    const uint32_t key_lane_bytes = (lane >> 5) * 16 * kRowBytes + (lane & 31) * 16;
+    const uint32_t value_lane_bytes = g * 4 * kRowBytes + m * 16;
+    const uint8_t* key_bytes = reinterpret_cast<const uint8_t*>(kbase);
+    const uint8_t* value_bytes = reinterpret_cast<const uint8_t*>(vbase);
     auto stage_keys = [&](uint32_t blk) {
-        const uint32_t key0 = (first_block + blk * block_stride) * kBlockKeys;
+        const uint32_t key0 = own_block(blk) * kBlockKeys;
         const uint32_t valid = min(kBlockKeys, key_end - key0);
-#pragma unroll
+        if (valid == kBlockKeys) {
+            const uint8_t* base = key_bytes + static_cast<uint64_t>(key0) * kRowBytes;
+            key_block_transfers(base + key_lane_bytes, stage, std::make_integer_sequence<uint32_t, 16>{});
+            return;
+        }
+#pragma unroll 1
         for (uint32_t i = 0; i < 16; ++i) {
             const uint32_t key = min(i + (lane >> 5) * 16, valid - 1);
             const uint16_t* src = kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8;
@@ -419,8 +666,17 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // V rows: contraction slot e of lane group g is key (e>>2)*16 + g*4 + (e&3);
     // one call fetches one 128-dim half (8 x 16 B per lane)
     auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
-        const uint32_t key0 = (first_block + blk * block_stride) * kBlockKeys;
+        const uint32_t key0 = own_block(blk) * kBlockKeys;
         const uint32_t valid = min(kBlockKeys, key_end - key0);
+        if (valid == kBlockKeys) {
+            const uint8_t* base = value_bytes + static_cast<uint64_t>(key0) * kRowBytes + hh * 256;
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) {
+                vhalf[e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
+                    base + (e >> 2) * 16 * kRowBytes + (e & 3) * kRowBytes + value_lane_bytes));
+            }
+            return;
+        }
 #pragma unroll
         for (uint32_t e = 0; e < 8; ++e) {
             const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
@@ -434,13 +690,45 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // requested as soon as the P.V products of block b have consumed that half's
     // registers, so a wave always has its next block in flight.
     u32x4 vreg[2][8];
-    if (wave < nblocks) {
+    if constexpr (kRope) {
+        // (by every wave, also one whose range holds no block for it: it fetches the last
+        // block again, and the norm below runs without a branch around the requests)
+        const uint32_t first = min(wave, nblocks - 1);
+        stage_keys(first);
+        load_values(vreg[0], first, 0);
+        load_values(vreg[1], first, 1);
+        // the requests above stay above the norm below (the scheduler would sink the
+        // value loads under it, towards their first use)
+        __builtin_amdgcn_sched_barrier(0);
+    } else if (wave < nblocks) {
         stage_keys(wave);
         load_values(vreg[0], wave, 0);
         load_values(vreg[1], wave, 1);
     }
+    if constexpr (kRope) {
+        // norm and rotation of the wave's two heads while the first blocks are under way;
+        // Q^T reaches the operand layout through 4 KiB of LDS behind the K stages.  The
+        // barrier waits for the LDS writes only, not for the transfers in flight.
+        __shared__ __attribute__((aligned(16))) uint16_t qs[kAttnHeadsPerKv * kD];
+        const RopeAngle angle = rope_angle_of(context, inverse_frequency);
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+            float nr[4];
+            norm_rope_head(ql[i], angle, lane, nr);
+#pragma unroll
+            for (uint32_t c = 0; c < 4; ++c) {
+                qs[(wave * 2 + i) * kD + lane + 64 * c] = f32_to_bf16_bits(nr[c]);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+        for (uint32_t kb = 0; kb < 8; ++kb) {
+            qreg[kb] = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4*>(qs + (m & 7) * kD + kb * 32 + g * 8));
+        }
+    }
     for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
-        const uint32_t valid = min(kBlockKeys, key_end - (first_block + blk * block_stride) * kBlockKeys);
+        const uint32_t valid = min(kBlockKeys, key_end - own_block(blk) * kBlockKeys);
         const bool more = blk + kWaves < nblocks;
         // every transfer issued so far (this block's K and V) has landed
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -718,67 +1006,6 @@ __device__ __forceinline__ StreamDeal deal_streams(const LayerArgs& a, uint32_t 
 // [g U / G, (g + 1) U / G): the largest g with g U / G <= u.
 __device__ __forceinline__ uint32_t group_of_unit(uint32_t u, uint32_t total, uint32_t groups) {
     return static_cast<uint32_t>(((static_cast<uint64_t>(u) + 1) * groups - 1) / total);
-}
-
-// One head of 256 values through RMS norm, weight and rotation by one wave; lane l
-// receives dims l, l + 64, l + 128, l + 192 as the fp32 of the stored bf16.  Operation for
-// operation attn_qk_rope_kernel: lane l's four squares are thread l's there, the same
-// half-wave tree, the same rounding points, the same cosine and sine.
-struct HeadLoads {
-    uint32_t run[2];      // values 4 l .. 4 l + 3 (sum of squares)
-    uint16_t x[4];        // values l + 64 c
-    uint16_t w[4];
-};
-__device__ __forceinline__ HeadLoads load_head(const uint16_t* x, const uint16_t* weight,
-                                               uint32_t lane) {
-    HeadLoads h;
-    const uint32_t* words = reinterpret_cast<const uint32_t*>(x + lane * 4);
-    h.run[0] = words[0];
-    h.run[1] = words[1];
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        h.x[c] = x[lane + 64 * c];
-        h.w[c] = weight[lane + 64 * c];
-    }
-    return h;
-}
-// Cosine and sine of the rotation of pair (lane & 31) at `position`: the same for every
-// head of a row, so a wave evaluates them once (one shared argument reduction) for all the
-// heads it norms.
-struct RopeAngle {
-    float c, s;
-};
-__device__ __forceinline__ RopeAngle rope_angle(uint32_t position, uint32_t lane) {
-    const uint32_t pair = lane & (kAttnRopePairs - 1);
-    const float inverse_frequency =
-        powf(kAttnRopeBase, static_cast<float>(pair) / static_cast<float>(kAttnRopePairs));
-    const float theta = static_cast<float>(position) / inverse_frequency;
-    RopeAngle a;
-    sincosf(theta, &a.s, &a.c);
-    return a;
-}
-__device__ __forceinline__ void norm_rope_head(const HeadLoads& h, const RopeAngle& angle,
-                                               uint32_t lane, float (&out)[4]) {
-    float acc = 0.0f;
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) {
-        const float v = __uint_as_float((j & 1) ? (h.run[j >> 1] & 0xFFFF0000u)
-                                                : (h.run[j >> 1] << 16));
-        acc += v * v;
-    }
-    acc = half_wave_sum(acc);
-    const float total = acc + __shfl_xor(acc, 32, 64);
-    const float inverse = 1.0f / sqrtf(total / static_cast<float>(kD) + kRmsNormEpsilon);
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        out[c] = round_bf16(bf16_bits_to_f32(h.w[c]) * round_bf16(bf16_bits_to_f32(h.x[c]) * inverse));
-    }
-    // dims below 64 rotate: lane l holds dim l, its partner (l ^ 32) the other half of the pair
-    const float n = out[0];
-    const float partner = __shfl_xor(n, kAttnRopePairs, 64);
-    const float rotated = lane < kAttnRopePairs ? fmaf(-partner, angle.s, n * angle.c)
-                                                : fmaf(partner, angle.s, n * angle.c);
-    out[0] = round_bf16(rotated);
 }
 
 // The new token's key (normed, rotated; fp32 of the stored bf16) and raw value for dims
@@ -1455,6 +1682,188 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
     a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
 }
 
+// ------------------------------------------- finish of the rope-form walk ----
+//
+// Second dispatch of the attention layer of a token wave whose first is
+// flash_decode_kernel<true>: merges the split records over the cached keys, folds in the
+// token itself - its key normed and rotated here, its value row as the projection holds
+// it - as one more record {numerator = V row, max = its score, sum = 1}, applies the gate
+// and appends the key and value rows to the cache.  Grid (16 heads, rows) x 256, thread d
+// = dimension d.  The norm and the rotation are attn_qk_rope_kernel's, operation for
+// operation, so the appended key row is that kernel's bit for bit.
+
+struct FinishArgs {
+    const uint16_t* projection;   // [rows][projection_stride]: {q | gate} x 16, K x 2, V x 2
+    const uint16_t* q_weight;
+    const uint16_t* k_weight;
+    uint16_t* keys;               // pools; row r's cache at + table[4 r] elements
+    uint16_t* values;
+    const uint32_t* table;        // per row {kv element offset, context, -, -}
+    const float* partials;        // [row][16][record_splits][258]
+    uint16_t* out;                // [rows][query_stride]
+    uint32_t capacity;
+    uint32_t projection_stride;
+    uint32_t query_stride;
+    uint32_t part;
+    uint32_t record_splits;
+    uint64_t partial_row_floats;
+};
+
+struct MergedParts {
+    float acc, denom, gmax;   // sum_p w_p num_p[d], sum_p w_p sum_p, w_p = exp(max_p - gmax)
+};
+
+// Numerators of up to kParts records requested at once by the thread that owns the
+// dimension; their maxima and sums go through LDS (one thread per record).  The caller
+// places a barrier between request_parts and reduce_parts.
+template <uint32_t kParts>
+__device__ __forceinline__ void request_parts(const float* base, uint32_t nparts, uint32_t d,
+                                              float (&numerator)[kParts], float* part_max,
+                                              float* part_sum) {
+    const uint32_t last = nparts == 0 ? 0u : nparts - 1;
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; ++p) {
+        numerator[p] = base[static_cast<uint64_t>(min(p, last)) * kAttnRecordFloats + d];
+    }
+    if (d < kParts) {
+        const float* rec = base + static_cast<uint64_t>(min(d, last)) * kAttnRecordFloats;
+        part_max[d] = d < nparts ? rec[kD] : -INFINITY;
+        part_sum[d] = rec[kD + 1];
+    }
+}
+template <uint32_t kParts>
+__device__ __forceinline__ MergedParts reduce_parts(const float (&numerator)[kParts], uint32_t nparts,
+                                                    const float* part_max, const float* part_sum) {
+    MergedParts r{0.0f, 0.0f, -INFINITY};
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; p += 4) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
+        r.gmax = fmaxf(fmaxf(r.gmax, m4[0]), fmaxf(fmaxf(m4[1], m4[2]), m4[3]));
+    }
+#pragma unroll
+    for (uint32_t p = 0; p < kParts; p += 4) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(part_sum + p);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            if (p + u < nparts) {
+                const float w = m4[u] == -INFINITY ? 0.0f : __expf(m4[u] - r.gmax);
+                r.acc = fmaf(w, numerator[p + u], r.acc);
+                r.denom += w * s4[u];
+            }
+        }
+    }
+    return r;
+}
+
+template <uint32_t kParts>
+__device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t head, uint32_t row,
+                                                uint32_t d, uint64_t kv_offset, uint32_t context,
+                                                uint32_t nparts) {
+    __shared__ __attribute__((aligned(16))) float part_max[kParts];
+    __shared__ __attribute__((aligned(16))) float part_sum[kParts];
+    __shared__ float wave_values[3][4];   // squares of the query head, of the key head, q . k
+    const uint32_t kvh = head / kAttnHeadsPerKv;
+    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
+    const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
+                        static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
+    // every load of the kernel is requested here, before the first is used
+    const float inverse_frequency = rope_inverse_frequency(d & (kAttnRopePairs - 1));
+    const uint16_t xq = proj[head * 2 * kD + d];
+    const uint16_t gate = proj[head * 2 * kD + kD + d];
+    const uint16_t xk = proj[kAttnQGateRows + kvh * kD + d];
+    const uint16_t vraw = proj[kAttnVRowOffset + kvh * kD + d];
+    const uint16_t wq = a.q_weight[d];
+    const uint16_t wk = a.k_weight[d];
+    float numerator[kParts];
+    request_parts<kParts>(base, nparts, d, numerator, part_max, part_sum);
+
+    // the rotation's cosine and sine, while the loads are in flight
+    float c = 1.0f, sn = 0.0f;
+    if (d < 2 * kAttnRopePairs) {
+        const RopeAngle angle = rope_angle_of(context, inverse_frequency);
+        c = angle.c;
+        sn = angle.s;
+    }
+    const float fq = bf16_bits_to_f32(xq);
+    const float fk = bf16_bits_to_f32(xk);
+    const float q_slices = wave_square_slices(fq * fq);
+    const float k_slices = wave_square_slices(fk * fk);
+    if ((d & 63) == 0) {
+        wave_values[0][d >> 6] = q_slices;
+        wave_values[1][d >> 6] = k_slices;
+    }
+    __syncthreads();   // also publishes the records' maxima and sums
+    const float q_total = (wave_values[0][0] + wave_values[0][1]) + (wave_values[0][2] + wave_values[0][3]);
+    const float k_total = (wave_values[1][0] + wave_values[1][1]) + (wave_values[1][2] + wave_values[1][3]);
+    const float q_inverse = 1.0f / sqrtf(q_total / static_cast<float>(kD) + kRmsNormEpsilon);
+    const float k_inverse = 1.0f / sqrtf(k_total / static_cast<float>(kD) + kRmsNormEpsilon);
+    const float nq = round_bf16(bf16_bits_to_f32(wq) * round_bf16(fq * q_inverse));
+    const float nk = round_bf16(bf16_bits_to_f32(wk) * round_bf16(fk * k_inverse));
+    const float q_partner = __shfl_xor(nq, static_cast<int>(kAttnRopePairs), 64);
+    const float k_partner = __shfl_xor(nk, static_cast<int>(kAttnRopePairs), 64);
+    float q_rotated = nq, k_rotated = nk;
+    if (d < 2 * kAttnRopePairs) {
+        q_rotated = d < kAttnRopePairs ? fmaf(-q_partner, sn, nq * c) : fmaf(q_partner, sn, nq * c);
+        k_rotated = d < kAttnRopePairs ? fmaf(-k_partner, sn, nk * c) : fmaf(k_partner, sn, nk * c);
+    }
+    const uint16_t k_bits = f32_to_bf16_bits(k_rotated);
+    // the token's score from the stored (bf16) query and key, as the walk scores cached keys
+    float dot = round_bf16(q_rotated) * bf16_bits_to_f32(k_bits);
+    dot = half_wave_sum(dot);
+    dot += __shfl_xor(dot, 32, 64);
+    if ((d & 63) == 0) wave_values[2][d >> 6] = dot;
+    MergedParts merged = reduce_parts<kParts>(numerator, nparts, part_max, part_sum);
+    __syncthreads();
+    if constexpr (kParts == 128) {
+        // more than 128 records (a cache far deeper than the split was chosen for): the same
+        // in batches of 128, merged as they come
+        for (uint32_t p0 = kParts; p0 < nparts; p0 += kParts) {
+            const uint32_t count = min(kParts, nparts - p0);
+            request_parts<kParts>(base + static_cast<uint64_t>(p0) * kAttnRecordFloats, count, d,
+                                  numerator, part_max, part_sum);
+            __syncthreads();
+            const MergedParts next = reduce_parts<kParts>(numerator, count, part_max, part_sum);
+            __syncthreads();
+            const float g = fmaxf(merged.gmax, next.gmax);
+            const float w_old = merged.gmax == -INFINITY ? 0.0f : __expf(merged.gmax - g);
+            const float w_next = next.gmax == -INFINITY ? 0.0f : __expf(next.gmax - g);
+            merged.acc = fmaf(w_old, merged.acc, w_next * next.acc);
+            merged.denom = fmaf(w_old, merged.denom, w_next * next.denom);
+            merged.gmax = g;
+        }
+    }
+    const float s_new =
+        ((wave_values[2][0] + wave_values[2][1]) + (wave_values[2][2] + wave_values[2][3])) * kAttnScale;
+    const float gmax = fmaxf(merged.gmax, s_new);
+    const float w_parts = merged.gmax == -INFINITY ? 0.0f : __expf(merged.gmax - gmax);
+    const float w_new = __expf(s_new - gmax);
+    const float acc = fmaf(w_new, bf16_bits_to_f32(vraw), w_parts * merged.acc);
+    const float denom = fmaf(w_parts, merged.denom, w_new);
+    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
+    a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(gate));
+    if (head % kAttnHeadsPerKv == 0) {
+        const uint64_t slot = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + d;
+        a.keys[slot] = k_bits;
+        a.values[slot] = vraw;
+    }
+}
+
+__global__ __launch_bounds__(256) void attention_finish_kernel(FinishArgs a) {
+    const uint32_t head = blockIdx.x;
+    const uint32_t row = blockIdx.y;
+    const uint32_t d = threadIdx.x;
+    const uint64_t kv_offset = a.table[row * 4];
+    const uint32_t context = a.table[row * 4 + 1];
+    // a row the table places outside its cache has no records and no slot to append to
+    if (context >= a.capacity) return;
+    const uint32_t nparts = (context + a.part - 1) / a.part;
+    if (nparts > a.record_splits) return;
+    if (nparts <= 32) return finish_row_head<32>(a, head, row, d, kv_offset, context, nparts);
+    if (nparts <= 64) return finish_row_head<64>(a, head, row, d, kv_offset, context, nparts);
+    return finish_row_head<128>(a, head, row, d, kv_offset, context, nparts);
+}
+
 // ---------------------------------------- separate score / value stages ------
 
 // attention_decode_scores_gqa4: one workgroup per (head, partition); thread t
@@ -1656,8 +2065,13 @@ int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream
 namespace {
 
 int32_t launch_flash(const FlashArgs& f, uint32_t splits, uint32_t rows, hipStream_t stream) {
-    hipLaunchKernelGGL(flash_decode_kernel, dim3(splits, kAttnKvHeads, rows), dim3(256),
-                       kWaves * kWaveLdsBytes, stream, f);
+    if (f.projection != nullptr) {
+        hipLaunchKernelGGL(flash_decode_kernel<true>, dim3(splits, kAttnKvHeads, rows), dim3(256),
+                           kWaves * kWaveLdsBytes, stream, f);
+    } else {
+        hipLaunchKernelGGL(flash_decode_kernel<false>, dim3(splits, kAttnKvHeads, rows), dim3(256),
+                           kWaves * kWaveLdsBytes, stream, f);
+    }
     return TT_OK;
 }
 
@@ -1787,6 +2201,7 @@ int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stre
     f.long_rows_only = a.constant(9) & 1;
     f.interleave = (a.constant(9) >> 1) & 1;
     f.compact = (a.constant(9) >> 2) & 1;
+    f.rotate = (a.constant(9) >> 3) & 31;
     f.single_partition = kAttnPartition;
     const uint32_t rows = static_cast<uint32_t>(g.gz);
     a.require(f.capacity != 0 && f.query_stride >= kAttnQueryValues && f.part != 0 &&
@@ -1838,6 +2253,87 @@ int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t st
     if (a.status != TT_OK || validate_only) return a.status;
     hipLaunchKernelGGL(attention_combine_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
                        c);
+    return TT_OK;
+}
+
+// Bindings shared by the two dispatches of a token wave's attention layer in the rope form:
+// b0 projection slab [rows][projection stride], b1 q_w, b2 k_w, b3 keys_pool, b4 values_pool,
+// b5 state_table, b6 split records [rows][16][max_splits][258] fp32, b7 out slab
+// [rows][query stride], c8 capacity, c9 projection stride, c10 query stride, c11 part (keys
+// per workgroup, multiple of 32), c12 max_splits, c13 bit 1 interleave, bit 2 compact, bits
+// 3..7 rotate (as c9 of attention_decode_split_ms).
+struct TokenLayer {
+    FlashArgs walk;
+    FinishArgs finish;
+    uint32_t rows;
+};
+TokenLayer token_layer_args(Args& a, uint32_t rows) {
+    TokenLayer t{};
+    FlashArgs& f = t.walk;
+    FinishArgs& n = t.finish;
+    t.rows = rows;
+    f.capacity = n.capacity = a.constant(8);
+    f.projection_stride = n.projection_stride = a.constant(9);
+    n.query_stride = a.constant(10);
+    f.part = n.part = a.constant(11);
+    f.record_splits = n.record_splits = a.constant(12);
+    const uint32_t flags = a.constant(13);
+    f.interleave = (flags >> 1) & 1;
+    f.compact = (flags >> 2) & 1;
+    f.rotate = (flags >> 3) & 31;
+    a.require(rows >= 1 && rows <= kMaxBatchRows, TT_CMD_INVALID_DISPATCH_EXTENT);
+    a.require(f.capacity != 0 && f.projection_stride >= kAttnProjectionRows &&
+                  f.projection_stride % 4 == 0 && n.query_stride >= kAttnQueryValues &&
+                  f.part != 0 && f.part % kBlockKeys == 0 && f.record_splits != 0 &&
+                  static_cast<uint64_t>(f.record_splits) * f.part >= f.capacity,
+              TT_CMD_INVALID_BUFFER);
+    if (a.status != TT_OK) return t;
+    const uint64_t last = rows - 1;
+    f.partial_row_floats = n.partial_row_floats =
+        static_cast<uint64_t>(kAttnQueryHeads) * f.record_splits * kAttnRecordFloats;
+    f.projection = n.projection =
+        a.buffer<const uint16_t>(0, (last * f.projection_stride + kAttnProjectionRows) * 2);
+    f.q_weight = n.q_weight = a.buffer<const uint16_t>(1, kD * 2);
+    n.k_weight = a.buffer<const uint16_t>(2, kD * 2);
+    n.keys = a.buffer<uint16_t>(3, cache_bytes(f.capacity));
+    n.values = a.buffer<uint16_t>(4, cache_bytes(f.capacity));
+    f.keys = n.keys;
+    f.values = n.values;
+    f.table = n.table = a.buffer<const uint32_t>(5, rows * 16);
+    f.partials = a.buffer<float>(6, f.partial_row_floats * rows * 4);
+    n.partials = f.partials;
+    n.out = a.buffer<uint16_t>(7, (last * n.query_stride + kAttnQueryValues) * 2);
+    // the table rows are read as 8-byte pairs
+    a.require(reinterpret_cast<uintptr_t>(f.table) % 8 == 0, TT_CMD_INVALID_BUFFER_OFFSET);
+    return t;
+}
+
+// attention_decode_token_ms (no reference counterpart; attn_qk_rope_ms and the split path of
+// decode_step.cpp:1231-1259 for every row in one dispatch): bindings above; grid
+// (max_splits, 2, rows) x 256.  Writes the split records over the cached keys; the token's
+// own key and value are folded in, and appended, by attention_decode_token_finish_ms.
+int32_t op_attention_token_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                              bool validate_only) {
+    Args a(b);
+    const uint32_t rows = static_cast<uint32_t>(std::min<uint64_t>(g.gz, 0xFFFF));
+    TokenLayer t = token_layer_args(a, rows);
+    a.require(g.gx == t.walk.record_splits && g.gy == 2 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    return launch_flash(t.walk, t.walk.record_splits, rows, stream);
+}
+
+// attention_decode_token_finish_ms: bindings above; grid (16, rows) x 256.
+int32_t op_attention_token_finish_ms(const Bindings& b, const Grid& g, hipStream_t stream,
+                                     bool validate_only) {
+    Args a(b);
+    const uint32_t rows = static_cast<uint32_t>(std::min<uint64_t>(g.gy, 0xFFFF));
+    TokenLayer t = token_layer_args(a, rows);
+    a.require(g.gx == kAttnQueryHeads && g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1,
+              TT_CMD_INVALID_DISPATCH_EXTENT);
+    if (a.status != TT_OK || validate_only) return a.status;
+    hipLaunchKernelGGL(attention_finish_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
+                       t.finish);
     return TT_OK;
 }
 
@@ -1997,7 +2493,10 @@ bool prepare_current_device() {
     }
     if (g_decode_ready[device]) return true;
     // 4 x 16.5 KiB of LDS is above the 64 KiB a kernel gets without opting in
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kWaves * kWaveLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWaves * kWaveLdsBytes) != hipSuccess ||
         hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel<true>),
@@ -2045,6 +2544,8 @@ const KernelDesc kAttentionDecodeKernels[] = {
     {"attention_decode_values_gqa8", op_attention_values},
     {"attention_decode_split_ms", op_attention_split_ms},
     {"attention_decode_combine_ms", op_attention_combine_ms},
+    {"attention_decode_token_ms", op_attention_token_ms},
+    {"attention_decode_token_finish_ms", op_attention_token_finish_ms},
     {"attention_decode_layer_ms", op_attention_layer_ms},
     {"attention_decode_layer_finish_ms", op_attention_layer_finish_ms},
 };
