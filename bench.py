@@ -6,10 +6,9 @@ family of the whole 40-layer hybrid stack, G,G,G,A x 10 (30 Gated DeltaNet layer
 full-attention layers), with the lane-batched operators:
     GDN:       gdn_decode_fused_ms (prepare + recurrence + gate-norm in one dispatch)
     attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms, or
-               with --attention layer attention_decode_layer_ms +
-               attention_decode_layer_finish_ms (qk-norm, rotation, K / V append, split-K
-               attention over keys dealt evenly to the workgroups and the gated combine in
-               two dispatches; same layer time, slower key walk)
+               with --attention token attention_decode_token_ms +
+               attention_decode_token_finish_ms (qk-norm and rotation inside the split-K walk;
+               the token's own key and value folded in and appended by the finishing dispatch)
 Projections (the reference's Q4 GEMVs) are not on the path: their outputs are resident
 random bf16 slabs.  Every layer has its own KV pools, recurrent state and inputs, all in
 HBM before the timed region (2.7 GB of keys and values: the 256 MB last-level cache cannot
@@ -68,10 +67,6 @@ CONFIG3 = {
 }
 
 
-def layer_scratch_bytes(groups, rows):
-    return 256 + 131072 + (groups + 2 * rows - 1) * 8 * 258 * 4
-
-
 class Wave:
     """Buffers and recorders of the attention family of one token wave."""
 
@@ -105,7 +100,6 @@ class Wave:
         self.b_q, self.b_gate, self.b_out = (dev.create_buffer(rows * 8192) for _ in range(3))
         # records down to the finest split the rule picks (128 keys)
         self.b_part = dev.create_buffer(rows * 16 * ((capacity + 127) // 128) * 258 * 4)
-        self.b_scratch = dev.create_buffer(layer_scratch_bytes(self.groups, rows))
         conv_elems, rec_elems = 3 * 8192, 32 * 128 * 128
         table = np.zeros(64, np.uint32)
         for r in range(rows):
@@ -148,7 +142,10 @@ class Wave:
         self.part = self.forced_split or stack_rules.choose_split_keys(visible, self.dev.compute_units)
         self.max_splits = (self.capacity + self.part - 1) // self.part
         self.interleave = 1 if self.rows <= 2 else 0
-        self.rotate = getattr(self, "rotate", 0)
+        # contiguous ranges are walked from a rotated starting block, so that the stride
+        # between ranges (the cache capacity) does not decide how the requests of the moment
+        # fall on the memory channels
+        self.rotate = 0 if self.interleave else 1
         live = stack_rules.split_workgroups(visible, self.part)
         grid = self.max_splits * 2 * self.rows
         self.compact = 1 if grid > live and grid > self.dev.compute_units else 0
@@ -173,23 +170,13 @@ class Wave:
     def record_attention(self, cb, index, walk_only=False):
         """All dispatches of one attention layer; walk_only: the key-walk kernel alone."""
         layer, rows, cap, P = self.attn[index], self.rows, self.capacity, self.lib.pipeline
-        if self.attention == "layer":
-            bind = {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: layer["keys"],
-                    4: layer["values"], 5: self.attn_table, 6: self.b_scratch, 7: self.b_out}
-            const = {8: cap, 9: 9216, 10: 4096}
-            cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: 0}, (self.groups, rows),
-                      (256,))
-            if not walk_only:
-                cb.barrier()
-                cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: self.groups},
-                          (16, rows), (64,))
-            return
         if self.attention == "token":
             splits = (cap + self.token_part - 1) // self.token_part
             bind = {0: layer["proj"], 1: layer["q_w"], 2: layer["k_w"], 3: layer["keys"],
                     4: layer["values"], 5: self.attn_table, 6: self.b_part, 7: self.b_out}
             const = {8: cap, 9: 9216, 10: 4096, 11: self.token_part, 12: splits,
-                     13: 2 * self.interleave + 4 * self.token_compact + 8 * self.rotate}
+                     13: 2 * self.interleave + 4 * self.token_compact + 8 * self.rotate,
+                     14: -(-max(self.contexts) // self.token_part)}
             cb.encode(P("attention_decode_token_ms"), bind, const, (splits, 2, rows), (256,))
             if not walk_only:
                 cb.barrier()
@@ -210,7 +197,7 @@ class Wave:
             cb.barrier()
             cb.encode(P("attention_decode_combine_ms"),
                       {0: self.b_part, 1: self.b_gate, 2: self.attn_table, 3: self.b_out},
-                      {4: self.part, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
+                      {4: self.part, 5: self.max_splits, 6: 4096, 7: 0, 8: cap}, (16, rows), (256,))
 
     def record_wave(self, cb):
         gdn = attn = 0
@@ -256,8 +243,8 @@ def attention_figures(queue, wave):
     algo = wave.visible_keys() * ATTN_BYTES_PER_KEY
     gbs = algo / (walk["median_us"] * 1e-6) / 1e9
     return {"lanes_visible_keys": [c + 1 for c in wave.contexts], "algorithmic_bytes": algo,
-            "split_keys": wave.part if wave.attention == "three" else None,
-            "workgroups_with_keys_first": bool(wave.compact) if wave.attention == "three" else None,
+            "split_keys": wave.part if wave.attention == "three" else wave.token_part,
+            "workgroups_with_keys_first": bool(wave.compact if wave.attention == "three" else wave.token_compact),
             "walk_kernel": walk, "walk_kernel_gbs": round(gbs, 1),
             "walk_kernel_frac": round(gbs / HBM_PEAK_GBS, 4),
             "layer_all_dispatches": layer,
@@ -473,9 +460,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--attention", choices=("layer", "three", "token"), default="three",
-                    help="three: rope, split and combine dispatches (the faster key walk); layer: one "
-                         "dispatch for the layer plus its finishing dispatch")
+    ap.add_argument("--attention", choices=("three", "token"), default="three",
+                    help="three: rope, split and combine dispatches (the faster key walk); token: the "
+                         "walk norms and rotates the query heads itself, a finishing dispatch folds "
+                         "in the token's own key and value")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the 16384-row block prefill figures in detail.prefill_16k")
@@ -534,8 +522,8 @@ def main():
                      len(wave.gdn))
     gdn_gbs = LANES * GDN_BYTES_PER_LANE_LAYER / (gdn["median_us"] * 1e-6) / 1e9
     walk = uniform["walk_kernel"]
-    kernel_name = ("attention_decode_layer_ms (attention_decode_layer_kernel)"
-                   if args.attention == "layer" else "attention_decode_split_ms (flash_decode_kernel)")
+    kernel_name = ("attention_decode_token_ms (flash_decode_kernel, rope form)"
+                   if args.attention == "token" else "attention_decode_split_ms (flash_decode_kernel)")
     line = {
         "metric": "decode attn+GDN us/layer @32k ctx x4 lanes",
         "value": round(ms_per_step * 1e3 / LAYERS, 3),
@@ -554,7 +542,7 @@ def main():
                                "own KV / state per layer), one HIP-graph replay per wave",
                    "lanes": LANES, "visible_keys": VISIBLE, "capacity": CAPACITY, "layers": LAYERS,
                    "attention_form": args.attention, "workgroups": wave.groups,
-                   "split_keys": wave.part if args.attention == "three" else None,
+                   "split_keys": wave.part if args.attention == "three" else wave.token_part,
                    "device": dev.name},
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": uniform["walk_kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -290,6 +290,22 @@ int32_t tt_attention_decode_lanes_static(tt_queue* queue, const void* q, uint64_
                                          uint64_t out_bytes, uint32_t rows, uint32_t capacity,
                                          uint32_t query_stride, uint32_t split_keys);
 
+/* ---- planning of the split-K walk of a token wave ----------------------------------
+ * The reference plans its split path per lane on the host (a fixed 256-key partition,
+ * src/runtime/decode_step.cpp:1249-1259; include/tatara/runtime/decode_geometry.h:133-146
+ * attention_partitions).  Here one grid serves every lane of a wave, and how many keys a
+ * workgroup takes decides how well that grid fills the chip; the rule lives in the library
+ * so that every caller (the C++ runtime, the Python mirror, a serving loop) plans alike.
+ *
+ * tt_split_workgroups: workgroups of one attention layer's split-K grid that hold keys
+ * when lane r sees visible_keys[r] keys and a workgroup takes split_keys of them
+ * (two kv heads x sum of ceil(keys / split_keys)); 0 for split_keys == 0.
+ * tt_choose_split_keys: the finest multiple of 32, at least 128, with which those
+ * workgroups fit compute_units one each (a lane count above compute_units / 2 cannot
+ * fit and gets the even share). */
+uint32_t tt_split_workgroups(const uint32_t* visible_keys, uint32_t rows, uint32_t split_keys);
+uint32_t tt_choose_split_keys(const uint32_t* visible_keys, uint32_t rows, uint32_t compute_units);
+
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = [
     "tt_command_buffer_reset", "tt_command_buffer_compile", "tt_command_buffer_set_profiling",
     "tt_command_name", "tt_command_gpu_ms", "tt_attention_decode_lanes_static",
     "tt_event_create", "tt_event_destroy", "tt_encode_signal_event", "tt_encode_wait_for_event",
+    "tt_split_workgroups", "tt_choose_split_keys",
 ]
 
 
@@ -102,6 +103,8 @@ def lib():
         "tt_command_name": (C.c_char_p, [vp, u32]),
         "tt_command_gpu_ms": (i32, [vp, u32, C.POINTER(C.c_double)]),
         "tt_attention_decode_lanes_static": (i32, [vp] + [vp, u64] * 6 + [u32] * 4),
+        "tt_split_workgroups": (u32, [C.POINTER(u32), u32, u32]),
+        "tt_choose_split_keys": (u32, [C.POINTER(u32), u32, u32]),
         "tt_event_create": (i32, [vp, pvp]), "tt_event_destroy": (None, [vp]),
         "tt_encode_signal_event": (i32, [vp, vp, u64]),
         "tt_encode_wait_for_event": (i32, [vp, vp, u64]),
@@ -435,3 +438,20 @@ class CommandBuffer:
 
     def __del__(self, _release=_release):
         _release(self, "tt_command_buffer_destroy")
+
+
+def _u32_array(values):
+    values = [int(v) for v in values]
+    return (C.c_uint32 * max(len(values), 1))(*values), len(values)
+
+
+def split_workgroups(visible_keys, split_keys):
+    """Workgroups of one attention layer's split-K grid that hold keys (tt_split_workgroups)."""
+    array, count = _u32_array(visible_keys)
+    return int(lib().tt_split_workgroups(array, count, int(split_keys)))
+
+
+def choose_split_keys(visible_keys, compute_units=256):
+    """Keys per split-K workgroup for a token wave (tt_choose_split_keys)."""
+    array, count = _u32_array(visible_keys)
+    return int(lib().tt_choose_split_keys(array, count, int(compute_units)))

@@ -182,27 +182,15 @@ std::uint32_t attention_partitions(std::uint32_t context) {
 
 std::uint32_t split_workgroups(std::span<const std::uint32_t> visible_keys,
                                std::uint32_t split_keys) noexcept {
-    std::uint64_t groups = 0;
-    for (const std::uint32_t keys : visible_keys) {
-        groups += 2 * ((std::uint64_t{keys} + split_keys - 1) / split_keys);   // two kv heads
-    }
-    return static_cast<std::uint32_t>(std::min<std::uint64_t>(groups, UINT32_MAX));
+    // the rule lives in the backend library, one implementation for every caller
+    return tt_split_workgroups(visible_keys.data(), static_cast<std::uint32_t>(visible_keys.size()),
+                               split_keys);
 }
 
 std::uint32_t choose_split_keys(std::span<const std::uint32_t> visible_keys,
                                 std::uint32_t compute_units) noexcept {
-    const std::uint64_t units = std::max<std::uint32_t>(compute_units, 1);
-    std::uint64_t total = 0;
-    for (const std::uint32_t keys : visible_keys) total += keys;
-    // an even share of all keys, then coarser until the last, partly filled split of every
-    // row fits too: one workgroup more than compute units costs a third of the walk
-    std::uint64_t split = std::max<std::uint64_t>(((2 * total + units - 1) / units + 31) / 32 * 32, 128);
-    while (split < UINT32_MAX - 31 &&
-           split_workgroups(visible_keys, static_cast<std::uint32_t>(split)) > units &&
-           2 * visible_keys.size() <= units) {
-        split += 32;
-    }
-    return static_cast<std::uint32_t>(split);
+    return tt_choose_split_keys(visible_keys.data(), static_cast<std::uint32_t>(visible_keys.size()),
+                                compute_units);
 }
 
 std::uint32_t choose_split_keys(std::uint32_t rows, std::uint32_t keys,
@@ -237,8 +225,8 @@ DecodePipelinesResult resolve_decode_pipelines(const HipLibrary& library) {
         resolve(library, p, &P::attention_decode_ms, "attention_decode_ms", error) &&
         resolve(library, p, &P::attention_split_ms, "attention_decode_split_ms", error) &&
         resolve(library, p, &P::attention_combine_ms, "attention_decode_combine_ms", error) &&
-        resolve(library, p, &P::attention_layer_ms, "attention_decode_layer_ms", error) &&
-        resolve(library, p, &P::attention_layer_finish_ms, "attention_decode_layer_finish_ms",
+        resolve(library, p, &P::attention_token_ms, "attention_decode_token_ms", error) &&
+        resolve(library, p, &P::attention_token_finish_ms, "attention_decode_token_finish_ms",
                 error);
     if (!ok) return {error, std::nullopt};
     return {HipPipelineError::None, std::move(p)};
@@ -411,16 +399,7 @@ DecodeBatchScratchResult create_decode_batch_scratch(const HipDevice& device,
         !allocate_zeroed(device, table_bytes, b.state_offsets)) {
         return {DecodeStepError::BufferAllocationFailed, std::nullopt};
     }
-    // whole-layer attention: one workgroup per compute unit; 256 B of tickets, 128 KiB of
-    // query heads, then one record of 8 x 258 floats per workgroup and stream boundary
     b.compute_units = std::max<std::uint32_t>(device.compute_units(), 1);
-    b.layer_groups = b.compute_units;
-    const std::uint64_t layer_scratch_bytes =
-        256 + 131072 +
-        (std::uint64_t{b.layer_groups} + 2 * rows - 1) * 8 * kAttentionRecordFloats * kF32Bytes;
-    if (!allocate_zeroed(device, layer_scratch_bytes, b.attn_layer_scratch)) {
-        return {DecodeStepError::BufferAllocationFailed, std::nullopt};
-    }
     return {DecodeStepError::None, std::move(b)};
 }
 
@@ -510,8 +489,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
     const std::uint32_t rows = static_cast<std::uint32_t>(streams.size());
     if (rows == 0 || rows > batch.rows || rows > kMaximumBatchRows ||
         pool.layers.size() != step.schedule.size() || pool.stripes == 0 || !batch.state_offsets ||
-        weights.size() != step.schedule.size() || batch.split_keys % 32u != 0 ||
-        (batch.attention_whole_layer && (batch.layer_groups == 0 || !batch.attn_layer_scratch))) {
+        weights.size() != step.schedule.size() || batch.split_keys % 32u != 0) {
         return HipCommandError::InvalidStreamGroup;
     }
     for (std::size_t index = 0; index < streams.size(); ++index) {
@@ -541,18 +519,25 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
 
     const DecodeGeometry& g = step.geometry;
     const std::uint64_t bucket_offset = step.schedule.size() * 256;
+    // Which rows take the split path: those with more than one 256-key partition - or, in the
+    // token form, every row (its walk covers the cached keys only, the token itself is folded
+    // in by the finishing dispatch).
+    const bool token_form = batch.attention_token_form;
     bool any_long = false;
     for (const DecodeStream& s : streams) any_long |= attention_partitions(s.context) != 1;
     // Keys per split-K workgroup: chosen from the depths of the rows that take the split
     // path, but no finer than 4096 workgroups over the capacity.  The grid always covers the
     // capacity (the operator reads the contexts on the device and refuses a grid that could
     // miss keys); where that leaves workgroups without keys in a grid larger than the chip,
-    // the ones with keys are placed first in the dispatch order (bit 2 of the operator's c9).
+    // the ones with keys are placed first in the dispatch order (bit 2 of the flags).
     std::array<std::uint32_t, kMaximumBatchRows> visible{};
     std::size_t long_rows = 0;
+    std::uint32_t deepest = 0;
     for (const DecodeStream& s : streams) {
-        if (attention_partitions(s.context) != 1 && long_rows < visible.size()) {
-            visible[long_rows++] = s.context + 1;
+        const bool splits = token_form ? s.context != 0 : attention_partitions(s.context) != 1;
+        if (splits && long_rows < visible.size()) {
+            visible[long_rows++] = token_form ? s.context : s.context + 1;
+            deepest = std::max(deepest, visible[long_rows - 1]);
         }
     }
     const std::span<const std::uint32_t> long_keys(visible.data(), long_rows);
@@ -565,10 +550,24 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                               static_cast<std::uint32_t>(std::min<std::uint64_t>(coarsest, 1u << 30)));
     }
     const std::uint32_t max_splits = (step.capacity + split_keys - 1) / split_keys;
-    if (any_long && batch.attn_partials.size_bytes() <
-                        std::uint64_t{rows} * 16 * max_splits * kAttentionRecordFloats * kF32Bytes) {
+    if ((any_long || token_form) &&
+        batch.attn_partials.size_bytes() <
+            std::uint64_t{rows} * 16 * max_splits * kAttentionRecordFloats * kF32Bytes) {
         return HipCommandError::InvalidBuffer;
     }
+    // Flags of the split-K walk.  Bit 1: waves of one or two lanes deal a lane's 32-key
+    // blocks to its workgroups in turn (measured 1-3 % faster there, 3 % slower at four
+    // lanes).  Bit 2: the grid is larger than the chip and part of it holds no keys, so the
+    // workgroups that do go first (0.4 us dearer than the order by grid position where that
+    // is not so).  Bits 3..7: workgroups that take consecutive ranges start a rotated number
+    // of blocks into them, so that the stride between ranges - the cache capacity - does
+    // not decide how their requests of the moment fall on the memory channels (the same
+    // 4 x 32768 keys took 46-77 us over capacities 32768 ... 131136 without, 46-48 us with).
+    const std::uint64_t grid_groups = std::uint64_t{max_splits} * 2 * rows;
+    const bool keyless_between =
+        grid_groups > units && grid_groups > split_workgroups(long_keys, split_keys);
+    const bool in_turn = rows <= 2;
+    const std::uint32_t walk_flags = (in_turn ? 2u : 8u) | (keyless_between ? 4u : 0u);
     Walk walk{pass};
     const DecodePipelines& k = step.pipelines;
     for (std::size_t layer = 0; layer < step.schedule.size(); ++layer) {
@@ -632,26 +631,29 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
             walk.buffer(batch.gdn_gated, 0, 3);
             walk.constant(static_cast<std::uint32_t>(g.gdn_value_bytes / 2), 4);
             walk.dispatch(g.gdn_gate_norm.groups, g.gdn_gate_norm.threads, rows);
-        } else if (batch.attention_whole_layer) {
+        } else if (token_form) {
             for (const bool finishing : {false, true}) {
                 if (finishing) walk.barrier();
-                walk.pipeline(finishing ? k.attention_layer_finish_ms : k.attention_layer_ms);
+                walk.pipeline(finishing ? k.attention_token_finish_ms : k.attention_token_ms);
                 walk.buffer(batch.attn_projection, 0, 0);
                 walk.weight(w.query_norm, 1);
                 walk.weight(w.key_norm, 2);
                 walk.buffer(pool.layers[layer].first, 0, 3);
                 walk.buffer(pool.layers[layer].second, 0, 4);
                 walk.buffer(batch.state_offsets, layer * 256, 5);
-                walk.buffer(batch.attn_layer_scratch, 0, 6);
+                walk.buffer(batch.attn_partials, 0, 6);
                 walk.buffer(batch.attn_attended, 0, 7);
                 walk.constant(step.capacity, 8);
                 walk.constant(static_cast<std::uint32_t>(g.attn_projection_bytes / 2), 9);
                 walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 10);
-                walk.constant(finishing ? batch.layer_groups : 0u, 11);
+                walk.constant(split_keys, 11);
+                walk.constant(max_splits, 12);
+                walk.constant(walk_flags, 13);
+                walk.constant((deepest + split_keys - 1) / split_keys, 14);
                 if (finishing) {
-                    walk.dispatch(HipSize{16, rows, 1}, HipSize{64, 1, 1});
+                    walk.dispatch(g.attention_head.groups, g.attention_head.threads, rows);
                 } else {
-                    walk.dispatch(HipSize{batch.layer_groups, rows, 1}, HipSize{256, 1, 1});
+                    walk.dispatch(HipSize{max_splits, 2, rows}, HipSize{256, 1, 1});
                 }
             }
         } else {
@@ -681,19 +683,8 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                 walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
                 walk.constant(split_keys, 7);
                 walk.constant(max_splits, 8);
-                // bit 0: short rows are left to the single-partition operator; bit 1: waves of
-                // one or two lanes deal a lane's 32-key blocks to its workgroups in turn
-                // (measured 1-3 % faster there, 3 % slower at four lanes); bit 2: the grid is
-                // larger than the chip and part of it holds no keys, so the workgroups that do
-                // go first (0.4 us dearer than the order by grid position where that is not so)
-                const std::uint64_t grid_groups = std::uint64_t{max_splits} * 2 * rows;
-                const bool keyless_between =
-                    grid_groups > units && grid_groups > split_workgroups(long_keys, split_keys);
-                const bool in_turn =
-                    batch.split_order == DecodeBatchScratch::SplitOrder::Automatic
-                        ? rows <= 2
-                        : batch.split_order == DecodeBatchScratch::SplitOrder::BlocksInTurn;
-                walk.constant(1u | (in_turn ? 2u : 0u) | (keyless_between ? 4u : 0u), 9);
+                // bit 0: short rows are left to the single-partition operator
+                walk.constant(1u | walk_flags, 9);
                 walk.dispatch(HipSize{max_splits, 2, rows}, HipSize{256, 1, 1});
                 walk.barrier();
                 walk.pipeline(k.attention_combine_ms);
@@ -705,6 +696,7 @@ HipCommandError encode_token_batch(DecodeStep& step, std::span<const DecodeStrea
                 walk.constant(max_splits, 5);
                 walk.constant(static_cast<std::uint32_t>(g.attn_query_bytes / 2), 6);
                 walk.constant(1u, 7);
+                walk.constant(step.capacity, 8);
                 walk.dispatch(g.attention_head.groups, g.attention_head.threads, rows);
             }
             if (table.bucket_rows != 0) {

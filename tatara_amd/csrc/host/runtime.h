@@ -176,7 +176,7 @@ struct DecodePipelines {
     HipComputePipeline gdn_prepare_ms, gdn_recurrence_ms, gate_norm_ms, gdn_decode_fused_ms;
     HipComputePipeline attn_qk_rope_ms, attention_decode_ms, attention_split_ms,
         attention_combine_ms;
-    HipComputePipeline attention_layer_ms, attention_layer_finish_ms;
+    HipComputePipeline attention_token_ms, attention_token_finish_ms;
 };
 struct DecodePipelinesResult {
     backend::hip::HipPipelineError error;
@@ -199,25 +199,15 @@ struct DecodeBatchScratch {
     std::uint32_t split_keys{0};
     // compute units of the device the scratch was made on: what the automatic split fills
     std::uint32_t compute_units{256};
-    // How a row's split-K workgroups share its keys: consecutive ranges of `split_keys`, or
-    // its 32-key blocks in turn.  Automatic: in turn for waves of one or two rows.  Ranges
-    // are the faster order at most depths, but their time depends on how the cache's strides
-    // fall on the memory channels (measured 47-77 us for the same 4 x 32768 keys over
-    // capacities 32768 ... 135168 at 1024 keys a workgroup), blocks in turn do not
-    // (48-49 us): a deployment whose capacity falls badly can pin the order here.
-    enum class SplitOrder : std::uint8_t { Automatic, Ranges, BlocksInTurn };
-    SplitOrder split_order{SplitOrder::Automatic};
     // One dispatch per Gated DeltaNet layer (gdn_decode_fused_ms) instead of the
     // reference's prepare / recurrence / gate-norm triple; same results bit for bit.
     bool gdn_fused{true};
-    // The attention layer of a wave as attention_decode_layer_ms +
-    // attention_decode_layer_finish_ms (norm, rotation, append, split-K over keys dealt evenly
-    // to `layer_groups` workgroups, gated combine) instead of rope, split path, combine and
-    // the short-row bucket: no split size to choose, every row through the same two
-    // dispatches.  `attn_layer_scratch` holds its tickets, query heads and records.
-    bool attention_whole_layer{false};
-    std::uint32_t layer_groups{0};
-    HipBuffer attn_layer_scratch;
+    // The attention layer of a wave as attention_decode_token_ms +
+    // attention_decode_token_finish_ms (norm and rotation inside the split-K walk over the
+    // cached keys; the token's own key and value folded in, and appended, by the finishing
+    // dispatch) instead of rope, split path, combine and the short-row bucket: every row
+    // through the same two dispatches, records in `attn_partials`.
+    bool attention_token_form{false};
 };
 
 // Keys per split-K workgroup for one attention layer of a wave whose rows see

@@ -10,7 +10,11 @@
 //   attention_decode_scores_gqa4 (:373), attention_decode_values_gqa8 (:995)
 // plus the lane-batched split path the reference lacks (it re-dispatches the
 // one-lane split path per long row, src/runtime/decode_step.cpp:1249-1259):
-//   attention_decode_split_ms, attention_decode_combine_ms.
+//   attention_decode_split_ms, attention_decode_combine_ms,
+// and the same layer of a token wave in two dispatches instead of three - the qk-norm and
+// rotation of attn_qk_rope_ms folded into the split-K walk, the token's own key and value
+// folded in and appended by the finishing dispatch:
+//   attention_decode_token_ms, attention_decode_token_finish_ms.
 //
 // Flash-decode layout.  One workgroup = 4 wave64 = one (row, kv head, key
 // range).  Each wave owns every 4th block of 32 keys and keeps an online
@@ -54,6 +58,7 @@ constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
 constexpr uint32_t kLdsPairBytes = 1040;    // key i row | key 16+i row | 16 B pad
 constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16640
 constexpr uint32_t kWaves = 4;
+constexpr uint32_t kHeadsPerWave = kAttnHeadsPerKv / kWaves;   // heads a wave norms and finishes
 // Cache policy of the K transfers and V loads: every key and value byte is used once per
 // dispatch, so it is requested nontemporal (the `nt` bit; V through
 // __builtin_nontemporal_load) and does not displace what the caches hold.  Measured on the
@@ -63,7 +68,6 @@ constexpr uint32_t kMergeTileFloats = 20;   // 16 accumulator words of one MFMA 
 constexpr uint32_t kMergeHeadFloats = 16 * kMergeTileFloats + 4;  // 324: head stride of the merge
 // Bound of the rows a state table may carry (decode_step.cpp:1007-1009).
 constexpr uint32_t kMaxBatchRows = 16;
-constexpr uint32_t kMaxStreams = kMaxBatchRows * kAttnKvHeads;  // (row, kv head) key streams
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -339,24 +343,12 @@ struct HeadLoads {
     uint32_t x32[4];      // the registers of load_head_untracked, narrowed by heads_landed
     uint32_t w32[4];
 };
-__device__ __forceinline__ HeadLoads load_head(const uint16_t* x, const uint16_t* weight,
-                                               uint32_t lane) {
-    HeadLoads h;
-    const uint32_t* words = reinterpret_cast<const uint32_t*>(x + lane * 4);
-    h.run[0] = words[0];
-    h.run[1] = words[1];
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        h.x[c] = x[lane + 64 * c];
-        h.w[c] = weight[lane + 64 * c];
-    }
-    return h;
-}
-// The same loads issued as assembly, which the compiler does not count, for a caller that
-// places them itself among the requests of a kernel's first microsecond and waits for
-// them with heads_landed() (left to the compiler, a wait for these values would also wait
-// for every request issued behind them: it does not wait for part of a queue that holds
-// LDS transfers).
+// The loads of one head for a wave (lane l: the run of values 4 l .. 4 l + 3 for the sum
+// of squares, values l + 64 c and their weights), issued as assembly, which the compiler
+// does not count: the caller places them itself among the requests of a kernel's first
+// microsecond and waits for them with heads_landed() (left to the compiler, a wait for
+// these values would also wait for every request issued behind them: it does not wait for
+// part of a queue that holds LDS transfers).
 __device__ __forceinline__ HeadLoads load_head_untracked(const uint16_t* x, const uint16_t* weight,
                                                          uint32_t lane) {
     HeadLoads h;
@@ -394,9 +386,6 @@ __device__ __forceinline__ void heads_landed(HeadLoads& a, HeadLoads& b) {
 // Cosine and sine of the rotation of pair (lane & 31) at `position`: the same for every
 // head of a row, so a wave evaluates them once (one shared argument reduction) for all the
 // heads it norms.
-__device__ __forceinline__ RopeAngle rope_angle(uint32_t position, uint32_t lane) {
-    return rope_angle_of(position, rope_inverse_frequency(lane & (kAttnRopePairs - 1)));
-}
 __device__ __forceinline__ void norm_rope_head(const HeadLoads& h, const RopeAngle& angle,
                                                uint32_t lane, float (&out)[4]) {
     float acc = 0.0f;
@@ -490,8 +479,10 @@ __device__ __forceinline__ void key_block_transfers(const uint8_t* from, uint8_t
     (key_row_transfer<kI>(from, stage), ...);
 }
 
-template <bool kRope>
-__global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
+// kFinal: one workgroup sees every key of its (row, kv head) and writes the gated bf16
+// output itself instead of a split record.
+template <bool kRope, bool kFinal = false>
+__global__ __launch_bounds__(kWaves * 64, 2) void flash_decode_kernel(FlashArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // (rope form) the rotation's inverse frequency of pair lane & 31
     float inverse_frequency = 1.0f;
@@ -507,13 +498,13 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // order, where the table names it, right behind the table.  Either way they are here
     // before the walk's first requests go out: requested among those, they would wait in
     // the memory system's queues behind the first blocks of every workgroup.
-    HeadLoads ql[2];
+    HeadLoads ql[kHeadsPerWave];
     auto request_heads = [&](uint32_t of_row, uint32_t of_kvh) {
         const uint16_t* proj = a.projection + static_cast<uint64_t>(of_row) * a.projection_stride;
 #pragma unroll
-        for (uint32_t i = 0; i < 2; ++i) {
+        for (uint32_t i = 0; i < kHeadsPerWave; ++i) {
             ql[i] = load_head_untracked(
-                proj + (of_kvh * kAttnHeadsPerKv + (threadIdx.x >> 6) * 2 + i) * 2 * kD, a.q_weight,
+                proj + (of_kvh * kAttnHeadsPerKv + (threadIdx.x >> 6) * kHeadsPerWave + i) * 2 * kD, a.q_weight,
                 threadIdx.x & 63);
         }
     };
@@ -570,7 +561,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     if (context >= a.capacity) return;  // a bad table row must not read outside the cache
     const uint32_t n = kRope ? context : context + 1;
     if (a.long_rows_only && n <= a.single_partition) return;
-    const uint32_t part = a.final_mode ? n : a.part;
+    const uint32_t part = kFinal ? n : a.part;
     if (split * part >= n) return;
     // The workgroup's blocks of 32 keys: block b of its own is block first_block + b *
     // block_stride of the row.  Contiguous: the keys [split * part, + part).  Interleaved: the
@@ -578,7 +569,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // they read one contiguous window of the cache and all get the same number of blocks.
     const uint32_t row_blocks = (n + kBlockKeys - 1) / kBlockKeys;
     const uint32_t row_splits = (n + part - 1) / part;
-    const bool interleave = a.interleave != 0 && a.final_mode == 0;
+    const bool interleave = a.interleave != 0 && !kFinal;
     const uint32_t first_block = interleave ? split : split * (part / kBlockKeys);
     const uint32_t block_stride = interleave ? row_splits : 1;
     const uint32_t key_end = interleave ? n : min(n, split * part + part);
@@ -595,7 +586,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     bf16x8 qreg[8];
     if constexpr (kRope) {
         if (a.compact) request_heads(row, kvh);
-        heads_landed(ql[0], ql[1]);
+        heads_landed(ql[0], ql[kHeadsPerWave - 1]);
     } else {
         const uint16_t* qh = a.q + static_cast<uint64_t>(row) * a.query_stride +
                              (kvh * kAttnHeadsPerKv + (m & 7)) * kD;
@@ -691,41 +682,42 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // registers, so a wave always has its next block in flight.
     u32x4 vreg[2][8];
     if constexpr (kRope) {
-        // (by every wave, also one whose range holds no block for it: it fetches the last
-        // block again, and the norm below runs without a branch around the requests)
+        // The first block is requested by every wave, also one whose range holds no block
+        // for it (it fetches the last block again), so that no branch surrounds what
+        // follows.  Its keys go out first; the norm and rotation of the wave's two query
+        // heads run next, while the memory system is busy with them - a wave that has
+        // issued all its requests cannot issue arithmetic any sooner, and one that still has
+        // requests to issue is held at them by the queues - and the values after that.
+        // Q^T reaches the operand layout through 4 KiB of LDS; the barrier waits for those
+        // LDS writes only, not for the transfers in flight.
         const uint32_t first = min(wave, nblocks - 1);
         stage_keys(first);
-        load_values(vreg[0], first, 0);
-        load_values(vreg[1], first, 1);
-        // the requests above stay above the norm below (the scheduler would sink the
-        // value loads under it, towards their first use)
         __builtin_amdgcn_sched_barrier(0);
-    } else if (wave < nblocks) {
-        stage_keys(wave);
-        load_values(vreg[0], wave, 0);
-        load_values(vreg[1], wave, 1);
-    }
-    if constexpr (kRope) {
-        // norm and rotation of the wave's two heads while the first blocks are under way;
-        // Q^T reaches the operand layout through 4 KiB of LDS behind the K stages.  The
-        // barrier waits for the LDS writes only, not for the transfers in flight.
         __shared__ __attribute__((aligned(16))) uint16_t qs[kAttnHeadsPerKv * kD];
         const RopeAngle angle = rope_angle_of(context, inverse_frequency);
 #pragma unroll
-        for (uint32_t i = 0; i < 2; ++i) {
+        for (uint32_t i = 0; i < kHeadsPerWave; ++i) {
             float nr[4];
             norm_rope_head(ql[i], angle, lane, nr);
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
-                qs[(wave * 2 + i) * kD + lane + 64 * c] = f32_to_bf16_bits(nr[c]);
+                qs[(wave * kHeadsPerWave + i) * kD + lane + 64 * c] = f32_to_bf16_bits(nr[c]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        load_values(vreg[0], first, 0);
+        load_values(vreg[1], first, 1);
+        __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
         for (uint32_t kb = 0; kb < 8; ++kb) {
             qreg[kb] = __builtin_bit_cast(
                 bf16x8, *reinterpret_cast<const u32x4*>(qs + (m & 7) * kD + kb * 32 + g * 8));
         }
+    } else if (wave < nblocks) {
+        stage_keys(wave);
+        load_values(vreg[0], wave, 0);
+        load_values(vreg[1], wave, 1);
     }
     for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
         const uint32_t valid = min(kBlockKeys, key_end - own_block(blk) * kBlockKeys);
@@ -846,8 +838,8 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
     // dimensions l, l+64, l+128, l+192 (coalesced stores).  Dimension d sits in
     // the stage at word ((d>>7)*8 + (d&7))*20 + ((d&127)>>3).
 #pragma unroll
-    for (uint32_t hl = 0; hl < 2; ++hl) {
-        const uint32_t h = wave * 2 + hl;
+    for (uint32_t hl = 0; hl < kHeadsPerWave; ++hl) {
+        const uint32_t h = wave * kHeadsPerWave + hl;
         float scale[kWaves];
         float gmax = -INFINITY;
         float lsum[kWaves];
@@ -865,7 +857,7 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
             denom = fmaf(scale[w], lsum[w], denom);
         }
         const uint32_t head = kvh * kAttnHeadsPerKv + h;
-        float* record = a.final_mode
+        float* record = kFinal
                             ? nullptr
                             : a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                                   (static_cast<uint64_t>(head) * a.record_splits + split) *
@@ -880,673 +872,20 @@ __global__ __launch_bounds__(256, 2) void flash_decode_kernel(FlashArgs a) {
                 const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
                 acc = fmaf(scale[w], wm[h * kMergeHeadFloats + slot], acc);
             }
-            if (a.final_mode) {
+            if constexpr (kFinal) {
                 const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + d;
                 a.out[at] = f32_to_bf16_bits((acc / denom) * sigmoid_gate(a.gate[at]));
             } else {
-                record[d] = acc;
+                // (nontemporal: the records are read once, by another dispatch, and a
+                // dispatch that ends on cached stores ends on their write-back)
+                __builtin_nontemporal_store(acc, record + d);
             }
         }
-        if (!a.final_mode && lane == 0) {
-            record[kD] = gmax;
-            record[kD + 1] = denom;
-        }
-    }
-}
-
-// ------------------------------------------------- whole decode layer -------
-//
-// attention_decode_layer_ms: the attention layer of a token wave in one dispatch - qk-norm
-// and rotation of the new token, its K / V append, split-K attention over every lane's
-// cache and the gated combine (attn_qk_rope_ms + the split path + the combine of
-// decode_step.cpp:1231-1259 folded together).
-//
-// Work is dealt by keys, not by lane: a (row, kv head) pair is a stream of
-// ceil(context / 32) units of 32 cached keys (one empty unit when the cache is empty), the
-// streams are laid end to end, and workgroup g of G takes units [g U / G, (g + 1) U / G) of
-// the U in total - ragged lanes and deep single lanes load every workgroup alike.  A
-// workgroup's range may cross stream boundaries; each piece inside one stream is a
-// segment, processed like a split of flash_decode_kernel and stored as one record per
-// head.  Everything is derived from the contexts in the state table, so one compiled walk
-// serves every token.
-//
-// The new token never goes through the cache: whoever finishes a stream folds it in as
-// one more record {numerator = V row, max = its score, sum = 1} from the projection row,
-// and appends its K / V rows for later tokens.
-//
-// Finishing.  finish_in_kernel = 0: a second dispatch (attention_layer_finish_kernel, one
-// wave per head and row).  finish_in_kernel = 1: the workgroups of a stream count their
-// arrivals on a ticket and the last to arrive finishes the stream, so the layer is a single
-// dispatch.  Records then travel between compute units that do not share an L2: they are
-// written with agent-scope atomic stores (write-through, no cache-wide write-back), the
-// ticket is taken after those stores have been acknowledged, and the finisher invalidates
-// its caches (acquire fence) before it reads them.  No workgroup ever waits for another.
-
-struct LayerArgs {
-    const uint16_t* projection;   // [rows][projection_stride]: {q | gate} x 16, K x 2, V x 2
-    const uint16_t* q_weight;
-    const uint16_t* k_weight;
-    uint16_t* keys;               // pools; row r's cache at + table[4 r] elements
-    uint16_t* values;
-    const uint32_t* table;        // per row {kv element offset, context, -, -}
-    float* records;               // [groups + streams - 1][8][258]
-    uint32_t* tickets;            // [streams] arrivals, zero between launches
-    uint16_t* queries;            // [streams][8][256] roped query heads (two-dispatch form)
-    uint16_t* out;                // [rows][query_stride]
-    uint32_t capacity;
-    uint32_t projection_stride;
-    uint32_t query_stride;
-    uint32_t rows;
-    uint32_t groups;              // G: workgroups the units are dealt to
-    uint32_t finish_in_kernel;
-};
-
-// How the key streams are dealt to the G workgroups, evaluated by one wave (lane s =
-// stream s) from the contexts in the state table.  A stream holds ceil(context / 32) units
-// (one empty unit for an empty cache; none when the table places the row outside its
-// cache, which every workgroup then skips alike).
-//   * G at least the number of streams that hold units: whole workgroups per stream.
-//     Stream s starts at workgroup b_s = the boundary g U / G nearest to its first unit,
-//     moved where needed so that every such stream keeps at least one workgroup; its
-//     units are split evenly among min(b_{s+1} - b_s, units) workgroups.  One segment per
-//     workgroup - none pays a second prologue at a stream boundary - and the loads differ by
-//     less than one part in the stream's workgroup count.
-//   * fewer workgroups than streams (`flat`): the streams are laid end to end and
-//     workgroup g takes units [g U / G', (g + 1) U / G'), G' = min(G, U), crossing stream
-//     boundaries as they come.
-struct StreamDeal {
-    uint32_t units;        // units of stream `lane`
-    uint32_t inclusive;    // units of streams 0 .. lane
-    uint32_t first_group;  // b_lane (G for lanes past the last stream); unused when flat
-    uint32_t total;        // U
-    bool flat;
-    uint32_t context;      // of the lane's row, as the table holds it
-};
-__device__ __forceinline__ StreamDeal deal_streams(const LayerArgs& a, uint32_t lane) {
-    StreamDeal d;
-    uint32_t units = 0;
-    d.context = 0;
-    if (lane < a.rows * kAttnKvHeads) {
-        d.context = a.table[(lane >> 1) * 4 + 1];
-        if (d.context < a.capacity) units = max(1u, (d.context + kBlockKeys - 1) / kBlockKeys);
-    }
-    uint32_t inclusive = units;
-#pragma unroll
-    for (uint32_t off = 1; off < 64; off <<= 1) {   // lane 32 must see the total as well
-        const uint32_t below = __shfl_up(inclusive, off, 64);
-        if (lane >= off) inclusive += below;
-    }
-    d.units = units;
-    d.inclusive = inclusive;
-    d.total = __shfl(inclusive, kMaxStreams - 1, 64);
-    const uint64_t holding = __builtin_amdgcn_ballot_w64(units != 0);
-    const uint32_t holders = __builtin_popcountll(holding);
-    d.flat = a.groups < holders;
-    const uint32_t before = __builtin_amdgcn_mbcnt_hi(
-        static_cast<uint32_t>(holding >> 32),
-        __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(holding), 0u));
-    d.first_group = 0;
-    if (!d.flat && d.total != 0) {
-        // 32-bit arithmetic: units x workgroups stays below 2^30 (layer_args bounds both)
-        const uint32_t first_unit = inclusive - units;
-        int32_t slack = static_cast<int32_t>((2 * first_unit * a.groups + d.total) / (2 * d.total)) -
-                        static_cast<int32_t>(before);
-#pragma unroll
-        for (uint32_t off = 1; off < 64; off <<= 1) {
-            const int32_t below = __shfl_up(slack, off, 64);
-            if (lane >= off) slack = max(slack, below);
-        }
-        slack = min(slack, static_cast<int32_t>(a.groups - holders));
-        d.first_group = static_cast<uint32_t>(slack) + before;
-    }
-    return d;
-}
-
-// Workgroup that holds unit u when U units are dealt to G workgroups in ranges
-// [g U / G, (g + 1) U / G): the largest g with g U / G <= u.
-__device__ __forceinline__ uint32_t group_of_unit(uint32_t u, uint32_t total, uint32_t groups) {
-    return static_cast<uint32_t>(((static_cast<uint64_t>(u) + 1) * groups - 1) / total);
-}
-
-// The new token's key (normed, rotated; fp32 of the stored bf16) and raw value for dims
-// lane + 64 c, from the projection row; with `append` the wave also writes both rows into
-// the cache at position `context`.
-__device__ __forceinline__ void new_token_rows(const LayerArgs& a, const uint16_t* proj,
-                                               uint32_t kvh, uint32_t context, uint64_t kv_offset,
-                                               const RopeAngle& angle, bool append, uint32_t lane,
-                                               float (&kn)[4], uint16_t (&vraw)[4]) {
-    const HeadLoads kl = load_head(proj + kAttnQGateRows + kvh * kD, a.k_weight, lane);
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) vraw[c] = proj[kAttnVRowOffset + kvh * kD + lane + 64 * c];
-    norm_rope_head(kl, angle, lane, kn);
-    if (append) {
-        const uint64_t at = kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
-#pragma unroll
-        for (uint32_t c = 0; c < 4; ++c) {
-            a.keys[at + 64 * c] = f32_to_bf16_bits(kn[c]);
-            a.values[at + 64 * c] = vraw[c];
+        if (!kFinal && lane == 0) {
+            __builtin_nontemporal_store(gmax, record + kD);
+            __builtin_nontemporal_store(denom, record + kD + 1);
         }
     }
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-    v = half_wave_sum(v);
-    return v + __shfl_xor(v, 32, 64);
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (uint32_t off = 32; off; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
-
-// One wave finishes one head of one row: merges the stream's `count` records (slots
-// first_slot ..), folds in the new token, applies the gate and writes the output row.
-// q: dims lane + 64 c of the roped query head (fp32 of bf16).  new_token(kn, vraw) delivers
-// the token's roped key (fp32 of bf16) and raw value row for the same dims; it is called
-// after the records have been requested, so whatever it loads or computes runs while they
-// are under way.
-template <uint32_t kFinishBatch, typename NewToken>   // kFinishBatch: records requested at once
-__device__ __forceinline__ void finish_head(const LayerArgs& a, uint32_t row, uint32_t head,
-                                            uint32_t first_slot, uint32_t count,
-                                            const float (&q)[4], NewToken&& new_token,
-                                            uint32_t lane) {
-    const uint32_t hl = head % kAttnHeadsPerKv;
-    const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
-    uint16_t gate[4];
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) gate[c] = proj[head * 2 * kD + kD + lane + 64 * c];
-    // The first 64 maxima and sums one per lane, the numerators of the first batch of
-    // records by the lane that owns the dimension: with a batch of 32, one trip to memory
-    // for a stream of up to 32 records.
-    const float* base = a.records + (static_cast<uint64_t>(first_slot) * kAttnHeadsPerKv + hl) *
-                                        kAttnRecordFloats;
-    constexpr uint64_t kSlotFloats = static_cast<uint64_t>(kAttnHeadsPerKv) * kAttnRecordFloats;
-    float first_max = -INFINITY, first_sum = 0.0f;
-    if (lane < count) {
-        first_max = base[lane * kSlotFloats + kD];
-        first_sum = base[lane * kSlotFloats + kD + 1];
-    }
-    float num[kFinishBatch][4];
-#pragma unroll
-    for (uint32_t u = 0; u < kFinishBatch; ++u) {
-        const float* rec = base + min(u, count - 1) * kSlotFloats + lane;
-#pragma unroll
-        for (uint32_t c = 0; c < 4; ++c) num[u][c] = rec[64 * c];
-    }
-    float kn[4];
-    uint16_t vraw[4];
-    new_token(kn, vraw);
-    float dot = 0.0f;
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) dot = fmaf(q[c], kn[c], dot);
-    const float s_new = wave_sum(dot) * kAttnScale;
-
-    // maxima beyond the first 64 records (only streams spread over more than 64 workgroups)
-    float lmax = first_max;
-    for (uint32_t p = lane + 64; p < count; p += 64) lmax = fmaxf(lmax, base[p * kSlotFloats + kD]);
-    const float gmax = fmaxf(wave_max(lmax), s_new);
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    float denom = 0.0f;
-    for (uint32_t p0 = 0; p0 < count; p0 += kFinishBatch) {
-        if (p0 != 0) {
-#pragma unroll
-            for (uint32_t u = 0; u < kFinishBatch; ++u) {
-                const float* rec = base + min(p0 + u, count - 1) * kSlotFloats + lane;
-#pragma unroll
-                for (uint32_t c = 0; c < 4; ++c) num[u][c] = rec[64 * c];
-            }
-        }
-        // lane j (and the lanes that repeat it) weighs record p0 + j
-        const uint32_t mine = p0 + (lane & (kFinishBatch - 1));
-        float record_max, record_sum;
-        if (p0 < 64) {
-            record_max = __shfl(first_max, mine & 63, 64);
-            record_sum = __shfl(first_sum, mine & 63, 64);
-        } else {
-            const float* rec = base + min(mine, count - 1) * kSlotFloats;
-            record_max = rec[kD];
-            record_sum = rec[kD + 1];
-        }
-        const float my_w =
-            (mine < count && record_max != -INFINITY) ? __expf(record_max - gmax) : 0.0f;
-        const float my_ws = my_w * record_sum;
-#pragma unroll
-        for (uint32_t u = 0; u < kFinishBatch; ++u) {
-            const float w = __shfl(my_w, u, 64);
-            const float ws = __shfl(my_ws, u, 64);
-#pragma unroll
-            for (uint32_t c = 0; c < 4; ++c) acc[c] = fmaf(w, num[u][c], acc[c]);
-            denom += ws;
-        }
-    }
-    const float w_new = __expf(s_new - gmax);
-    denom += w_new;
-    const uint64_t at = static_cast<uint64_t>(row) * a.query_stride + head * kD + lane;
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        const float value = fmaf(w_new, bf16_bits_to_f32(vraw[c]), acc[c]);
-        a.out[at + 64 * c] = f32_to_bf16_bits((value / denom) * sigmoid_gate(gate[c]));
-    }
-}
-
-template <bool kFinishInKernel>
-__global__ __launch_bounds__(256, 2) void attention_decode_layer_kernel(LayerArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    // after the four K stages: the roped query heads of the segment's kv group (bf16),
-    // the stream offsets and the ticket broadcast
-    uint16_t* qs = reinterpret_cast<uint16_t*>(lds + kWaves * kWaveLdsBytes);
-    uint32_t* s_off = reinterpret_cast<uint32_t*>(lds + kWaves * kWaveLdsBytes +
-                                                  kAttnHeadsPerKv * kD * 2);
-    uint32_t* s_ticket = s_off + kMaxStreams + 1;
-    uint32_t* s_context = s_ticket + 1;            // per row, as the table holds them
-    uint32_t* s_kv_offset = s_context + kMaxBatchRows;
-    uint32_t* s_group = s_kv_offset + kMaxBatchRows;   // first workgroup per stream, then G
-    uint32_t* s_flat = s_group + kMaxStreams + 1;
-    uint32_t* s_range = s_flat + 1;                    // this workgroup's {first unit, end, stream}
-
-    const uint32_t group = blockIdx.x;
-    const uint32_t streams = a.rows * kAttnKvHeads;
-
-    if (threadIdx.x < 64) {
-        // one read of the state table: the contexts size the streams, and both words of a
-        // row are kept in LDS for the segments (no second trip to memory per segment)
-        const uint32_t lane = threadIdx.x;
-        const StreamDeal deal = deal_streams(a, lane);
-        if (lane < streams && (lane & 1) == 0) {
-            s_context[lane >> 1] = deal.context;
-            s_kv_offset[lane >> 1] = a.table[(lane >> 1) * 4];
-        }
-        if (lane < kMaxStreams) s_off[lane + 1] = deal.inclusive;
-        if (lane <= kMaxStreams) s_group[lane] = deal.first_group;
-        if (lane == 0) {
-            s_off[0] = 0;
-            *s_flat = deal.flat ? 1u : 0u;
-        }
-        // this workgroup's own units {first, end, stream of the first}: found by the lane of
-        // the stream whose workgroups include it
-        const uint32_t total = deal.total;
-        if (deal.flat) {
-            if (lane == 0) {
-                const uint32_t flat_groups = min(a.groups, total);
-                const bool idle = total == 0 || group >= flat_groups;
-                s_range[0] = idle ? 0u : static_cast<uint32_t>(static_cast<uint64_t>(group) * total / flat_groups);
-                s_range[1] = idle ? 0u : static_cast<uint32_t>((static_cast<uint64_t>(group) + 1) * total / flat_groups);
-                s_range[2] = 0;
-            }
-        } else {
-            const uint32_t next_group = __shfl_down(deal.first_group, 1, 64);
-            if (lane == 0) s_range[0] = s_range[1] = s_range[2] = 0;   // idle unless a stream claims it
-            if (lane < streams && deal.units != 0 && deal.first_group <= group && group < next_group) {
-                const uint32_t sharers = min(next_group - deal.first_group, deal.units);
-                const uint32_t place = group - deal.first_group;
-                const uint32_t first_unit = deal.inclusive - deal.units;
-                if (place < sharers) {                                 // else more workgroups than units
-                    s_range[0] = first_unit + place * deal.units / sharers;
-                    s_range[1] = first_unit + (place + 1) * deal.units / sharers;
-                    s_range[2] = lane;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    // values read back from LDS are the same in every lane: moved to scalar registers so
-    // that the segment walk, the key ranges and the row's table entries stay scalar
-    // (the builtin returns int: as uint32_t, so that a 32-bit offset widens without its sign)
-    const auto uniform = [](uint32_t v) -> uint32_t { return __builtin_amdgcn_readfirstlane(v); };
-    uint32_t unit = uniform(s_range[0]);
-    const uint32_t unit_end = uniform(s_range[1]);
-    if (unit >= unit_end) return;
-    const uint32_t total = uniform(s_off[streams]);
-    const bool flat = uniform(*s_flat) != 0;
-    const uint32_t flat_groups = min(a.groups, total);
-    uint32_t stream = uniform(s_range[2]);
-
-    while (unit < unit_end) {
-        // Everything derived from the thread index is derived inside the segment, from an
-        // opaque copy: hoisted out of this loop it would be carried in registers across
-        // the key walk (which has none to spare) and spilled.
-        uint32_t thread_early = threadIdx.x;
-        asm volatile("" : "+v"(thread_early));
-        const uint32_t wave = thread_early >> 6;
-        const uint32_t lane = thread_early & 63;
-        const uint32_t m = lane & 15;
-        const uint32_t g = lane >> 4;
-        uint8_t* stage = lds + wave * kWaveLdsBytes;
-        while (uniform(s_off[stream + 1]) <= unit) ++stream;
-        const uint32_t stream_first = uniform(s_off[stream]);
-        const uint32_t stream_last = uniform(s_off[stream + 1]);
-        const uint32_t segment_end = min(unit_end, stream_last);
-        const uint32_t row = stream >> 1;
-        const uint32_t kvh = stream & 1;
-        const uint64_t kv_offset = uniform(s_kv_offset[row]);
-        const uint32_t context = uniform(s_context[row]);
-        const uint32_t k0 = (unit - stream_first) * kBlockKeys;
-        const uint32_t k1 = min(context, (segment_end - stream_first) * kBlockKeys);
-        const uint32_t nblocks = k1 > k0 ? (k1 - k0 + kBlockKeys - 1) / kBlockKeys : 0u;
-        const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
-        const uint16_t* kbase = a.keys + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
-        const uint16_t* vbase = a.values + kv_offset + static_cast<uint64_t>(kvh) * a.capacity * kD;
-
-        // the wave's two query heads: their loads go out first, then the first block of
-        // keys and values, and the norm / rotation runs while that block is in flight
-        HeadLoads ql[2];
-#pragma unroll
-        for (uint32_t i = 0; i < 2; ++i) {
-            ql[i] = load_head(proj + (kvh * kAttnHeadsPerKv + wave * 2 + i) * 2 * kD, a.q_weight, lane);
-        }
-
-        auto stage_keys = [&](uint32_t blk) {
-            const uint32_t key0 = k0 + blk * kBlockKeys;
-            const uint32_t valid = min(kBlockKeys, k1 - key0);
-#pragma unroll
-            for (uint32_t i = 0; i < 16; ++i) {
-                const uint32_t key = min(i + (lane >> 5) * 16, valid - 1);
-                const uint16_t* src = kbase + static_cast<uint64_t>(key0 + key) * kD + (lane & 31) * 8;
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(src),
-                    (__attribute__((address_space(3))) void*)(stage + i * kLdsPairBytes),
-                    16, 0, kStreamOnce);
-            }
-        };
-        auto load_values = [&](u32x4 (&vhalf)[8], uint32_t blk, uint32_t hh) {
-            const uint32_t key0 = k0 + blk * kBlockKeys;
-            const uint32_t valid = min(kBlockKeys, k1 - key0);
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) {
-                const uint32_t key = min((e >> 2) * 16 + g * 4 + (e & 3), valid - 1);
-                vhalf[e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(
-                    vbase + static_cast<uint64_t>(key0 + key) * kD + hh * 128 + m * 8));
-            }
-        };
-
-        u32x4 vreg[2][8];
-        if (wave < nblocks) {
-            stage_keys(wave);
-            load_values(vreg[0], wave, 0);
-            load_values(vreg[1], wave, 1);
-        }
-        // two-dispatch form: the workgroup that holds a stream's first unit leaves the roped
-        // query heads in the scratch and appends the token's key and value rows (no key walk
-        // reads position `context`), so the finishing dispatch only loads them
-        const bool publishes = !kFinishInKernel && unit == stream_first;
-        const RopeAngle angle = rope_angle(context, lane);
-#pragma unroll
-        for (uint32_t i = 0; i < 2; ++i) {
-            float n[4];
-            norm_rope_head(ql[i], angle, lane, n);
-#pragma unroll
-            for (uint32_t c = 0; c < 4; ++c) {
-                const uint16_t bits = f32_to_bf16_bits(n[c]);
-                qs[(wave * 2 + i) * kD + lane + 64 * c] = bits;
-                if (publishes) {
-                    a.queries[(static_cast<uint64_t>(stream) * kAttnHeadsPerKv + wave * 2 + i) * kD +
-                              lane + 64 * c] = bits;
-                }
-            }
-        }
-        if (publishes && wave == 0) {
-            float kn[4];
-            uint16_t vraw[4];
-            new_token_rows(a, proj, kvh, context, kv_offset, angle, true, lane, kn, vraw);
-        }
-        __syncthreads();
-        // B operand of S^T: Q^T, column m holds head (m & 7)
-        bf16x8 qreg[8];
-#pragma unroll
-        for (uint32_t kb = 0; kb < 8; ++kb) {
-            qreg[kb] = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u32x4*>(qs + (m & 7) * kD + kb * 32 + g * 8));
-        }
-
-        f32x4 o[16];
-#pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) o[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        float m_run = -INFINITY;
-        float l_run = 0.0f;
-
-        for (uint32_t blk = wave; blk < nblocks; blk += kWaves) {
-            const uint32_t valid = min(kBlockKeys, k1 - (k0 + blk * kBlockKeys));
-            const bool more = blk + kWaves < nblocks;
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            __builtin_amdgcn_wave_barrier();
-            f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f};
-            f32x4 s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (uint32_t kb = 0; kb < 8; ++kb) {
-                const bf16x8 a0 = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes +
-                                                            (kb * 4 + g) * 16));
-                const bf16x8 a1 = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const u32x4*>(stage + m * kLdsPairBytes + 512 +
-                                                            (kb * 4 + g) * 16));
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[kb], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[kb], s1, 0, 0, 0);
-            }
-            float sc[8];
-            float block_max = -INFINITY;
-#pragma unroll
-            for (uint32_t i = 0; i < 4; ++i) {
-                sc[i] = (g * 4 + i) < valid ? s0[i] * kAttnScale : -INFINITY;
-                sc[4 + i] = (16 + g * 4 + i) < valid ? s1[i] * kAttnScale : -INFINITY;
-                block_max = fmaxf(block_max, fmaxf(sc[i], sc[4 + i]));
-            }
-            __builtin_amdgcn_wave_barrier();
-            if (more) stage_keys(blk + kWaves);
-            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
-            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
-            const float m_new = fmaxf(m_run, block_max);
-            const float alpha = __expf(m_run - m_new);
-            float p[8];
-            float block_sum = 0.0f;
-#pragma unroll
-            for (uint32_t e = 0; e < 8; ++e) {
-                p[e] = __expf(sc[e] - m_new);
-                block_sum += p[e];
-            }
-            block_sum += __shfl_xor(block_sum, 16, 64);
-            block_sum += __shfl_xor(block_sum, 32, 64);
-            l_run = l_run * alpha + block_sum;
-            m_run = m_new;
-            uint32_t pw[4];
-#pragma unroll
-            for (uint32_t c = 0; c < 4; ++c) {
-                float x0 = p[2 * c];
-                float x1 = p[2 * c + 1];
-                if (m >= 8) {
-                    x0 -= round_bf16(x0);
-                    x1 -= round_bf16(x1);
-                }
-                pw[c] = static_cast<uint32_t>(f32_to_bf16_bits(x0)) |
-                        (static_cast<uint32_t>(f32_to_bf16_bits(x1)) << 16);
-            }
-            const bf16x8 pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-                for (uint32_t j = 0; j < 16; ++j) o[j] *= alpha;
-            }
-#pragma unroll
-            for (uint32_t hh = 0; hh < 2; ++hh) {
-#pragma unroll
-                for (uint32_t dw = 0; dw < 4; ++dw) {
-                    u32x4 lo, hi;
-                    lo.x = pack_low(vreg[hh][0][dw], vreg[hh][1][dw]);
-                    lo.y = pack_low(vreg[hh][2][dw], vreg[hh][3][dw]);
-                    lo.z = pack_low(vreg[hh][4][dw], vreg[hh][5][dw]);
-                    lo.w = pack_low(vreg[hh][6][dw], vreg[hh][7][dw]);
-                    hi.x = pack_high(vreg[hh][0][dw], vreg[hh][1][dw]);
-                    hi.y = pack_high(vreg[hh][2][dw], vreg[hh][3][dw]);
-                    hi.z = pack_high(vreg[hh][4][dw], vreg[hh][5][dw]);
-                    hi.w = pack_high(vreg[hh][6][dw], vreg[hh][7][dw]);
-                    o[hh * 8 + 2 * dw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, lo), pb, o[hh * 8 + 2 * dw], 0, 0, 0);
-                    o[hh * 8 + 2 * dw + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, hi), pb, o[hh * 8 + 2 * dw + 1], 0, 0, 0);
-                }
-                if (more) load_values(vreg[hh], blk + kWaves, hh);
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-
-        // the same for the addresses of the merge below
-        uint32_t thread_late = threadIdx.x;
-        asm volatile("" : "+v"(thread_late));
-        const uint32_t wave_l = thread_late >> 6;
-        const uint32_t lane_l = thread_late & 63;
-        const uint32_t m_l = lane_l & 15;
-        const uint32_t g_l = lane_l >> 4;
-
-        // the wave's {O[8][256], max, sum} into its own stage (layout as in flash_decode_kernel)
-        float* merge = reinterpret_cast<float*>(lds + wave_l * kWaveLdsBytes);
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) {
-            f32x4 sum4;
-#pragma unroll
-            for (uint32_t i = 0; i < 4; ++i) sum4[i] = o[j][i] + dpp_row_ror8(o[j][i]);
-            if (m_l < 8) {
-                *reinterpret_cast<f32x4*>(merge + m_l * kMergeHeadFloats + j * kMergeTileFloats +
-                                          g_l * 4) = sum4;
-            }
-        }
-        if (lane_l < 8) {
-            merge[8 * kMergeHeadFloats + lane_l * 2] = m_run;
-            merge[8 * kMergeHeadFloats + lane_l * 2 + 1] = l_run;
-        }
-        __syncthreads();
-
-        // cross-wave merge into the segment's record: slot = workgroup + stream
-        const uint32_t slot = group + stream;
-#pragma unroll
-        for (uint32_t hl = 0; hl < 2; ++hl) {
-            const uint32_t h = wave_l * 2 + hl;
-            float scale[kWaves];
-            float gmax = -INFINITY;
-            float lsum[kWaves];
-#pragma unroll
-            for (uint32_t w = 0; w < kWaves; ++w) {
-                const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
-                scale[w] = wm[8 * kMergeHeadFloats + h * 2];
-                lsum[w] = wm[8 * kMergeHeadFloats + h * 2 + 1];
-                gmax = fmaxf(gmax, scale[w]);
-            }
-            float denom = 0.0f;
-#pragma unroll
-            for (uint32_t w = 0; w < kWaves; ++w) {
-                scale[w] = scale[w] == -INFINITY ? 0.0f : __expf(scale[w] - gmax);
-                denom = fmaf(scale[w], lsum[w], denom);
-            }
-            float* record = a.records + (static_cast<uint64_t>(slot) * kAttnHeadsPerKv + h) *
-                                            kAttnRecordFloats;
-#pragma unroll
-            for (uint32_t c = 0; c < 4; ++c) {
-                const uint32_t d = lane_l + 64 * c;
-                const uint32_t at = ((d >> 7) * 8 + (d & 7)) * kMergeTileFloats + ((d & 127) >> 3);
-                float acc = 0.0f;
-#pragma unroll
-                for (uint32_t w = 0; w < kWaves; ++w) {
-                    const float* wm = reinterpret_cast<const float*>(lds + w * kWaveLdsBytes);
-                    acc = fmaf(scale[w], wm[h * kMergeHeadFloats + at], acc);
-                }
-                __hip_atomic_store(record + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (lane_l == 0) {
-                __hip_atomic_store(record + kD, gmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(record + kD + 1, denom, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-
-        if constexpr (kFinishInKernel) {
-            // the record stores have been acknowledged before the ticket is taken
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            uint32_t first_group, count;
-            if (flat) {
-                first_group = group_of_unit(stream_first, total, flat_groups);
-                count = group_of_unit(stream_last - 1, total, flat_groups) - first_group + 1;
-            } else {
-                first_group = uniform(s_group[stream]);
-                count = min(uniform(s_group[stream + 1]) - first_group, stream_last - stream_first);
-            }
-            if (threadIdx.x == 0) {
-                *s_ticket = __hip_atomic_fetch_add(a.tickets + stream, 1u, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-            }
-            __syncthreads();
-            if (uniform(*s_ticket) == count - 1) {
-                // last to arrive: every record of the stream is in memory; drop what this
-                // compute unit's caches may hold of that memory, then finish two heads a wave
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-#pragma unroll 1
-                for (uint32_t hl = 0; hl < 2; ++hl) {
-                    const uint32_t h = wave * 2 + hl;
-                    float q[4];
-#pragma unroll
-                    for (uint32_t c = 0; c < 4; ++c) q[c] = bf16_bits_to_f32(qs[h * kD + lane + 64 * c]);
-                    // eight records at a time: the key walk above leaves no registers for more
-                    finish_head<8>(a, row, kvh * kAttnHeadsPerKv + h, first_group + stream, count, q,
-                                   [&](float (&kn)[4], uint16_t (&vraw)[4]) {
-                                       new_token_rows(a, proj, kvh, context, kv_offset, angle,
-                                                      h == 0, lane, kn, vraw);
-                                   },
-                                   lane);
-                }
-                if (threadIdx.x == 0) {
-                    __hip_atomic_store(a.tickets + stream, 0u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-        }
-        __syncthreads();  // the stages and the query heads are free for the next segment
-        unit = segment_end;
-    }
-}
-
-// Second dispatch of the two-dispatch form: grid (16 heads, rows) x 64, one wave per head.
-__global__ __launch_bounds__(64) void attention_layer_finish_kernel(LayerArgs a) {
-    const uint32_t head = blockIdx.x;
-    const uint32_t row = blockIdx.y;
-    const uint32_t lane = threadIdx.x;
-    const uint32_t stream = row * kAttnKvHeads + head / kAttnHeadsPerKv;
-    const StreamDeal deal = deal_streams(a, lane);
-    const uint32_t total = deal.total;
-    const uint32_t stream_last = __shfl(deal.inclusive, stream, 64);
-    const uint32_t below = __shfl(deal.inclusive, stream == 0 ? 0 : stream - 1, 64);
-    const uint32_t stream_first = stream == 0 ? 0u : below;
-    if (stream_last == stream_first) return;   // a row the table places outside its cache
-    uint32_t first_group, count;
-    if (deal.flat) {
-        const uint32_t groups = min(a.groups, total);
-        first_group = group_of_unit(stream_first, total, groups);
-        count = group_of_unit(stream_last - 1, total, groups) - first_group + 1;
-    } else {
-        first_group = __shfl(deal.first_group, stream, 64);
-        count = min(__shfl(deal.first_group, stream + 1, 64) - first_group,
-                    stream_last - stream_first);
-    }
-    // The first dispatch left the roped query heads in the scratch and the token's key and
-    // value rows in the cache: nothing is normed or rotated again here.
-    const uint64_t kv_offset = a.table[row * 4];
-    const uint32_t context = a.table[row * 4 + 1];
-    const uint32_t kvh = head / kAttnHeadsPerKv;
-    float q[4];
-#pragma unroll
-    for (uint32_t c = 0; c < 4; ++c) {
-        q[c] = bf16_bits_to_f32(
-            a.queries[(static_cast<uint64_t>(stream) * kAttnHeadsPerKv + head % kAttnHeadsPerKv) * kD +
-                      lane + 64 * c]);
-    }
-    finish_head<32>(a, row, head, first_group + stream, count, q,
-                    [&](float (&kn)[4], uint16_t (&vraw)[4]) {
-                        const uint64_t at =
-                            kv_offset + (static_cast<uint64_t>(kvh) * a.capacity + context) * kD + lane;
-#pragma unroll
-                        for (uint32_t c = 0; c < 4; ++c) {
-                            kn[c] = bf16_bits_to_f32(a.keys[at + 64 * c]);
-                            vraw[c] = a.values[at + 64 * c];
-                        }
-                    },
-                    lane);
 }
 
 // ----------------------------------------------------------------- combine ---
@@ -1563,6 +902,7 @@ struct CombineArgs {
     uint64_t partial_row_floats;
     uint32_t long_rows_only;
     uint32_t single_partition;
+    uint32_t capacity;       // with a table: a row whose context is not a cache position is left alone
 };
 
 // Up to kParts partitions: every load is requested before the first is used - the
@@ -1617,11 +957,14 @@ __global__ __launch_bounds__(256) void attention_combine_kernel(CombineArgs a) {
     const uint32_t d = threadIdx.x;
     uint32_t nparts = a.nparts;
     if (a.table != nullptr) {
-        const uint32_t n = a.table[row * 4 + 1] + 1;
+        const uint32_t context = a.table[row * 4 + 1];
+        // a table row the split kernel refused (its context is not a position of the cache)
+        // has no records of this launch: its output is left alone, whatever earlier launches
+        // left in the record buffer and whatever the context wraps to
+        if (context >= a.capacity) return;
+        const uint32_t n = context + 1;
         if (a.long_rows_only && n <= a.single_partition) return;
         nparts = (n + a.part - 1) / a.part;
-        // a table row the split kernel refused (context past the capacity the records were
-        // sized for) has no records: leave its output alone rather than read past them
         if (nparts > a.record_splits) return;
     }
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
@@ -1706,6 +1049,7 @@ struct FinishArgs {
     uint32_t query_stride;
     uint32_t part;
     uint32_t record_splits;
+    uint32_t parts_hint;          // records per head the caller expects the deepest row to have
     uint64_t partial_row_floats;
 };
 
@@ -1714,23 +1058,26 @@ struct MergedParts {
 };
 
 // Numerators of up to kParts records requested at once by the thread that owns the
-// dimension; their maxima and sums go through LDS (one thread per record).  The caller
-// places a barrier between request_parts and reduce_parts.
+// dimension; their maxima and sums go through LDS (one thread per record).  `held` = how
+// many records the buffer holds from `base` on (requests beyond it repeat the last one);
+// which of them count is decided in reduce_parts, so nothing here waits for the state
+// table.  The caller places a barrier between request_parts and reduce_parts.
 template <uint32_t kParts>
-__device__ __forceinline__ void request_parts(const float* base, uint32_t nparts, uint32_t d,
+__device__ __forceinline__ void request_parts(const float* base, uint32_t held, uint32_t d,
                                               float (&numerator)[kParts], float* part_max,
                                               float* part_sum) {
-    const uint32_t last = nparts == 0 ? 0u : nparts - 1;
+    const uint32_t last = held - 1;
 #pragma unroll
     for (uint32_t p = 0; p < kParts; ++p) {
         numerator[p] = base[static_cast<uint64_t>(min(p, last)) * kAttnRecordFloats + d];
     }
     if (d < kParts) {
         const float* rec = base + static_cast<uint64_t>(min(d, last)) * kAttnRecordFloats;
-        part_max[d] = d < nparts ? rec[kD] : -INFINITY;
+        part_max[d] = rec[kD];
         part_sum[d] = rec[kD + 1];
     }
 }
+// Merge of the first `nparts` (at most kParts) of the requested records.
 template <uint32_t kParts>
 __device__ __forceinline__ MergedParts reduce_parts(const float (&numerator)[kParts], uint32_t nparts,
                                                     const float* part_max, const float* part_sum) {
@@ -1738,7 +1085,10 @@ __device__ __forceinline__ MergedParts reduce_parts(const float (&numerator)[kPa
 #pragma unroll
     for (uint32_t p = 0; p < kParts; p += 4) {
         const f32x4 m4 = *reinterpret_cast<const f32x4*>(part_max + p);
-        r.gmax = fmaxf(fmaxf(r.gmax, m4[0]), fmaxf(fmaxf(m4[1], m4[2]), m4[3]));
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            if (p + u < nparts) r.gmax = fmaxf(r.gmax, m4[u]);
+        }
     }
 #pragma unroll
     for (uint32_t p = 0; p < kParts; p += 4) {
@@ -1756,10 +1106,12 @@ __device__ __forceinline__ MergedParts reduce_parts(const float (&numerator)[kPa
     return r;
 }
 
+// One (row, head) by one workgroup.  Every load - the state table entry, the projection
+// row's four slices, the two norm weights and the first kParts records - is requested
+// before the first is used: the kernel is one trip to memory deep.
 template <uint32_t kParts>
 __device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t head, uint32_t row,
-                                                uint32_t d, uint64_t kv_offset, uint32_t context,
-                                                uint32_t nparts) {
+                                                uint32_t d) {
     __shared__ __attribute__((aligned(16))) float part_max[kParts];
     __shared__ __attribute__((aligned(16))) float part_sum[kParts];
     __shared__ float wave_values[3][4];   // squares of the query head, of the key head, q . k
@@ -1767,7 +1119,7 @@ __device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t he
     const uint16_t* proj = a.projection + static_cast<uint64_t>(row) * a.projection_stride;
     const float* base = a.partials + static_cast<uint64_t>(row) * a.partial_row_floats +
                         static_cast<uint64_t>(head) * a.record_splits * kAttnRecordFloats;
-    // every load of the kernel is requested here, before the first is used
+    const u32x2 entry = *reinterpret_cast<const u32x2*>(a.table + row * 4);
     const float inverse_frequency = rope_inverse_frequency(d & (kAttnRopePairs - 1));
     const uint16_t xq = proj[head * 2 * kD + d];
     const uint16_t gate = proj[head * 2 * kD + kD + d];
@@ -1776,9 +1128,14 @@ __device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t he
     const uint16_t wq = a.q_weight[d];
     const uint16_t wk = a.k_weight[d];
     float numerator[kParts];
-    request_parts<kParts>(base, nparts, d, numerator, part_max, part_sum);
+    request_parts<kParts>(base, min(kParts, a.record_splits), d, numerator, part_max, part_sum);
 
-    // the rotation's cosine and sine, while the loads are in flight
+    const uint64_t kv_offset = entry[0];
+    const uint32_t context = entry[1];
+    // a row the table places outside its cache has no records and no slot to append to
+    if (context >= a.capacity) return;
+    const uint32_t nparts = (context + a.part - 1) / a.part;
+    if (nparts > a.record_splits) return;
     float c = 1.0f, sn = 0.0f;
     if (d < 2 * kAttnRopePairs) {
         const RopeAngle angle = rope_angle_of(context, inverse_frequency);
@@ -1813,11 +1170,11 @@ __device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t he
     dot = half_wave_sum(dot);
     dot += __shfl_xor(dot, 32, 64);
     if ((d & 63) == 0) wave_values[2][d >> 6] = dot;
-    MergedParts merged = reduce_parts<kParts>(numerator, nparts, part_max, part_sum);
+    MergedParts merged = reduce_parts<kParts>(numerator, min(nparts, kParts), part_max, part_sum);
     __syncthreads();
-    if constexpr (kParts == 128) {
-        // more than 128 records (a cache far deeper than the split was chosen for): the same
-        // in batches of 128, merged as they come
+    {
+        // more records than were requested up front (a context that has grown past the
+        // caller's hint, or more than 128 records): the rest in batches, merged as they come
         for (uint32_t p0 = kParts; p0 < nparts; p0 += kParts) {
             const uint32_t count = min(kParts, nparts - p0);
             request_parts<kParts>(base + static_cast<uint64_t>(p0) * kAttnRecordFloats, count, d,
@@ -1849,19 +1206,17 @@ __device__ __forceinline__ void finish_row_head(const FinishArgs& a, uint32_t he
     }
 }
 
+// The batch of records requested up front is sized by a launch constant - how many records
+// the caller expects the deepest row to have, at most what the buffer holds per head - not
+// by the contexts in the state table, which arrive with the records.
 __global__ __launch_bounds__(256) void attention_finish_kernel(FinishArgs a) {
     const uint32_t head = blockIdx.x;
     const uint32_t row = blockIdx.y;
     const uint32_t d = threadIdx.x;
-    const uint64_t kv_offset = a.table[row * 4];
-    const uint32_t context = a.table[row * 4 + 1];
-    // a row the table places outside its cache has no records and no slot to append to
-    if (context >= a.capacity) return;
-    const uint32_t nparts = (context + a.part - 1) / a.part;
-    if (nparts > a.record_splits) return;
-    if (nparts <= 32) return finish_row_head<32>(a, head, row, d, kv_offset, context, nparts);
-    if (nparts <= 64) return finish_row_head<64>(a, head, row, d, kv_offset, context, nparts);
-    return finish_row_head<128>(a, head, row, d, kv_offset, context, nparts);
+    const uint32_t expected = min(a.parts_hint == 0 ? a.record_splits : a.parts_hint, a.record_splits);
+    if (expected <= 32) return finish_row_head<32>(a, head, row, d);
+    if (expected <= 64) return finish_row_head<64>(a, head, row, d);
+    return finish_row_head<128>(a, head, row, d);
 }
 
 // ---------------------------------------- separate score / value stages ------
@@ -2066,10 +1421,13 @@ namespace {
 
 int32_t launch_flash(const FlashArgs& f, uint32_t splits, uint32_t rows, hipStream_t stream) {
     if (f.projection != nullptr) {
-        hipLaunchKernelGGL(flash_decode_kernel<true>, dim3(splits, kAttnKvHeads, rows), dim3(256),
+        hipLaunchKernelGGL(flash_decode_kernel<true>, dim3(splits, kAttnKvHeads, rows), dim3(kWaves * 64),
                            kWaves * kWaveLdsBytes, stream, f);
+    } else if (f.final_mode) {
+        hipLaunchKernelGGL((flash_decode_kernel<false, true>), dim3(splits, kAttnKvHeads, rows),
+                           dim3(kWaves * 64), kWaves * kWaveLdsBytes, stream, f);
     } else {
-        hipLaunchKernelGGL(flash_decode_kernel<false>, dim3(splits, kAttnKvHeads, rows), dim3(256),
+        hipLaunchKernelGGL(flash_decode_kernel<false>, dim3(splits, kAttnKvHeads, rows), dim3(kWaves * 64),
                            kWaves * kWaveLdsBytes, stream, f);
     }
     return TT_OK;
@@ -2226,7 +1584,8 @@ int32_t op_attention_split_ms(const Bindings& b, const Grid& g, hipStream_t stre
 }
 
 // attention_decode_combine_ms: b0 partials, b1 gate slab, b2 state_table,
-// b3 out slab, c4 part, c5 max_splits, c6 query stride, c7 long_rows_only;
+// b3 out slab, c4 part, c5 max_splits, c6 query stride, c7 long_rows_only, c8 capacity
+// (the one the split dispatch ran with: rows it refused are left alone here too);
 // grid (16, rows) x 256.
 int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t stream,
                                 bool validate_only) {
@@ -2236,9 +1595,11 @@ int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t st
     c.record_splits = a.constant(5);
     c.query_stride = a.constant(6);
     c.long_rows_only = a.constant(7);
+    c.capacity = a.constant(8);
     c.single_partition = kAttnPartition;
     const uint32_t rows = static_cast<uint32_t>(g.gy);
-    a.require(c.part != 0 && c.record_splits != 0 && c.query_stride >= kAttnQueryValues,
+    a.require(c.part != 0 && c.record_splits != 0 && c.query_stride >= kAttnQueryValues &&
+                  c.capacity != 0,
               TT_CMD_INVALID_BUFFER);
     a.require(g.gx == 16 && g.gz == 1 && rows >= 1 && rows <= kMaxBatchRows && g.tx == 256 &&
                   g.ty == 1 && g.tz == 1,
@@ -2261,7 +1622,9 @@ int32_t op_attention_combine_ms(const Bindings& b, const Grid& g, hipStream_t st
 // b5 state_table, b6 split records [rows][16][max_splits][258] fp32, b7 out slab
 // [rows][query stride], c8 capacity, c9 projection stride, c10 query stride, c11 part (keys
 // per workgroup, multiple of 32), c12 max_splits, c13 bit 1 interleave, bit 2 compact, bits
-// 3..7 rotate (as c9 of attention_decode_split_ms).
+// 3..7 rotate (as c9 of attention_decode_split_ms), c14 records per head the deepest row is
+// expected to have (0: as many as the buffer holds; a hint that sizes the finishing
+// dispatch's first batch of requests, any value gives the same result).
 struct TokenLayer {
     FlashArgs walk;
     FinishArgs finish;
@@ -2278,6 +1641,7 @@ TokenLayer token_layer_args(Args& a, uint32_t rows) {
     f.part = n.part = a.constant(11);
     f.record_splits = n.record_splits = a.constant(12);
     const uint32_t flags = a.constant(13);
+    n.parts_hint = a.constant(14);
     f.interleave = (flags >> 1) & 1;
     f.compact = (flags >> 2) & 1;
     f.rotate = (flags >> 3) & 31;
@@ -2334,92 +1698,6 @@ int32_t op_attention_token_finish_ms(const Bindings& b, const Grid& g, hipStream
     if (a.status != TT_OK || validate_only) return a.status;
     hipLaunchKernelGGL(attention_finish_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
                        t.finish);
-    return TT_OK;
-}
-
-constexpr uint32_t kLayerLdsBytes = kWaves * kWaveLdsBytes + kAttnHeadsPerKv * kD * 2 +
-                                    (2 * kMaxStreams + 8 + 2 * kMaxBatchRows) * 4;
-constexpr uint32_t kLayerTicketBytes = 256;   // tickets lead the scratch
-constexpr uint32_t kLayerQueryBytes = kMaxStreams * kAttnHeadsPerKv * kD * 2;  // then the queries
-constexpr uint32_t kMaxLayerGroups = 2048;   // keeps units x workgroups in 32 bits
-
-uint64_t layer_scratch_bytes(uint32_t groups, uint32_t rows) {
-    return kLayerTicketBytes + kLayerQueryBytes +
-           static_cast<uint64_t>(groups + rows * kAttnKvHeads - 1) * kAttnHeadsPerKv *
-               kAttnRecordFloats * 4;
-}
-
-// Bindings shared by the two dispatches of the whole-layer decode: b0 projection slab
-// [rows][projection stride], b1 q_w, b2 k_w, b3 keys_pool, b4 values_pool, b5 state_table,
-// b6 scratch (256 B of tickets, 128 KiB of query heads, then (groups + 2 rows - 1) x 8
-// records of 258 floats; zero before the first use, tickets left zeroed by every launch), b7 out slab [rows][query stride],
-// c8 capacity, c9 projection stride, c10 query stride.
-LayerArgs layer_args(Args& a, uint32_t rows, uint32_t groups) {
-    LayerArgs l{};
-    l.capacity = a.constant(8);
-    l.projection_stride = a.constant(9);
-    l.query_stride = a.constant(10);
-    l.rows = rows;
-    l.groups = groups;
-    a.require(rows >= 1 && rows <= kMaxBatchRows && groups >= 1 && groups <= kMaxLayerGroups,
-              TT_CMD_INVALID_DISPATCH_EXTENT);
-    a.require(l.capacity != 0 && l.projection_stride >= kAttnProjectionRows &&
-                  l.projection_stride % 4 == 0 && l.query_stride >= kAttnQueryValues,
-              TT_CMD_INVALID_BUFFER);
-    if (a.status != TT_OK) return l;
-    const uint64_t last = rows - 1;
-    l.projection =
-        a.buffer<const uint16_t>(0, (last * l.projection_stride + kAttnProjectionRows) * 2);
-    l.q_weight = a.buffer<const uint16_t>(1, kD * 2);
-    l.k_weight = a.buffer<const uint16_t>(2, kD * 2);
-    l.keys = a.buffer<uint16_t>(3, cache_bytes(l.capacity));
-    l.values = a.buffer<uint16_t>(4, cache_bytes(l.capacity));
-    l.table = a.buffer<const uint32_t>(5, rows * 16);
-    uint8_t* scratch_base = a.buffer<uint8_t>(6, layer_scratch_bytes(groups, rows));
-    l.out = a.buffer<uint16_t>(7, (last * l.query_stride + kAttnQueryValues) * 2);
-    if (scratch_base != nullptr) {
-        l.tickets = reinterpret_cast<uint32_t*>(scratch_base);
-        l.queries = reinterpret_cast<uint16_t*>(scratch_base + kLayerTicketBytes);
-        l.records = reinterpret_cast<float*>(scratch_base + kLayerTicketBytes + kLayerQueryBytes);
-    }
-    return l;
-}
-
-// attention_decode_layer_ms (no reference counterpart; attn_qk_rope_ms, the split path of
-// every row and the combine of decode_step.cpp:1231-1259 in one dispatch): bindings as
-// above, c11 finish mode (1: finished inside the dispatch by the last workgroup of each
-// stream; 0: attention_decode_layer_finish_ms follows); grid (groups, rows) x 256 -
-// `groups` workgroups are launched, the keys of all rows are dealt evenly among them.
-int32_t op_attention_layer_ms(const Bindings& b, const Grid& g, hipStream_t stream,
-                              bool validate_only) {
-    Args a(b);
-    a.require(g.gz == 1 && g.tx == 256 && g.ty == 1 && g.tz == 1, TT_CMD_INVALID_DISPATCH_EXTENT);
-    LayerArgs l = layer_args(a, static_cast<uint32_t>(std::min<uint64_t>(g.gy, 0xFFFF)),
-                             static_cast<uint32_t>(std::min<uint64_t>(g.gx, 0xFFFF)));
-    l.finish_in_kernel = a.constant(11) != 0 ? 1u : 0u;
-    if (a.status != TT_OK || validate_only) return a.status;
-    if (l.finish_in_kernel) {
-        hipLaunchKernelGGL(attention_decode_layer_kernel<true>, dim3(l.groups), dim3(256),
-                           kLayerLdsBytes, stream, l);
-    } else {
-        hipLaunchKernelGGL(attention_decode_layer_kernel<false>, dim3(l.groups), dim3(256),
-                           kLayerLdsBytes, stream, l);
-    }
-    return TT_OK;
-}
-
-// attention_decode_layer_finish_ms: bindings as above, c11 groups of the dispatch whose
-// records it merges; grid (16, rows) x 64.
-int32_t op_attention_layer_finish_ms(const Bindings& b, const Grid& g, hipStream_t stream,
-                                     bool validate_only) {
-    Args a(b);
-    a.require(g.gx == kAttnQueryHeads && g.gz == 1 && g.tx == 64 && g.ty == 1 && g.tz == 1,
-              TT_CMD_INVALID_DISPATCH_EXTENT);
-    LayerArgs l = layer_args(a, static_cast<uint32_t>(std::min<uint64_t>(g.gy, 0xFFFF)),
-                             a.constant(11));
-    if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(attention_layer_finish_kernel, dim3(kAttnQueryHeads, l.rows), dim3(64), 0,
-                       stream, l);
     return TT_OK;
 }
 
@@ -2496,15 +1774,12 @@ bool prepare_current_device() {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWaves * kWaveLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<true>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<false, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             kWaves * kWaveLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel<true>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(flash_decode_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLayerLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(attention_decode_layer_kernel<false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLayerLdsBytes) != hipSuccess) {
+                            kWaves * kWaveLdsBytes) != hipSuccess) {
         (void)hipGetLastError();
         return false;
     }
@@ -2546,8 +1821,6 @@ const KernelDesc kAttentionDecodeKernels[] = {
     {"attention_decode_combine_ms", op_attention_combine_ms},
     {"attention_decode_token_ms", op_attention_token_ms},
     {"attention_decode_token_finish_ms", op_attention_token_finish_ms},
-    {"attention_decode_layer_ms", op_attention_layer_ms},
-    {"attention_decode_layer_finish_ms", op_attention_layer_finish_ms},
 };
 const uint32_t kAttentionDecodeKernelCount =
     sizeof(kAttentionDecodeKernels) / sizeof(kAttentionDecodeKernels[0]);
@@ -2586,7 +1859,18 @@ extern "C" int32_t tt_attention_decode_lanes_static(
     const uint32_t splits = (capacity + split_keys - 1) / split_keys;
     const uint64_t row_floats = static_cast<uint64_t>(kAttnQueryHeads) * splits * kAttnRecordFloats;
     if (row_floats * rows * 4 > TT_STATIC_SCRATCH_BYTES) return TT_CMD_STATIC_SCRATCH_EXCEEDED;
-    if (!prepare_current_device()) return TT_CMD_INVALID_DEVICE;
+    // The device's one-time set-up is done when a queue is created; a caller that reaches
+    // this point without it (a queue of another device made current by hand) gets it here,
+    // unless the stream is capturing - the set-up calls are not capture-safe.
+    if (static_scratch() == nullptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
+            capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return TT_CMD_INVALID_DEVICE;
+        }
+        if (!prepare_current_device()) return TT_CMD_INVALID_DEVICE;
+    }
     float* records = static_cast<float*>(static_scratch());
     if (records == nullptr) return TT_CMD_INVALID_DEVICE;
 
@@ -2604,8 +1888,10 @@ extern "C" int32_t tt_attention_decode_lanes_static(
     f.single_partition = kAttnPartition;
     // a grid larger than the chip may hold workgroups without keys: the ones with keys first
     // (the contexts are on the device, so this cannot be decided more finely here)
-    f.compact = static_cast<uint64_t>(splits) * kAttnKvHeads * rows > 256 &&
+    const uint32_t units = queue_compute_units(queue);
+    f.compact = static_cast<uint64_t>(splits) * kAttnKvHeads * rows > (units != 0 ? units : 256u) &&
                 reinterpret_cast<uintptr_t>(state_table) % 8 == 0;
+    f.rotate = 1;   // ranges walked from a rotated starting block, whatever the capacity
     launch_flash(f, splits, rows, stream);
 
     CombineArgs c{};
@@ -2618,6 +1904,7 @@ extern "C" int32_t tt_attention_decode_lanes_static(
     c.query_stride = query_stride;
     c.partial_row_floats = row_floats;
     c.single_partition = kAttnPartition;
+    c.capacity = capacity;
     hipLaunchKernelGGL(attention_combine_kernel, dim3(kAttnQueryHeads, rows), dim3(256), 0, stream,
                        c);
     return hipGetLastError() == hipSuccess ? TT_OK : TT_CMD_INVALID_PENDING_EXECUTION;

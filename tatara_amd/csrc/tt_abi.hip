@@ -6,6 +6,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <new>
@@ -60,6 +61,10 @@ struct tt_pipeline {
 };
 
 namespace tt {
+uint32_t queue_compute_units(const tt_queue* queue) {
+    return queue != nullptr && queue->device != nullptr ? queue->device->compute_units : 0;
+}
+
 hipStream_t queue_stream(const tt_queue* queue) {
     return queue != nullptr ? queue->stream : nullptr;
 }
@@ -197,6 +202,30 @@ extern "C" {
 
 uint32_t tt_abi_version(void) { return TT_ABI_VERSION; }
 
+uint32_t tt_split_workgroups(const uint32_t* visible_keys, uint32_t rows, uint32_t split_keys) {
+    if (visible_keys == nullptr || split_keys == 0) return 0;
+    uint64_t groups = 0;
+    for (uint32_t r = 0; r < rows; ++r) {
+        groups += 2 * ((static_cast<uint64_t>(visible_keys[r]) + split_keys - 1) / split_keys);
+    }
+    return static_cast<uint32_t>(groups < UINT32_MAX ? groups : UINT32_MAX);
+}
+
+uint32_t tt_choose_split_keys(const uint32_t* visible_keys, uint32_t rows, uint32_t compute_units) {
+    const uint64_t units = compute_units == 0 ? 1 : compute_units;
+    uint64_t total = 0;
+    for (uint32_t r = 0; visible_keys != nullptr && r < rows; ++r) total += visible_keys[r];
+    // an even share of all keys, then coarser until the last, partly filled split of every
+    // row fits too: one workgroup more than compute units costs a third of the walk
+    uint64_t split = ((2 * total + units - 1) / units + 31) / 32 * 32;
+    if (split < 128) split = 128;
+    while (split < UINT32_MAX - 31 && 2 * static_cast<uint64_t>(rows) <= units &&
+           tt_split_workgroups(visible_keys, rows, static_cast<uint32_t>(split)) > units) {
+        split += 32;
+    }
+    return static_cast<uint32_t>(split);
+}
+
 const char* tt_status_name(int32_t status) {
     switch (status) {
     case TT_OK: return "None";
@@ -291,6 +320,10 @@ int32_t tt_queue_create(tt_device* device, tt_queue** out) {
     }
     queue->device = device;
     queue->stream = stream;
+    // The decode kernels' one-time set-up for this device (kernel attributes, the address
+    // of the static scratch): done here so that an entry point that launches directly on
+    // the queue never has to do it inside a stream capture.  A failure shows at that call.
+    (void)tt::prepare_decode_kernels();
     *out = queue;
     return TT_OK;
 }
@@ -714,6 +747,26 @@ static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool
         }
         (void)hipEventRecord(cb->marks[0], stream);
     }
+    // A wait whose signal has not been committed fails the whole commit before anything is
+    // launched: found at its own position, it would leave the command buffer half executed.
+    // (A signal earlier in this same command buffer reaches a later wait of it.)
+    {
+        std::map<const tt_event*, uint64_t> signalled_here;
+        for (const Command& command : cb->commands) {
+            if (command.kind == CommandKind::Signal) {
+                uint64_t& highest = signalled_here[command.event];
+                highest = std::max(highest, command.event_value);
+            } else if (command.kind == CommandKind::Wait) {
+                const auto here = signalled_here.find(command.event);
+                if (here != signalled_here.end() && here->second >= command.event_value) continue;
+                std::lock_guard<std::mutex> lock(command.event->mutex);
+                if (command.event->reached.lower_bound(command.event_value) ==
+                    command.event->reached.end()) {
+                    return hipErrorNotReady;
+                }
+            }
+        }
+    }
     size_t index = 0;
     for (const Command& command : cb->commands) {
         hipError_t error = hipSuccess;
@@ -725,10 +778,14 @@ static hipError_t issue_commands(tt_command_buffer* cb, hipStream_t stream, bool
             // a fresh HIP event per signalled value, recorded behind everything issued so far
             std::lock_guard<std::mutex> lock(command.event->mutex);
             hipEvent_t& reached = command.event->reached[command.event_value];
-            if (reached == nullptr) {
-                error = hipEventCreateWithFlags(&reached, hipEventDisableTiming);
-            }
+            const bool fresh = reached == nullptr;
+            if (fresh) error = hipEventCreateWithFlags(&reached, hipEventDisableTiming);
             if (error == hipSuccess) error = hipEventRecord(reached, stream);
+            if (error != hipSuccess && fresh) {
+                // no entry without a recorded event behind it: a later wait must not find one
+                if (reached != nullptr) (void)hipEventDestroy(reached);
+                command.event->reached.erase(command.event_value);
+            }
             // A wait takes the smallest committed value that reaches the one it asks for, so
             // the oldest values can go once there are many: a late wait for one of them is
             // served by a newer signal, which the counter has passed as well.

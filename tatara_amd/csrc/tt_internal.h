@@ -90,6 +90,8 @@ int32_t op_attn_qk_rope_blk(const Bindings& b, const Grid& g, hipStream_t stream
 // The HIP stream of a queue (tt_queue is defined by the C-ABI core), for entry points
 // that launch directly instead of recording.
 hipStream_t queue_stream(const tt_queue* queue);
+// Compute units of the device the queue was made on (0 for a null queue).
+uint32_t queue_compute_units(const tt_queue* queue);
 
 // One-time kernel attribute set-up (large dynamic LDS opt-in); called when a
 // library is created, so it never runs inside a stream capture.

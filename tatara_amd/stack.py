@@ -20,6 +20,8 @@ GDN planes ping-pong, attention caches append at the lane's context.
 """
 import numpy as np
 
+from tatara_amd import backend
+
 HIDDEN = 2048
 GDN_PROJ = 12352
 ATTN_PROJ = 9216
@@ -86,20 +88,17 @@ def make_weights(layers, vocab, seed, quantized=False):
 
 
 def split_workgroups(visible_keys, split_keys):
-    """Workgroups of one attention layer's split-K grid that hold keys (two kv heads)."""
-    return 2 * sum(-(-keys // split_keys) for keys in visible_keys)
+    """Workgroups of one attention layer's split-K grid that hold keys (two kv heads); the
+    backend library's rule, which the C++ runtime calls as well."""
+    return backend.split_workgroups(list(visible_keys), split_keys)
 
 
 def choose_split_keys(visible_keys, compute_units=256):
     """Keys per split-K workgroup for a token wave whose lanes see `visible_keys[r]` keys
     each: the finest multiple of 32, at least 128, with which the workgroups that hold
-    keys fit the compute units one each (runtime.cpp choose_split_keys)."""
-    visible_keys = list(visible_keys)
-    share = -(-2 * sum(visible_keys) // compute_units)
-    split = max(128, -(-share // 32) * 32)
-    while split_workgroups(visible_keys, split) > compute_units and 2 * len(visible_keys) <= compute_units:
-        split += 32
-    return split
+    keys fit the compute units one each.  The backend library's rule (tt_choose_split_keys),
+    the same call the C++ runtime makes."""
+    return backend.choose_split_keys(list(visible_keys), compute_units)
 
 
 class StubStack:
@@ -109,14 +108,15 @@ class StubStack:
     def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
                  split_keys=None, attention_form="three", fused_wave_steps=False):
         """attention_form: "three" records a token wave's attention layer as rope, split-K
-        and combine dispatches (split_keys keys per workgroup); "layer" as the whole-layer
-        dispatch plus its finishing dispatch (keys dealt evenly to one workgroup per compute
-        unit, whatever the lanes' depths).
+        and combine dispatches (split_keys keys per workgroup); "token" as the two-dispatch
+        form (attention_decode_token_ms norms and rotates the query heads inside the split-K
+        walk, attention_decode_token_finish_ms folds in and appends the token's own key and
+        value).
         fused_wave_steps: decode waves of several lanes over 4-bit weights take the norm in
         the prologue of the input projection and the residual sum in the epilogue of the
         output projection (same bits, one dispatch less per layer; measured slower, because
         every workgroup of the projection norms the rows again)."""
-        assert attention_form in ("three", "layer")
+        assert attention_form in ("three", "token")
         self.dev, self.lib = dev, lib
         self.attention_form = attention_form
         self.fused_wave_steps = fused_wave_steps
@@ -162,7 +162,6 @@ class StubStack:
         self.q, self.gate = mk(rows * 8192), mk(rows * 8192)
         self.decay, self.beta = mk(rows * 128), mk(rows * 128)
         self.partials = mk(lanes * 16 * self.max_splits * 258 * 4)
-        self.layer_scratch = mk(256 + 131072 + (self.groups + 2 * lanes - 1) * 8 * 258 * 4)
         self.chunk = mk(((min(block_rows, 2048) + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
         self.logits = mk(rows * vocab * 2)
         self._write_tables()
@@ -270,7 +269,8 @@ class StubStack:
         holds no keys, the workgroups that do go first (bit 2)."""
         live = split_workgroups([c + 1 for c in self.context[:rows]], self.split_keys)
         grid = self.max_splits * 2 * rows
-        return (2 if rows <= 2 else 0) | (4 if grid > live and grid > self.groups else 0)
+        # (bits 3..7: contiguous ranges are walked from a rotated starting block)
+        return (2 if rows <= 2 else 8) | (4 if grid > live and grid > self.groups else 0)
 
     # ---- one token for every lane ----
     def record_token_wave(self, cb, with_head=True):
@@ -286,15 +286,17 @@ class StubStack:
                           {0: self.proj, 1: layer["conv"], 2: layer["conv_w"], 3: layer["a_log"],
                            4: layer["dt_bias"], 5: layer["rec"], 6: layer["norm_w"], 7: self.mixed,
                            8: layer["table"]}, {9: GDN_PROJ, 10: 4096}, (32, rows), (512,))
-            elif self.attention_form == "layer":
+            elif self.attention_form == "token":
                 bind = {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: layer["keys"],
-                        4: layer["values"], 5: layer["table"], 6: self.layer_scratch, 7: self.mixed}
-                const = {8: self.capacity, 9: ATTN_PROJ, 10: 4096}
-                cb.encode(P("attention_decode_layer_ms"), bind, {**const, 11: 0},
-                          (self.groups, rows), (256,))
+                        4: layer["values"], 5: layer["table"], 6: self.partials, 7: self.mixed}
+                deepest = max(self.context[:rows])
+                const = {8: self.capacity, 9: ATTN_PROJ, 10: 4096, 11: self.split_keys,
+                         12: self.max_splits, 13: self._split_flags(rows),
+                         14: -(-deepest // self.split_keys)}
+                cb.encode(P("attention_decode_token_ms"), bind, const, (self.max_splits, 2, rows),
+                          (256,))
                 cb.barrier()
-                cb.encode(P("attention_decode_layer_finish_ms"), bind, {**const, 11: self.groups},
-                          (16, rows), (64,))
+                cb.encode(P("attention_decode_token_finish_ms"), bind, const, (16, rows), (256,))
             else:
                 cb.encode(P("attn_qk_rope_ms"),
                           {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,
@@ -310,7 +312,8 @@ class StubStack:
                 cb.barrier()
                 cb.encode(P("attention_decode_combine_ms"),
                           {0: self.partials, 1: self.gate, 2: layer["table"], 3: self.mixed},
-                          {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0}, (16, rows), (256,))
+                          {4: self.split_keys, 5: self.max_splits, 6: 4096, 7: 0, 8: self.capacity},
+                          (16, rows), (256,))
             cb.barrier()
             self._project_out(cb, layer, rows, block=False)
             if not self._fused_wave(layer, rows):

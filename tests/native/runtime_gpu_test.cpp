@@ -276,12 +276,12 @@ int main() {
             streams.push_back({&pooled.slots[stripes[r]], contexts[r], stripes[r]});
         }
         // first wave: rope, split path, combine and the short-row bucket; second wave: the
-        // whole-layer dispatch and its finishing dispatch - both held to the same checker rows
-        batch.attention_whole_layer = token == 1;
+        // token form (rope inside the walk) and its finishing dispatch - both held to the same checker rows
+        batch.attention_token_form = token == 1;
         const int rc = submit.run([&](HipComputePass& pass) {
             return encode_token_batch(step, streams, *pooled.pool, batch, bound, no_hooks, pass);
         });
-        batch.attention_whole_layer = false;
+        batch.attention_token_form = false;
         if (rc != 0) return 20 + rc;
         const auto gated = download<std::uint16_t>(batch.gdn_gated, kLanes * 4096);
         const auto attended = download<std::uint16_t>(batch.attn_attended, kLanes * 4096);
@@ -403,10 +403,7 @@ int main() {
             // hold keys are placed first in the dispatch order
             batch.split_keys = wave == 0 ? 256 : 0;
             const std::uint32_t chip_units = batch.compute_units;
-            if (wave == 1) {
-                batch.compute_units = 4;
-                batch.split_order = DecodeBatchScratch::SplitOrder::BlocksInTurn;   // pinned, three rows
-            }
+            if (wave == 1) batch.compute_units = 4;
             std::vector<std::uint16_t> x = gauss16(7400 + wave, kLanes * 2048);
             if (!upload(hidden.input, x)) return 206;
             std::vector<DecodeStream> streams;
@@ -418,7 +415,6 @@ int main() {
                                           pass);
             });
             batch.compute_units = chip_units;
-            batch.split_order = DecodeBatchScratch::SplitOrder::Automatic;
             if (rc != 0) return 210 + rc;
             const auto got_residual = download<std::uint16_t>(hidden.residual, kLanes * 2048);
             const auto got_normed = download<std::uint16_t>(hidden.normed, kLanes * 2048);

@@ -246,7 +246,7 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
                   {0: b_part, 1: b_g, 2: b_tab, 3: b_o},
-                  {4: part, 5: max_splits, 6: 4096, 7: 1}, (16, rows), (256,))
+                  {4: part, 5: max_splits, 6: 4096, 7: 1, 8: cap}, (16, rows), (256,))
         if short:
             cb.encode(lib.pipeline("attention_decode_ms"),
                       {0: b_q, 1: b_g, 2: k_pool, 3: v_pool, 4: b_tab, 5: b_o,
@@ -331,7 +331,7 @@ def test_compact_walk_compiled_once_replayed_while_contexts_grow():
               {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 4}, (max_splits, 2, rows), (256,))
     cb.barrier()
     cb.encode(lib.pipeline("attention_decode_combine_ms"),
-              {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0},
+              {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0, 8: cap},
               (16, rows), (256,))
     cb.end_compute_pass()
     cb.compile()
@@ -388,7 +388,7 @@ def test_table_rows_past_the_capacity_are_left_alone(compact):
                   (max_splits, 2, rows), (256,))
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
-                  {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0},
+                  {0: b_part, 1: b_g, 2: b_tab, 3: b_o}, {4: part, 5: max_splits, 6: 4096, 7: 0, 8: cap},
                   (16, rows), (256,))
     run(rec)
     got = b_o.read(np.uint16).reshape(rows, 4096)

@@ -138,10 +138,13 @@ def test_scores_far_above_the_first_tile_take_the_exact_loop():
 
 def test_config4_prefill_16384_rows():
     """Config 4: 16384 new tokens into an empty capacity-16384 cache.  The checker
-    computes a strided subset of query rows (every 256th plus the first and last
-    16); the K/V cache written by the rope stage is compared in full."""
+    computes a strided subset of query rows (every 257th plus the first and last
+    16: a stride coprime with the kernel's 32-row tile, so every row of a tile is
+    compared somewhere at depth); the K/V cache written by the rope stage is compared in
+    full."""
     print("[case] config 4: prefill 16384 rows", flush=True)
     rows = 16384
-    sel = sorted(set(list(range(16)) + list(range(0, rows, 256)) + list(range(rows - 16, rows))))
+    sel = sorted(set(list(range(16)) + list(range(0, rows, 257)) + list(range(rows - 16, rows))))
+    assert {r % 32 for r in sel} == set(range(32))
     ms, _ = _prefill_case(rows, 0, rows, 0xC0F4, select=sel)
     print(f"[time] rope + flash prefill 16384 rows (first run): {ms:.3f} ms", flush=True)

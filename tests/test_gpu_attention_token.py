@@ -28,7 +28,8 @@ def flags(interleave=0, compact=0, rotate=0):
 
 
 def token_batch(contexts, cap, forms, seed, replays=0, projection_stride=9216,
-                query_stride=4096, stripes=None, pool_stripes=None, against_rope=False):
+                query_stride=4096, stripes=None, pool_stripes=None, against_rope=False,
+                parts_hint=None):
     """forms: list of (part, flags).  Returns the outputs per form."""
     B, dev, queue, lib = gpu()
     rows = len(contexts)
@@ -73,7 +74,9 @@ def token_batch(contexts, cap, forms, seed, replays=0, projection_stride=9216,
             v_pool.write(v, stripes[r] * stride)
         b_o = dev.create_buffer(rows * query_stride * 2)
         bind = {0: b_proj, 1: b_qw, 2: b_kw, 3: k_pool, 4: v_pool, 5: b_tab, 6: b_rec, 7: b_o}
-        const = {8: cap, 9: projection_stride, 10: query_stride, 11: part, 12: splits, 13: flag}
+        hint = parts_hint if parts_hint is not None else -(-max(contexts) // part)
+        const = {8: cap, 9: projection_stride, 10: query_stride, 11: part, 12: splits, 13: flag,
+                 14: hint}
 
         def rec(cb, bind=bind, const=const, splits=splits):
             cb.encode(lib.pipeline("attention_decode_token_ms"), bind, const, (splits, 2, rows), (256,))
@@ -156,3 +159,12 @@ def test_token_sixteen_lanes():
     print("[case] token layer, 16 lanes", flush=True)
     contexts = [37 * (i + 1) + (i % 3) * 200 for i in range(16)]
     token_batch(contexts, 1024, [(256, flags(compact=1, rotate=1)), (1024, 0)], 0x1616, replays=1)
+
+
+@pytest.mark.parametrize("hint", [0, 1, 3, 40, 200])
+def test_token_finish_hint_is_only_a_hint(hint):
+    """The finishing dispatch sizes its first batch of record requests by the caller's hint;
+    whatever the hint (none, too small, too large), every record is merged: 1..157 records
+    per head here, past the largest batch of 128."""
+    print(f"[case] token layer, finish hint {hint}", flush=True)
+    token_batch([5000, 31, 2100, 0], 5024, [(32, flags(rotate=1))], 0x7117, parts_hint=hint)

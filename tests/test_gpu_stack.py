@@ -105,16 +105,19 @@ def _compare(step, got, want):
           f"argmax {got.argmax()} / {want.argmax()} top-2 gap {top2[1] - top2[0]:.3e}", flush=True)
     assert np.isfinite(got).all()
     assert err.mean() <= 2e-2 * max(1.0, np.abs(want).max())
+    # no single logit far off either: eight bf16 steps of the largest logit (the logits are
+    # bf16 values of a 2048-term sum behind a stack of bf16 stages)
+    step16 = 2.0 ** (np.floor(np.log2(max(np.abs(want).max(), 1e-30))) - 7)
+    assert err.max() <= 8 * step16, f"{step}: a logit is off by {err.max():.3e} (bf16 step {step16:.3e})"
     if got.argmax() != want.argmax():
         # a tie within the noise of the run: the checker itself ranks the GPU's choice below its
         # own by no more than two bf16 steps of the winning logit, or by no more than the two
-        # vectors differ anywhere (a gap smaller than the error of a logit decides nothing; the
-        # error itself is held by the mean bar above)
-        step16 = 2.0 ** (np.floor(np.log2(max(abs(want.max()), 1e-30))) - 7)
+        # competing logits themselves are off (a gap smaller than their error decides nothing)
         margin = want.max() - want[got.argmax()]
+        competing = err[got.argmax()] + err[want.argmax()]
         print(f"[parity] {step}: argmax differs on a margin of {margin:.3e} (bf16 step {step16:.3e}, "
-              f"largest logit error {err.max():.3e})", flush=True)
-        assert margin <= max(2 * step16, err.max()), step
+              f"error of the two logits {competing:.3e})", flush=True)
+        assert margin <= max(2 * step16, competing), step
 
 
 @pytest.mark.parametrize("layers,quantized,fused", [(40, False, False), (12, True, False), (12, True, True)],
@@ -341,13 +344,14 @@ def _depth_reference(layers, vocab, capacity, prompts, waves):
     return _DEPTH[key]
 
 
-@pytest.mark.parametrize("form", ["three", "layer"])
+@pytest.mark.parametrize("form", ["three", "token"])
 def test_stacked_run_at_depth_four_ragged_lanes(form):
     """Config 5 at depth: 12 layers (G,G,G,A x 3), four lanes with prompts of 1024, 640,
     384 and 160 tokens prefilled in blocks of 512 rows (two blocks for the longer ones), then
     three greedy token waves of all four lanes through the pooled-state operators, with the
-    split size the stack chooses for itself (form "three") or the whole-layer dispatch (form
-    "layer").  Every greedy token must be the checker's (ties within two bf16 steps of the
+    split size the stack chooses for itself, as rope + split-K + combine (form "three") or
+    with the rope inside the walk and the token folded in by the finishing dispatch (form
+    "token").  Every greedy token must be the checker's (ties within two bf16 steps of the
     winning logit aside, as in the shallow run)."""
     print(f"[case] stacked run at depth, attention form {form}", flush=True)
     from tatara_amd import stack as S

@@ -47,11 +47,11 @@ def _case(contexts, cap, part, seed):
     def rec(cb):
         cb.encode(lib.pipeline("attention_decode_split_ms"),
                   {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
-                  {5: cap, 6: 4096, 7: part, 8: splits, 9: 0}, (splits, 2, rows), (256,))
+                  {5: cap, 6: 4096, 7: part, 8: splits, 9: 8}, (splits, 2, rows), (256,))   # rotated ranges, as the entry point walks them
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
                   {0: b_part, 1: b_g, 2: b_tab, 3: b_ref},
-                  {4: part, 5: splits, 6: 4096, 7: 0}, (16, rows), (256,))
+                  {4: part, 5: splits, 6: 4096, 7: 0, 8: cap}, (16, rows), (256,))
     run(rec)
     reference = b_ref.read(np.uint16).reshape(rows, 4096)
     b_out = dev.create_buffer(rows * 8192)
@@ -114,3 +114,26 @@ def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
     assert e.value.status == 15
     # nothing above launched anything: the valid call still gives the reference bits
     _call_and_check(queue, case, "after rejected calls")
+
+
+def test_static_scratch_row_outside_its_cache_is_left_alone():
+    """A table row whose context is not a position of the cache (here: equal to the capacity,
+    and the all-ones word) has no records of the call; its output row must stay untouched,
+    whatever an earlier, larger call left in the shared scratch."""
+    print("[case] no-alloc entry: a row outside its cache after a larger call", flush=True)
+    B, dev, queue, lib = gpu()
+    large = _case([4095, 2500, 100], 4096, 128, 0x2A05)
+    _call_and_check(queue, large, "larger call first")
+    small = _case([500, 300], 1000, 96, 0x2A06)      # capacity not a multiple of the split
+    b_q, b_g, k_pool, v_pool, b_tab, b_out = small["operands"]
+    for bad in (1000, 0xFFFFFFFF):
+        table = b_tab.read(np.uint32)
+        table[1 * 4 + 1] = bad
+        b_bad = dev.buffer_from(table)
+        sentinel = np.full(2 * 4096, 0x1234, np.uint16)
+        b_out.write(sentinel)
+        queue.attention_decode_lanes_static(b_q, b_g, k_pool, v_pool, b_bad, b_out, 2, 1000, 4096, 96)
+        queue.synchronize()
+        got = b_out.read(np.uint16).reshape(2, 4096)
+        assert np.array_equal(got[0], small["reference"][0]), f"context {bad}: the good row changed"
+        assert np.array_equal(got[1], sentinel[:4096]), f"context {bad}: the refused row was written"
