@@ -183,6 +183,30 @@ class StubStack:
         for layer in self.layers:
             layer["table"].write(gdn if layer["kind"] == "G" else att)
 
+    def install_lane_state(self, lane, context, states):
+        """Writes a lane's whole state as it would stand after `context` tokens, without
+        running them: states[i] holds layer i's arrays - {"conv": [3 x 8192] bf16, "rec":
+        [32 x 128 x 128] fp32} for a Gated DeltaNet layer, {"keys", "values"}: [2 x capacity
+        x 256] bf16 for an attention layer - the record body of the reference's state record
+        (tools/native/decode_harness.cpp:339-460) in host arrays.  GDN planes go to the
+        lane's live plane; the tables are rewritten."""
+        assert 0 <= context < self.capacity and len(states) == len(self.layers)
+        live, _ = self._gdn_planes(lane)
+        stripe_bytes = 2 * self.capacity * 256 * 2
+        for layer, state in zip(self.layers, states):
+            if layer["kind"] == "G":
+                layer["conv"].write(np.ascontiguousarray(state["conv"], np.uint16).reshape(-1),
+                                    live * CONV_ELEMS * 2)
+                layer["rec"].write(np.ascontiguousarray(state["rec"], np.float32).reshape(-1),
+                                   live * REC_ELEMS * 4)
+            else:
+                layer["keys"].write(np.ascontiguousarray(state["keys"], np.uint16).reshape(-1),
+                                    lane * stripe_bytes)
+                layer["values"].write(np.ascontiguousarray(state["values"], np.uint16).reshape(-1),
+                                      lane * stripe_bytes)
+        self.context[lane] = context
+        self._write_tables()
+
     # ---- shared steps ----
     def _dense(self, cb, x, w, out, rows, k, n):
         cb.encode(self.lib.pipeline("dense_bf16"), {0: x, 1: w, 2: out}, {3: rows, 4: k, 5: n},

@@ -390,3 +390,105 @@ def test_stacked_run_at_depth_four_ragged_lanes(form):
         for lane in range(len(prompts)):
             _compare(f"depth wave {step} lane {lane} (context {stack.context[lane] - 1})",
                      got[lane], want_rows[lane])
+
+
+# ---- token waves over deep, installed state -----------------------------------------------
+
+_DEEP = {}
+
+
+def _deep_states(weights, capacity, contexts, seed):
+    """Synthetic lane states as they might stand after `contexts[lane]` tokens: caches of
+    N(0, 1) keys and values up to the context (NaN beyond it: a row past the context must
+    never be read), conv windows N(0, 0.5), recurrent states N(0, 0.02).  A generator of
+    (lane, states): the same seeds give the same arrays for the checker and for the GPU."""
+    for lane, context in enumerate(contexts):
+        rng = np.random.default_rng(seed + 101 * lane)
+        states = []
+        for lw in weights["layers"]:
+            if lw["kind"] == "G":
+                conv = (rng.standard_normal(3 * 8192, dtype=np.float32) * np.float32(0.5))
+                rec = rng.standard_normal(32 * 128 * 128, dtype=np.float32) * np.float32(0.02)
+                states.append({"conv": ol.f32_to_bf16(conv), "rec": rec})
+            else:
+                def cache():
+                    c = np.full((2, capacity, 256), 0x7FC0, np.uint16)
+                    c[:, :context] = ol.f32_to_bf16(
+                        rng.standard_normal(2 * context * 256, dtype=np.float32)).reshape(2, context, 256)
+                    return c.reshape(-1)
+                states.append({"keys": cache(), "values": cache()})
+        yield lane, states
+
+
+def _deep_reference(layers, vocab, capacity, contexts, waves, seed):
+    """The checker's side of greedy token waves over installed deep state, evaluated once
+    for both attention forms.  Its dense projections are numpy float32 products (another
+    summation order than tto_dense_bf16, which the operator-level test holds the kernel to);
+    everything of the attention family is the checker's own arithmetic."""
+    from tatara_amd import stack as S
+    key = (layers, vocab, capacity, tuple(contexts), waves, seed)
+    if key in _DEEP:
+        return _DEEP[key]
+    weights = S.make_weights(layers, vocab, seed)
+    embed = weights["embed"].reshape(vocab, 2048)
+    lanes = []
+    for lane, states in _deep_states(weights, capacity, contexts, seed):
+        checker = OracleLane(weights, capacity, vocab, fast_dense=True)
+        checker.state = states
+        checker.context = contexts[lane]
+        lanes.append(checker)
+    tokens = [int(t) for t in np.random.default_rng(seed ^ 0x70C).integers(0, vocab, len(contexts))]
+    steps = []
+    for step in range(waves):
+        print(f"[checker] deep greedy wave {step}", flush=True)
+        row = [lanes[lane].block(np.ascontiguousarray(embed[tokens[lane]]), 1)[0]
+               for lane in range(len(contexts))]
+        steps.append((list(tokens), row))
+        tokens = [int(r.argmax()) for r in row]
+    _DEEP[key] = (weights, steps)
+    return _DEEP[key]
+
+
+def _deep_waves(form, layers, capacity, contexts, seed, waves=2, vocab=4096):
+    from tatara_amd import stack as S
+    B, dev, queue, lib = gpu()
+    weights, want_steps = _deep_reference(layers, vocab, capacity, contexts, waves, seed)
+    embed = weights["embed"].reshape(vocab, 2048)
+    stack = S.StubStack(dev, lib, weights, len(contexts), capacity, vocab, block_rows=64,
+                        attention_form=form)
+    print(f"[plan] {len(contexts)} lanes, capacity {capacity}: {stack.split_keys} keys per "
+          f"workgroup, {stack.max_splits} splits", flush=True)
+    assert stack.split_keys == S.choose_split_keys([capacity] * len(contexts), dev.compute_units)
+    for lane, states in _deep_states(weights, capacity, contexts, seed):
+        stack.install_lane_state(lane, contexts[lane], states)
+    for step, (tokens, want_rows) in enumerate(want_steps):
+        stack.x.write(np.ascontiguousarray(embed[tokens]).reshape(-1))
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass()
+        stack.record_token_wave(cb)
+        cb.end_compute_pass()
+        cb.commit().wait()
+        stack.advance_token_wave()
+        got = ol.bf16_to_f32(stack.logits.read(np.uint16, len(contexts) * vocab)).reshape(-1, vocab)
+        for lane in range(len(contexts)):
+            _compare(f"deep wave {step} lane {lane} (context {stack.context[lane] - 1}, {form})",
+                     got[lane], want_rows[lane])
+
+
+@pytest.mark.parametrize("form", ["three", "token"])
+def test_token_waves_at_32k_depth_forty_layers(form):
+    """Config 5 where the sweep times it: all 40 layers, four ragged lanes around 32k keys
+    (32767 - the last position but one of the cache -, 30000, 24576, 8191), their state
+    installed directly, two greedy token waves through state table, split planner (the split
+    the stack picks for the capacity, with whatever dispatch order and block order follow
+    from it) and both attention forms.  Every greedy token must be the checker's."""
+    print(f"[case] 40 layers, 4 ragged lanes at 32k depth, form {form}", flush=True)
+    _deep_waves(form, 40, 32768 + 64, [32767, 30000, 24576, 8191], 0xDEE9)
+
+
+@pytest.mark.parametrize("form", ["three", "token"])
+def test_token_waves_one_lane_at_100k_depth(form):
+    """One lane of 100000 cached keys through 12 layers (three attention layers): the deep
+    single-lane shape of config 3 inside the stack, blocks dealt in turn."""
+    print(f"[case] 12 layers, 1 lane at 100k depth, form {form}", flush=True)
+    _deep_waves(form, 12, 100096, [100000], 0xDEEA)
