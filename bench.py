@@ -336,6 +336,130 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
             "kernel_ms": {k: round(v, 3) for k, v in best.items()}}
 
 
+CONFIG5_DECODE_CONTEXTS = (1024, 4096, 16384, 32768, 65536, 100000)
+CONFIG5_PREFILL_TOKENS = (4096, 32768)
+CONFIG5_LANES = (1, 4)
+CONFIG5_BLOCK_ROWS = 2048
+
+
+def config5_decode_point(dev, queue, lib, torch, attention, lanes, visible):
+    """One decode token wave of `lanes` lanes at `visible` visible keys through the
+    attention family of all 40 layers (own caches and state per layer), compiled into one
+    graph and replayed: device time of whole replays, launch gaps and all."""
+    capacity = (visible + 1023) // 1024 * 1024
+    attention_layers = LAYERS // PERIOD
+    wave = Wave(dev, lib, torch, attention, 0, attention_layers, LAYERS - attention_layers,
+                [visible - 1] * lanes, capacity)
+    step = time_graph(queue, wave.record_wave, 1, replays=10, warm=2)
+    us = step["median_us"]
+    kv = attention_layers * wave.visible_keys() * ATTN_BYTES_PER_KEY
+    gdn = (LAYERS - attention_layers) * lanes * GDN_BYTES_PER_LANE_LAYER
+    split = wave.part if attention == "three" else wave.token_part
+    del wave
+    torch.cuda.empty_cache()
+    return {"lanes": lanes, "visible_keys": visible, "capacity": capacity, "split_keys": split,
+            "wave_us": us, "wave_p10_us": step["p10_us"], "wave_p90_us": step["p90_us"],
+            "us_per_layer": round(us / LAYERS, 3), "tok_per_s": round(lanes / (us * 1e-6)),
+            "algorithmic_gbs": round((kv + gdn) / (us * 1e-6) / 1e9, 1)}
+
+
+def config5_prefill_point(dev, queue, lib, torch, lanes, tokens):
+    """`tokens` new tokens of each of `lanes` lanes, lane after lane, through the attention
+    family of all 40 layers in blocks of 2048 rows: per Gated DeltaNet layer conv, gates,
+    chunk-64 recurrence and gate-norm, per attention layer rope and causal flash attention
+    over the lane's cache so far.  Own caches and recurrent state per layer and lane;
+    the projections (resident random slabs) are shared by the layers of a kind.  Device time
+    of each block's command buffer (launch gaps included), summed."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0xC5F1 + tokens)
+    rows_max = min(CONFIG5_BLOCK_ROWS, tokens)
+    mk = dev.create_buffer
+
+    def rb(n, sigma=1.0):
+        t = (torch.randn(n, generator=gen, device="cuda") * sigma).to(torch.bfloat16)
+        return dev.wrap(t.data_ptr(), n * 2, keepalive=t)
+
+    P = lib.pipeline
+    ones256 = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
+    ones128 = dev.buffer_from(np.full(128, 0x3F80, np.uint16))
+    a_proj, g_proj = rb(rows_max * 9216), rb(rows_max * 12352, 0.5)
+    conv_w = rb(4 * 8192, 0.5)
+    rng = np.random.default_rng(5)
+    a_log = dev.buffer_from((rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16)
+                            .astype(np.uint16))
+    dt_bias = dev.buffer_from(np.zeros(32, np.uint16))
+    q, gate, out = (mk(rows_max * 8192) for _ in range(3))
+    qk, v, z, y = (mk(rows_max * 8192) for _ in range(4))
+    decay, beta = mk(rows_max * 128), mk(rows_max * 128)
+    chunk = mk(((rows_max + 63) // 64) * 32 * 115712)
+    attention_layers = LAYERS // PERIOD
+    stripe_bytes = 2 * tokens * 256 * 2
+    caches = [(mk(lanes * stripe_bytes), mk(lanes * stripe_bytes)) for _ in range(attention_layers)]
+    conv_bytes, rec_bytes = 3 * 8192 * 2, 32 * 128 * 128 * 4
+    states = [(mk(2 * lanes * conv_bytes), mk(2 * lanes * rec_bytes))
+              for _ in range(LAYERS - attention_layers)]
+    total_ms = 0.0
+    for lane in range(lanes):
+        swapped = False
+        for base in range(0, tokens, CONFIG5_BLOCK_ROWS):
+            rows = min(CONFIG5_BLOCK_ROWS, tokens - base)
+            cb = queue.create_command_buffer()
+            cb.begin_compute_pass()
+            attn = gdn = 0
+            for layer in range(LAYERS):
+                if layer % PERIOD == PERIOD - 1:
+                    keys = (caches[attn][0], lane * stripe_bytes)
+                    values = (caches[attn][1], lane * stripe_bytes)
+                    attn += 1
+                    cb.encode(P("attn_qk_rope_blk"),
+                              {0: a_proj, 1: ones256, 2: ones256, 3: q, 4: gate, 5: keys, 6: values},
+                              {7: base, 8: tokens}, (18, rows), (256,))
+                    cb.barrier()
+                    cb.encode(P("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: out},
+                              {5: base + rows, 6: tokens, 7: rows, 8: base},
+                              (16, (rows + 15) // 16), (256,))
+                else:
+                    conv, rec = states[gdn]
+                    gdn += 1
+                    plane_in, plane_out = (2 * lane + 1, 2 * lane) if swapped else (2 * lane, 2 * lane + 1)
+                    cb.encode(P("gdn_conv_blk"),
+                              {0: g_proj, 1: (conv, plane_in * conv_bytes), 2: conv_w, 3: qk, 4: v, 5: z,
+                               6: (conv, plane_out * conv_bytes)}, {7: rows}, (96, rows), (128,))
+                    cb.encode(P("gdn_gates_blk"), {0: g_proj, 1: a_log, 2: dt_bias, 3: decay, 4: beta},
+                              {5: rows}, (1, (rows + 3) // 4, 1), (32, 4, 1))
+                    cb.barrier()
+                    cb.encode(P("gdn_chunk_recurrence_blk"),
+                              {0: qk, 1: v, 2: decay, 3: beta, 4: chunk, 5: (rec, plane_in * rec_bytes),
+                               6: y, 7: (rec, plane_out * rec_bytes)}, {8: rows}, (8, 32), (256,))
+                    cb.barrier()
+                    cb.encode(P("gdn_gate_norm_blk"), {0: y, 1: z, 2: ones128, 3: out}, {},
+                              (32, rows), (128,))
+                cb.barrier()
+            cb.end_compute_pass()
+            total_ms += cb.commit().wait()
+            swapped = not swapped
+    total = lanes * tokens
+    del caches, states
+    torch.cuda.empty_cache()
+    return {"lanes": lanes, "tokens": tokens, "block_rows": CONFIG5_BLOCK_ROWS,
+            "family_ms": round(total_ms, 3), "tok_per_s": round(total / (total_ms * 1e-3)),
+            "us_per_layer_token": round(total_ms * 1e3 / (LAYERS * total), 4)}
+
+
+def config5_figures(dev, queue, lib, torch, attention):
+    """The hybrid stack sweep: decode waves at six depths and blocked prefill of two prompt
+    lengths, one lane and four, attention family of all 40 layers only (the projections are
+    resident inputs, as in the headline)."""
+    decode = [config5_decode_point(dev, queue, lib, torch, attention, lanes, visible)
+              for lanes in CONFIG5_LANES for visible in CONFIG5_DECODE_CONTEXTS]
+    prefill = [config5_prefill_point(dev, queue, lib, torch, lanes, tokens)
+               for lanes in CONFIG5_LANES for tokens in CONFIG5_PREFILL_TOKENS]
+    return {"layers": LAYERS, "pattern": "G,G,G,A x 10", "attention_form": attention,
+            "decode": decode, "prefill": prefill,
+            "how": "decode: one HIP-graph replay per token wave, median of 10; prefill: device "
+                   "time of every 2048-row block's command buffer, summed, lane after lane"}
+
+
 def _oracle():
     path = os.path.join(ROOT, "oracle", "liboracle.so")
     if not os.path.exists(path):
@@ -467,6 +591,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the 16384-row block prefill figures in detail.prefill_16k")
+    ap.add_argument("--no-config5", action="store_true",
+                    help="skip the stack sweep in detail.config5 (decode waves at 1k ... 100k keys and "
+                         "blocked prefill of 4k / 32k tokens, 1 and 4 lanes)")
     ap.add_argument("--no-config3", action="store_true",
                     help="skip the ragged-lane and deep-lane figures in detail.config3")
     ap.add_argument("--split-keys", type=int, default=0,
@@ -575,6 +702,8 @@ def main():
     else:
         del wave, step
         torch.cuda.empty_cache()
+    if not args.no_config5:
+        line["detail"]["config5"] = config5_figures(dev, queue, lib, torch, args.attention)
     # host threads of the CPU legs: what this process may run on, bounded by the box's CPU
     # share where the environment states one (OMP_NUM_THREADS)
     threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
