@@ -57,7 +57,7 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
 # counter read for a plain 256 MiB copy of known size; see the file named here.
 TRAFFIC_SOURCE = "profiles/flash_decode_4x32768_hbm_counters.md"
-TRAFFIC_BYTES = round((131297.1 * 262144.0 / 131083.3 + 2112.0) * 1024)   # 271,035,969
+TRAFFIC_BYTES = round((131289.6 * 262144.0 / 131083.3 + 2181.5) * 1024)   # 271,091,778
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 CONFIG3 = {
