@@ -65,6 +65,7 @@ CONFIG3 = {
     "ragged": ([32767, 29999, 24575, 8191], CAPACITY),
     "lane100k": ([99999], 100096),
 }
+CAPACITY_SWEEP = (33024, 100096, 131072, 131136, 262144)
 
 
 class Wave:
@@ -698,6 +699,22 @@ def main():
         config3["lane100k"] = attention_figures(queue, deep)
         del deep
         torch.cuda.empty_cache()
+        # the uniform wave again in caches of other capacities: the stride between the ranges
+        # of a lane's workgroups, between heads and between lanes is the capacity's, and the
+        # walk must not depend on how those strides fall on the memory channels
+        config3["uniform_by_capacity"] = []
+        for capacity in CAPACITY_SWEEP:
+            other = Wave(dev, lib, torch, args.attention, args.split_keys, 4, 0,
+                         CONFIG3["uniform"][0], capacity)
+            figures = attention_figures(queue, other)
+            config3["uniform_by_capacity"].append(
+                {"capacity": capacity, "split_keys": figures["split_keys"],
+                 "workgroups_with_keys_first": figures["workgroups_with_keys_first"],
+                 "walk_kernel": figures["walk_kernel"], "walk_kernel_frac": figures["walk_kernel_frac"],
+                 "layer_all_dispatches": figures["layer_all_dispatches"],
+                 "layer_frac": figures["layer_frac"]})
+            del other
+            torch.cuda.empty_cache()
         line["detail"]["config3"] = config3
     else:
         del wave, step

@@ -187,10 +187,12 @@ def test_decode_context_edges(ctx):
 
 
 def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=False,
-                stripes=None, pool_stripes=None, sharpen=0):
+                stripes=None, pool_stripes=None, sharpen=0, rotate=0):
     """Lane-batched decode over a striped pool with a state table, long rows
     through attention_decode_split_ms and short rows through attention_decode_ms.
     interleave: a lane's workgroups take its 32-key blocks in turn (bit 1 of c9).
+    rotate: a workgroup starts (split + 5 kv head + 11 row) * rotate blocks into its range
+    and wraps (bits 3-7 of c9); the same keys per record in another order.
     compact: the workgroups whose splits hold keys lead the dispatch order (bit 2 of c9);
     the records, and so the output bits, are those of the plain order.
     stripes / pool_stripes: which stripe of a pool of `pool_stripes` each lane lives on
@@ -241,7 +243,8 @@ def _lane_batch(contexts, cap, part, seed, replays=0, interleave=False, compact=
     def rec(cb):
         cb.encode(lib.pipeline("attention_decode_split_ms"),
                   {0: b_q, 1: k_pool, 2: v_pool, 3: b_tab, 4: b_part},
-                  {5: cap, 6: 4096, 7: part, 8: max_splits, 9: 1 + 2 * int(interleave) + 4 * int(compact)},
+                  {5: cap, 6: 4096, 7: part, 8: max_splits,
+                   9: 1 + 2 * int(interleave) + 4 * int(compact) + 8 * int(rotate)},
                   (max_splits, 2, rows), (256,))
         cb.barrier()
         cb.encode(lib.pipeline("attention_decode_combine_ms"),
@@ -605,10 +608,11 @@ def test_lane_batch_drawn_shapes():
         part = 32 * rng.randint(1, 16)
         contexts = [rng.choice([0, cap - 1, rng.randrange(cap), rng.randrange(cap)]) for _ in range(rows)]
         interleave, compact = rng.random() < 0.5, rng.random() < 0.5
+        rotate = 0 if interleave else (0, 1, 1, 3, 31)[case % 5]
         print(f"[case] drawn wave {case}: contexts {contexts} cap {cap} part {part} "
-              f"interleave {interleave} compact {compact}", flush=True)
+              f"interleave {interleave} compact {compact} rotate {rotate}", flush=True)
         _lane_batch(contexts, cap, part, 0xD1CE00 + case, replays=case % 2, interleave=interleave,
-                    compact=compact)
+                    compact=compact, rotate=rotate)
 
 
 def test_lane_batch_with_scores_in_the_hundreds():
@@ -651,6 +655,25 @@ def test_headline_shape_four_lanes_32768_split_1024_graph_replay():
     compiled walk."""
     print("[case] headline shape: 4 x 32768, split 1024, graph replay", flush=True)
     _lane_batch([32767] * 4, 32768, 1024, 0xBE7C, replays=3)
+
+
+@pytest.mark.parametrize("cap", [33024, 131136])
+def test_rotated_walk_at_capacities_that_alias(cap):
+    """The benchmark's lanes in caches whose capacity used to put the ranges of the 256
+    workgroups on the same memory channels: the host walks such ranges from a rotated starting
+    block (and, the grid being larger than the chip, with the workgroups that hold keys
+    first).  Same bar as every other order, eager and replayed."""
+    print(f"[case] 4 x 32768 in capacity {cap}, rotated ranges, keyed first", flush=True)
+    _lane_batch([32767] * 4, cap, 1024, 0xA11A5 + cap, replays=2, compact=True, rotate=1)
+
+
+def test_rotated_ranges_with_partial_and_single_blocks():
+    """Rotation where it has little room: ranges of one block (nothing to rotate), a last range
+    with a partial block, a last range of a single partial block, contexts of 0 and 31."""
+    print("[case] rotated ranges, partial and single blocks", flush=True)
+    _lane_batch([2000, 1499, 700, 100, 255, 256, 0, 31, 32, 319], 2048, 32, 0x2071, rotate=1)
+    _lane_batch([5000, 4999, 31, 1024, 1025], 5120, 1024, 0x2072, replays=1, rotate=1)
+    _lane_batch([5000, 4127, 4128, 63], 5120, 96, 0x2073, compact=True, rotate=7)
 
 
 def test_lane_batch_record_counts_straddle_32():
