@@ -11,6 +11,9 @@
 //       same row norm over the rounded sums, both written
 //   dense_bf16, add_bf16   no reference counterpart: the reference projects with
 //       4-bit weights (q4_dot.metal); here the weights are plain bf16.
+#include <algorithm>
+#include <type_traits>
+
 #include "../tt_internal.h"
 #include "lane_sums.h"
 #include "rms_row.h"
@@ -123,6 +126,238 @@ __global__ __launch_bounds__(256) void dense_bf16_kernel(const uint16_t* input,
             const uint32_t n = n0 + g * 4 + i;
             if (n < out_dim) output[static_cast<uint64_t>(row) * out_dim + n] = store16(acc0[i] + acc1[i]);
         }
+    }
+}
+
+// The same for a block of rows, sized for the matrix unit.  A workgroup of eight waves owns
+// 256 rows x 256 outputs (128 flop per operand byte it fetches: what reaches the compute
+// units from the L2 is what bounds a bf16 product of this size) and walks K in steps of
+// 32 columns:
+//   * both operands go from global memory straight into LDS (16 bytes per lane and
+//     transfer, no registers), five stages of 32 KiB, four steps ahead, one barrier per
+//     step; the fragments of a step are read into registers while the step before it is
+//     multiplied.  The transfers are issued as assembly, so that the only waits are the ones
+//     written below (M0 is used for nothing else in this kernel).  A stage row is one
+//     row's 64 bytes of the step; 16-byte piece p of row r sits in slot p ^ ((r >> 1) & 3),
+//     with which the 16-byte fragment reads of a wave (sixteen consecutive rows, one piece
+//     per quarter wave) were measured free of bank conflicts (p ^ ((r >> 2) & 3), p ^ (r & 3)
+//     and the plain order all cost a second pass).
+//   * wave (mh, nq) multiplies rows [128 mh, +128) with outputs [64 nq, +64) as 8 x 4 tiles
+//     of v_mfma_f32_16x16x32_bf16 (twelve fragment reads for 32 products), the weights as
+//     the left operand: a lane then holds four consecutive outputs of one row per tile and
+//     stores them as 8 bytes.
+// Rows and outputs past the end are clamped on the way in and not stored.
+constexpr uint32_t kDenseTileM = 256;
+constexpr uint32_t kDenseTileN = 256;
+constexpr uint32_t kDenseThreads = 512;
+constexpr uint32_t kDenseStages = 5;
+constexpr uint32_t kDenseStepColumns = 32;
+constexpr uint32_t kDenseRowBytes = kDenseStepColumns * 2;
+constexpr uint32_t kDenseXStageBytes = kDenseTileM * kDenseRowBytes;
+constexpr uint32_t kDenseStageBytes = (kDenseTileM + kDenseTileN) * kDenseRowBytes;
+constexpr uint32_t kDenseLdsBytes = kDenseStages * kDenseStageBytes;      // 163840
+static_assert(kDenseLdsBytes <= 160 * 1024, "one workgroup per compute unit");
+
+// lane l's 16 bytes at base + offset land at lds_address + 16 l
+__device__ __forceinline__ void dense_transfer(const uint8_t* base, uint32_t offset,
+                                               uint32_t lds_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_address)), "v"(offset), "s"(base)
+                 : "memory");
+}
+
+// two sums to a packed bf16 pair: hardware round to nearest even, then results below the
+// normal range flushed to signed zero
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+__device__ __forceinline__ uint32_t dense_pack(float a, float b) {
+    const uint32_t pair = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+    const uint32_t keep = ((pair & 0x00007F80u) ? 0x0000FFFFu : 0x00008000u) |
+                          ((pair & 0x7F800000u) ? 0xFFFF0000u : 0x80000000u);
+    return pair & keep;
+}
+
+__global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16_t* input,
+                                                                   const uint16_t* weights,
+                                                                   uint16_t* output, uint32_t rows,
+                                                                   uint32_t in_dim, uint32_t out_dim) {
+    extern __shared__ __align__(16) uint8_t dense_lds[];
+    const uint32_t t = threadIdx.x;
+    const uint32_t lane = t & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t i16 = lane & 15, g = lane >> 4;
+    const uint32_t steps = in_dim / kDenseStepColumns;
+    const uint32_t n_tiles = (out_dim + kDenseTileN - 1) / kDenseTileN;
+    const uint32_t tiles = n_tiles * ((rows + kDenseTileM - 1) / kDenseTileM);
+    const uint32_t lds_base = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)dense_lds));
+    const uint32_t nq = wave & 3, mh = wave >> 2;
+
+    // staging roles: transfers 0, 1 of wave w fill x rows 32 w + 16 j .. + 15, transfers 2, 3
+    // the weight rows of the same numbers; lane l lands in row + (l >> 2), slot l & 3, so it
+    // fetches piece (l & 3) ^ ((l >> 3) & 3) of that row
+    const uint8_t* x_base = reinterpret_cast<const uint8_t*>(input);
+    const uint8_t* w_base = reinterpret_cast<const uint8_t*>(weights);
+    const uint32_t piece = ((lane & 3) ^ ((lane >> 3) & 3)) * 16;
+    uint32_t x_offset[2], w_offset[2];
+    auto aim = [&](uint32_t tile) {
+        const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
+#pragma unroll
+        for (uint32_t j = 0; j < 2; ++j) {
+            const uint32_t in_tile = 32 * wave + 16 * j + (lane >> 2);
+            x_offset[j] = min(m0 + in_tile, rows - 1) * in_dim * 2 + piece;
+            w_offset[j] = min(n0 + in_tile, out_dim - 1) * in_dim * 2 + piece;
+        }
+    };
+    auto request = [&](uint32_t step) {
+        const uint32_t stage = lds_base + (step % kDenseStages) * kDenseStageBytes;
+        const uint8_t* x_step = x_base + step * kDenseRowBytes;   // uniform: scalar arithmetic
+        const uint8_t* w_step = w_base + step * kDenseRowBytes;
+#pragma unroll
+        for (uint32_t j = 0; j < 2; ++j) {
+            dense_transfer(x_step, x_offset[j], stage + (32 * wave + 16 * j) * kDenseRowBytes);
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 2; ++j) {
+            dense_transfer(w_step, w_offset[j],
+                           stage + kDenseXStageBytes + (32 * wave + 16 * j) * kDenseRowBytes);
+        }
+    };
+    // in_dim is a multiple of 64: an even number of steps, at least two
+    auto request_first_steps = [&]() {
+        request(0);
+        request(1);
+        if (steps > 2) {
+            request(2);
+            request(3);
+        }
+    };
+
+    // fragment of a row: piece g, stored at slot g ^ ((row >> 1) & 3)
+    const uint32_t frag = i16 * kDenseRowBytes + ((g ^ ((i16 >> 1) & 3)) * 16);
+    const uint32_t x_frag = 128 * mh * kDenseRowBytes + frag;
+    const uint32_t w_frag = kDenseXStageBytes + 64 * nq * kDenseRowBytes + frag;
+    f32x4 acc[4][8];   // [tn][tm]
+
+    struct Fragments {
+        bf16x8 x[8], w[4];
+    };
+    auto read_fragments = [&](uint32_t step, Fragments& f) __attribute__((always_inline)) {
+        const uint8_t* stage = dense_lds + (step % kDenseStages) * kDenseStageBytes;
+#pragma unroll
+        for (uint32_t tile = 0; tile < 4; ++tile) {
+            f.w[tile] = *reinterpret_cast<const bf16x8*>(stage + w_frag + tile * 16 * kDenseRowBytes);
+        }
+#pragma unroll
+        for (uint32_t tile = 0; tile < 8; ++tile) {
+            f.x[tile] = *reinterpret_cast<const bf16x8*>(stage + x_frag + tile * 16 * kDenseRowBytes);
+        }
+    };
+    auto multiply = [&](const Fragments& f) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t tm = 0; tm < 8; ++tm) {
+#pragma unroll
+            for (uint32_t tn = 0; tn < 4; ++tn) {
+                acc[tn][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.w[tn], f.x[tm], acc[tn][tm],
+                                                                      0, 0, 0);
+            }
+        }
+    };
+    // One slot of the walk: the fragments of `step` are in registers (read a slot ago);
+    // wait for the operands of step + 1 (kAhead later steps of four transfers each may stay
+    // in flight), request step + 4 into the stage whose fragments were multiplied a slot
+    // ago, read the fragments of step + 1 and multiply those of `step` while they arrive.
+    // No branch between the reads and the products: at a join the compiler would wait for
+    // the reads first.
+    auto slot = [&](uint32_t step, const Fragments& now, Fragments& next, auto ahead,
+                    auto with_request) __attribute__((always_inline)) {
+        constexpr uint32_t kAhead = decltype(ahead)::value;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (4 * kAhead));   // vmcnt(4 kAhead): mine have landed
+        __syncthreads();                                     // ... and everybody's
+        if constexpr (decltype(with_request)::value) request(step + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        read_fragments(step + 1, next);
+        multiply(now);
+        // issue order: a read, then two products, so that the eight waves' reads are spread
+        // over the slot instead of queueing at the LDS right after the barrier while the
+        // matrix unit waits (left alone the scheduler sinks each read to the product that
+        // needs it, a slot later)
+#pragma unroll
+        for (uint32_t i = 0; i < 12; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    using std::bool_constant;
+
+    // A workgroup takes every gridDim.x-th tile (outputs fastest); the first steps of its
+    // next tile are requested before it converts and stores the sums of this one.
+    uint32_t tile = blockIdx.x;
+    if (tile >= tiles) return;
+    aim(tile);
+    request_first_steps();
+    while (true) {
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+#pragma unroll
+            for (uint32_t tm = 0; tm < 8; ++tm) acc[tn][tm] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        // the first steps have landed (and the stores of the tile before are on their way:
+        // reads and writes do not retire in one order, so the count must reach zero)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        Fragments even, odd;
+        read_fragments(0, even);
+        uint32_t step = 0;
+        if (steps > 2) {
+            // steps 1, 2, 3 have landed too: the first three slots wait for nothing
+            for (; step + 4 < steps; step += 2) {
+                slot(step, even, odd, integral_constant<uint32_t, 2>{}, bool_constant<true>{});
+                slot(step + 1, odd, even, integral_constant<uint32_t, 2>{}, bool_constant<true>{});
+            }
+            // step == steps - 4
+            slot(step, even, odd, integral_constant<uint32_t, 2>{}, bool_constant<false>{});
+            slot(step + 1, odd, even, integral_constant<uint32_t, 1>{}, bool_constant<false>{});
+            step += 2;
+        }
+        slot(step, even, odd, integral_constant<uint32_t, 0>{}, bool_constant<false>{});
+        multiply(odd);
+
+        const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
+        const uint32_t next_tile = tile + gridDim.x;
+        __syncthreads();   // nobody reads the stages any more
+        if (next_tile < tiles) {
+            aim(next_tile);
+            request_first_steps();
+        }
+        // the lane holds outputs n0 + 64 nq + 16 tn + 4 g + j of row m0 + 128 mh + 16 tm + i16
+        const bool wide = ((reinterpret_cast<uintptr_t>(output) | (out_dim * 2)) & 7) == 0;
+#pragma unroll
+        for (uint32_t tm = 0; tm < 8; ++tm) {
+            const uint32_t row = m0 + 128 * mh + 16 * tm + i16;
+            if (row >= rows) continue;
+            uint16_t* out_row = output + static_cast<uint64_t>(row) * out_dim;
+#pragma unroll
+            for (uint32_t tn = 0; tn < 4; ++tn) {
+                const uint32_t n = n0 + 64 * nq + 16 * tn + 4 * g;
+                if (n >= out_dim) continue;
+                const f32x4 v = acc[tn][tm];
+                const u32x2 four = u32x2{dense_pack(v[0], v[1]), dense_pack(v[2], v[3])};
+                if (wide && n + 4 <= out_dim) {
+                    *reinterpret_cast<u32x2*>(out_row + n) = four;
+                } else {
+                    for (uint32_t j = 0; j < 4 && n + j < out_dim; ++j) {
+                        out_row[n + j] = static_cast<uint16_t>(four[j >> 1] >> (16 * (j & 1)));
+                    }
+                }
+            }
+        }
+        if (next_tile >= tiles) break;
+        tile = next_tile;
     }
 }
 
@@ -262,6 +497,27 @@ int32_t op_rms_only_ms(const Bindings& b, const Grid& g, hipStream_t stream, boo
     return launch_rms(b, g, stream, validate_only, true);
 }
 
+// Compute units of the current device (one workgroup of the block kernel each); recorded
+// when a library is created on the device.
+uint32_t g_compute_units[64] = {};
+uint32_t current_device_compute_units() {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    return g_compute_units[device] != 0 ? g_compute_units[device] : 256;
+}
+
+// Blocks of more rows than this take the LDS-staged kernel (below it a 256-row tile is
+// mostly padding).
+constexpr uint32_t kDenseBlockRowsFrom = 64;
+// What the block kernel assumes beyond the sizes: 16-byte pieces of both operands and
+// 32-bit byte offsets into them.
+bool dense_block_operands_fit(const uint16_t* input, const uint16_t* weights, uint32_t rows,
+                              uint32_t in_dim, uint32_t out_dim) {
+    return ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(weights)) & 15) == 0 &&
+           static_cast<uint64_t>(rows) * in_dim * 2 < (1ull << 32) &&
+           static_cast<uint64_t>(out_dim) * in_dim * 2 < (1ull << 32);
+}
+
 // dense_bf16: b0 input [rows][in], b1 weights [out][in], b2 output [rows][out], c3 rows,
 // c4 in (multiple of 64), c5 out; grid (ceil(out/64), ceil(rows/16)) x 256.
 int32_t op_dense_bf16(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only) {
@@ -285,6 +541,12 @@ int32_t op_dense_bf16(const Bindings& b, const Grid& g, hipStream_t stream, bool
     } else if (rows <= 16 && in_dim == 4096) {
         hipLaunchKernelGGL(dense_rows_kernel<8>, dim3((out_dim + 15) / 16), dim3(512), 0, stream, input,
                            weights, output, rows, out_dim);
+    } else if (rows > kDenseBlockRowsFrom && dense_block_operands_fit(input, weights, rows, in_dim, out_dim)) {
+        const uint32_t tiles = ((out_dim + kDenseTileN - 1) / kDenseTileN) *
+                               ((rows + kDenseTileM - 1) / kDenseTileM);
+        hipLaunchKernelGGL(dense_block_kernel, dim3(std::min(tiles, current_device_compute_units())),
+                           dim3(kDenseThreads), kDenseLdsBytes, stream, input, weights, output, rows,
+                           in_dim, out_dim);
     } else {
         hipLaunchKernelGGL(dense_bf16_kernel, dim3((out_dim + 63) / 64, (rows + 15) / 16), dim3(256), 0,
                            stream, input, weights, output, rows, in_dim, out_dim);
@@ -321,6 +583,17 @@ const KernelDesc kStackStepKernels[] = {
     {"add_bf16", op_add_bf16},
 };
 const uint32_t kStackStepKernelCount = sizeof(kStackStepKernels) / sizeof(kStackStepKernels[0]);
+bool prepare_stack_kernels() {
+    int device = 0, units = 0;
+    if (hipGetDevice(&device) == hipSuccess && device >= 0 && device < 64 &&
+        hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess &&
+        units > 0) {
+        g_compute_units[device] = static_cast<uint32_t>(units);
+    }
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(dense_block_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kDenseLdsBytes) == hipSuccess;
+}
 #endif
 
 }  // namespace tt

@@ -511,7 +511,7 @@ int32_t tt_library_create(tt_device* device, tt_library** out) {
     if (library == nullptr) return TT_PIPE_LIBRARY_COMPILATION_FAILED;
     library->device = device;
     if (!tt::prepare_decode_kernels() || !tt::prepare_prefill_kernels() ||
-        !tt::prepare_q4_kernels()) {
+        !tt::prepare_q4_kernels() || !tt::prepare_stack_kernels()) {
         delete library;
         return TT_PIPE_LIBRARY_COMPILATION_FAILED;
     }

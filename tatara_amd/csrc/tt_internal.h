@@ -98,6 +98,7 @@ uint32_t queue_compute_units(const tt_queue* queue);
 bool prepare_decode_kernels();
 bool prepare_prefill_kernels();
 bool prepare_q4_kernels();
+bool prepare_stack_kernels();
 
 extern const KernelDesc kAttentionDecodeKernels[];
 extern const uint32_t kAttentionDecodeKernelCount;

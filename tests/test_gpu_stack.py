@@ -301,6 +301,55 @@ def test_dense_bf16_operator(rows, in_dim, out_dim):
     assert np.mean(got == want) > 0.97
 
 
+def _dense_block_case(rows, in_dim, out_dim, sample_rows, seed):
+    """dense_bf16 on a block of rows; the checker evaluates `sample_rows` of them."""
+    B, dev, queue, lib = gpu()
+    x = ol.gaussian_bf16(seed, rows * in_dim).reshape(rows, in_dim)
+    w = ol.gaussian_bf16(seed + 1, out_dim * in_dim, 0.0, 1.0 / np.sqrt(in_dim))
+    b_x, b_w = dev.buffer_from(x), dev.buffer_from(w)
+    b_o = dev.create_buffer(rows * out_dim * 2)
+    b_o.write(np.full(rows * out_dim, 0x7FC0, np.uint16))       # NaN wherever nothing is stored
+    run(lambda cb: cb.encode(lib.pipeline("dense_bf16"), {0: b_x, 1: b_w, 2: b_o},
+                             {3: rows, 4: in_dim, 5: out_dim},
+                             ((out_dim + 63) // 64, (rows + 15) // 16), (256,)))
+    got = b_o.read(np.uint16).reshape(rows, out_dim)
+    sample = np.asarray(sorted(set(sample_rows)))
+    want = np.zeros(sample.size * out_dim, np.uint16)
+    o.tto_dense_bf16(np.ascontiguousarray(x[sample]).reshape(-1), w, sample.size, in_dim, out_dim,
+                     want, THREADS)
+    from gpu_util import check_bf16
+    check_bf16(got[sample].reshape(-1), want, f"dense_bf16 block {rows}x{in_dim}x{out_dim}", ulps=1)
+    assert np.mean(got[sample].reshape(-1) == want) > 0.97
+    return got
+
+
+@pytest.mark.parametrize("rows,in_dim,out_dim", [
+    (65, 64, 70),          # the smallest block: two steps, one tile mostly padding, narrow stores
+    (257, 2048, 300),      # one row and 44 outputs into a second tile either way
+    (300, 4096, 2048),     # the output projection's shape
+    (1000, 2048, 515),     # an odd output width: rows are not 8-byte aligned
+    (513, 128, 256),       # four steps: the walk's lead-in and lead-out only
+    (640, 192, 1024),      # six steps: one round of the steady loop
+], ids=["65x64x70", "257x2048x300", "300x4096x2048", "1000x2048x515", "513x128x256", "640x192x1024"])
+def test_dense_bf16_block_kernel(rows, in_dim, out_dim):
+    """Blocks of more than 64 rows take the LDS-staged 256 x 256 kernel: every row against the
+    checker, partial tiles either way, every length of the K walk's lead-in and lead-out."""
+    print(f"[case] dense_bf16 block rows={rows} in={in_dim} out={out_dim}", flush=True)
+    _dense_block_case(rows, in_dim, out_dim, range(rows), 0xB10C + rows)
+
+
+def test_dense_bf16_block_kernel_at_the_prefill_shape():
+    """16384 rows x 2048 -> 9216 (the attention input projection of a 16384-row block): 2304
+    tiles on one workgroup per compute unit, nine tiles each.  The checker evaluates every
+    251st row (66 rows, each at another position inside its tile) and the last rows."""
+    rows, in_dim, out_dim = 16384, 2048, 9216
+    print(f"[case] dense_bf16 block rows={rows} in={in_dim} out={out_dim}, sampled rows", flush=True)
+    sample = list(range(0, rows, 251)) + [rows - 2, rows - 1]
+    assert len({r % 256 for r in range(0, rows, 251)}) > 60
+    got = _dense_block_case(rows, in_dim, out_dim, sample, 0xB16B)
+    assert not np.any((got & 0x7F80) == 0x7F80), "an output was not stored"
+
+
 def test_add_bf16_operator_bit_for_bit():
     print("[case] add_bf16", flush=True)
     B, dev, queue, lib = gpu()
