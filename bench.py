@@ -52,6 +52,7 @@ CAPACITY = 32768
 LAYERS = 40
 PERIOD = 4                      # G,G,G,A
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0   # dense bf16
 CALIBRATION_COPY_BYTES = 256 << 20
 # HBM traffic of one launch of the key-walk kernel at 4 lanes x 32768 keys, from two rocprofv3
 # counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
@@ -341,6 +342,31 @@ CONFIG5_DECODE_CONTEXTS = (1024, 4096, 16384, 32768, 65536, 100000)
 CONFIG5_PREFILL_TOKENS = (4096, 32768)
 CONFIG5_LANES = (1, 4)
 CONFIG5_BLOCK_ROWS = 2048
+
+
+def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=5):
+    """dense_bf16 (the stub stack's stand-in for the projections) on a block of rows at the
+    three projection shapes of the family: device time per dispatch and MFMA rate."""
+    out = []
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0xDE75E)
+    for in_dim, out_dim in ((2048, 9216), (2048, 12352), (4096, 2048)):
+        x = torch.randn(rows * in_dim, generator=gen, device="cuda").to(torch.bfloat16)
+        w = (torch.randn(out_dim * in_dim, generator=gen, device="cuda") * in_dim ** -0.5).to(torch.bfloat16)
+        y = torch.empty(rows * out_dim, device="cuda", dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        b_x, b_w, b_y = (dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t) for t in (x, w, y))
+        figures = time_graph(queue, lambda cb: cb.encode(
+            lib.pipeline("dense_bf16"), {0: b_x, 1: b_w, 2: b_y}, {3: rows, 4: in_dim, 5: out_dim},
+            ((out_dim + 63) // 64, (rows + 15) // 16), (256,)), 1, replays=repeats, warm=2)
+        flops = 2.0 * rows * in_dim * out_dim
+        tflops = flops / (figures["median_us"] * 1e-6) / 1e12
+        out.append({"operator": "dense_bf16", "rows": rows, "in": in_dim, "out": out_dim,
+                    "us": figures["median_us"], "tflops": round(tflops, 1),
+                    "frac_of_bf16_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4)})
+        del x, w, y
+        torch.cuda.empty_cache()
+    return out
 
 
 def config5_decode_point(dev, queue, lib, torch, attention, lanes, visible):
@@ -730,6 +756,7 @@ def main():
         line["detail"]["prefill_16k"] = prefill_figures(B, dev, queue, lib, torch)
         if not args.no_cpu_baseline:
             line["detail"]["prefill_16k"]["cpu_baseline"] = cpu_prefill_baseline(threads)
+        line["detail"]["dense_bf16_block"] = dense_block_figures(dev, queue, lib, torch)
         from tatara_amd import q4_sweep
         line["detail"]["q4_projections"] = (
             [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)

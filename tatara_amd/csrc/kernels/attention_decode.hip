@@ -21,7 +21,7 @@
 // softmax state for the 8 query heads of the kv group:
 //   S^T[key][head] = K[key][:] . Q[head][:]   v_mfma_f32_16x16x32_bf16,
 //       A = K tile read from a per-wave LDS stage that HBM fills directly
-//       (global_load_lds, no registers; row pairs padded to 1040 B so the
+//       (global_load_lds, no registers; row pairs padded to 1056 B so the
 //       16-lane operand reads spread over the banks), B = Q^T in registers.
 //       MFMA columns 8..15 repeat heads 0..7.
 //   O^T[dim][head] += V^T[dim][key] P^T[key][head]
@@ -55,8 +55,8 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr uint32_t kD = kAttnHeadDim;
 constexpr uint32_t kBlockKeys = 32;         // keys per wave iteration
-constexpr uint32_t kLdsPairBytes = 1040;    // key i row | key 16+i row | 16 B pad
-constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16640
+constexpr uint32_t kLdsPairBytes = 1056;    // key i row | key 16+i row | 32 B pad
+constexpr uint32_t kWaveLdsBytes = 16 * kLdsPairBytes;  // 16896
 constexpr uint32_t kWaves = 4;
 constexpr uint32_t kHeadsPerWave = kAttnHeadsPerKv / kWaves;   // heads a wave norms and finishes
 // Cache policy of the K transfers and V loads: every key and value byte is used once per

@@ -34,8 +34,8 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr uint32_t kD = kAttnHeadDim;
 constexpr uint32_t kTileKeys = 32;
-constexpr uint32_t kKeyPairBytes = 1040;                 // key i | key 16+i | 16 B pad
-constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16640
+constexpr uint32_t kKeyPairBytes = 1056;                 // key i | key 16+i | 32 B pad
+constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16896
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kReferenceSlack = 100.0f;  // log2 units a score may exceed the fixed reference by
 
@@ -86,10 +86,10 @@ struct FlashPrefillArgs {
 // SIMD (256 registers each): one wave's softmax (VALU) runs under the other's
 // products (MFMA), and LDS operand reads are issued from eight waves.
 //   K and V tiles: HBM/L2 -> LDS rings of 3 stages, two tiles ahead (global_load_lds).
-//   Both are stored as 16 row pairs (row i | row 16+i | pad): K pairs of 1040 bytes so
-//   the 16-byte S^T operand reads are conflict-free, V pairs of 1056 bytes so that the
-//   eight rows one half-wave touches in a transposing read fall into eight different
-//   32-byte bank groups.
+//   Both are stored as 16 row pairs (row i | row 16+i | 32 B pad): with pairs of 1056 bytes
+//   both the 16-byte S^T operand reads (sixteen pairs, one piece per quarter wave) and the
+//   transposing V reads were measured free of bank conflicts (pairs of 1040 bytes cost the
+//   16-byte reads a second pass, pairs of 1024 seven).
 //   V^T operands come straight from the row-major V stage with ds_read_b64_tr_b16:
 //   16 lanes hand in the addresses of 4 key rows x 16 dims (4 lanes per row, 4 dims
 //   each) and lane i receives dim i of the 4 rows - two such reads are the 8 contraction
@@ -102,10 +102,10 @@ struct FlashPrefillArgs {
 constexpr uint32_t kFlashWaves = 8;
 constexpr uint32_t kTilePositions = 32;
 constexpr uint32_t kRing = 3;
-constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 49920
+constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 50688
 constexpr uint32_t kValuePairBytes = 1056;                             // row i | row 16+i | 32 B pad
 constexpr uint32_t kValuePairedStageBytes = 16 * kValuePairBytes;      // 16896
-constexpr uint32_t kFlashLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 100608
+constexpr uint32_t kFlashLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 101376
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 

@@ -129,33 +129,33 @@ __global__ __launch_bounds__(256) void dense_bf16_kernel(const uint16_t* input,
     }
 }
 
-// The same for a block of rows, sized for the matrix unit.  A workgroup of eight waves owns
-// 256 rows x 256 outputs (128 flop per operand byte it fetches: what reaches the compute
-// units from the L2 is what bounds a bf16 product of this size) and walks K in steps of
-// 32 columns:
+// The same for a block of rows, sized for the matrix unit.  One persistent workgroup of
+// eight waves per compute unit; a workgroup owns tiles of 256 rows x 256 outputs (128 flop
+// per operand byte it fetches) and walks K in units of 64 columns, two steps of 32 each:
 //   * both operands go from global memory straight into LDS (16 bytes per lane and
-//     transfer, no registers), five stages of 32 KiB, four steps ahead, one barrier per
-//     step; the fragments of a step are read into registers while the step before it is
-//     multiplied.  The transfers are issued as assembly, so that the only waits are the ones
-//     written below (M0 is used for nothing else in this kernel).  A stage row is one
-//     row's 64 bytes of the step; 16-byte piece p of row r sits in slot p ^ ((r >> 1) & 3),
-//     with which the 16-byte fragment reads of a wave (sixteen consecutive rows, one piece
-//     per quarter wave) were measured free of bank conflicts (p ^ ((r >> 2) & 3), p ^ (r & 3)
-//     and the plain order all cost a second pass).
+//     transfer, whole 128-byte lines of a row, no registers), a ring of two units of
+//     64 KiB.  The transfers are issued as assembly, so that the only waits are the ones
+//     written below (M0 is used for nothing else in this kernel).  A ring row is one
+//     row's 128 bytes of the unit; 16-byte piece p of row r sits in slot p ^ (r & 7), with
+//     which the 16-byte fragment reads of a wave (sixteen consecutive rows, one piece per
+//     quarter wave) were measured free of bank conflicts.
 //   * wave (mh, nq) multiplies rows [128 mh, +128) with outputs [64 nq, +64) as 8 x 4 tiles
 //     of v_mfma_f32_16x16x32_bf16 (twelve fragment reads for 32 products), the weights as
 //     the left operand: a lane then holds four consecutive outputs of one row per tile and
-//     stores them as 8 bytes.
+//     stores them as 8 bytes.  The fragments of a step are read into registers while the
+//     step before it is multiplied; one barrier per unit.
+//   * the first two units of a workgroup's next tile are requested before it converts and
+//     stores the sums of this one.
 // Rows and outputs past the end are clamped on the way in and not stored.
 constexpr uint32_t kDenseTileM = 256;
 constexpr uint32_t kDenseTileN = 256;
 constexpr uint32_t kDenseThreads = 512;
-constexpr uint32_t kDenseStages = 5;
-constexpr uint32_t kDenseStepColumns = 32;
-constexpr uint32_t kDenseRowBytes = kDenseStepColumns * 2;
-constexpr uint32_t kDenseXStageBytes = kDenseTileM * kDenseRowBytes;
-constexpr uint32_t kDenseStageBytes = (kDenseTileM + kDenseTileN) * kDenseRowBytes;
-constexpr uint32_t kDenseLdsBytes = kDenseStages * kDenseStageBytes;      // 163840
+constexpr uint32_t kDenseRing = 2;
+constexpr uint32_t kDenseUnitColumns = 64;
+constexpr uint32_t kDenseRowBytes = kDenseUnitColumns * 2;
+constexpr uint32_t kDenseXUnitBytes = kDenseTileM * kDenseRowBytes;
+constexpr uint32_t kDenseUnitBytes = (kDenseTileM + kDenseTileN) * kDenseRowBytes;
+constexpr uint32_t kDenseLdsBytes = kDenseRing * kDenseUnitBytes;      // 131072
 static_assert(kDenseLdsBytes <= 160 * 1024, "one workgroup per compute unit");
 
 // lane l's 16 bytes at base + offset land at lds_address + 16 l
@@ -187,71 +187,63 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
     const uint32_t lane = t & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t i16 = lane & 15, g = lane >> 4;
-    const uint32_t steps = in_dim / kDenseStepColumns;
+    const uint32_t units = in_dim / kDenseUnitColumns;
     const uint32_t n_tiles = (out_dim + kDenseTileN - 1) / kDenseTileN;
     const uint32_t tiles = n_tiles * ((rows + kDenseTileM - 1) / kDenseTileM);
     const uint32_t lds_base = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)dense_lds));
     const uint32_t nq = wave & 3, mh = wave >> 2;
 
-    // staging roles: transfers 0, 1 of wave w fill x rows 32 w + 16 j .. + 15, transfers 2, 3
-    // the weight rows of the same numbers; lane l lands in row + (l >> 2), slot l & 3, so it
-    // fetches piece (l & 3) ^ ((l >> 3) & 3) of that row
+    // staging roles: transfers 0..3 of wave w fill x rows 32 w + 8 j .. + 7, transfers 4..7
+    // the weight rows of the same numbers; lane l lands in row + (l >> 3), slot l & 7, so it
+    // fetches piece (l & 7) ^ (l >> 3) of that row
     const uint8_t* x_base = reinterpret_cast<const uint8_t*>(input);
     const uint8_t* w_base = reinterpret_cast<const uint8_t*>(weights);
-    const uint32_t piece = ((lane & 3) ^ ((lane >> 3) & 3)) * 16;
-    uint32_t x_offset[2], w_offset[2];
+    const uint32_t piece = ((lane & 7) ^ (lane >> 3)) * 16;
+    uint32_t x_offset[4], w_offset[4];
     auto aim = [&](uint32_t tile) {
         const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
 #pragma unroll
-        for (uint32_t j = 0; j < 2; ++j) {
-            const uint32_t in_tile = 32 * wave + 16 * j + (lane >> 2);
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t in_tile = 32 * wave + 8 * j + (lane >> 3);
             x_offset[j] = min(m0 + in_tile, rows - 1) * in_dim * 2 + piece;
             w_offset[j] = min(n0 + in_tile, out_dim - 1) * in_dim * 2 + piece;
         }
     };
-    auto request = [&](uint32_t step) {
-        const uint32_t stage = lds_base + (step % kDenseStages) * kDenseStageBytes;
-        const uint8_t* x_step = x_base + step * kDenseRowBytes;   // uniform: scalar arithmetic
-        const uint8_t* w_step = w_base + step * kDenseRowBytes;
+    auto request = [&](uint32_t unit) {
+        const uint32_t place = lds_base + (unit % kDenseRing) * kDenseUnitBytes;
+        const uint8_t* x_unit = x_base + unit * kDenseRowBytes;   // uniform: scalar arithmetic
+        const uint8_t* w_unit = w_base + unit * kDenseRowBytes;
 #pragma unroll
-        for (uint32_t j = 0; j < 2; ++j) {
-            dense_transfer(x_step, x_offset[j], stage + (32 * wave + 16 * j) * kDenseRowBytes);
+        for (uint32_t j = 0; j < 4; ++j) {
+            dense_transfer(x_unit, x_offset[j], place + (32 * wave + 8 * j) * kDenseRowBytes);
         }
 #pragma unroll
-        for (uint32_t j = 0; j < 2; ++j) {
-            dense_transfer(w_step, w_offset[j],
-                           stage + kDenseXStageBytes + (32 * wave + 16 * j) * kDenseRowBytes);
-        }
-    };
-    // in_dim is a multiple of 64: an even number of steps, at least two
-    auto request_first_steps = [&]() {
-        request(0);
-        request(1);
-        if (steps > 2) {
-            request(2);
-            request(3);
+        for (uint32_t j = 0; j < 4; ++j) {
+            dense_transfer(w_unit, w_offset[j],
+                           place + kDenseXUnitBytes + (32 * wave + 8 * j) * kDenseRowBytes);
         }
     };
 
-    // fragment of a row: piece g, stored at slot g ^ ((row >> 1) & 3)
-    const uint32_t frag = i16 * kDenseRowBytes + ((g ^ ((i16 >> 1) & 3)) * 16);
-    const uint32_t x_frag = 128 * mh * kDenseRowBytes + frag;
-    const uint32_t w_frag = kDenseXStageBytes + 64 * nq * kDenseRowBytes + frag;
+    // fragment of (row, step of the unit): piece 4 step + g, stored at slot piece ^ (row & 7)
+    const uint32_t frag_row = i16 * kDenseRowBytes;
+    const uint32_t frag_piece[2] = {(g ^ (i16 & 7)) * 16, ((4 + g) ^ (i16 & 7)) * 16};
+    const uint32_t x_frag = 128 * mh * kDenseRowBytes + frag_row;
+    const uint32_t w_frag = kDenseXUnitBytes + 64 * nq * kDenseRowBytes + frag_row;
     f32x4 acc[4][8];   // [tn][tm]
 
     struct Fragments {
         bf16x8 x[8], w[4];
     };
-    auto read_fragments = [&](uint32_t step, Fragments& f) __attribute__((always_inline)) {
-        const uint8_t* stage = dense_lds + (step % kDenseStages) * kDenseStageBytes;
+    auto read_fragments = [&](uint32_t unit, uint32_t step, Fragments& f) __attribute__((always_inline)) {
+        const uint8_t* place = dense_lds + (unit % kDenseRing) * kDenseUnitBytes + frag_piece[step];
 #pragma unroll
         for (uint32_t tile = 0; tile < 4; ++tile) {
-            f.w[tile] = *reinterpret_cast<const bf16x8*>(stage + w_frag + tile * 16 * kDenseRowBytes);
+            f.w[tile] = *reinterpret_cast<const bf16x8*>(place + w_frag + tile * 16 * kDenseRowBytes);
         }
 #pragma unroll
         for (uint32_t tile = 0; tile < 8; ++tile) {
-            f.x[tile] = *reinterpret_cast<const bf16x8*>(stage + x_frag + tile * 16 * kDenseRowBytes);
+            f.x[tile] = *reinterpret_cast<const bf16x8*>(place + x_frag + tile * 16 * kDenseRowBytes);
         }
     };
     auto multiply = [&](const Fragments& f) __attribute__((always_inline)) {
@@ -264,25 +256,12 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
             }
         }
     };
-    // One slot of the walk: the fragments of `step` are in registers (read a slot ago);
-    // wait for the operands of step + 1 (kAhead later steps of four transfers each may stay
-    // in flight), request step + 4 into the stage whose fragments were multiplied a slot
-    // ago, read the fragments of step + 1 and multiply those of `step` while they arrive.
-    // No branch between the reads and the products: at a join the compiler would wait for
-    // the reads first.
-    auto slot = [&](uint32_t step, const Fragments& now, Fragments& next, auto ahead,
-                    auto with_request) __attribute__((always_inline)) {
-        constexpr uint32_t kAhead = decltype(ahead)::value;
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (4 * kAhead));   // vmcnt(4 kAhead): mine have landed
-        __syncthreads();                                     // ... and everybody's
-        if constexpr (decltype(with_request)::value) request(step + 4);
-        __builtin_amdgcn_sched_barrier(0);
-        read_fragments(step + 1, next);
-        multiply(now);
-        // issue order: a read, then two products, so that the eight waves' reads are spread
-        // over the slot instead of queueing at the LDS right after the barrier while the
-        // matrix unit waits (left alone the scheduler sinks each read to the product that
-        // needs it, a slot later)
+    // issue order of a slot: a read, then two products, so that the eight waves' reads are
+    // spread over the slot instead of queueing at the LDS while the matrix unit waits (left
+    // alone the scheduler sinks each read to the product that needs it, a slot later).  No
+    // branch between the reads and the products: at a join the compiler would wait for the
+    // reads first.
+    auto interleave = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (uint32_t i = 0; i < 12; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -291,48 +270,68 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
         __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
-    using std::integral_constant;
+    // first step of `unit` (its fragments are in `first`): read the second step's while
+    // multiplying; the unit was published a slot ago, so nothing to wait for
+    auto first_step = [&](uint32_t unit, const Fragments& first, Fragments& second)
+                          __attribute__((always_inline)) {
+        __builtin_amdgcn_sched_barrier(0);
+        read_fragments(unit, 1, second);
+        multiply(first);
+        interleave();
+    };
+    // second step of `unit`: the next unit (requested a unit ago) has landed - mine, then
+    // everybody's -, and nobody reads the unit before this one any more, so the unit after
+    // the next goes into its place; read the next unit's first fragments while multiplying
+    auto second_step = [&](uint32_t unit, const Fragments& second, Fragments& first_of_next,
+                           auto with_request) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        __syncthreads();
+        if constexpr (decltype(with_request)::value) request(unit + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        read_fragments(unit + 1, 0, first_of_next);
+        multiply(second);
+        interleave();
+    };
     using std::bool_constant;
 
-    // A workgroup takes every gridDim.x-th tile (outputs fastest); the first steps of its
-    // next tile are requested before it converts and stores the sums of this one.
+    // A workgroup takes every gridDim.x-th tile (outputs fastest)
     uint32_t tile = blockIdx.x;
     if (tile >= tiles) return;
     aim(tile);
-    request_first_steps();
+    request(0);
+    if (units > 1) request(1);
     while (true) {
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
 #pragma unroll
             for (uint32_t tm = 0; tm < 8; ++tm) acc[tn][tm] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
-        // the first steps have landed (and the stores of the tile before are on their way:
-        // reads and writes do not retire in one order, so the count must reach zero)
+        // unit 0 has landed (the second unit may be in flight; so may the stores of the tile
+        // before, and reads and writes do not retire in one order: wait for everything)
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-        Fragments even, odd;
-        read_fragments(0, even);
-        uint32_t step = 0;
-        if (steps > 2) {
-            // steps 1, 2, 3 have landed too: the first three slots wait for nothing
-            for (; step + 4 < steps; step += 2) {
-                slot(step, even, odd, integral_constant<uint32_t, 2>{}, bool_constant<true>{});
-                slot(step + 1, odd, even, integral_constant<uint32_t, 2>{}, bool_constant<true>{});
-            }
-            // step == steps - 4
-            slot(step, even, odd, integral_constant<uint32_t, 2>{}, bool_constant<false>{});
-            slot(step + 1, odd, even, integral_constant<uint32_t, 1>{}, bool_constant<false>{});
-            step += 2;
+        Fragments a, b;
+        read_fragments(0, 0, a);
+        uint32_t unit = 0;
+        for (; unit + 2 < units; ++unit) {
+            first_step(unit, a, b);
+            second_step(unit, b, a, bool_constant<true>{});
         }
-        slot(step, even, odd, integral_constant<uint32_t, 0>{}, bool_constant<false>{});
-        multiply(odd);
+        if (units > 1) {   // unit == units - 2
+            first_step(unit, a, b);
+            second_step(unit, b, a, bool_constant<false>{});
+            ++unit;
+        }
+        first_step(unit, a, b);
+        multiply(b);
 
         const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
         const uint32_t next_tile = tile + gridDim.x;
         __syncthreads();   // nobody reads the stages any more
         if (next_tile < tiles) {
             aim(next_tile);
-            request_first_steps();
+            request(0);
+            if (units > 1) request(1);
         }
         // the lane holds outputs n0 + 64 nq + 16 tn + 4 g + j of row m0 + 128 mh + 16 tm + i16
         const bool wide = ((reinterpret_cast<uintptr_t>(output) | (out_dim * 2)) & 7) == 0;
