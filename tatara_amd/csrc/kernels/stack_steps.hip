@@ -200,27 +200,28 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
     const uint8_t* x_base = reinterpret_cast<const uint8_t*>(input);
     const uint8_t* w_base = reinterpret_cast<const uint8_t*>(weights);
     const uint32_t piece = ((lane & 7) ^ (lane >> 3)) * 16;
-    uint32_t x_offset[4], w_offset[4];
+    const uint32_t staged_row = 32 * wave + (lane >> 3);
+    const uint32_t row_bytes = in_dim * 2;
+    uint32_t m_aim = 0, n_aim = 0;   // first row and output of the tile the requests go to
     auto aim = [&](uint32_t tile) {
-        const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t in_tile = 32 * wave + 8 * j + (lane >> 3);
-            x_offset[j] = min(m0 + in_tile, rows - 1) * in_dim * 2 + piece;
-            w_offset[j] = min(n0 + in_tile, out_dim - 1) * in_dim * 2 + piece;
-        }
+        m_aim = (tile / n_tiles) * kDenseTileM;
+        n_aim = (tile % n_tiles) * kDenseTileN;
     };
+    // the lane offsets are worked out per request (a handful of instructions per 64
+    // products) rather than held in eight registers the products need
     auto request = [&](uint32_t unit) {
         const uint32_t place = lds_base + (unit % kDenseRing) * kDenseUnitBytes;
         const uint8_t* x_unit = x_base + unit * kDenseRowBytes;   // uniform: scalar arithmetic
         const uint8_t* w_unit = w_base + unit * kDenseRowBytes;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            dense_transfer(x_unit, x_offset[j], place + (32 * wave + 8 * j) * kDenseRowBytes);
+            const uint32_t offset = min(m_aim + staged_row + 8 * j, rows - 1) * row_bytes + piece;
+            dense_transfer(x_unit, offset, place + (32 * wave + 8 * j) * kDenseRowBytes);
         }
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            dense_transfer(w_unit, w_offset[j],
+            const uint32_t offset = min(n_aim + staged_row + 8 * j, out_dim - 1) * row_bytes + piece;
+            dense_transfer(w_unit, offset,
                            place + kDenseXUnitBytes + (32 * wave + 8 * j) * kDenseRowBytes);
         }
     };
