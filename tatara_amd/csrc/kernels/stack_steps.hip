@@ -203,10 +203,18 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
     const uint32_t staged_row = 32 * wave + (lane >> 3);
     const uint32_t row_bytes = in_dim * 2;
     uint32_t m_aim = 0, n_aim = 0;   // first row and output of the tile the requests go to
-    auto aim = [&](uint32_t tile) {
-        m_aim = (tile / n_tiles) * kDenseTileM;
-        n_aim = (tile % n_tiles) * kDenseTileN;
+    // Tiles are numbered along bands of eight tile rows, down a band's columns first, so that
+    // a run of consecutive numbers is a compact patch (32 of them: eight rows x four columns,
+    // twelve operand panels for 32 tiles).
+    const uint32_t m_tiles = (rows + kDenseTileM - 1) / kDenseTileM;
+    auto place = [&](uint32_t tile, uint32_t& m0, uint32_t& n0) {
+        const uint32_t band = tile / (8 * n_tiles);
+        const uint32_t band_rows = min(8u, m_tiles - 8 * band);
+        const uint32_t within = tile - band * 8 * n_tiles;
+        m0 = (8 * band + within % band_rows) * kDenseTileM;
+        n0 = (within / band_rows) * kDenseTileN;
     };
+    auto aim = [&](uint32_t tile) { place(tile, m_aim, n_aim); };
     // the lane offsets are worked out per request (a handful of instructions per 64
     // products) rather than held in eight registers the products need
     auto request = [&](uint32_t unit) {
@@ -295,8 +303,15 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
     };
     using std::bool_constant;
 
-    // A workgroup takes every gridDim.x-th tile (outputs fastest)
-    uint32_t tile = blockIdx.x;
+    // Workgroup b of the dispatch order runs on XCD b mod 8, each XCD with an L2 of its own:
+    // the workgroups of an XCD (b / 8 = 0, 1, ...) take a run of consecutive tiles together,
+    // the XCDs take the runs in turn - the operand panels a patch shares are then fetched into
+    // one L2 once instead of into several.  (A grid that is no multiple of eight - fewer tiles
+    // than compute units - takes every gridDim.x-th tile.)
+    const bool by_xcd = gridDim.x % 8 == 0;
+    const uint32_t per_xcd = gridDim.x / 8;
+    const uint32_t stride = by_xcd ? 8 * per_xcd : gridDim.x;
+    uint32_t tile = by_xcd ? (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
     if (tile >= tiles) return;
     aim(tile);
     request(0);
@@ -326,8 +341,9 @@ __global__ __launch_bounds__(kDenseThreads) void dense_block_kernel(const uint16
         first_step(unit, a, b);
         multiply(b);
 
-        const uint32_t m0 = (tile / n_tiles) * kDenseTileM, n0 = (tile % n_tiles) * kDenseTileN;
-        const uint32_t next_tile = tile + gridDim.x;
+        uint32_t m0, n0;
+        place(tile, m0, n0);
+        const uint32_t next_tile = tile + stride;
         __syncthreads();   // nobody reads the stages any more
         if (next_tile < tiles) {
             aim(next_tile);
