@@ -58,7 +58,7 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
 # counter read for a plain 256 MiB copy of known size; see the file named here.
 TRAFFIC_SOURCE = "profiles/flash_decode_4x32768_hbm_counters.md"
-TRAFFIC_BYTES = round((131289.6 * 262144.0 / 131083.3 + 2181.5) * 1024)   # 271,091,778
+TRAFFIC_BYTES = round((131289.6 * 262144.0 / 131083.3 + 2151.0) * 1024)   # 271,060,546
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 CONFIG3 = {
@@ -253,7 +253,7 @@ def attention_figures(queue, wave):
             "layer_frac": round(algo / (layer["median_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
-def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
+def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=16, warm=6):
     """Block prefill of `rows` new tokens into an empty cache, one lane, resident
     random inputs: the causal flash attention kernel (rope stage timed beside it) and
     the chunk-64 Gated DeltaNet recurrence (conv, gates and gate-norm beside it).
@@ -287,7 +287,9 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
     qk, v, z, y, gated = (mk(rows * 8192) for _ in range(5))
     decay, beta = mk(rows * 128), mk(rows * 128)
     chunk = mk(((min(rows, 2048) + 63) // 64) * 32 * 115712)
-    best = {}
+    # the first passes run at the clock the device idles at; the figures are medians of the
+    # passes after them (a block prefill is a long run of such passes)
+    times = {}
     for _ in range(repeats):
         cb = queue.create_command_buffer()
         cb.set_profiling(True)
@@ -310,7 +312,8 @@ def prefill_figures(B, dev, queue, lib, torch, rows=16384, repeats=3):
         cb.end_compute_pass()
         cb.commit().wait()
         for name, ms in cb.command_times():
-            best[name] = min(best.get(name, ms), ms)
+            times.setdefault(name, []).append(ms)
+    best = {name: statistics.median(ms[warm:]) for name, ms in times.items()}
     flash_ms = best["attention_flash_v2_blk"]
     flops = 16 * 4 * 256 * rows * (rows + 1) / 2
     attn_ms = flash_ms + best["attn_qk_rope_blk"]
@@ -344,7 +347,7 @@ CONFIG5_LANES = (1, 4)
 CONFIG5_BLOCK_ROWS = 2048
 
 
-def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=5):
+def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=15):
     """dense_bf16 (the stub stack's stand-in for the projections) on a block of rows at the
     three projection shapes of the family: device time per dispatch and MFMA rate."""
     out = []
@@ -358,7 +361,7 @@ def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=5):
         b_x, b_w, b_y = (dev.wrap(t.data_ptr(), t.numel() * 2, keepalive=t) for t in (x, w, y))
         figures = time_graph(queue, lambda cb: cb.encode(
             lib.pipeline("dense_bf16"), {0: b_x, 1: b_w, 2: b_y}, {3: rows, 4: in_dim, 5: out_dim},
-            ((out_dim + 63) // 64, (rows + 15) // 16), (256,)), 1, replays=repeats, warm=2)
+            ((out_dim + 63) // 64, (rows + 15) // 16), (256,)), 1, replays=repeats, warm=10)
         flops = 2.0 * rows * in_dim * out_dim
         tflops = flops / (figures["median_us"] * 1e-6) / 1e12
         out.append({"operator": "dense_bf16", "rows": rows, "in": in_dim, "out": out_dim,
@@ -761,7 +764,7 @@ def main():
         line["detail"]["q4_projections"] = (
             [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)
              for name in q4_sweep.FAMILIES] +
-            [q4_sweep.measure(dev, queue, lib, name, 16384, True, 2) for name in q4_sweep.FAMILIES])
+            [q4_sweep.measure(dev, queue, lib, name, 16384, True, 6) for name in q4_sweep.FAMILIES])
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(threads)
     print(json.dumps(line))
