@@ -68,6 +68,38 @@ __device__ __forceinline__ float sigmoid_bf16(float x) {
     return x < 0.0f ? low : rb(1.0f - low);
 }
 
+// The same bf16 steps for two values at once, rounded by the hardware's packed conversion
+// (round to nearest even: the bits of rb for every finite value and for infinities; a NaN
+// comes out quiet instead of with its upper bits kept) - one instruction and two to pull the
+// halves apart again where rb takes five a value.  For the block kernels, whose time is these
+// roundings.
+typedef __attribute__((ext_vector_type(2))) float rb_f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 rb_bf16x2;
+__device__ __forceinline__ uint32_t rb_pair_bits(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(rb_f32x2{a, b}, rb_bf16x2));
+}
+__device__ __forceinline__ void rb_pair(float& a, float& b) {
+    const uint32_t pair = rb_pair_bits(a, b);
+    a = __uint_as_float(pair << 16);
+    b = __uint_as_float(pair & 0xFFFF0000u);
+}
+__device__ __forceinline__ float reciprocal_for_bf16(float d) {   // see rb_reciprocal
+    const float size = fabsf(d);
+    return (size >= 0x1p-100f && size <= 0x1p+100f) ? __builtin_amdgcn_rcpf(d) : 1.0f / d;
+}
+__device__ __forceinline__ void sigmoid_bf16_pair(float x0, float x1, float& s0, float& s1) {
+    float e0 = expf(fabsf(x0)), e1 = expf(fabsf(x1));
+    rb_pair(e0, e1);
+    float d0 = 1.0f + e0, d1 = 1.0f + e1;
+    rb_pair(d0, d1);
+    float low0 = reciprocal_for_bf16(d0), low1 = reciprocal_for_bf16(d1);
+    rb_pair(low0, low1);
+    float high0 = 1.0f - low0, high1 = 1.0f - low1;
+    rb_pair(high0, high1);
+    s0 = x0 < 0.0f ? low0 : high0;
+    s1 = x1 < 0.0f ? low1 : high1;
+}
+
 // decay and beta of one value head from the a / b projection rows
 // (gdn.metal:133-150): softplus as bf16 LogAddExp, outer exponentials in fp32
 __device__ __forceinline__ void head_gates(uint16_t a_bits, uint16_t b_bits, uint16_t a_log,
@@ -233,14 +265,20 @@ __global__ __launch_bounds__(256) void gdn_prepare_block_kernel(PrepareArgs a) {
             a.projection + static_cast<uint64_t>(row) * a.projection_stride + c);
         float act[8];
 #pragma unroll
-        for (uint32_t j = 0; j < 8; ++j) {
+        for (uint32_t j = 0; j < 8; j += 2) {
             // fixed four-term shape; bf16 x bf16 products are exact in fp32
-            const float convolved = w[j][0] * widen_half(t0[j >> 1], j) +
-                                    w[j][1] * widen_half(t1[j >> 1], j) +
-                                    w[j][2] * widen_half(t2[j >> 1], j) +
-                                    w[j][3] * widen_half(t3[j >> 1], j);
-            const float conv_b = rb(convolved);
-            act[j] = rb(conv_b * sigmoid_bf16(conv_b));
+            float conv[2];
+#pragma unroll
+            for (uint32_t e = 0; e < 2; ++e) {
+                conv[e] = w[j + e][0] * widen_half(t0[j >> 1], e) + w[j + e][1] * widen_half(t1[j >> 1], e) +
+                          w[j + e][2] * widen_half(t2[j >> 1], e) + w[j + e][3] * widen_half(t3[j >> 1], e);
+            }
+            rb_pair(conv[0], conv[1]);
+            float gate0, gate1;
+            sigmoid_bf16_pair(conv[0], conv[1], gate0, gate1);
+            act[j] = conv[0] * gate0;
+            act[j + 1] = conv[1] * gate1;
+            rb_pair(act[j], act[j + 1]);
         }
         if (row == a.rows - 1) {
             *reinterpret_cast<u32x4*>(a.conv_out + c) = t1;
@@ -265,13 +303,17 @@ __global__ __launch_bounds__(256) void gdn_prepare_block_kernel(PrepareArgs a) {
             const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
-                packed[j] = narrow_pair(rb(act[2 * j] * inverse) * scale,
-                                        rb(act[2 * j + 1] * inverse) * scale);
+                float n0 = act[2 * j] * inverse, n1 = act[2 * j + 1] * inverse;
+                rb_pair(n0, n1);
+                packed[j] = rb_pair_bits(n0 * scale, n1 * scale);
             }
             *reinterpret_cast<u32x4*>(a.qk + static_cast<uint64_t>(row) * a.qk_stride + c) = packed;
         } else {
+            // already bf16 values: their upper halves are the bits
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) packed[j] = narrow_pair(act[2 * j], act[2 * j + 1]);
+            for (uint32_t j = 0; j < 4; ++j) {
+                packed[j] = (__float_as_uint(act[2 * j]) >> 16) | (__float_as_uint(act[2 * j + 1]) & 0xFFFF0000u);
+            }
             *reinterpret_cast<u32x4*>(a.value + static_cast<uint64_t>(row) * a.value_stride + c -
                                       kGdnQkValues) = packed;
         }
@@ -498,18 +540,25 @@ __global__ __launch_bounds__(256) void gdn_gate_norm_block_kernel(
         float total = run0 + run1;
         total = row_sum(total);
         const float inverse = 1.0f / sqrtf(total / static_cast<float>(kGD) + kRmsNormEpsilon);
-        float r[8];
-#pragma unroll
-        for (uint32_t j = 0; j < 8; ++j) {
-            const float normed = rb(w[j] * rb(v[j] * inverse));
-            const float g = widen_half(zb[j >> 1], j);
-            const float low = 1.0f / (1.0f + expf(fabsf(g)));
-            const float sig = g < 0.0f ? low : 1.0f - low;
-            r[j] = (g * sig) * normed;
-        }
         u32x4 packed;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) packed[j] = narrow_pair(r[2 * j], r[2 * j + 1]);
+        for (uint32_t j = 0; j < 8; j += 2) {
+            float r[2];
+            float n0 = v[j] * inverse, n1 = v[j + 1] * inverse;
+            rb_pair(n0, n1);
+            n0 *= w[j];
+            n1 *= w[j + 1];
+            rb_pair(n0, n1);
+            const float normed[2] = {n0, n1};
+#pragma unroll
+            for (uint32_t e = 0; e < 2; ++e) {
+                const float g = widen_half(zb[j >> 1], e);
+                const float low = 1.0f / (1.0f + expf(fabsf(g)));
+                const float sig = g < 0.0f ? low : 1.0f - low;
+                r[e] = (g * sig) * normed[e];
+            }
+            packed[j >> 1] = rb_pair_bits(r[0], r[1]);
+        }
         *reinterpret_cast<u32x4*>(out + at) = packed;
     }
 }
