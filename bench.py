@@ -5,10 +5,11 @@ A step is one decode token wave of 4 lanes at 32768 visible keys through the att
 family of the whole 40-layer hybrid stack, G,G,G,A x 10 (30 Gated DeltaNet layers, 10
 full-attention layers), with the lane-batched operators:
     GDN:       gdn_decode_fused_ms (prepare + recurrence + gate-norm in one dispatch)
-    attention: attn_qk_rope_ms -> attention_decode_split_ms -> attention_decode_combine_ms, or
-               with --attention token attention_decode_token_ms +
-               attention_decode_token_finish_ms (qk-norm and rotation inside the split-K walk;
-               the token's own key and value folded in and appended by the finishing dispatch)
+    attention: attention_decode_token_ms -> attention_decode_token_finish_ms (qk-norm and
+               rotation inside the split-K walk; the token's own key and value folded in and
+               appended by the finishing dispatch: what the host runtime records), or with
+               --attention three the reference's own sequence attn_qk_rope_ms ->
+               attention_decode_split_ms -> attention_decode_combine_ms
 Projections (the reference's Q4 GEMVs) are not on the path: their outputs are resident
 random bf16 slabs.  Every layer has its own KV pools, recurrent state and inputs, all in
 HBM before the timed region (2.7 GB of keys and values: the 256 MB last-level cache cannot
@@ -58,7 +59,8 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # counter runs (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
 # counter read for a plain 256 MiB copy of known size; see the file named here.
 TRAFFIC_SOURCE = "profiles/flash_decode_4x32768_hbm_counters.md"
-TRAFFIC_BYTES = round((131289.6 * 262144.0 / 131083.3 + 2151.0) * 1024)   # 271,060,546
+TRAFFIC_BYTES = {"three": round((131289.6 * 262144.0 / 131083.3 + 2151.0) * 1024),    # 271,060,546
+                 "token": round((131303.6 * 262144.0 / 131083.3 + 2146.9) * 1024)}    # 271,085,019
 ATTN_BYTES_PER_KEY = 2048       # K and V rows of both kv heads, bf16
 GDN_BYTES_PER_LANE_LAYER = 4194304 + 2 * 49152 + 65536 + 24704 + 4 * 8192
 CONFIG3 = {
@@ -614,10 +616,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--attention", choices=("three", "token"), default="three",
-                    help="three: rope, split and combine dispatches (the faster key walk); token: the "
-                         "walk norms and rotates the query heads itself, a finishing dispatch folds "
-                         "in the token's own key and value")
+    ap.add_argument("--attention", choices=("three", "token"), default="token",
+                    help="token: the walk norms and rotates the query heads itself, a finishing "
+                         "dispatch folds in the token's own key and value (what the host runtime "
+                         "records: the shorter wave); three: rope, split and combine dispatches, "
+                         "the reference's own sequence")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true",
                     help="skip the 16384-row block prefill figures in detail.prefill_16k")
@@ -627,7 +630,7 @@ def main():
     ap.add_argument("--no-config3", action="store_true",
                     help="skip the ragged-lane and deep-lane figures in detail.config3")
     ap.add_argument("--split-keys", type=int, default=0,
-                    help="keys per split-K workgroup of --attention three (multiple of 32); 0: what "
+                    help="keys per split-K workgroup of the key walk (multiple of 32); 0: what "
                          "the host runtime picks for the wave (1024 at 4 x 32768, 800 at 1 x 100000)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device-to-device copies first, so a "
@@ -704,8 +707,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": uniform["walk_kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": uniform["walk_kernel_frac"],
-                     "traffic": TRAFFIC_BYTES if args.attention == "three" else None,
-                     "traffic_source": TRAFFIC_SOURCE if args.attention == "three" else None,
+                     "traffic": TRAFFIC_BYTES[args.attention],
+                     "traffic_source": TRAFFIC_SOURCE,
                      "algorithmic_bytes": uniform["algorithmic_bytes"],
                      "avg_launch_us": walk["mean_us"], "median_launch_us": walk["median_us"],
                      "p10_launch_us": walk["p10_us"], "p90_launch_us": walk["p90_us"],

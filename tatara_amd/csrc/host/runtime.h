@@ -206,8 +206,9 @@ struct DecodeBatchScratch {
     // attention_decode_token_finish_ms (norm and rotation inside the split-K walk over the
     // cached keys; the token's own key and value folded in, and appended, by the finishing
     // dispatch) instead of rope, split path, combine and the short-row bucket: every row
-    // through the same two dispatches, records in `attn_partials`.
-    bool attention_token_form{false};
+    // through the same two dispatches, records in `attn_partials`.  The default: a 40-layer
+    // wave is 2 to 7 % shorter with it (one dispatch less per attention layer), at any depth.
+    bool attention_token_form{true};
 };
 
 // Keys per split-K workgroup for one attention layer of a wave whose rows see

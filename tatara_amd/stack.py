@@ -106,12 +106,12 @@ class StubStack:
     state and the scratch, and records token waves and prefill blocks."""
 
     def __init__(self, dev, lib, weights, lanes, capacity, vocab, block_rows=2048,
-                 split_keys=None, attention_form="three", fused_wave_steps=False):
-        """attention_form: "three" records a token wave's attention layer as rope, split-K
-        and combine dispatches (split_keys keys per workgroup); "token" as the two-dispatch
+                 split_keys=None, attention_form="token", fused_wave_steps=False):
+        """attention_form: "token" records a token wave's attention layer as the two-dispatch
         form (attention_decode_token_ms norms and rotates the query heads inside the split-K
         walk, attention_decode_token_finish_ms folds in and appends the token's own key and
-        value).
+        value: the shorter wave at every depth); "three" as rope, split-K and combine
+        dispatches (split_keys keys per workgroup), the reference's own sequence.
         fused_wave_steps: decode waves of several lanes over 4-bit weights take the norm in
         the prologue of the input projection and the residual sum in the epilogue of the
         output projection (same bits, one dispatch less per layer; measured slower, because

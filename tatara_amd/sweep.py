@@ -7,6 +7,8 @@ family, projections and norms together, without the per-command events).
 
     python -m tatara_amd.sweep [--layers 40] [--decode 1024,4096,...] [--prefill 4096,32768]
                                [--quantized]   (4-bit projections instead of dense bf16)
+                               [--attention three]   (rope, split and combine dispatches instead
+                                                      of the two-dispatch token form)
 prints one JSON line per measured point and a closing summary line."""
 import argparse
 import json
@@ -29,9 +31,10 @@ def _family_ms(times):
     return family, stub
 
 
-def measure_decode(dev, queue, lib, weights, layers, lanes, context, repeats=5):
+def measure_decode(dev, queue, lib, weights, layers, lanes, context, repeats=5, attention="token"):
     capacity = ((context + 1 + 1023) // 1024) * 1024
-    st = S.StubStack(dev, lib, weights, lanes, capacity, vocab=1024, block_rows=16)
+    st = S.StubStack(dev, lib, weights, lanes, capacity, vocab=1024, block_rows=16,
+                     attention_form=attention)
     st.context = [context] * lanes
     st._write_tables()
     st.x.write(np.full(lanes * S.HIDDEN, 0x3C00, np.uint16))
@@ -96,6 +99,7 @@ def main(argv=None):
     ap.add_argument("--prefill", default="4096,32768")
     ap.add_argument("--lanes", default="1,4")
     ap.add_argument("--quantized", action="store_true")
+    ap.add_argument("--attention", choices=("token", "three"), default="token")
     args = ap.parse_args(argv)
     dev = B.Device()
     queue = dev.create_queue()
@@ -104,7 +108,8 @@ def main(argv=None):
     points = []
     for lanes in [int(v) for v in args.lanes.split(",") if v]:
         for context in [int(v) for v in args.decode.split(",") if v]:
-            points.append(measure_decode(dev, queue, lib, weights, args.layers, lanes, context))
+            points.append(measure_decode(dev, queue, lib, weights, args.layers, lanes, context,
+                                         attention=args.attention))
             print(json.dumps(points[-1]), flush=True)
         for tokens in [int(v) for v in args.prefill.split(",") if v]:
             points.append(measure_prefill(dev, queue, lib, weights, args.layers, lanes, tokens))
