@@ -102,11 +102,11 @@ struct FlashPrefillArgs {
 // raised per tile, O rescaled), which finishes the walk.
 constexpr uint32_t kFlashWaves = 8;
 constexpr uint32_t kTilePositions = 32;
-constexpr uint32_t kRing = 3;
-constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 50688
+constexpr uint32_t kRing = 4;
+constexpr uint32_t kKeyRingBytes = kRing * kKeyStageBytes;             // 67584
 constexpr uint32_t kValuePairBytes = 1056;                             // row i | row 16+i | 32 B pad
 constexpr uint32_t kValuePairedStageBytes = 16 * kValuePairBytes;      // 16896
-constexpr uint32_t kFlashLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 101376
+constexpr uint32_t kFlashLdsBytes = kKeyRingBytes + kRing * kValuePairedStageBytes;  // 135168
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
@@ -197,6 +197,15 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
 
     const uint32_t key_read_bytes = m * kKeyPairBytes + g * 16;
     // S^T of the tile in key stage `slot`; operand reads run one contraction step ahead
+    // The operands of a tile's first contraction step are requested while the tile before it
+    // is still being accumulated (its keys have landed by then), those of the first V^T
+    // product before the softmax: neither phase starts on an LDS round trip.
+    u32x4 first_keys[2];
+    auto request_first_keys = [&](uint32_t slot) {
+        const uint8_t* stage = key_ring + slot * kKeyStageBytes + key_read_bytes;
+        first_keys[0] = *reinterpret_cast<const u32x4*>(stage);
+        first_keys[1] = *reinterpret_cast<const u32x4*>(stage + 512);
+    };
     auto scores = [&](uint32_t slot, f32x4 (&s)[2][NB]) {
         const uint8_t* stage = key_ring + slot * kKeyStageBytes + key_read_bytes;
 #pragma unroll
@@ -205,8 +214,8 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
             for (uint32_t b = 0; b < NB; ++b) s[kt][b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
         u32x4 ka[2][2];
-        ka[0][0] = *reinterpret_cast<const u32x4*>(stage);
-        ka[0][1] = *reinterpret_cast<const u32x4*>(stage + 512);
+        ka[0][0] = first_keys[0];
+        ka[0][1] = first_keys[1];
 #pragma unroll
         for (uint32_t kk = 0; kk < 8; ++kk) {
             if (kk + 1 < 8) {
@@ -238,12 +247,22 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         const u32x2 h = __builtin_bit_cast(u32x2, hi);
         return u32x4{l[0], l[1], h[0], h[1]};
     };
+    u32x4 first_values;
+    auto request_first_values = [&](uint32_t slot) {
+        first_values = read_values(value_ring + slot * kValuePairedStageBytes + value_read_bytes);
+    };
     auto accumulate = [&](uint32_t slot, const bf16x8 (&pb)[NB]) {
         const uint8_t* vt = value_ring + slot * kValuePairedStageBytes + value_read_bytes;
         u32x4 va[2];
-        va[0] = read_values(vt);
+        va[0] = first_values;
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
+            if (j == 10) {
+                // far enough from the barrier to have arrived by then, late enough for the
+                // registers of the last score step to be free
+                request_first_keys((slot + 1) & 3);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (j + 1 < 16) va[(j + 1) & 1] = read_values(vt + (j + 1) * 32);
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) {
@@ -306,31 +325,35 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         return alpha;
     };
 
-    // Batch j, issued on entering tile j: keys and values of tile j+2.
+    // Batch j, issued on entering tile j: keys and values of tile j+3.
     stage_tile(0, 0);
     stage_tile(1, 1);
-    // Ring position of the tile being entered: kslot = kb % 3; tile kb+2 goes to
-    // (kb+2) % 3, the stage tile kb-1 has just left.
+    stage_tile(2, 2);
+    // Ring position of the tile being entered: kslot = kb % 4; tile kb+3 goes to
+    // (kb+3) % 4, the stage tile kb-1 has just left.
     uint32_t kb = 0;
     uint32_t kslot = 0;
-    // Entering tile kb: batch kb-2 (this tile) has landed for every wave and every wave
-    // is done with tile kb-1.
+    // Entering tile kb: batches up to kb-2 (tiles up to kb+1) have landed for every wave, so
+    // the next tile's first operands may be read while this one is accumulated, and every
+    // wave is done with tile kb-1.
     auto enter_tile = [&]() {
         __builtin_amdgcn_s_waitcnt(0x0F74);  // all but the 4 transfers of batch kb-1
         __syncthreads();
-        stage_tile(kb + 2, kslot == 0 ? kRing - 1 : kslot - 1);
+        stage_tile(kb + 3, (kslot + 3) & 3);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto advance = [&]() {
         ++kb;
-        kslot = kslot == kRing - 1 ? 0 : kslot + 1;
+        kslot = (kslot + 1) & 3;
     };
 
     bf16x8 pb[NB];
     enter_tile();
+    request_first_keys(kslot);
     {
         f32x4 s[2][NB];
         scores(kslot, s);
+        request_first_values(kslot);
 #pragma unroll
         for (uint32_t b = 0; b < NB; ++b) {
             float x[8];
@@ -349,6 +372,7 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         while (kb < end) {
             f32x4 s[2][NB];
             scores(kslot, s);
+            request_first_values(kslot);
             __builtin_amdgcn_sched_barrier(0);
             float sums[NB];
             bf16x8 next[NB];
@@ -376,9 +400,13 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
     bool above = steady(std::false_type{}, min(first_masked, nkb));
     if (!above) above = steady(std::true_type{}, nkb);
     if (above) {
+        // (a wave that leaves the steady loop has taken the scores of tile kb, so it asks for
+        // that tile's first keys again)
+        request_first_keys(kslot);
         for (;;) {
             f32x4 s[2][NB];
             scores(kslot, s);
+            request_first_values(kslot);
 #pragma unroll
             for (uint32_t b = 0; b < NB; ++b) {
                 float x[8];
