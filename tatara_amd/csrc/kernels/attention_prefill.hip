@@ -84,9 +84,14 @@ struct FlashPrefillArgs {
 // Workgroup = 8 wave64 = 32 consecutive query positions x the 8 query heads of one
 // kv head.  Wave w owns heads 2(w&3), 2(w&3)+1 at positions 16(w>>2)..+15: two 16x16
 // blocks that share every K and V fragment the wave reads from LDS.  Two waves per
-// SIMD (256 registers each): one wave's softmax (VALU) runs under the other's
-// products (MFMA), and LDS operand reads are issued from eight waves.
-//   K and V tiles: HBM/L2 -> LDS rings of 3 stages, two tiles ahead (global_load_lds).
+// SIMD (256 registers each): LDS operand reads are issued from eight waves and one
+// wave's LDS round trips are covered by the other's products.  (The two waves of a SIMD
+// pass every phase nearly together - the barrier keeps them in step - so the softmax
+// itself is not hidden; forms that keep them a phase apart were measured and are slower,
+// because a wave alone in its products waits for its own operand reads.)
+//   K and V tiles: HBM/L2 -> LDS rings of 4 stages, three tiles ahead (global_load_lds), so
+//   that a tile has landed one barrier before it is entered and its first operands can be
+//   read while the tile before it is still being accumulated.
 //   Both are stored as 16 row pairs (row i | row 16+i | 32 B pad): with pairs of 1056 bytes
 //   both the 16-byte S^T operand reads (sixteen pairs, one piece per quarter wave) and the
 //   transposing V reads were measured free of bank conflicts (pairs of 1040 bytes cost the
@@ -196,7 +201,6 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
     const float scale = kAttnScale * kLog2e;
 
     const uint32_t key_read_bytes = m * kKeyPairBytes + g * 16;
-    // S^T of the tile in key stage `slot`; operand reads run one contraction step ahead
     // The operands of a tile's first contraction step are requested while the tile before it
     // is still being accumulated (its keys have landed by then), those of the first V^T
     // product before the softmax: neither phase starts on an LDS round trip.
@@ -206,6 +210,7 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         first_keys[0] = *reinterpret_cast<const u32x4*>(stage);
         first_keys[1] = *reinterpret_cast<const u32x4*>(stage + 512);
     };
+    // S^T of the tile in key stage `slot`; operand reads run one contraction step ahead
     auto scores = [&](uint32_t slot, f32x4 (&s)[2][NB]) {
         const uint8_t* stage = key_ring + slot * kKeyStageBytes + key_read_bytes;
 #pragma unroll
