@@ -374,6 +374,42 @@ def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=15):
     return out
 
 
+def block_2048_figures(B, dev, queue, lib, torch, capacity=32768, repeats=12):
+    """The causal flash kernel on the reference's block size: 2048 new rows behind 30720, 14336
+    and 0 cached tokens of one lane, as attention_flash_v2_blk (one workgroup per 32 rows and kv
+    head: 128 workgroups) and as attention_flash_split_blk with the sharers the library plans
+    for the device.  Device time per dispatch (the split form's clearing dispatch included)."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x2048)
+    rows = 2048
+
+    def rb(n):
+        t = torch.randn(n, generator=gen, device="cuda").to(torch.bfloat16)
+        return dev.wrap(t.data_ptr(), n * 2, keepalive=t)
+
+    keys, values = rb(2 * capacity * 256), rb(2 * capacity * 256)
+    q, gate = rb(rows * 4096), rb(rows * 4096)
+    out = dev.create_buffer(rows * 8192)
+    points = []
+    for base in (capacity - rows, 14336, 0):
+        sharers = B.flash_prefill_splits(rows, base + rows, dev.compute_units)
+        scratch = dev.create_buffer(max(B.flash_prefill_scratch_bytes(rows, sharers), 256))
+        flops = 16 * 1024.0 * (rows * base + rows * (rows + 1) / 2)
+        point = {"rows": rows, "cached_tokens": base, "sharers": sharers}
+        for name, bind, const in (
+                ("attention_flash_v2_blk", {}, {}),
+                ("attention_flash_split_blk", {9: scratch}, {10: sharers})):
+            figures = time_graph(queue, lambda cb: cb.encode(
+                lib.pipeline(name), {0: q, 1: keys, 2: values, 3: gate, 4: out, **bind},
+                {5: base + rows, 6: capacity, 7: rows, 8: base, **const},
+                (16, (rows + 15) // 16), (256,)), 1, replays=repeats, warm=6)
+            tflops = flops / (figures["median_us"] * 1e-6) / 1e12
+            point[name] = {"us": figures["median_us"], "tflops": round(tflops, 1),
+                           "frac_of_bf16_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4)}
+        points.append(point)
+    return points
+
+
 def config5_decode_point(dev, queue, lib, torch, attention, lanes, visible):
     """One decode token wave of `lanes` lanes at `visible` visible keys through the
     attention family of all 40 layers (own caches and state per layer), compiled into one
@@ -402,6 +438,7 @@ def config5_prefill_point(dev, queue, lib, torch, lanes, tokens):
     over the lane's cache so far.  Own caches and recurrent state per layer and lane;
     the projections (resident random slabs) are shared by the layers of a kind.  Device time
     of each block's command buffer (launch gaps included), summed."""
+    from tatara_amd import backend as B
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0xC5F1 + tokens)
     rows_max = min(CONFIG5_BLOCK_ROWS, tokens)
@@ -424,6 +461,11 @@ def config5_prefill_point(dev, queue, lib, torch, lanes, tokens):
     qk, v, z, y = (mk(rows_max * 8192) for _ in range(4))
     decay, beta = mk(rows_max * 128), mk(rows_max * 128)
     chunk = mk(((rows_max + 63) // 64) * 32 * 115712)
+    # a 2048-row block is 128 workgroups of the flash kernel: the host shares each position
+    # tile's key walk between as many workgroups as fill the device (attention_flash_split_blk)
+    units = dev.compute_units
+    shared_walk = mk(max([B.flash_prefill_scratch_bytes(r, B.flash_prefill_splits(r, tokens, units))
+                          for r in range(32, rows_max + 1, 32)] + [256]))
     attention_layers = LAYERS // PERIOD
     stripe_bytes = 2 * tokens * 256 * 2
     caches = [(mk(lanes * stripe_bytes), mk(lanes * stripe_bytes)) for _ in range(attention_layers)]
@@ -447,9 +489,16 @@ def config5_prefill_point(dev, queue, lib, torch, lanes, tokens):
                               {0: a_proj, 1: ones256, 2: ones256, 3: q, 4: gate, 5: keys, 6: values},
                               {7: base, 8: tokens}, (18, rows), (256,))
                     cb.barrier()
-                    cb.encode(P("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: out},
-                              {5: base + rows, 6: tokens, 7: rows, 8: base},
-                              (16, (rows + 15) // 16), (256,))
+                    sharers = B.flash_prefill_splits(rows, base + rows, units)
+                    if sharers > 1:
+                        cb.encode(P("attention_flash_split_blk"),
+                                  {0: q, 1: keys, 2: values, 3: gate, 4: out, 9: shared_walk},
+                                  {5: base + rows, 6: tokens, 7: rows, 8: base, 10: sharers},
+                                  (16, (rows + 15) // 16), (256,))
+                    else:
+                        cb.encode(P("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: out},
+                                  {5: base + rows, 6: tokens, 7: rows, 8: base},
+                                  (16, (rows + 15) // 16), (256,))
                 else:
                     conv, rec = states[gdn]
                     gdn += 1
@@ -763,6 +812,7 @@ def main():
         if not args.no_cpu_baseline:
             line["detail"]["prefill_16k"]["cpu_baseline"] = cpu_prefill_baseline(threads)
         line["detail"]["dense_bf16_block"] = dense_block_figures(dev, queue, lib, torch)
+        line["detail"]["prefill_block_2048"] = block_2048_figures(B, dev, queue, lib, torch)
         from tatara_amd import q4_sweep
         line["detail"]["q4_projections"] = (
             [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)

@@ -306,6 +306,19 @@ int32_t tt_attention_decode_lanes_static(tt_queue* queue, const void* q, uint64_
 uint32_t tt_split_workgroups(const uint32_t* visible_keys, uint32_t rows, uint32_t split_keys);
 uint32_t tt_choose_split_keys(const uint32_t* visible_keys, uint32_t rows, uint32_t compute_units);
 
+/* Planning of attention_flash_split_blk (no counterpart in the reference, whose prefill walks
+ * 256-row query tiles of blocks of at most 2048 rows, prefill_step.cpp:1469-1475): a block of
+ * few rows is few workgroups - 2048 rows are 128 on 256 compute units - while each of them
+ * walks the whole prefix, so the operator lets several workgroups share a position tile's
+ * key walk.
+ *
+ * tt_flash_prefill_splits: the sharers per tile (1..8) with which a block of `rows` rows, the
+ * last of which sees visible_keys keys, fills compute_units (1 where the longest walk is
+ * under 16 tiles of 32 keys); tt_flash_prefill_scratch_bytes: what the operator's scratch binding must
+ * hold for that many (0 for one). */
+uint32_t tt_flash_prefill_splits(uint32_t rows, uint32_t visible_keys, uint32_t compute_units);
+uint64_t tt_flash_prefill_scratch_bytes(uint32_t rows, uint32_t splits);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = [
     "tt_command_name", "tt_command_gpu_ms", "tt_attention_decode_lanes_static",
     "tt_event_create", "tt_event_destroy", "tt_encode_signal_event", "tt_encode_wait_for_event",
     "tt_split_workgroups", "tt_choose_split_keys",
+    "tt_flash_prefill_splits", "tt_flash_prefill_scratch_bytes",
 ]
 
 
@@ -105,6 +106,8 @@ def lib():
         "tt_attention_decode_lanes_static": (i32, [vp] + [vp, u64] * 6 + [u32] * 4),
         "tt_split_workgroups": (u32, [C.POINTER(u32), u32, u32]),
         "tt_choose_split_keys": (u32, [C.POINTER(u32), u32, u32]),
+        "tt_flash_prefill_splits": (u32, [u32, u32, u32]),
+        "tt_flash_prefill_scratch_bytes": (u64, [u32, u32]),
         "tt_event_create": (i32, [vp, pvp]), "tt_event_destroy": (None, [vp]),
         "tt_encode_signal_event": (i32, [vp, vp, u64]),
         "tt_encode_wait_for_event": (i32, [vp, vp, u64]),
@@ -455,3 +458,15 @@ def choose_split_keys(visible_keys, compute_units=256):
     """Keys per split-K workgroup for a token wave (tt_choose_split_keys)."""
     array, count = _u32_array(visible_keys)
     return int(lib().tt_choose_split_keys(array, count, int(compute_units)))
+
+
+def flash_prefill_splits(rows, visible_keys, compute_units=256):
+    """Workgroups that share a position tile's key walk in attention_flash_split_blk so that a
+    block of `rows` rows, whose last row sees `visible_keys` keys, fills the device
+    (tt_flash_prefill_splits)."""
+    return int(lib().tt_flash_prefill_splits(int(rows), int(visible_keys), int(compute_units)))
+
+
+def flash_prefill_scratch_bytes(rows, splits):
+    """Bytes the scratch binding of attention_flash_split_blk must hold (0 for one split)."""
+    return int(lib().tt_flash_prefill_scratch_bytes(int(rows), int(splits)))

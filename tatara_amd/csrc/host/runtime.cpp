@@ -1351,6 +1351,7 @@ PrefillPipelinesResult resolve_prefill_pipelines(const HipLibrary& library) {
     const bool ok =
         resolve(library, p, &P::attn_qk_rope_blk, "attn_qk_rope_blk", error) &&
         resolve(library, p, &P::attention_flash_blk, "attention_flash_v2_blk", error) &&
+        resolve(library, p, &P::attention_flash_split_blk, "attention_flash_split_blk", error) &&
         resolve(library, p, &P::gdn_conv_blk, "gdn_conv_blk", error) &&
         resolve(library, p, &P::gdn_gates_blk, "gdn_gates_blk", error) &&
         resolve(library, p, &P::gdn_recurrence_gates_blk, "gdn_recurrence_gates_blk", error) &&
@@ -1370,6 +1371,15 @@ PrefillScratchResult create_prefill_scratch(const HipDevice& device,
     if (!device) return {DecodeStepError::InvalidDevice, std::nullopt};
     PrefillScratch s;
     s.block_rows = geometry.policy.maximum_block_rows;
+    s.compute_units = std::max<std::uint32_t>(device.compute_units(), 1);
+    // the most any block of up to block_rows rows needs when its key walks are shared
+    std::uint64_t shared_walk_bytes = 0;
+    for (std::uint32_t rows = 32; rows <= std::max<std::uint32_t>(s.block_rows, 32); rows += 32) {
+        shared_walk_bytes = std::max<std::uint64_t>(
+            shared_walk_bytes,
+            tt_flash_prefill_scratch_bytes(
+                rows, tt_flash_prefill_splits(rows, geometry.policy.context_capacity, s.compute_units)));
+    }
     const std::uint64_t parameter_bytes =
         std::uint64_t{s.block_rows} * 32u * kF32Bytes;  // [rows][32] decay / beta
     if (!allocate_zeroed(device, geometry.gdn_projection_bytes, s.gdn_projection) ||
@@ -1388,7 +1398,8 @@ PrefillScratchResult create_prefill_scratch(const HipDevice& device,
         !allocate_zeroed(device, geometry.attention_projection_bytes, s.attn_projection) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_query) ||
         !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_gate) ||
-        !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_attended)) {
+        !allocate_zeroed(device, geometry.attention_vector_bytes, s.attn_attended) ||
+        (shared_walk_bytes != 0 && !allocate_zeroed(device, shared_walk_bytes, s.attn_shared_walk))) {
         return {DecodeStepError::BufferAllocationFailed, std::nullopt};
     }
     return {DecodeStepError::None, std::move(s)};
@@ -1417,16 +1428,23 @@ HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
     walk.constant(capacity, 8);
     walk.dispatch(18, 256, rows);
     walk.barrier();
-    walk.pipeline(pipelines.attention_flash_blk);
+    const std::uint32_t visible = static_cast<std::uint32_t>(position) + rows;
+    const std::uint32_t sharers =
+        scratch.attn_shared_walk ? tt_flash_prefill_splits(rows, visible, scratch.compute_units) : 1;
+    walk.pipeline(sharers > 1 ? pipelines.attention_flash_split_blk : pipelines.attention_flash_blk);
     walk.buffer(scratch.attn_query, 0, 0);
     walk.buffer(state.first, 0, 1);
     walk.buffer(state.second, 0, 2);
     walk.buffer(scratch.attn_gate, 0, 3);
     walk.buffer(scratch.attn_attended, 0, 4);
-    walk.constant(static_cast<std::uint32_t>(position) + rows, 5);
+    walk.constant(visible, 5);
     walk.constant(capacity, 6);
     walk.constant(rows, 7);
     walk.constant(static_cast<std::uint32_t>(position), 8);
+    if (sharers > 1) {
+        walk.buffer(scratch.attn_shared_walk, 0, 9);
+        walk.constant(sharers, 10);
+    }
     walk.dispatch(16, 256, (rows + 15u) / 16u);
     return walk.error;
 }

@@ -580,7 +580,7 @@ PrefillChunk prefill_chunk_at(const PrefillPolicy& policy, std::uint32_t context
                               std::uint32_t total_rows, std::uint32_t ordinal);
 
 struct PrefillPipelines {
-    HipComputePipeline attn_qk_rope_blk, attention_flash_blk;
+    HipComputePipeline attn_qk_rope_blk, attention_flash_blk, attention_flash_split_blk;
     HipComputePipeline gdn_conv_blk, gdn_gates_blk, gdn_recurrence_gates_blk, gdn_recurrence_blk,
         gdn_gate_norm_blk, gdn_chunk_recurrence_blk;
     HipComputePipeline gdn_conv_tape_blk, gdn_recurrence_gates_tape_blk, gdn_tape_replay_blk;
@@ -601,6 +601,10 @@ struct PrefillScratch {
     HipBuffer gdn_decay, gdn_beta, gdn_chunk;
     HipBuffer gdn_tape, gdn_conv_tape;
     HipBuffer attn_projection, attn_query, attn_gate, attn_attended;
+    // attention_flash_split_blk: a block of few rows is few workgroups, so several share each
+    // position tile's key walk (tt_flash_prefill_splits) and exchange their results here
+    HipBuffer attn_shared_walk;
+    std::uint32_t compute_units{256};
 };
 struct PrefillScratchResult {
     DecodeStepError error;
@@ -614,7 +618,8 @@ PrefillScratchResult create_prefill_scratch(const HipDevice& device,
 
 // encode_attention (prefill_step.cpp:1386-1851): rope + append the chunk's rows
 // at context_base + chunk.offset, then causal attention of the chunk (one flash
-// dispatch for the whole chunk; the reference walks 256-row query tiles).
+// dispatch for the whole chunk; the reference walks 256-row query tiles).  Chunks of too
+// few rows to fill the device take attention_flash_split_blk.
 HipCommandError encode_prefill_attention(const PrefillPipelines& pipelines,
                                          const PrefillGeometry& geometry, PrefillScratch& scratch,
                                          const DecodeLayerState& state, const LayerWeights& weights,

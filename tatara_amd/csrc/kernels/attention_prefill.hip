@@ -37,8 +37,7 @@ constexpr uint32_t kTileKeys = 32;
 constexpr uint32_t kKeyPairBytes = 1056;                 // key i | key 16+i | 32 B pad
 constexpr uint32_t kKeyStageBytes = 16 * kKeyPairBytes;  // 16896
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kReferenceSlack = 100.0f;  // log2 units a score may exceed the fixed reference by
-constexpr float kReferenceSlackPower = 0x1p100f;   // 2^kReferenceSlack
+constexpr float kReferenceSlackPower = 0x1p100f;   // a score may exceed the fixed reference by 100 log2 units
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
     return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -77,7 +76,25 @@ struct FlashPrefillArgs {
     uint32_t rows;
     uint32_t tile_context;   // cache position of row 0
     uint32_t capacity;
+    uint32_t splits;         // workgroups that share the key walk of a position tile (grid z)
+    uint8_t* scratch;        // splits > 1: arrival counts, then the partial results
 };
+
+// Key walk shared between workgroups.  A block of few rows is few position tiles - 2048 rows
+// are 128 workgroups on 256 compute units - while each of them walks the whole prefix.  With
+// splits > 1 the key tiles of a position tile are dealt to that many workgroups in equal
+// ranges; each range is an ordinary walk with its own softmax reference.  A workgroup that is
+// not the last of its position tile to finish leaves {O, reference, row sum} in scratch, fp32,
+// in the register order of its lanes; the last one - told by an arrival count, nobody waits
+// for anybody - adds the others' to its own with the usual reference change and writes the
+// rows.  A walk of fewer than kMinTilesPerSplit key tiles per workgroup is shared by fewer.
+constexpr uint32_t kMaxFlashSplits = 8;
+constexpr uint32_t kMinTilesPerSplit = 4;
+constexpr uint32_t kPartialBytes = 512 * 132 * 4;   // per lane 128 values of O, two references, two row-sum shares
+constexpr uint32_t kArrivalBytesPerTile = 4;
+__host__ __device__ constexpr uint64_t flash_arrival_bytes(uint32_t rows) {
+    return ((static_cast<uint64_t>((rows + 31) / 32) * kAttnKvHeads * kArrivalBytesPerTile + 255) / 256) * 256;
+}
 
 // ---------------------------------------------------------- flash kernel ------
 //
@@ -132,7 +149,13 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
     const uint32_t head0 = kvh * kAttnHeadsPerKv + (wave & 3) * 2;
     const uint32_t p0 = tile * kTilePositions;
     const uint32_t tile_keys = a.tile_context + min(p0 + kTilePositions, a.rows);  // visible count
-    const uint32_t nkb = (tile_keys + kTileKeys - 1) / kTileKeys;
+    const uint32_t walk_tiles = (tile_keys + kTileKeys - 1) / kTileKeys;
+    // this workgroup's share of the walk: key tiles [kb_begin, nkb)
+    const uint32_t sharers = min(a.splits, max(walk_tiles / kMinTilesPerSplit, 1u));
+    const uint32_t share = blockIdx.z;
+    if (share >= sharers) return;
+    const uint32_t kb_begin = static_cast<uint32_t>(static_cast<uint64_t>(walk_tiles) * share / sharers);
+    const uint32_t nkb = static_cast<uint32_t>(static_cast<uint64_t>(walk_tiles) * (share + 1) / sharers);
     // this lane's column: query row p0 + 16*half + m, whose last visible key is limit
     const uint32_t row = p0 + half * 16 + m;
     const uint32_t limit = a.tile_context + row;
@@ -330,13 +353,13 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         return alpha;
     };
 
-    // Batch j, issued on entering tile j: keys and values of tile j+3.
-    stage_tile(0, 0);
-    stage_tile(1, 1);
-    stage_tile(2, 2);
-    // Ring position of the tile being entered: kslot = kb % 4; tile kb+3 goes to
-    // (kb+3) % 4, the stage tile kb-1 has just left.
-    uint32_t kb = 0;
+    // Batch j, issued on entering the walk's tile j: keys and values of its tile j+3.
+    stage_tile(kb_begin, 0);
+    stage_tile(kb_begin + 1, 1);
+    stage_tile(kb_begin + 2, 2);
+    // Ring position of the tile being entered: kslot = (kb - kb_begin) % 4; tile kb+3 goes
+    // to the stage tile kb-1 has just left.
+    uint32_t kb = kb_begin;
     uint32_t kslot = 0;
     // Entering tile kb: batches up to kb-2 (tiles up to kb+1) have landed for every wave, so
     // the next tile's first operands may be read while this one is accumulated, and every
@@ -362,7 +385,7 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
 #pragma unroll
         for (uint32_t b = 0; b < NB; ++b) {
             float x[8];
-            (void)exact_step(0, s, b, x);  // O and the sums are still zero
+            (void)exact_step(kb, s, b, x);  // O and the sums are still zero
             l_run[b] += probabilities(x, pb[b]);
         }
         accumulate(kslot, pb);
@@ -427,6 +450,70 @@ void attention_flash_prefill_kernel(FlashPrefillArgs a) {
         }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // transfers of the tiles past the walk
+
+    if (sharers > 1) {
+        // Arrival: every workgroup but the last to finish leaves its result and goes; the
+        // last one takes the others' in.  The count starts at zero (the launcher clears it).
+        // Results travel as device-scope stores and loads of single words, which go through
+        // to memory and come from it whatever the L2 of either side holds: the writer waits
+        // for their acknowledgement before it counts itself in, and no cache is written back
+        // or dropped (fences of that scope, one per wave, cost 60 us a launch: the L2s of
+        // eight dies written back 2000 times).
+        __shared__ uint32_t arrival;
+        const uint32_t pair = tile * kAttnKvHeads + kvh;
+        float* const partials = reinterpret_cast<float*>(a.scratch + flash_arrival_bytes(a.rows)) +
+                                static_cast<uint64_t>(pair) * a.splits * (kPartialBytes / 4);
+        const auto publish = [](float* at, float value) {
+            __hip_atomic_store(reinterpret_cast<uint32_t*>(at), __float_as_uint(value), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        };
+        const auto collect = [](const float* at) {
+            return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(at),
+                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        };
+        // element e of a lane's 132 (O of head b, dim block j, value i at (b*16+j)*4+i, then
+        // the two references and the two row-sum shares) lies at [e][thread]
+        float* const mine = partials + static_cast<uint64_t>(share) * (kPartialBytes / 4) + threadIdx.x;
+#pragma unroll
+        for (uint32_t b = 0; b < NB; ++b) {
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) publish(mine + ((b * 16 + j) * 4 + i) * 512, o[b][j][i]);
+            }
+            publish(mine + (128 + b) * 512, m_run[b]);
+            publish(mine + (130 + b) * 512, l_run[b]);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // every store of this wave acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            arrival = __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(a.scratch) + pair, 1u,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (arrival != sharers - 1) return;
+        for (uint32_t other = 0; other < sharers; ++other) {
+            if (other == share) continue;
+            const float* theirs = partials + static_cast<uint64_t>(other) * (kPartialBytes / 4) + threadIdx.x;
+#pragma unroll
+            for (uint32_t b = 0; b < NB; ++b) {
+                const float m_other = collect(theirs + (128 + b) * 512);
+                const float l_other = collect(theirs + (130 + b) * 512);
+                const float m_new = fmaxf(m_run[b], m_other);
+                const float keep = __builtin_amdgcn_exp2f(m_run[b] - m_new);
+                const float take = __builtin_amdgcn_exp2f(m_other - m_new);
+                m_run[b] = m_new;
+                l_run[b] = l_run[b] * keep + l_other * take;
+#pragma unroll
+                for (uint32_t j = 0; j < 16; ++j) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; ++i) {
+                        o[b][j][i] = o[b][j][i] * keep + collect(theirs + ((b * 16 + j) * 4 + i) * 512) * take;
+                    }
+                }
+            }
+        }
+    }
 
     // out[(row*16 + head)*256 + dim] = bf16((O/l) * sigmoid(gate)); lane holds, for
     // position column m, dims 16j + 4g + i
@@ -562,6 +649,24 @@ __global__ __launch_bounds__(256) void attention_combine_blk_kernel(const float*
 
 // ---------------------------------------------------------------- launchers --
 
+}  // namespace
+
+uint32_t flash_prefill_splits(uint32_t rows, uint32_t visible, uint32_t compute_units) {
+    const uint64_t groups = static_cast<uint64_t>((rows + kTilePositions - 1) / kTilePositions) * kAttnKvHeads;
+    // a longest walk that two workgroups would not share is not worth the clearing dispatch
+    if (groups == 0 || (static_cast<uint64_t>(visible) + kTileKeys - 1) / kTileKeys < 4 * kMinTilesPerSplit) return 1;
+    const uint64_t fit = compute_units / groups;
+    return static_cast<uint32_t>(fit < 1 ? 1 : fit > kMaxFlashSplits ? kMaxFlashSplits : fit);
+}
+
+uint64_t flash_prefill_scratch_bytes(uint32_t rows, uint32_t splits) {
+    if (splits <= 1) return 0;
+    const uint64_t groups = static_cast<uint64_t>((rows + kTilePositions - 1) / kTilePositions) * kAttnKvHeads;
+    return flash_arrival_bytes(rows) + groups * splits * kPartialBytes;
+}
+
+namespace {
+
 uint64_t cache_bytes(uint32_t capacity) {
     return static_cast<uint64_t>(kAttnKvHeads) * capacity * kD * 2;
 }
@@ -571,8 +676,13 @@ uint64_t cache_bytes(uint32_t capacity) {
 // c7 tile_rows, c8 tile_context; grid (16, ceil(tile_rows/16)) x 256
 // (prefill_step.cpp:1657-1717).  tile_rows is not limited to the reference's
 // 256-row query tile: one dispatch may cover a whole block.
-int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t stream,
-                               bool validate_only) {
+__global__ void clear_arrivals_kernel(uint32_t* words, uint32_t count) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) words[i] = 0;
+}
+
+int32_t flash_blk(const Bindings& b, const Grid& g, hipStream_t stream, bool validate_only,
+                  bool shared_walk) {
     Args a(b);
     FlashPrefillArgs f{};
     const uint32_t visible = a.constant(5);
@@ -596,11 +706,38 @@ int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t str
     f.values = a.buffer<const uint16_t>(2, cache_bytes(f.capacity));
     f.gate = a.buffer<const uint16_t>(3, row_bytes);
     f.out = a.buffer<uint16_t>(4, row_bytes);
+    f.splits = 1;
+    if (shared_walk) {
+        f.splits = a.constant(10);
+        a.require(f.splits >= 1 && f.splits <= kMaxFlashSplits, TT_CMD_INVALID_DISPATCH_EXTENT);
+        if (a.status != TT_OK) return a.status;
+        if (f.splits > 1) f.scratch = a.buffer<uint8_t>(9, flash_prefill_scratch_bytes(f.rows, f.splits));
+    }
     if (a.status != TT_OK || validate_only) return a.status;
-    hipLaunchKernelGGL(attention_flash_prefill_kernel,
-                       dim3((f.rows + kTilePositions - 1) / kTilePositions, kAttnKvHeads),
+    const uint32_t tiles = (f.rows + kTilePositions - 1) / kTilePositions;
+    if (f.splits > 1) {
+        const uint32_t words = tiles * kAttnKvHeads;
+        hipLaunchKernelGGL(clear_arrivals_kernel, dim3((words + 255) / 256), dim3(256), 0, stream,
+                           reinterpret_cast<uint32_t*>(f.scratch), words);
+    }
+    hipLaunchKernelGGL(attention_flash_prefill_kernel, dim3(tiles, kAttnKvHeads, f.splits),
                        dim3(kFlashWaves * 64), kFlashLdsBytes, stream, f);
     return TT_OK;
+}
+
+int32_t op_attention_flash_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                               bool validate_only) {
+    return flash_blk(b, g, stream, validate_only, false);
+}
+
+// attention_flash_split_blk (no counterpart in the reference): the bindings, constants and
+// grid of attention_flash_v2_blk, plus b9 scratch and c10 splits (1..8) - the workgroups that
+// share each position tile's key walk.  tt_flash_prefill_splits gives the count that fills
+// the device for a block of `rows` rows that sees `visible` keys, tt_flash_prefill_scratch_bytes the bytes b9 must hold
+// (none for one split).  Same results as attention_flash_v2_blk up to the order of fp32 sums.
+int32_t op_attention_flash_split_blk(const Bindings& b, const Grid& g, hipStream_t stream,
+                                     bool validate_only) {
+    return flash_blk(b, g, stream, validate_only, true);
 }
 
 // attention_partial_blk: b0 query(+tile), b1 keys, b2 values, c3 tile_context,
@@ -671,6 +808,7 @@ const KernelDesc kAttentionPrefillKernels[] = {
     {"attn_qk_rope_blk", op_attn_qk_rope_blk},
     {"attention_streaming_blk", op_attention_flash_blk},
     {"attention_flash_v2_blk", op_attention_flash_blk},
+    {"attention_flash_split_blk", op_attention_flash_split_blk},
     {"attention_partial_blk", op_attention_partial_blk},
     {"attention_combine_blk", op_attention_combine_blk},
 };

@@ -226,6 +226,14 @@ uint32_t tt_choose_split_keys(const uint32_t* visible_keys, uint32_t rows, uint3
     return static_cast<uint32_t>(split);
 }
 
+uint32_t tt_flash_prefill_splits(uint32_t rows, uint32_t visible_keys, uint32_t compute_units) {
+    return tt::flash_prefill_splits(rows, visible_keys, compute_units);
+}
+
+uint64_t tt_flash_prefill_scratch_bytes(uint32_t rows, uint32_t splits) {
+    return tt::flash_prefill_scratch_bytes(rows, splits);
+}
+
 const char* tt_status_name(int32_t status) {
     switch (status) {
     case TT_OK: return "None";

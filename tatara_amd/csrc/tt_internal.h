@@ -93,6 +93,12 @@ hipStream_t queue_stream(const tt_queue* queue);
 // Compute units of the device the queue was made on (0 for a null queue).
 uint32_t queue_compute_units(const tt_queue* queue);
 
+// attention_flash_split_blk: the workgroups that share a position tile's key walk so that a
+// block of `rows` rows whose last row sees `visible` keys fills `compute_units`, and the
+// scratch bytes that many need.
+uint32_t flash_prefill_splits(uint32_t rows, uint32_t visible, uint32_t compute_units);
+uint64_t flash_prefill_scratch_bytes(uint32_t rows, uint32_t splits);
+
 // One-time kernel attribute set-up (large dynamic LDS opt-in); called when a
 // library is created, so it never runs inside a stream capture.
 bool prepare_decode_kernels();

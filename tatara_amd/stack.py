@@ -163,6 +163,11 @@ class StubStack:
         self.decay, self.beta = mk(rows * 128), mk(rows * 128)
         self.partials = mk(lanes * 16 * self.max_splits * 258 * 4)
         self.chunk = mk(((min(block_rows, 2048) + 63) // 64) * 32 * CHUNK_RECORD_BYTES)
+        # blocks of few rows share each position tile's key walk between workgroups; the most
+        # scratch any block up to block_rows needs is at one workgroup per compute unit
+        self.flash_scratch = mk(max(
+            [backend.flash_prefill_scratch_bytes(r, backend.flash_prefill_splits(r, 1 << 20, self.groups))
+             for r in range(32, max(block_rows, 32) + 1, 32)] + [256]))
         self.logits = mk(rows * vocab * 2)
         self._write_tables()
 
@@ -399,10 +404,18 @@ class StubStack:
                           {0: self.proj, 1: layer["q_norm"], 2: layer["k_norm"], 3: self.q, 4: self.gate,
                            5: keys, 6: values}, {7: base, 8: self.capacity}, (18, rows), (256,))
                 cb.barrier()
-                cb.encode(P("attention_flash_v2_blk"),
-                          {0: self.q, 1: keys, 2: values, 3: self.gate, 4: self.mixed},
-                          {5: base + rows, 6: self.capacity, 7: rows, 8: base},
-                          (16, (rows + 15) // 16), (256,))
+                splits = backend.flash_prefill_splits(rows, base + rows, self.groups)
+                if splits > 1:
+                    cb.encode(P("attention_flash_split_blk"),
+                              {0: self.q, 1: keys, 2: values, 3: self.gate, 4: self.mixed,
+                               9: self.flash_scratch},
+                              {5: base + rows, 6: self.capacity, 7: rows, 8: base, 10: splits},
+                              (16, (rows + 15) // 16), (256,))
+                else:
+                    cb.encode(P("attention_flash_v2_blk"),
+                              {0: self.q, 1: keys, 2: values, 3: self.gate, 4: self.mixed},
+                              {5: base + rows, 6: self.capacity, 7: rows, 8: base},
+                              (16, (rows + 15) // 16), (256,))
             cb.barrier()
             self._project_out(cb, layer, rows, block=True)
             self._residual_and_norm(cb, rows, index)

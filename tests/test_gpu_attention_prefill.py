@@ -18,9 +18,12 @@ def _weights():
     return q_w, k_w
 
 
-def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, weights=None):
+def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, weights=None,
+                  splits=None, replays=0):
     """Runs rope + flash prefill on the GPU for `rows` new tokens after `base`
-    cached ones and compares the selected rows with the checker."""
+    cached ones and compares the selected rows with the checker.  splits: through
+    attention_flash_split_blk with that many workgroups sharing each position tile's key walk,
+    and held to the one-workgroup operator's result as well."""
     B, dev, queue, lib = gpu()
     q_w, k_w = _weights() if weights is None else weights
     if proj is None:
@@ -41,20 +44,52 @@ def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, 
     b_qw, b_kw = dev.buffer_from(q_w), dev.buffer_from(k_w)
     b_q, b_g, b_o = (dev.create_buffer(rows * 8192) for _ in range(3))
     tiles = (rows + 15) // 16
+    if splits:
+        # scratch starts as 0xFF bytes: the operator clears its arrival counts itself
+        need = B.flash_prefill_scratch_bytes(rows, splits)
+        b_s = dev.buffer_from(np.full(max(need, 256), 0xFF, np.uint8))
+
+    def flash(cb, out):
+        if splits:
+            cb.encode(lib.pipeline("attention_flash_split_blk"),
+                      {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: out, 9: b_s},
+                      {5: base + rows, 6: cap, 7: rows, 8: base, 10: splits}, (16, tiles), (256,))
+        else:
+            # the reference's two names of the streaming path resolve to the one kernel
+            cb.encode(lib.pipeline("attention_streaming_blk" if base % 2 else "attention_flash_v2_blk"),
+                      {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: out},
+                      {5: base + rows, 6: cap, 7: rows, 8: base}, (16, tiles), (256,))
 
     def rec(cb):
         cb.encode(lib.pipeline("attn_qk_rope_blk"),
                   {0: b_p, 1: b_qw, 2: b_kw, 3: b_q, 4: b_g, 5: b_k, 6: b_v}, {7: base, 8: cap},
                   (18, rows), (256,))
         cb.barrier()
-        # the reference's two names of the streaming path resolve to the one kernel
-        cb.encode(lib.pipeline("attention_streaming_blk" if base % 2 else "attention_flash_v2_blk"),
-                  {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: b_o},
-                  {5: base + rows, 6: cap, 7: rows, 8: base}, (16, tiles), (256,))
+        flash(cb, b_o)
     ms = run(rec)
     got = b_o.read(np.uint16).reshape(rows, 4096)
     w = want.reshape(rows, 4096)
-    check_bf16(got[sel], w[sel], f"flash prefill rows {rows} base {base}")
+    what = f"flash prefill rows {rows} base {base}" + (f" splits {splits}" if splits else "")
+    check_bf16(got[sel], w[sel], what)
+    if splits:
+        # against one workgroup per position tile: each share rounds its probabilities to bf16
+        # against its own reference, so the two differ like either does from the checker
+        b_o1 = dev.create_buffer(rows * 8192)
+        run(lambda cb: cb.encode(lib.pipeline("attention_flash_v2_blk"),
+                                 {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: b_o1},
+                                 {5: base + rows, 6: cap, 7: rows, 8: base}, (16, tiles), (256,)))
+        check_bf16(got, b_o1.read(np.uint16).reshape(rows, 4096), what + " vs one workgroup a tile",
+                   max_abs=8e-3, mean_abs=2e-4, ulps=2)
+    if replays:
+        # a compiled command buffer replayed: every replay clears and counts again
+        cb = queue.create_command_buffer()
+        cb.begin_compute_pass(); flash(cb, b_o); cb.end_compute_pass()
+        cb.compile()
+        for replay in range(replays):
+            b_o.write(np.zeros(rows * 4096, np.uint16))
+            cb.commit().wait()
+            again = b_o.read(np.uint16).reshape(rows, 4096)
+            check_bf16(again, got, what + f" replay {replay}", max_abs=8e-3, mean_abs=1e-5, ulps=1)
     # cache: raw V exact, roped K at the decode bar, rows beyond untouched
     gk = b_k.read(np.uint16).reshape(2, cap, 256)
     gv = b_v.read(np.uint16).reshape(2, cap, 256)
@@ -134,6 +169,45 @@ def test_scores_far_above_the_first_tile_take_the_exact_loop():
     w = np.full(256, 0x4040, np.uint16)                     # 3.0
     _prefill_case(rows, 0, 128, 0xE8AD, proj=np.ascontiguousarray(proj).reshape(-1), weights=(w, w),
                   control=True)
+
+
+@pytest.mark.parametrize("rows,base,splits", [(64, 1000, 2), (64, 1000, 8), (37, 700, 4), (13, 300, 8),
+                                              (1, 0, 8), (1, 4000, 3), (300, 33, 2), (100, 5000, 8),
+                                              (40, 95, 5)])
+def test_key_walk_shared_between_workgroups(rows, base, splits):
+    """attention_flash_split_blk: up to eight workgroups share a position tile's key walk and the
+    last to finish adds the others' results to its own.  Walks too short for the count asked
+    are shared by fewer (13 rows at 300: two of eight; the first tiles of a block at context
+    0 or 33: one), rows that are not whole tiles, one row."""
+    print(f"[case] shared key walk rows {rows} base {base} splits {splits}", flush=True)
+    _prefill_case(rows, base, 8192, 0x5A1E + rows + splits, splits=splits, replays=2)
+
+
+def test_shared_walk_with_a_share_in_the_exact_loop():
+    """The upper share of the last position tiles meets scores 150 log2 units above its first
+    tile's and finishes in the exact loop; its reference then lies far above the lower share's,
+    whose result the merge scales to nothing."""
+    print("[case] shared key walk, one share in the exact softmax loop", flush=True)
+    rows = 320
+    proj = ol.gaussian_bf16(0xE8B0, rows * 9216).reshape(rows, 9216)
+    for r in range(288, rows):
+        proj[r, 8192:8448] = proj[rows - 1, 0:256]
+        proj[r, 8448:8704] = proj[rows - 1, 4096:4352]
+    w = np.full(256, 0x4040, np.uint16)                     # 3.0
+    _prefill_case(rows, 0, 512, 0xE8B1, proj=np.ascontiguousarray(proj).reshape(-1), weights=(w, w),
+                  splits=2, select=list(range(0, 320, 7)) + list(range(280, 320)))
+
+
+def test_shared_walk_of_a_2048_row_block_deep_in_a_cache():
+    """The shape the operator is for: a 2048-row block behind 6144 cached tokens, as many shares
+    as fill the device (two on 256 compute units); sampled rows against the checker, every row
+    against the one-workgroup operator."""
+    B, dev, queue, lib = gpu()
+    splits = B.flash_prefill_splits(2048, 8192, dev.compute_units)
+    print(f"[case] shared key walk, 2048 rows at context 6144, splits {splits}", flush=True)
+    rows = [0, 1, 31, 32, 33, 1000, 1023, 1024, 2016, 2047] + list(range(300, 2048, 97))
+    ms, _ = _prefill_case(2048, 6144, 8192, 0x2048, select=sorted(set(rows)), splits=max(splits, 2))
+    print(f"[time] rope + flash, 2048 rows at 6144: {ms:.3f} ms", flush=True)
 
 
 def test_config4_prefill_16384_rows():

@@ -41,3 +41,21 @@ def test_split_keys_rule_never_oversubscribes():
             if split > 128:
                 share = -(-2 * sum(visible) // units)
                 assert split - 32 < share or S.split_workgroups(visible, split - 32) > units
+
+
+@pytest.mark.parametrize("rows,units,splits,scratch", [
+    (2048, 256, 2, 512 + 128 * 2 * 270336), (1024, 256, 4, 256 + 64 * 4 * 270336),
+    (512, 256, 8, 256 + 32 * 8 * 270336), (256, 256, 8, 256 + 16 * 8 * 270336),
+    (13, 256, 8, 256 + 2 * 8 * 270336), (4096, 256, 1, 0), (16384, 256, 1, 0),
+    (2048, 304, 2, 512 + 128 * 2 * 270336), (2048, 128, 1, 0), (2049, 256, 1, 0), (0, 256, 1, 0)])
+def test_flash_prefill_sharing_plan(rows, units, splits, scratch):
+    """tt_flash_prefill_splits: as many workgroups per position tile (32 rows x 2 kv heads) as fit
+    the compute units, between one and eight; tt_flash_prefill_scratch_bytes: a 4-byte arrival
+    count per tile and kv head, padded to 256 bytes, and 270,336 bytes per sharer - 32 f32x4 of O
+    and one of {reference, row sum} for each of 512 lanes."""
+    from tatara_amd import backend as B
+    assert B.flash_prefill_splits(rows, 32768, units) == splits
+    assert B.flash_prefill_splits(rows, 480, units) == 1     # a longest walk under 16 key tiles
+    assert B.flash_prefill_splits(rows, 481, units) == splits
+    assert B.flash_prefill_scratch_bytes(rows, splits) == scratch
+    assert B.flash_prefill_scratch_bytes(rows, 1) == 0
