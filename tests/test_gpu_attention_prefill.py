@@ -210,6 +210,38 @@ def test_shared_walk_of_a_2048_row_block_deep_in_a_cache():
     print(f"[time] rope + flash, 2048 rows at 6144: {ms:.3f} ms", flush=True)
 
 
+def test_shared_walk_on_drawn_shapes_against_one_workgroup_a_tile():
+    """Twenty drawn blocks (1-700 rows behind 0-9000 cached tokens, 2-8 sharers asked for, random
+    bf16 operands straight into the flash operators): the shared walk against the unshared one
+    on the same buffers, and no row left unwritten."""
+    B, dev, queue, lib = gpu()
+    rng = np.random.default_rng(0x5A4E)
+    cap = 9728
+    keys = dev.buffer_from(ol.gaussian_bf16(0x5A4F, 2 * cap * 256))
+    values = dev.buffer_from(ol.gaussian_bf16(0x5A50, 2 * cap * 256))
+    for case in range(20):
+        rows = int(rng.integers(1, 701))
+        base = int(rng.integers(0, 9001)) if case % 4 else 0
+        splits = int(rng.integers(2, 9))
+        print(f"[case] drawn block {case}: rows {rows} base {base} splits {splits}", flush=True)
+        q = dev.buffer_from(ol.gaussian_bf16(0x6000 + case, rows * 4096, 0.0, 0.25))
+        gate = dev.buffer_from(ol.gaussian_bf16(0x7000 + case, rows * 4096))
+        outs = [dev.buffer_from(np.full(rows * 4096, 0x7FC0, np.uint16)) for _ in range(2)]
+        scratch = dev.buffer_from(np.full(max(B.flash_prefill_scratch_bytes(rows, splits), 256), 0xA5, np.uint8))
+        const = {5: base + rows, 6: cap, 7: rows, 8: base}
+        grid = (16, (rows + 15) // 16)
+
+        def rec(cb):
+            cb.encode(lib.pipeline("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: outs[0]},
+                      const, grid, (256,))
+            cb.encode(lib.pipeline("attention_flash_split_blk"),
+                      {0: q, 1: keys, 2: values, 3: gate, 4: outs[1], 9: scratch}, {**const, 10: splits},
+                      grid, (256,))
+        run(rec)
+        one, shared = (o_.read(np.uint16) for o_ in outs)
+        check_bf16(shared, one, f"drawn block {case}", max_abs=8e-3, mean_abs=2e-4, ulps=2)
+
+
 def test_config4_prefill_16384_rows():
     """Config 4: 16384 new tokens into an empty capacity-16384 cache.  The checker
     computes a strided subset of query rows (every 257th plus the first and last
