@@ -376,9 +376,11 @@ def dense_block_figures(dev, queue, lib, torch, rows=16384, repeats=15):
 
 def block_2048_figures(B, dev, queue, lib, torch, capacity=32768, repeats=12):
     """The causal flash kernel on the reference's block size: 2048 new rows behind 30720, 14336
-    and 0 cached tokens of one lane, as attention_flash_v2_blk (one workgroup per 32 rows and kv
-    head: 128 workgroups) and as attention_flash_split_blk with the sharers the library plans
-    for the device.  Device time per dispatch (the split form's clearing dispatch included)."""
+    and 0 cached tokens of one lane, with one workgroup per 32 rows and kv head (128 workgroups:
+    attention_flash_split_blk told to share nothing), with the sharers the library plans for the
+    device in the caller's scratch, and as attention_flash_v2_blk, which plans the same in its
+    queue's workspace.  Device time per dispatch (the clearing dispatch of a shared walk
+    included)."""
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0x2048)
     rows = 2048
@@ -396,16 +398,17 @@ def block_2048_figures(B, dev, queue, lib, torch, capacity=32768, repeats=12):
         scratch = dev.create_buffer(max(B.flash_prefill_scratch_bytes(rows, sharers), 256))
         flops = 16 * 1024.0 * (rows * base + rows * (rows + 1) / 2)
         point = {"rows": rows, "cached_tokens": base, "sharers": sharers}
-        for name, bind, const in (
-                ("attention_flash_v2_blk", {}, {}),
-                ("attention_flash_split_blk", {9: scratch}, {10: sharers})):
+        for label, name, bind, const in (
+                ("one_workgroup_a_tile", "attention_flash_split_blk", {}, {10: 1}),
+                ("attention_flash_split_blk", "attention_flash_split_blk", {9: scratch}, {10: sharers}),
+                ("attention_flash_v2_blk", "attention_flash_v2_blk", {}, {})):
             figures = time_graph(queue, lambda cb: cb.encode(
                 lib.pipeline(name), {0: q, 1: keys, 2: values, 3: gate, 4: out, **bind},
                 {5: base + rows, 6: capacity, 7: rows, 8: base, **const},
                 (16, (rows + 15) // 16), (256,)), 1, replays=repeats, warm=6)
             tflops = flops / (figures["median_us"] * 1e-6) / 1e12
-            point[name] = {"us": figures["median_us"], "tflops": round(tflops, 1),
-                           "frac_of_bf16_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4)}
+            point[label] = {"us": figures["median_us"], "tflops": round(tflops, 1),
+                            "frac_of_bf16_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4)}
         points.append(point)
     return points
 

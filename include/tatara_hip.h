@@ -138,7 +138,11 @@ const char* tt_device_name(const tt_device* device);
 /* Number of compute units of the device (no reference counterpart; used to size
  * split-K grids). */
 uint32_t tt_device_compute_units(const tt_device* device);
-/* create_command_queue (resources.h:239): one in-order HIP stream. */
+/* create_command_queue (resources.h:239): one in-order HIP stream.  A queue also owns a
+ * workspace in device memory (270,336 bytes per compute unit: 69 MB on 256) for operators
+ * whose reference bindings carry no scratch - attention_flash_v2_blk / attention_streaming_blk
+ * share the key walks of a block of few rows through it; a queue whose workspace could not be
+ * allocated works without. */
 int32_t tt_queue_create(tt_device* device, tt_queue** out);
 void tt_queue_destroy(tt_queue* queue);
 /* The HIP stream (hipStream_t) behind a queue, for event timing by the caller. */
@@ -310,7 +314,8 @@ uint32_t tt_choose_split_keys(const uint32_t* visible_keys, uint32_t rows, uint3
  * 256-row query tiles of blocks of at most 2048 rows, prefill_step.cpp:1469-1475): a block of
  * few rows is few workgroups - 2048 rows are 128 on 256 compute units - while each of them
  * walks the whole prefix, so the operator lets several workgroups share a position tile's
- * key walk.
+ * key walk, with the count and the scratch in the caller's hands.  (attention_flash_v2_blk
+ * plans the same by itself and uses its queue's workspace.)
  *
  * tt_flash_prefill_splits: the sharers per tile (1..8) with which a block of `rows` rows, the
  * last of which sees visible_keys keys, fills compute_units (1 where the longest walk is

@@ -659,6 +659,12 @@ uint32_t flash_prefill_splits(uint32_t rows, uint32_t visible, uint32_t compute_
     return static_cast<uint32_t>(fit < 1 ? 1 : fit > kMaxFlashSplits ? kMaxFlashSplits : fit);
 }
 
+uint64_t stream_workspace_bytes(uint32_t compute_units) {
+    // the shared walk never has more workgroups than compute units; their arrival counts
+    // (at most one per two of them) stay under a page
+    return 4096 + static_cast<uint64_t>(compute_units) * kPartialBytes;
+}
+
 uint64_t flash_prefill_scratch_bytes(uint32_t rows, uint32_t splits) {
     if (splits <= 1) return 0;
     const uint64_t groups = static_cast<uint64_t>((rows + kTilePositions - 1) / kTilePositions) * kAttnKvHeads;
@@ -714,6 +720,18 @@ int32_t flash_blk(const Bindings& b, const Grid& g, hipStream_t stream, bool val
         if (f.splits > 1) f.scratch = a.buffer<uint8_t>(9, flash_prefill_scratch_bytes(f.rows, f.splits));
     }
     if (a.status != TT_OK || validate_only) return a.status;
+    if (!shared_walk) {
+        // the reference's bindings carry no scratch: the walk is shared through the queue's
+        // own workspace where the block is too few rows to fill the device
+        const StreamWorkspace workspace = stream_workspace(stream);
+        if (workspace.base != nullptr) {
+            const uint32_t planned = flash_prefill_splits(f.rows, visible, workspace.compute_units);
+            if (planned > 1 && flash_prefill_scratch_bytes(f.rows, planned) <= workspace.bytes) {
+                f.splits = planned;
+                f.scratch = workspace.base;
+            }
+        }
+    }
     const uint32_t tiles = (f.rows + kTilePositions - 1) / kTilePositions;
     if (f.splits > 1) {
         const uint32_t words = tiles * kAttnKvHeads;

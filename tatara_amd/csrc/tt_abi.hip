@@ -28,6 +28,8 @@ struct tt_device {
 struct tt_queue {
     tt_device* device = nullptr;
     hipStream_t stream = nullptr;
+    uint8_t* workspace = nullptr;   // see tt::StreamWorkspace
+    uint64_t workspace_bytes = 0;
 };
 
 struct tt_buffer {
@@ -67,6 +69,17 @@ uint32_t queue_compute_units(const tt_queue* queue) {
 
 hipStream_t queue_stream(const tt_queue* queue) {
     return queue != nullptr ? queue->stream : nullptr;
+}
+
+namespace {
+std::mutex g_workspace_mutex;
+std::map<hipStream_t, StreamWorkspace> g_workspaces;
+}  // namespace
+
+StreamWorkspace stream_workspace(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    const auto found = g_workspaces.find(stream);
+    return found == g_workspaces.end() ? StreamWorkspace{} : found->second;
 }
 }  // namespace tt
 
@@ -332,6 +345,18 @@ int32_t tt_queue_create(tt_device* device, tt_queue** out) {
     // of the static scratch): done here so that an entry point that launches directly on
     // the queue never has to do it inside a stream capture.  A failure shows at that call.
     (void)tt::prepare_decode_kernels();
+    // The queue's workspace.  Doing without it is not an error: the operators that would
+    // use it run as they do on a foreign stream.
+    const uint64_t bytes = tt::stream_workspace_bytes(device->compute_units);
+    void* workspace = nullptr;
+    if (bytes != 0 && hipMalloc(&workspace, bytes) == hipSuccess) {
+        queue->workspace = static_cast<uint8_t*>(workspace);
+        queue->workspace_bytes = bytes;
+        std::lock_guard<std::mutex> lock(tt::g_workspace_mutex);
+        tt::g_workspaces[stream] = tt::StreamWorkspace{queue->workspace, bytes, device->compute_units};
+    } else {
+        (void)hipGetLastError();
+    }
     *out = queue;
     return TT_OK;
 }
@@ -340,8 +365,13 @@ void tt_queue_destroy(tt_queue* queue) {
     if (queue == nullptr) return;
     if (queue->stream != nullptr) {
         (void)hipStreamSynchronize(queue->stream);
+        {
+            std::lock_guard<std::mutex> lock(tt::g_workspace_mutex);
+            tt::g_workspaces.erase(queue->stream);
+        }
         (void)hipStreamDestroy(queue->stream);
     }
+    if (queue->workspace != nullptr) (void)hipFree(queue->workspace);
     delete queue;
 }
 

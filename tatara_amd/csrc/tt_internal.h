@@ -93,6 +93,20 @@ hipStream_t queue_stream(const tt_queue* queue);
 // Compute units of the device the queue was made on (0 for a null queue).
 uint32_t queue_compute_units(const tt_queue* queue);
 
+// Device memory a queue owns for operators whose reference bindings carry no scratch (the
+// shared key walk of attention_flash_v2_blk on blocks of few rows).  Allocated when the queue
+// is created, so never under a stream capture; commands of one queue run in order, so one
+// operator at a time uses it.  base is null for a stream no queue of this library made, or
+// where the allocation failed.
+struct StreamWorkspace {
+    uint8_t* base = nullptr;
+    uint64_t bytes = 0;
+    uint32_t compute_units = 0;
+};
+StreamWorkspace stream_workspace(hipStream_t stream);
+// the bytes a queue's workspace holds on a device of that many compute units
+uint64_t stream_workspace_bytes(uint32_t compute_units);
+
 // attention_flash_split_blk: the workgroups that share a position tile's key walk so that a
 // block of `rows` rows whose last row sees `visible` keys fills `compute_units`, and the
 // scratch bytes that many need.

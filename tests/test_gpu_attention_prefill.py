@@ -74,10 +74,11 @@ def _prefill_case(rows, base, cap, seed, select=None, control=False, proj=None, 
     if splits:
         # against one workgroup per position tile: each share rounds its probabilities to bf16
         # against its own reference, so the two differ like either does from the checker
+        # (c10 = 1; attention_flash_v2_blk shares walks by itself through its queue's workspace)
         b_o1 = dev.create_buffer(rows * 8192)
-        run(lambda cb: cb.encode(lib.pipeline("attention_flash_v2_blk"),
+        run(lambda cb: cb.encode(lib.pipeline("attention_flash_split_blk"),
                                  {0: b_q, 1: b_k, 2: b_v, 3: b_g, 4: b_o1},
-                                 {5: base + rows, 6: cap, 7: rows, 8: base}, (16, tiles), (256,)))
+                                 {5: base + rows, 6: cap, 7: rows, 8: base, 10: 1}, (16, tiles), (256,)))
         check_bf16(got, b_o1.read(np.uint16).reshape(rows, 4096), what + " vs one workgroup a tile",
                    max_abs=8e-3, mean_abs=2e-4, ulps=2)
     if replays:
@@ -212,8 +213,9 @@ def test_shared_walk_of_a_2048_row_block_deep_in_a_cache():
 
 def test_shared_walk_on_drawn_shapes_against_one_workgroup_a_tile():
     """Twenty drawn blocks (1-700 rows behind 0-9000 cached tokens, 2-8 sharers asked for, random
-    bf16 operands straight into the flash operators): the shared walk against the unshared one
-    on the same buffers, and no row left unwritten."""
+    bf16 operands straight into the flash operators): the shared walk - with the caller's scratch
+    and count, and as attention_flash_v2_blk plans it in its queue's workspace - against the
+    unshared one on the same buffers, and no row left unwritten."""
     B, dev, queue, lib = gpu()
     rng = np.random.default_rng(0x5A4E)
     cap = 9728
@@ -226,20 +228,24 @@ def test_shared_walk_on_drawn_shapes_against_one_workgroup_a_tile():
         print(f"[case] drawn block {case}: rows {rows} base {base} splits {splits}", flush=True)
         q = dev.buffer_from(ol.gaussian_bf16(0x6000 + case, rows * 4096, 0.0, 0.25))
         gate = dev.buffer_from(ol.gaussian_bf16(0x7000 + case, rows * 4096))
-        outs = [dev.buffer_from(np.full(rows * 4096, 0x7FC0, np.uint16)) for _ in range(2)]
+        outs = [dev.buffer_from(np.full(rows * 4096, 0x7FC0, np.uint16)) for _ in range(3)]
         scratch = dev.buffer_from(np.full(max(B.flash_prefill_scratch_bytes(rows, splits), 256), 0xA5, np.uint8))
         const = {5: base + rows, 6: cap, 7: rows, 8: base}
         grid = (16, (rows + 15) // 16)
 
         def rec(cb):
-            cb.encode(lib.pipeline("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: outs[0]},
-                      const, grid, (256,))
+            cb.encode(lib.pipeline("attention_flash_split_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: outs[0]},
+                      {**const, 10: 1}, grid, (256,))
             cb.encode(lib.pipeline("attention_flash_split_blk"),
                       {0: q, 1: keys, 2: values, 3: gate, 4: outs[1], 9: scratch}, {**const, 10: splits},
                       grid, (256,))
+            cb.encode(lib.pipeline("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: outs[2]},
+                      const, grid, (256,))
         run(rec)
-        one, shared = (o_.read(np.uint16) for o_ in outs)
+        one, shared, planned = (o_.read(np.uint16) for o_ in outs)
         check_bf16(shared, one, f"drawn block {case}", max_abs=8e-3, mean_abs=2e-4, ulps=2)
+        check_bf16(planned, one, f"drawn block {case}, planned by the operator", max_abs=8e-3,
+                   mean_abs=2e-4, ulps=2)
 
 
 def test_config4_prefill_16384_rows():
