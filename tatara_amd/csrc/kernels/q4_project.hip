@@ -69,6 +69,11 @@ struct Q4Projection {
     const uint16_t* norm_weight;           // not null: the input rows go through the RMS norm first
     const uint16_t* residual;              // not null: output = bf16(residual + bf16(projection)),
     uint64_t residual_stride;              //   [rows][residual_stride]; may be the output itself
+    // the block kernel only: how its tiles are dealt to workgroups (see launch_block)
+    uint32_t tiles_n;                      // tiles along the output rows
+    uint32_t whole_tiles;                  // tiles 0 .. whole_tiles - 1 have a workgroup each
+    uint32_t sharers;                      // the others are shared by this many, a slice of K each
+    uint8_t* exchange;                     // arrival counts, then the sharers' partial sums
 };
 
 // The weight matrix that holds output row `n`, with n the same for every lane (matrices have
@@ -276,6 +281,8 @@ constexpr uint32_t kMetaKindBytes = kBlockN * 16;
 constexpr uint32_t kMetaWindowBytes = 2 * kMetaKindBytes;
 constexpr uint32_t kBlockLdsBytes = kMetaBase + 2 * kMetaWindowBytes;    // 163840
 constexpr uint32_t kOutRowBytes = 144;               // a wave's 64 results of one m on the way out
+constexpr uint32_t kExchangeCountBytes = 4096;       // arrival counts of the shared tiles (at most 1024)
+constexpr uint64_t kExchangeShareBytes = 512 * 64 * 4;   // a sharer's partial sums: 64 floats a lane
 static_assert(kBlockLdsBytes <= 160 * 1024, "one workgroup per compute unit");
 static_assert(8 * 64 * kOutRowBytes <= kWordBase, "the results leave through the idle x stages");
 
@@ -334,8 +341,18 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     const uint32_t wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t i16 = lane & 15, g = lane >> 4;
     const uint32_t out_rows = p.first_row[p.segments];
-    const uint32_t n0 = blockIdx.x * kBlockN, m0 = blockIdx.y * kBlockM;
-    const uint32_t groups = p.k_size / kQ4Group;
+    // tiles in rounds of one per compute unit, n fastest; those of the last, partly filled
+    // round are shared: `sharers` workgroups each take a slice of K (whole windows of eight
+    // groups) and the last to finish adds the others' sums to its own
+    const uint32_t shared = blockIdx.x >= p.whole_tiles;
+    const uint32_t beyond = shared ? blockIdx.x - p.whole_tiles : 0;
+    const uint32_t tile_index = shared ? p.whole_tiles + beyond / p.sharers : blockIdx.x;
+    const uint32_t sharers = shared ? p.sharers : 1;
+    const uint32_t share = shared ? beyond % p.sharers : 0;
+    const uint32_t n0 = (tile_index % p.tiles_n) * kBlockN, m0 = (tile_index / p.tiles_n) * kBlockM;
+    const uint32_t all_groups = p.k_size / kQ4Group;
+    const uint32_t first_group = all_groups / sharers * share;   // a multiple of 8
+    const uint32_t groups = first_group + all_groups / sharers;   // this workgroup's end
     const uint32_t lds_base = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds));
     // multiply role: the waves form two sets of four, the two waves that share a SIMD in
@@ -351,8 +368,8 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         while (segment + 1 < p.segments && n >= p.first_row[segment + 1]) ++segment;
         const uint64_t local = n - p.first_row[segment];
         words = p.words[segment] + local * (p.k_size / 8);
-        scales = p.scales[segment] + local * groups;
-        biases = p.biases[segment] + local * groups;
+        scales = p.scales[segment] + local * all_groups;
+        biases = p.biases[segment] + local * all_groups;
     };
 
     // ---- staging roles
@@ -524,7 +541,7 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
             scale[tn] = __uint_as_float(__builtin_amdgcn_perm(
                 0u, *reinterpret_cast<const uint32_t*>(scale_pairs + (64 * nh + 16 * tn + i16) * 16), pick));
         }
-        if ((group & 3) == 0 && group != 0) read_affine_terms(group - 4);
+        if ((group & 3) == 0 && group != first_group) read_affine_terms(group - 4);
         // the transfers overlap the reads above; they go into the x stage that both sets read
         // in their fetch (g - 1)
         if (group + 2 < groups) request(group + 2);
@@ -533,7 +550,7 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     auto multiply = [&](uint32_t group) __attribute__((always_inline)) {
         __builtin_amdgcn_s_setprio(1);
         // the four groups before this one are complete since this set's last multiply
-        if ((group & 3) == 0 && group != 0) add_affine_terms();
+        if ((group & 3) == 0 && group != first_group) add_affine_terms();
 #pragma unroll
         for (uint32_t tn = 0; tn < 4; ++tn) {
 #pragma unroll
@@ -575,15 +592,15 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
         __builtin_amdgcn_s_setprio(0);
     };
 
-    request(0);
-    request(1);   // the group count is a multiple of 8
+    request(first_group);
+    request(first_group + 1);   // the group count of a share is a multiple of 8
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    commit(0, read_words(0));
+    commit(first_group, read_words(first_group));
     __syncthreads();
     // every wave passes 2 * groups + 1 barriers: the second set one before its first slot,
     // the first set one after its last
     if (second_set) __syncthreads();
-    for (uint32_t group = 0; group < groups; ++group) {
+    for (uint32_t group = first_group; group < groups; ++group) {
         fetch(group);
         __syncthreads();
         multiply(group);
@@ -593,9 +610,57 @@ __global__ __launch_bounds__(kBlockThreads) void q4_block_kernel(Q4Projection p)
     read_affine_terms(groups - 4);
     add_affine_terms();
 
+    __syncthreads();   // nobody reads the stages any more (nor the sums, which the tiles do not reach)
+    if (sharers > 1) {
+        // Every sharer but the last to finish leaves its sums - device-scope stores of single
+        // words, which go through to memory whatever an L2 holds, [value][thread] so that a
+        // store instruction writes 256 contiguous bytes - waits for their acknowledgement,
+        // counts itself in and goes; the one whose count comes back sharers - 1 adds the
+        // others' to its own and stores the tile.  The launcher clears the counts.
+        uint32_t* const arrival = reinterpret_cast<uint32_t*>(lds + kBlockLdsBytes - 16);
+        float* const sums = reinterpret_cast<float*>(p.exchange + kExchangeCountBytes) +
+                            static_cast<uint64_t>(beyond / p.sharers) * p.sharers * (kBlockThreads * 64);
+        float* const mine = sums + static_cast<uint64_t>(share) * (kBlockThreads * 64) + t;
+#pragma unroll
+        for (uint32_t tn = 0; tn < 4; ++tn) {
+#pragma unroll
+            for (uint32_t tm = 0; tm < 4; ++tm) {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    __hip_atomic_store(reinterpret_cast<uint32_t*>(mine + ((tn * 4 + tm) * 4 + j) * kBlockThreads),
+                                       __float_as_uint(acc[tn][tm][j]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        if (t == 0) {
+            *arrival = __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(p.exchange) + beyond / p.sharers, 1u,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (*arrival != sharers - 1) return;
+        for (uint32_t other = 0; other < sharers; ++other) {
+            if (other == share) continue;
+            const float* theirs = sums + static_cast<uint64_t>(other) * (kBlockThreads * 64) + t;
+#pragma unroll
+            for (uint32_t tn = 0; tn < 4; ++tn) {
+#pragma unroll
+                for (uint32_t tm = 0; tm < 4; ++tm) {
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j) {
+                        acc[tn][tm][j] += __uint_as_float(__hip_atomic_load(
+                            reinterpret_cast<const uint32_t*>(theirs + ((tn * 4 + tm) * 4 + j) * kBlockThreads),
+                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    }
+                }
+            }
+        }
+        __syncthreads();   // the count has been read by every wave before the tiles reach its place
+    }
     // ---- store: through a tile of the wave's own in LDS ([m][n], rows 16 B apart from a
     // multiple of 128), read back as 16-byte pieces: 128 contiguous bytes per m
-    __syncthreads();   // nobody reads the stages any more (nor the sums, which the tiles do not reach)
     uint8_t* tile = lds + wave * 64 * kOutRowBytes;
 #pragma unroll
     for (uint32_t tm = 0; tm < 4; ++tm) {
@@ -644,11 +709,48 @@ int32_t check_block_operands(const Q4Projection& p) {
     return TT_OK;
 }
 
-int32_t launch_block(const Q4Projection& p, hipStream_t stream) {
+__global__ void clear_counts_kernel(uint32_t* words, uint32_t count) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) words[i] = 0;
+}
+
+// Tiles go to workgroups in rounds of one per compute unit.  A block of the reference's size
+// leaves the last round partly filled - 2048 rows of the attention in-projection are 576 tiles,
+// two rounds and a quarter on 256 compute units, of the out-projection 128, half a round - and
+// a partly filled round costs a whole one.  Where the queue has a workspace, the tiles of that
+// round are shared: 2, 4 or 8 workgroups (as many as fit the idle compute units and divide
+// the windows of eight groups) take a slice of K each and exchange their sums through it.
+int32_t launch_block(const Q4Projection& projection, hipStream_t stream) {
+    Q4Projection p = projection;
     const uint32_t out_rows = p.first_row[p.segments];
-    hipLaunchKernelGGL(q4_block_kernel,
-                       dim3((out_rows + kBlockN - 1) / kBlockN, (p.rows + kBlockM - 1) / kBlockM),
-                       dim3(kBlockThreads), kBlockLdsBytes, stream, p);
+    p.tiles_n = (out_rows + kBlockN - 1) / kBlockN;
+    const uint32_t tiles = p.tiles_n * ((p.rows + kBlockM - 1) / kBlockM);
+    p.whole_tiles = tiles;
+    p.sharers = 1;
+    p.exchange = nullptr;
+    const StreamWorkspace workspace = stream_workspace(stream);
+    if (workspace.base != nullptr && workspace.compute_units != 0) {
+        const uint32_t units = workspace.compute_units;
+        const uint32_t last_round = tiles % units;
+        const uint32_t windows = p.k_size / (8 * kQ4Group);
+        uint32_t sharers = 1;
+        for (uint32_t s = 8; s >= 2 && last_round != 0; s >>= 1) {
+            if (last_round * s <= units && windows % s == 0) {
+                sharers = s;
+                break;
+            }
+        }
+        if (sharers > 1 && last_round * 4 <= kExchangeCountBytes &&
+            kExchangeCountBytes + last_round * sharers * kExchangeShareBytes <= workspace.bytes) {
+            p.whole_tiles = tiles - last_round;
+            p.sharers = sharers;
+            p.exchange = workspace.base;
+            hipLaunchKernelGGL(clear_counts_kernel, dim3((last_round + 255) / 256), dim3(256), 0, stream,
+                               reinterpret_cast<uint32_t*>(p.exchange), last_round);
+        }
+    }
+    const uint32_t workgroups = p.whole_tiles + (tiles - p.whole_tiles) * p.sharers;
+    hipLaunchKernelGGL(q4_block_kernel, dim3(workgroups), dim3(kBlockThreads), kBlockLdsBytes, stream, p);
     return TT_OK;
 }
 
