@@ -141,8 +141,9 @@ uint32_t tt_device_compute_units(const tt_device* device);
 /* create_command_queue (resources.h:239): one in-order HIP stream.  A queue also owns a
  * workspace in device memory (270,336 bytes per compute unit: 69 MB on 256) for operators
  * whose reference bindings carry no scratch - attention_flash_v2_blk / attention_streaming_blk
- * share the key walks of a block of few rows through it; a queue whose workspace could not be
- * allocated works without. */
+ * share the key walks of a block of few rows through it, attn_project_blk / gdn_project_blk /
+ * outproj_blk the tiles of their last, partly filled round; a queue whose workspace could not
+ * be allocated works without. */
 int32_t tt_queue_create(tt_device* device, tt_queue** out);
 void tt_queue_destroy(tt_queue* queue);
 /* The HIP stream (hipStream_t) behind a queue, for event timing by the caller. */
