@@ -820,7 +820,9 @@ def main():
         line["detail"]["q4_projections"] = (
             [q4_sweep.measure(dev, queue, lib, name, LANES, False, 3, matrix_unit=True)
              for name in q4_sweep.FAMILIES] +
-            [q4_sweep.measure(dev, queue, lib, name, 16384, True, 6) for name in q4_sweep.FAMILIES])
+            [q4_sweep.measure(dev, queue, lib, name, 16384, True, 6) for name in q4_sweep.FAMILIES] +
+            # the reference's block size: the last, partly filled round of tiles is shared
+            [q4_sweep.measure(dev, queue, lib, name, 2048, True, 6) for name in q4_sweep.FAMILIES])
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(threads)
     print(json.dumps(line))
