@@ -434,96 +434,122 @@ def config5_decode_point(dev, queue, lib, torch, attention, lanes, visible):
             "algorithmic_gbs": round((kv + gdn) / (us * 1e-6) / 1e9, 1)}
 
 
+class PrefillFamily:
+    """The attention family of all 40 layers over blocks of 2048 rows: per Gated DeltaNet layer
+    conv, gates, chunk-64 recurrence and gate-norm, per attention layer rope and causal flash
+    attention over the lane's cache so far.  Own caches and recurrent state per layer and
+    lane; the projections (resident random slabs) are shared by the layers of a kind."""
+
+    def __init__(self, dev, lib, torch, lanes, tokens):
+        from tatara_amd import backend as B
+        self.B, self.dev, self.lib = B, dev, lib
+        self.lanes, self.tokens = lanes, tokens
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(0xC5F1 + tokens)
+        self.rows_max = min(CONFIG5_BLOCK_ROWS, tokens)
+        mk = dev.create_buffer
+
+        def rb(n, sigma=1.0):
+            t = (torch.randn(n, generator=gen, device="cuda") * sigma).to(torch.bfloat16)
+            return dev.wrap(t.data_ptr(), n * 2, keepalive=t)
+
+        self.ones256 = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
+        self.ones128 = dev.buffer_from(np.full(128, 0x3F80, np.uint16))
+        self.a_proj, self.g_proj = rb(self.rows_max * 9216), rb(self.rows_max * 12352, 0.5)
+        self.conv_w = rb(4 * 8192, 0.5)
+        rng = np.random.default_rng(5)
+        self.a_log = dev.buffer_from((rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16)
+                                     .astype(np.uint16))
+        self.dt_bias = dev.buffer_from(np.zeros(32, np.uint16))
+        attention_layers = LAYERS // PERIOD
+        self.stripe_bytes = 2 * tokens * 256 * 2
+        self.caches = [(mk(lanes * self.stripe_bytes), mk(lanes * self.stripe_bytes))
+                       for _ in range(attention_layers)]
+        self.conv_bytes, self.rec_bytes = 3 * 8192 * 2, 32 * 128 * 128 * 4
+        self.states = [(mk(2 * lanes * self.conv_bytes), mk(2 * lanes * self.rec_bytes))
+                       for _ in range(LAYERS - attention_layers)]
+
+    def working_set(self):
+        """The block-sized buffers one stream of blocks works in."""
+        B, mk, rows_max, units = self.B, self.dev.create_buffer, self.rows_max, self.dev.compute_units
+        work = {name: mk(rows_max * 8192) for name in ("q", "gate", "out", "qk", "v", "z", "y")}
+        work["decay"], work["beta"] = mk(rows_max * 128), mk(rows_max * 128)
+        work["chunk"] = mk(((rows_max + 63) // 64) * 32 * 115712)
+        # a 2048-row block is 128 workgroups of the flash kernel: the host shares each position
+        # tile's key walk between as many workgroups as fill the device (attention_flash_split_blk)
+        work["shared_walk"] = mk(max(
+            [B.flash_prefill_scratch_bytes(r, B.flash_prefill_splits(r, self.tokens, units))
+             for r in range(32, rows_max + 1, 32)] + [256]))
+        return work
+
+    def record_block(self, cb, w, lane, base, rows, swapped):
+        B, P, tokens = self.B, self.lib.pipeline, self.tokens
+        units = self.dev.compute_units
+        attn = gdn = 0
+        for layer in range(LAYERS):
+            if layer % PERIOD == PERIOD - 1:
+                keys = (self.caches[attn][0], lane * self.stripe_bytes)
+                values = (self.caches[attn][1], lane * self.stripe_bytes)
+                attn += 1
+                cb.encode(P("attn_qk_rope_blk"),
+                          {0: self.a_proj, 1: self.ones256, 2: self.ones256, 3: w["q"], 4: w["gate"],
+                           5: keys, 6: values}, {7: base, 8: tokens}, (18, rows), (256,))
+                cb.barrier()
+                sharers = B.flash_prefill_splits(rows, base + rows, units)
+                if sharers > 1:
+                    cb.encode(P("attention_flash_split_blk"),
+                              {0: w["q"], 1: keys, 2: values, 3: w["gate"], 4: w["out"], 9: w["shared_walk"]},
+                              {5: base + rows, 6: tokens, 7: rows, 8: base, 10: sharers},
+                              (16, (rows + 15) // 16), (256,))
+                else:
+                    cb.encode(P("attention_flash_v2_blk"),
+                              {0: w["q"], 1: keys, 2: values, 3: w["gate"], 4: w["out"]},
+                              {5: base + rows, 6: tokens, 7: rows, 8: base},
+                              (16, (rows + 15) // 16), (256,))
+            else:
+                conv, rec = self.states[gdn]
+                gdn += 1
+                plane_in, plane_out = (2 * lane + 1, 2 * lane) if swapped else (2 * lane, 2 * lane + 1)
+                cb.encode(P("gdn_conv_blk"),
+                          {0: self.g_proj, 1: (conv, plane_in * self.conv_bytes), 2: self.conv_w, 3: w["qk"],
+                           4: w["v"], 5: w["z"], 6: (conv, plane_out * self.conv_bytes)}, {7: rows},
+                          (96, rows), (128,))
+                cb.encode(P("gdn_gates_blk"),
+                          {0: self.g_proj, 1: self.a_log, 2: self.dt_bias, 3: w["decay"], 4: w["beta"]},
+                          {5: rows}, (1, (rows + 3) // 4, 1), (32, 4, 1))
+                cb.barrier()
+                cb.encode(P("gdn_chunk_recurrence_blk"),
+                          {0: w["qk"], 1: w["v"], 2: w["decay"], 3: w["beta"], 4: w["chunk"],
+                           5: (rec, plane_in * self.rec_bytes), 6: w["y"], 7: (rec, plane_out * self.rec_bytes)},
+                          {8: rows}, (8, 32), (256,))
+                cb.barrier()
+                cb.encode(P("gdn_gate_norm_blk"), {0: w["y"], 1: w["z"], 2: self.ones128, 3: w["out"]}, {},
+                          (32, rows), (128,))
+            cb.barrier()
+
+    def blocks(self):
+        return [(base, min(CONFIG5_BLOCK_ROWS, self.tokens - base))
+                for base in range(0, self.tokens, CONFIG5_BLOCK_ROWS)]
+
+
 def config5_prefill_point(dev, queue, lib, torch, lanes, tokens):
-    """`tokens` new tokens of each of `lanes` lanes, lane after lane, through the attention
-    family of all 40 layers in blocks of 2048 rows: per Gated DeltaNet layer conv, gates,
-    chunk-64 recurrence and gate-norm, per attention layer rope and causal flash attention
-    over the lane's cache so far.  Own caches and recurrent state per layer and lane;
-    the projections (resident random slabs) are shared by the layers of a kind.  Device time
-    of each block's command buffer (launch gaps included), summed."""
-    from tatara_amd import backend as B
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0xC5F1 + tokens)
-    rows_max = min(CONFIG5_BLOCK_ROWS, tokens)
-    mk = dev.create_buffer
-
-    def rb(n, sigma=1.0):
-        t = (torch.randn(n, generator=gen, device="cuda") * sigma).to(torch.bfloat16)
-        return dev.wrap(t.data_ptr(), n * 2, keepalive=t)
-
-    P = lib.pipeline
-    ones256 = dev.buffer_from(np.full(256, 0x3F80, np.uint16))
-    ones128 = dev.buffer_from(np.full(128, 0x3F80, np.uint16))
-    a_proj, g_proj = rb(rows_max * 9216), rb(rows_max * 12352, 0.5)
-    conv_w = rb(4 * 8192, 0.5)
-    rng = np.random.default_rng(5)
-    a_log = dev.buffer_from((rng.uniform(-4.0, -2.5, 32).astype(np.float32).view(np.uint32) >> 16)
-                            .astype(np.uint16))
-    dt_bias = dev.buffer_from(np.zeros(32, np.uint16))
-    q, gate, out = (mk(rows_max * 8192) for _ in range(3))
-    qk, v, z, y = (mk(rows_max * 8192) for _ in range(4))
-    decay, beta = mk(rows_max * 128), mk(rows_max * 128)
-    chunk = mk(((rows_max + 63) // 64) * 32 * 115712)
-    # a 2048-row block is 128 workgroups of the flash kernel: the host shares each position
-    # tile's key walk between as many workgroups as fill the device (attention_flash_split_blk)
-    units = dev.compute_units
-    shared_walk = mk(max([B.flash_prefill_scratch_bytes(r, B.flash_prefill_splits(r, tokens, units))
-                          for r in range(32, rows_max + 1, 32)] + [256]))
-    attention_layers = LAYERS // PERIOD
-    stripe_bytes = 2 * tokens * 256 * 2
-    caches = [(mk(lanes * stripe_bytes), mk(lanes * stripe_bytes)) for _ in range(attention_layers)]
-    conv_bytes, rec_bytes = 3 * 8192 * 2, 32 * 128 * 128 * 4
-    states = [(mk(2 * lanes * conv_bytes), mk(2 * lanes * rec_bytes))
-              for _ in range(LAYERS - attention_layers)]
+    """`tokens` new tokens of each of `lanes` lanes, lane after lane on one queue, through the
+    attention family of all 40 layers in blocks of 2048 rows.  Device time of each block's
+    command buffer (launch gaps included), summed."""
+    family = PrefillFamily(dev, lib, torch, lanes, tokens)
+    work = family.working_set()
     total_ms = 0.0
     for lane in range(lanes):
         swapped = False
-        for base in range(0, tokens, CONFIG5_BLOCK_ROWS):
-            rows = min(CONFIG5_BLOCK_ROWS, tokens - base)
+        for base, rows in family.blocks():
             cb = queue.create_command_buffer()
             cb.begin_compute_pass()
-            attn = gdn = 0
-            for layer in range(LAYERS):
-                if layer % PERIOD == PERIOD - 1:
-                    keys = (caches[attn][0], lane * stripe_bytes)
-                    values = (caches[attn][1], lane * stripe_bytes)
-                    attn += 1
-                    cb.encode(P("attn_qk_rope_blk"),
-                              {0: a_proj, 1: ones256, 2: ones256, 3: q, 4: gate, 5: keys, 6: values},
-                              {7: base, 8: tokens}, (18, rows), (256,))
-                    cb.barrier()
-                    sharers = B.flash_prefill_splits(rows, base + rows, units)
-                    if sharers > 1:
-                        cb.encode(P("attention_flash_split_blk"),
-                                  {0: q, 1: keys, 2: values, 3: gate, 4: out, 9: shared_walk},
-                                  {5: base + rows, 6: tokens, 7: rows, 8: base, 10: sharers},
-                                  (16, (rows + 15) // 16), (256,))
-                    else:
-                        cb.encode(P("attention_flash_v2_blk"), {0: q, 1: keys, 2: values, 3: gate, 4: out},
-                                  {5: base + rows, 6: tokens, 7: rows, 8: base},
-                                  (16, (rows + 15) // 16), (256,))
-                else:
-                    conv, rec = states[gdn]
-                    gdn += 1
-                    plane_in, plane_out = (2 * lane + 1, 2 * lane) if swapped else (2 * lane, 2 * lane + 1)
-                    cb.encode(P("gdn_conv_blk"),
-                              {0: g_proj, 1: (conv, plane_in * conv_bytes), 2: conv_w, 3: qk, 4: v, 5: z,
-                               6: (conv, plane_out * conv_bytes)}, {7: rows}, (96, rows), (128,))
-                    cb.encode(P("gdn_gates_blk"), {0: g_proj, 1: a_log, 2: dt_bias, 3: decay, 4: beta},
-                              {5: rows}, (1, (rows + 3) // 4, 1), (32, 4, 1))
-                    cb.barrier()
-                    cb.encode(P("gdn_chunk_recurrence_blk"),
-                              {0: qk, 1: v, 2: decay, 3: beta, 4: chunk, 5: (rec, plane_in * rec_bytes),
-                               6: y, 7: (rec, plane_out * rec_bytes)}, {8: rows}, (8, 32), (256,))
-                    cb.barrier()
-                    cb.encode(P("gdn_gate_norm_blk"), {0: y, 1: z, 2: ones128, 3: out}, {},
-                              (32, rows), (128,))
-                cb.barrier()
+            family.record_block(cb, work, lane, base, rows, swapped)
             cb.end_compute_pass()
             total_ms += cb.commit().wait()
             swapped = not swapped
     total = lanes * tokens
-    del caches, states
+    del family, work
     torch.cuda.empty_cache()
     return {"lanes": lanes, "tokens": tokens, "block_rows": CONFIG5_BLOCK_ROWS,
             "family_ms": round(total_ms, 3), "tok_per_s": round(total / (total_ms * 1e-3)),
