@@ -180,12 +180,13 @@ def test_block_projection(family, name, rows):
 
 @pytest.mark.parametrize("family,name", [(ATTN, "attn_project_blk"), (GDN, "gdn_project_blk"),
                                          (OUT, "outproj_blk")], ids=["attn", "gdn", "out"])
-@pytest.mark.parametrize("rows", [256, 257, 700, 16384])
+@pytest.mark.parametrize("rows", [256, 257, 700, 2048, 16384])
 def test_block_projection_over_several_row_tiles(family, name, rows):
     """Blocks that span more than one 256-row tile of the block kernel, up to the 16384 rows
-    the benchmark times: every output row is produced, and a sample of rows - the first and
-    last of the block, the rows either side of each tile boundary sampled, a few inside -
-    is held to the checker."""
+    the benchmark times, among them the reference's 2048-row block, whose last, partly filled
+    round of tiles is shared between workgroups (as that of most sizes here is): every output
+    row is produced, and a sample of rows - the first and last of the block, the rows either
+    side of each tile boundary sampled, a few inside - is held to the checker."""
     print(f"[case] {name} rows={rows} (sampled rows)", flush=True)
     B, dev, queue, lib = gpu()
     host, bindings = _family(dev, family, 0x9600)
